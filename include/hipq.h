@@ -1,0 +1,175 @@
+/* SPDX-License-Identifier: Apache-2.0 */
+/**
+ * @file   hipq.h
+ * @brief  C ABI of the MI355X (gfx950) quantized-weight matmul back-end.
+ *
+ * One shared library (libhipq.so) exports exactly these symbols. Signatures use
+ * plain pointers and sizes only. Every function returns 0 on success or a
+ * negative hipq_status and never throws; hipq_last_error() gives the message
+ * of the calling thread's last failure. All entry points may be called from
+ * several host threads at once (the reference's MoE layer calls its matmul
+ * from inside an OpenMP loop).
+ *
+ * Reference interfaces replaced (paths relative to the reference checkout):
+ *   nntrainer/tensor/cpu_backend/cpu_backend.h:937-1165  (gemm_q4_0, gemm_q4_K,
+ *       gemm_q6_K, quantize_q4_0/q4_K/q6_K, repack_q4_0/q4_K, init_backend)
+ *   nntrainer/tensor/cpu_backend/ggml_interface/ggml_interface.h:28-342
+ *   nntrainer/tensor/float_tensor.cpp:923-969            (dotQnK dispatch)
+ *   Applications/CausalLM/layers/qwen_moe_layer.cpp:394-503 (MoE block)
+ *
+ * Memory: `mem` says where the caller's buffers live. HIPQ_MEM_DEVICE buffers are
+ * device pointers; the call only enqueues work on `stream` and returns.
+ * HIPQ_MEM_HOST buffers are ordinary host memory; the call copies in, runs,
+ * copies out and returns when the result is in the host buffer.
+ * `stream` is a hipStream_t passed as void* (NULL = the default stream).
+ */
+#ifndef HIPQ_H
+#define HIPQ_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#if defined(__GNUC__)
+#define HIPQ_API __attribute__((visibility("default")))
+#else
+#define HIPQ_API
+#endif
+
+typedef enum hipq_status {
+  HIPQ_OK = 0,
+  HIPQ_ERR_INVALID_ARGUMENT = -1, /* bad dims / null pointer / unknown enum  */
+  HIPQ_ERR_NOT_INITIALIZED = -2,  /* hipq_init has not succeeded             */
+  HIPQ_ERR_RUNTIME = -3,          /* a HIP call failed (message has details) */
+  HIPQ_ERR_NOT_SUPPORTED = -4,    /* valid request this build cannot serve   */
+  HIPQ_ERR_OUT_OF_MEMORY = -5
+} hipq_status;
+
+/** Weight formats; values are the ggml type ids the reference uses
+ *  (nntr_ggml_impl_common.h:166-176). */
+typedef enum hipq_dtype { HIPQ_Q4_0 = 2, HIPQ_Q4_K = 12, HIPQ_Q6_K = 14 } hipq_dtype;
+
+/** Byte layout of weights handed to hipq_weight_create.
+ *  CANONICAL: rows of plain ggml blocks (block_q4_0 18 B / block_q4_K 144 B /
+ *             block_q6_K 210 B), row n = output column n (W^T, N x K).
+ *  X8:        the 8-row interleave NNTrainer stores in its tensors and model
+ *             files for Q4_0 and Q4_K (repack_q4_0 / repack_q4_K,
+ *             nntr_ggml_impl.cpp:8189-8245). Not defined for Q6_K. */
+typedef enum hipq_layout { HIPQ_LAYOUT_CANONICAL = 0, HIPQ_LAYOUT_X8 = 1 } hipq_layout;
+
+typedef enum hipq_mem { HIPQ_MEM_HOST = 0, HIPQ_MEM_DEVICE = 1 } hipq_mem;
+
+/** Which of the reference's two Q8_K activation quantizers to reproduce.
+ *  ROW: quantize_row_q8_K (nntr_ggml_impl_quant.cpp:1334-1374) -- used for
+ *       M == 1, for leftover rows M % 4 and for every Q6_K row.
+ *  MAT: per-row content of quantize_mat_q8_K_4x8 (nntr_ggml_impl.cpp:7504-7737)
+ *       -- used for rows [0, 4*(M/4)) of a Q4_K matmul with M > 1.
+ *  They differ only in rare roundings and in the sign convention when +amax and
+ *  -amax both occur. */
+typedef enum hipq_q8k_variant { HIPQ_Q8K_ROW = 0, HIPQ_Q8K_MAT = 1 } hipq_q8k_variant;
+
+/** Opaque device-resident weight matrix. */
+typedef struct hipq_weight *hipq_weight_t;
+
+/** Replaces init_backend() (x86_compute_backend.cpp:31): selects the GPU and
+ *  creates the library state. Idempotent for the same device. */
+HIPQ_API int hipq_init(int device);
+/** Frees every cached buffer. Weights must be destroyed first. */
+HIPQ_API int hipq_shutdown(void);
+HIPQ_API const char *hipq_last_error(void);
+/** Library version, "major.minor". */
+HIPQ_API const char *hipq_version(void);
+
+/** Bytes of an N x K weight matrix in canonical or x8 form (same size), or a
+ *  negative status when K is not a multiple of the block size (32 for Q4_0,
+ *  256 for Q4_K / Q6_K; q4_0_tensor.cpp:25-28, q4_k_tensor.cpp:23-27). */
+HIPQ_API int64_t hipq_weight_nbytes(int dtype, int64_t N, int64_t K);
+
+/** Uploads a weight matrix and re-lays it out once for the GPU kernels
+ *  (structure-of-arrays: quants, scales and headers in separate 16-byte-aligned
+ *  planes). `bytes` may be host or device memory (`mem`). The handle is what
+ *  FullyConnectedLayer's weight tensor becomes on this back-end. */
+HIPQ_API int hipq_weight_create(int dtype, int layout, int64_t N, int64_t K,
+                                const void *bytes, int mem, hipq_weight_t *out);
+HIPQ_API int hipq_weight_destroy(hipq_weight_t w);
+HIPQ_API int hipq_weight_dims(hipq_weight_t w, int *dtype, int64_t *N, int64_t *K);
+
+/** Activation quantizer fp32 -> Q8_0, canonical block_q8_0 output (34 B per 32
+ *  values), M rows of K values (K % 32 == 0). Replaces nntr_quantize_row_q8_0 /
+ *  nntr_quantize_mat_q8_0_4x8 (nntr_ggml_impl_quant.cpp:532-875,
+ *  nntr_ggml_impl.cpp:7788-8012), whose per-row content is identical. */
+HIPQ_API int hipq_quantize_q8_0(const float *A, int64_t M, int64_t K, int64_t lda,
+                                void *out_blocks, int mem, void *stream);
+/** Activation quantizer fp32 -> Q8_K, canonical block_q8_K output (292 B per
+ *  256 values: fp32 d, 256 int8, 16 int16 group sums), K % 256 == 0. */
+HIPQ_API int hipq_quantize_q8_K(const float *A, int64_t M, int64_t K, int64_t lda,
+                                int variant, void *out_blocks, int mem, void *stream);
+
+/** C[M x N] = A[M x K] . W^T with on-the-fly activation quantization; the GPU
+ *  form of gemm_q4_0 / gemm_q4_K / gemm_q6_K (x86_compute_backend.cpp:301-341)
+ *  as reached from FloatTensor::dotQnK (float_tensor.cpp:923-969). M == 1 runs
+ *  the decode GEMV kernels, M > 1 the prefill GEMM kernels. lda >= K and
+ *  ldc >= N are row strides in elements. */
+HIPQ_API int hipq_matmul(hipq_weight_t w, const float *A, int64_t M, int64_t lda,
+                         float *C, int64_t ldc, int mem, void *stream);
+
+/** One fp32 activation against several weights sharing K (the QKV layer's
+ *  vector dot, float_tensor.cpp:724-798): quantizes A once. */
+HIPQ_API int hipq_matmul_multi(int count, const hipq_weight_t *w, const float *A,
+                               int64_t M, int64_t lda, float *const *C,
+                               const int64_t *ldc, int mem, void *stream);
+
+/** Mixture-of-experts feed-forward block (MoELayer::incremental_forwarding,
+ *  qwen_moe_layer.cpp:394-503): softmax over E router logits, top-k, weights
+ *  renormalised to sum 1, per (token, expert) SwiGLU MLP
+ *  down(silu(gate(x)) * up(x)), outputs combined in ascending expert order.
+ *  Tokens are sorted by expert on the device and each projection is one grouped
+ *  launch over the active experts. */
+typedef struct hipq_moe_desc {
+  int32_t tokens;       /* T                                   */
+  int32_t hidden;       /* H, K of gate/up, N of down          */
+  int32_t intermediate; /* I, N of gate/up, K of down          */
+  int32_t experts;      /* E                                   */
+  int32_t topk;         /* experts per token                   */
+  int32_t renormalize;  /* 1: divide top-k weights by their sum (incremental
+                           path); 0: use softmax values as is (forwarding path,
+                           qwen_moe_layer.cpp:161-259)           */
+} hipq_moe_desc;
+
+/** gate/up/down: E handles each. x [T x H]. Exactly one of `router_logits`
+ *  [T x E] (logits already computed) and `router_weight` [H x E] fp32 (the
+ *  layer's "gate" weight; logits = x . router_weight) must be non-NULL.
+ *  y [T x H]. topk_idx [T x topk] int32 and topk_w [T x topk] fp32 are optional
+ *  outputs of the routing. */
+HIPQ_API int hipq_moe_forward(const hipq_moe_desc *desc, const hipq_weight_t *gate,
+                              const hipq_weight_t *up, const hipq_weight_t *down,
+                              const float *x, const float *router_logits,
+                              const float *router_weight, float *y,
+                              int32_t *topk_idx, float *topk_w, int mem,
+                              void *stream);
+
+/** Offline weight quantizers fp32 [N x K] -> canonical blocks, on the GPU.
+ *  Replace quantize_q4_0 / quantize_q4_K / quantize_q6_K
+ *  (x86_compute_backend.cpp:343-370 -> nntr_ggml_impl_quant.cpp:452-467,
+ *  1062-1077, 1274-1289). */
+HIPQ_API int hipq_quantize_weights(int dtype, const float *W, int64_t N, int64_t K,
+                                   void *out_blocks, int mem, void *stream);
+
+/** Timing helper for benchmarks: runs the matmul `iters` times on device
+ *  buffers, rotating over `n_weights` handles (distinct copies defeat the
+ *  last-level cache), brackets the launches with HIP events recorded on
+ *  `stream` and returns the average milliseconds per call.
+ *  phase 0: whole call (activation quantizer + block-dot kernel);
+ *  phase 1: block-dot kernel only, on activations quantized once beforehand;
+ *  phase 2: activation quantizer only. */
+HIPQ_API int hipq_time_matmul(int n_weights, const hipq_weight_t *w, const float *A,
+                              int64_t M, int64_t lda, float *C, int64_t ldc,
+                              int iters, int phase, void *stream, float *ms_per_call);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HIPQ_H */

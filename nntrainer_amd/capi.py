@@ -1,0 +1,178 @@
+"""ctypes binding of the libhipq C ABI (include/hipq.h).
+
+Device buffers are passed as raw addresses (``tensor.data_ptr()``); torch is only
+the allocator and stream provider of the callers, it is not imported here.
+"""
+import ctypes as C
+import os
+import subprocess
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "lib", "libhipq.so")
+CSRC = os.path.join(HERE, "csrc")
+
+Q4_0, Q4_K, Q6_K = 2, 12, 14
+LAYOUT_CANONICAL, LAYOUT_X8 = 0, 1
+MEM_HOST, MEM_DEVICE = 0, 1
+Q8K_ROW, Q8K_MAT = 0, 1
+DTYPES = {"q4_0": Q4_0, "q4_K": Q4_K, "q6_K": Q6_K}
+
+SYMBOLS = [
+    "hipq_init", "hipq_shutdown", "hipq_last_error", "hipq_version", "hipq_weight_nbytes",
+    "hipq_weight_create", "hipq_weight_destroy", "hipq_weight_dims", "hipq_quantize_q8_0",
+    "hipq_quantize_q8_K", "hipq_matmul", "hipq_matmul_multi", "hipq_moe_forward",
+    "hipq_quantize_weights", "hipq_time_matmul",
+]
+
+
+class HipqError(RuntimeError):
+    def __init__(self, code, msg):
+        super().__init__("hipq error %d: %s" % (code, msg))
+        self.code = code
+
+
+class MoeDesc(C.Structure):
+    _fields_ = [("tokens", C.c_int32), ("hidden", C.c_int32), ("intermediate", C.c_int32),
+                ("experts", C.c_int32), ("topk", C.c_int32), ("renormalize", C.c_int32)]
+
+
+def build(force=False):
+    """Compile libhipq.so for gfx950 with hipcc (cross-compiles without a GPU)."""
+    if force:
+        subprocess.check_call(["make", "-C", CSRC, "clean"], stdout=subprocess.DEVNULL)
+    subprocess.check_call(["make", "-C", CSRC, "-j8"], stdout=subprocess.DEVNULL)
+    return LIB_PATH
+
+
+_lib = None
+
+
+def lib():
+    """The loaded library. Fails loudly if it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.exists(LIB_PATH):
+            raise FileNotFoundError(
+                "%s is missing: build it with `make -C %s` (there is no fallback path)" % (LIB_PATH, CSRC))
+        L = C.CDLL(LIB_PATH)
+        vp, i64, i32 = C.c_void_p, C.c_int64, C.c_int
+        L.hipq_last_error.restype = C.c_char_p
+        L.hipq_version.restype = C.c_char_p
+        L.hipq_init.argtypes = [i32]
+        L.hipq_weight_nbytes.restype = i64
+        L.hipq_weight_nbytes.argtypes = [i32, i64, i64]
+        L.hipq_weight_create.argtypes = [i32, i32, i64, i64, vp, i32, C.POINTER(vp)]
+        L.hipq_weight_destroy.argtypes = [vp]
+        L.hipq_weight_dims.argtypes = [vp, C.POINTER(i32), C.POINTER(i64), C.POINTER(i64)]
+        L.hipq_quantize_q8_0.argtypes = [vp, i64, i64, i64, vp, i32, vp]
+        L.hipq_quantize_q8_K.argtypes = [vp, i64, i64, i64, i32, vp, i32, vp]
+        L.hipq_matmul.argtypes = [vp, vp, i64, i64, vp, i64, i32, vp]
+        L.hipq_matmul_multi.argtypes = [i32, C.POINTER(vp), vp, i64, i64, C.POINTER(vp),
+                                        C.POINTER(i64), i32, vp]
+        L.hipq_moe_forward.argtypes = [C.POINTER(MoeDesc), C.POINTER(vp), C.POINTER(vp),
+                                       C.POINTER(vp), vp, vp, vp, vp, vp, vp, i32, vp]
+        L.hipq_quantize_weights.argtypes = [i32, vp, i64, i64, vp, i32, vp]
+        L.hipq_time_matmul.argtypes = [i32, C.POINTER(vp), vp, i64, i64, vp, i64, i32, i32, vp,
+                                       C.POINTER(C.c_float)]
+        _lib = L
+    return _lib
+
+
+def check(rc):
+    if rc != 0:
+        raise HipqError(rc, lib().hipq_last_error().decode())
+
+
+def init(device=0):
+    check(lib().hipq_init(device))
+
+
+def shutdown():
+    check(lib().hipq_shutdown())
+
+
+def _addr(x):
+    """Address of a numpy array, a torch tensor, an int, or None."""
+    if x is None:
+        return None
+    if isinstance(x, int):
+        return x
+    if hasattr(x, "data_ptr"):
+        return x.data_ptr()
+    return x.ctypes.data
+
+
+class Weight:
+    """Device-resident quantized weight matrix (W^T: N rows of K values)."""
+
+    def __init__(self, dtype, n, k, blocks, layout=LAYOUT_CANONICAL, mem=MEM_HOST):
+        self.dtype = DTYPES.get(dtype, dtype)
+        self.n, self.k = n, k
+        self._h = C.c_void_p()
+        check(lib().hipq_weight_create(self.dtype, layout, n, k, _addr(blocks), mem, C.byref(self._h)))
+
+    @property
+    def handle(self):
+        return self._h
+
+    def destroy(self):
+        if self._h:
+            check(lib().hipq_weight_destroy(self._h))
+            self._h = C.c_void_p()
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass
+
+
+def weight_nbytes(dtype, n, k):
+    r = lib().hipq_weight_nbytes(DTYPES.get(dtype, dtype), n, k)
+    if r < 0:
+        raise HipqError(int(r), lib().hipq_last_error().decode())
+    return int(r)
+
+
+def quantize_q8_0(a, m, k, out, lda=None, mem=MEM_DEVICE, stream=None):
+    check(lib().hipq_quantize_q8_0(_addr(a), m, k, lda or k, _addr(out), mem, stream))
+
+
+def quantize_q8_K(a, m, k, out, variant=Q8K_ROW, lda=None, mem=MEM_DEVICE, stream=None):
+    check(lib().hipq_quantize_q8_K(_addr(a), m, k, lda or k, variant, _addr(out), mem, stream))
+
+
+def matmul(w, a, m, c, lda=None, ldc=None, mem=MEM_DEVICE, stream=None):
+    check(lib().hipq_matmul(w.handle, _addr(a), m, lda or w.k, _addr(c), ldc or w.n, mem, stream))
+
+
+def matmul_multi(ws, a, m, cs, mem=MEM_DEVICE, stream=None):
+    n = len(ws)
+    hs = (C.c_void_p * n)(*[w.handle.value for w in ws])
+    cp = (C.c_void_p * n)(*[_addr(c) for c in cs])
+    ld = (C.c_int64 * n)(*[w.n for w in ws])
+    check(lib().hipq_matmul_multi(n, hs, _addr(a), m, ws[0].k, cp, ld, mem, stream))
+
+
+def quantize_weights(dtype, w, n, k, out, mem=MEM_DEVICE, stream=None):
+    check(lib().hipq_quantize_weights(DTYPES.get(dtype, dtype), _addr(w), n, k, _addr(out), mem, stream))
+
+
+def moe_forward(tokens, hidden, inter, experts, topk, gate, up, down, x, y, router_logits=None,
+                router_weight=None, topk_idx=None, topk_w=None, renormalize=True, mem=MEM_DEVICE,
+                stream=None):
+    d = MoeDesc(tokens, hidden, inter, experts, topk, 1 if renormalize else 0)
+    arr = lambda ws: (C.c_void_p * experts)(*[w.handle.value for w in ws])
+    check(lib().hipq_moe_forward(C.byref(d), arr(gate), arr(up), arr(down), _addr(x),
+                                 _addr(router_logits), _addr(router_weight), _addr(y),
+                                 _addr(topk_idx), _addr(topk_w), mem, stream))
+
+
+def time_matmul(ws, a, m, c, iters, phase=0, stream=None):
+    """Average milliseconds per call, HIP events on `stream`, rotating over `ws`."""
+    n = len(ws)
+    hs = (C.c_void_p * n)(*[w.handle.value for w in ws])
+    ms = C.c_float()
+    check(lib().hipq_time_matmul(n, hs, _addr(a), m, ws[0].k, _addr(c), ws[0].n, iters, phase,
+                                 stream, C.byref(ms)))
+    return ms.value

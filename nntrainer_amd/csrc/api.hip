@@ -1,0 +1,607 @@
+// SPDX-License-Identifier: Apache-2.0
+/**
+ * @file   api.hip
+ * @brief  C ABI of libhipq (include/hipq.h): library state, per-stream
+ *         workspaces, weight upload, and the matmul / quantize / MoE dispatch.
+ *
+ * The dispatch in hipq_matmul restates the control flow of the reference
+ * wrappers (nntrainer/tensor/cpu_backend/ggml_interface/ggml_interface_omp.cpp:
+ * 303-390 Q4_0, 404-487 Q4_K, 500-566 Q6_K in the reference checkout):
+ * which activation quantizer each row gets (Q8_0; Q8_K row semantics for M == 1,
+ * for the M % 4 leftover rows and for every Q6_K row; Q8_K 4-row semantics for
+ * rows [0, 4*(M/4)) of a Q4_K matmul with M > 1), then GEMV for decode shapes
+ * and the matrix-core GEMM for prefill shapes. There is no CPU fallback: without
+ * a gfx950 device hipq_init fails and every other call reports
+ * HIPQ_ERR_NOT_INITIALIZED.
+ */
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <mutex>
+#include <unordered_map>
+#include <vector>
+
+#include "hipq_internal.h"
+
+namespace {
+
+thread_local char tl_error[768] = "";
+
+struct Workspace {
+  void *ptr = nullptr;
+  size_t bytes = 0;
+};
+
+struct MoeTable {
+  std::vector<const hipq_weight *> key;
+  WView *dev = nullptr;
+};
+
+struct State {
+  std::mutex mu;
+  bool ready = false;
+  int device = -1;
+  std::unordered_map<hipStream_t, Workspace> ws;
+  std::unordered_map<hipStream_t, MoeTable> moe_tables;
+  int64_t live_weights = 0;
+};
+State g;
+
+} // namespace
+
+namespace hipq {
+
+int fail(int code, const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(tl_error, sizeof(tl_error), fmt, ap);
+  va_end(ap);
+  return code;
+}
+
+} // namespace hipq
+
+using hipq::fail;
+
+namespace {
+
+int require_ready() {
+  if (!g.ready) return fail(HIPQ_ERR_NOT_INITIALIZED, "hipq_init has not succeeded");
+  hipError_t e = hipSetDevice(g.device);
+  if (e != hipSuccess) return fail(HIPQ_ERR_RUNTIME, "hipSetDevice(%d): %s", g.device, hipGetErrorString(e));
+  return HIPQ_OK;
+}
+
+/* Per-stream scratch, grown on demand. Work queued on one stream runs in order,
+ * so consecutive calls on a stream may share it; different streams never do. */
+int workspace(hipStream_t s, size_t bytes, void **out) {
+  std::lock_guard<std::mutex> lk(g.mu);
+  Workspace &w = g.ws[s];
+  if (w.bytes < bytes) {
+    if (w.ptr) {
+      HIPQ_HIP(hipStreamSynchronize(s));
+      HIPQ_HIP(hipFree(w.ptr));
+      w.ptr = nullptr;
+      w.bytes = 0;
+    }
+    size_t want = (bytes + ((size_t)1 << 20) - 1) & ~(((size_t)1 << 20) - 1);
+    hipError_t e = hipMalloc(&w.ptr, want);
+    if (e != hipSuccess) {
+      w.ptr = nullptr;
+      return fail(HIPQ_ERR_OUT_OF_MEMORY, "workspace of %zu bytes: %s", want, hipGetErrorString(e));
+    }
+    w.bytes = want;
+  }
+  *out = w.ptr;
+  return HIPQ_OK;
+}
+
+bool dtype_ok(int dt) { return dt == HIPQ_Q4_0 || dt == HIPQ_Q4_K || dt == HIPQ_Q6_K; }
+int64_t block_elems(int dt) { return dt == HIPQ_Q4_0 ? 32 : 256; }
+int64_t block_bytes(int dt) { return dt == HIPQ_Q4_0 ? 18 : dt == HIPQ_Q4_K ? 144 : 210; }
+
+QAct qact_rows(const QAct &a, int is_k, int64_t r0, int64_t rows) {
+  QAct v = a;
+  v.q = a.q + r0 * a.K;
+  if (is_k) {
+    v.d = a.d + r0 * (a.K / 256);
+    v.bsum = a.bsum + r0 * (a.K / 16);
+  } else {
+    v.meta = a.meta + r0 * (a.K / 32);
+  }
+  v.M = (int)rows;
+  return v;
+}
+
+/* Quantize the activations the way the reference does for this weight type. */
+int quantize_for(const hipq_weight *w, const float *A, int64_t M, int64_t lda, const QAct &qa,
+                 hipStream_t s) {
+  if (w->dtype == HIPQ_Q4_0) return hipq::launch_quantize_q8_0(A, M, w->K, lda, &qa, nullptr, s);
+  const int64_t mat_rows = (w->dtype == HIPQ_Q4_K && M > 1) ? (M / 4) * 4 : 0;
+  return hipq::launch_quantize_q8_K(A, M, w->K, lda, mat_rows, &qa, nullptr, s);
+}
+
+/* Block-dot stage on already quantized activations. */
+int multiply(const hipq_weight *w, const QAct &qa, int64_t M, float *C, int64_t ldc,
+             hipStream_t s) {
+  const int is_k = w->dtype != HIPQ_Q4_0;
+  if (M <= 8) return hipq::launch_gemv(w, &qa, (int)M, C, ldc, s);
+  if (w->dtype != HIPQ_Q6_K && w->K % 256 == 0) return hipq::launch_gemm(w, &qa, (int)M, C, ldc, s);
+  for (int64_t r0 = 0; r0 < M; r0 += 8) {
+    const int64_t rows = (M - r0) < 8 ? (M - r0) : 8;
+    QAct sub = qact_rows(qa, is_k, r0, rows);
+    int rc = hipq::launch_gemv(w, &sub, (int)rows, C + r0 * ldc, ldc, s);
+    if (rc) return rc;
+  }
+  return HIPQ_OK;
+}
+
+int check_matmul_args(hipq_weight_t w, const float *A, int64_t M, int64_t lda, const float *C,
+                      int64_t ldc) {
+  if (!w || !A || !C) return fail(HIPQ_ERR_INVALID_ARGUMENT, "null weight, activation or output");
+  if (M < 0) return fail(HIPQ_ERR_INVALID_ARGUMENT, "M = %lld", (long long)M);
+  if (lda < w->K) return fail(HIPQ_ERR_INVALID_ARGUMENT, "lda %lld < K %lld", (long long)lda, (long long)w->K);
+  if (ldc < w->N) return fail(HIPQ_ERR_INVALID_ARGUMENT, "ldc %lld < N %lld", (long long)ldc, (long long)w->N);
+  return HIPQ_OK;
+}
+
+int matmul_device(hipq_weight_t w, const float *A, int64_t M, int64_t lda, float *C, int64_t ldc,
+                  hipStream_t s) {
+  if (M == 0) return HIPQ_OK;
+  const int is_k = w->dtype != HIPQ_Q4_0;
+  void *mem = nullptr;
+  int rc = workspace(s, qact_bytes(is_k, M, w->K), &mem);
+  if (rc) return rc;
+  QAct qa = qact_carve(is_k, mem, M, w->K);
+  rc = quantize_for(w, A, M, lda, qa, s);
+  if (rc) return rc;
+  return multiply(w, qa, M, C, ldc, s);
+}
+
+struct DevBuf {
+  void *p = nullptr;
+  ~DevBuf() {
+    if (p) (void)hipFree(p);
+  }
+  int alloc(size_t n) {
+    hipError_t e = hipMalloc(&p, n ? n : 16);
+    if (e != hipSuccess) {
+      p = nullptr;
+      return fail(HIPQ_ERR_OUT_OF_MEMORY, "hipMalloc(%zu): %s", n, hipGetErrorString(e));
+    }
+    return HIPQ_OK;
+  }
+};
+
+} // namespace
+
+extern "C" {
+
+const char *hipq_last_error(void) { return tl_error; }
+const char *hipq_version(void) { return "0.1"; }
+
+int hipq_init(int device) {
+  std::lock_guard<std::mutex> lk(g.mu);
+  if (g.ready) {
+    if (g.device == device) return HIPQ_OK;
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "already initialised on device %d", g.device);
+  }
+  int count = 0;
+  hipError_t e = hipGetDeviceCount(&count);
+  if (e != hipSuccess || count <= 0)
+    return fail(HIPQ_ERR_RUNTIME, "no HIP device available (%s)", hipGetErrorString(e));
+  if (device < 0 || device >= count)
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "device %d out of range [0, %d)", device, count);
+  hipDeviceProp_t prop;
+  HIPQ_HIP(hipGetDeviceProperties(&prop, device));
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+    return fail(HIPQ_ERR_NOT_SUPPORTED, "device %d is %s; this library is built for gfx950 only",
+                device, prop.gcnArchName);
+  HIPQ_HIP(hipSetDevice(device));
+  g.device = device;
+  g.ready = true;
+  return HIPQ_OK;
+}
+
+int hipq_shutdown(void) {
+  std::lock_guard<std::mutex> lk(g.mu);
+  if (!g.ready) return HIPQ_OK;
+  if (g.live_weights)
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "%lld weights still alive", (long long)g.live_weights);
+  (void)hipSetDevice(g.device);
+  (void)hipDeviceSynchronize();
+  for (auto &kv : g.ws)
+    if (kv.second.ptr) (void)hipFree(kv.second.ptr);
+  g.ws.clear();
+  for (auto &kv : g.moe_tables)
+    if (kv.second.dev) (void)hipFree(kv.second.dev);
+  g.moe_tables.clear();
+  g.ready = false;
+  g.device = -1;
+  return HIPQ_OK;
+}
+
+int64_t hipq_weight_nbytes(int dtype, int64_t N, int64_t K) {
+  if (!dtype_ok(dtype)) return fail(HIPQ_ERR_INVALID_ARGUMENT, "unknown weight dtype %d", dtype);
+  if (N <= 0 || K <= 0 || K % block_elems(dtype))
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "N=%lld K=%lld: K must be a positive multiple of %lld",
+                (long long)N, (long long)K, (long long)block_elems(dtype));
+  return N * (K / block_elems(dtype)) * block_bytes(dtype);
+}
+
+int hipq_weight_create(int dtype, int layout, int64_t N, int64_t K, const void *bytes, int mem,
+                       hipq_weight_t *out) {
+  int rc = require_ready();
+  if (rc) return rc;
+  if (!out || !bytes) return fail(HIPQ_ERR_INVALID_ARGUMENT, "null argument");
+  *out = nullptr;
+  const int64_t nbytes = hipq_weight_nbytes(dtype, N, K);
+  if (nbytes < 0) return (int)nbytes;
+  if (layout != HIPQ_LAYOUT_CANONICAL && layout != HIPQ_LAYOUT_X8)
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "unknown layout %d", layout);
+  if (layout == HIPQ_LAYOUT_X8) {
+    if (dtype == HIPQ_Q6_K) return fail(HIPQ_ERR_INVALID_ARGUMENT, "Q6_K has no x8 layout");
+    /* same rule as the reference's repack: 8 rows interleaved, K % 8 == 0 */
+    if (N % 8 || K % 8)
+      return fail(HIPQ_ERR_INVALID_ARGUMENT, "x8 layout needs N %% 8 == 0 and K %% 8 == 0 (N=%lld K=%lld)",
+                  (long long)N, (long long)K);
+  }
+  if (N > INT32_MAX || K > INT32_MAX) return fail(HIPQ_ERR_INVALID_ARGUMENT, "dimension too large");
+
+  hipq_weight *w = new (std::nothrow) hipq_weight();
+  if (!w) return fail(HIPQ_ERR_OUT_OF_MEMORY, "host allocation failed");
+  w->dtype = dtype;
+  w->device = g.device;
+  w->N = N;
+  w->K = K;
+  /* planes, each 256-byte aligned */
+  auto up = [](size_t x) { return (x + 255) & ~(size_t)255; };
+  size_t o_qs = 0, o_qh = 0, o_hdr = 0, o_sc = 0, o_d = 0, total = 0;
+  if (dtype == HIPQ_Q4_0) {
+    o_qs = 0;
+    o_d = up((size_t)N * K / 2);
+    total = o_d + up((size_t)N * (K / 32) * 2);
+  } else if (dtype == HIPQ_Q4_K) {
+    o_qs = 0;
+    o_hdr = up((size_t)N * K / 2);
+    total = o_hdr + up((size_t)N * (K / 256) * 16);
+  } else {
+    o_qs = 0;
+    o_qh = up((size_t)N * K / 2);
+    o_sc = o_qh + up((size_t)N * K / 4);
+    o_d = o_sc + up((size_t)N * K / 16);
+    total = o_d + up((size_t)N * (K / 256) * 2);
+  }
+  hipError_t e = hipMalloc((void **)&w->base, total);
+  if (e != hipSuccess) {
+    delete w;
+    return fail(HIPQ_ERR_OUT_OF_MEMORY, "weight planes of %zu bytes: %s", total, hipGetErrorString(e));
+  }
+  w->bytes = total;
+  w->qs = w->base + o_qs;
+  w->qh = dtype == HIPQ_Q6_K ? w->base + o_qh : nullptr;
+  w->hdr = dtype == HIPQ_Q4_K ? w->base + o_hdr : nullptr;
+  w->sc = dtype == HIPQ_Q6_K ? (const int8_t *)(w->base + o_sc) : nullptr;
+  w->d = dtype != HIPQ_Q4_K ? (const uint16_t *)(w->base + o_d) : nullptr;
+
+  const uint8_t *src = (const uint8_t *)bytes;
+  DevBuf staging;
+  if (mem == HIPQ_MEM_HOST) {
+    rc = staging.alloc((size_t)nbytes);
+    if (!rc) {
+      e = hipMemcpy(staging.p, bytes, (size_t)nbytes, hipMemcpyHostToDevice);
+      if (e != hipSuccess) rc = fail(HIPQ_ERR_RUNTIME, "weight upload: %s", hipGetErrorString(e));
+    }
+    src = (const uint8_t *)staging.p;
+  } else if (mem != HIPQ_MEM_DEVICE) {
+    rc = fail(HIPQ_ERR_INVALID_ARGUMENT, "unknown mem kind %d", mem);
+  }
+  if (!rc) rc = hipq::launch_relayout(w, layout, src, nullptr);
+  if (!rc) {
+    e = hipStreamSynchronize(nullptr);
+    if (e != hipSuccess) rc = fail(HIPQ_ERR_RUNTIME, "weight relayout: %s", hipGetErrorString(e));
+  }
+  if (rc) {
+    (void)hipFree(w->base);
+    delete w;
+    return rc;
+  }
+  {
+    std::lock_guard<std::mutex> lk(g.mu);
+    g.live_weights++;
+  }
+  *out = w;
+  return HIPQ_OK;
+}
+
+int hipq_weight_destroy(hipq_weight_t w) {
+  if (!w) return HIPQ_OK;
+  int rc = require_ready();
+  if (rc) return rc;
+  (void)hipDeviceSynchronize();
+  (void)hipFree(w->base);
+  {
+    std::lock_guard<std::mutex> lk(g.mu);
+    g.live_weights--;
+    for (auto &kv : g.moe_tables) kv.second.key.clear(); /* tables may name w */
+  }
+  delete w;
+  return HIPQ_OK;
+}
+
+int hipq_weight_dims(hipq_weight_t w, int *dtype, int64_t *N, int64_t *K) {
+  if (!w) return fail(HIPQ_ERR_INVALID_ARGUMENT, "null weight");
+  if (dtype) *dtype = w->dtype;
+  if (N) *N = w->N;
+  if (K) *K = w->K;
+  return HIPQ_OK;
+}
+
+/* ---- activation quantizers (canonical output) ---------------------------- */
+
+static int quantize_api(int is_k, const float *A, int64_t M, int64_t K, int64_t lda, int variant,
+                        void *out, int mem, void *stream) {
+  int rc = require_ready();
+  if (rc) return rc;
+  if (!A || !out) return fail(HIPQ_ERR_INVALID_ARGUMENT, "null argument");
+  if (M < 0 || K <= 0 || K % (is_k ? 256 : 32) || lda < K)
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "M=%lld K=%lld lda=%lld", (long long)M, (long long)K, (long long)lda);
+  if (is_k && variant != HIPQ_Q8K_ROW && variant != HIPQ_Q8K_MAT)
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "unknown Q8_K variant %d", variant);
+  if (M == 0) return HIPQ_OK;
+  hipStream_t s = (hipStream_t)stream;
+  const size_t out_bytes = (size_t)M * (K / (is_k ? 256 : 32)) * (is_k ? 292 : 34);
+  const int64_t mat_rows = (is_k && variant == HIPQ_Q8K_MAT) ? M : 0;
+  if (mem == HIPQ_MEM_DEVICE) {
+    return is_k ? hipq::launch_quantize_q8_K(A, M, K, lda, mat_rows, nullptr, out, s)
+                : hipq::launch_quantize_q8_0(A, M, K, lda, nullptr, out, s);
+  }
+  if (mem != HIPQ_MEM_HOST) return fail(HIPQ_ERR_INVALID_ARGUMENT, "unknown mem kind %d", mem);
+  DevBuf dA, dOut;
+  if ((rc = dA.alloc((size_t)M * K * 4))) return rc;
+  if ((rc = dOut.alloc(out_bytes))) return rc;
+  HIPQ_HIP(hipMemcpy2D(dA.p, (size_t)K * 4, A, (size_t)lda * 4, (size_t)K * 4, (size_t)M,
+                       hipMemcpyHostToDevice));
+  rc = is_k ? hipq::launch_quantize_q8_K((const float *)dA.p, M, K, K, mat_rows, nullptr, dOut.p, s)
+            : hipq::launch_quantize_q8_0((const float *)dA.p, M, K, K, nullptr, dOut.p, s);
+  if (rc) return rc;
+  HIPQ_HIP(hipStreamSynchronize(s));
+  HIPQ_HIP(hipMemcpy(out, dOut.p, out_bytes, hipMemcpyDeviceToHost));
+  return HIPQ_OK;
+}
+
+int hipq_quantize_q8_0(const float *A, int64_t M, int64_t K, int64_t lda, void *out_blocks,
+                       int mem, void *stream) {
+  return quantize_api(0, A, M, K, lda, 0, out_blocks, mem, stream);
+}
+
+int hipq_quantize_q8_K(const float *A, int64_t M, int64_t K, int64_t lda, int variant,
+                       void *out_blocks, int mem, void *stream) {
+  return quantize_api(1, A, M, K, lda, variant, out_blocks, mem, stream);
+}
+
+/* ---- matmul --------------------------------------------------------------- */
+
+int hipq_matmul(hipq_weight_t w, const float *A, int64_t M, int64_t lda, float *C, int64_t ldc,
+                int mem, void *stream) {
+  int rc = require_ready();
+  if (rc) return rc;
+  if ((rc = check_matmul_args(w, A, M, lda, C, ldc))) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  if (mem == HIPQ_MEM_DEVICE) return matmul_device(w, A, M, lda, C, ldc, s);
+  if (mem != HIPQ_MEM_HOST) return fail(HIPQ_ERR_INVALID_ARGUMENT, "unknown mem kind %d", mem);
+  if (M == 0) return HIPQ_OK;
+  DevBuf dA, dC;
+  if ((rc = dA.alloc((size_t)M * w->K * 4))) return rc;
+  if ((rc = dC.alloc((size_t)M * w->N * 4))) return rc;
+  HIPQ_HIP(hipMemcpy2D(dA.p, (size_t)w->K * 4, A, (size_t)lda * 4, (size_t)w->K * 4, (size_t)M,
+                       hipMemcpyHostToDevice));
+  rc = matmul_device(w, (const float *)dA.p, M, w->K, (float *)dC.p, w->N, s);
+  if (rc) return rc;
+  HIPQ_HIP(hipStreamSynchronize(s));
+  HIPQ_HIP(hipMemcpy2D(C, (size_t)ldc * 4, dC.p, (size_t)w->N * 4, (size_t)w->N * 4, (size_t)M,
+                       hipMemcpyDeviceToHost));
+  return HIPQ_OK;
+}
+
+int hipq_matmul_multi(int count, const hipq_weight_t *w, const float *A, int64_t M, int64_t lda,
+                      float *const *C, const int64_t *ldc, int mem, void *stream) {
+  int rc = require_ready();
+  if (rc) return rc;
+  if (count <= 0 || !w || !C || !ldc) return fail(HIPQ_ERR_INVALID_ARGUMENT, "bad weight list");
+  for (int i = 0; i < count; ++i) {
+    if ((rc = check_matmul_args(w[i], A, M, lda, C[i], ldc[i]))) return rc;
+    if (w[i]->K != w[0]->K) return fail(HIPQ_ERR_INVALID_ARGUMENT, "weights disagree on K");
+  }
+  if (mem != HIPQ_MEM_DEVICE) {
+    for (int i = 0; i < count; ++i)
+      if ((rc = hipq_matmul(w[i], A, M, lda, C[i], ldc[i], mem, stream))) return rc;
+    return HIPQ_OK;
+  }
+  if (M == 0) return HIPQ_OK;
+  hipStream_t s = (hipStream_t)stream;
+  /* one quantization per distinct activation format among the weights */
+  auto klass = [&](const hipq_weight *x) {
+    if (x->dtype == HIPQ_Q4_0) return 0;
+    return (x->dtype == HIPQ_Q4_K && M > 1) ? 1 : 2;
+  };
+  for (int k = 0; k < 3; ++k) {
+    int first = -1;
+    for (int i = 0; i < count; ++i)
+      if (klass(w[i]) == k) {
+        first = i;
+        break;
+      }
+    if (first < 0) continue;
+    const int is_k = k != 0;
+    void *memp = nullptr;
+    if ((rc = workspace(s, qact_bytes(is_k, M, w[0]->K), &memp))) return rc;
+    QAct qa = qact_carve(is_k, memp, M, w[0]->K);
+    if ((rc = quantize_for(w[first], A, M, lda, qa, s))) return rc;
+    for (int i = 0; i < count; ++i)
+      if (klass(w[i]) == k)
+        if ((rc = multiply(w[i], qa, M, C[i], ldc[i], s))) return rc;
+  }
+  return HIPQ_OK;
+}
+
+int hipq_time_matmul(int n_weights, const hipq_weight_t *w, const float *A, int64_t M, int64_t lda,
+                     float *C, int64_t ldc, int iters, int phase, void *stream,
+                     float *ms_per_call) {
+  int rc = require_ready();
+  if (rc) return rc;
+  if (n_weights <= 0 || !w || iters <= 0 || !ms_per_call || phase < 0 || phase > 2)
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "bad timing arguments");
+  for (int i = 0; i < n_weights; ++i) {
+    if ((rc = check_matmul_args(w[i], A, M, lda, C, ldc))) return rc;
+    if (w[i]->K != w[0]->K || w[i]->dtype != w[0]->dtype)
+      return fail(HIPQ_ERR_INVALID_ARGUMENT, "timed weights must share dtype and K");
+  }
+  hipStream_t s = (hipStream_t)stream;
+  const int is_k = w[0]->dtype != HIPQ_Q4_0;
+  void *memp = nullptr;
+  if ((rc = workspace(s, qact_bytes(is_k, M, w[0]->K), &memp))) return rc;
+  QAct qa = qact_carve(is_k, memp, M, w[0]->K);
+  if ((rc = quantize_for(w[0], A, M, lda, qa, s))) return rc;
+  hipEvent_t e0, e1;
+  HIPQ_HIP(hipEventCreate(&e0));
+  HIPQ_HIP(hipEventCreate(&e1));
+  HIPQ_HIP(hipStreamSynchronize(s));
+  HIPQ_HIP(hipEventRecord(e0, s));
+  for (int it = 0; it < iters && !rc; ++it) {
+    const hipq_weight *wi = w[it % n_weights];
+    if (phase == 0 || phase == 2) rc = quantize_for(wi, A, M, lda, qa, s);
+    if (!rc && (phase == 0 || phase == 1)) rc = multiply(wi, qa, M, C, ldc, s);
+  }
+  hipError_t er = hipEventRecord(e1, s);
+  if (er == hipSuccess) er = hipEventSynchronize(e1);
+  float ms = 0.f;
+  if (er == hipSuccess) er = hipEventElapsedTime(&ms, e0, e1);
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  if (rc) return rc;
+  if (er != hipSuccess) return fail(HIPQ_ERR_RUNTIME, "timing: %s", hipGetErrorString(er));
+  *ms_per_call = ms / (float)iters;
+  return HIPQ_OK;
+}
+
+/* ---- mixture of experts ---------------------------------------------------- */
+
+int hipq_moe_forward(const hipq_moe_desc *desc, const hipq_weight_t *gate, const hipq_weight_t *up,
+                     const hipq_weight_t *down, const float *x, const float *router_logits,
+                     const float *router_weight, float *y, int32_t *topk_idx, float *topk_w,
+                     int mem, void *stream) {
+  int rc = require_ready();
+  if (rc) return rc;
+  if (!desc || !gate || !up || !down || !x || !y)
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "null argument");
+  const hipq_moe_desc d = *desc;
+  if (d.tokens < 0 || d.hidden <= 0 || d.intermediate <= 0 || d.experts <= 0 || d.topk <= 0 ||
+      d.topk > d.experts || d.topk > 32 || d.experts > 1024)
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "bad MoE shape T=%d H=%d I=%d E=%d k=%d", d.tokens,
+                d.hidden, d.intermediate, d.experts, d.topk);
+  if ((router_logits == nullptr) == (router_weight == nullptr))
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "pass exactly one of router_logits and router_weight");
+  const int dt = gate[0] ? gate[0]->dtype : -1;
+  for (int e = 0; e < d.experts; ++e) {
+    if (!gate[e] || !up[e] || !down[e]) return fail(HIPQ_ERR_INVALID_ARGUMENT, "null expert weight %d", e);
+    if (gate[e]->dtype != dt || up[e]->dtype != dt || down[e]->dtype != dt)
+      return fail(HIPQ_ERR_INVALID_ARGUMENT, "expert weights must share one dtype");
+    if (gate[e]->N != d.intermediate || gate[e]->K != d.hidden || up[e]->N != d.intermediate ||
+        up[e]->K != d.hidden || down[e]->N != d.hidden || down[e]->K != d.intermediate)
+      return fail(HIPQ_ERR_INVALID_ARGUMENT, "expert %d weight dims do not match the block", e);
+  }
+  if (d.tokens == 0) return HIPQ_OK;
+  hipStream_t s = (hipStream_t)stream;
+
+  /* device table of the 3E weight views, rebuilt only when the handles change */
+  WView *dev_views = nullptr;
+  {
+    std::lock_guard<std::mutex> lk(g.mu);
+    MoeTable &t = g.moe_tables[s];
+    std::vector<const hipq_weight *> key;
+    key.reserve(3 * (size_t)d.experts);
+    for (int e = 0; e < d.experts; ++e) key.push_back(gate[e]);
+    for (int e = 0; e < d.experts; ++e) key.push_back(up[e]);
+    for (int e = 0; e < d.experts; ++e) key.push_back(down[e]);
+    if (t.key != key || !t.dev) {
+      std::vector<WView> host(key.size());
+      for (size_t i = 0; i < key.size(); ++i) host[i] = wview(key[i]);
+      if (t.dev) {
+        HIPQ_HIP(hipStreamSynchronize(s));
+        HIPQ_HIP(hipFree(t.dev));
+        t.dev = nullptr;
+      }
+      HIPQ_HIP(hipMalloc((void **)&t.dev, host.size() * sizeof(WView)));
+      HIPQ_HIP(hipMemcpy(t.dev, host.data(), host.size() * sizeof(WView), hipMemcpyHostToDevice));
+      t.key = key;
+    }
+    dev_views = t.dev;
+  }
+
+  const size_t ws_bytes = hipq::moe_workspace_bytes(&d);
+  void *ws = nullptr;
+  if ((rc = workspace(s, ws_bytes, &ws))) return rc;
+
+  hipq::MoeArgs a;
+  a.desc = d;
+  a.gate = gate;
+  a.up = up;
+  a.down = down;
+  const size_t T = (size_t)d.tokens, H = (size_t)d.hidden, E = (size_t)d.experts, k = (size_t)d.topk;
+  if (mem == HIPQ_MEM_DEVICE) {
+    a.x = x;
+    a.router_logits = router_logits;
+    a.router_weight = router_weight;
+    a.y = y;
+    a.topk_idx = topk_idx;
+    a.topk_w = topk_w;
+    return hipq::launch_moe(&a, ws, ws_bytes, dev_views, s);
+  }
+  if (mem != HIPQ_MEM_HOST) return fail(HIPQ_ERR_INVALID_ARGUMENT, "unknown mem kind %d", mem);
+  DevBuf dx, dr, dy, di, dw;
+  if ((rc = dx.alloc(T * H * 4))) return rc;
+  if ((rc = dr.alloc((router_logits ? T * E : H * E) * 4))) return rc;
+  if ((rc = dy.alloc(T * H * 4))) return rc;
+  if ((rc = di.alloc(T * k * 4))) return rc;
+  if ((rc = dw.alloc(T * k * 4))) return rc;
+  HIPQ_HIP(hipMemcpy(dx.p, x, T * H * 4, hipMemcpyHostToDevice));
+  HIPQ_HIP(hipMemcpy(dr.p, router_logits ? router_logits : router_weight,
+                     (router_logits ? T * E : H * E) * 4, hipMemcpyHostToDevice));
+  a.x = (const float *)dx.p;
+  a.router_logits = router_logits ? (const float *)dr.p : nullptr;
+  a.router_weight = router_weight ? (const float *)dr.p : nullptr;
+  a.y = (float *)dy.p;
+  a.topk_idx = (int32_t *)di.p;
+  a.topk_w = (float *)dw.p;
+  if ((rc = hipq::launch_moe(&a, ws, ws_bytes, dev_views, s))) return rc;
+  HIPQ_HIP(hipStreamSynchronize(s));
+  HIPQ_HIP(hipMemcpy(y, dy.p, T * H * 4, hipMemcpyDeviceToHost));
+  if (topk_idx) HIPQ_HIP(hipMemcpy(topk_idx, di.p, T * k * 4, hipMemcpyDeviceToHost));
+  if (topk_w) HIPQ_HIP(hipMemcpy(topk_w, dw.p, T * k * 4, hipMemcpyDeviceToHost));
+  return HIPQ_OK;
+}
+
+/* ---- offline weight quantizers ---------------------------------------------- */
+
+int hipq_quantize_weights(int dtype, const float *W, int64_t N, int64_t K, void *out_blocks,
+                          int mem, void *stream) {
+  int rc = require_ready();
+  if (rc) return rc;
+  if (!W || !out_blocks) return fail(HIPQ_ERR_INVALID_ARGUMENT, "null argument");
+  const int64_t nbytes = hipq_weight_nbytes(dtype, N, K);
+  if (nbytes < 0) return (int)nbytes;
+  hipStream_t s = (hipStream_t)stream;
+  if (mem == HIPQ_MEM_DEVICE) return hipq::launch_quantize_weights(dtype, W, N, K, out_blocks, s);
+  if (mem != HIPQ_MEM_HOST) return fail(HIPQ_ERR_INVALID_ARGUMENT, "unknown mem kind %d", mem);
+  DevBuf dW, dOut;
+  if ((rc = dW.alloc((size_t)N * K * 4))) return rc;
+  if ((rc = dOut.alloc((size_t)nbytes))) return rc;
+  HIPQ_HIP(hipMemcpy(dW.p, W, (size_t)N * K * 4, hipMemcpyHostToDevice));
+  if ((rc = hipq::launch_quantize_weights(dtype, (const float *)dW.p, N, K, dOut.p, s))) return rc;
+  HIPQ_HIP(hipStreamSynchronize(s));
+  HIPQ_HIP(hipMemcpy(out_blocks, dOut.p, (size_t)nbytes, hipMemcpyDeviceToHost));
+  return HIPQ_OK;
+}
+
+} /* extern "C" */

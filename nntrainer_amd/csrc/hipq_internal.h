@@ -1,0 +1,218 @@
+// SPDX-License-Identifier: Apache-2.0
+/**
+ * @file   hipq_internal.h
+ * @brief  Shared declarations of the gfx950 quantized-matmul library: device
+ *         data layouts, launch entry points of each kernel family and the
+ *         device-side helpers (wave reductions over DPP, int8 dot, half
+ *         conversion) they have in common.
+ */
+#ifndef HIPQ_INTERNAL_H
+#define HIPQ_INTERNAL_H
+
+#include <hip/hip_fp16.h>
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "hipq.h"
+
+/* ------------------------------------------------------------------------- */
+/* Device-resident weight matrix (W^T, N rows of K quantized values).         */
+/*                                                                            */
+/* The ggml array-of-structs blocks are split once, at creation, into planes  */
+/* so that every lane of a wavefront can issue aligned 128-bit loads:         */
+/*   Q4_0: qs [N][K/2]  (16 B per 32-block, nibble order of block_q4_0)       */
+/*         d  [N][K/32] fp16                                                  */
+/*   Q4_K: qs [N][K/2]  (128 B per super-block, byte order of block_q4_K)     */
+/*         hdr[N][K/256][16] = {fp16 d, fp16 dmin, scales[12]}                */
+/*   Q6_K: qs [N][K/2]  (ql, 128 B per super-block, byte order of block_q6_K) */
+/*         qh [N][K/4]  (64 B per super-block, same byte order)               */
+/*         sc [N][K/16] int8, regrouped per super-block as [unit u][group g]  */
+/*                      = scales[(u>>1)*8 + g*2 + (u&1)]                      */
+/*         d  [N][K/256] fp16                                                 */
+/* The total size equals the packed ggml size; nothing is expanded in HBM.    */
+/* ------------------------------------------------------------------------- */
+struct hipq_weight {
+  int dtype;
+  int device;
+  int64_t N, K;
+  uint8_t *base;   /* one allocation holding all planes */
+  size_t bytes;
+  const uint8_t *qs;
+  const uint8_t *qh;
+  const uint8_t *hdr;
+  const int8_t *sc;
+  const uint16_t *d;
+};
+
+/* Plain-data view of a weight passed to kernels by value. */
+struct WView {
+  const uint8_t *qs;
+  const uint8_t *qh;
+  const uint8_t *hdr;
+  const int8_t *sc;
+  const uint16_t *d;
+  int N, K;
+};
+static inline WView wview(const hipq_weight *w) {
+  WView v;
+  v.qs = w->qs;
+  v.qh = w->qh;
+  v.hdr = w->hdr;
+  v.sc = w->sc;
+  v.d = w->d;
+  v.N = (int)w->N;
+  v.K = (int)w->K;
+  return v;
+}
+
+/* ------------------------------------------------------------------------- */
+/* Internal (device) form of quantized activations, structure of arrays.      */
+/*   Q8_0: q [M][K] int8; meta [M][K/32] = fp16 d bits | (int16 sum of the    */
+/*         block's 32 quants) << 16                                           */
+/*   Q8_K: q [M][K] int8; d [M][K/256] fp32; bsum [M][K/16] int16             */
+/* The quantizers can alternatively emit the canonical ggml blocks.           */
+/* ------------------------------------------------------------------------- */
+struct QAct {
+  int8_t *q;
+  uint32_t *meta; /* Q8_0 */
+  float *d;       /* Q8_K */
+  int16_t *bsum;  /* Q8_K */
+  int M, K;
+};
+size_t qact_bytes(int dtype_is_k, int64_t M, int64_t K);
+QAct qact_carve(int dtype_is_k, void *mem, int64_t M, int64_t K);
+
+namespace hipq {
+
+/* error plumbing (api.hip) */
+int fail(int code, const char *fmt, ...);
+#define HIPQ_HIP(call)                                                        \
+  do {                                                                        \
+    hipError_t e_ = (call);                                                   \
+    if (e_ != hipSuccess)                                                     \
+      return ::hipq::fail(HIPQ_ERR_RUNTIME, "%s failed: %s (%s:%d)", #call,   \
+                          hipGetErrorString(e_), __FILE__, __LINE__);         \
+  } while (0)
+
+/* quantize.hip ------------------------------------------------------------ */
+/* Rows [0, M) of A (row stride lda). `canonical_out` != nullptr writes ggml
+ * blocks there, otherwise the internal planes of `qa` are written.
+ * mat_rows: rows [0, mat_rows) use the 4-row ("MAT") Q8_K semantics, the rest
+ * the row semantics. */
+int launch_quantize_q8_0(const float *A, int64_t M, int64_t K, int64_t lda,
+                         const QAct *qa, void *canonical_out, hipStream_t s);
+int launch_quantize_q8_K(const float *A, int64_t M, int64_t K, int64_t lda,
+                         int64_t mat_rows, const QAct *qa, void *canonical_out,
+                         hipStream_t s);
+
+/* gemv.hip ---------------------------------------------------------------- */
+/* C[m][n] for m < M <= 8: one pass over the weights, M activation rows. */
+int launch_gemv(const hipq_weight *w, const QAct *qa, int M, float *C,
+                int64_t ldc, hipStream_t s);
+
+/* gemm.hip ---------------------------------------------------------------- */
+int launch_gemm(const hipq_weight *w, const QAct *qa, int M, float *C,
+                int64_t ldc, hipStream_t s);
+
+/* moe.hip ----------------------------------------------------------------- */
+struct MoeArgs {
+  hipq_moe_desc desc;
+  const hipq_weight *const *gate;
+  const hipq_weight *const *up;
+  const hipq_weight *const *down;
+  const float *x;             /* device */
+  const float *router_logits; /* device or null */
+  const float *router_weight; /* device or null */
+  float *y;                   /* device */
+  int32_t *topk_idx;          /* device or null */
+  float *topk_w;              /* device or null */
+};
+size_t moe_workspace_bytes(const hipq_moe_desc *d);
+int launch_moe(const MoeArgs *a, void *workspace, size_t workspace_bytes,
+               const WView *dev_views /* [3*E] gate|up|down, device */,
+               hipStream_t s);
+
+/* wquant.hip -------------------------------------------------------------- */
+int launch_quantize_weights(int dtype, const float *W, int64_t N, int64_t K,
+                            void *out_blocks, hipStream_t s);
+
+/* relayout.hip ------------------------------------------------------------ */
+int launch_relayout(hipq_weight *w, int layout, const uint8_t *src_dev,
+                    hipStream_t s);
+
+} // namespace hipq
+
+/* ------------------------------------------------------------------------- */
+/* device helpers                                                             */
+/* ------------------------------------------------------------------------- */
+#if defined(__HIPCC__)
+
+#define HIPQ_WAVE 64
+
+__device__ __forceinline__ float hipq_h2f(uint16_t bits) {
+  return __half2float(__ushort_as_half(bits));
+}
+__device__ __forceinline__ uint16_t hipq_f2h(float f) {
+  return __half_as_ushort(__float2half_rn(f));
+}
+
+/* signed 4 x int8 dot product with int32 accumulate (v_dot4_i32_i8) */
+__device__ __forceinline__ int hipq_dot4(int a, int b, int c) {
+  return __builtin_amdgcn_sdot4(a, b, c, false);
+}
+
+template <int CTRL> __device__ __forceinline__ int hipq_dpp_i(int v) {
+  return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xf, 0xf, true);
+}
+template <int CTRL> __device__ __forceinline__ float hipq_dpp_f(float v) {
+  return __builtin_bit_cast(float, hipq_dpp_i<CTRL>(__builtin_bit_cast(int, v)));
+}
+
+/* DPP controls: quad_perm [1,0,3,2], quad_perm [2,3,0,1], row_half_mirror,
+ * row_mirror. After the first four steps every lane of a 16-lane row holds the
+ * row's total; rows are then combined with two cross-row exchanges. All lanes
+ * of a group end with bit-identical values (each step adds the same two
+ * operands in both partners). */
+#define HIPQ_DPP_XOR1 0xB1
+#define HIPQ_DPP_XOR2 0x4E
+#define HIPQ_DPP_HALF_MIRROR 0x141
+#define HIPQ_DPP_MIRROR 0x140
+
+template <int T> __device__ __forceinline__ float hipq_group_sum(float v) {
+  if (T >= 2) v += hipq_dpp_f<HIPQ_DPP_XOR1>(v);
+  if (T >= 4) v += hipq_dpp_f<HIPQ_DPP_XOR2>(v);
+  if (T >= 8) v += hipq_dpp_f<HIPQ_DPP_HALF_MIRROR>(v);
+  if (T >= 16) v += hipq_dpp_f<HIPQ_DPP_MIRROR>(v);
+  if (T >= 32) v += __shfl_xor(v, 16, HIPQ_WAVE);
+  if (T >= 64) v += __shfl_xor(v, 32, HIPQ_WAVE);
+  return v;
+}
+template <int T> __device__ __forceinline__ int hipq_group_sum_i(int v) {
+  if (T >= 2) v += hipq_dpp_i<HIPQ_DPP_XOR1>(v);
+  if (T >= 4) v += hipq_dpp_i<HIPQ_DPP_XOR2>(v);
+  if (T >= 8) v += hipq_dpp_i<HIPQ_DPP_HALF_MIRROR>(v);
+  if (T >= 16) v += hipq_dpp_i<HIPQ_DPP_MIRROR>(v);
+  if (T >= 32) v += __shfl_xor(v, 16, HIPQ_WAVE);
+  if (T >= 64) v += __shfl_xor(v, 32, HIPQ_WAVE);
+  return v;
+}
+template <int T> __device__ __forceinline__ float hipq_group_max(float v) {
+  if (T >= 2) v = fmaxf(v, hipq_dpp_f<HIPQ_DPP_XOR1>(v));
+  if (T >= 4) v = fmaxf(v, hipq_dpp_f<HIPQ_DPP_XOR2>(v));
+  if (T >= 8) v = fmaxf(v, hipq_dpp_f<HIPQ_DPP_HALF_MIRROR>(v));
+  if (T >= 16) v = fmaxf(v, hipq_dpp_f<HIPQ_DPP_MIRROR>(v));
+  if (T >= 32) v = fmaxf(v, __shfl_xor(v, 16, HIPQ_WAVE));
+  if (T >= 64) v = fmaxf(v, __shfl_xor(v, 32, HIPQ_WAVE));
+  return v;
+}
+
+/* 128-bit streaming load of weight data: marked non-temporal so the one-pass
+ * weight stream does not evict the (re-used) quantized activations. */
+typedef unsigned int hipq_u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 hipq_ld_stream(const uint4 *p) {
+  hipq_u32x4 v = __builtin_nontemporal_load((const hipq_u32x4 *)p);
+  return make_uint4(v.x, v.y, v.z, v.w);
+}
+
+#endif /* __HIPCC__ */
+#endif /* HIPQ_INTERNAL_H */

@@ -1,0 +1,225 @@
+// SPDX-License-Identifier: Apache-2.0
+/**
+ * @file   quantize.hip
+ * @brief  Activation quantizers fp32 -> Q8_0 / Q8_K for gfx950.
+ *
+ * Bit-exact with the reference CPU quantizers in an x86 AVX2 GCC build
+ * (paths relative to the reference checkout, IMPL =
+ * nntrainer/tensor/cpu_backend/ggml_interface/nntr_ggml_impl):
+ *   Q8_0      IMPL/nntr_ggml_impl_quant.cpp:613-701 and the per-row content of
+ *             IMPL/nntr_ggml_impl.cpp:7879-7980
+ *   Q8_K ROW  IMPL/nntr_ggml_impl_quant.cpp:1334-1374, where the compiler fuses
+ *             iscale*x + 1.5*2^23 into a single rounding
+ *   Q8_K MAT  IMPL/nntr_ggml_impl.cpp:7504-7737 (product rounded to fp32, then
+ *             to the nearest-even integer; scale negative iff some x == +amax)
+ * Every floating-point step that decides a bit is an explicit round-to-nearest
+ * intrinsic (__fdiv_rn, __fmul_rn, __fmaf_rn, rintf), so the compiler can
+ * neither contract nor approximate it.
+ *
+ * Work mapping: Q8_0 uses 8 lanes per 32-value block (one 128-bit load per
+ * lane, 8 blocks per wavefront); Q8_K uses one wavefront per 256-value
+ * super-block (one 128-bit load per lane). Reductions run over DPP.
+ */
+#include "hipq_internal.h"
+
+namespace {
+
+constexpr float kRoundMagic = 12582912.f; /* 1.5 * 2^23 */
+
+__device__ __forceinline__ int magic_to_int(float biased) {
+  return (int)(__float_as_uint(biased) & 0x007fffffu) - 0x00400000;
+}
+
+__device__ __forceinline__ int pack4(int a, int b, int c, int d) {
+  return (a & 0xff) | ((b & 0xff) << 8) | ((c & 0xff) << 16) | ((d & 0xff) << 24);
+}
+
+/* ---- Q8_0 ---------------------------------------------------------------- */
+template <bool CANONICAL>
+__global__ __launch_bounds__(256) void quantize_q8_0_kernel(
+  const float *__restrict__ A, int64_t n_blocks_total, int nb, int64_t lda,
+  int8_t *__restrict__ q_out, uint32_t *__restrict__ meta_out,
+  uint8_t *__restrict__ canon_out) {
+  const int64_t gtid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  int64_t blk = gtid >> 3;
+  const int sub = (int)(gtid & 7);
+  const bool live = blk < n_blocks_total;
+  if (!live) blk = n_blocks_total - 1; /* keep the lane in the reductions */
+  const int64_t m = blk / nb;
+  const int b = (int)(blk - m * nb);
+  const float4 x = *(const float4 *)(A + m * lda + (int64_t)b * 32 + sub * 4);
+
+  float amax = fmaxf(fmaxf(fabsf(x.x), fabsf(x.y)), fmaxf(fabsf(x.z), fabsf(x.w)));
+  amax = hipq_group_max<8>(amax);
+
+  const float d = __fdiv_rn(amax, 127.f);
+  const float id = (amax != 0.0f) ? __fdiv_rn(127.f, amax) : 0.0f;
+  const int q0 = (int)rintf(__fmul_rn(x.x, id));
+  const int q1 = (int)rintf(__fmul_rn(x.y, id));
+  const int q2 = (int)rintf(__fmul_rn(x.z, id));
+  const int q3 = (int)rintf(__fmul_rn(x.w, id));
+  const int packed = pack4(q0, q1, q2, q3);
+  const uint16_t dh = hipq_f2h(d);
+
+  if (CANONICAL) {
+    if (!live) return;
+    uint8_t *o = canon_out + blk * 34;
+    if (sub == 0) *(uint16_t *)o = dh;
+    uint16_t *qs = (uint16_t *)(o + 2 + sub * 4);
+    qs[0] = (uint16_t)(packed & 0xffff);
+    qs[1] = (uint16_t)((unsigned)packed >> 16);
+  } else {
+    int bsum = hipq_group_sum_i<8>(q0 + q1 + q2 + q3);
+    if (!live) return;
+    *(int *)(q_out + (m * nb + b) * 32 + sub * 4) = packed;
+    if (sub == 0) meta_out[m * nb + b] = (uint32_t)dh | ((uint32_t)(bsum & 0xffff) << 16);
+  }
+}
+
+/* ---- Q8_K ---------------------------------------------------------------- */
+template <bool CANONICAL>
+__global__ __launch_bounds__(256) void quantize_q8_K_kernel(
+  const float *__restrict__ A, int64_t n_sb_total, int nsb, int64_t lda,
+  int64_t mat_rows, int8_t *__restrict__ q_out, float *__restrict__ d_out,
+  int16_t *__restrict__ bsum_out, uint8_t *__restrict__ canon_out) {
+  const int lane = threadIdx.x & 63;
+  int64_t sb = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  const bool live = sb < n_sb_total; /* uniform per wavefront */
+  if (!live) return;
+  const int64_t m = sb / nsb;
+  const int b = (int)(sb - m * nsb);
+  const float4 xv = *(const float4 *)(A + m * lda + (int64_t)b * 256 + lane * 4);
+  const float x[4] = {xv.x, xv.y, xv.z, xv.w};
+
+  float amax = fmaxf(fmaxf(fabsf(x[0]), fabsf(x[1])), fmaxf(fabsf(x[2]), fabsf(x[3])));
+  amax = hipq_group_max<64>(amax);
+
+  int q[4];
+  float d;
+  if (amax == 0.0f) {
+    q[0] = q[1] = q[2] = q[3] = 0;
+    d = 0.f;
+  } else if (m < mat_rows) {
+    /* 4-row quantizer semantics */
+    const bool hit = (x[0] == amax) | (x[1] == amax) | (x[2] == amax) | (x[3] == amax);
+    const bool pos_hit = __ballot(hit) != 0ull;
+    const float iscale = pos_hit ? __fdiv_rn(-127.f, amax) : __fdiv_rn(127.f, amax);
+    d = __fdiv_rn(1.f, iscale);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int v = (int)rintf(__fmul_rn(x[i], iscale));
+      q[i] = max(-128, min(127, v));
+    }
+  } else {
+    /* row quantizer semantics: sign of the FIRST element of maximal magnitude */
+    float cand = 0.f;
+    bool has = false;
+#pragma unroll
+    for (int i = 3; i >= 0; --i)
+      if (fabsf(x[i]) == amax) {
+        cand = x[i];
+        has = true;
+      }
+    const unsigned long long mask = __ballot(has);
+    const int first = __ffsll((long long)mask) - 1;
+    const float vmax = __shfl(cand, first, HIPQ_WAVE);
+    const float iscale = __fdiv_rn(-127.f, vmax);
+    d = __fdiv_rn(1.f, iscale);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      q[i] = min(127, magic_to_int(__fmaf_rn(iscale, x[i], kRoundMagic)));
+  }
+
+  const int packed = pack4(q[0], q[1], q[2], q[3]);
+  int gsum = q[0] + q[1] + q[2] + q[3];
+  gsum = hipq_group_sum_i<4>(gsum); /* 4 lanes = one 16-value group */
+
+  if (CANONICAL) {
+    uint8_t *o = canon_out + sb * 292;
+    if (lane == 0) *(float *)o = d;
+    *(int *)(o + 4 + lane * 4) = packed;
+    if ((lane & 3) == 0) *(int16_t *)(o + 260 + (lane >> 2) * 2) = (int16_t)gsum;
+  } else {
+    *(int *)(q_out + sb * 256 + lane * 4) = packed;
+    if (lane == 0) d_out[sb] = d;
+    if ((lane & 3) == 0) bsum_out[sb * 16 + (lane >> 2)] = (int16_t)gsum;
+  }
+}
+
+} // namespace
+
+namespace hipq {
+
+int launch_quantize_q8_0(const float *A, int64_t M, int64_t K, int64_t lda,
+                         const QAct *qa, void *canonical_out, hipStream_t s) {
+  if (M <= 0) return HIPQ_OK;
+  if (K % 32 || lda < K) return fail(HIPQ_ERR_INVALID_ARGUMENT, "Q8_0: K=%lld must be a multiple of 32 and lda >= K", (long long)K);
+  if (((uintptr_t)A & 15) || (lda & 3))
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "activation rows must be 16-byte aligned");
+  const int nb = (int)(K / 32);
+  const int64_t total = M * nb;
+  const int64_t threads = total * 8;
+  const unsigned grid = (unsigned)((threads + 255) / 256);
+  if (canonical_out)
+    hipLaunchKernelGGL(quantize_q8_0_kernel<true>, dim3(grid), dim3(256), 0, s, A, total, nb, lda,
+                       nullptr, nullptr, (uint8_t *)canonical_out);
+  else
+    hipLaunchKernelGGL(quantize_q8_0_kernel<false>, dim3(grid), dim3(256), 0, s, A, total, nb, lda,
+                       qa->q, qa->meta, nullptr);
+  HIPQ_HIP(hipGetLastError());
+  return HIPQ_OK;
+}
+
+int launch_quantize_q8_K(const float *A, int64_t M, int64_t K, int64_t lda,
+                         int64_t mat_rows, const QAct *qa, void *canonical_out,
+                         hipStream_t s) {
+  if (M <= 0) return HIPQ_OK;
+  if (K % 256 || lda < K) return fail(HIPQ_ERR_INVALID_ARGUMENT, "Q8_K: K=%lld must be a multiple of 256 and lda >= K", (long long)K);
+  if (((uintptr_t)A & 15) || (lda & 3))
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "activation rows must be 16-byte aligned");
+  const int nsb = (int)(K / 256);
+  const int64_t total = M * nsb;
+  const unsigned grid = (unsigned)((total + 3) / 4);
+  if (canonical_out)
+    hipLaunchKernelGGL(quantize_q8_K_kernel<true>, dim3(grid), dim3(256), 0, s, A, total, nsb, lda,
+                       mat_rows, nullptr, nullptr, nullptr, (uint8_t *)canonical_out);
+  else
+    hipLaunchKernelGGL(quantize_q8_K_kernel<false>, dim3(grid), dim3(256), 0, s, A, total, nsb, lda,
+                       mat_rows, qa->q, qa->d, qa->bsum, nullptr);
+  HIPQ_HIP(hipGetLastError());
+  return HIPQ_OK;
+}
+
+} // namespace hipq
+
+size_t qact_bytes(int is_k, int64_t M, int64_t K) {
+  /* q plane rounded to 256 B, then metadata planes */
+  size_t q = ((size_t)M * K + 255) & ~(size_t)255;
+  if (is_k) {
+    size_t d = ((size_t)M * (K / 256) * 4 + 255) & ~(size_t)255;
+    size_t bs = ((size_t)M * (K / 16) * 2 + 255) & ~(size_t)255;
+    return q + d + bs;
+  }
+  size_t meta = ((size_t)M * (K / 32) * 4 + 255) & ~(size_t)255;
+  return q + meta;
+}
+
+QAct qact_carve(int is_k, void *mem, int64_t M, int64_t K) {
+  QAct a;
+  uint8_t *p = (uint8_t *)mem;
+  a.M = (int)M;
+  a.K = (int)K;
+  a.q = (int8_t *)p;
+  p += ((size_t)M * K + 255) & ~(size_t)255;
+  a.meta = nullptr;
+  a.d = nullptr;
+  a.bsum = nullptr;
+  if (is_k) {
+    a.d = (float *)p;
+    p += ((size_t)M * (K / 256) * 4 + 255) & ~(size_t)255;
+    a.bsum = (int16_t *)p;
+  } else {
+    a.meta = (uint32_t *)p;
+  }
+  return a;
+}

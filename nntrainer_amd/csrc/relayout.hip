@@ -1,0 +1,129 @@
+// SPDX-License-Identifier: Apache-2.0
+/**
+ * @file   relayout.hip
+ * @brief  One-time conversion of ggml weight blocks (canonical rows, or the
+ *         8-row interleave NNTrainer stores on disk) into the plane layout the
+ *         gfx950 kernels read (see hipq_internal.h).
+ *
+ * Inverse of the reference's repack (nntr_make_block_q4_0x8 /
+ * make_block_q4_Kx8, nntrainer/tensor/cpu_backend/ggml_interface/
+ * nntr_ggml_impl/nntr_ggml_impl.cpp:8056-8158 in the reference checkout) fused
+ * with the array-of-structs -> planes split. Pure byte movement; runs once per
+ * weight at load time, one thread per source block.
+ */
+#include "hipq_internal.h"
+
+namespace {
+
+/* 6-bit scale/min j of a 12-byte packed group (get_scale_min_k4). */
+__device__ __forceinline__ void scale_min(int j, const uint8_t *s, int &sc, int &mn) {
+  if (j < 4) {
+    sc = s[j] & 63;
+    mn = s[j + 4] & 63;
+  } else {
+    sc = (s[j + 4] & 0x0f) | ((s[j - 4] >> 6) << 4);
+    mn = (s[j + 4] >> 4) | ((s[j] >> 6) << 4);
+  }
+}
+
+__global__ void relayout_q4_0(const uint8_t *__restrict__ src, int x8, int64_t N, int nb,
+                              uint8_t *__restrict__ qs, uint16_t *__restrict__ d) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= N * nb) return;
+  const int64_t n = i / nb;
+  const int b = (int)(i - n * nb);
+  uint8_t *oq = qs + i * 16;
+  if (!x8) {
+    const uint8_t *blk = src + i * 18;
+    d[i] = (uint16_t)(blk[0] | (blk[1] << 8));
+    for (int k = 0; k < 16; ++k) oq[k] = blk[2 + k];
+  } else {
+    const int r = (int)(n & 7);
+    const uint8_t *grp = src + ((n >> 3) * nb + b) * 144;
+    d[i] = (uint16_t)(grp[2 * r] | (grp[2 * r + 1] << 8));
+    for (int k = 0; k < 16; ++k)
+      oq[k] = grp[16 + (k >> 3) * 64 + r * 8 + (k & 7)] ^ 0x88;
+  }
+}
+
+__global__ void relayout_q4_K(const uint8_t *__restrict__ src, int x8, int64_t N, int nb,
+                              uint8_t *__restrict__ qs, uint8_t *__restrict__ hdr) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= N * nb) return;
+  const int64_t n = i / nb;
+  const int b = (int)(i - n * nb);
+  uint8_t *oq = qs + i * 128;
+  uint8_t *oh = hdr + i * 16;
+  if (!x8) {
+    const uint8_t *blk = src + i * 144;
+    for (int k = 0; k < 16; ++k) oh[k] = blk[k];
+    for (int k = 0; k < 128; ++k) oq[k] = blk[16 + k];
+  } else {
+    const int r = (int)(n & 7);
+    const uint8_t *grp = src + ((n >> 3) * nb + b) * 1152;
+    oh[0] = grp[2 * r];
+    oh[1] = grp[2 * r + 1];
+    oh[2] = grp[16 + 2 * r];
+    oh[3] = grp[16 + 2 * r + 1];
+    /* group g of the interleaved scales holds sub-block g of all 8 rows,
+     * indexed by row; rebuild this row's 12 bytes indexed by sub-block */
+    uint8_t s[12];
+    for (int k = 0; k < 12; ++k) s[k] = 0;
+    for (int g = 0; g < 8; ++g) {
+      int sc, mn;
+      scale_min(r, grp + 32 + 12 * g, sc, mn);
+      if (g < 4) {
+        s[g] |= (uint8_t)sc;
+        s[g + 4] |= (uint8_t)mn;
+      } else {
+        s[g + 4] = (uint8_t)((sc & 0x0f) | ((mn & 0x0f) << 4));
+        s[g - 4] |= (uint8_t)((sc >> 4) << 6);
+        s[g] |= (uint8_t)((mn >> 4) << 6);
+      }
+    }
+    for (int k = 0; k < 12; ++k) oh[4 + k] = s[k];
+    for (int k = 0; k < 128; ++k) oq[k] = grp[128 + (k >> 3) * 64 + r * 8 + (k & 7)];
+  }
+}
+
+__global__ void relayout_q6_K(const uint8_t *__restrict__ src, int64_t total,
+                              uint8_t *__restrict__ ql, uint8_t *__restrict__ qh,
+                              int8_t *__restrict__ sc, uint16_t *__restrict__ d) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= total) return;
+  const uint8_t *blk = src + i * 210;
+  for (int k = 0; k < 128; ++k) ql[i * 128 + k] = blk[k];
+  for (int k = 0; k < 64; ++k) qh[i * 64 + k] = blk[128 + k];
+  for (int u = 0; u < 4; ++u)
+    for (int g = 0; g < 4; ++g)
+      sc[i * 16 + u * 4 + g] = (int8_t)blk[192 + (u >> 1) * 8 + g * 2 + (u & 1)];
+  d[i] = (uint16_t)(blk[208] | (blk[209] << 8));
+}
+
+} // namespace
+
+namespace hipq {
+
+int launch_relayout(hipq_weight *w, int layout, const uint8_t *src, hipStream_t s) {
+  const int x8 = layout == HIPQ_LAYOUT_X8;
+  if (w->dtype == HIPQ_Q4_0) {
+    const int nb = (int)(w->K / 32);
+    const int64_t total = w->N * nb;
+    hipLaunchKernelGGL(relayout_q4_0, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, src,
+                       x8, w->N, nb, (uint8_t *)w->qs, (uint16_t *)w->d);
+  } else if (w->dtype == HIPQ_Q4_K) {
+    const int nb = (int)(w->K / 256);
+    const int64_t total = w->N * nb;
+    hipLaunchKernelGGL(relayout_q4_K, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, src,
+                       x8, w->N, nb, (uint8_t *)w->qs, (uint8_t *)w->hdr);
+  } else {
+    const int64_t total = w->N * (w->K / 256);
+    hipLaunchKernelGGL(relayout_q6_K, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, src,
+                       total, (uint8_t *)w->qs, (uint8_t *)w->qh, (int8_t *)w->sc,
+                       (uint16_t *)w->d);
+  }
+  HIPQ_HIP(hipGetLastError());
+  return HIPQ_OK;
+}
+
+} // namespace hipq

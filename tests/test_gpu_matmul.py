@@ -1,0 +1,129 @@
+"""GPU parity: fp32 outputs of the quantized matmul (decode GEMV and prefill GEMM)
+against the oracle on the same seeded inputs, through the C ABI.
+
+Bar: max|gpu - ref| / max|ref| <= 1e-4 per matrix (only the order of the fp32
+additions may differ; integer inner sums are exact on both sides)."""
+import numpy as np
+import pytest
+
+from nntrainer_amd import capi, synth
+
+pytestmark = pytest.mark.gpu
+
+KINDS = ["q4_0", "q4_K", "q6_K"]
+
+
+def _weights(cr, kind, n, k, seed):
+    w = synth.normal(seed, (n, k), 0.02)
+    return cr.quantize_weights(cr.oracle(), kind, w)
+
+
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("n,k", [(256, 256), (512, 1024), (1000, 768), (4096, 4096), (768, 2048)])
+def test_gemv_matches_oracle(hipq, cr, kind, n, k):
+    import gpu_util as gu
+    if kind != "q4_0" and k % 256:
+        pytest.skip("K must be a multiple of 256")
+    blocks = _weights(cr, kind, n, k, seed=100 + n)
+    a = synth.normal(200 + k, (1, k))
+    ref = cr.gemm(cr.oracle(), kind, a, blocks, n)
+    w = capi.Weight(kind, n, k, blocks)
+    got = gu.gpu_matmul(w, a)
+    w.destroy()
+    assert not np.isnan(got).any()
+    assert gu.rel_err(got, ref) <= gu.TOL, gu.rel_err(got, ref)
+
+
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("m", [2, 3, 4, 5, 7, 8])
+def test_small_m_matches_oracle(hipq, cr, kind, m):
+    """M = 2..8 runs the multi-row GEMV; rows below 4*(M/4) of a Q4_K matmul must be
+    quantized with the 4-row rule, the rest with the row rule."""
+    import gpu_util as gu
+    n, k = 512, 1024
+    blocks = _weights(cr, kind, n, k, seed=31)
+    a = synth.normal(300 + m, (m, k))
+    ref = cr.gemm(cr.oracle(), kind, a, blocks, n)
+    w = capi.Weight(kind, n, k, blocks)
+    got = gu.gpu_matmul(w, a)
+    w.destroy()
+    assert gu.rel_err(got, ref) <= gu.TOL, gu.rel_err(got, ref)
+
+
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("m,n,k", [(16, 256, 256), (64, 512, 1024), (130, 384, 512), (457, 512, 512),
+                                   (459, 512, 512), (512, 1024, 2048)])
+def test_gemm_matches_oracle(hipq, cr, kind, m, n, k):
+    """Prefill shapes, including M % 4 != 0 (the reference's leftover-row path,
+    unittest_nntrainer_cpu_backend.cpp:457-515 uses M = 457, 458, 459) and tiles that
+    do not divide M or N."""
+    import gpu_util as gu
+    blocks = _weights(cr, kind, n, k, seed=41 + m)
+    a = synth.normal(400 + m, (m, k))
+    ref = cr.gemm(cr.oracle(), kind, a, blocks, n)
+    w = capi.Weight(kind, n, k, blocks)
+    got = gu.gpu_matmul(w, a)
+    w.destroy()
+    assert not np.isnan(got).any()
+    assert gu.rel_err(got, ref) <= gu.TOL, gu.rel_err(got, ref)
+
+
+@pytest.mark.parametrize("kind", ["q4_0", "q4_K"])
+def test_x8_layout_equals_canonical(hipq, cr, kind):
+    """Weights handed over in NNTrainer's 8-row interleave give the same outputs."""
+    import gpu_util as gu
+    n, k = 512, 1024
+    blocks = _weights(cr, kind, n, k, seed=51)
+    x8 = cr.repack_x8(cr.oracle(), kind, blocks, n, k)
+    a = synth.normal(52, (5, k))
+    w0 = capi.Weight(kind, n, k, blocks)
+    w1 = capi.Weight(kind, n, k, x8, layout=capi.LAYOUT_X8)
+    c0, c1 = gu.gpu_matmul(w0, a), gu.gpu_matmul(w1, a)
+    w0.destroy(); w1.destroy()
+    assert np.array_equal(c0, c1)
+
+
+def test_host_memory_entry(hipq, cr):
+    """HIPQ_MEM_HOST: plain host pointers in and out, with row strides."""
+    import gpu_util as gu
+    n, k, m = 256, 512, 3
+    blocks = _weights(cr, "q4_K", n, k, seed=61)
+    a = np.zeros((m, k + 64), np.float32)
+    a[:, :k] = synth.normal(62, (m, k))
+    c = np.full((m, n + 16), np.nan, np.float32)
+    w = capi.Weight("q4_K", n, k, blocks)
+    capi.matmul(w, a, m, c, lda=k + 64, ldc=n + 16, mem=capi.MEM_HOST)
+    w.destroy()
+    ref = cr.gemm(cr.oracle(), "q4_K", a[:, :k], blocks, n)
+    assert gu.rel_err(c[:, :n], ref) <= gu.TOL
+    assert np.isnan(c[:, n:]).all()
+
+
+def test_matmul_multi_shares_quantization(hipq, cr):
+    import gpu_util as gu
+    import torch
+    k, m = 1024, 1
+    ns = [512, 256, 256]
+    blocks = [_weights(cr, "q4_0", n, k, seed=70 + i) for i, n in enumerate(ns)]
+    ws = [capi.Weight("q4_0", n, k, b) for n, b in zip(ns, blocks)]
+    a = synth.normal(73, (m, k))
+    da = gu.dev(a)
+    outs = [torch.empty((m, n), device="cuda") for n in ns]
+    capi.matmul_multi(ws, da, m, outs, stream=gu.stream())
+    torch.cuda.synchronize()
+    for n, b, o in zip(ns, blocks, outs):
+        assert gu.rel_err(o.cpu().numpy(), cr.gemm(cr.oracle(), "q4_0", a, b, n)) <= gu.TOL
+    for w in ws:
+        w.destroy()
+
+
+def test_bad_arguments_are_reported(hipq):
+    with pytest.raises(capi.HipqError) as e:
+        capi.weight_nbytes("q4_K", 16, 100)  # K not a multiple of 256 (q4_k_tensor.cpp:23-27)
+    assert e.value.code == -1
+    blocks = np.zeros(capi.weight_nbytes("q6_K", 8, 256), np.uint8)
+    with pytest.raises(capi.HipqError):
+        capi.Weight("q6_K", 8, 256, blocks, layout=capi.LAYOUT_X8)  # no x8 form of Q6_K
+    blocks = np.zeros(capi.weight_nbytes("q4_0", 12, 64), np.uint8)
+    with pytest.raises(capi.HipqError):
+        capi.Weight("q4_0", 12, 64, blocks, layout=capi.LAYOUT_X8)  # N % 8 != 0 (repack returns -1)
