@@ -125,12 +125,14 @@ int quantize_for(const hipq_weight *w, const float *A, int64_t M, int64_t lda, c
 int multiply(const hipq_weight *w, const QAct &qa, int64_t M, float *C, int64_t ldc,
              hipStream_t s) {
   const int is_k = w->dtype != HIPQ_Q4_0;
-  if (M <= 8) return hipq::launch_gemv(w, &qa, (int)M, C, ldc, s);
+  /* rows the reference sends through its 4-row GEMM kernel (Q4_K, M > 1) */
+  const int pair_rows = (w->dtype == HIPQ_Q4_K && M > 1) ? (int)((M / 4) * 4) : 0;
+  if (M <= 8) return hipq::launch_gemv(w, &qa, (int)M, pair_rows, C, ldc, s);
   if (w->dtype != HIPQ_Q6_K && w->K % 256 == 0) return hipq::launch_gemm(w, &qa, (int)M, C, ldc, s);
   for (int64_t r0 = 0; r0 < M; r0 += 8) {
     const int64_t rows = (M - r0) < 8 ? (M - r0) : 8;
     QAct sub = qact_rows(qa, is_k, r0, rows);
-    int rc = hipq::launch_gemv(w, &sub, (int)rows, C + r0 * ldc, ldc, s);
+    int rc = hipq::launch_gemv(w, &sub, (int)rows, 0, C + r0 * ldc, ldc, s);
     if (rc) return rc;
   }
   return HIPQ_OK;

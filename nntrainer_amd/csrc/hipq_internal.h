@@ -106,9 +106,10 @@ int launch_quantize_q8_K(const float *A, int64_t M, int64_t K, int64_t lda,
                          hipStream_t s);
 
 /* gemv.hip ---------------------------------------------------------------- */
-/* C[m][n] for m < M <= 8: one pass over the weights, M activation rows. */
-int launch_gemv(const hipq_weight *w, const QAct *qa, int M, float *C,
-                int64_t ldc, hipStream_t s);
+/* C[m][n] for m < M <= 8: one pass over the weights, M activation rows.
+ * Rows below pair_rows use the reference GEMM kernel's fp32 order (Q4_K). */
+int launch_gemv(const hipq_weight *w, const QAct *qa, int M, int pair_rows,
+                float *C, int64_t ldc, hipStream_t s);
 
 /* gemm.hip ---------------------------------------------------------------- */
 int launch_gemm(const hipq_weight *w, const QAct *qa, int M, float *C,
@@ -152,8 +153,11 @@ int launch_relayout(hipq_weight *w, int layout, const uint8_t *src_dev,
 __device__ __forceinline__ float hipq_h2f(uint16_t bits) {
   return __half2float(__ushort_as_half(bits));
 }
+/* fp32 -> fp16, round to nearest even (F16C _cvtss_sh semantics). The sign is
+ * copied from the fp32 bits: the compiler's conversion turns -0.0f into +0. */
 __device__ __forceinline__ uint16_t hipq_f2h(float f) {
-  return __half_as_ushort(__float2half_rn(f));
+  const uint16_t h = __half_as_ushort(__float2half_rn(f));
+  return (uint16_t)((h & 0x7fffu) | ((__float_as_uint(f) >> 16) & 0x8000u));
 }
 
 /* signed 4 x int8 dot product with int32 accumulate (v_dot4_i32_i8) */

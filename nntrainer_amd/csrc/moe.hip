@@ -24,7 +24,8 @@
  * scatter (pairs sorted by expert) -> quantize x -> grouped gate+up GEMV with
  * fused SwiGLU over (column tiles x experts) -> quantize h -> grouped down GEMV
  * scaled by the routing weight -> combine. Within an expert the weight rows are
- * streamed once per group of four tokens.
+ * streamed once per group of four tokens. Each single-row product is computed by
+ * the same engine as the decode GEMV, so it carries the reference's bits.
  */
 #include "gemv_device.h"
 
@@ -214,15 +215,15 @@ __global__ __launch_bounds__(256) void gate_up_kernel(const WView *__restrict__ 
                                                       QView xq, const int *__restrict__ offsets,
                                                       const int *__restrict__ slot_pair, int topk,
                                                       int I, float *__restrict__ h) {
-  constexpr int ROWS_PER_WAVE = 64 / T;
+  constexpr int G = GemvGroup<DT, RTOK>::G;
+  extern __shared__ uint32_t moe_lds[];
   const int e = blockIdx.y;
   const int begin = offsets[e], end = offsets[e + 1];
   if (begin == end) return;
   const WView wg = views[e], wu = views[E + e];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, tl = lane % T;
-  int col = (blockIdx.x * 4 + wave) * ROWS_PER_WAVE + lane / T;
-  const bool live = col < I;
-  if (!live) col = I - 1;
+  const int wave = threadIdx.x >> 6;
+  uint32_t *lds = moe_lds + wave * GemvGroup<DT, RTOK>::LDS_DWORDS;
+  const int col0 = (blockIdx.x * 4 + wave) * G;
   for (int s0 = begin; s0 < end; s0 += RTOK) {
     int arow[RTOK];
 #pragma unroll
@@ -230,14 +231,10 @@ __global__ __launch_bounds__(256) void gate_up_kernel(const WView *__restrict__ 
       const int slot = min(s0 + r, end - 1);
       arow[r] = slot_pair[slot] / topk; /* token of the pair */
     }
-    float g[RTOK], u[RTOK];
-    gemv_rows<DT, T, RTOK>(wg, col, tl, xq, arow, g);
-    gemv_rows<DT, T, RTOK>(wu, col, tl, xq, arow, u);
-    if (live && tl == 0) {
-#pragma unroll
-      for (int r = 0; r < RTOK; ++r)
-        if (s0 + r < end) h[(size_t)(s0 + r) * I + col] = silu_ref(g[r]) * u[r];
-    }
+    const GemvOut g = gemv_engine<DT, T, RTOK, G>(wg, col0, xq, arow, 0, lds);
+    const GemvOut u = gemv_engine<DT, T, RTOK, G>(wu, col0, xq, arow, 0, lds);
+    if (g.valid && col0 + g.g < I && s0 + g.r < end)
+      h[(size_t)(s0 + g.r) * I + col0 + g.g] = silu_ref(g.v) * u.v;
   }
 }
 
@@ -248,27 +245,22 @@ __global__ __launch_bounds__(256) void down_kernel(const WView *__restrict__ vie
                                                    const int *__restrict__ slot_pair,
                                                    const float *__restrict__ wgt, int H,
                                                    float *__restrict__ contrib) {
-  constexpr int ROWS_PER_WAVE = 64 / T;
+  constexpr int G = GemvGroup<DT, RTOK>::G;
+  extern __shared__ uint32_t moe_lds[];
   const int e = blockIdx.y;
   const int begin = offsets[e], end = offsets[e + 1];
   if (begin == end) return;
   const WView wd = views[2 * E + e];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, tl = lane % T;
-  int col = (blockIdx.x * 4 + wave) * ROWS_PER_WAVE + lane / T;
-  const bool live = col < H;
-  if (!live) col = H - 1;
+  const int wave = threadIdx.x >> 6;
+  uint32_t *lds = moe_lds + wave * GemvGroup<DT, RTOK>::LDS_DWORDS;
+  const int col0 = (blockIdx.x * 4 + wave) * G;
   for (int s0 = begin; s0 < end; s0 += RTOK) {
     int arow[RTOK];
 #pragma unroll
     for (int r = 0; r < RTOK; ++r) arow[r] = min(s0 + r, end - 1); /* hq rows are slots */
-    float o[RTOK];
-    gemv_rows<DT, T, RTOK>(wd, col, tl, hq, arow, o);
-    if (live && tl == 0) {
-#pragma unroll
-      for (int r = 0; r < RTOK; ++r)
-        if (s0 + r < end)
-          contrib[(size_t)(s0 + r) * H + col] = o[r] * wgt[slot_pair[s0 + r]];
-    }
+    const GemvOut o = gemv_engine<DT, T, RTOK, G>(wd, col0, hq, arow, 0, lds);
+    if (o.valid && col0 + o.g < H && s0 + o.r < end)
+      contrib[(size_t)(s0 + o.r) * H + col0 + o.g] = o.v * wgt[slot_pair[s0 + o.r]];
   }
 }
 
@@ -304,18 +296,21 @@ template <int DT>
 int launch_grouped(const hipq::MoeArgs *a, const MoeBufs &b, const WView *views, const QAct &xq,
                    const QAct &hq, hipStream_t s) {
   const hipq_moe_desc &d = a->desc;
+  constexpr int G = GemvGroup<DT, RTOK>::G;
+  constexpr int TS = GemvGroup<DT, RTOK>::T16_OK ? 16 : 64; /* lanes per row for short K */
+  const size_t lds = 4 * GemvGroup<DT, RTOK>::LDS_DWORDS * sizeof(uint32_t);
   const int64_t units_gu = (DT == HIPQ_Q6_K) ? d.hidden / 64 : d.hidden / 32;
   const int64_t units_dn = (DT == HIPQ_Q6_K) ? d.intermediate / 64 : d.intermediate / 32;
   const int64_t P = (int64_t)d.tokens * d.topk;
   int rc;
-  if (units_gu >= 64) {
-    const dim3 grid((d.intermediate + 3) / 4, d.experts);
-    hipLaunchKernelGGL((gate_up_kernel<DT, 64>), grid, dim3(256), 0, s, views, d.experts, qview(xq),
-                       b.offsets, b.slot_pair, d.topk, d.intermediate, b.h);
-  } else {
-    const dim3 grid((d.intermediate + 15) / 16, d.experts);
-    hipLaunchKernelGGL((gate_up_kernel<DT, 16>), grid, dim3(256), 0, s, views, d.experts, qview(xq),
-                       b.offsets, b.slot_pair, d.topk, d.intermediate, b.h);
+  {
+    const dim3 grid((d.intermediate + 4 * G - 1) / (4 * G), d.experts);
+    if (units_gu >= 64)
+      hipLaunchKernelGGL((gate_up_kernel<DT, 64>), grid, dim3(256), lds, s, views, d.experts,
+                         qview(xq), b.offsets, b.slot_pair, d.topk, d.intermediate, b.h);
+    else
+      hipLaunchKernelGGL((gate_up_kernel<DT, TS>), grid, dim3(256), lds, s, views, d.experts,
+                         qview(xq), b.offsets, b.slot_pair, d.topk, d.intermediate, b.h);
   }
   HIPQ_HIP(hipGetLastError());
   if (DT == HIPQ_Q4_0)
@@ -323,14 +318,14 @@ int launch_grouped(const hipq::MoeArgs *a, const MoeBufs &b, const WView *views,
   else
     rc = hipq::launch_quantize_q8_K(b.h, P, d.intermediate, d.intermediate, 0, &hq, nullptr, s);
   if (rc) return rc;
-  if (units_dn >= 64) {
-    const dim3 grid((d.hidden + 3) / 4, d.experts);
-    hipLaunchKernelGGL((down_kernel<DT, 64>), grid, dim3(256), 0, s, views, d.experts, qview(hq),
-                       b.offsets, b.slot_pair, b.wgt, d.hidden, b.contrib);
-  } else {
-    const dim3 grid((d.hidden + 15) / 16, d.experts);
-    hipLaunchKernelGGL((down_kernel<DT, 16>), grid, dim3(256), 0, s, views, d.experts, qview(hq),
-                       b.offsets, b.slot_pair, b.wgt, d.hidden, b.contrib);
+  {
+    const dim3 grid((d.hidden + 4 * G - 1) / (4 * G), d.experts);
+    if (units_dn >= 64)
+      hipLaunchKernelGGL((down_kernel<DT, 64>), grid, dim3(256), lds, s, views, d.experts,
+                         qview(hq), b.offsets, b.slot_pair, b.wgt, d.hidden, b.contrib);
+    else
+      hipLaunchKernelGGL((down_kernel<DT, TS>), grid, dim3(256), lds, s, views, d.experts,
+                         qview(hq), b.offsets, b.slot_pair, b.wgt, d.hidden, b.contrib);
   }
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;

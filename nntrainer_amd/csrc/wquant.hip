@@ -42,7 +42,8 @@ __global__ void quantize_w_q4_0(const float *__restrict__ src, int64_t nblk,
       vmax = x[j];
     }
   }
-  const float d = __fdiv_rn(vmax, -8.f);
+  /* max / -8 as an exact scaling plus a sign flip (keeps -0 for an all-zero block) */
+  const float d = -(vmax * 0.125f);
   const float id = d != 0.f ? __fdiv_rn(1.0f, d) : 0.0f;
   const uint16_t hd = hipq_f2h(d);
   y[0] = (uint8_t)(hd & 0xff);
@@ -144,7 +145,8 @@ __global__ __launch_bounds__(64) void quantize_w_q4_K(const float *__restrict__ 
     const float *xs = x + 32 * j;
     float sum_x2 = 0;
     for (int l = 0; l < 32; ++l) sum_x2 = __fmaf_rn(xs[l], xs[l], sum_x2);
-    const float av_x = __fsqrt_rn(__fdiv_rn(sum_x2, 32.f));
+    /* sqrtf: correctly rounded (the __fsqrt_rn intrinsic maps to the native approximation) */
+    const float av_x = sqrtf(__fdiv_rn(sum_x2, 32.f));
     for (int l = 0; l < 32; ++l) w[l] = __fadd_rn(av_x, fabsf(xs[l]));
     scales[j] = q4k_fit(xs, w, L + 32 * j, &mins[j]);
     if (scales[j] > max_scale) max_scale = scales[j];

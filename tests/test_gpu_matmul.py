@@ -19,7 +19,8 @@ def _weights(cr, kind, n, k, seed):
 
 
 @pytest.mark.parametrize("kind", KINDS)
-@pytest.mark.parametrize("n,k", [(256, 256), (512, 1024), (1000, 768), (4096, 4096), (768, 2048)])
+@pytest.mark.parametrize("n,k", [(256, 256), (512, 1024), (1000, 768), (4096, 4096), (768, 2048),
+                                 (130, 8192), (64, 12288)])
 def test_gemv_matches_oracle(hipq, cr, kind, n, k):
     import gpu_util as gu
     if kind != "q4_0" and k % 256:
@@ -32,6 +33,9 @@ def test_gemv_matches_oracle(hipq, cr, kind, n, k):
     w.destroy()
     assert not np.isnan(got).any()
     assert gu.rel_err(got, ref) <= gu.TOL, gu.rel_err(got, ref)
+    # the decode path reproduces the reference's fp32 evaluation order: same bits
+    assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), \
+        "%d of %d outputs differ in bits" % ((got.view(np.uint32) != ref.view(np.uint32)).sum(), got.size)
 
 
 @pytest.mark.parametrize("kind", KINDS)
@@ -48,6 +52,7 @@ def test_small_m_matches_oracle(hipq, cr, kind, m):
     got = gu.gpu_matmul(w, a)
     w.destroy()
     assert gu.rel_err(got, ref) <= gu.TOL, gu.rel_err(got, ref)
+    assert np.array_equal(got.view(np.uint32), ref.view(np.uint32))
 
 
 @pytest.mark.parametrize("kind", KINDS)

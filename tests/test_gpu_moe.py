@@ -39,7 +39,9 @@ def test_moe_matches_oracle(hipq, cr, t, h, i, e, k):
     assert np.abs(wt.cpu().numpy() - ref_w).max() <= 1e-6
     got = y.cpu().numpy()
     assert not np.isnan(got).any()
-    assert gu.rel_err(got, ref_y) <= gu.TOL, gu.rel_err(got, ref_y)
+    # every single-row product carries the reference's bits; only the softmax
+    # row sum (order unspecified in the reference, BLAS) may move the last bits
+    assert gu.rel_err(got, ref_y) <= 2e-6, gu.rel_err(got, ref_y)
     # second call on the same handles (cached expert table) gives the same bits
     y2 = torch.empty_like(y)
     capi.moe_forward(t, h, i, e, k, wg, wu, wd, dx, y2, router_logits=dl, stream=gu.stream())
