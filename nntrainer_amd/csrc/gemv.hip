@@ -11,59 +11,83 @@
  * they call; outputs are bit-identical to those kernels (see gemv_device.h).
  *
  * Launch shape: 256 threads = 4 wavefronts per workgroup, each wavefront owns G
- * consecutive output columns (G = 8 for one activation row), so a matrix with N
- * columns launches N / 32 workgroups: 384 for N = 12288, 4748 for the 151936-row
- * lm_head. The kernel is bound by HBM: per output column it reads the column's
- * packed weights exactly once, 16 bytes per lane per load.
+ * consecutive output columns; G = 4 from N = 8192 up (9497 workgroups for the
+ * 151936-row lm_head, 768 for N = 12288), 2 or 1 for smaller matrices so that
+ * they still fill the 1024 SIMDs. The kernel is bound by
+ * HBM: per output column it reads the column's packed weights exactly once,
+ * 16 bytes per lane per load, all loads of a group in flight together.
  */
+#include <cstdlib>
+
 #include "gemv_device.h"
 
 namespace {
 
-template <int DT, int T, int R>
+template <int DT, int T, int R, int G, bool PW>
 __global__ __launch_bounds__(256) void gemv_kernel(WView w, QView qa, int M, int pair_rows,
                                                    float *__restrict__ C, int64_t ldc) {
-  constexpr int G = GemvGroup<DT, R>::G;
   extern __shared__ uint32_t gemv_lds[];
   const int wave = threadIdx.x >> 6;
-  uint32_t *lds = gemv_lds + wave * GemvGroup<DT, R>::LDS_DWORDS;
+  uint32_t *lds = gemv_lds + wave * GemvLds<DT, R, G, PW>::DWORDS;
   const int row0 = (blockIdx.x * 4 + wave) * G;
   int arow[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) arow[r] = r < M ? r : M - 1;
-  const GemvOut o = gemv_engine<DT, T, R, G>(w, row0, qa, arow, pair_rows, lds);
+  const GemvOut o = gemv_engine<DT, T, R, G, PW>(w, row0, qa, arow, pair_rows, lds);
   if (o.valid && row0 + o.g < w.N && o.r < M) C[(int64_t)o.r * ldc + row0 + o.g] = o.v;
 }
 
-template <int DT, int T, int R>
+template <int DT, int T, int R, int G, bool PW>
 int launch_one(const hipq_weight *w, const QAct *qa, int M, int pair_rows, float *C, int64_t ldc,
                hipStream_t s) {
-  constexpr int G = GemvGroup<DT, R>::G;
   const unsigned grid = (unsigned)((w->N + 4 * G - 1) / (4 * G));
-  const size_t lds = 4 * GemvGroup<DT, R>::LDS_DWORDS * sizeof(uint32_t);
-  hipLaunchKernelGGL((gemv_kernel<DT, T, R>), dim3(grid), dim3(256), lds, s, wview(w), qview(*qa), M,
-                     pair_rows, C, ldc);
+  const size_t lds = 4 * GemvLds<DT, R, G, PW>::DWORDS * sizeof(uint32_t);
+  hipLaunchKernelGGL((gemv_kernel<DT, T, R, G, PW>), dim3(grid), dim3(256), lds, s, wview(w),
+                     qview(*qa), M, pair_rows, C, ldc);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
 }
 
-template <int DT, int R>
-int launch_t(const hipq_weight *w, const QAct *qa, int M, int pair_rows, float *C, int64_t ldc,
-             hipStream_t s) {
-  /* units of work per row: 32-weight units for Q4_0 / Q4_K, 64-weight for Q6_K */
-  const int64_t units = (DT == HIPQ_Q6_K) ? w->K / 64 : w->K / 32;
-  if (GemvGroup<DT, R>::T16_OK && units < 64)
-    return launch_one<DT, (GemvGroup<DT, R>::T16_OK ? 16 : 64), R>(w, qa, M, pair_rows, C, ldc, s);
-  return launch_one<DT, 64, R>(w, qa, M, pair_rows, C, ldc, s);
+/* Largest group size not above gmax that still gives ~6000 wavefronts. */
+int pick_group(int64_t N, int gmax) {
+  if (const char *e = getenv("HIPQ_GEMV_G")) return atoi(e);
+  /* measured: 4 rows per wavefront is best from N = 8192 up to the 151936-row
+   * lm_head; smaller matrices want more, shorter wavefronts */
+  int g = N >= 8192 ? 4 : (N >= 2048 ? 2 : 1);
+  return g < gmax ? g : gmax;
 }
 
+/* One activation row: the decode shape, tuned for parallelism. */
 template <int DT>
-int launch_r(const hipq_weight *w, const QAct *qa, int M, int pair_rows, float *C, int64_t ldc,
-             hipStream_t s) {
-  if (M == 1) return launch_t<DT, 1>(w, qa, M, pair_rows, C, ldc, s);
-  if (M == 2) return launch_t<DT, 2>(w, qa, M, pair_rows, C, ldc, s);
-  if (M <= 4) return launch_t<DT, 4>(w, qa, M, pair_rows, C, ldc, s);
-  return launch_t<DT, 8>(w, qa, M, pair_rows, C, ldc, s);
+int launch_m1(const hipq_weight *w, const QAct *qa, float *C, int64_t ldc, hipStream_t s) {
+  const int64_t units = w->K / GemvRec<DT, false>::UNIT;
+  if (units < 64) { /* short rows: 16 lanes per row, 4 rows streamed at once */
+    if (pick_group(w->N, 8) == 8) return launch_one<DT, 16, 1, 8, false>(w, qa, 1, 0, C, ldc, s);
+    return launch_one<DT, 16, 1, 4, false>(w, qa, 1, 0, C, ldc, s);
+  }
+  switch (pick_group(w->N, 8)) {
+  case 8:
+    return launch_one<DT, 64, 1, 8, false>(w, qa, 1, 0, C, ldc, s);
+  case 4:
+    return launch_one<DT, 64, 1, 4, false>(w, qa, 1, 0, C, ldc, s);
+  case 2:
+    return launch_one<DT, 64, 1, 2, false>(w, qa, 1, 0, C, ldc, s);
+  default:
+    /* Q4_0's fp32 chain has one step per 32 weights: keep two rows per pass */
+    if (DT == HIPQ_Q4_0) return launch_one<DT, 64, 1, 2, false>(w, qa, 1, 0, C, ldc, s);
+    return launch_one<DT, 64, 1, 1, false>(w, qa, 1, 0, C, ldc, s);
+  }
+}
+
+/* 2..8 activation rows in one pass (small prefill chunks, leftover rows). */
+template <int DT>
+int launch_mr(const hipq_weight *w, const QAct *qa, int M, int pair_rows, float *C, int64_t ldc,
+              hipStream_t s) {
+  constexpr bool K4 = DT == HIPQ_Q4_K;
+  if (M == 2) return launch_one<DT, 64, 2, (K4 ? 4 : 2), false>(w, qa, M, 0, C, ldc, s);
+  if (M == 3) return launch_one<DT, 64, 4, 2, false>(w, qa, M, 0, C, ldc, s);
+  if (M == 4) return launch_one<DT, 64, 4, 2, K4>(w, qa, M, pair_rows, C, ldc, s);
+  return launch_one<DT, 64, 8, 1, K4>(w, qa, M, pair_rows, C, ldc, s);
 }
 
 } // namespace
@@ -75,11 +99,14 @@ int launch_gemv(const hipq_weight *w, const QAct *qa, int M, int pair_rows, floa
   if (M < 1 || M > 8) return fail(HIPQ_ERR_INVALID_ARGUMENT, "gemv handles 1..8 rows, got %d", M);
   switch (w->dtype) {
   case HIPQ_Q4_0:
-    return launch_r<HIPQ_Q4_0>(w, qa, M, pair_rows, C, ldc, s);
+    return M == 1 ? launch_m1<HIPQ_Q4_0>(w, qa, C, ldc, s)
+                  : launch_mr<HIPQ_Q4_0>(w, qa, M, pair_rows, C, ldc, s);
   case HIPQ_Q4_K:
-    return launch_r<HIPQ_Q4_K>(w, qa, M, pair_rows, C, ldc, s);
+    return M == 1 ? launch_m1<HIPQ_Q4_K>(w, qa, C, ldc, s)
+                  : launch_mr<HIPQ_Q4_K>(w, qa, M, pair_rows, C, ldc, s);
   case HIPQ_Q6_K:
-    return launch_r<HIPQ_Q6_K>(w, qa, M, pair_rows, C, ldc, s);
+    return M == 1 ? launch_m1<HIPQ_Q6_K>(w, qa, C, ldc, s)
+                  : launch_mr<HIPQ_Q6_K>(w, qa, M, pair_rows, C, ldc, s);
   }
   return fail(HIPQ_ERR_INVALID_ARGUMENT, "unknown weight dtype %d", w->dtype);
 }

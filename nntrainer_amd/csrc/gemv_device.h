@@ -23,12 +23,15 @@
  *   phase 1  T lanes (16 or 64) stream one weight row with 128-bit non-temporal
  *            loads, unpack nibbles in registers and form exact integer partial
  *            sums with v_dot4_i32_i8 against R rows of quantized activations;
- *            partials of a block / sub-block pair are combined over DPP
- *            (integers, exact) and written to LDS as per-block records;
+ *            partials of a block / sub-block pair / super-block are combined
+ *            over DPP (integers, exact) and written to LDS as per-block records.
+ *            The activations a lane needs are the same for every weight row, so
+ *            they are loaded into registers once per chunk; the weight loads of
+ *            all rows of the group are issued before the first is consumed.
  *   phase 2  one lane per (weight row, activation row) [x 8 for Q6_K] walks the
  *            records of its output in ascending K order and performs the fp32
  *            chain above. G weight rows share one pass so that the sequential
- *            chains run on many lanes at once.
+ *            chains run on several lanes at once.
  */
 #ifndef HIPQ_GEMV_DEVICE_H
 #define HIPQ_GEMV_DEVICE_H
@@ -64,179 +67,336 @@ __device__ __forceinline__ int hipq_dot16(const uint32_t (&w)[4], const int4 &a)
   return s;
 }
 
-/* Dwords of LDS per (weight row, activation row) and K-chunk. The odd-ish
- * strides keep the phase-2 lanes, which read the same record index of
- * different outputs, on different banks. */
-template <int DT> struct GemvRec;
-template <> struct GemvRec<HIPQ_Q4_0> {
+/* ---- per-format traits --------------------------------------------------------- */
+/* UNIT: weights covered by one lane-unit. PER_CHUNK: dwords of LDS per (weight
+ * row, activation row) and K-chunk; the strides keep the phase-2 lanes, which
+ * read the same record index of different outputs, on different banks.
+ * PW = records per sub-block pair (needed when some rows use the pairwise order). */
+template <int DT, bool PW> struct GemvRec;
+template <bool PW> struct GemvRec<HIPQ_Q4_0, PW> {
+  static constexpr int UNIT = 32;
   static constexpr int PER_CHUNK = (HIPQ_KCHUNK / 32) * 2 + 2; /* {float isum, float scale} per block */
   static constexpr int LANES_PER_OUT = 1;
 };
-template <> struct GemvRec<HIPQ_Q4_K> {
+template <> struct GemvRec<HIPQ_Q4_K, false> {
+  static constexpr int UNIT = 64;
+  static constexpr int PER_CHUNK = (HIPQ_KCHUNK / 256) * 4 + 4; /* {fI, sd, fIm, sm} per super-block */
+  static constexpr int LANES_PER_OUT = 1;
+};
+template <> struct GemvRec<HIPQ_Q4_K, true> {
+  static constexpr int UNIT = 64;
   static constexpr int PER_CHUNK = (HIPQ_KCHUNK / 256) * 10 + 2; /* {I[4], Im[4], sd, sm} per super-block */
   static constexpr int LANES_PER_OUT = 1;
 };
-template <> struct GemvRec<HIPQ_Q6_K> {
+template <bool PW> struct GemvRec<HIPQ_Q6_K, PW> {
+  static constexpr int UNIT = 64;
   static constexpr int PER_CHUNK = (HIPQ_KCHUNK / 256) * 9 + 1; /* {S[8], d} per super-block */
   static constexpr int LANES_PER_OUT = 8;
 };
 
-/* ---- phase 1 ---------------------------------------------------------------- */
+/* Units a lane handles per chunk: 64 lanes cover a 4096-weight chunk in 2 (Q4_0) or
+ * 1 (Q4_K, Q6_K) steps; 16 lanes are only used for rows shorter than 64 units. */
+template <int DT, int T> struct GemvUnits {
+  static constexpr int MAXU = (T == 64) ? (HIPQ_KCHUNK / GemvRec<DT, false>::UNIT) / 64 : 4;
+};
 
-/* Q4_0: a unit is one 32-value block; a lane owns whole blocks, no cross-lane
- * step is needed. rec points at this weight row's records [R][PER_CHUNK]. */
-template <int T, int R>
-__device__ __forceinline__ void gemv_p1_q4_0(const WView &w, int row, int tl, const QView &qa,
-                                             const int (&arow)[R], int k0, int kc, uint32_t *rec) {
-  const int units = w.K >> 5, u0 = k0 >> 5, un = kc >> 5;
-  const uint4 *qs = (const uint4 *)w.qs + (size_t)row * units + u0;
-  const uint16_t *dw = w.d + (size_t)row * units + u0;
-#pragma unroll 2
-  for (int u = tl; u < un; u += T) {
-    const uint4 q = hipq_ld_stream(qs + u);
-    const float d = hipq_h2f(dw[u]);
-    const uint32_t lo[4] = {q.x & HIPQ_M4, q.y & HIPQ_M4, q.z & HIPQ_M4, q.w & HIPQ_M4};
-    const uint32_t hi[4] = {(q.x >> 4) & HIPQ_M4, (q.y >> 4) & HIPQ_M4, (q.z >> 4) & HIPQ_M4,
-                            (q.w >> 4) & HIPQ_M4};
+/* ---- Q4_0 ----------------------------------------------------------------------- */
+template <int T, int R, bool PW> struct GemvQ40 {
+  static constexpr int MAXU = GemvUnits<HIPQ_Q4_0, T>::MAXU;
+  static constexpr int PER = GemvRec<HIPQ_Q4_0, PW>::PER_CHUNK;
+  struct Act {
+    int4 a0[MAXU][R], a1[MAXU][R];
+    float da[MAXU][R];
+    int bsum[MAXU][R];
+  };
+  struct Wt {
+    uint4 q[MAXU];
+    uint16_t d[MAXU];
+  };
+  __device__ static __forceinline__ void load_act(Act &A, const QView &qa, const int (&arow)[R],
+                                                  int tl, int k0, int kc) {
+    const int units = qa.K >> 5, u0 = k0 >> 5, un = kc >> 5;
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const int4 *a = (const int4 *)(qa.q + (size_t)arow[r] * qa.K + (size_t)(u0 + u) * 32);
-      const int4 a0 = a[0], a1 = a[1];
-      const uint32_t meta = qa.meta[(size_t)arow[r] * units + u0 + u];
-      const float da = hipq_h2f((uint16_t)(meta & 0xffff));
-      const int bsum = (int)(int16_t)(meta >> 16);
-      const int isum = hipq_dot16(lo, a0) + hipq_dot16(hi, a1) - 8 * bsum; /* weights are nibble - 8 */
-      float2 v;
-      v.x = (float)isum;
-      v.y = d * da;
-      *(float2 *)(rec + r * GemvRec<HIPQ_Q4_0>::PER_CHUNK + 2 * u) = v;
+    for (int i = 0; i < MAXU; ++i) {
+      if (i * T >= un) break; /* uniform: this step lies beyond the chunk */
+      const int u = min(tl + i * T, un - 1);
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const int4 *a = (const int4 *)(qa.q + (size_t)arow[r] * qa.K + (size_t)(u0 + u) * 32);
+        A.a0[i][r] = a[0];
+        A.a1[i][r] = a[1];
+        const uint32_t meta = qa.meta[(size_t)arow[r] * units + u0 + u];
+        A.da[i][r] = hipq_h2f((uint16_t)(meta & 0xffff));
+        A.bsum[i][r] = (int)(int16_t)(meta >> 16);
+      }
     }
   }
-}
-
-/* Q4_K: a unit is 16 bytes = halves (h) of sub-blocks 2c and 2c+1 of a
- * super-block; lanes u and u^1 hold the two halves of pair c. */
-template <int T, int R>
-__device__ __forceinline__ void gemv_p1_q4_K(const WView &w, int row, int tl, const QView &qa,
-                                             const int (&arow)[R], int k0, int kc, uint32_t *rec) {
-  const int units = w.K >> 5, nsb = w.K >> 8, u0 = k0 >> 5, un = kc >> 5, b0 = k0 >> 8;
-  const uint4 *qs = (const uint4 *)w.qs + (size_t)row * units + u0;
-  const uint4 *hdr = (const uint4 *)w.hdr + (size_t)row * nsb + b0;
-  /* all lanes run the same trip count: the DPP exchange needs both partners */
-  const int trips = (un + T - 1) / T;
-#pragma unroll 2
-  for (int it = 0; it < trips; ++it) {
-    const int u = tl + it * T;
-    const bool on = u < un;
-    const int uc = on ? u : un - 1;
-    const int b = uc >> 3, c = (uc >> 1) & 3, h = uc & 1;
-    const uint4 q = hipq_ld_stream(qs + uc);
-    const uint4 hd = hdr[b];
-    uint32_t scw, mnw;
-    if (c < 2) {
-      scw = (hd.y >> (16 * c)) & 0x3f3fu;
-      mnw = (hd.z >> (16 * c)) & 0x3f3fu;
-    } else {
-      const int sh = 16 * (c - 2);
-      scw = ((hd.w >> sh) & 0x0f0fu) | ((((hd.y >> sh) >> 6) & 0x0303u) << 4);
-      mnw = (((hd.w >> sh) >> 4) & 0x0f0fu) | ((((hd.z >> sh) >> 6) & 0x0303u) << 4);
-    }
-    const int sc0 = (int)(scw & 0xff), sc1 = (int)(scw >> 8);
-    const int mn = (int)((mnw >> (8 * h)) & 0xff);
-    const uint32_t lo[4] = {q.x & HIPQ_M4, q.y & HIPQ_M4, q.z & HIPQ_M4, q.w & HIPQ_M4};
-    const uint32_t hi[4] = {(q.x >> 4) & HIPQ_M4, (q.y >> 4) & HIPQ_M4, (q.z >> 4) & HIPQ_M4,
-                            (q.w >> 4) & HIPQ_M4};
-    const int j = 2 * c + h;
-    const float dw = hipq_h2f((uint16_t)(hd.x & 0xffff));
-    const float dmin = hipq_h2f((uint16_t)(hd.x >> 16));
+  __device__ static __forceinline__ void load_w(Wt &W, const WView &w, int row, int tl, int k0,
+                                                int kc) {
+    const int units = w.K >> 5, u0 = k0 >> 5, un = kc >> 5;
+    const uint4 *qs = (const uint4 *)w.qs + (size_t)row * units + u0;
+    const uint16_t *dw = w.d + (size_t)row * units + u0;
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const int8_t *ab = qa.q + (size_t)arow[r] * qa.K + (size_t)(b0 + b) * 256 + c * 64 + h * 16;
-      const int4 alo = *(const int4 *)(ab);
-      const int4 ahi = *(const int4 *)(ab + 32);
-      int I = sc0 * hipq_dot16(lo, alo) + sc1 * hipq_dot16(hi, ahi);
-      const int bsw =
-        *(const int *)(qa.bsum + (size_t)arow[r] * (qa.K >> 4) + (b0 + b) * 16 + 2 * j);
-      int Im = mn * ((int)(int16_t)(bsw & 0xffff) + (bsw >> 16));
-      I += hipq_dpp_i<HIPQ_DPP_XOR1>(I); /* both halves of the sub-block pair */
-      Im += hipq_dpp_i<HIPQ_DPP_XOR1>(Im);
-      if (on && h == 0) {
-        uint32_t *o = rec + r * GemvRec<HIPQ_Q4_K>::PER_CHUNK + b * 10;
-        o[c] = (uint32_t)I;
-        o[4 + c] = (uint32_t)Im;
-        if (c == 0) {
-          const float dA = qa.d[(size_t)arow[r] * nsb + b0 + b];
-          o[8] = __float_as_uint(dw * dA);
-          o[9] = __float_as_uint(dmin * dA);
+    for (int i = 0; i < MAXU; ++i) {
+      if (i * T >= un) break;
+      const int u = min(tl + i * T, un - 1);
+      W.q[i] = hipq_ld_stream(qs + u);
+      W.d[i] = dw[u];
+    }
+  }
+  __device__ static __forceinline__ void compute(const Wt &W, const Act &A, int tl, int kc,
+                                                 uint32_t *rec) {
+    const int un = kc >> 5;
+#pragma unroll
+    for (int i = 0; i < MAXU; ++i) {
+      if (i * T >= un) break;
+      const int u = tl + i * T;
+      const uint4 q = W.q[i];
+      const float d = hipq_h2f(W.d[i]);
+      const uint32_t lo[4] = {q.x & HIPQ_M4, q.y & HIPQ_M4, q.z & HIPQ_M4, q.w & HIPQ_M4};
+      const uint32_t hi[4] = {(q.x >> 4) & HIPQ_M4, (q.y >> 4) & HIPQ_M4, (q.z >> 4) & HIPQ_M4,
+                              (q.w >> 4) & HIPQ_M4};
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        /* weights are nibble - 8 */
+        const int isum = hipq_dot16(lo, A.a0[i][r]) + hipq_dot16(hi, A.a1[i][r]) - 8 * A.bsum[i][r];
+        float2 v;
+        v.x = (float)isum;
+        v.y = d * A.da[i][r];
+        if (u < un) *(float2 *)(rec + r * PER + 2 * u) = v;
+      }
+    }
+  }
+};
+
+/* ---- Q4_K ----------------------------------------------------------------------- */
+/* A unit is one sub-block pair: 32 bytes whose low nibbles are sub-block 2c and
+ * whose high nibbles are sub-block 2c+1 of a super-block; 4 consecutive lanes
+ * hold one super-block, so its integer sums meet in two quad-permute DPP steps. */
+template <int T, int R, bool PW> struct GemvQ4K {
+  static constexpr int MAXU = GemvUnits<HIPQ_Q4_K, T>::MAXU;
+  static constexpr int PER = GemvRec<HIPQ_Q4_K, PW>::PER_CHUNK;
+  struct Act {
+    int4 lo0[MAXU][R], lo1[MAXU][R], hi0[MAXU][R], hi1[MAXU][R];
+    int bs0[MAXU][R], bs1[MAXU][R]; /* sums of the activations of sub-blocks 2c, 2c+1 */
+    float dA[MAXU][R];
+  };
+  struct Wt {
+    uint4 q0[MAXU], q1[MAXU];
+    uint4 hd[MAXU];
+  };
+  __device__ static __forceinline__ void load_act(Act &A, const QView &qa, const int (&arow)[R],
+                                                  int tl, int k0, int kc) {
+    const int nsb = qa.K >> 8, un = kc >> 6, b0 = k0 >> 8;
+#pragma unroll
+    for (int i = 0; i < MAXU; ++i) {
+      if (i * T >= un) break;
+      const int u = min(tl + i * T, un - 1);
+      const int b = u >> 2, c = u & 3;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const int4 *ab =
+          (const int4 *)(qa.q + (size_t)arow[r] * qa.K + (size_t)(b0 + b) * 256 + c * 64);
+        A.lo0[i][r] = ab[0];
+        A.lo1[i][r] = ab[1];
+        A.hi0[i][r] = ab[2];
+        A.hi1[i][r] = ab[3];
+        const int2 bsw = *(const int2 *)(qa.bsum + (size_t)arow[r] * (qa.K >> 4) +
+                                         (b0 + b) * 16 + 4 * c);
+        A.bs0[i][r] = (int)(int16_t)(bsw.x & 0xffff) + (bsw.x >> 16);
+        A.bs1[i][r] = (int)(int16_t)(bsw.y & 0xffff) + (bsw.y >> 16);
+        A.dA[i][r] = qa.d[(size_t)arow[r] * nsb + b0 + b];
+      }
+    }
+  }
+  __device__ static __forceinline__ void load_w(Wt &W, const WView &w, int row, int tl, int k0,
+                                                int kc) {
+    const int nsb = w.K >> 8, un = kc >> 6, b0 = k0 >> 8;
+    const uint4 *qs = (const uint4 *)(w.qs + (size_t)row * (w.K >> 1) + (size_t)b0 * 128);
+    const uint4 *hdr = (const uint4 *)w.hdr + (size_t)row * nsb + b0;
+#pragma unroll
+    for (int i = 0; i < MAXU; ++i) {
+      if (i * T >= un) break;
+      const int u = min(tl + i * T, un - 1);
+      W.q0[i] = hipq_ld_stream(qs + 2 * u);
+      W.q1[i] = hipq_ld_stream(qs + 2 * u + 1);
+      W.hd[i] = hdr[u >> 2];
+    }
+  }
+  __device__ static __forceinline__ void compute(const Wt &W, const Act &A, int tl, int kc,
+                                                 uint32_t *rec) {
+    const int un = kc >> 6;
+#pragma unroll
+    for (int i = 0; i < MAXU; ++i) {
+      if (i * T >= un) break;
+      const int u = tl + i * T;
+      const bool on = u < un;
+      const int uc = on ? u : un - 1;
+      const int b = uc >> 2, c = uc & 3;
+      const uint4 q0 = W.q0[i], q1 = W.q1[i];
+      const uint4 hd = W.hd[i];
+      /* 6-bit scales / mins of sub-blocks 2c, 2c+1: two adjacent bytes */
+      const int sh = 16 * (c & 1);
+      const uint32_t y = hd.y >> sh, z = hd.z >> sh, ww = hd.w >> sh;
+      const uint32_t sc_hi = (ww & 0x0f0fu) | (((y >> 6) & 0x0303u) << 4);
+      const uint32_t mn_hi = ((ww >> 4) & 0x0f0fu) | (((z >> 6) & 0x0303u) << 4);
+      const uint32_t scw = c < 2 ? (y & 0x3f3fu) : sc_hi;
+      const uint32_t mnw = c < 2 ? (z & 0x3f3fu) : mn_hi;
+      const int sc0 = (int)(scw & 0xff), sc1 = (int)(scw >> 8);
+      const int mn0 = (int)(mnw & 0xff), mn1 = (int)(mnw >> 8);
+      const uint32_t lo0[4] = {q0.x & HIPQ_M4, q0.y & HIPQ_M4, q0.z & HIPQ_M4, q0.w & HIPQ_M4};
+      const uint32_t lo1[4] = {q1.x & HIPQ_M4, q1.y & HIPQ_M4, q1.z & HIPQ_M4, q1.w & HIPQ_M4};
+      const uint32_t hi0[4] = {(q0.x >> 4) & HIPQ_M4, (q0.y >> 4) & HIPQ_M4, (q0.z >> 4) & HIPQ_M4,
+                               (q0.w >> 4) & HIPQ_M4};
+      const uint32_t hi1[4] = {(q1.x >> 4) & HIPQ_M4, (q1.y >> 4) & HIPQ_M4, (q1.z >> 4) & HIPQ_M4,
+                               (q1.w >> 4) & HIPQ_M4};
+      const float dw = hipq_h2f((uint16_t)(hd.x & 0xffff));
+      const float dmin = hipq_h2f((uint16_t)(hd.x >> 16));
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const int dlo = hipq_dot16(lo0, A.lo0[i][r]) + hipq_dot16(lo1, A.lo1[i][r]);
+        const int dhi = hipq_dot16(hi0, A.hi0[i][r]) + hipq_dot16(hi1, A.hi1[i][r]);
+        int I = __mul24(sc0, dlo) + __mul24(sc1, dhi);
+        int Im = __mul24(mn0, A.bs0[i][r]) + __mul24(mn1, A.bs1[i][r]);
+        if (PW) {
+          if (on) {
+            uint32_t *o = rec + r * PER + b * 10;
+            o[c] = (uint32_t)I;
+            o[4 + c] = (uint32_t)Im;
+            if (c == 0) {
+              o[8] = __float_as_uint(dw * A.dA[i][r]);
+              o[9] = __float_as_uint(dmin * A.dA[i][r]);
+            }
+          }
+        } else {
+          I += hipq_dpp_i<HIPQ_DPP_XOR1>(I); /* the four pairs of the super-block */
+          Im += hipq_dpp_i<HIPQ_DPP_XOR1>(Im);
+          I += hipq_dpp_i<HIPQ_DPP_XOR2>(I);
+          Im += hipq_dpp_i<HIPQ_DPP_XOR2>(Im);
+          if (on && c == 0) {
+            float4 v;
+            v.x = (float)I;
+            v.y = dw * A.dA[i][r];
+            v.z = (float)Im;
+            v.w = dmin * A.dA[i][r];
+            *(float4 *)(rec + r * PER + b * 4) = v;
+          }
         }
       }
     }
   }
-}
+};
 
-/* Q6_K: a unit is 64 weights = 2 x 16 B of ql + 16 B of qh, unit uu = half*2 + hl
- * of a super-block. Dword t of the unit belongs to partial l = hl*4 + t; lanes
- * uu and uu^2 hold the two halves. */
-template <int T, int R>
-__device__ __forceinline__ void gemv_p1_q6_K(const WView &w, int row, int tl, const QView &qa,
-                                             const int (&arow)[R], int k0, int kc, uint32_t *rec) {
-  const int nsb = w.K >> 8, b0 = k0 >> 8, un = kc >> 6;
-  const uint8_t *qlrow = w.qs + (size_t)row * (w.K >> 1) + (size_t)b0 * 128;
-  const uint8_t *qhrow = w.qh + (size_t)row * (w.K >> 2) + (size_t)b0 * 64;
-  const int8_t *scrow = w.sc + (size_t)row * (w.K >> 4) + (size_t)b0 * 16;
-  const uint16_t *drow = w.d + (size_t)row * nsb + b0;
-  const int trips = (un + T - 1) / T;
-  for (int it = 0; it < trips; ++it) {
-    const int u = tl + it * T;
-    const bool on = u < un;
-    const int uc = on ? u : un - 1;
-    const int b = uc >> 2, uu = uc & 3, half = uu >> 1, hl = uu & 1;
-    const uint8_t *ql = qlrow + b * 128 + half * 64 + hl * 16;
-    const uint4 qa_ = hipq_ld_stream((const uint4 *)ql);
-    const uint4 qb_ = hipq_ld_stream((const uint4 *)(ql + 32));
-    const uint4 qh_ = hipq_ld_stream((const uint4 *)(qhrow + b * 64 + half * 32 + hl * 16));
-    const int scw = *(const int *)(scrow + b * 16 + uu * 4);
-    const uint32_t A[4] = {qa_.x, qa_.y, qa_.z, qa_.w};
-    const uint32_t B[4] = {qb_.x, qb_.y, qb_.z, qb_.w};
-    const uint32_t H[4] = {qh_.x, qh_.y, qh_.z, qh_.w};
-    const int s0 = (int)(int8_t)(scw & 0xff), s1 = (int)(int8_t)((scw >> 8) & 0xff);
-    const int s2 = (int)(int8_t)((scw >> 16) & 0xff), s3 = (int)(int8_t)((scw >> 24) & 0xff);
-    const float dwt = hipq_h2f(drow[b]);
+/* ---- Q6_K ----------------------------------------------------------------------- */
+/* A unit is 64 weights = 2 x 16 B of ql + 16 B of qh, unit uu = half*2 + hl of a
+ * super-block. Dword t of the unit belongs to partial l = hl*4 + t; lanes uu and
+ * uu^2 hold the two 128-element halves. */
+template <int T, int R, bool PW> struct GemvQ6K {
+  static constexpr int MAXU = GemvUnits<HIPQ_Q6_K, T>::MAXU;
+  static constexpr int PER = GemvRec<HIPQ_Q6_K, PW>::PER_CHUNK;
+  struct Act {
+    int4 a[MAXU][R][4];
+    float dA[MAXU][R];
+  };
+  struct Wt {
+    uint4 qa[MAXU], qb[MAXU], qh[MAXU];
+    int scw[MAXU];
+    uint16_t d[MAXU];
+  };
+  __device__ static __forceinline__ void load_act(Act &A, const QView &qa, const int (&arow)[R],
+                                                  int tl, int k0, int kc) {
+    const int nsb = qa.K >> 8, un = kc >> 6, b0 = k0 >> 8;
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const int8_t *ab =
-        qa.q + (size_t)arow[r] * qa.K + (size_t)(b0 + b) * 256 + half * 128 + hl * 16;
-      const int4 a0 = *(const int4 *)(ab), a1 = *(const int4 *)(ab + 32);
-      const int4 a2 = *(const int4 *)(ab + 64), a3 = *(const int4 *)(ab + 96);
-      const int a0w[4] = {a0.x, a0.y, a0.z, a0.w}, a1w[4] = {a1.x, a1.y, a1.z, a1.w};
-      const int a2w[4] = {a2.x, a2.y, a2.z, a2.w}, a3w[4] = {a3.x, a3.y, a3.z, a3.w};
-      int P[4];
+    for (int i = 0; i < MAXU; ++i) {
+      if (i * T >= un) break;
+      const int u = min(tl + i * T, un - 1);
+      const int b = u >> 2, uu = u & 3, half = uu >> 1, hl = uu & 1;
 #pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        /* 6-bit values of the four 32-element groups, 4 at a time; (q6 - 32) . a
-         * = q6 . a - 32 . a, both via v_dot4 */
-        const int v0 = (int)((A[t] & HIPQ_M4) | ((H[t] << 4) & 0x30303030u));
-        const int v1 = (int)((B[t] & HIPQ_M4) | ((H[t] << 2) & 0x30303030u));
-        const int v2 = (int)(((A[t] >> 4) & HIPQ_M4) | (H[t] & 0x30303030u));
-        const int v3 = (int)(((B[t] >> 4) & HIPQ_M4) | ((H[t] >> 2) & 0x30303030u));
-        const int c32 = 0x20202020;
-        int p = s0 * (hipq_dot4(v0, a0w[t], 0) - hipq_dot4(c32, a0w[t], 0));
-        p += s1 * (hipq_dot4(v1, a1w[t], 0) - hipq_dot4(c32, a1w[t], 0));
-        p += s2 * (hipq_dot4(v2, a2w[t], 0) - hipq_dot4(c32, a2w[t], 0));
-        p += s3 * (hipq_dot4(v3, a3w[t], 0) - hipq_dot4(c32, a3w[t], 0));
-        P[t] = p + hipq_dpp_i<HIPQ_DPP_XOR2>(p); /* both 128-element halves */
-      }
-      if (on && half == 0) {
-        uint32_t *o = rec + r * GemvRec<HIPQ_Q6_K>::PER_CHUNK + b * 9;
+      for (int r = 0; r < R; ++r) {
+        const int8_t *ab =
+          qa.q + (size_t)arow[r] * qa.K + (size_t)(b0 + b) * 256 + half * 128 + hl * 16;
 #pragma unroll
-        for (int t = 0; t < 4; ++t) o[hl * 4 + t] = (uint32_t)P[t];
-        if (hl == 0) o[8] = __float_as_uint(qa.d[(size_t)arow[r] * nsb + b0 + b] * dwt);
+        for (int g = 0; g < 4; ++g) A.a[i][r][g] = *(const int4 *)(ab + 32 * g);
+        A.dA[i][r] = qa.d[(size_t)arow[r] * nsb + b0 + b];
       }
     }
   }
-}
+  __device__ static __forceinline__ void load_w(Wt &W, const WView &w, int row, int tl, int k0,
+                                                int kc) {
+    const int nsb = w.K >> 8, b0 = k0 >> 8, un = kc >> 6;
+    const uint8_t *qlrow = w.qs + (size_t)row * (w.K >> 1) + (size_t)b0 * 128;
+    const uint8_t *qhrow = w.qh + (size_t)row * (w.K >> 2) + (size_t)b0 * 64;
+    const int8_t *scrow = w.sc + (size_t)row * (w.K >> 4) + (size_t)b0 * 16;
+    const uint16_t *drow = w.d + (size_t)row * nsb + b0;
+#pragma unroll
+    for (int i = 0; i < MAXU; ++i) {
+      if (i * T >= un) break;
+      const int u = min(tl + i * T, un - 1);
+      const int b = u >> 2, uu = u & 3, half = uu >> 1, hl = uu & 1;
+      const uint8_t *ql = qlrow + b * 128 + half * 64 + hl * 16;
+      W.qa[i] = hipq_ld_stream((const uint4 *)ql);
+      W.qb[i] = hipq_ld_stream((const uint4 *)(ql + 32));
+      W.qh[i] = hipq_ld_stream((const uint4 *)(qhrow + b * 64 + half * 32 + hl * 16));
+      W.scw[i] = *(const int *)(scrow + b * 16 + uu * 4);
+      W.d[i] = drow[b];
+    }
+  }
+  __device__ static __forceinline__ void compute(const Wt &W, const Act &A, int tl, int kc,
+                                                 uint32_t *rec) {
+    const int un = kc >> 6;
+#pragma unroll
+    for (int i = 0; i < MAXU; ++i) {
+      if (i * T >= un) break;
+      const int u = tl + i * T;
+      const bool on = u < un;
+      const int uc = on ? u : un - 1;
+      const int b = uc >> 2, uu = uc & 3, half = uu >> 1, hl = uu & 1;
+      const uint32_t QA[4] = {W.qa[i].x, W.qa[i].y, W.qa[i].z, W.qa[i].w};
+      const uint32_t QB[4] = {W.qb[i].x, W.qb[i].y, W.qb[i].z, W.qb[i].w};
+      const uint32_t H[4] = {W.qh[i].x, W.qh[i].y, W.qh[i].z, W.qh[i].w};
+      const int scw = W.scw[i];
+      const int s0 = (int)(int8_t)(scw & 0xff), s1 = (int)(int8_t)((scw >> 8) & 0xff);
+      const int s2 = (int)(int8_t)((scw >> 16) & 0xff), s3 = (int)(int8_t)((scw >> 24) & 0xff);
+      const float dwt = hipq_h2f(W.d[i]);
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        const int a0w[4] = {A.a[i][r][0].x, A.a[i][r][0].y, A.a[i][r][0].z, A.a[i][r][0].w};
+        const int a1w[4] = {A.a[i][r][1].x, A.a[i][r][1].y, A.a[i][r][1].z, A.a[i][r][1].w};
+        const int a2w[4] = {A.a[i][r][2].x, A.a[i][r][2].y, A.a[i][r][2].z, A.a[i][r][2].w};
+        const int a3w[4] = {A.a[i][r][3].x, A.a[i][r][3].y, A.a[i][r][3].z, A.a[i][r][3].w};
+        int P[4];
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          /* 6-bit values of the four 32-element groups, 4 at a time;
+           * (q6 - 32) . a = q6 . a - 32 . a, both via v_dot4 */
+          const int v0 = (int)((QA[t] & HIPQ_M4) | ((H[t] << 4) & 0x30303030u));
+          const int v1 = (int)((QB[t] & HIPQ_M4) | ((H[t] << 2) & 0x30303030u));
+          const int v2 = (int)(((QA[t] >> 4) & HIPQ_M4) | (H[t] & 0x30303030u));
+          const int v3 = (int)(((QB[t] >> 4) & HIPQ_M4) | ((H[t] >> 2) & 0x30303030u));
+          const int c32 = 0x20202020;
+          int p = __mul24(s0, hipq_dot4(v0, a0w[t], 0) - hipq_dot4(c32, a0w[t], 0));
+          p += __mul24(s1, hipq_dot4(v1, a1w[t], 0) - hipq_dot4(c32, a1w[t], 0));
+          p += __mul24(s2, hipq_dot4(v2, a2w[t], 0) - hipq_dot4(c32, a2w[t], 0));
+          p += __mul24(s3, hipq_dot4(v3, a3w[t], 0) - hipq_dot4(c32, a3w[t], 0));
+          P[t] = p + hipq_dpp_i<HIPQ_DPP_XOR2>(p); /* both 128-element halves */
+        }
+        if (on && half == 0) {
+          uint32_t *o = rec + r * PER + b * 9;
+#pragma unroll
+          for (int t = 0; t < 4; ++t) o[hl * 4 + t] = (uint32_t)P[t];
+          if (hl == 0) o[8] = __float_as_uint(A.dA[i][r] * dwt);
+        }
+      }
+    }
+  }
+};
 
-/* ---- engine ------------------------------------------------------------------ */
+template <int DT, int T, int R, bool PW> struct GemvFmt;
+template <int T, int R, bool PW> struct GemvFmt<HIPQ_Q4_0, T, R, PW> { typedef GemvQ40<T, R, PW> type; };
+template <int T, int R, bool PW> struct GemvFmt<HIPQ_Q4_K, T, R, PW> { typedef GemvQ4K<T, R, PW> type; };
+template <int T, int R, bool PW> struct GemvFmt<HIPQ_Q6_K, T, R, PW> { typedef GemvQ6K<T, R, PW> type; };
+
+/* ---- engine --------------------------------------------------------------------- */
 
 struct GemvOut {
   float v;    /* finished output                                   */
@@ -248,16 +408,18 @@ struct GemvOut {
  * Computes, for the G weight rows starting at row0 (clamped to the matrix) and
  * the R activation rows arow[], all G*R outputs. Must be called by every lane
  * of every wavefront of the workgroup (it uses __syncthreads); `lds` is this
- * wavefront's private region of G*R*PER_CHUNK dwords. `pair_rows`: activation
- * rows with arow[r] < pair_rows use the per-sub-block-pair order (Q4_K only).
+ * wavefront's private region of G*R*PER_CHUNK dwords. With PW, activation rows
+ * arow[r] < pair_rows use the per-sub-block-pair order (Q4_K only).
  */
-template <int DT, int T, int R, int G>
+template <int DT, int T, int R, int G, bool PW>
 __device__ __forceinline__ GemvOut gemv_engine(const WView &w, int row0, const QView &qa,
                                                const int (&arow)[R], int pair_rows,
                                                uint32_t *lds) {
+  typedef typename GemvFmt<DT, T, R, PW>::type F;
   constexpr int RW = 64 / T; /* weight rows streamed at once */
-  constexpr int PER = GemvRec<DT>::PER_CHUNK;
-  constexpr int LPO = GemvRec<DT>::LANES_PER_OUT;
+  constexpr int NP = G / RW; /* passes per group */
+  constexpr int PER = GemvRec<DT, PW>::PER_CHUNK;
+  constexpr int LPO = GemvRec<DT, PW>::LANES_PER_OUT;
   static_assert(G % RW == 0, "group must be a multiple of the rows streamed at once");
   static_assert(G * R * LPO <= 64, "one lane per fp32 chain");
   const int lane = threadIdx.x & 63, tl = lane % T;
@@ -266,29 +428,44 @@ __device__ __forceinline__ GemvOut gemv_engine(const WView &w, int row0, const Q
   const int cg = chain ? ci / R : 0, cr = chain ? ci % R : 0;
   const uint32_t *crec = lds + (cg * R + cr) * PER;
   float acc = 0.f, accm = 0.f;
-  const bool pairwise = DT == HIPQ_Q4_K && arow[cr] < pair_rows;
+  bool pairwise = false;
+  if (PW) {
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+      if (r == cr) pairwise = arow[r] < pair_rows;
+  }
 
   for (int k0 = 0; k0 < w.K; k0 += HIPQ_KCHUNK) {
     const int kc = min(HIPQ_KCHUNK, w.K - k0);
+    typename F::Act A;
+    F::load_act(A, qa, arow, tl, k0, kc);
+    typename F::Wt W[NP];
 #pragma unroll
-    for (int pass = 0; pass < G / RW; ++pass) {
+    for (int pass = 0; pass < NP; ++pass) {
       const int g = pass * RW + lane / T;
-      const int row = min(row0 + g, w.N - 1);
-      uint32_t *rec = lds + g * R * PER;
-      if (DT == HIPQ_Q4_0)
-        gemv_p1_q4_0<T, R>(w, row, tl, qa, arow, k0, kc, rec);
-      else if (DT == HIPQ_Q4_K)
-        gemv_p1_q4_K<T, R>(w, row, tl, qa, arow, k0, kc, rec);
-      else
-        gemv_p1_q6_K<T, R>(w, row, tl, qa, arow, k0, kc, rec);
+      F::load_w(W[pass], w, min(row0 + g, w.N - 1), tl, k0, kc);
+    }
+#pragma unroll
+    for (int pass = 0; pass < NP; ++pass) {
+      const int g = pass * RW + lane / T;
+      F::compute(W[pass], A, tl, kc, lds + g * R * PER);
     }
     __syncthreads();
     if (chain) {
       if (DT == HIPQ_Q4_0) {
         const int nb = kc >> 5;
+#pragma unroll 4
         for (int b = 0; b < nb; ++b) {
           const float2 v = *(const float2 *)(crec + 2 * b);
           acc = fmaf(v.x, v.y, acc);
+        }
+      } else if (DT == HIPQ_Q4_K && !PW) {
+        const int nb = kc >> 8;
+#pragma unroll 4
+        for (int b = 0; b < nb; ++b) {
+          const float4 v = *(const float4 *)(crec + 4 * b);
+          acc = fmaf(v.x, v.y, acc);
+          accm = fmaf(v.z, v.w, accm);
         }
       } else if (DT == HIPQ_Q4_K) {
         const int nb = kc >> 8;
@@ -313,6 +490,7 @@ __device__ __forceinline__ GemvOut gemv_engine(const WView &w, int row0, const Q
         }
       } else {
         const int nb = kc >> 8;
+#pragma unroll 4
         for (int b = 0; b < nb; ++b) {
           const uint32_t *o = crec + b * 9;
           acc = fmaf(__uint_as_float(o[8]), (float)(int)o[l], acc);
@@ -343,15 +521,9 @@ __device__ __forceinline__ GemvOut gemv_engine(const WView &w, int row0, const Q
   return out;
 }
 
-/* Weight rows per group for a given number of activation rows: G * R fp32
- * chains per wavefront (16 for Q4_K, whose records are small; 8 otherwise),
- * at most 8 rows. */
-template <int DT, int R> struct GemvGroup {
-  static constexpr int CHAINS = DT == HIPQ_Q4_K ? 16 : 8;
-  static constexpr int G = (CHAINS / R) >= 8 ? 8 : (CHAINS / R);
-  static constexpr int LDS_DWORDS = G * R * GemvRec<DT>::PER_CHUNK; /* per wavefront */
-  /* 16 lanes per weight row stream 4 rows at once, so G must be a multiple of 4 */
-  static constexpr bool T16_OK = (G % 4) == 0;
+/* LDS dwords one wavefront needs for G weight rows x R activation rows. */
+template <int DT, int R, int G, bool PW> struct GemvLds {
+  static constexpr int DWORDS = G * R * GemvRec<DT, PW>::PER_CHUNK;
 };
 
 #endif /* HIPQ_GEMV_DEVICE_H */

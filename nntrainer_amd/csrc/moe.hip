@@ -32,6 +32,7 @@
 namespace {
 
 constexpr int RTOK = 4; /* tokens sharing one pass over an expert's weight rows */
+constexpr int GROW = 2; /* weight rows (output columns) per wavefront and pass      */
 
 struct MoeBufs {
   float *logits;
@@ -215,14 +216,14 @@ __global__ __launch_bounds__(256) void gate_up_kernel(const WView *__restrict__ 
                                                       QView xq, const int *__restrict__ offsets,
                                                       const int *__restrict__ slot_pair, int topk,
                                                       int I, float *__restrict__ h) {
-  constexpr int G = GemvGroup<DT, RTOK>::G;
+  constexpr int G = GROW;
   extern __shared__ uint32_t moe_lds[];
   const int e = blockIdx.y;
   const int begin = offsets[e], end = offsets[e + 1];
   if (begin == end) return;
   const WView wg = views[e], wu = views[E + e];
   const int wave = threadIdx.x >> 6;
-  uint32_t *lds = moe_lds + wave * GemvGroup<DT, RTOK>::LDS_DWORDS;
+  uint32_t *lds = moe_lds + wave * GemvLds<DT, RTOK, GROW, false>::DWORDS;
   const int col0 = (blockIdx.x * 4 + wave) * G;
   for (int s0 = begin; s0 < end; s0 += RTOK) {
     int arow[RTOK];
@@ -231,8 +232,8 @@ __global__ __launch_bounds__(256) void gate_up_kernel(const WView *__restrict__ 
       const int slot = min(s0 + r, end - 1);
       arow[r] = slot_pair[slot] / topk; /* token of the pair */
     }
-    const GemvOut g = gemv_engine<DT, T, RTOK, G>(wg, col0, xq, arow, 0, lds);
-    const GemvOut u = gemv_engine<DT, T, RTOK, G>(wu, col0, xq, arow, 0, lds);
+    const GemvOut g = gemv_engine<DT, T, RTOK, G, false>(wg, col0, xq, arow, 0, lds);
+    const GemvOut u = gemv_engine<DT, T, RTOK, G, false>(wu, col0, xq, arow, 0, lds);
     if (g.valid && col0 + g.g < I && s0 + g.r < end)
       h[(size_t)(s0 + g.r) * I + col0 + g.g] = silu_ref(g.v) * u.v;
   }
@@ -245,20 +246,20 @@ __global__ __launch_bounds__(256) void down_kernel(const WView *__restrict__ vie
                                                    const int *__restrict__ slot_pair,
                                                    const float *__restrict__ wgt, int H,
                                                    float *__restrict__ contrib) {
-  constexpr int G = GemvGroup<DT, RTOK>::G;
+  constexpr int G = GROW;
   extern __shared__ uint32_t moe_lds[];
   const int e = blockIdx.y;
   const int begin = offsets[e], end = offsets[e + 1];
   if (begin == end) return;
   const WView wd = views[2 * E + e];
   const int wave = threadIdx.x >> 6;
-  uint32_t *lds = moe_lds + wave * GemvGroup<DT, RTOK>::LDS_DWORDS;
+  uint32_t *lds = moe_lds + wave * GemvLds<DT, RTOK, GROW, false>::DWORDS;
   const int col0 = (blockIdx.x * 4 + wave) * G;
   for (int s0 = begin; s0 < end; s0 += RTOK) {
     int arow[RTOK];
 #pragma unroll
     for (int r = 0; r < RTOK; ++r) arow[r] = min(s0 + r, end - 1); /* hq rows are slots */
-    const GemvOut o = gemv_engine<DT, T, RTOK, G>(wd, col0, hq, arow, 0, lds);
+    const GemvOut o = gemv_engine<DT, T, RTOK, G, false>(wd, col0, hq, arow, 0, lds);
     if (o.valid && col0 + o.g < H && s0 + o.r < end)
       contrib[(size_t)(s0 + o.r) * H + col0 + o.g] = o.v * wgt[slot_pair[s0 + o.r]];
   }
@@ -296,9 +297,9 @@ template <int DT>
 int launch_grouped(const hipq::MoeArgs *a, const MoeBufs &b, const WView *views, const QAct &xq,
                    const QAct &hq, hipStream_t s) {
   const hipq_moe_desc &d = a->desc;
-  constexpr int G = GemvGroup<DT, RTOK>::G;
-  constexpr int TS = GemvGroup<DT, RTOK>::T16_OK ? 16 : 64; /* lanes per row for short K */
-  const size_t lds = 4 * GemvGroup<DT, RTOK>::LDS_DWORDS * sizeof(uint32_t);
+  constexpr int G = GROW;
+  constexpr int TS = 64;
+  const size_t lds = 4 * GemvLds<DT, RTOK, GROW, false>::DWORDS * sizeof(uint32_t);
   const int64_t units_gu = (DT == HIPQ_Q6_K) ? d.hidden / 64 : d.hidden / 32;
   const int64_t units_dn = (DT == HIPQ_Q6_K) ? d.intermediate / 64 : d.intermediate / 32;
   const int64_t P = (int64_t)d.tokens * d.topk;

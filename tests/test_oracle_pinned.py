@@ -1,0 +1,231 @@
+"""CPU: pin the oracle (oracle/nntr_oracle.c).
+
+Three kinds of evidence, none of which retypes the oracle's own formulas:
+ 1. bit-for-bit equality with the reference library built from the reference's own
+    sources (oracle/_ref), when that library is present;
+ 2. closed forms the block formats fix: matmul == dot(dequant(W), dequant(QA)) in
+    double; repack is an invertible byte permutation; quantizer invariants;
+ 3. committed golden digests of oracle outputs on seeded inputs (tests/golden),
+    produced where the reference library was available, so drift of the oracle is
+    caught on machines without it.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import cpuref as cr
+from nntrainer_amd import synth
+
+KINDS = ["q4_0", "q4_K", "q6_K"]
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden", "oracle_digests.json")
+needs_ref = pytest.mark.skipif(cr.ref() is None, reason="reference library not built here")
+
+
+def _w(seed, n, k, sigma=0.02):
+    w = synth.normal(seed, (n, k), sigma)
+    w[1, :256] = 0.0       # all-zero super-block / blocks
+    w[2, 256:288] = 0.0    # one zero sub-block
+    w[3, 0:32] = 0.01      # constant sub-block (max == min)
+    return w
+
+
+# ------------------------------------------------------------------ 1. vs reference
+@needs_ref
+def test_fp16_conversions_match_reference():
+    o, r = cr.oracle(), cr.ref()
+    for h in range(0, 65536, 1):
+        a, b = o.orc_fp16_to_fp32(h), r.ref_fp16_to_fp32(h)
+        assert np.float32(a).view(np.uint32) == np.float32(b).view(np.uint32) or (a != a and b != b)
+    rng = np.random.default_rng(0)
+    fs = np.concatenate([rng.standard_normal(20000).astype(np.float32) * s
+                         for s in (1, 1e-3, 1e-5, 1e-7, 300, 7e4)])
+    edge = np.array([65504, 65519.99, 65520, 65536, 1e-8, 5.96e-8, 2.98e-8, 2.9802322e-8, 0, -0.0,
+                     np.inf, -np.inf, 6.1e-5, 6.0975e-5], np.float32)
+    for f in np.concatenate([fs, edge]):
+        assert o.orc_fp32_to_fp16(float(f)) == r.ref_fp32_to_fp16(float(f)), f
+
+
+@needs_ref
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("sigma", [0.02, 1.0])
+def test_weight_quantizer_bytes_match_reference(kind, sigma):
+    w = _w(3, 256, 2048, sigma)
+    assert np.array_equal(cr.quantize_weights(cr.oracle(), kind, w), cr.quantize_weights(cr.ref(), kind, w))
+
+
+@needs_ref
+@pytest.mark.parametrize("kind", KINDS)
+def test_dequantize_matches_reference(kind):
+    q = cr.quantize_weights(cr.ref(), kind, _w(4, 64, 1024))
+    a, b = cr.dequantize(cr.oracle(), kind, q, 64 * 1024), cr.dequantize(cr.ref(), kind, q, 64 * 1024)
+    assert np.array_equal(a.view(np.uint32), b.view(np.uint32))
+
+
+@needs_ref
+@pytest.mark.parametrize("kind", ["q4_0", "q4_K"])
+def test_repack_matches_reference(kind):
+    q = cr.quantize_weights(cr.ref(), kind, _w(5, 64, 1024))
+    assert np.array_equal(cr.repack_x8(cr.oracle(), kind, q, 64, 1024), cr.repack_x8(cr.ref(), kind, q, 64, 1024))
+
+
+def _act_cases(k):
+    x = synth.normal(11, (16, k))
+    x[0, :] = 0.0
+    x[2, 5] = 9.5; x[2, 9] = -9.5
+    x[3, 5] = -9.5; x[3, 9] = 9.5
+    x[4, :] *= 1e-6
+    x[5, :] *= 1e4
+    return x
+
+
+@needs_ref
+@pytest.mark.parametrize("kind", ["q8_0", "q8_K"])
+def test_activation_quantizers_match_reference(kind):
+    x = _act_cases(1024)
+    adv = np.load(os.path.join(os.path.dirname(__file__), "golden", "q8k_rounding_adversaries.npy"))
+    x = np.concatenate([x, adv.reshape(-1, 256)[:24].reshape(-1, 1024)])
+    x = x[: (len(x) // 4) * 4]
+    o, r = cr.oracle(), cr.ref()
+    assert np.array_equal(cr.quantize_act(o, kind, x, "row"), cr.quantize_act(r, kind, x, "row"))
+    mo = cr.quantize_act(o, kind, x, "mat")
+    inter = np.stack([cr.interleave4(kind, mo[4 * g:4 * g + 4], 1024) for g in range(len(x) // 4)])
+    assert np.array_equal(inter, cr.quantize_act(r, kind, x, "mat"))
+
+
+@needs_ref
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("m", [1, 3, 4, 7, 16, 35])
+def test_matmul_bits_match_reference(kind, m):
+    """Same bits as the reference wrapper, for GEMV (M=1), the 4-row GEMM path and the
+    leftover-row path (M % 4 != 0)."""
+    n, k = 128, 1024
+    q = cr.quantize_weights(cr.ref(), kind, _w(6, n, k))
+    a = synth.normal(60 + m, (m, k))
+    co, cc = cr.gemm(cr.oracle(), kind, a, q, n), cr.gemm(cr.ref(), kind, a, q, n)
+    assert np.array_equal(co.view(np.uint32), cc.view(np.uint32))
+
+
+# ------------------------------------------------------------------ 2. closed forms
+@pytest.mark.parametrize("kind", KINDS)
+def test_matmul_equals_dequantized_dot(kind):
+    """C == dequant(QA) . dequant(W)^T evaluated in double (a textbook dot product):
+    catches a wrong nibble order, scale index, sign or a dropped min term."""
+    n, k, m = 96, 1024, 5
+    o = cr.oracle()
+    q = cr.quantize_weights(o, kind, _w(7, n, k))
+    a = synth.normal(70, (m, k))
+    wd = cr.dequantize(o, kind, q, n * k).reshape(n, k).astype(np.float64)
+    if kind == "q4_0":
+        qa = cr.quantize_act(o, "q8_0", a)
+        ad = np.stack([cr.dequantize(o, "q8_0", qa[i], k) for i in range(m)]).astype(np.float64)
+    else:
+        var = ["mat" if (kind == "q4_K" and i < (m // 4) * 4) else "row" for i in range(m)]
+        ad = np.stack([cr.dequantize(o, "q8_K", cr.quantize_act(o, "q8_K", a[i:i + 1], var[i])[0], k)
+                       for i in range(m)]).astype(np.float64)
+    want = ad @ wd.T
+    got = cr.gemm(o, kind, a, q, n)
+    assert np.abs(got - want).max() / np.abs(want).max() < 2e-6
+
+
+@pytest.mark.parametrize("kind", KINDS)
+def test_weight_quantizer_round_trip_error(kind):
+    """Quantize -> dequantize error stays within the format's step (the reference's own
+    acceptance is an mse bound, unittest_nntrainer_cpu_backend.cpp:182-293)."""
+    o = cr.oracle()
+    w = synth.normal(8, (64, 1024), 0.02)
+    back = cr.dequantize(o, kind, cr.quantize_weights(o, kind, w), w.size).reshape(w.shape)
+    rel = np.abs(back - w).max() / np.abs(w).max()
+    assert rel < {"q4_0": 0.09, "q4_K": 0.07, "q6_K": 0.02}[kind]
+    mse = float(((back - w) ** 2).mean())
+    assert mse < 1e-5
+
+
+@pytest.mark.parametrize("kind", ["q4_0", "q4_K"])
+def test_repack_is_an_invertible_permutation(kind):
+    o = cr.oracle()
+    q = cr.quantize_weights(o, kind, _w(9, 64, 1024))
+    x8 = cr.repack_x8(o, kind, q, 64, 1024)
+    assert x8.size == q.size and not np.array_equal(x8, q)
+    assert np.array_equal(cr.unpack_x8(kind, x8, 64, 1024), q)
+    # repack refuses row counts that are not multiples of 8 (reference returns -1)
+    out = np.zeros(18 * 12 * 2, np.uint8)
+    assert o.orc_repack_q4_0_x8(out.ctypes.data, out.ctypes.data, 12, 64) == -1
+
+
+def test_activation_quantizer_invariants():
+    o = cr.oracle()
+    x = _act_cases(1024)
+    for variant in ("row", "mat"):
+        blk = cr.quantize_act(o, "q8_K", x, variant).reshape(len(x), -1, 292)
+        d = blk[..., :4].copy().view(np.float32)[..., 0]
+        qs = blk[..., 4:260].copy().view(np.int8).astype(np.int32)
+        bs = blk[..., 260:].copy().view(np.int16).astype(np.int32)
+        assert (np.abs(qs) <= 127).all() or variant == "mat"
+        assert np.array_equal(qs.reshape(len(x), -1, 16, 16).sum(-1), bs)       # group sums consistent
+        xb = x.reshape(len(x), -1, 256)
+        assert (np.abs(d[..., None] * qs - xb) <= np.abs(d[..., None]) * 0.5000001 + 1e-30).all()
+        assert (d[0] == 0).all() and (qs[0] == 0).all()                         # all-zero row
+    # sign rule when +amax and -amax both occur: row follows the first, mat a positive hit
+    r2 = cr.quantize_act(o, "q8_K", x[2:4], "row").reshape(2, -1, 292)[:, 0, :4].copy().view(np.float32)
+    m2 = cr.quantize_act(o, "q8_K", x[2:4], "mat").reshape(2, -1, 292)[:, 0, :4].copy().view(np.float32)
+    assert r2[0, 0] < 0 and r2[1, 0] > 0 and m2[0, 0] < 0 and m2[1, 0] < 0
+    b0 = cr.quantize_act(o, "q8_0", x).reshape(len(x), -1, 34)
+    q0 = b0[..., 2:].copy().view(np.int8)
+    assert (np.abs(q0.astype(np.int32)) <= 127).all()
+    assert (np.abs(q0).max(-1)[1] == 127).all()  # the max element maps to +-127
+
+
+def test_moe_equals_dense_per_token_evaluation():
+    """MoE block == for every token, softmax over its top-k logits as weights of the
+    SwiGLU MLPs of those experts, each built from the oracle's single-row matmul."""
+    o = cr.oracle()
+    t, h, i, e, k = 6, 256, 256, 8, 3
+    gate = [cr.quantize_weights(o, "q4_K", synth.normal(100 + 3 * x, (i, h), 0.02)) for x in range(e)]
+    up = [cr.quantize_weights(o, "q4_K", synth.normal(101 + 3 * x, (i, h), 0.02)) for x in range(e)]
+    down = [cr.quantize_weights(o, "q4_K", synth.normal(102 + 3 * x, (h, i), 0.02)) for x in range(e)]
+    x = synth.normal(200, (t, h))
+    logits = synth.normal(201, (t, e))
+    y, idx, wt = cr.moe_forward(x, logits, gate, up, down, k)
+    want = np.zeros((t, h), np.float64)
+    for tt in range(t):
+        order = np.argsort(-logits[tt], kind="stable")[:k]
+        assert set(order) == set(idx[tt])
+        lw = np.exp(logits[tt, order].astype(np.float64) - logits[tt, order].max())
+        lw /= lw.sum()  # renormalised softmax == softmax over the selected logits
+        for ee, ww in zip(order, lw):
+            g = cr.gemm(o, "q4_K", x[tt:tt + 1], gate[ee], i)[0].astype(np.float64)
+            u = cr.gemm(o, "q4_K", x[tt:tt + 1], up[ee], i)[0].astype(np.float64)
+            hh = (g / (1 + np.exp(-g)) * u).astype(np.float32)
+            want[tt] += ww * cr.gemm(o, "q4_K", hh[None], down[ee], h)[0]
+    assert np.abs(y - want).max() / np.abs(want).max() < 2e-3  # h re-rounded to fp32 / requantized
+    assert np.abs(wt.sum(1) - 1).max() < 1e-6
+
+
+# ------------------------------------------------------------------ 3. golden digests
+def _digest_cases():
+    o = cr.oracle()
+    out = {}
+    for kind in KINDS:
+        w = _w(20, 64, 1024)
+        q = cr.quantize_weights(o, kind, w)
+        out["wquant_" + kind] = synth.digest(q)
+        for m in (1, 6):
+            out["gemm_%s_m%d" % (kind, m)] = synth.digest(cr.gemm(o, kind, synth.normal(21 + m, (m, 1024)), q, 64))
+    x = _act_cases(1024)
+    out["q8_0"] = synth.digest(cr.quantize_act(o, "q8_0", x))
+    out["q8_K_row"] = synth.digest(cr.quantize_act(o, "q8_K", x, "row"))
+    out["q8_K_mat"] = synth.digest(cr.quantize_act(o, "q8_K", x, "mat"))
+    out["input_w"] = synth.digest(_w(20, 64, 1024))
+    return out
+
+
+def test_golden_digests():
+    """tests/golden/oracle_digests.json was written by tests/golden/make_golden.py on a
+    machine where every digest's output had just been compared bit-for-bit with the
+    reference library."""
+    want = json.load(open(GOLDEN))
+    got = _digest_cases()
+    assert got["input_w"] == want["input_w"], "input generator drifted, not the oracle"
+    assert got == want
