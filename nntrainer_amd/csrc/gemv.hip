@@ -17,8 +17,6 @@
  * HBM: per output column it reads the column's packed weights exactly once,
  * 16 bytes per lane per load, all loads of a group in flight together.
  */
-#include <cstdlib>
-
 #include "gemv_device.h"
 
 namespace {
@@ -50,7 +48,6 @@ int launch_one(const hipq_weight *w, const QAct *qa, int M, int pair_rows, float
 
 /* Largest group size not above gmax that still gives ~6000 wavefronts. */
 int pick_group(int64_t N, int gmax) {
-  if (const char *e = getenv("HIPQ_GEMV_G")) return atoi(e);
   /* measured: 4 rows per wavefront is best from N = 8192 up to the 151936-row
    * lm_head; smaller matrices want more, shorter wavefronts */
   int g = N >= 8192 ? 4 : (N >= 2048 ? 2 : 1);
