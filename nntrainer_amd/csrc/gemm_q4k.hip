@@ -65,8 +65,8 @@ struct BBlock { /* one super-block of weights: 64 columns x 128 bytes + headers 
   uint4 hd;
 };
 struct RowBlock { /* per-row data of one super-block (threads 0..127) */
-  uint4 bs0, bs1;
-  float dA;
+  uint4 bs0 = {0, 0, 0, 0}, bs1 = {0, 0, 0, 0};
+  float dA = 0.f;
 };
 
 /* per 16-bit half: (two bytes <= 15) * (digit <= 7): no carry between bytes */
@@ -127,6 +127,8 @@ __device__ __forceinline__ void load_b(BBlock &b, const Addr &ad, int sb) {
   b.hd = *(const uint4 *)(ad.hdr + (ad.hd + (uint32_t)(sb * 16)));
 }
 __device__ __forceinline__ void load_row(RowBlock &r, const Addr &ad, int sb) {
+  /* whole wavefronts 0 and 1 own the 128 rows; the branch is uniform per wavefront */
+  if (__builtin_amdgcn_readfirstlane((int)threadIdx.x) >= BM) return;
   const uint4 *bp = (const uint4 *)((const char *)ad.bsum + (ad.bs + (uint32_t)(sb * 32)));
   r.bs0 = bp[0];
   r.bs1 = bp[1];
@@ -176,7 +178,7 @@ __device__ __forceinline__ void store_b(const BBlock &b, Smem &sm) {
 
 __device__ __forceinline__ void store_row(const RowBlock &rb, Smem &sm) {
   const int t = threadIdx.x;
-  if (t < BM) {
+  if (__builtin_amdgcn_readfirstlane(t) < BM) {
     const uint32_t wds[8] = {rb.bs0.x, rb.bs0.y, rb.bs0.z, rb.bs0.w,
                              rb.bs1.x, rb.bs1.y, rb.bs1.z, rb.bs1.w};
     v8h vlo, vhi;
@@ -204,23 +206,49 @@ __device__ __forceinline__ int acc_row(int r, int lane) {
   return 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
 }
 
-/* One 32-deep step of both digit chains over the wavefront's 2 x 1 tiles. */
-template <bool FIRST>
-__device__ __forceinline__ void kstep(const Smem &sm, int buf, int ks, int wm, int wn, int i32,
-                                      int g, v16i (&Dlo)[2], v16i (&Dhi)[2]) {
-  const v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-  v4i a[2], bl, bh;
-#pragma unroll
-  for (int tm = 0; tm < 2; ++tm)
-    a[tm] = *(const v4i *)(sm.a[buf] + (wm * 64 + tm * 32 + i32) * STRIDE + ks * 32 + g * 16);
+/* Operands of one 32-deep step of the wavefront's 2 x 1 tiles. */
+struct Ops {
+  v4i a0, a1, bl, bh;
+};
+__device__ __forceinline__ void read_ops(Ops &o, const Smem &sm, int buf, int ks, int wm, int wn,
+                                         int i32, int g) {
+  const int8_t *pa = sm.a[buf] + (wm * 64 + i32) * STRIDE + ks * 32 + g * 16;
+  o.a0 = *(const v4i *)pa;
+  o.a1 = *(const v4i *)(pa + 32 * STRIDE);
   const int off = (wn * 32 + i32) * STRIDE + ks * 32 + g * 16;
-  bl = *(const v4i *)(sm.blo[buf] + off);
-  bh = *(const v4i *)(sm.bhi[buf] + off);
-#pragma unroll
-  for (int tm = 0; tm < 2; ++tm) {
-    Dlo[tm] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[tm], bl, FIRST ? zero16 : Dlo[tm], 0, 0, 0);
-    Dhi[tm] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[tm], bh, FIRST ? zero16 : Dhi[tm], 0, 0, 0);
-  }
+  o.bl = *(const v4i *)(sm.blo[buf] + off);
+  o.bh = *(const v4i *)(sm.bhi[buf] + off);
+}
+template <bool FIRST>
+__device__ __forceinline__ void mma_ops(const Ops &o, v16i (&Dlo)[2], v16i (&Dhi)[2]) {
+  const v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  Dlo[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(o.a0, o.bl, FIRST ? zero16 : Dlo[0], 0, 0, 0);
+  Dhi[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(o.a0, o.bh, FIRST ? zero16 : Dhi[0], 0, 0, 0);
+  Dlo[1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(o.a1, o.bl, FIRST ? zero16 : Dlo[1], 0, 0, 0);
+  Dhi[1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(o.a1, o.bh, FIRST ? zero16 : Dhi[1], 0, 0, 0);
+}
+
+/* The four 32-deep steps of one stage; the operands of step k+1 are read from
+ * LDS while the matrix core works on step k. */
+template <bool FIRST>
+__device__ __forceinline__ void stage_mma(const Smem &sm, int buf, int wm, int wn, int i32, int g,
+                                          v16i (&Dlo)[2], v16i (&Dhi)[2]) {
+  Ops o0, o1;
+  read_ops(o0, sm, buf, 0, wm, wn, i32, g);
+  read_ops(o1, sm, buf, 1, wm, wn, i32, g);
+  __builtin_amdgcn_sched_barrier(0);
+  mma_ops<FIRST>(o0, Dlo, Dhi);
+  __builtin_amdgcn_sched_barrier(0);
+  read_ops(o0, sm, buf, 2, wm, wn, i32, g);
+  __builtin_amdgcn_sched_barrier(0);
+  mma_ops<false>(o1, Dlo, Dhi);
+  __builtin_amdgcn_sched_barrier(0);
+  read_ops(o1, sm, buf, 3, wm, wn, i32, g);
+  __builtin_amdgcn_sched_barrier(0);
+  mma_ops<false>(o0, Dlo, Dhi);
+  __builtin_amdgcn_sched_barrier(0);
+  mma_ops<false>(o1, Dlo, Dhi);
+  __builtin_amdgcn_sched_barrier(0);
 }
 
 struct Ctx {
@@ -283,13 +311,7 @@ __device__ __forceinline__ void super_block(Smem &sm, const Addr &ad, const Ctx 
   const int sb1 = min(sb + 1, nsb - 1), sb2 = min(sb + 2, nsb - 1);
   load_a(as, ad, sb, 1);
   __builtin_amdgcn_sched_barrier(0);
-  kstep<true>(sm, 0, 0, c.wm, c.wn, c.i32, c.g, Dlo, Dhi);
-#pragma unroll
-  for (int ks = 1; ks < 4; ++ks) {
-    __builtin_amdgcn_sched_barrier(0); /* keep the operand reads of later steps from piling up */
-    kstep<false>(sm, 0, ks, c.wm, c.wn, c.i32, c.g, Dlo, Dhi);
-  }
-  __builtin_amdgcn_sched_barrier(0);
+  stage_mma<true>(sm, 0, c.wm, c.wn, c.i32, c.g, Dlo, Dhi);
   store_a(as, sm, 1);
   store_b<1>(bcur, sm);
   sync_lds();
@@ -297,12 +319,7 @@ __device__ __forceinline__ void super_block(Smem &sm, const Addr &ad, const Ctx 
   load_row(rb, ad, sb1);
   load_b(bcur, ad, sb2); /* bcur's registers are free: they become the weights of sb + 2 */
   __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-  for (int ks = 0; ks < 4; ++ks) {
-    __builtin_amdgcn_sched_barrier(0);
-    kstep<false>(sm, 1, ks, c.wm, c.wn, c.i32, c.g, Dlo, Dhi);
-  }
-  __builtin_amdgcn_sched_barrier(0);
+  stage_mma<false>(sm, 1, c.wm, c.wn, c.i32, c.g, Dlo, Dhi);
   epilogue(sm, c, Dlo, Dhi, acc);
   sync_lds(); /* every wavefront is done with stage (sb, 0) and the row/column data */
   __builtin_amdgcn_sched_barrier(0);
