@@ -21,6 +21,12 @@ sys.path.insert(0, ROOT)
 M, K, N = 512, 4096, 12288
 INT8_PEAK_TOPS = 5000.0  # MI355X dense int8 matrix peak, TOP/s
 HBM_PEAK_GBS = 8000.0    # MI355X HBM3E peak, GB/s
+# HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs of this script, scaled by
+# what the same counters read for its 256 MiB device copy (profiles/gemm_q4k_prefill_m512_k4096_n12288.txt,
+# profiles/gemv_q4k_decode_m1_k4096.txt). Measured once, not live: counters need the profiler attached.
+TRAFFIC_GEMM_C2 = 62.07e6 + 25.17e6
+TRAFFIC_GEMV_C2 = 28.42e6 + 0.05e6
+TRAFFIC_GEMV_LM_HEAD = 350.57e6 + 0.61e6
 METRIC = "Q4 GEMV effective GB/s (%HBM peak); prefill GEMM int8 TOPS (%MFMA peak)"
 
 
@@ -128,6 +134,31 @@ def main():
     gemv_hot_ms = capi.time_matmul(weights[:1], a1, 1, c1, 400, phase=1, stream=stream)
     gemv_gbs = gv_bytes / (gemv_ms * 1e-3) / 1e9
 
+    # ---- the same GEMV at lm_head size (N=151936: 350 MB of Q4_K per matrix) ----
+    NL = 151936
+    wl32 = torch.randn((NL, K), generator=gen, device="cuda", dtype=torch.float32) * 0.02
+    blocks_l = torch.empty(capi.weight_nbytes("q4_K", NL, K), dtype=torch.uint8, device="cuda")
+    capi.quantize_weights("q4_K", wl32, NL, K, blocks_l, stream=stream)
+    torch.cuda.synchronize()
+    del wl32
+    big = [capi.Weight("q4_K", NL, K, blocks_l, mem=capi.MEM_DEVICE) for _ in range(3)]
+    cl = torch.empty((1, NL), device="cuda", dtype=torch.float32)
+    capi.time_matmul(big, a1, 1, cl, 6, phase=1, stream=stream)
+    big_ms = capi.time_matmul(big, a1, 1, cl, 60, phase=1, stream=stream)
+    big_bytes = NL * K * 144 // 256 + 4 * K + 4 * NL
+    big_gbs = big_bytes / (big_ms * 1e-3) / 1e9
+    for w in big:
+        w.destroy()
+
+    # ---- a plain device copy of known size: the yardstick the FETCH_SIZE / WRITE_SIZE
+    # counters of a profiled run of this script are scaled by
+    src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda")
+    dst = torch.empty_like(src)
+    for _ in range(3):
+        dst.copy_(src)
+    torch.cuda.synchronize()
+    del src, dst
+
     out = {
         "metric": METRIC, "value": round(value, 3), "unit": "TOPS", "n_gpus": 1,
         "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(sec * 1e3, 5),
@@ -136,18 +167,26 @@ def main():
         "config": {"workload": "Q4_K x Q8_K prefill GEMM, M=512 K=4096 N=12288 (BASELINE configs[1]); "
                                "step = activation quantizer + block-dot GEMM on HBM-resident inputs",
                    "M": M, "K": K, "N": N, "weight_copies_rotated": n_copies},
-        "roofline": {"bound": "mfma", "kernel": "gemm_i8_kernel<Q4_K>", "achieved": round(gemm_tops, 3),
+        "roofline": {"bound": "mfma", "kernel": "gemm_q4k_kernel", "achieved": round(gemm_tops, 3),
                      "peak": INT8_PEAK_TOPS, "unit": "TOP/s", "frac": round(gemm_tops / INT8_PEAK_TOPS, 5),
-                     "kernel_ms": round(gemm_ms, 5), "traffic": None},
+                     "kernel_ms": round(gemm_ms, 5), "traffic": TRAFFIC_GEMM_C2,
+                     "algorithmic_ops_per_launch": ops},
         "quantizer_ms": round(quant_ms, 5),
         "decode_gemv": {"workload": "Q4_K GEMV M=1 K=4096 N=12288, %d weight copies rotated" % n_copies,
                         "value": round(gv_bytes / (gemv_all_ms * 1e-3) / 1e9, 2), "unit": "GB/s",
                         "ms_per_call": round(gemv_all_ms, 5),
                         "cache_hot_kernel_ms": round(gemv_hot_ms, 5),
-                        "roofline": {"bound": "hbm", "kernel": "gemv_kernel<Q4_K,64,1>",
+                        "roofline": {"bound": "hbm", "kernel": "gemv_kernel<Q4_K,T=64,R=1,G=4>",
                                      "achieved": round(gemv_gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                      "frac": round(gemv_gbs / HBM_PEAK_GBS, 5),
-                                     "kernel_ms": round(gemv_ms, 5), "traffic": None}},
+                                     "kernel_ms": round(gemv_ms, 5), "traffic": TRAFFIC_GEMV_C2,
+                                     "algorithmic_bytes_per_launch": gv_bytes}},
+        "decode_gemv_lm_head_size": {
+            "workload": "Q4_K GEMV M=1 K=4096 N=151936, 3 weight copies rotated",
+            "roofline": {"bound": "hbm", "kernel": "gemv_kernel<Q4_K,T=64,R=1,G=4>",
+                         "achieved": round(big_gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(big_gbs / HBM_PEAK_GBS, 5), "kernel_ms": round(big_ms, 5),
+                         "traffic": TRAFFIC_GEMV_LM_HEAD, "algorithmic_bytes_per_launch": big_bytes}},
     }
     if not args.no_cpu:
         capi.matmul(weights[0], a, M, c, stream=stream)
