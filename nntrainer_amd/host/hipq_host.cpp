@@ -1,0 +1,159 @@
+// SPDX-License-Identifier: Apache-2.0
+/**
+ * @file   hipq_host.cpp
+ * @brief  Host core of the HIP plug-in: status -> exception translation, the
+ *         weight cache and thin typed wrappers over the C ABI (see hipq_host.h).
+ */
+#include "hipq_host.h"
+
+#include <atomic>
+#include <sstream>
+
+namespace hipq_host {
+
+void check(int status, const char *what) {
+  if (status == HIPQ_OK)
+    return;
+  std::ostringstream msg;
+  const char *detail = hipq_last_error();
+  msg << "[hipq] " << what << " failed (" << status << ")";
+  if (detail && *detail)
+    msg << ": " << detail;
+  switch (status) {
+  case HIPQ_ERR_INVALID_ARGUMENT:
+    throw std::invalid_argument(msg.str());
+  case HIPQ_ERR_NOT_SUPPORTED:
+    throw not_supported(msg.str());
+  case HIPQ_ERR_OUT_OF_MEMORY:
+    throw std::bad_alloc();
+  default:
+    throw std::runtime_error(msg.str());
+  }
+}
+
+bool runtime_available(int device) noexcept {
+  /* 0 = not tried, 1 = up, 2 = unavailable */
+  static std::atomic<int> state{0};
+  static std::mutex mtx;
+  int s = state.load(std::memory_order_acquire);
+  if (s)
+    return s == 1;
+  std::lock_guard<std::mutex> lock(mtx);
+  s = state.load(std::memory_order_relaxed);
+  if (s)
+    return s == 1;
+  s = hipq_init(device) == HIPQ_OK ? 1 : 2;
+  state.store(s, std::memory_order_release);
+  return s == 1;
+}
+
+WeightCache::~WeightCache() { clear(); }
+
+hipq_weight_t WeightCache::get(const void *host_bytes, const WeightSpec &spec) {
+  if (!host_bytes)
+    throw std::invalid_argument("[hipq] weight tensor has no data");
+  std::lock_guard<std::mutex> lock(mtx);
+  auto it = map.find(host_bytes);
+  if (it != map.end()) {
+    const WeightSpec &o = it->second.spec;
+    if (o.dtype == spec.dtype && o.layout == spec.layout && o.N == spec.N && o.K == spec.K)
+      return it->second.w;
+    /* the allocator handed the address to another tensor: replace */
+    hipq_weight_destroy(it->second.w);
+    map.erase(it);
+  }
+  hipq_weight_t w = nullptr;
+  check(hipq_weight_create(spec.dtype, spec.layout, spec.N, spec.K, host_bytes, HIPQ_MEM_HOST, &w),
+        "hipq_weight_create");
+  map.emplace(host_bytes, Entry{w, spec});
+  return w;
+}
+
+void WeightCache::invalidate(const void *host_bytes) {
+  std::lock_guard<std::mutex> lock(mtx);
+  auto it = map.find(host_bytes);
+  if (it == map.end())
+    return;
+  hipq_weight_destroy(it->second.w);
+  map.erase(it);
+}
+
+void WeightCache::clear() {
+  std::lock_guard<std::mutex> lock(mtx);
+  for (auto &kv : map)
+    hipq_weight_destroy(kv.second.w);
+  map.clear();
+}
+
+size_t WeightCache::size() const {
+  std::lock_guard<std::mutex> lock(mtx);
+  return map.size();
+}
+
+WeightCache &global_cache() {
+  /* never destroyed: contexts live as long as the process
+   * (nntrainer/engine.h:52-57) and the device may be gone at exit */
+  static WeightCache *cache = new WeightCache();
+  return *cache;
+}
+
+static void require_runtime() {
+  if (!runtime_available())
+    throw std::runtime_error(std::string("[hipq] no usable HIP device: ") + hipq_last_error());
+}
+
+void matmul(WeightCache &cache, const void *weight_bytes, const WeightSpec &spec, const float *A,
+            int64_t M, int64_t lda, float *C, int64_t ldc) {
+  require_runtime();
+  hipq_weight_t w = cache.get(weight_bytes, spec);
+  check(hipq_matmul(w, A, M, lda, C, ldc, HIPQ_MEM_HOST, nullptr), "hipq_matmul");
+}
+
+void matmul_multi(WeightCache &cache, const std::vector<const void *> &weight_bytes,
+                  const std::vector<WeightSpec> &specs, const float *A, int64_t M, int64_t lda,
+                  const std::vector<float *> &C) {
+  require_runtime();
+  if (weight_bytes.size() != specs.size() || weight_bytes.size() != C.size() || specs.empty())
+    throw std::invalid_argument("[hipq] matmul_multi: weights, specs and outputs differ in number");
+  std::vector<hipq_weight_t> ws(specs.size());
+  std::vector<int64_t> ldc(specs.size());
+  for (size_t i = 0; i < specs.size(); ++i) {
+    ws[i] = cache.get(weight_bytes[i], specs[i]);
+    ldc[i] = specs[i].N;
+  }
+  check(hipq_matmul_multi((int)ws.size(), ws.data(), A, M, lda, C.data(), ldc.data(), HIPQ_MEM_HOST,
+                          nullptr),
+        "hipq_matmul_multi");
+}
+
+void moe_forward(WeightCache &cache, const MoeShape &shape, int dtype,
+                 const std::vector<const void *> &gate_bytes,
+                 const std::vector<const void *> &up_bytes,
+                 const std::vector<const void *> &down_bytes, const float *x,
+                 const float *router_weight, float *y) {
+  require_runtime();
+  const size_t E = (size_t)shape.experts;
+  if (gate_bytes.size() != E || up_bytes.size() != E || down_bytes.size() != E)
+    throw std::invalid_argument("[hipq] moe_forward: one gate, up and down weight per expert");
+  const int layout = framework_layout(dtype);
+  const WeightSpec gu{dtype, layout, shape.intermediate, shape.hidden};
+  const WeightSpec dn{dtype, layout, shape.hidden, shape.intermediate};
+  std::vector<hipq_weight_t> g(E), u(E), d(E);
+  for (size_t e = 0; e < E; ++e) {
+    g[e] = cache.get(gate_bytes[e], gu);
+    u[e] = cache.get(up_bytes[e], gu);
+    d[e] = cache.get(down_bytes[e], dn);
+  }
+  hipq_moe_desc desc;
+  desc.tokens = shape.tokens;
+  desc.hidden = shape.hidden;
+  desc.intermediate = shape.intermediate;
+  desc.experts = shape.experts;
+  desc.topk = shape.topk;
+  desc.renormalize = shape.renormalize ? 1 : 0;
+  check(hipq_moe_forward(&desc, g.data(), u.data(), d.data(), x, nullptr, router_weight, y, nullptr,
+                         nullptr, HIPQ_MEM_HOST, nullptr),
+        "hipq_moe_forward");
+}
+
+} // namespace hipq_host

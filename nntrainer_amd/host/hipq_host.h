@@ -1,0 +1,129 @@
+// SPDX-License-Identifier: Apache-2.0
+/**
+ * @file   hipq_host.h
+ * @brief  C++ host core between the framework adapters (HipContext, FC and MoE
+ *         layers) and the C ABI of libhipq (include/hipq.h).
+ *
+ * Nothing in here knows the framework's types. It provides
+ *  - the translation of C-ABI status codes into the exceptions the framework
+ *    uses on this path (std::invalid_argument for bad properties and
+ *    dimensions, std::runtime_error for a failed kernel or dispatch,
+ *    cf. nntrainer/tensor/cl_operations/blas_kernels.cpp:246-319, and
+ *    nntrainer::exception::not_supported = a std::invalid_argument,
+ *    nntrainer/nntrainer_error.h:157-159);
+ *  - the device-side cache of weights keyed by the host pointer of the tensor
+ *    the framework owns: layers may not allocate in finalize()
+ *    (nntrainer/layers/layer_devel.h:187-189), so a weight is uploaded and put
+ *    into the device layout the first time a forward call sees it;
+ *  - the quantized matmul and the MoE block on host pointers.
+ */
+#ifndef HIPQ_HOST_H
+#define HIPQ_HOST_H
+
+#include <cstdint>
+#include <mutex>
+#include <stdexcept>
+#include <string>
+#include <unordered_map>
+#include <vector>
+
+#include <hipq.h>
+
+namespace hipq_host {
+
+/** raised for HIPQ_ERR_NOT_SUPPORTED; an invalid_argument like the framework's own */
+struct not_supported : public std::invalid_argument {
+  using std::invalid_argument::invalid_argument;
+};
+
+/** throws the exception that corresponds to a non-zero status code */
+void check(int status, const char *what);
+
+/**
+ * Brings the device up once per process. Never throws: a machine without a
+ * usable GPU leaves the runtime marked unavailable, as ClContext::initialize
+ * does for a missing OpenCL device (nntrainer/cl_context.cpp:70-90).
+ * @return true if kernels can be launched
+ */
+bool runtime_available(int device = 0) noexcept;
+
+/** Layout of weight bytes as the framework hands them over. */
+struct WeightSpec {
+  int dtype;  /**< HIPQ_Q4_0 | HIPQ_Q4_K | HIPQ_Q6_K */
+  int layout; /**< HIPQ_LAYOUT_X8 for Q4_0/Q4_K tensors of a loaded model
+                   (ggml_interface.cpp:109-122), canonical for Q6_K */
+  int64_t N;  /**< output features */
+  int64_t K;  /**< input features  */
+};
+
+/** layout a framework tensor of this dtype uses for its bytes */
+inline int framework_layout(int dtype) {
+  return dtype == HIPQ_Q6_K ? HIPQ_LAYOUT_CANONICAL : HIPQ_LAYOUT_X8;
+}
+
+/**
+ * Device copies of the weights, keyed by the host address of the bytes.
+ * Thread safe: MoE calls its experts from an OpenMP loop
+ * (Applications/CausalLM/layers/qwen_moe_layer.cpp:478-490) and weights are
+ * read by one thread per node at load time (nntrainer/models/neuralnet.cpp:742-751).
+ */
+class WeightCache {
+public:
+  WeightCache() = default;
+  ~WeightCache();
+  WeightCache(const WeightCache &) = delete;
+  WeightCache &operator=(const WeightCache &) = delete;
+
+  /** the device weight for these host bytes; uploads on first use */
+  hipq_weight_t get(const void *host_bytes, const WeightSpec &spec);
+  /** forget (and free) the device copy of a host buffer whose content changed */
+  void invalidate(const void *host_bytes);
+  void clear();
+  size_t size() const;
+
+private:
+  struct Entry {
+    hipq_weight_t w;
+    WeightSpec spec;
+  };
+  mutable std::mutex mtx;
+  std::unordered_map<const void *, Entry> map;
+};
+
+/** process-wide cache used by the layers */
+WeightCache &global_cache();
+
+/**
+ * C[M x N] = A[M x K] * W^T with W given as quantized bytes in host memory;
+ * A and C are host fp32. M == 1 runs the decode GEMV, M > 1 the prefill GEMM,
+ * exactly the dispatch of FloatTensor::dotQnK
+ * (nntrainer/tensor/float_tensor.cpp:923-969).
+ */
+void matmul(WeightCache &cache, const void *weight_bytes, const WeightSpec &spec,
+            const float *A, int64_t M, int64_t lda, float *C, int64_t ldc);
+
+/** one activation against several weights (shared activation quantization),
+ *  the vector overload of dot (float_tensor.cpp:724-798) */
+void matmul_multi(WeightCache &cache, const std::vector<const void *> &weight_bytes,
+                  const std::vector<WeightSpec> &specs, const float *A, int64_t M,
+                  int64_t lda, const std::vector<float *> &C);
+
+struct MoeShape {
+  int tokens, hidden, intermediate, experts, topk;
+  bool renormalize;
+};
+
+/**
+ * The MoE block of qwen_moe_layer.cpp:394-503 on host pointers: router matmul
+ * with the fp32 gate weight [hidden x experts], softmax, top-k, renormalise,
+ * per-expert SwiGLU MLP on quantized weights, combine in ascending expert order.
+ */
+void moe_forward(WeightCache &cache, const MoeShape &shape, int dtype,
+                 const std::vector<const void *> &gate_bytes,
+                 const std::vector<const void *> &up_bytes,
+                 const std::vector<const void *> &down_bytes, const float *x,
+                 const float *router_weight, float *y);
+
+} // namespace hipq_host
+
+#endif /* HIPQ_HOST_H */

@@ -1,0 +1,186 @@
+// SPDX-License-Identifier: Apache-2.0
+/**
+ * @file   moe_layer_hip.cpp
+ * @brief  MoELayerHip (see moe_layer_hip.h).
+ */
+#include "moe_layer_hip.h"
+
+#include "hipq_host.h"
+#include "layer_props.h"
+
+namespace nntrainer {
+
+static constexpr unsigned int SINGLE_INOUT_IDX = 0;
+
+void MoELayerHip::setProperty(const std::vector<std::string> &values) {
+  for (const auto &kv : hipq_host::split_properties(values)) {
+    const std::string &key = kv.first, &val = kv.second;
+    if (key == "num_experts") {
+      num_experts = hipq_host::parse_positive(key, val);
+    } else if (key == "num_experts_per_token") {
+      topk = hipq_host::parse_positive(key, val);
+    } else if (key == "unit") {
+      intermediate = hipq_host::parse_positive(key, val);
+    } else if (key == "moe_activation") {
+      /* the expert MLP is SwiGLU: silu(gate) * up (qwen_moe_layer.cpp:357-372) */
+      const std::string a = hipq_host::lower(val);
+      if (a != "swish" && a != "silu")
+        throw exception::not_supported("MoELayerHip computes the swish activation only, got " + val);
+      activation_set = true;
+    } else if (key == "weight_initializer" || key == "weight_regularizer" ||
+               key == "weight_regularizer_constant" || key == "weight_decay" || key == "print" ||
+               key == "disable_bias" || key == "bias_initializer" || key == "bias_decay") {
+      /* training-time properties of the CPU layer: accepted, without effect on inference */
+    } else {
+      throw std::invalid_argument("Unknown Layer Properties count 1: " + key);
+    }
+  }
+}
+
+void MoELayerHip::finalize(InitLayerContext &context) {
+  NNTR_THROW_IF(context.getNumInputs() != 1, std::invalid_argument)
+    << "MoE layer only supports single input";
+  NNTR_THROW_IF(num_experts == 0 || topk == 0 || intermediate == 0, std::invalid_argument)
+    << "MoE layer needs num_experts, num_experts_per_token and unit";
+  NNTR_THROW_IF(topk > num_experts, std::invalid_argument)
+    << "num_experts_per_token " << topk << " exceeds num_experts " << num_experts;
+  if (!activation_set)
+    throw std::runtime_error("Activation type is not set for MoE layer");
+  if (context.getActivationDataType() != Tdatatype::FP32)
+    throw std::runtime_error("Unsupported activation data type for MoE layer");
+  NNTR_THROW_IF(context.getFormat() != Tformat::NCHW, exception::not_supported)
+    << "MoELayerHip supports the NCHW format only";
+
+  switch (context.getWeightDataType()) {
+  case Tdatatype::Q4_0:
+    weight_dtype = HIPQ_Q4_0;
+    break;
+  case Tdatatype::Q4_K:
+    weight_dtype = HIPQ_Q4_K;
+    break;
+  case Tdatatype::Q6_K:
+    weight_dtype = HIPQ_Q6_K;
+    break;
+  default:
+    throw exception::not_supported("MoELayerHip serves Q4_0, Q4_K and Q6_K expert weights");
+  }
+
+  const auto &in_dim = context.getInputDimensions()[SINGLE_INOUT_IDX];
+  std::vector<TensorDim> output_dims(1);
+  output_dims[SINGLE_INOUT_IDX] = in_dim;
+  context.setOutputDimensions(output_dims);
+
+  hidden = in_dim.width();
+  const unsigned int block = weight_dtype == HIPQ_Q4_0 ? 32 : 256;
+  NNTR_THROW_IF(hidden % block != 0 || intermediate % block != 0, std::invalid_argument)
+    << "hidden " << hidden << " and unit " << intermediate << " must be multiples of the quantization block "
+    << block;
+
+  /* 1. router weight, always fp32 */
+  TensorDim gate_dim(1, 1, hidden, num_experts,
+                     TensorDim::TensorType(context.getFormat(), Tdatatype::FP32), 0b0011);
+  gate_idx = context.requestWeight(gate_dim, Initializer::NONE, WeightRegularizer::NONE, 1.0f, 0.0f,
+                                   "gate", true);
+
+  /* 2. experts, in the order the model file stores them: up, gate, down */
+  expert_gate_proj_indices.clear();
+  expert_up_proj_indices.clear();
+  expert_down_proj_indices.clear();
+  expert_gate_proj_indices.reserve(num_experts);
+  expert_up_proj_indices.reserve(num_experts);
+  expert_down_proj_indices.reserve(num_experts);
+
+  TensorDim expert_gate_dim(1, 1, hidden, intermediate,
+                            TensorDim::TensorType(context.getFormat(), context.getWeightDataType()),
+                            0b0011);
+  TensorDim expert_down_dim(1, 1, intermediate, hidden,
+                            TensorDim::TensorType(context.getFormat(), context.getWeightDataType()),
+                            0b0011);
+  for (unsigned int i = 0; i < num_experts; ++i) {
+    expert_up_proj_indices.push_back(
+      context.requestWeight(expert_gate_dim, Initializer::NONE, WeightRegularizer::NONE, 1.0f, 0.0f,
+                            "expert_up_" + std::to_string(i), false));
+    expert_gate_proj_indices.push_back(
+      context.requestWeight(expert_gate_dim, Initializer::NONE, WeightRegularizer::NONE, 1.0f, 0.0f,
+                            "expert_gate_" + std::to_string(i), false));
+    expert_down_proj_indices.push_back(
+      context.requestWeight(expert_down_dim, Initializer::NONE, WeightRegularizer::NONE, 1.0f, 0.0f,
+                            "expert_down_" + std::to_string(i), false));
+  }
+
+  /* 3. the scratch tensors of the CPU layer, kept so that tensor indices and
+   *    memory planning of a model do not depend on the engine */
+  const unsigned int total_tokens = in_dim.batch() * in_dim.height();
+  router_logits_idx =
+    context.requestTensor({total_tokens, 1, 1, num_experts}, "router_logits", Initializer::NONE, false,
+                          TensorLifespan::FORWARD_FUNC_LIFESPAN);
+  expert_mask_idx =
+    context.requestTensor({num_experts, 1, topk, total_tokens}, "expert_mask", Initializer::ZEROS,
+                          false, TensorLifespan::FORWARD_FUNC_LIFESPAN);
+}
+
+void MoELayerHip::run(RunLayerContext &context, const float *x, float *y, unsigned int tokens,
+                      bool renormalize) const {
+  std::vector<const void *> g(num_experts), u(num_experts), d(num_experts);
+  for (unsigned int e = 0; e < num_experts; ++e) {
+    g[e] = context.getWeight(expert_gate_proj_indices[e]).getData<uint8_t>();
+    u[e] = context.getWeight(expert_up_proj_indices[e]).getData<uint8_t>();
+    d[e] = context.getWeight(expert_down_proj_indices[e]).getData<uint8_t>();
+  }
+  const float *router = context.getWeight(gate_idx).getData<float>();
+  hipq_host::MoeShape shape;
+  shape.tokens = (int)tokens;
+  shape.hidden = (int)hidden;
+  shape.intermediate = (int)intermediate;
+  shape.experts = (int)num_experts;
+  shape.topk = (int)topk;
+  shape.renormalize = renormalize;
+  hipq_host::moe_forward(hipq_host::global_cache(), shape, weight_dtype, g, u, d, x, router, y);
+}
+
+void MoELayerHip::forwarding(RunLayerContext &context, bool training) {
+  NNTR_THROW_IF(training, exception::not_supported) << "MoELayerHip is an inference layer";
+  Tensor &input_ = context.getInput(SINGLE_INOUT_IDX);
+  Tensor &output_ = context.getOutput(SINGLE_INOUT_IDX);
+  const unsigned int total_tokens = input_.batch() * input_.height();
+  /* the whole-tensor path keeps the softmax weights as they are
+   * (qwen_moe_layer.cpp:161-259 does not renormalise) */
+  run(context, input_.getData<float>(), output_.getData<float>(), total_tokens, false);
+}
+
+void MoELayerHip::incremental_forwarding(RunLayerContext &context, unsigned int from,
+                                         unsigned int to, bool training) {
+  NNTR_THROW_IF(training, exception::not_supported) << "MoELayerHip is an inference layer";
+  NNTR_THROW_IF(to <= from, std::invalid_argument)
+    << "incremental step [" << from << ", " << to << ") is empty";
+  Tensor &input_ = context.getInput(SINGLE_INOUT_IDX);
+  Tensor &output_ = context.getOutput(SINGLE_INOUT_IDX);
+  NNTR_THROW_IF(to - from > input_.height(), std::invalid_argument)
+    << "incremental step of " << (to - from) << " rows exceeds the input height " << input_.height();
+
+  TensorDim input_step_dim = input_.getDim();
+  TensorDim output_step_dim = output_.getDim();
+  input_step_dim.batch(1);
+  output_step_dim.batch(1);
+  input_step_dim.height(to - from);
+  output_step_dim.height(to - from);
+
+  /* rows [0, to - from) of every batch entry, as qwen_moe_layer.cpp:417-424 */
+  for (unsigned int b = 0; b < input_.batch(); ++b) {
+    Tensor input =
+      input_.getSharedDataTensor(input_step_dim, b * input_.getDim().getFeatureLen(), true);
+    Tensor output =
+      output_.getSharedDataTensor(output_step_dim, b * output_.getDim().getFeatureLen(), true);
+    run(context, input.getData<float>(), output.getData<float>(), to - from, true);
+  }
+}
+
+void MoELayerHip::calcDerivative(RunLayerContext &) {
+  throw exception::not_supported("MoELayerHip does not support backwarding");
+}
+
+void MoELayerHip::calcGradient(RunLayerContext &) {
+  throw exception::not_supported("MoELayerHip does not support backwarding");
+}
+
+} // namespace nntrainer
