@@ -129,11 +129,10 @@ int multiply(const hipq_weight *w, const QAct &qa, int64_t M, float *C, int64_t 
   /* rows the reference sends through its 4-row GEMM kernel (Q4_K, M > 1) */
   const int pair_rows = (w->dtype == HIPQ_Q4_K && M > 1) ? (int)((M / 4) * 4) : 0;
   if (M <= 8) return hipq::launch_gemv(w, &qa, (int)M, pair_rows, C, ldc, s);
-  if (w->dtype == HIPQ_Q4_K) {
-    static const bool v1 = getenv("HIPQ_GEMM_V1") != nullptr;
-    return v1 ? hipq::launch_gemm(w, &qa, (int)M, C, ldc, s)
-              : hipq::launch_gemm_q4k(w, &qa, (int)M, C, ldc, s);
-  }
+  /* the Q4_K GEMM addresses its planes with 32-bit byte offsets */
+  const bool fits32 = w->N * (w->K / 2) < (int64_t(1) << 32) && M * w->K < (int64_t(1) << 32);
+  if (w->dtype == HIPQ_Q4_K && fits32) return hipq::launch_gemm_q4k(w, &qa, (int)M, C, ldc, s);
+  if (w->dtype == HIPQ_Q4_K) return hipq::launch_gemm(w, &qa, (int)M, C, ldc, s);
   if (w->dtype == HIPQ_Q4_0 && w->K % 256 == 0) return hipq::launch_gemm(w, &qa, (int)M, C, ldc, s);
   for (int64_t r0 = 0; r0 < M; r0 += 8) {
     const int64_t rows = (M - r0) < 8 ? (M - r0) : 8;
