@@ -114,6 +114,15 @@ QAct qact_rows(const QAct &a, int is_k, int64_t r0, int64_t rows) {
   return v;
 }
 
+/* The Q4_K prefill GEMM takes its activations in the tiled form and addresses
+ * the weight planes with 32-bit byte offsets. */
+bool wants_tiled(const hipq_weight *w, int64_t M) {
+  return w->dtype == HIPQ_Q4_K && M > 8 && w->N * (w->K / 2) < (int64_t(1) << 32);
+}
+
+int matmul_tiled(const hipq_weight *w, const float *A, int64_t M, int64_t lda, float *C, int64_t ldc,
+                 hipStream_t s, int phase);
+
 /* Quantize the activations the way the reference does for this weight type. */
 int quantize_for(const hipq_weight *w, const float *A, int64_t M, int64_t lda, const QAct &qa,
                  hipStream_t s) {
@@ -129,9 +138,6 @@ int multiply(const hipq_weight *w, const QAct &qa, int64_t M, float *C, int64_t 
   /* rows the reference sends through its 4-row GEMM kernel (Q4_K, M > 1) */
   const int pair_rows = (w->dtype == HIPQ_Q4_K && M > 1) ? (int)((M / 4) * 4) : 0;
   if (M <= 8) return hipq::launch_gemv(w, &qa, (int)M, pair_rows, C, ldc, s);
-  /* the Q4_K GEMM addresses its planes with 32-bit byte offsets */
-  const bool fits32 = w->N * (w->K / 2) < (int64_t(1) << 32) && M * w->K < (int64_t(1) << 32);
-  if (w->dtype == HIPQ_Q4_K && fits32) return hipq::launch_gemm_q4k(w, &qa, (int)M, C, ldc, s);
   if (w->dtype == HIPQ_Q4_K) return hipq::launch_gemm(w, &qa, (int)M, C, ldc, s);
   if (w->dtype == HIPQ_Q4_0 && w->K % 256 == 0) return hipq::launch_gemm(w, &qa, (int)M, C, ldc, s);
   for (int64_t r0 = 0; r0 < M; r0 += 8) {
@@ -152,9 +158,22 @@ int check_matmul_args(hipq_weight_t w, const float *A, int64_t M, int64_t lda, c
   return HIPQ_OK;
 }
 
+/* phase: 0 quantizer + GEMM, 1 GEMM only (activations from the previous call), 2 quantizer only */
+int matmul_tiled(const hipq_weight *w, const float *A, int64_t M, int64_t lda, float *C, int64_t ldc,
+                 hipStream_t s, int phase) {
+  void *mem = nullptr;
+  int rc = workspace(s, qact_tiled_bytes(M, w->K), &mem);
+  if (rc) return rc;
+  QActTiled qa = qact_tiled_carve(mem, M, w->K);
+  if (phase != 1) rc = hipq::launch_quantize_q8_K_tiled(A, M, w->K, lda, (M / 4) * 4, &qa, s);
+  if (!rc && phase != 2) rc = hipq::launch_gemm_q4k(w, &qa, (int)M, C, ldc, s);
+  return rc;
+}
+
 int matmul_device(hipq_weight_t w, const float *A, int64_t M, int64_t lda, float *C, int64_t ldc,
                   hipStream_t s) {
   if (M == 0) return HIPQ_OK;
+  if (wants_tiled(w, M)) return matmul_tiled(w, A, M, lda, C, ldc, s, 0);
   const int is_k = w->dtype != HIPQ_Q4_0;
   void *mem = nullptr;
   int rc = workspace(s, qact_bytes(is_k, M, w->K), &mem);
@@ -430,8 +449,17 @@ int hipq_matmul_multi(int count, const hipq_weight_t *w, const float *A, int64_t
   /* one quantization per distinct activation format among the weights */
   auto klass = [&](const hipq_weight *x) {
     if (x->dtype == HIPQ_Q4_0) return 0;
+    if (wants_tiled(x, M)) return 3;
     return (x->dtype == HIPQ_Q4_K && M > 1) ? 1 : 2;
   };
+  {
+    bool first = true;
+    for (int i = 0; i < count; ++i)
+      if (klass(w[i]) == 3) {
+        if ((rc = matmul_tiled(w[i], A, M, lda, C[i], ldc[i], s, first ? 0 : 1))) return rc;
+        first = false;
+      }
+  }
   for (int k = 0; k < 3; ++k) {
     int first = -1;
     for (int i = 0; i < count; ++i)
@@ -466,10 +494,17 @@ int hipq_time_matmul(int n_weights, const hipq_weight_t *w, const float *A, int6
   }
   hipStream_t s = (hipStream_t)stream;
   const int is_k = w[0]->dtype != HIPQ_Q4_0;
+  bool tiled = true;
+  for (int i = 0; i < n_weights; ++i) tiled = tiled && wants_tiled(w[i], M);
   void *memp = nullptr;
-  if ((rc = workspace(s, qact_bytes(is_k, M, w[0]->K), &memp))) return rc;
-  QAct qa = qact_carve(is_k, memp, M, w[0]->K);
-  if ((rc = quantize_for(w[0], A, M, lda, qa, s))) return rc;
+  QAct qa{};
+  if (tiled) {
+    if ((rc = matmul_tiled(w[0], A, M, lda, C, ldc, s, 2))) return rc;
+  } else {
+    if ((rc = workspace(s, qact_bytes(is_k, M, w[0]->K), &memp))) return rc;
+    qa = qact_carve(is_k, memp, M, w[0]->K);
+    if ((rc = quantize_for(w[0], A, M, lda, qa, s))) return rc;
+  }
   hipEvent_t e0, e1;
   HIPQ_HIP(hipEventCreate(&e0));
   HIPQ_HIP(hipEventCreate(&e1));
@@ -477,6 +512,10 @@ int hipq_time_matmul(int n_weights, const hipq_weight_t *w, const float *A, int6
   HIPQ_HIP(hipEventRecord(e0, s));
   for (int it = 0; it < iters && !rc; ++it) {
     const hipq_weight *wi = w[it % n_weights];
+    if (tiled) {
+      rc = matmul_tiled(wi, A, M, lda, C, ldc, s, phase);
+      continue;
+    }
     if (phase == 0 || phase == 2) rc = quantize_for(wi, A, M, lda, qa, s);
     if (!rc && (phase == 0 || phase == 1)) rc = multiply(wi, qa, M, C, ldc, s);
   }

@@ -22,14 +22,21 @@
  * result is exact (< 2^24). Per super-block and output the ALU does
  *       acc += dA * (d * float(Dlo + 8*Dhi) - dmin * Im).
  *
- * Tiling. A workgroup (4 wavefronts, 2 x 2) owns a 128 x 128 tile of C.
- * K is walked in stages of 128; per stage the int8 activations and the two
- * digit planes of the weights (expanded from nibbles once per workgroup, on the
- * way from HBM to LDS; HBM only carries the packed 4.5-bit form) sit in LDS,
- * double-buffered, rows padded to 144 bytes so that the 16 lanes of a
- * ds_read_b128 phase hit 16 disjoint 4-bank groups. Each wavefront computes
- * 2 x 2 MFMA tiles (64 x 64). Workgroup ids are mapped so that the M-tiles
- * sharing a weight tile run on the same XCD (same L2).
+ * Tiling. A workgroup (4 wavefronts, 2 x 2) owns a 128 x 64 tile of C, each
+ * wavefront 64 x 32 (2 MFMA tiles x 2 digit chains). K is walked in stages of
+ * 128. Two workgroups share a CU (80 KB of LDS and at most 256 registers each),
+ * so one's matrix phase overlaps the other's expansion and epilogue.
+ *  - Activations come from the quantizer already in operand order, 16 KB per
+ *    128-row stage (hipq_internal.h, QActTiled), and go from HBM/L2 straight
+ *    into LDS with global_load_lds_dwordx4: no registers, no ALU work, and the
+ *    ds_read_b128 of a wavefront covers 1 KB of consecutive LDS.
+ *  - Weights are read as packed nibbles two super-blocks ahead (registers) and
+ *    expanded into the two digit planes once per workgroup on the way to LDS;
+ *    HBM only carries the 4.5-bit form. Plane rows are padded to 144 bytes so
+ *    that the 16 lanes of a ds_read_b128 phase hit 16 disjoint 4-bank groups.
+ *  - The per-row data of a super-block (bsum parts, d) is copied the same way.
+ * Workgroup ids are mapped so that the M-tiles sharing a weight tile run on the
+ * same XCD (same L2).
  */
 #include "gemv_device.h"
 
@@ -43,30 +50,23 @@ typedef unsigned short v2us __attribute__((ext_vector_type(2)));
 
 constexpr int BM = 128, BN = 64, KS = 128;
 constexpr int NT = 256;         /* 4 wavefronts (2 x 2), 64 x 32 outputs each */
-constexpr int STRIDE = KS + 16; /* bytes per staged row */
+constexpr int STRIDE = KS + 16; /* bytes per staged weight row */
+constexpr int ATILE = BM * KS;  /* bytes of one activation stage */
 
 struct Smem {
-  int8_t a[2][BM * STRIDE];
+  int8_t a[2][ATILE]; /* [row/32][k/32][k%32/16][row%32][16] */
   int8_t blo[2][BN * STRIDE];
   int8_t bhi[2][BN * STRIDE];
-  /* per super-block, single-buffered (a barrier separates readers and writer) */
-  _Float16 amin[BM * 16]; /* per row: 8 low parts, 8 high parts of bsum32_j */
-  float dA[BM];
-  uint4 colhd[BN]; /* per column: the super-block header {d, dmin, scales[12]} */
+  /* per super-block, double-buffered */
+  _Float16 amin[2][BM * 16]; /* per row: 8 low parts, 8 high parts of bsum32_j */
+  float dA[2][BM];
+  uint4 colhd[2][BN]; /* per column: the super-block header {d, dmin, scales[12]} */
 };
 static_assert(sizeof(Smem) <= 80 * 1024, "two workgroups per CU must fit the 160 KB LDS");
 
-/* Registers of one workgroup thread between the global loads and the LDS. */
-struct AStage { /* one 128-deep stage of activations: 128 rows x 128 bytes */
-  v4i a0, a1, a2, a3; /* plain vectors: struct copies would stay in scratch memory */
-};
 struct BBlock { /* one super-block of weights: 64 columns x 128 bytes + headers */
   uint4 q0, q1; /* the 16 bytes this thread expands in stage 0 and in stage 1 */
   uint4 hd;
-};
-struct RowBlock { /* per-row data of one super-block (threads 0..127) */
-  uint4 bs0 = {0, 0, 0, 0}, bs1 = {0, 0, 0, 0};
-  float dA = 0.f;
 };
 
 /* per 16-bit half: (two bytes <= 15) * (digit <= 7): no carry between bytes */
@@ -75,79 +75,53 @@ __device__ __forceinline__ uint32_t pk_scale(uint32_t x, uint32_t digit2) {
   return __builtin_bit_cast(uint32_t, r);
 }
 
-/* Per-thread constant parts of the addresses. Rows past the end of the
- * matrices are clamped (their results are never stored), so no load sits under
- * a lane-dependent branch and the hardware counters wait for each one exactly. */
-struct Addr { /* byte offsets from the (uniform) plane pointers; planes are < 4 GiB */
-  const int8_t *q;
+/* 64 lanes x 16 bytes (or x 4 bytes) from global memory to LDS without passing
+ * through registers: lane l's bytes land at lds + l * size. lds is uniform. */
+__device__ __forceinline__ void dma16(const void *gptr_lane, void *lds_wave) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gptr_lane,
+                                   (__attribute__((address_space(3))) void *)lds_wave, 16, 0, 0);
+}
+__device__ __forceinline__ void dma4(const void *gptr_lane, void *lds_wave) {
+  __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)gptr_lane,
+                                   (__attribute__((address_space(3))) void *)lds_wave, 4, 0, 0);
+}
+
+/* Everything a thread needs to find its share of the inputs. */
+struct Src {
+  const int8_t *qt;     /* activation stages of this M-tile, + stage * ATILE, + lane part */
+  const uint16_t *amin; /* + sb * BM * 16 halfs */
+  const float *dAt;     /* + sb * BM */
   const uint8_t *qs, *hdr;
-  const int16_t *bsum;
-  const float *d;
-  uint32_t a[4]; /* + sb * 256 + h * 128 */
-  uint32_t bq;   /* + sb * 128 + h * 64 */
-  uint32_t hd;   /* + sb * 16 */
-  uint32_t bs;   /* + sb * 32 */
-  uint32_t dA;   /* + sb * 4 */
+  uint32_t bq; /* byte offset of this thread's weight bytes, + sb * 128 (+ 64) */
+  uint32_t hd; /* byte offset of its column's headers, + sb * 16 */
+  int wave, lane;
 };
 
-__device__ __forceinline__ Addr make_addr(const WView &w, const QView &qa, int M, int m0, int n0) {
-  const int t = threadIdx.x;
-  const int nsb = w.K >> 8;
-  Addr ad;
-  ad.q = qa.q;
-  ad.qs = w.qs;
-  ad.hdr = w.hdr;
-  ad.bsum = qa.bsum;
-  ad.d = qa.d;
+/* stage s of the activations -> LDS buffer buf: wavefront w copies rows 32w..32w+31 */
+__device__ __forceinline__ void dma_a(const Src &sr, Smem &sm, int s, int buf) {
+  const int8_t *g = sr.qt + (size_t)s * ATILE + sr.wave * 4096 + sr.lane * 16;
+  int8_t *l = sm.a[buf] + sr.wave * 4096;
 #pragma unroll
-  for (int it = 0; it < 4; ++it) {
-    const int idx = it * NT + t;
-    const int row = idx >> 3, c16 = idx & 7;
-    ad.a[it] = (uint32_t)min(m0 + row, M - 1) * (uint32_t)qa.K + c16 * 16;
-  }
-  const uint32_t n = (uint32_t)min(n0 + (t >> 2), w.N - 1);
-  ad.bq = n * (uint32_t)(w.K >> 1) + (t & 3) * 16;
-  ad.hd = n * (uint32_t)nsb * 16;
-  const uint32_t m = (uint32_t)min(m0 + (t & (BM - 1)), M - 1);
-  ad.bs = m * (uint32_t)(qa.K >> 4) * 2;
-  ad.dA = m * (uint32_t)nsb * 4;
-  return ad;
+  for (int c = 0; c < 4; ++c) dma16(g + c * 1024, l + c * 1024);
 }
 
-__device__ __forceinline__ void load_a(AStage &st, const Addr &ad, int sb, int h) {
-  const uint32_t k0 = (uint32_t)(sb * 256 + h * 128);
-  st.a0 = *(const v4i *)(ad.q + (ad.a[0] + k0));
-  st.a1 = *(const v4i *)(ad.q + (ad.a[1] + k0));
-  st.a2 = *(const v4i *)(ad.q + (ad.a[2] + k0));
-  st.a3 = *(const v4i *)(ad.q + (ad.a[3] + k0));
-}
-__device__ __forceinline__ void load_b(BBlock &b, const Addr &ad, int sb) {
-  b.q0 = hipq_ld_stream((const uint4 *)(ad.qs + (ad.bq + (uint32_t)(sb * 128))));
-  b.q1 = hipq_ld_stream((const uint4 *)(ad.qs + (ad.bq + (uint32_t)(sb * 128 + 64))));
-  b.hd = *(const uint4 *)(ad.hdr + (ad.hd + (uint32_t)(sb * 16)));
-}
-__device__ __forceinline__ void load_row(RowBlock &r, const Addr &ad, int sb) {
-  /* whole wavefronts 0 and 1 own the 128 rows; the branch is uniform per wavefront */
-  if (__builtin_amdgcn_readfirstlane((int)threadIdx.x) >= BM) return;
-  const uint4 *bp = (const uint4 *)((const char *)ad.bsum + (ad.bs + (uint32_t)(sb * 32)));
-  r.bs0 = bp[0];
-  r.bs1 = bp[1];
-  r.dA = *(const float *)((const char *)ad.d + (ad.dA + (uint32_t)(sb * 4)));
+/* per-row data of super-block sb -> LDS buffer buf */
+__device__ __forceinline__ void dma_rows(const Src &sr, Smem &sm, int sb, int buf) {
+  dma16((const char *)(sr.amin + (size_t)sb * BM * 16) + sr.wave * 1024 + sr.lane * 16,
+        (char *)sm.amin[buf] + sr.wave * 1024);
+  if (sr.wave < 2) /* uniform per wavefront */
+    dma4(sr.dAt + (size_t)sb * BM + sr.wave * 64 + sr.lane, sm.dA[buf] + sr.wave * 64);
 }
 
-__device__ __forceinline__ void store_a(const AStage &st, Smem &sm, int buf) {
-  const int t = threadIdx.x;
-  /* thread t owns 16 bytes of rows t/8, t/8 + 32, t/8 + 64, t/8 + 96 */
-  int8_t *p = sm.a[buf] + (t >> 3) * STRIDE + (t & 7) * 16;
-  *(v4i *)(p) = st.a0;
-  *(v4i *)(p + 32 * STRIDE) = st.a1;
-  *(v4i *)(p + 64 * STRIDE) = st.a2;
-  *(v4i *)(p + 96 * STRIDE) = st.a3;
+__device__ __forceinline__ void load_b(BBlock &b, const Src &sr, int sb) {
+  b.q0 = hipq_ld_stream((const uint4 *)(sr.qs + (sr.bq + (uint32_t)(sb * 128))));
+  b.q1 = hipq_ld_stream((const uint4 *)(sr.qs + (sr.bq + (uint32_t)(sb * 128 + 64))));
+  b.hd = *(const uint4 *)(sr.hdr + (sr.hd + (uint32_t)(sb * 16)));
 }
 
-/* Expand this thread's 32 weights of stage h into the two digit planes. */
+/* Expand this thread's 32 weights of stage H into the two digit planes. */
 template <int H>
-__device__ __forceinline__ void store_b(const BBlock &b, Smem &sm) {
+__device__ __forceinline__ void store_b(const BBlock &b, Smem &sm, int hdbuf) {
   const int t = threadIdx.x;
   const int row = t >> 2, c16 = t & 3;
   const int p = c16 >> 1, hh = c16 & 1; /* sub-block pair 2*H + p of the super-block */
@@ -165,41 +139,25 @@ __device__ __forceinline__ void store_b(const BBlock &b, Smem &sm) {
                           (q.w >> 4) & HIPQ_M4};
   const int d0 = row * STRIDE + (2 * p) * 32 + hh * 16; /* even sub-block: low nibbles */
   const int d1 = d0 + 32;                               /* odd sub-block: high nibbles */
-  *(uint4 *)(sm.blo[H] + d0) =
-    make_uint4(pk_scale(L[0], lo0), pk_scale(L[1], lo0), pk_scale(L[2], lo0), pk_scale(L[3], lo0));
-  *(uint4 *)(sm.bhi[H] + d0) =
-    make_uint4(pk_scale(L[0], hi0), pk_scale(L[1], hi0), pk_scale(L[2], hi0), pk_scale(L[3], hi0));
-  *(uint4 *)(sm.blo[H] + d1) = make_uint4(pk_scale(Hn[0], lo1), pk_scale(Hn[1], lo1),
-                                          pk_scale(Hn[2], lo1), pk_scale(Hn[3], lo1));
-  *(uint4 *)(sm.bhi[H] + d1) = make_uint4(pk_scale(Hn[0], hi1), pk_scale(Hn[1], hi1),
-                                          pk_scale(Hn[2], hi1), pk_scale(Hn[3], hi1));
-  if (H == 0 && c16 == 0) sm.colhd[row] = hd;
+  auto put = [](int8_t *dst, const uint32_t (&v)[4], uint32_t digit2) {
+    *(v4i *)dst = v4i{(int)pk_scale(v[0], digit2), (int)pk_scale(v[1], digit2),
+                      (int)pk_scale(v[2], digit2), (int)pk_scale(v[3], digit2)};
+  };
+  put(sm.blo[H] + d0, L, lo0);
+  put(sm.bhi[H] + d0, L, hi0);
+  put(sm.blo[H] + d1, Hn, lo1);
+  put(sm.bhi[H] + d1, Hn, hi1);
+  if (H == 0 && c16 == 0)
+    *(v4i *)((int8_t *)sm.colhd[hdbuf] + row * 16) = v4i{(int)hd.x, (int)hd.y, (int)hd.z, (int)hd.w};
 }
 
-__device__ __forceinline__ void store_row(const RowBlock &rb, Smem &sm) {
-  const int t = threadIdx.x;
-  if (__builtin_amdgcn_readfirstlane(t) < BM) {
-    const uint32_t wds[8] = {rb.bs0.x, rb.bs0.y, rb.bs0.z, rb.bs0.w,
-                             rb.bs1.x, rb.bs1.y, rb.bs1.z, rb.bs1.w};
-    v8h vlo, vhi;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const int bs = (int)(int16_t)(wds[j] & 0xffff) + ((int)wds[j] >> 16); /* |bs| <= 4064 */
-      const int l6 = bs & 63;
-      vlo[j] = (_Float16)(float)l6;        /* 0..63 */
-      vhi[j] = (_Float16)(float)(bs - l6); /* multiple of 64, 7 significant bits */
-    }
-    *(v8h *)(sm.amin + t * 16) = vlo;
-    *(v8h *)(sm.amin + t * 16 + 8) = vhi;
-    sm.dA[t] = rb.dA;
-  }
-}
-
-/* Workgroup barrier that only waits for this wavefront's LDS traffic. The
- * generic __syncthreads() also drains the global loads in flight, which would
- * throw away the prefetch of the next stages. */
+/* Workgroup barrier after this wavefront's LDS stores and after all but the
+ * youngest `VM` of its global loads (direct-to-LDS copies included) are done.
+ * The generic __syncthreads() would drain every load in flight and throw away
+ * the prefetch of the weights. */
+template <int VM>
 __device__ __forceinline__ void sync_lds() {
-  asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+  asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)\n\ts_barrier" ::"n"(VM) : "memory");
 }
 
 __device__ __forceinline__ int acc_row(int r, int lane) {
@@ -211,11 +169,11 @@ struct Ops {
   v4i a0, a1, bl, bh;
 };
 __device__ __forceinline__ void read_ops(Ops &o, const Smem &sm, int buf, int ks, int wm, int wn,
-                                         int i32, int g) {
-  const int8_t *pa = sm.a[buf] + (wm * 64 + i32) * STRIDE + ks * 32 + g * 16;
+                                         int lane) {
+  const int8_t *pa = sm.a[buf] + ((wm * 2) * 4 + ks) * 1024 + lane * 16;
   o.a0 = *(const v4i *)pa;
-  o.a1 = *(const v4i *)(pa + 32 * STRIDE);
-  const int off = (wn * 32 + i32) * STRIDE + ks * 32 + g * 16;
+  o.a1 = *(const v4i *)(pa + 4096);
+  const int off = (wn * 32 + (lane & 31)) * STRIDE + ks * 32 + (lane >> 5) * 16;
   o.bl = *(const v4i *)(sm.blo[buf] + off);
   o.bh = *(const v4i *)(sm.bhi[buf] + off);
 }
@@ -231,19 +189,19 @@ __device__ __forceinline__ void mma_ops(const Ops &o, v16i (&Dlo)[2], v16i (&Dhi
 /* The four 32-deep steps of one stage; the operands of step k+1 are read from
  * LDS while the matrix core works on step k. */
 template <bool FIRST>
-__device__ __forceinline__ void stage_mma(const Smem &sm, int buf, int wm, int wn, int i32, int g,
+__device__ __forceinline__ void stage_mma(const Smem &sm, int buf, int wm, int wn, int lane,
                                           v16i (&Dlo)[2], v16i (&Dhi)[2]) {
   Ops o0, o1;
-  read_ops(o0, sm, buf, 0, wm, wn, i32, g);
-  read_ops(o1, sm, buf, 1, wm, wn, i32, g);
+  read_ops(o0, sm, buf, 0, wm, wn, lane);
+  read_ops(o1, sm, buf, 1, wm, wn, lane);
   __builtin_amdgcn_sched_barrier(0);
   mma_ops<FIRST>(o0, Dlo, Dhi);
   __builtin_amdgcn_sched_barrier(0);
-  read_ops(o0, sm, buf, 2, wm, wn, i32, g);
+  read_ops(o0, sm, buf, 2, wm, wn, lane);
   __builtin_amdgcn_sched_barrier(0);
   mma_ops<false>(o1, Dlo, Dhi);
   __builtin_amdgcn_sched_barrier(0);
-  read_ops(o1, sm, buf, 3, wm, wn, i32, g);
+  read_ops(o1, sm, buf, 3, wm, wn, lane);
   __builtin_amdgcn_sched_barrier(0);
   mma_ops<false>(o0, Dlo, Dhi);
   __builtin_amdgcn_sched_barrier(0);
@@ -256,10 +214,14 @@ struct Ctx {
 };
 
 /* acc += dA * (d * (Dlo + 8 Dhi) - dmin * sum_j m_j bsum_j) for one super-block */
-__device__ __forceinline__ void epilogue(const Smem &sm, const Ctx &c, const v16i (&Dlo)[2],
+__device__ __forceinline__ void epilogue(const Smem &sm, int buf, const Ctx &c, const v16i (&Dlo)[2],
                                          const v16i (&Dhi)[2], float (&acc)[2][16]) {
   const v16f zero16f = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-  const uint4 hd = sm.colhd[c.wn * 32 + c.i32];
+  /* every LDS access of this kernel is a plain 4 x int vector: the compiler then
+   * tells them apart from the direct-to-LDS copies in flight instead of waiting
+   * for all of those before each access */
+  const v4i hdv = *(const v4i *)((const int8_t *)sm.colhd[buf] + (c.wn * 32 + c.i32) * 16);
+  const uint4 hd = make_uint4((uint32_t)hdv[0], (uint32_t)hdv[1], (uint32_t)hdv[2], (uint32_t)hdv[3]);
   const float dcol = hipq_h2f((uint16_t)(hd.x & 0xffff));
   const float ndmin = -hipq_h2f((uint16_t)(hd.x >> 16));
   const uint32_t mlo = hd.z & 0x3f3f3f3fu;
@@ -274,12 +236,14 @@ __device__ __forceinline__ void epilogue(const Smem &sm, const Ctx &c, const v16
   for (int tm = 0; tm < 2; ++tm) {
     const int rbase = c.wm * 64 + tm * 32;
     /* lanes 0-31 feed the low parts of bsum, lanes 32-63 the high parts */
-    const v8h amin = *(const v8h *)(sm.amin + (rbase + c.i32) * 16 + c.g * 8);
+    const v8h amin = __builtin_bit_cast(
+      v8h, *(const v4i *)((const int8_t *)sm.amin[buf] + ((rbase + c.i32) * 16 + c.g * 8) * 2));
     const v16f Sm = __builtin_amdgcn_mfma_f32_32x32x16_f16(amin, bmin, zero16f, 0, 0, 0);
 #pragma unroll
     for (int q4 = 0; q4 < 4; ++q4) {
-      const float4 dv = *(const float4 *)(sm.dA + rbase + 8 * q4 + 4 * c.g);
-      const float dA[4] = {dv.x, dv.y, dv.z, dv.w};
+      const v4i dv = *(const v4i *)((const int8_t *)sm.dA[buf] + (rbase + 8 * q4 + 4 * c.g) * 4);
+      const float dA[4] = {__int_as_float(dv[0]), __int_as_float(dv[1]), __int_as_float(dv[2]),
+                           __int_as_float(dv[3])};
 #pragma unroll
       for (int e = 0; e < 4; ++e) {
         const int r = 4 * q4 + e;
@@ -297,41 +261,42 @@ __device__ __forceinline__ void epilogue(const Smem &sm, const Ctx &c, const v16
   }
 }
 
-/* One super-block. On entry LDS holds stage (sb, 0), the row/column data of sb,
- * and registers hold the weights of sb (bcur) and sb+1 (bnext). The order of the
- * global loads matters: the counters retire loads in issue order, so the far
- * prefetch of the weights (from HBM) is issued after the activation loads (L2
- * hits) that are needed first. */
-__device__ __forceinline__ void super_block(Smem &sm, const Addr &ad, const Ctx &c, int sb,
-                                            int nsb, BBlock &bcur, const BBlock &bnext,
-                                            v16i (&Dlo)[2], v16i (&Dhi)[2],
-                                            float (&acc)[2][16]) {
-  AStage as;
-  RowBlock rb;
+/* One super-block sb (eb = sb & 1 selects its row/column data buffers).
+ * On entry LDS holds activation stage (sb, 0) in a[0], the digit planes of
+ * stage (sb, 0) in blo/bhi[0], the row data and headers of sb in buffer eb;
+ * registers hold the packed weights of sb (bcur) and sb + 1 (bnext).
+ * The hardware retires loads in issue order, so each wait names how many
+ * younger loads may stay in flight: the weight prefetch (HBM, two super-blocks
+ * ahead) is always issued after the copies that are needed first. */
+template <int EB>
+__device__ __forceinline__ void super_block(Smem &sm, const Src &sr, const Ctx &c, int sb, int nsb,
+                                            BBlock &bcur, const BBlock &bnext, v16i (&Dlo)[2],
+                                            v16i (&Dhi)[2], float (&acc)[2][16]) {
   const int sb1 = min(sb + 1, nsb - 1), sb2 = min(sb + 2, nsb - 1);
-  load_a(as, ad, sb, 1);
+  dma_rows(sr, sm, sb1, EB ^ 1); /* last read by the epilogue of sb - 1 */
+  dma_a(sr, sm, sb * 2 + 1, 1);  /* last read by the second stage of sb - 1 */
   __builtin_amdgcn_sched_barrier(0);
-  stage_mma<true>(sm, 0, c.wm, c.wn, c.i32, c.g, Dlo, Dhi);
-  store_a(as, sm, 1);
-  store_b<1>(bcur, sm);
-  sync_lds();
-  load_a(as, ad, sb1, 0);
-  load_row(rb, ad, sb1);
-  load_b(bcur, ad, sb2); /* bcur's registers are free: they become the weights of sb + 2 */
+  stage_mma<true>(sm, 0, c.wm, c.wn, c.lane, Dlo, Dhi);
+  store_b<1>(bcur, sm, 0);
+  sync_lds<0>(); /* a[1], the planes of stage 1 and the row data of sb + 1 are in place */
+  /* The compiler guards every LDS store that follows a direct-to-LDS copy with a
+   * wait for all loads in flight, so the stores go where nothing is in flight:
+   * right after the barrier, before the next copies and loads are issued. */
+  store_b<0>(bnext, sm, EB ^ 1); /* planes and headers of stage (sb + 1, 0) */
   __builtin_amdgcn_sched_barrier(0);
-  stage_mma<false>(sm, 1, c.wm, c.wn, c.i32, c.g, Dlo, Dhi);
-  epilogue(sm, c, Dlo, Dhi, acc);
-  sync_lds(); /* every wavefront is done with stage (sb, 0) and the row/column data */
+  dma_a(sr, sm, sb1 * 2, 0);
+  load_b(bcur, sr, sb2); /* bcur's registers are free: they become the weights of sb + 2 */
   __builtin_amdgcn_sched_barrier(0);
-  store_a(as, sm, 0);
-  store_b<0>(bnext, sm);
-  store_row(rb, sm);
-  sync_lds();
+  stage_mma<false>(sm, 1, c.wm, c.wn, c.lane, Dlo, Dhi);
+  epilogue(sm, EB, c, Dlo, Dhi, acc);
+  sync_lds<3>(); /* a[0] has landed; the three weight loads stay in flight */
 }
 
-__global__ __launch_bounds__(NT, 2) void gemm_q4k_kernel(WView w, QView qa, int M, int mtiles,
-                                                         int ntiles, float *__restrict__ C,
-                                                         int64_t ldc) {
+__global__ __launch_bounds__(NT, 2) void gemm_q4k_kernel(WView w, const int8_t *__restrict__ qt,
+                                                         const uint16_t *__restrict__ amin,
+                                                         const float *__restrict__ dAt, int M,
+                                                         int mtiles, int ntiles,
+                                                         float *__restrict__ C, int64_t ldc) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   Smem &sm = *reinterpret_cast<Smem *>(smem_raw);
   /* workgroup id -> tile: the M-tiles of one weight tile share id % 8 (one XCD) */
@@ -340,14 +305,29 @@ __global__ __launch_bounds__(NT, 2) void gemm_q4k_kernel(WView w, QView qa, int 
   const int mt = qd % mtiles, nt = (qd / mtiles) * 8 + xcd;
   if (nt >= ntiles) return; /* uniform per workgroup */
   const int m0 = mt * BM, n0 = nt * BN;
+  const int nsb = w.K >> 8;
   Ctx c;
   c.lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   c.wm = wave >> 1;
   c.wn = wave & 1;
   c.i32 = c.lane & 31;
   c.g = c.lane >> 5;
-  const int nsb = w.K >> 8;
+
+  Src sr;
+  sr.qt = qt + (size_t)mt * (2 * nsb) * ATILE;
+  sr.amin = amin + (size_t)mt * nsb * BM * 16;
+  sr.dAt = dAt + (size_t)mt * nsb * BM;
+  sr.qs = w.qs;
+  sr.hdr = w.hdr;
+  {
+    const int t = threadIdx.x;
+    const uint32_t n = (uint32_t)min(n0 + (t >> 2), w.N - 1); /* columns past N are never stored */
+    sr.bq = n * (uint32_t)(w.K >> 1) + (t & 3) * 16;
+    sr.hd = n * (uint32_t)nsb * 16;
+  }
+  sr.wave = wave;
+  sr.lane = c.lane;
 
   v16i Dlo[2], Dhi[2];
   float acc[2][16];
@@ -356,26 +336,21 @@ __global__ __launch_bounds__(NT, 2) void gemm_q4k_kernel(WView w, QView qa, int 
 #pragma unroll
     for (int r = 0; r < 16; ++r) acc[a][r] = 0.f;
 
-  const Addr ad = make_addr(w, qa, M, m0, n0);
   BBlock b0, b1;
-  {
-    AStage as;
-    RowBlock rb;
-    load_a(as, ad, 0, 0);
-    load_row(rb, ad, 0);
-    load_b(b0, ad, 0);
-    load_b(b1, ad, min(1, nsb - 1));
-    store_a(as, sm, 0);
-    store_b<0>(b0, sm);
-    store_row(rb, sm);
-    sync_lds();
-  }
+  dma_rows(sr, sm, 0, 0);
+  dma_a(sr, sm, 0, 0);
+  load_b(b0, sr, 0);
+  load_b(b1, sr, min(1, nsb - 1));
+  store_b<0>(b0, sm, 0);
+  sync_lds<0>();
+
   int sb = 0;
   for (; sb + 1 < nsb; sb += 2) {
-    super_block(sm, ad, c, sb, nsb, b0, b1, Dlo, Dhi, acc);
-    super_block(sm, ad, c, sb + 1, nsb, b1, b0, Dlo, Dhi, acc);
+    super_block<0>(sm, sr, c, sb, nsb, b0, b1, Dlo, Dhi, acc);
+    super_block<1>(sm, sr, c, sb + 1, nsb, b1, b0, Dlo, Dhi, acc);
   }
-  if (sb < nsb) super_block(sm, ad, c, sb, nsb, b0, b1, Dlo, Dhi, acc);
+  if (sb < nsb) super_block<0>(sm, sr, c, sb, nsb, b0, b1, Dlo, Dhi, acc);
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); /* no copy may outlive the workgroup's LDS */
 
   const int n = n0 + c.wn * 32 + c.i32;
 #pragma unroll
@@ -391,9 +366,11 @@ __global__ __launch_bounds__(NT, 2) void gemm_q4k_kernel(WView w, QView qa, int 
 
 namespace hipq {
 
-int launch_gemm_q4k(const hipq_weight *w, const QAct *qa, int M, float *C, int64_t ldc,
+int launch_gemm_q4k(const hipq_weight *w, const QActTiled *qa, int M, float *C, int64_t ldc,
                     hipStream_t s) {
   const int mtiles = (M + BM - 1) / BM;
+  if (mtiles != qa->mtiles || qa->K != w->K)
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "tiled activations do not match the matmul shape");
   const int ntiles = (int)((w->N + BN - 1) / BN);
   const int ngroups = (ntiles + 7) / 8;
   const unsigned grid = (unsigned)(mtiles * ngroups * 8);
@@ -403,8 +380,8 @@ int launch_gemm_q4k(const hipq_weight *w, const QAct *qa, int M, float *C, int64
                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(Smem)));
     lds_opt_in = true;
   }
-  hipLaunchKernelGGL(gemm_q4k_kernel, dim3(grid), dim3(NT), sizeof(Smem), s, wview(w), qview(*qa),
-                     M, mtiles, ntiles, C, ldc);
+  hipLaunchKernelGGL(gemm_q4k_kernel, dim3(grid), dim3(NT), sizeof(Smem), s, wview(w), qa->qt, qa->amin,
+                     qa->dAt, M, mtiles, ntiles, C, ldc);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
 }

@@ -82,6 +82,26 @@ struct QAct {
 size_t qact_bytes(int dtype_is_k, int64_t M, int64_t K);
 QAct qact_carve(int dtype_is_k, void *mem, int64_t M, int64_t K);
 
+/* ------------------------------------------------------------------------- */
+/* Q8_K activations in the form the Q4_K prefill GEMM copies straight from    */
+/* HBM into LDS, tiled by 128 rows (mt = m / 128, rows padded to 128):         */
+/*   qt   [mt][K/128][16384]: one 128-row x 128-deep stage, laid out as        */
+/*        [m%128/32][k%128/32][k%32/16][m%32][16 bytes], i.e. in the order the  */
+/*        lanes of the 32x32x32 int8 matrix instruction take their operands    */
+/*   amin [mt][K/256][128][16] fp16: per row and super-block the eight         */
+/*        sub-block sums (bsum[2j] + bsum[2j+1]) split into a part in 0..63    */
+/*        (first 8) and a multiple of 64 (last 8), both exact in fp16          */
+/*   dAt  [mt][K/256][128] fp32: the block scales d                            */
+/* ------------------------------------------------------------------------- */
+struct QActTiled {
+  int8_t *qt;
+  uint16_t *amin;
+  float *dAt;
+  int M, K, mtiles;
+};
+size_t qact_tiled_bytes(int64_t M, int64_t K);
+QActTiled qact_tiled_carve(void *mem, int64_t M, int64_t K);
+
 namespace hipq {
 
 /* error plumbing (api.hip) */
@@ -104,6 +124,9 @@ int launch_quantize_q8_0(const float *A, int64_t M, int64_t K, int64_t lda,
 int launch_quantize_q8_K(const float *A, int64_t M, int64_t K, int64_t lda,
                          int64_t mat_rows, const QAct *qa, void *canonical_out,
                          hipStream_t s);
+/* same values, written in the tiled form; rows M .. 128 * mtiles are zero-filled */
+int launch_quantize_q8_K_tiled(const float *A, int64_t M, int64_t K, int64_t lda,
+                               int64_t mat_rows, const QActTiled *qa, hipStream_t s);
 
 /* gemv.hip ---------------------------------------------------------------- */
 /* C[m][n] for m < M <= 8: one pass over the weights, M activation rows.
@@ -115,7 +138,7 @@ int launch_gemv(const hipq_weight *w, const QAct *qa, int M, int pair_rows,
 int launch_gemm(const hipq_weight *w, const QAct *qa, int M, float *C,
                 int64_t ldc, hipStream_t s);
 /* gemm_q4k.hip: Q4_K with the sub-block scales folded into two int8 digit planes */
-int launch_gemm_q4k(const hipq_weight *w, const QAct *qa, int M, float *C,
+int launch_gemm_q4k(const hipq_weight *w, const QActTiled *qa, int M, float *C,
                     int64_t ldc, hipStream_t s);
 
 /* moe.hip ----------------------------------------------------------------- */

@@ -77,18 +77,24 @@ __global__ __launch_bounds__(256) void quantize_q8_0_kernel(
 }
 
 /* ---- Q8_K ---------------------------------------------------------------- */
-template <bool CANONICAL>
+enum { Q8K_PLANES = 0, Q8K_CANONICAL = 1, Q8K_TILED = 2 };
+
+/* One wavefront per (row, super-block). In the tiled mode the grid also covers
+ * the padding rows M .. n_sb_total / nsb - 1, which are written as zeros. */
+template <int MODE>
 __global__ __launch_bounds__(256) void quantize_q8_K_kernel(
-  const float *__restrict__ A, int64_t n_sb_total, int nsb, int64_t lda,
+  const float *__restrict__ A, int64_t M, int64_t n_sb_total, int nsb, int64_t lda,
   int64_t mat_rows, int8_t *__restrict__ q_out, float *__restrict__ d_out,
-  int16_t *__restrict__ bsum_out, uint8_t *__restrict__ canon_out) {
+  int16_t *__restrict__ bsum_out, uint8_t *__restrict__ canon_out,
+  uint16_t *__restrict__ amin_out) {
   const int lane = threadIdx.x & 63;
   int64_t sb = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   const bool live = sb < n_sb_total; /* uniform per wavefront */
   if (!live) return;
   const int64_t m = sb / nsb;
   const int b = (int)(sb - m * nsb);
-  const float4 xv = *(const float4 *)(A + m * lda + (int64_t)b * 256 + lane * 4);
+  float4 xv = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (m < M) xv = *(const float4 *)(A + m * lda + (int64_t)b * 256 + lane * 4);
   const float x[4] = {xv.x, xv.y, xv.z, xv.w};
 
   float amax = fmaxf(fmaxf(fabsf(x[0]), fabsf(x[1])), fmaxf(fabsf(x[2]), fabsf(x[3])));
@@ -134,11 +140,28 @@ __global__ __launch_bounds__(256) void quantize_q8_K_kernel(
   int gsum = q[0] + q[1] + q[2] + q[3];
   gsum = hipq_group_sum_i<4>(gsum); /* 4 lanes = one 16-value group */
 
-  if (CANONICAL) {
+  if (MODE == Q8K_CANONICAL) {
     uint8_t *o = canon_out + sb * 292;
     if (lane == 0) *(float *)o = d;
     *(int *)(o + 4 + lane * 4) = packed;
     if ((lane & 3) == 0) *(int16_t *)(o + 260 + (lane >> 2) * 2) = (int16_t)gsum;
+  } else if (MODE == Q8K_TILED) {
+    const int64_t mt = m >> 7;
+    const int r = (int)(m & 127);
+    /* lane holds elements 4*lane .. 4*lane+3 of the super-block */
+    const int stage = b * 2 + (lane >> 5);
+    const int kk = (lane * 4) & 127;
+    const int64_t tile = (mt * (2 * nsb) + stage) * 16384;
+    const int off = (((r >> 5) * 4 + (kk >> 5)) * 2 + ((kk >> 4) & 1)) * 512 + (r & 31) * 16 + (kk & 15);
+    *(int *)(q_out + tile + off) = packed;
+    const int64_t rb = (mt * nsb + b) * 128 + r;
+    if (lane == 0) d_out[rb] = d;
+    const int bs = gsum + __shfl_xor(gsum, 4, HIPQ_WAVE); /* two 16-value groups = one sub-block */
+    if ((lane & 7) == 0) {
+      const int l6 = bs & 63;
+      amin_out[rb * 16 + (lane >> 3)] = __half_as_ushort(__float2half_rn((float)l6));
+      amin_out[rb * 16 + 8 + (lane >> 3)] = __half_as_ushort(__float2half_rn((float)(bs - l6)));
+    }
   } else {
     *(int *)(q_out + sb * 256 + lane * 4) = packed;
     if (lane == 0) d_out[sb] = d;
@@ -181,11 +204,26 @@ int launch_quantize_q8_K(const float *A, int64_t M, int64_t K, int64_t lda,
   const int64_t total = M * nsb;
   const unsigned grid = (unsigned)((total + 3) / 4);
   if (canonical_out)
-    hipLaunchKernelGGL(quantize_q8_K_kernel<true>, dim3(grid), dim3(256), 0, s, A, total, nsb, lda,
-                       mat_rows, nullptr, nullptr, nullptr, (uint8_t *)canonical_out);
+    hipLaunchKernelGGL(quantize_q8_K_kernel<Q8K_CANONICAL>, dim3(grid), dim3(256), 0, s, A, M, total,
+                       nsb, lda, mat_rows, nullptr, nullptr, nullptr, (uint8_t *)canonical_out, nullptr);
   else
-    hipLaunchKernelGGL(quantize_q8_K_kernel<false>, dim3(grid), dim3(256), 0, s, A, total, nsb, lda,
-                       mat_rows, qa->q, qa->d, qa->bsum, nullptr);
+    hipLaunchKernelGGL(quantize_q8_K_kernel<Q8K_PLANES>, dim3(grid), dim3(256), 0, s, A, M, total, nsb,
+                       lda, mat_rows, qa->q, qa->d, qa->bsum, nullptr, nullptr);
+  HIPQ_HIP(hipGetLastError());
+  return HIPQ_OK;
+}
+
+int launch_quantize_q8_K_tiled(const float *A, int64_t M, int64_t K, int64_t lda, int64_t mat_rows,
+                               const QActTiled *qa, hipStream_t s) {
+  if (M <= 0) return HIPQ_OK;
+  if (K % 256 || lda < K) return fail(HIPQ_ERR_INVALID_ARGUMENT, "Q8_K: K=%lld must be a multiple of 256 and lda >= K", (long long)K);
+  if (((uintptr_t)A & 15) || (lda & 3))
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "activation rows must be 16-byte aligned");
+  const int nsb = (int)(K / 256);
+  const int64_t total = (int64_t)qa->mtiles * 128 * nsb;
+  const unsigned grid = (unsigned)((total + 3) / 4);
+  hipLaunchKernelGGL(quantize_q8_K_kernel<Q8K_TILED>, dim3(grid), dim3(256), 0, s, A, M, total, nsb, lda,
+                     mat_rows, qa->qt, qa->dAt, nullptr, nullptr, qa->amin);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
 }
@@ -202,6 +240,26 @@ size_t qact_bytes(int is_k, int64_t M, int64_t K) {
   }
   size_t meta = ((size_t)M * (K / 32) * 4 + 255) & ~(size_t)255;
   return q + meta;
+}
+
+size_t qact_tiled_bytes(int64_t M, int64_t K) {
+  const size_t mpad = (size_t)((M + 127) / 128) * 128, nsb = (size_t)(K / 256);
+  return mpad * K + mpad * nsb * 32 + mpad * nsb * 4; /* each a multiple of 256 */
+}
+
+QActTiled qact_tiled_carve(void *mem, int64_t M, int64_t K) {
+  QActTiled a;
+  const size_t mpad = (size_t)((M + 127) / 128) * 128, nsb = (size_t)(K / 256);
+  uint8_t *p = (uint8_t *)mem;
+  a.M = (int)M;
+  a.K = (int)K;
+  a.mtiles = (int)(mpad / 128);
+  a.qt = (int8_t *)p;
+  p += mpad * K;
+  a.amin = (uint16_t *)p;
+  p += mpad * nsb * 32;
+  a.dAt = (float *)p;
+  return a;
 }
 
 QAct qact_carve(int is_k, void *mem, int64_t M, int64_t K) {
