@@ -107,6 +107,8 @@ QAct qact_rows(const QAct &a, int is_k, int64_t r0, int64_t rows) {
   if (is_k) {
     v.d = a.d + r0 * (a.K / 256);
     v.bsum = a.bsum + r0 * (a.K / 16);
+    v.ql = a.ql + r0 * (a.K / 2);
+    v.qh = a.qh + r0 * (a.K / 2);
   } else {
     v.meta = a.meta + r0 * (a.K / 32);
   }
@@ -138,7 +140,6 @@ int multiply(const hipq_weight *w, const QAct &qa, int64_t M, float *C, int64_t 
   /* rows the reference sends through its 4-row GEMM kernel (Q4_K, M > 1) */
   const int pair_rows = (w->dtype == HIPQ_Q4_K && M > 1) ? (int)((M / 4) * 4) : 0;
   if (M <= 8) return hipq::launch_gemv(w, &qa, (int)M, pair_rows, C, ldc, s);
-  if (w->dtype == HIPQ_Q4_K) return hipq::launch_gemm(w, &qa, (int)M, C, ldc, s);
   if (w->dtype == HIPQ_Q4_0 && w->K % 256 == 0) return hipq::launch_gemm(w, &qa, (int)M, C, ldc, s);
   for (int64_t r0 = 0; r0 < M; r0 += 8) {
     const int64_t rows = (M - r0) < 8 ? (M - r0) : 8;

@@ -1,14 +1,13 @@
 // SPDX-License-Identifier: Apache-2.0
 /**
  * @file   gemm.hip
- * @brief  Prefill GEMM (M > 8) for Q4_0 x Q8_0 and Q4_K x Q8_K on gfx950 int8
- *         matrix cores.
+ * @brief  Prefill GEMM (M > 8) for Q4_0 x Q8_0 on gfx950 int8 matrix cores.
+ *         (Q4_K x Q8_K has its own kernel, gemm_q4k.hip.)
  *
- * Replaces the M > 1 branches of __ggml_q4_0_8x8_q8_0_GEMM and
- * __ggml_q4_K_8x8_q8_K_GEMM (nntrainer/tensor/cpu_backend/ggml_interface/
- * ggml_interface_omp.cpp:330-389, 432-486 in the reference checkout) and the
- * nntr_gemm_q4_0_8x8_q8_0 / nntr_gemm_q4_K_8x8_q8_K kernels behind them
- * (nntr_ggml_impl/nntr_ggml_impl.cpp:650-3259, 3261-7078).
+ * Replaces the M > 1 branch of __ggml_q4_0_8x8_q8_0_GEMM
+ * (nntrainer/tensor/cpu_backend/ggml_interface/ggml_interface_omp.cpp:330-389 in
+ * the reference checkout) and the nntr_gemm_q4_0_8x8_q8_0 kernel behind it
+ * (nntr_ggml_impl/nntr_ggml_impl.cpp:650-3259).
  *
  * Structure. A workgroup (4 wavefronts, 2 x 2) owns a 128 x 128 tile of C and
  * walks K in chunks of 256. Per chunk it stages into LDS
@@ -17,12 +16,9 @@
  *     registers on the way from HBM to LDS, so HBM only ever carries the packed
  *     4.5-bit form,
  * then every wavefront runs v_mfma_i32_32x32x32_i8 over its 64 x 64 quadrant,
- * one instruction per 32-deep quantization group, so each instruction's int32
- * result is exactly the group's dot product. The per-group scale epilogue runs
- * on the vector ALU:
- *   Q4_K: I += sc_j * dot_j (int32, exact), and per 256-value super-block
- *         acc += dA * (d * float(I) - dmin * float(sum_j m_j * bsum_j));
- *   Q4_0: acc += float(dot) * (dw * da) per 32-value block.
+ * one instruction per 32-value block, so each instruction's int32 result is
+ * exactly the block's dot product. The per-block scale epilogue runs on the
+ * vector ALU: acc += float(dot) * (dw * da).
  * In the MFMA result layout a lane holds one column n and 16 rows m, so the
  * weight-side scales are per-lane registers and the activation-side scales are
  * broadcast reads from LDS.
@@ -36,17 +32,10 @@ namespace {
 
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
-typedef short v2s __attribute__((ext_vector_type(2)));
 
 constexpr int BM = 128, BN = 128, KC = 256;
 constexpr int LDS_STRIDE = KC + 16; /* bytes per staged row */
 
-struct SmemQ4K {
-  int8_t a[BM * LDS_STRIDE];
-  int8_t b[BN * LDS_STRIDE];
-  float dA[BM];
-  int bs[BM * 4]; /* per row: 4 x (bsum32[2p] | bsum32[2p+1] << 16) */
-};
 struct SmemQ40 {
   int8_t a[BM * LDS_STRIDE];
   int8_t b[BN * LDS_STRIDE];
@@ -86,12 +75,7 @@ __device__ __forceinline__ void stage_b(int8_t *sb, const WView &w, int n0, int 
     uint4 lo = make_uint4(q.x & HIPQ_M4, q.y & HIPQ_M4, q.z & HIPQ_M4, q.w & HIPQ_M4);
     uint4 hi = make_uint4((q.x >> 4) & HIPQ_M4, (q.y >> 4) & HIPQ_M4, (q.z >> 4) & HIPQ_M4,
                           (q.w >> 4) & HIPQ_M4);
-    if (DT == HIPQ_Q4_K) {
-      /* 16 bytes = elements c*64 + h*16 .. (low nibbles) and +32 (high) */
-      int8_t *dst = sb + row * LDS_STRIDE + (c16 >> 1) * 64 + (c16 & 1) * 16;
-      *(uint4 *)dst = lo;
-      *(uint4 *)(dst + 32) = hi;
-    } else {
+    {
       /* one 32-value block: low nibbles = elements 0..15, high = 16..31 */
       if (live) {
         lo = make_uint4(nib_to_s8(lo.x), nib_to_s8(lo.y), nib_to_s8(lo.z), nib_to_s8(lo.w));
@@ -137,105 +121,7 @@ __global__ __launch_bounds__(256) void gemm_i8_kernel(WView w, QView qa, int M,
   }
   const v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 
-  if (DT == HIPQ_Q4_K) {
-    SmemQ4K &sm = *reinterpret_cast<SmemQ4K *>(smem_raw);
-    const int nsb = w.K >> 8;
-    for (int kc = 0; kc < nchunks; ++kc) {
-      stage_a(sm.a, qa, M, m0, kc);
-      stage_b<HIPQ_Q4_K>(sm.b, w, n0, kc);
-      if (threadIdx.x < BM) {
-        const int row = threadIdx.x;
-        sm.dA[row] = (m0 + row < M) ? qa.d[(size_t)(m0 + row) * nsb + kc] : 0.f;
-      } else {
-        const int row = threadIdx.x - BM;
-        int p[4] = {0, 0, 0, 0};
-        if (m0 + row < M) {
-          const uint4 *bp =
-            (const uint4 *)(qa.bsum + (size_t)(m0 + row) * (qa.K >> 4) + (size_t)kc * 16);
-          const uint4 b0 = bp[0], b1 = bp[1];
-          const uint32_t wds[8] = {b0.x, b0.y, b0.z, b0.w, b1.x, b1.y, b1.z, b1.w};
-          int s32[8];
-#pragma unroll
-          for (int j = 0; j < 8; ++j)
-            s32[j] = (int)(int16_t)(wds[j] & 0xffff) + ((int)wds[j] >> 16);
-#pragma unroll
-          for (int k = 0; k < 4; ++k) p[k] = (s32[2 * k] & 0xffff) | (s32[2 * k + 1] << 16);
-        }
-        *(int4 *)(sm.bs + row * 4) = make_int4(p[0], p[1], p[2], p[3]);
-      }
-      /* weight-side scales of this lane's two columns */
-      float dcol[2], dmincol[2];
-      uint32_t sc4[2][2];
-      int mpair[2][4];
-#pragma unroll
-      for (int tn = 0; tn < 2; ++tn) {
-        const uint4 hd = *((const uint4 *)w.hdr + (size_t)ncol[tn] * nsb + kc);
-        dcol[tn] = hipq_h2f((uint16_t)(hd.x & 0xffff));
-        dmincol[tn] = hipq_h2f((uint16_t)(hd.x >> 16));
-        sc4[tn][0] = hd.y & 0x3f3f3f3fu;
-        sc4[tn][1] = (hd.w & 0x0f0f0f0fu) | (((hd.y >> 6) & 0x03030303u) << 4);
-        const uint32_t mlo = hd.z & 0x3f3f3f3fu;
-        const uint32_t mhi = ((hd.w >> 4) & 0x0f0f0f0fu) | (((hd.z >> 6) & 0x03030303u) << 4);
-        mpair[tn][0] = (int)((mlo & 0xff) | (((mlo >> 8) & 0xff) << 16));
-        mpair[tn][1] = (int)(((mlo >> 16) & 0xff) | ((mlo >> 24) << 16));
-        mpair[tn][2] = (int)((mhi & 0xff) | (((mhi >> 8) & 0xff) << 16));
-        mpair[tn][3] = (int)(((mhi >> 16) & 0xff) | ((mhi >> 24) << 16));
-      }
-      __syncthreads();
-
-      int I[2][2][16];
-#pragma unroll
-      for (int i = 0; i < 2; ++i)
-#pragma unroll
-        for (int j = 0; j < 2; ++j)
-#pragma unroll
-          for (int r = 0; r < 16; ++r) I[i][j][r] = 0;
-
-#pragma unroll 1
-      for (int j = 0; j < 8; ++j) {
-        v4i a[2], b[2];
-#pragma unroll
-        for (int t = 0; t < 2; ++t) {
-          a[t] = *(const v4i *)(sm.a + (wm * 64 + t * 32 + l32) * LDS_STRIDE + j * 32 + kg * 16);
-          b[t] = *(const v4i *)(sm.b + (wn * 64 + t * 32 + l32) * LDS_STRIDE + j * 32 + kg * 16);
-        }
-#pragma unroll
-        for (int tm = 0; tm < 2; ++tm)
-#pragma unroll
-          for (int tn = 0; tn < 2; ++tn) {
-            const v16i dot = __builtin_amdgcn_mfma_i32_32x32x32_i8(a[tm], b[tn], zero16, 0, 0, 0);
-            const uint32_t scw = (j < 4) ? sc4[tn][0] : sc4[tn][1];
-            const int sc = (int)((scw >> (8 * (j & 3))) & 0xff);
-#pragma unroll
-            for (int r = 0; r < 16; ++r) I[tm][tn][r] += __mul24(dot[r], sc);
-          }
-      }
-      /* per super-block fp32 epilogue */
-#pragma unroll
-      for (int tm = 0; tm < 2; ++tm)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int row = wm * 64 + tm * 32 + acc_row(r, lane);
-          const float dA = sm.dA[row];
-          const int4 bs = *(const int4 *)(sm.bs + row * 4);
-#pragma unroll
-          for (int tn = 0; tn < 2; ++tn) {
-            int Im = __builtin_amdgcn_sdot2(__builtin_bit_cast(v2s, mpair[tn][0]),
-                                            __builtin_bit_cast(v2s, bs.x), 0, false);
-            Im = __builtin_amdgcn_sdot2(__builtin_bit_cast(v2s, mpair[tn][1]),
-                                        __builtin_bit_cast(v2s, bs.y), Im, false);
-            Im = __builtin_amdgcn_sdot2(__builtin_bit_cast(v2s, mpair[tn][2]),
-                                        __builtin_bit_cast(v2s, bs.z), Im, false);
-            Im = __builtin_amdgcn_sdot2(__builtin_bit_cast(v2s, mpair[tn][3]),
-                                        __builtin_bit_cast(v2s, bs.w), Im, false);
-            float t = dcol[tn] * (float)I[tm][tn][r];
-            t = fmaf(-dmincol[tn], (float)Im, t);
-            accf[tm][tn][r] = fmaf(dA, t, accf[tm][tn][r]);
-          }
-        }
-      __syncthreads();
-    }
-  } else {
+  {
     SmemQ40 &sm = *reinterpret_cast<SmemQ40 *>(smem_raw);
     const int nb = w.K >> 5;
     for (int kc = 0; kc < nchunks; ++kc) {
@@ -318,16 +204,11 @@ int launch_gemm(const hipq_weight *w, const QAct *qa, int M, float *C, int64_t l
   /* the staged tiles need more than the default 64 KB of dynamic LDS */
   static bool lds_opt_in = false;
   if (!lds_opt_in) {
-    HIPQ_HIP(hipFuncSetAttribute((const void *)gemm_i8_kernel<HIPQ_Q4_K>,
-                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(SmemQ4K)));
     HIPQ_HIP(hipFuncSetAttribute((const void *)gemm_i8_kernel<HIPQ_Q4_0>,
                                  hipFuncAttributeMaxDynamicSharedMemorySize, (int)sizeof(SmemQ40)));
     lds_opt_in = true;
   }
-  if (w->dtype == HIPQ_Q4_K) {
-    hipLaunchKernelGGL(gemm_i8_kernel<HIPQ_Q4_K>, grid, dim3(256), sizeof(SmemQ4K), s, wview(w),
-                       qview(*qa), M, C, ldc);
-  } else if (w->dtype == HIPQ_Q4_0) {
+  if (w->dtype == HIPQ_Q4_0) {
     hipLaunchKernelGGL(gemm_i8_kernel<HIPQ_Q4_0>, grid, dim3(256), sizeof(SmemQ40), s, wview(w),
                        qview(*qa), M, C, ldc);
   } else {

@@ -119,35 +119,36 @@ __device__ __forceinline__ void load_b(BBlock &b, const Src &sr, int sb) {
   b.hd = *(const uint4 *)(sr.hdr + (sr.hd + (uint32_t)(sb * 16)));
 }
 
-/* Expand this thread's 32 weights of stage H into the two digit planes. */
+/* Expand this thread's 32 weights of stage H into the two digit planes. Its 16
+ * bytes are ONE sub-block (weight 2i / 2i+1 in the low / high nibble of byte i),
+ * i.e. one 32-deep matrix step of its column: the even weights become the 16
+ * operand bytes of lanes 0-31 of that step, the odd ones those of lanes 32-63
+ * (the quantizer lays the activations out the same way). */
 template <int H>
 __device__ __forceinline__ void store_b(const BBlock &b, Smem &sm, int hdbuf) {
   const int t = threadIdx.x;
-  const int row = t >> 2, c16 = t & 3;
-  const int p = c16 >> 1, hh = c16 & 1; /* sub-block pair 2*H + p of the super-block */
+  const int row = t >> 2, ks = t & 3; /* sub-block 4*H + ks of the super-block */
   const uint4 hd = b.hd;
-  const int sh = 16 * p;
-  const uint32_t y = hd.y >> sh, ww = hd.w >> sh;
-  /* scales of sub-blocks 4..7 are spread over two header words */
-  const uint32_t scw = H == 0 ? (y & 0x3f3fu) : ((ww & 0x0f0fu) | (((y >> 6) & 0x0303u) << 4));
-  const uint32_t sc0 = scw & 0xff, sc1 = scw >> 8;
-  const uint32_t lo0 = (sc0 & 7) * 0x00010001u, hi0 = (sc0 >> 3) * 0x00010001u;
-  const uint32_t lo1 = (sc1 & 7) * 0x00010001u, hi1 = (sc1 >> 3) * 0x00010001u;
+  /* 6-bit scale of sub-block j: byte j of y for j < 4, else low nibble of byte
+   * j of w and bits 6-7 of byte j-4 of y */
+  const int sh = 8 * ks;
+  const uint32_t sc = H == 0 ? ((hd.y >> sh) & 0x3fu)
+                             : (((hd.w >> sh) & 0x0fu) | (((hd.y >> (sh + 6)) & 0x03u) << 4));
+  const uint32_t lo = (sc & 7) * 0x00010001u, hi = (sc >> 3) * 0x00010001u;
   const uint4 q = H == 0 ? b.q0 : b.q1;
-  const uint32_t L[4] = {q.x & HIPQ_M4, q.y & HIPQ_M4, q.z & HIPQ_M4, q.w & HIPQ_M4};
-  const uint32_t Hn[4] = {(q.x >> 4) & HIPQ_M4, (q.y >> 4) & HIPQ_M4, (q.z >> 4) & HIPQ_M4,
-                          (q.w >> 4) & HIPQ_M4};
-  const int d0 = row * STRIDE + (2 * p) * 32 + hh * 16; /* even sub-block: low nibbles */
-  const int d1 = d0 + 32;                               /* odd sub-block: high nibbles */
+  const uint32_t E[4] = {q.x & HIPQ_M4, q.y & HIPQ_M4, q.z & HIPQ_M4, q.w & HIPQ_M4};
+  const uint32_t O[4] = {(q.x >> 4) & HIPQ_M4, (q.y >> 4) & HIPQ_M4, (q.z >> 4) & HIPQ_M4,
+                         (q.w >> 4) & HIPQ_M4};
+  const int d0 = row * STRIDE + ks * 32; /* even weights; the odd ones 16 bytes on */
   auto put = [](int8_t *dst, const uint32_t (&v)[4], uint32_t digit2) {
     *(v4i *)dst = v4i{(int)pk_scale(v[0], digit2), (int)pk_scale(v[1], digit2),
                       (int)pk_scale(v[2], digit2), (int)pk_scale(v[3], digit2)};
   };
-  put(sm.blo[H] + d0, L, lo0);
-  put(sm.bhi[H] + d0, L, hi0);
-  put(sm.blo[H] + d1, Hn, lo1);
-  put(sm.bhi[H] + d1, Hn, hi1);
-  if (H == 0 && c16 == 0)
+  put(sm.blo[H] + d0, E, lo);
+  put(sm.bhi[H] + d0, E, hi);
+  put(sm.blo[H] + d0 + 16, O, lo);
+  put(sm.bhi[H] + d0 + 16, O, hi);
+  if (H == 0 && ks == 0)
     *(v4i *)((int8_t *)sm.colhd[hdbuf] + row * 16) = v4i{(int)hd.x, (int)hd.y, (int)hd.z, (int)hd.w};
 }
 

@@ -47,6 +47,7 @@ struct QView {
   const uint32_t *meta;
   const float *d;
   const int16_t *bsum;
+  const uint8_t *ql, *qh; /* Q8_K as 4-bit digits: q = 16 * (qh - 8) + ql */
   int K;
 };
 static inline QView qview(const QAct &a) {
@@ -55,8 +56,30 @@ static inline QView qview(const QAct &a) {
   v.meta = a.meta;
   v.d = a.d;
   v.bsum = a.bsum;
+  v.ql = a.ql;
+  v.qh = a.qh;
   v.K = a.K;
   return v;
+}
+
+/* Exact dot product of one Q4_K sub-block (32 unsigned 4-bit weights, eight per
+ * dword) with 32 int8 activations given as 4-bit digits lo in 0..15 and
+ * hi = (q >> 4) + 8 in 0..15:  sum w*q = 16*sum w*hi + sum w*lo - 128*sum w.
+ * Three v_dot8_u32_u4 per eight weights and no nibble unpacking. */
+__device__ __forceinline__ int hipq_dot32_u4(const uint4 &w, const uint4 &lo, const uint4 &hi) {
+  uint32_t l = __builtin_amdgcn_udot8(w.x, lo.x, 0u, false);
+  uint32_t h = __builtin_amdgcn_udot8(w.x, hi.x, 0u, false);
+  uint32_t s = __builtin_amdgcn_udot8(w.x, 0x11111111u, 0u, false);
+  l = __builtin_amdgcn_udot8(w.y, lo.y, l, false);
+  h = __builtin_amdgcn_udot8(w.y, hi.y, h, false);
+  s = __builtin_amdgcn_udot8(w.y, 0x11111111u, s, false);
+  l = __builtin_amdgcn_udot8(w.z, lo.z, l, false);
+  h = __builtin_amdgcn_udot8(w.z, hi.z, h, false);
+  s = __builtin_amdgcn_udot8(w.z, 0x11111111u, s, false);
+  l = __builtin_amdgcn_udot8(w.w, lo.w, l, false);
+  h = __builtin_amdgcn_udot8(w.w, hi.w, h, false);
+  s = __builtin_amdgcn_udot8(w.w, 0x11111111u, s, false);
+  return (int)((h << 4) + l) - (int)(s << 7);
 }
 
 __device__ __forceinline__ int hipq_dot16(const uint32_t (&w)[4], const int4 &a) {
@@ -170,14 +193,15 @@ template <int T, int R, bool PW> struct GemvQ40 {
 };
 
 /* ---- Q4_K ----------------------------------------------------------------------- */
-/* A unit is one sub-block pair: 32 bytes whose low nibbles are sub-block 2c and
- * whose high nibbles are sub-block 2c+1 of a super-block; 4 consecutive lanes
+/* A unit is one sub-block pair: 16 bytes of sub-block 2c then 16 bytes of
+ * sub-block 2c+1 of a super-block (eight weights per dword); 4 consecutive lanes
  * hold one super-block, so its integer sums meet in two quad-permute DPP steps. */
 template <int T, int R, bool PW> struct GemvQ4K {
   static constexpr int MAXU = GemvUnits<HIPQ_Q4_K, T>::MAXU;
   static constexpr int PER = GemvRec<HIPQ_Q4_K, PW>::PER_CHUNK;
   struct Act {
-    int4 lo0[MAXU][R], lo1[MAXU][R], hi0[MAXU][R], hi1[MAXU][R];
+    /* digits of the activations of sub-blocks 2c (l0, h0) and 2c+1 (l1, h1) */
+    uint4 l0[MAXU][R], l1[MAXU][R], h0[MAXU][R], h1[MAXU][R];
     int bs0[MAXU][R], bs1[MAXU][R]; /* sums of the activations of sub-blocks 2c, 2c+1 */
     float dA[MAXU][R];
   };
@@ -195,12 +219,12 @@ template <int T, int R, bool PW> struct GemvQ4K {
       const int b = u >> 2, c = u & 3;
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        const int4 *ab =
-          (const int4 *)(qa.q + (size_t)arow[r] * qa.K + (size_t)(b0 + b) * 256 + c * 64);
-        A.lo0[i][r] = ab[0];
-        A.lo1[i][r] = ab[1];
-        A.hi0[i][r] = ab[2];
-        A.hi1[i][r] = ab[3];
+        const size_t off = (size_t)arow[r] * (qa.K >> 1) + (size_t)(b0 + b) * 128 + c * 32;
+        const uint4 *al = (const uint4 *)(qa.ql + off), *ah = (const uint4 *)(qa.qh + off);
+        A.l0[i][r] = al[0];
+        A.l1[i][r] = al[1];
+        A.h0[i][r] = ah[0];
+        A.h1[i][r] = ah[1];
         const int2 bsw = *(const int2 *)(qa.bsum + (size_t)arow[r] * (qa.K >> 4) +
                                          (b0 + b) * 16 + 4 * c);
         A.bs0[i][r] = (int)(int16_t)(bsw.x & 0xffff) + (bsw.x >> 16);
@@ -244,18 +268,13 @@ template <int T, int R, bool PW> struct GemvQ4K {
       const uint32_t mnw = c < 2 ? (z & 0x3f3fu) : mn_hi;
       const int sc0 = (int)(scw & 0xff), sc1 = (int)(scw >> 8);
       const int mn0 = (int)(mnw & 0xff), mn1 = (int)(mnw >> 8);
-      const uint32_t lo0[4] = {q0.x & HIPQ_M4, q0.y & HIPQ_M4, q0.z & HIPQ_M4, q0.w & HIPQ_M4};
-      const uint32_t lo1[4] = {q1.x & HIPQ_M4, q1.y & HIPQ_M4, q1.z & HIPQ_M4, q1.w & HIPQ_M4};
-      const uint32_t hi0[4] = {(q0.x >> 4) & HIPQ_M4, (q0.y >> 4) & HIPQ_M4, (q0.z >> 4) & HIPQ_M4,
-                               (q0.w >> 4) & HIPQ_M4};
-      const uint32_t hi1[4] = {(q1.x >> 4) & HIPQ_M4, (q1.y >> 4) & HIPQ_M4, (q1.z >> 4) & HIPQ_M4,
-                               (q1.w >> 4) & HIPQ_M4};
       const float dw = hipq_h2f((uint16_t)(hd.x & 0xffff));
       const float dmin = hipq_h2f((uint16_t)(hd.x >> 16));
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        const int dlo = hipq_dot16(lo0, A.lo0[i][r]) + hipq_dot16(lo1, A.lo1[i][r]);
-        const int dhi = hipq_dot16(hi0, A.hi0[i][r]) + hipq_dot16(hi1, A.hi1[i][r]);
+        /* q0 / q1: the 32 weights of sub-block 2c / 2c+1 */
+        const int dlo = hipq_dot32_u4(q0, A.l0[i][r], A.h0[i][r]);
+        const int dhi = hipq_dot32_u4(q1, A.l1[i][r], A.h1[i][r]);
         int I = __mul24(sc0, dlo) + __mul24(sc1, dhi);
         int Im = __mul24(mn0, A.bs0[i][r]) + __mul24(mn1, A.bs1[i][r]);
         if (PW) {
@@ -411,6 +430,15 @@ struct GemvOut {
  * wavefront's private region of G*R*PER_CHUNK dwords. With PW, activation rows
  * arow[r] < pair_rows use the per-sub-block-pair order (Q4_K only).
  */
+/* The records are private to one wavefront. Its lanes run in lockstep, so LDS
+ * stores only have to be complete before other lanes read them: no workgroup
+ * barrier, and the wavefronts of a workgroup stay free to drift apart (one
+ * streams weights while another computes). */
+__device__ __forceinline__ void hipq_wave_lds_sync() {
+  asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  __builtin_amdgcn_wave_barrier();
+}
+
 template <int DT, int T, int R, int G, bool PW>
 __device__ __forceinline__ GemvOut gemv_engine(const WView &w, int row0, const QView &qa,
                                                const int (&arow)[R], int pair_rows,
@@ -450,7 +478,7 @@ __device__ __forceinline__ GemvOut gemv_engine(const WView &w, int row0, const Q
       const int g = pass * RW + lane / T;
       F::compute(W[pass], A, tl, kc, lds + g * R * PER);
     }
-    __syncthreads();
+    hipq_wave_lds_sync();
     if (chain) {
       if (DT == HIPQ_Q4_0) {
         const int nb = kc >> 5;
@@ -497,7 +525,7 @@ __device__ __forceinline__ GemvOut gemv_engine(const WView &w, int row0, const Q
         }
       }
     }
-    __syncthreads();
+    hipq_wave_lds_sync();
   }
 
   GemvOut out;

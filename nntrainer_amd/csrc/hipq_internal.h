@@ -22,7 +22,8 @@
 /* so that every lane of a wavefront can issue aligned 128-bit loads:         */
 /*   Q4_0: qs [N][K/2]  (16 B per 32-block, nibble order of block_q4_0)       */
 /*         d  [N][K/32] fp16                                                  */
-/*   Q4_K: qs [N][K/2]  (128 B per super-block, byte order of block_q4_K)     */
+/*   Q4_K: qs [N][K/2]  (128 B per super-block: sub-block j = bytes 16j..16j+15, */
+/*                      weight 2i low / 2i+1 high nibble of byte i)             */
 /*         hdr[N][K/256][16] = {fp16 d, fp16 dmin, scales[12]}                */
 /*   Q6_K: qs [N][K/2]  (ql, 128 B per super-block, byte order of block_q6_K) */
 /*         qh [N][K/4]  (64 B per super-block, same byte order)               */
@@ -69,7 +70,9 @@ static inline WView wview(const hipq_weight *w) {
 /* Internal (device) form of quantized activations, structure of arrays.      */
 /*   Q8_0: q [M][K] int8; meta [M][K/32] = fp16 d bits | (int16 sum of the    */
 /*         block's 32 quants) << 16                                           */
-/*   Q8_K: q [M][K] int8; d [M][K/256] fp32; bsum [M][K/16] int16             */
+/*   Q8_K: q [M][K] int8; d [M][K/256] fp32; bsum [M][K/16] int16;            */
+/*         ql, qh [M][K/2]: the same values split into 4-bit digits,           */
+/*         q = 16 * (qh - 8) + ql, element 2i in the low nibble of byte i      */
 /* The quantizers can alternatively emit the canonical ggml blocks.           */
 /* ------------------------------------------------------------------------- */
 struct QAct {
@@ -77,6 +80,8 @@ struct QAct {
   uint32_t *meta; /* Q8_0 */
   float *d;       /* Q8_K */
   int16_t *bsum;  /* Q8_K */
+  uint8_t *ql;    /* Q8_K */
+  uint8_t *qh;    /* Q8_K */
   int M, K;
 };
 size_t qact_bytes(int dtype_is_k, int64_t M, int64_t K);
@@ -86,8 +91,9 @@ QAct qact_carve(int dtype_is_k, void *mem, int64_t M, int64_t K);
 /* Q8_K activations in the form the Q4_K prefill GEMM copies straight from    */
 /* HBM into LDS, tiled by 128 rows (mt = m / 128, rows padded to 128):         */
 /*   qt   [mt][K/128][16384]: one 128-row x 128-deep stage, laid out as        */
-/*        [m%128/32][k%128/32][k%32/16][m%32][16 bytes], i.e. in the order the  */
-/*        lanes of the 32x32x32 int8 matrix instruction take their operands    */
+/*        [m%128/32][k%128/32][k%2][m%32][k%32/2], i.e. 16-byte operands in the  */
+/*        order the lanes of the 32x32x32 int8 matrix instruction take them,    */
+/*        even k in lanes 0-31 and odd k in lanes 32-63 (as the weights' nibbles) */
 /*   amin [mt][K/256][128][16] fp16: per row and super-block the eight         */
 /*        sub-block sums (bsum[2j] + bsum[2j+1]) split into a part in 0..63    */
 /*        (first 8) and a multiple of 64 (last 8), both exact in fp16          */

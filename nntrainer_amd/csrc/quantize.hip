@@ -86,7 +86,7 @@ __global__ __launch_bounds__(256) void quantize_q8_K_kernel(
   const float *__restrict__ A, int64_t M, int64_t n_sb_total, int nsb, int64_t lda,
   int64_t mat_rows, int8_t *__restrict__ q_out, float *__restrict__ d_out,
   int16_t *__restrict__ bsum_out, uint8_t *__restrict__ canon_out,
-  uint16_t *__restrict__ amin_out) {
+  uint16_t *__restrict__ amin_out, uint16_t *__restrict__ ql_out, uint16_t *__restrict__ qh_out) {
   const int lane = threadIdx.x & 63;
   int64_t sb = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
   const bool live = sb < n_sb_total; /* uniform per wavefront */
@@ -152,8 +152,11 @@ __global__ __launch_bounds__(256) void quantize_q8_K_kernel(
     const int stage = b * 2 + (lane >> 5);
     const int kk = (lane * 4) & 127;
     const int64_t tile = (mt * (2 * nsb) + stage) * 16384;
-    const int off = (((r >> 5) * 4 + (kk >> 5)) * 2 + ((kk >> 4) & 1)) * 512 + (r & 31) * 16 + (kk & 15);
-    *(int *)(q_out + tile + off) = packed;
+    /* element k of a 32-deep step goes to half k % 2, byte k / 2: this lane's four
+     * values are two even and two odd elements */
+    const int off = ((r >> 5) * 4 + (kk >> 5)) * 1024 + (r & 31) * 16 + ((kk & 31) >> 1);
+    *(uint16_t *)(q_out + tile + off) = (uint16_t)((q[0] & 0xff) | ((q[2] & 0xff) << 8));
+    *(uint16_t *)(q_out + tile + off + 512) = (uint16_t)((q[1] & 0xff) | ((q[3] & 0xff) << 8));
     const int64_t rb = (mt * nsb + b) * 128 + r;
     if (lane == 0) d_out[rb] = d;
     const int bs = gsum + __shfl_xor(gsum, 4, HIPQ_WAVE); /* two 16-value groups = one sub-block */
@@ -166,6 +169,15 @@ __global__ __launch_bounds__(256) void quantize_q8_K_kernel(
     *(int *)(q_out + sb * 256 + lane * 4) = packed;
     if (lane == 0) d_out[sb] = d;
     if ((lane & 3) == 0) bsum_out[sb * 16 + (lane >> 2)] = (int16_t)gsum;
+    /* 4-bit digits for the v_dot8_u32_u4 kernels: q = 16 * (qh - 8) + ql */
+    uint32_t lo = 0, hi = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      lo |= (uint32_t)(q[i] & 15) << (4 * i);
+      hi |= (uint32_t)(((q[i] >> 4) + 8) & 15) << (4 * i);
+    }
+    ql_out[sb * 64 + lane] = (uint16_t)lo;
+    qh_out[sb * 64 + lane] = (uint16_t)hi;
   }
 }
 
@@ -205,10 +217,12 @@ int launch_quantize_q8_K(const float *A, int64_t M, int64_t K, int64_t lda,
   const unsigned grid = (unsigned)((total + 3) / 4);
   if (canonical_out)
     hipLaunchKernelGGL(quantize_q8_K_kernel<Q8K_CANONICAL>, dim3(grid), dim3(256), 0, s, A, M, total,
-                       nsb, lda, mat_rows, nullptr, nullptr, nullptr, (uint8_t *)canonical_out, nullptr);
+                       nsb, lda, mat_rows, nullptr, nullptr, nullptr, (uint8_t *)canonical_out, nullptr, nullptr,
+                       nullptr);
   else
     hipLaunchKernelGGL(quantize_q8_K_kernel<Q8K_PLANES>, dim3(grid), dim3(256), 0, s, A, M, total, nsb,
-                       lda, mat_rows, qa->q, qa->d, qa->bsum, nullptr, nullptr);
+                       lda, mat_rows, qa->q, qa->d, qa->bsum, nullptr, nullptr, (uint16_t *)qa->ql,
+                       (uint16_t *)qa->qh);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
 }
@@ -223,7 +237,7 @@ int launch_quantize_q8_K_tiled(const float *A, int64_t M, int64_t K, int64_t lda
   const int64_t total = (int64_t)qa->mtiles * 128 * nsb;
   const unsigned grid = (unsigned)((total + 3) / 4);
   hipLaunchKernelGGL(quantize_q8_K_kernel<Q8K_TILED>, dim3(grid), dim3(256), 0, s, A, M, total, nsb, lda,
-                     mat_rows, qa->qt, qa->dAt, nullptr, nullptr, qa->amin);
+                     mat_rows, qa->qt, qa->dAt, nullptr, nullptr, qa->amin, nullptr, nullptr);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
 }
@@ -236,7 +250,8 @@ size_t qact_bytes(int is_k, int64_t M, int64_t K) {
   if (is_k) {
     size_t d = ((size_t)M * (K / 256) * 4 + 255) & ~(size_t)255;
     size_t bs = ((size_t)M * (K / 16) * 2 + 255) & ~(size_t)255;
-    return q + d + bs;
+    size_t dg = ((size_t)M * (K / 2) + 255) & ~(size_t)255;
+    return q + d + bs + 2 * dg;
   }
   size_t meta = ((size_t)M * (K / 32) * 4 + 255) & ~(size_t)255;
   return q + meta;
@@ -272,10 +287,16 @@ QAct qact_carve(int is_k, void *mem, int64_t M, int64_t K) {
   a.meta = nullptr;
   a.d = nullptr;
   a.bsum = nullptr;
+  a.ql = nullptr;
+  a.qh = nullptr;
   if (is_k) {
     a.d = (float *)p;
     p += ((size_t)M * (K / 256) * 4 + 255) & ~(size_t)255;
     a.bsum = (int16_t *)p;
+    p += ((size_t)M * (K / 16) * 2 + 255) & ~(size_t)255;
+    a.ql = p;
+    p += ((size_t)M * (K / 2) + 255) & ~(size_t)255;
+    a.qh = p;
   } else {
     a.meta = (uint32_t *)p;
   }

@@ -54,10 +54,11 @@ __global__ void relayout_q4_K(const uint8_t *__restrict__ src, int x8, int64_t N
   const int b = (int)(i - n * nb);
   uint8_t *oq = qs + i * 128;
   uint8_t *oh = hdr + i * 16;
+  uint8_t cq[128]; /* the super-block's qs in the byte order of block_q4_K */
   if (!x8) {
     const uint8_t *blk = src + i * 144;
     for (int k = 0; k < 16; ++k) oh[k] = blk[k];
-    for (int k = 0; k < 128; ++k) oq[k] = blk[16 + k];
+    for (int k = 0; k < 128; ++k) cq[k] = blk[16 + k];
   } else {
     const int r = (int)(n & 7);
     const uint8_t *grp = src + ((n >> 3) * nb + b) * 1152;
@@ -82,7 +83,17 @@ __global__ void relayout_q4_K(const uint8_t *__restrict__ src, int x8, int64_t N
       }
     }
     for (int k = 0; k < 12; ++k) oh[4 + k] = s[k];
-    for (int k = 0; k < 128; ++k) oq[k] = grp[128 + (k >> 3) * 64 + r * 8 + (k & 7)];
+    for (int k = 0; k < 128; ++k) cq[k] = grp[128 + (k >> 3) * 64 + r * 8 + (k & 7)];
+  }
+  /* block_q4_K keeps sub-blocks 2c / 2c+1 in the low / high nibbles of 32 bytes.
+   * The device plane stores each sub-block's 32 weights as 16 consecutive bytes,
+   * weight 2i in the low and 2i+1 in the high nibble of byte i, so that one
+   * dword is eight weights of ONE sub-block (the unit of v_dot8_u32_u4). */
+  for (int j = 0; j < 8; ++j) {
+    const uint8_t *ch = cq + 32 * (j >> 1);
+    const int sh = 4 * (j & 1);
+    for (int k = 0; k < 16; ++k)
+      oq[16 * j + k] = (uint8_t)(((ch[2 * k] >> sh) & 15) | (((ch[2 * k + 1] >> sh) & 15) << 4));
   }
 }
 
