@@ -193,6 +193,9 @@ template <bool FIRST>
 __device__ __forceinline__ void stage_mma(const Smem &sm, int buf, int wm, int wn, int lane,
                                           v16i (&Dlo)[2], v16i (&Dhi)[2]) {
   Ops o0, o1;
+  /* the matrix phase goes first when both wavefronts of a SIMD want to issue:
+   * the other workgroup's vector work then fills the gaps between MFMAs */
+  __builtin_amdgcn_s_setprio(2);
   read_ops(o0, sm, buf, 0, wm, wn, lane);
   read_ops(o1, sm, buf, 1, wm, wn, lane);
   __builtin_amdgcn_sched_barrier(0);
@@ -207,6 +210,7 @@ __device__ __forceinline__ void stage_mma(const Smem &sm, int buf, int wm, int w
   mma_ops<false>(o0, Dlo, Dhi);
   __builtin_amdgcn_sched_barrier(0);
   mma_ops<false>(o1, Dlo, Dhi);
+  __builtin_amdgcn_s_setprio(0);
   __builtin_amdgcn_sched_barrier(0);
 }
 
