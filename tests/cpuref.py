@@ -173,6 +173,26 @@ def gemm(lib, kind, a, w_blocks, n):
     return c
 
 
+def prepack(lib, kind, w_blocks, n, k):
+    """Weights in the form `gemm_prepacked` takes: as they are for the oracle, in the
+    x8 layout (done once) for the reference library's Q4_0 / Q4_K kernels."""
+    w_blocks = np.ascontiguousarray(w_blocks)
+    if lib is oracle() or kind == "q6_K":
+        return w_blocks
+    return repack_x8(lib, kind, w_blocks, n, k)
+
+
+def gemm_prepacked(lib, kind, a, packed, n):
+    a = np.ascontiguousarray(a, dtype=np.float32)
+    m, k = a.shape
+    c = np.zeros((m, n), np.float32)
+    if lib is oracle():
+        getattr(lib, "orc_gemm_" + kind)(_i32(m), _i32(n), _i32(k), _ptr(a), _ptr(packed), _ptr(c))
+    else:
+        getattr(lib, "ref_gemm_" + kind)(_c.c_uint(m), _c.c_uint(n), _c.c_uint(k), _ptr(a), _ptr(packed), _ptr(c))
+    return c
+
+
 def moe_forward(x, logits, gate, up, down, topk):
     """Oracle MoE block. gate/up/down: lists (len E) of canonical Q4_K block arrays."""
     lib = oracle()
