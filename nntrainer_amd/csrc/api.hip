@@ -43,7 +43,8 @@ struct State {
   bool ready = false;
   int device = -1;
   std::unordered_map<hipStream_t, Workspace> ws;
-  std::unordered_map<hipStream_t, MoeTable> moe_tables;
+  /* one table of expert weight views per MoE layer, found by its first gate weight */
+  std::unordered_map<const hipq_weight *, MoeTable> moe_tables;
   int64_t live_weights = 0;
 };
 State g;
@@ -350,7 +351,10 @@ int hipq_weight_destroy(hipq_weight_t w) {
   {
     std::lock_guard<std::mutex> lk(g.mu);
     g.live_weights--;
-    for (auto &kv : g.moe_tables) kv.second.key.clear(); /* tables may name w */
+    /* tables may name w: drop them (the device was synchronized above) */
+    for (auto &kv : g.moe_tables)
+      if (kv.second.dev) (void)hipFree(kv.second.dev);
+    g.moe_tables.clear();
   }
   delete w;
   return HIPQ_OK;
@@ -565,7 +569,7 @@ int hipq_moe_forward(const hipq_moe_desc *desc, const hipq_weight_t *gate, const
   WView *dev_views = nullptr;
   {
     std::lock_guard<std::mutex> lk(g.mu);
-    MoeTable &t = g.moe_tables[s];
+    MoeTable &t = g.moe_tables[gate[0]];
     std::vector<const hipq_weight *> key;
     key.reserve(3 * (size_t)d.experts);
     for (int e = 0; e < d.experts; ++e) key.push_back(gate[e]);
@@ -575,7 +579,7 @@ int hipq_moe_forward(const hipq_moe_desc *desc, const hipq_weight_t *gate, const
       std::vector<WView> host(key.size());
       for (size_t i = 0; i < key.size(); ++i) host[i] = wview(key[i]);
       if (t.dev) {
-        HIPQ_HIP(hipStreamSynchronize(s));
+        HIPQ_HIP(hipDeviceSynchronize()); /* another stream may still read the old table */
         HIPQ_HIP(hipFree(t.dev));
         t.dev = nullptr;
       }

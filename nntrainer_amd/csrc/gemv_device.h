@@ -117,15 +117,17 @@ template <bool PW> struct GemvRec<HIPQ_Q6_K, PW> {
   static constexpr int LANES_PER_OUT = 8;
 };
 
-/* Units a lane handles per chunk: 64 lanes cover a 4096-weight chunk in 2 (Q4_0) or
- * 1 (Q4_K, Q6_K) steps; 16 lanes are only used for rows shorter than 64 units. */
-template <int DT, int T> struct GemvUnits {
-  static constexpr int MAXU = (T == 64) ? (HIPQ_KCHUNK / GemvRec<DT, false>::UNIT) / 64 : 4;
+/* Units a lane handles per chunk of KC weights: 64 lanes cover a 4096-weight chunk
+ * in 2 (Q4_0) or 1 (Q4_K, Q6_K) steps. Kernels for short rows (MoE experts) pick
+ * fewer lanes per row and a smaller chunk so that no lane and no register idles. */
+template <int DT, int T, int KC> struct GemvUnits {
+  static constexpr int MAXU = (KC / GemvRec<DT, false>::UNIT + T - 1) / T;
+  static_assert(KC <= HIPQ_KCHUNK && KC % 256 == 0, "chunk must fit the LDS records");
 };
 
 /* ---- Q4_0 ----------------------------------------------------------------------- */
-template <int T, int R, bool PW> struct GemvQ40 {
-  static constexpr int MAXU = GemvUnits<HIPQ_Q4_0, T>::MAXU;
+template <int T, int R, bool PW, int KC> struct GemvQ40 {
+  static constexpr int MAXU = GemvUnits<HIPQ_Q4_0, T, KC>::MAXU;
   static constexpr int PER = GemvRec<HIPQ_Q4_0, PW>::PER_CHUNK;
   struct Act {
     int4 a0[MAXU][R], a1[MAXU][R];
@@ -196,8 +198,8 @@ template <int T, int R, bool PW> struct GemvQ40 {
 /* A unit is one sub-block pair: 16 bytes of sub-block 2c then 16 bytes of
  * sub-block 2c+1 of a super-block (eight weights per dword); 4 consecutive lanes
  * hold one super-block, so its integer sums meet in two quad-permute DPP steps. */
-template <int T, int R, bool PW> struct GemvQ4K {
-  static constexpr int MAXU = GemvUnits<HIPQ_Q4_K, T>::MAXU;
+template <int T, int R, bool PW, int KC> struct GemvQ4K {
+  static constexpr int MAXU = GemvUnits<HIPQ_Q4_K, T, KC>::MAXU;
   static constexpr int PER = GemvRec<HIPQ_Q4_K, PW>::PER_CHUNK;
   struct Act {
     /* digits of the activations of sub-blocks 2c (l0, h0) and 2c+1 (l1, h1) */
@@ -310,8 +312,8 @@ template <int T, int R, bool PW> struct GemvQ4K {
 /* A unit is 64 weights = 2 x 16 B of ql + 16 B of qh, unit uu = half*2 + hl of a
  * super-block. Dword t of the unit belongs to partial l = hl*4 + t; lanes uu and
  * uu^2 hold the two 128-element halves. */
-template <int T, int R, bool PW> struct GemvQ6K {
-  static constexpr int MAXU = GemvUnits<HIPQ_Q6_K, T>::MAXU;
+template <int T, int R, bool PW, int KC> struct GemvQ6K {
+  static constexpr int MAXU = GemvUnits<HIPQ_Q6_K, T, KC>::MAXU;
   static constexpr int PER = GemvRec<HIPQ_Q6_K, PW>::PER_CHUNK;
   struct Act {
     int4 a[MAXU][R][4];
@@ -410,10 +412,10 @@ template <int T, int R, bool PW> struct GemvQ6K {
   }
 };
 
-template <int DT, int T, int R, bool PW> struct GemvFmt;
-template <int T, int R, bool PW> struct GemvFmt<HIPQ_Q4_0, T, R, PW> { typedef GemvQ40<T, R, PW> type; };
-template <int T, int R, bool PW> struct GemvFmt<HIPQ_Q4_K, T, R, PW> { typedef GemvQ4K<T, R, PW> type; };
-template <int T, int R, bool PW> struct GemvFmt<HIPQ_Q6_K, T, R, PW> { typedef GemvQ6K<T, R, PW> type; };
+template <int DT, int T, int R, bool PW, int KC> struct GemvFmt;
+template <int T, int R, bool PW, int KC> struct GemvFmt<HIPQ_Q4_0, T, R, PW, KC> { typedef GemvQ40<T, R, PW, KC> type; };
+template <int T, int R, bool PW, int KC> struct GemvFmt<HIPQ_Q4_K, T, R, PW, KC> { typedef GemvQ4K<T, R, PW, KC> type; };
+template <int T, int R, bool PW, int KC> struct GemvFmt<HIPQ_Q6_K, T, R, PW, KC> { typedef GemvQ6K<T, R, PW, KC> type; };
 
 /* ---- engine --------------------------------------------------------------------- */
 
@@ -439,46 +441,76 @@ __device__ __forceinline__ void hipq_wave_lds_sync() {
   __builtin_amdgcn_wave_barrier();
 }
 
-template <int DT, int T, int R, int G, bool PW>
-__device__ __forceinline__ GemvOut gemv_engine(const WView &w, int row0, const QView &qa,
-                                               const int (&arow)[R], int pair_rows,
-                                               uint32_t *lds) {
-  typedef typename GemvFmt<DT, T, R, PW>::type F;
-  constexpr int RW = 64 / T; /* weight rows streamed at once */
-  constexpr int NP = G / RW; /* passes per group */
-  constexpr int PER = GemvRec<DT, PW>::PER_CHUNK;
-  constexpr int LPO = GemvRec<DT, PW>::LANES_PER_OUT;
+/* The pieces of the engine, so that callers with several weight-row groups per
+ * wavefront can keep the loads of the next group in flight while this one is
+ * computed (see gemv_engine for the plain sequence). */
+template <int DT, int T, int R, int G, bool PW, int KC = HIPQ_KCHUNK> struct GemvCore {
+  typedef typename GemvFmt<DT, T, R, PW, KC>::type F;
+  typedef typename F::Act Act;
+  static constexpr int RW = 64 / T; /* weight rows streamed at once */
+  static constexpr int NP = G / RW; /* passes per group */
+  static constexpr int PER = GemvRec<DT, PW>::PER_CHUNK;
+  static constexpr int LPO = GemvRec<DT, PW>::LANES_PER_OUT;
   static_assert(G % RW == 0, "group must be a multiple of the rows streamed at once");
   static_assert(G * R * LPO <= 64, "one lane per fp32 chain");
-  const int lane = threadIdx.x & 63, tl = lane % T;
-  const int ci = lane / LPO, l = lane % LPO; /* chain of this lane in phase 2 */
-  const bool chain = ci < G * R;
-  const int cg = chain ? ci / R : 0, cr = chain ? ci % R : 0;
-  const uint32_t *crec = lds + (cg * R + cr) * PER;
-  float acc = 0.f, accm = 0.f;
-  bool pairwise = false;
-  if (PW) {
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-      if (r == cr) pairwise = arow[r] < pair_rows;
-  }
-
-  for (int k0 = 0; k0 < w.K; k0 += HIPQ_KCHUNK) {
-    const int kc = min(HIPQ_KCHUNK, w.K - k0);
-    typename F::Act A;
-    F::load_act(A, qa, arow, tl, k0, kc);
+  struct Wts {
     typename F::Wt W[NP];
+  };
+  /* the fp32 chain this lane runs in phase 2 */
+  struct Chain {
+    int cg, cr, l;
+    bool on, pairwise;
+    float acc, accm;
+  };
+
+  __device__ static __forceinline__ void load_act(Act &A, const QView &qa, const int (&arow)[R],
+                                                  int k0, int kc) {
+    F::load_act(A, qa, arow, (threadIdx.x & 63) % T, k0, kc);
+  }
+  /* issue the loads of the G weight rows from row0 (clamped to the matrix) */
+  __device__ static __forceinline__ void load_w(Wts &w, const WView &wv, int row0, int k0, int kc) {
+    const int lane = threadIdx.x & 63, tl = lane % T;
 #pragma unroll
     for (int pass = 0; pass < NP; ++pass) {
       const int g = pass * RW + lane / T;
-      F::load_w(W[pass], w, min(row0 + g, w.N - 1), tl, k0, kc);
+      F::load_w(w.W[pass], wv, min(row0 + g, wv.N - 1), tl, k0, kc);
     }
+  }
+  /* phase 1: integer partial sums of this chunk into the wavefront's LDS records */
+  __device__ static __forceinline__ void compute(const Wts &w, const Act &A, int kc, uint32_t *lds) {
+    const int lane = threadIdx.x & 63, tl = lane % T;
 #pragma unroll
     for (int pass = 0; pass < NP; ++pass) {
       const int g = pass * RW + lane / T;
-      F::compute(W[pass], A, tl, kc, lds + g * R * PER);
+      F::compute(w.W[pass], A, tl, kc, lds + g * R * PER);
     }
-    hipq_wave_lds_sync();
+  }
+  __device__ static __forceinline__ Chain begin(const int (&arow)[R], int pair_rows) {
+    const int lane = threadIdx.x & 63;
+    Chain c;
+    const int ci = lane / LPO;
+    c.l = lane % LPO;
+    c.on = ci < G * R;
+    c.cg = c.on ? ci / R : 0;
+    c.cr = c.on ? ci % R : 0;
+    c.acc = 0.f;
+    c.accm = 0.f;
+    c.pairwise = false;
+    if (PW) {
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+        if (r == c.cr) c.pairwise = arow[r] < pair_rows;
+    }
+    return c;
+  }
+  /* phase 2: this lane's fp32 chain over the records of one chunk, reference order */
+  __device__ static __forceinline__ void chain(Chain &c, int kc, const uint32_t *lds) {
+    const uint32_t *crec = lds + (c.cg * R + c.cr) * PER;
+    const bool chain = c.on, pairwise = c.pairwise;
+    const int l = c.l;
+    float acc = c.acc, accm = c.accm;
+    (void)pairwise;
+    (void)l;
     if (chain) {
       if (DT == HIPQ_Q4_0) {
         const int nb = kc >> 5;
@@ -525,9 +557,15 @@ __device__ __forceinline__ GemvOut gemv_engine(const WView &w, int row0, const Q
         }
       }
     }
-    hipq_wave_lds_sync();
+    c.acc = acc;
+    c.accm = accm;
   }
-
+  __device__ static __forceinline__ GemvOut finish(const Chain &c) {
+    const bool chain = c.on;
+    const int cg = c.cg, cr = c.cr, l = c.l;
+    const float acc = c.acc, accm = c.accm;
+    (void)l;
+    (void)accm;
   GemvOut out;
   out.g = cg;
   out.r = cr;
@@ -547,6 +585,27 @@ __device__ __forceinline__ GemvOut gemv_engine(const WView &w, int row0, const Q
     out.valid = chain;
   }
   return out;
+  }
+};
+
+template <int DT, int T, int R, int G, bool PW, int KC = HIPQ_KCHUNK>
+__device__ __forceinline__ GemvOut gemv_engine(const WView &w, int row0, const QView &qa,
+                                               const int (&arow)[R], int pair_rows,
+                                               uint32_t *lds) {
+  typedef GemvCore<DT, T, R, G, PW, KC> E;
+  typename E::Chain c = E::begin(arow, pair_rows);
+  for (int k0 = 0; k0 < w.K; k0 += KC) {
+    const int kc = min(KC, w.K - k0);
+    typename E::Act A;
+    E::load_act(A, qa, arow, k0, kc);
+    typename E::Wts W;
+    E::load_w(W, w, row0, k0, kc);
+    E::compute(W, A, kc, lds);
+    hipq_wave_lds_sync();
+    E::chain(c, kc, lds);
+    hipq_wave_lds_sync();
+  }
+  return E::finish(c);
 }
 
 /* LDS dwords one wavefront needs for G weight rows x R activation rows. */

@@ -32,7 +32,6 @@
 namespace {
 
 constexpr int RTOK = 4; /* tokens sharing one pass over an expert's weight rows */
-constexpr int GROW = 2; /* weight rows (output columns) per wavefront and pass      */
 
 struct MoeBufs {
   float *logits;
@@ -169,6 +168,45 @@ __global__ __launch_bounds__(256) void route_kernel(const float *__restrict__ lo
   }
 }
 
+/* Count, scan and scatter of the (token, k) pairs by expert in one workgroup:
+ * the sort of a decode step or a short prefill chunk is a few thousand pairs, and
+ * four tiny launches would cost more than the work. E <= 1024. */
+__global__ __launch_bounds__(1024) void sort_pairs_kernel(const int32_t *__restrict__ idx, int P,
+                                                          int E, int *__restrict__ offsets,
+                                                          int *__restrict__ slot_pair,
+                                                          int *__restrict__ pair_slot) {
+  __shared__ int cnt[1024];
+  __shared__ int off[1024];
+  const int t = threadIdx.x;
+  cnt[t] = 0;
+  __syncthreads();
+  for (int i = t; i < P; i += 1024) atomicAdd(&cnt[idx[i]], 1);
+  __syncthreads();
+  /* inclusive scan over the 1024 slots (Hillis-Steele), exclusive = inclusive - own */
+  const int own = cnt[t];
+  off[t] = own;
+  __syncthreads();
+  for (int d = 1; d < 1024; d <<= 1) {
+    const int v = t >= d ? off[t - d] : 0;
+    __syncthreads();
+    off[t] += v;
+    __syncthreads();
+  }
+  const int excl = off[t] - own;
+  if (t < E) offsets[t] = excl;
+  if (t == E - 1) offsets[E] = off[t];
+  __syncthreads();
+  off[t] = excl;
+  cnt[t] = 0;
+  __syncthreads();
+  for (int i = t; i < P; i += 1024) {
+    const int e = idx[i];
+    const int slot = off[e] + atomicAdd(&cnt[e], 1);
+    slot_pair[slot] = i;
+    pair_slot[i] = slot;
+  }
+}
+
 __global__ void fill_int_kernel(int *p, int n, int v) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i < n) p[i] = v;
@@ -210,21 +248,42 @@ __device__ __forceinline__ float silu_ref(float g) {
   return sig * g;
 }
 
-/* h[slot][col] = silu(x_tok . Wgate[e][col]) * (x_tok . Wup[e][col]) */
-template <int DT, int T>
-__global__ __launch_bounds__(256) void gate_up_kernel(const WView *__restrict__ views, int E,
+/* One group of G weight rows against the cached activations: phase 1 into the
+ * wavefront's LDS records, phase 2 fp32 chains, result of this lane's chain. */
+template <typename E>
+__device__ __forceinline__ GemvOut run_group(const typename E::Wts &W, const typename E::Act &A,
+                                             const int (&arow)[RTOK], int K, uint32_t *lds) {
+  typename E::Chain c = E::begin(arow, 0);
+  E::compute(W, A, K, lds);
+  hipq_wave_lds_sync();
+  E::chain(c, K, lds);
+  hipq_wave_lds_sync();
+  return E::finish(c);
+}
+
+/* h[slot][col] = silu(x_tok . Wgate[e][col]) * (x_tok . Wup[e][col])
+ *
+ * A workgroup serves one expert; each wavefront owns CPW groups of G columns.
+ * Per group of RTOK tokens it loads their quantized activations once, then walks
+ * its column groups with the gate rows and the up rows of a group as two work
+ * items; the weight loads of the next item are always in flight while the current
+ * one is computed. Requires K <= KC (one chunk). */
+template <int DT, int T, int KC, int G, int CPW>
+__global__ __launch_bounds__(256) void gate_up_kernel(const WView *__restrict__ views, int E_,
                                                       QView xq, const int *__restrict__ offsets,
                                                       const int *__restrict__ slot_pair, int topk,
                                                       int I, float *__restrict__ h) {
-  constexpr int G = GROW;
+  typedef GemvCore<DT, T, RTOK, G, false, KC> E;
   extern __shared__ uint32_t moe_lds[];
   const int e = blockIdx.y;
   const int begin = offsets[e], end = offsets[e + 1];
   if (begin == end) return;
-  const WView wg = views[e], wu = views[E + e];
+  const WView wg = views[e], wu = views[E_ + e];
   const int wave = threadIdx.x >> 6;
-  uint32_t *lds = moe_lds + wave * GemvLds<DT, RTOK, GROW, false>::DWORDS;
-  const int col0 = (blockIdx.x * 4 + wave) * G;
+  uint32_t *lds = moe_lds + wave * GemvLds<DT, RTOK, G, false>::DWORDS;
+  const int cbase = (blockIdx.x * 4 + wave) * CPW * G;
+  if (cbase >= I) return; /* uniform per wavefront; the syncs below are wavefront-local */
+  const int K = wg.K;
   for (int s0 = begin; s0 < end; s0 += RTOK) {
     int arow[RTOK];
 #pragma unroll
@@ -232,34 +291,112 @@ __global__ __launch_bounds__(256) void gate_up_kernel(const WView *__restrict__ 
       const int slot = min(s0 + r, end - 1);
       arow[r] = slot_pair[slot] / topk; /* token of the pair */
     }
-    const GemvOut g = gemv_engine<DT, T, RTOK, G, false>(wg, col0, xq, arow, 0, lds);
-    const GemvOut u = gemv_engine<DT, T, RTOK, G, false>(wu, col0, xq, arow, 0, lds);
+    typename E::Act A;
+    E::load_act(A, xq, arow, 0, K);
+    typename E::Wts Wg, Wu;
+    E::load_w(Wg, wg, cbase, 0, K);
+#pragma unroll
+    for (int cg = 0; cg < CPW; ++cg) {
+      const int col0 = cbase + cg * G;
+      if (col0 >= I) break; /* uniform */
+      E::load_w(Wu, wu, col0, 0, K);
+      const GemvOut g = run_group<E>(Wg, A, arow, K, lds);
+      if (cg + 1 < CPW && col0 + G < I) E::load_w(Wg, wg, col0 + G, 0, K);
+      const GemvOut u = run_group<E>(Wu, A, arow, K, lds);
+      if (g.valid && col0 + g.g < I && s0 + g.r < end)
+        h[(size_t)(s0 + g.r) * I + col0 + g.g] = silu_ref(g.v) * u.v;
+    }
+  }
+}
+
+/* contrib[slot][col] = (h_slot . Wdown[e][col]) * weight(pair); same structure */
+template <int DT, int T, int KC, int G, int CPW>
+__global__ __launch_bounds__(256) void down_kernel(const WView *__restrict__ views, int E_, QView hq,
+                                                   const int *__restrict__ offsets,
+                                                   const int *__restrict__ slot_pair,
+                                                   const float *__restrict__ wgt, int H,
+                                                   float *__restrict__ contrib) {
+  typedef GemvCore<DT, T, RTOK, G, false, KC> E;
+  extern __shared__ uint32_t moe_lds[];
+  const int e = blockIdx.y;
+  const int begin = offsets[e], end = offsets[e + 1];
+  if (begin == end) return;
+  const WView wd = views[2 * E_ + e];
+  const int wave = threadIdx.x >> 6;
+  uint32_t *lds = moe_lds + wave * GemvLds<DT, RTOK, G, false>::DWORDS;
+  const int cbase = (blockIdx.x * 4 + wave) * CPW * G;
+  if (cbase >= H) return;
+  const int K = wd.K;
+  for (int s0 = begin; s0 < end; s0 += RTOK) {
+    int arow[RTOK];
+#pragma unroll
+    for (int r = 0; r < RTOK; ++r) arow[r] = min(s0 + r, end - 1); /* hq rows are slots */
+    typename E::Act A;
+    E::load_act(A, hq, arow, 0, K);
+    typename E::Wts W[2];
+    E::load_w(W[0], wd, cbase, 0, K);
+#pragma unroll
+    for (int cg = 0; cg < CPW; ++cg) {
+      const int col0 = cbase + cg * G;
+      if (col0 >= H) break;
+      if (cg + 1 < CPW && col0 + G < H) E::load_w(W[(cg + 1) & 1], wd, col0 + G, 0, K);
+      const GemvOut o = run_group<E>(W[cg & 1], A, arow, K, lds);
+      if (o.valid && col0 + o.g < H && s0 + o.r < end)
+        contrib[(size_t)(s0 + o.r) * H + col0 + o.g] = o.v * wgt[slot_pair[s0 + o.r]];
+    }
+  }
+}
+
+/* The same two products for rows longer than one chunk (K > 4096): one engine call
+ * per column group, no cross-group prefetch. */
+template <int DT>
+__global__ __launch_bounds__(256) void gate_up_long_kernel(const WView *__restrict__ views, int E_,
+                                                           QView xq, const int *__restrict__ offsets,
+                                                           const int *__restrict__ slot_pair,
+                                                           int topk, int I, float *__restrict__ h) {
+  constexpr int G = 2;
+  extern __shared__ uint32_t moe_lds[];
+  const int e = blockIdx.y;
+  const int begin = offsets[e], end = offsets[e + 1];
+  if (begin == end) return;
+  const WView wg = views[e], wu = views[E_ + e];
+  const int wave = threadIdx.x >> 6;
+  uint32_t *lds = moe_lds + wave * GemvLds<DT, RTOK, G, false>::DWORDS;
+  const int col0 = (blockIdx.x * 4 + wave) * G;
+  for (int s0 = begin; s0 < end; s0 += RTOK) {
+    int arow[RTOK];
+#pragma unroll
+    for (int r = 0; r < RTOK; ++r) {
+      const int slot = min(s0 + r, end - 1);
+      arow[r] = slot_pair[slot] / topk;
+    }
+    const GemvOut g = gemv_engine<DT, 64, RTOK, G, false>(wg, col0, xq, arow, 0, lds);
+    const GemvOut u = gemv_engine<DT, 64, RTOK, G, false>(wu, col0, xq, arow, 0, lds);
     if (g.valid && col0 + g.g < I && s0 + g.r < end)
       h[(size_t)(s0 + g.r) * I + col0 + g.g] = silu_ref(g.v) * u.v;
   }
 }
 
-/* contrib[slot][col] = (h_slot . Wdown[e][col]) * weight(pair) */
-template <int DT, int T>
-__global__ __launch_bounds__(256) void down_kernel(const WView *__restrict__ views, int E, QView hq,
-                                                   const int *__restrict__ offsets,
-                                                   const int *__restrict__ slot_pair,
-                                                   const float *__restrict__ wgt, int H,
-                                                   float *__restrict__ contrib) {
-  constexpr int G = GROW;
+template <int DT>
+__global__ __launch_bounds__(256) void down_long_kernel(const WView *__restrict__ views, int E_,
+                                                        QView hq, const int *__restrict__ offsets,
+                                                        const int *__restrict__ slot_pair,
+                                                        const float *__restrict__ wgt, int H,
+                                                        float *__restrict__ contrib) {
+  constexpr int G = 2;
   extern __shared__ uint32_t moe_lds[];
   const int e = blockIdx.y;
   const int begin = offsets[e], end = offsets[e + 1];
   if (begin == end) return;
-  const WView wd = views[2 * E + e];
+  const WView wd = views[2 * E_ + e];
   const int wave = threadIdx.x >> 6;
-  uint32_t *lds = moe_lds + wave * GemvLds<DT, RTOK, GROW, false>::DWORDS;
+  uint32_t *lds = moe_lds + wave * GemvLds<DT, RTOK, G, false>::DWORDS;
   const int col0 = (blockIdx.x * 4 + wave) * G;
   for (int s0 = begin; s0 < end; s0 += RTOK) {
     int arow[RTOK];
 #pragma unroll
-    for (int r = 0; r < RTOK; ++r) arow[r] = min(s0 + r, end - 1); /* hq rows are slots */
-    const GemvOut o = gemv_engine<DT, T, RTOK, G, false>(wd, col0, hq, arow, 0, lds);
+    for (int r = 0; r < RTOK; ++r) arow[r] = min(s0 + r, end - 1);
+    const GemvOut o = gemv_engine<DT, 64, RTOK, G, false>(wd, col0, hq, arow, 0, lds);
     if (o.valid && col0 + o.g < H && s0 + o.r < end)
       contrib[(size_t)(s0 + o.r) * H + col0 + o.g] = o.v * wgt[slot_pair[s0 + o.r]];
   }
@@ -293,41 +430,91 @@ __global__ __launch_bounds__(256) void combine_kernel(const int32_t *__restrict_
   y[(size_t)t * H + c] = acc;
 }
 
+/* Lanes per weight row, chunk size and weight rows per wavefront for rows of K
+ * weights: expert matrices are short (K = 768 .. 4096), so the lanes of a
+ * wavefront are split over 4, 2 or 1 rows such that (nearly) all of them hold a
+ * unit, and more rows per wavefront amortise the activation loads. Q6_K has eight
+ * fp32 chains per output, which bounds the rows per wavefront. */
+constexpr int CPW = 4; /* column groups per wavefront */
+
+template <int DT, int T, int KC, int G>
+void launch_gate_up(const hipq_moe_desc &d, const WView *views, const QAct &xq, const MoeBufs &b,
+                    hipStream_t s) {
+  const size_t lds = 4 * GemvLds<DT, RTOK, G, false>::DWORDS * sizeof(uint32_t);
+  if (d.hidden > KC) {
+    const dim3 grid((d.intermediate + 7) / 8, d.experts);
+    const size_t lds_long = 4 * GemvLds<DT, RTOK, 2, false>::DWORDS * sizeof(uint32_t);
+    hipLaunchKernelGGL((gate_up_long_kernel<DT>), grid, dim3(256), lds_long, s, views, d.experts,
+                       qview(xq), b.offsets, b.slot_pair, d.topk, d.intermediate, b.h);
+    return;
+  }
+  const dim3 grid((d.intermediate + 4 * G * CPW - 1) / (4 * G * CPW), d.experts);
+  hipLaunchKernelGGL((gate_up_kernel<DT, T, KC, G, CPW>), grid, dim3(256), lds, s, views, d.experts,
+                     qview(xq), b.offsets, b.slot_pair, d.topk, d.intermediate, b.h);
+}
+template <int DT, int T, int KC, int G>
+void launch_down(const hipq_moe_desc &d, const WView *views, const QAct &hq, const MoeBufs &b,
+                 hipStream_t s) {
+  const size_t lds = 4 * GemvLds<DT, RTOK, G, false>::DWORDS * sizeof(uint32_t);
+  if (d.intermediate > KC) {
+    const dim3 grid((d.hidden + 7) / 8, d.experts);
+    const size_t lds_long = 4 * GemvLds<DT, RTOK, 2, false>::DWORDS * sizeof(uint32_t);
+    hipLaunchKernelGGL((down_long_kernel<DT>), grid, dim3(256), lds_long, s, views, d.experts,
+                       qview(hq), b.offsets, b.slot_pair, b.wgt, d.hidden, b.contrib);
+    return;
+  }
+  const dim3 grid((d.hidden + 4 * G * CPW - 1) / (4 * G * CPW), d.experts);
+  hipLaunchKernelGGL((down_kernel<DT, T, KC, G, CPW>), grid, dim3(256), lds, s, views, d.experts,
+                     qview(hq), b.offsets, b.slot_pair, b.wgt, d.hidden, b.contrib);
+}
+
+/* calls f.template operator()<T, KC, G>() for the shape class of K */
+template <int DT, typename F> void for_row_length(int64_t K, F f) {
+  if constexpr (DT == HIPQ_Q4_K) {
+    if (K <= 1024) f.template operator()<16, 1024, 8>();
+    else if (K <= 2048) f.template operator()<32, 2048, 4>();
+    else f.template operator()<64, 4096, 4>();
+  } else if constexpr (DT == HIPQ_Q4_0) {
+    if (K <= 1024) f.template operator()<32, 1024, 2>();
+    else if (K <= 2048) f.template operator()<64, 2048, 2>();
+    else f.template operator()<64, 4096, 2>();
+  } else {
+    if (K <= 2048) f.template operator()<32, 2048, 2>();
+    else f.template operator()<64, 4096, 2>();
+  }
+}
+
+template <int DT> struct GateUpLauncher {
+  const hipq_moe_desc &d;
+  const WView *views;
+  const QAct &xq;
+  const MoeBufs &b;
+  hipStream_t s;
+  template <int T, int KC, int G> void operator()() const { launch_gate_up<DT, T, KC, G>(d, views, xq, b, s); }
+};
+template <int DT> struct DownLauncher {
+  const hipq_moe_desc &d;
+  const WView *views;
+  const QAct &hq;
+  const MoeBufs &b;
+  hipStream_t s;
+  template <int T, int KC, int G> void operator()() const { launch_down<DT, T, KC, G>(d, views, hq, b, s); }
+};
+
 template <int DT>
 int launch_grouped(const hipq::MoeArgs *a, const MoeBufs &b, const WView *views, const QAct &xq,
                    const QAct &hq, hipStream_t s) {
   const hipq_moe_desc &d = a->desc;
-  constexpr int G = GROW;
-  constexpr int TS = 64;
-  const size_t lds = 4 * GemvLds<DT, RTOK, GROW, false>::DWORDS * sizeof(uint32_t);
-  const int64_t units_gu = (DT == HIPQ_Q6_K) ? d.hidden / 64 : d.hidden / 32;
-  const int64_t units_dn = (DT == HIPQ_Q6_K) ? d.intermediate / 64 : d.intermediate / 32;
   const int64_t P = (int64_t)d.tokens * d.topk;
   int rc;
-  {
-    const dim3 grid((d.intermediate + 4 * G - 1) / (4 * G), d.experts);
-    if (units_gu >= 64)
-      hipLaunchKernelGGL((gate_up_kernel<DT, 64>), grid, dim3(256), lds, s, views, d.experts,
-                         qview(xq), b.offsets, b.slot_pair, d.topk, d.intermediate, b.h);
-    else
-      hipLaunchKernelGGL((gate_up_kernel<DT, TS>), grid, dim3(256), lds, s, views, d.experts,
-                         qview(xq), b.offsets, b.slot_pair, d.topk, d.intermediate, b.h);
-  }
+  for_row_length<DT>(d.hidden, GateUpLauncher<DT>{d, views, xq, b, s});
   HIPQ_HIP(hipGetLastError());
   if (DT == HIPQ_Q4_0)
     rc = hipq::launch_quantize_q8_0(b.h, P, d.intermediate, d.intermediate, &hq, nullptr, s);
   else
     rc = hipq::launch_quantize_q8_K(b.h, P, d.intermediate, d.intermediate, 0, &hq, nullptr, s);
   if (rc) return rc;
-  {
-    const dim3 grid((d.hidden + 4 * G - 1) / (4 * G), d.experts);
-    if (units_dn >= 64)
-      hipLaunchKernelGGL((down_kernel<DT, 64>), grid, dim3(256), lds, s, views, d.experts,
-                         qview(hq), b.offsets, b.slot_pair, b.wgt, d.hidden, b.contrib);
-    else
-      hipLaunchKernelGGL((down_kernel<DT, TS>), grid, dim3(256), lds, s, views, d.experts,
-                         qview(hq), b.offsets, b.slot_pair, b.wgt, d.hidden, b.contrib);
-  }
+  for_row_length<DT>(d.intermediate, DownLauncher<DT>{d, views, hq, b, s});
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
 }
@@ -368,11 +555,16 @@ int launch_moe(const MoeArgs *a, void *workspace, size_t workspace_bytes, const 
                      d.renormalize, idx, wgt);
   HIPQ_HIP(hipGetLastError());
   b.wgt = wgt;
-  hipLaunchKernelGGL(fill_int_kernel, dim3((E + 255) / 256), dim3(256), 0, s, b.counts, E, 0);
-  hipLaunchKernelGGL(count_kernel, dim3((P + 255) / 256), dim3(256), 0, s, idx, P, b.counts);
-  hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(64), 0, s, b.counts, E, b.offsets, b.cursor);
-  hipLaunchKernelGGL(scatter_kernel, dim3((P + 255) / 256), dim3(256), 0, s, idx, P, b.offsets,
-                     b.cursor, b.slot_pair, b.pair_slot);
+  if (P <= 16384 && E <= 1024) {
+    hipLaunchKernelGGL(sort_pairs_kernel, dim3(1), dim3(1024), 0, s, idx, P, E, b.offsets, b.slot_pair,
+                       b.pair_slot);
+  } else {
+    hipLaunchKernelGGL(fill_int_kernel, dim3((E + 255) / 256), dim3(256), 0, s, b.counts, E, 0);
+    hipLaunchKernelGGL(count_kernel, dim3((P + 255) / 256), dim3(256), 0, s, idx, P, b.counts);
+    hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(64), 0, s, b.counts, E, b.offsets, b.cursor);
+    hipLaunchKernelGGL(scatter_kernel, dim3((P + 255) / 256), dim3(256), 0, s, idx, P, b.offsets,
+                       b.cursor, b.slot_pair, b.pair_slot);
+  }
   HIPQ_HIP(hipGetLastError());
 
   QAct xq = qact_carve(is_k, b.xq_mem, T, d.hidden);
