@@ -23,10 +23,10 @@ INT8_PEAK_TOPS = 5000.0  # MI355X dense int8 matrix peak, TOP/s
 HBM_PEAK_GBS = 8000.0    # MI355X HBM3E peak, GB/s
 # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs of this script, scaled by
 # what the same counters read for its 256 MiB device copy (profiles/gemm_q4k_prefill_m512_k4096_n12288.txt,
-# profiles/gemv_q4k_decode_m1_k4096.txt). Measured once, not live: counters need the profiler attached.
-TRAFFIC_GEMM_C2 = 62.07e6 + 25.17e6
+# profiles/gemv_q4k_decode_m1_k4096.txt, profiles/moe_block_q4k_64tok_128experts.txt). Measured once, not live: counters need the profiler attached.
+TRAFFIC_GEMM_C2 = 66.76e6 + 25.17e6
 TRAFFIC_GEMV_C2 = 28.42e6 + 0.05e6
-TRAFFIC_GEMV_LM_HEAD = 350.57e6 + 0.61e6
+TRAFFIC_GEMV_LM_HEAD = 354.17e6 + 0.61e6
 METRIC = "Q4 GEMV effective GB/s (%HBM peak); prefill GEMM int8 TOPS (%MFMA peak)"
 
 
@@ -150,6 +150,44 @@ def main():
     for w in big:
         w.destroy()
 
+    # ---- the MoE block of configs[3]: 64 tokens, 128 experts, top-8, Q4_K ----------
+    mt, mh, me, mi, mk = 64, 2048, 128, 768, 8
+
+    def mk_expert(n, k):
+        e32 = torch.randn((n, k), generator=gen, device="cuda", dtype=torch.float32) * 0.02
+        eb = torch.empty(capi.weight_nbytes("q4_K", n, k), dtype=torch.uint8, device="cuda")
+        capi.quantize_weights("q4_K", e32, n, k, eb, stream=stream)
+        torch.cuda.synchronize()
+        return capi.Weight("q4_K", n, k, eb, mem=capi.MEM_DEVICE)
+
+    # two sets of experts (2 x 340 MB) so that consecutive calls do not hit the last-level cache
+    sets = [([mk_expert(mi, mh) for _ in range(me)], [mk_expert(mi, mh) for _ in range(me)],
+             [mk_expert(mh, mi) for _ in range(me)]) for _ in range(2)]
+    mx = torch.randn((mt, mh), generator=gen, device="cuda")
+    ml = torch.randn((mt, me), generator=gen, device="cuda")
+    my = torch.empty((mt, mh), device="cuda")
+    midx = torch.zeros((mt, mk), dtype=torch.int32, device="cuda")
+    for i in range(4):
+        g_, u_, d_ = sets[i % 2]
+        capi.moe_forward(mt, mh, mi, me, mk, g_, u_, d_, mx, my, router_logits=ml, topk_idx=midx, stream=stream)
+    torch.cuda.synchronize()
+    active = int(torch.unique(midx).numel())
+    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    reps = 40
+    ev0.record()
+    for i in range(reps):
+        g_, u_, d_ = sets[i % 2]
+        capi.moe_forward(mt, mh, mi, me, mk, g_, u_, d_, mx, my, router_logits=ml, stream=stream)
+    ev1.record()
+    torch.cuda.synchronize()
+    moe_ms = ev0.elapsed_time(ev1) / reps
+    moe_bytes = active * 3 * (mi * mh * 144 // 256) + 2 * mt * mh * 4
+    moe_gbs = moe_bytes / (moe_ms * 1e-3) / 1e9
+    for st_ in sets:
+        for lst in st_:
+            for w_ in lst:
+                w_.destroy()
+
     # ---- a plain device copy of known size: the yardstick the FETCH_SIZE / WRITE_SIZE
     # counters of a profiled run of this script are scaled by
     src = torch.empty(256 << 20, dtype=torch.uint8, device="cuda")
@@ -183,10 +221,18 @@ def main():
                                      "algorithmic_bytes_per_launch": gv_bytes}},
         "decode_gemv_lm_head_size": {
             "workload": "Q4_K GEMV M=1 K=4096 N=151936, 3 weight copies rotated",
-            "roofline": {"bound": "hbm", "kernel": "gemv_kernel<Q4_K,T=64,R=1,G=4>",
+            "roofline": {"bound": "hbm", "kernel": "gemv_stream_kernel<Q4_K,G=4,GPW=2>",
                          "achieved": round(big_gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(big_gbs / HBM_PEAK_GBS, 5), "kernel_ms": round(big_ms, 5),
                          "traffic": TRAFFIC_GEMV_LM_HEAD, "algorithmic_bytes_per_launch": big_bytes}},
+        "moe_block": {
+            "workload": "MoE FFN block (BASELINE configs[3]): 64 tokens, hidden 2048, 128 experts x "
+                        "(gate/up 2048->768, down 768->2048) Q4_K, top-8; router, sort, experts, combine; "
+                        "two expert sets alternated; whole call incl. launches",
+            "ms_per_block": round(moe_ms, 5), "active_experts": active,
+            "roofline": {"bound": "hbm", "achieved": round(moe_gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                         "frac": round(moe_gbs / HBM_PEAK_GBS, 5), "algorithmic_bytes_per_block": moe_bytes,
+                         "traffic": 290.0e6 + 141.5e6 + 5.8e6}},
     }
     if not args.no_cpu:
         capi.matmul(weights[0], a, M, c, stream=stream)
