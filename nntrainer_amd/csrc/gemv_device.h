@@ -166,7 +166,7 @@ template <int T, int R, bool PW, int KC> struct GemvQ40 {
       if (i * T >= un) break;
       const int u = min(tl + i * T, un - 1);
       W.q[i] = hipq_ld_stream(qs + u);
-      W.d[i] = dw[u];
+      W.d[i] = hipq_ld_global(dw + u);
     }
   }
   __device__ static __forceinline__ void compute(const Wt &W, const Act &A, int tl, int kc,
@@ -246,7 +246,7 @@ template <int T, int R, bool PW, int KC> struct GemvQ4K {
       const int u = min(tl + i * T, un - 1);
       W.q0[i] = hipq_ld_stream(qs + 2 * u);
       W.q1[i] = hipq_ld_stream(qs + 2 * u + 1);
-      W.hd[i] = hdr[u >> 2];
+      W.hd[i] = hipq_ld_global(hdr + (u >> 2));
     }
   }
   __device__ static __forceinline__ void compute(const Wt &W, const Act &A, int tl, int kc,
@@ -358,8 +358,8 @@ template <int T, int R, bool PW, int KC> struct GemvQ6K {
       W.qa[i] = hipq_ld_stream((const uint4 *)ql);
       W.qb[i] = hipq_ld_stream((const uint4 *)(ql + 32));
       W.qh[i] = hipq_ld_stream((const uint4 *)(qhrow + b * 64 + half * 32 + hl * 16));
-      W.scw[i] = *(const int *)(scrow + b * 16 + uu * 4);
-      W.d[i] = drow[b];
+      W.scw[i] = hipq_ld_global((const int *)(scrow + b * 16 + uu * 4));
+      W.d[i] = hipq_ld_global(drow + b);
     }
   }
   __device__ static __forceinline__ void compute(const Wt &W, const Act &A, int tl, int kc,

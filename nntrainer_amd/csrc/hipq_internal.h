@@ -130,7 +130,15 @@ int launch_quantize_q8_0(const float *A, int64_t M, int64_t K, int64_t lda,
 int launch_quantize_q8_K(const float *A, int64_t M, int64_t K, int64_t lda,
                          int64_t mat_rows, const QAct *qa, void *canonical_out,
                          hipStream_t s);
-/* same values, written in the tiled form; rows M .. 128 * mtiles are zero-filled */
+/* Row quantizer into a QAct whose planes take the form the grouped MFMA expert
+ * kernels read: q row-major with every 16-value group stored as its 8 even then
+ * its 8 odd values, d as usual, and in place of bsum 16 fp16 per super-block:
+ * the eight sub-block sums split into a part in 0..63 (first 8) and a multiple
+ * of 64 (last 8). ql / qh are not written. */
+int launch_quantize_q8_K_rowmma(const float *A, int64_t M, int64_t K, int64_t lda, const QAct *qa,
+                                hipStream_t s);
+/* the values of launch_quantize_q8_K, written in the tiled form; rows M .. 128 * mtiles
+ * are zero-filled */
 int launch_quantize_q8_K_tiled(const float *A, int64_t M, int64_t K, int64_t lda,
                                int64_t mat_rows, const QActTiled *qa, hipStream_t s);
 
@@ -242,11 +250,26 @@ template <int T> __device__ __forceinline__ float hipq_group_max(float v) {
   return v;
 }
 
+/* Loads of weight data name the global address space. A pointer that a kernel
+ * read from memory (a table of weight views) is generic to the compiler, which
+ * then emits flat loads; those count against the LDS counter as well, so every
+ * wait for an LDS read would also wait for the weight prefetch. */
+#define HIPQ_GLOBAL __attribute__((address_space(1)))
+typedef unsigned int hipq_u32x4 __attribute__((ext_vector_type(4)));
+template <typename T> __device__ __forceinline__ T hipq_ld_global(const T *p) {
+  if constexpr (sizeof(T) == 16) {
+    return __builtin_bit_cast(T, *(const HIPQ_GLOBAL hipq_u32x4 *)p);
+  } else if constexpr (sizeof(T) == 4) {
+    return __builtin_bit_cast(T, *(const HIPQ_GLOBAL uint32_t *)p);
+  } else {
+    static_assert(sizeof(T) == 2, "16-, 4- and 2-byte loads only");
+    return __builtin_bit_cast(T, *(const HIPQ_GLOBAL uint16_t *)p);
+  }
+}
 /* 128-bit streaming load of weight data: marked non-temporal so the one-pass
  * weight stream does not evict the (re-used) quantized activations. */
-typedef unsigned int hipq_u32x4 __attribute__((ext_vector_type(4)));
 __device__ __forceinline__ uint4 hipq_ld_stream(const uint4 *p) {
-  hipq_u32x4 v = __builtin_nontemporal_load((const hipq_u32x4 *)p);
+  hipq_u32x4 v = __builtin_nontemporal_load((const HIPQ_GLOBAL hipq_u32x4 *)p);
   return make_uint4(v.x, v.y, v.z, v.w);
 }
 

@@ -38,7 +38,8 @@ struct MoeBufs {
   int32_t *idx;
   float *wgt;
   int *counts, *offsets, *cursor;
-  int *slot_pair, *pair_slot;
+  int *slot_pair; /* pair (token * topk + k) of each slot */
+  int *tok_slots; /* [T][topk]: a token's slots in ascending expert id */
   float *h;       /* [P][I] by slot */
   float *contrib; /* [P][H] by slot */
   void *xq_mem, *hq_mem;
@@ -70,7 +71,7 @@ size_t carve(const hipq_moe_desc &d, int is_k, uint8_t *base, MoeBufs *b) {
   p = take(P * 4);
   if (b) b->slot_pair = (int *)p;
   p = take(P * 4);
-  if (b) b->pair_slot = (int *)p;
+  if (b) b->tok_slots = (int *)p;
   p = take(P * I * 4);
   if (b) b->h = (float *)p;
   p = take(P * H * 4);
@@ -107,25 +108,32 @@ __global__ __launch_bounds__(256) void route_kernel(const float *__restrict__ lo
   float p[MAXV];
   const float *lg = logits + (size_t)t * E;
   float mx = -INFINITY;
+  /* the guards on 64 * i are uniform: rounds past E cost nothing (the double
+   * exponential is a few hundred instructions) */
 #pragma unroll
   for (int i = 0; i < MAXV; ++i) {
-    const int e = lane + 64 * i;
-    p[i] = e < E ? lg[e] : -INFINITY;
-    mx = fmaxf(mx, p[i]);
+    p[i] = -INFINITY;
+    if (64 * i < E) {
+      const int e = lane + 64 * i;
+      if (e < E) p[i] = lg[e];
+      mx = fmaxf(mx, p[i]);
+    }
   }
   mx = hipq_group_max<64>(mx);
   float sum = 0.f;
 #pragma unroll
   for (int i = 0; i < MAXV; ++i) {
-    const int e = lane + 64 * i;
-    p[i] = e < E ? (float)exp((double)(p[i] - mx)) : 0.f;
-    sum += p[i];
+    if (64 * i < E) {
+      const int e = lane + 64 * i;
+      p[i] = e < E ? (float)exp((double)(p[i] - mx)) : 0.f;
+      sum += p[i];
+    }
   }
   sum = hipq_group_sum<64>(sum);
 #pragma unroll
   for (int i = 0; i < MAXV; ++i) {
     const int e = lane + 64 * i;
-    p[i] = e < E ? __fdiv_rn(p[i], sum) : -1.f; /* -1: never selected */
+    p[i] = (64 * i < E && e < E) ? __fdiv_rn(p[i], sum) : -1.f; /* -1: never selected */
   }
   float ksum = 0.f;
   float myw = 0.f; /* lane kk keeps the kk-th weight */
@@ -136,20 +144,22 @@ __global__ __launch_bounds__(256) void route_kernel(const float *__restrict__ lo
 #pragma unroll
     for (int i = 0; i < MAXV; ++i) {
       const int e = lane + 64 * i;
-      if (p[i] > bv) { /* ascending e within the lane: first maximum wins */
+      if (64 * i < E && p[i] > bv) { /* ascending e within the lane: first maximum wins */
         bv = p[i];
         bi = e;
       }
     }
-#pragma unroll
-    for (int off = 1; off < 64; off <<= 1) {
-      const float ov = __shfl_xor(bv, off, 64);
-      const int oi = __shfl_xor(bi, off, 64);
-      if (ov > bv || (ov == bv && oi < bi)) {
-        bv = ov;
-        bi = oi;
-      }
-    }
+    /* the wavefront's maximum, then the lowest expert id that holds it */
+    const float mxv = hipq_group_max<64>(bv);
+    int cand = bv == mxv ? bi : 0x7fffffff;
+    cand = min(cand, hipq_dpp_i<HIPQ_DPP_XOR1>(cand));
+    cand = min(cand, hipq_dpp_i<HIPQ_DPP_XOR2>(cand));
+    cand = min(cand, hipq_dpp_i<HIPQ_DPP_HALF_MIRROR>(cand));
+    cand = min(cand, hipq_dpp_i<HIPQ_DPP_MIRROR>(cand));
+    cand = min(cand, __shfl_xor(cand, 16, 64));
+    cand = min(cand, __shfl_xor(cand, 32, 64));
+    bv = mxv;
+    bi = cand;
     /* every lane now agrees on (bv, bi); retire it in its owner */
     if ((bi & 63) == lane) {
 #pragma unroll
@@ -168,13 +178,24 @@ __global__ __launch_bounds__(256) void route_kernel(const float *__restrict__ lo
   }
 }
 
+/* Where the slot of pair i goes in tok_slots: a token's slots in ascending expert
+ * id, the order in which its contributions are added. */
+__device__ __forceinline__ int rank_in_token(const int32_t *__restrict__ idx, int i, int topk) {
+  const int t = i / topk;
+  const int e = idx[i];
+  int r = 0;
+  for (int j = 0; j < topk; ++j) r += idx[t * topk + j] < e;
+  return t * topk + r;
+}
+
 /* Count, scan and scatter of the (token, k) pairs by expert in one workgroup:
  * the sort of a decode step or a short prefill chunk is a few thousand pairs, and
  * four tiny launches would cost more than the work. E <= 1024. */
 __global__ __launch_bounds__(1024) void sort_pairs_kernel(const int32_t *__restrict__ idx, int P,
-                                                          int E, int *__restrict__ offsets,
+                                                          int E, int topk,
+                                                          int *__restrict__ offsets,
                                                           int *__restrict__ slot_pair,
-                                                          int *__restrict__ pair_slot) {
+                                                          int *__restrict__ tok_slots) {
   __shared__ int cnt[1024];
   __shared__ int off[1024];
   const int t = threadIdx.x;
@@ -203,7 +224,7 @@ __global__ __launch_bounds__(1024) void sort_pairs_kernel(const int32_t *__restr
     const int e = idx[i];
     const int slot = off[e] + atomicAdd(&cnt[e], 1);
     slot_pair[slot] = i;
-    pair_slot[i] = slot;
+    tok_slots[rank_in_token(idx, i, topk)] = slot;
   }
 }
 
@@ -230,15 +251,15 @@ __global__ void scan_kernel(const int *__restrict__ counts, int E, int *__restri
   }
 }
 
-__global__ void scatter_kernel(const int32_t *__restrict__ idx, int P,
+__global__ void scatter_kernel(const int32_t *__restrict__ idx, int P, int topk,
                                const int *__restrict__ offsets, int *__restrict__ cursor,
-                               int *__restrict__ slot_pair, int *__restrict__ pair_slot) {
+                               int *__restrict__ slot_pair, int *__restrict__ tok_slots) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= P) return;
   const int e = idx[i];
   const int slot = offsets[e] + atomicAdd(&cursor[e], 1);
   slot_pair[slot] = i;
-  pair_slot[i] = slot;
+  tok_slots[rank_in_token(idx, i, topk)] = slot;
 }
 
 __device__ __forceinline__ float silu_ref(float g) {
@@ -402,30 +423,416 @@ __global__ __launch_bounds__(256) void down_long_kernel(const WView *__restrict_
   }
 }
 
+/* ---- Q4_K experts on the matrix cores --------------------------------------------
+ *
+ * With a handful of tokens per expert the products above redo the nibble unpacking
+ * per token group. Here a wavefront owns 32 weight rows and up to 32 tokens and
+ * forms the 32 x 32 integer block sums of a super-block with
+ * v_mfma_i32_32x32x32_i8: the tokens' Q8_K values are the row operand (from LDS,
+ * staged once per workgroup), the weights the column operand, expanded in registers
+ * from the packed nibbles into two digit planes (scale = 8 * high digit + low
+ * digit, as the prefill GEMM does). Lane (n, g) holds the 64 bytes of sub-blocks
+ * 4g .. 4g+3 of weight row n; a matrix step takes 16 consecutive weights per lane,
+ * even ones (low nibbles) in operand bytes 0-7 and odd ones in bytes 8-15, and the
+ * quantizer stores every 16-value group of the activations in that order. The mins
+ * go through one v_mfma_f32_32x32x16_f16 per super-block with the sub-block sums
+ * split into two fp16-exact parts. Every integer is exact and the fp32 chain per
+ * output is the single-row kernel's, so the results carry the same bits:
+ *   acc = fma(float(I), d * dA, acc); accm = fma(float(Im), dmin * dA, accm). */
+typedef int mv4i __attribute__((ext_vector_type(4)));
+typedef int mv16i __attribute__((ext_vector_type(16)));
+typedef float mv16f __attribute__((ext_vector_type(16)));
+typedef _Float16 mv8h __attribute__((ext_vector_type(8)));
+typedef unsigned short mv2us __attribute__((ext_vector_type(2)));
+
+__device__ __forceinline__ uint32_t mma_pk_scale(uint32_t x, uint32_t digit2) {
+  const mv2us r = __builtin_bit_cast(mv2us, x) * __builtin_bit_cast(mv2us, digit2);
+  return __builtin_bit_cast(uint32_t, r);
+}
+
+/* LDS of a workgroup: TC activation rows, padded so that the lanes of a 128-bit
+ * read fall into different banks, then one ring of weight tiles per wavefront. */
+constexpr int XDEPTH = 3;       /* super-blocks of weights in the ring of a wavefront */
+constexpr int XTILE = 32 * 128 + 64 * 16; /* nibbles of 32 weight rows for one super-block, then their headers (twice) */
+struct XLds {
+  int8_t *q;           /* [TC][K + 16] */
+  uint8_t *amin;       /* [TC][nsb][32 bytes] */
+  float *dA;           /* [nsb][TC] */
+  int *rows;           /* [TC] source rows of the chunk */
+  unsigned char *ring; /* this wavefront's [XDEPTH][XTILE] */
+};
+__host__ __device__ inline size_t xlds_act_bytes(int TC, int K) {
+  const size_t b = (size_t)TC * (K + 16) + (size_t)TC * (K / 256) * 32 + (size_t)TC * (K / 256) * 4 + TC * 4;
+  return (b + 255) & ~(size_t)255;
+}
+__host__ __device__ inline size_t xlds_bytes(int TC, int K) {
+  return xlds_act_bytes(TC, K) + 4 * XDEPTH * XTILE;
+}
+__device__ __forceinline__ XLds xlds_carve(unsigned char *base, int TC, int K, int wave) {
+  XLds l;
+  l.q = (int8_t *)base;
+  l.amin = (uint8_t *)base + (size_t)TC * (K + 16);
+  l.dA = (float *)(l.amin + (size_t)TC * (K / 256) * 32);
+  l.rows = (int *)(l.dA + (size_t)TC * (K / 256));
+  l.ring = base + xlds_act_bytes(TC, K) + wave * (XDEPTH * XTILE);
+  return l;
+}
+
+/* Copy the chunk's activation rows (l.rows, already in LDS) from the planes of a.
+ * Loads are issued four at a time before their stores so that their latencies overlap. */
+template <int TC>
+__device__ __forceinline__ void stage_rows(const XLds &l, const QView &a) {
+  const int K = a.K, nsb = K >> 8;
+  const int cpr = K >> 4; /* 16-byte pieces per row */
+  const int nt = blockDim.x;
+  for (int c0 = threadIdx.x; c0 < TC * cpr; c0 += 4 * nt) {
+    mv4i v0, v1, v2, v3;
+    int d0, d1, d2, d3;
+    auto ld = [&](int u, mv4i &v, int &dst) {
+      const int c = min(c0 + u * nt, TC * cpr - 1);
+      const int r = c / cpr, o = c - r * cpr;
+      v = *(const mv4i *)(a.q + (size_t)l.rows[r] * K + o * 16);
+      dst = r * (K + 16) + o * 16;
+    };
+    ld(0, v0, d0), ld(1, v1, d1), ld(2, v2, d2), ld(3, v3, d3);
+    *(mv4i *)(l.q + d0) = v0;
+    if (c0 + nt < TC * cpr) *(mv4i *)(l.q + d1) = v1;
+    if (c0 + 2 * nt < TC * cpr) *(mv4i *)(l.q + d2) = v2;
+    if (c0 + 3 * nt < TC * cpr) *(mv4i *)(l.q + d3) = v3;
+  }
+  for (int c = threadIdx.x; c < TC * nsb * 2; c += nt) {
+    const int r = c / (nsb * 2), o = c - r * (nsb * 2);
+    const mv4i v = *(const mv4i *)((const uint8_t *)a.bsum + ((size_t)l.rows[r] * nsb) * 32 + o * 16);
+    *(mv4i *)(l.amin + ((size_t)r * nsb) * 32 + o * 16) = v;
+  }
+  for (int c = threadIdx.x; c < TC * nsb; c += nt) {
+    const int r = c / nsb, b = c - r * nsb;
+    l.dA[b * TC + r] = a.d[(size_t)l.rows[r] * nsb + b];
+  }
+}
+
+/* The weight stream of a wavefront. A super-block of a tile's 32 rows is 32 lines of
+ * 128 bytes; four direct-to-LDS copies fetch 8 whole lines each (8 lanes per line:
+ * fully coalesced) into the next ring slot, so no registers hold weights in flight
+ * and the ring can run several super-blocks ahead. Lane L of copy i fetches piece
+ * (L % 8) ^ (L / 8) of row 8i + L / 8 and the hardware stores it at slot byte
+ * 1024 i + 16 L: row r of the slot holds its eight 16-byte pieces XOR-swizzled by
+ * r % 8, which spreads the later 128-bit reads of a column of pieces over the banks.
+ * A fifth copy brings each lane the 16-byte header of its row. */
+typedef __amdgpu_buffer_rsrc_t xrsrc_t;
+struct XStream {
+  xrsrc_t rs;       /* the tile's nibble plane */
+  uint32_t voff[4]; /* this lane's byte offset for each of the four copies, super-block 0 */
+  uint32_t so;      /* + byte offset of the super-block under the cursor */
+  xrsrc_t rh;       /* the tile's header plane */
+  uint32_t hoff;    /* this lane's row (lane % 32) in it, super-block 0 */
+  uint32_t hso;     /* + byte offset of the super-block under the cursor */
+};
+__device__ __forceinline__ void xs_open(XStream &x, const WView &w, int col0, int lane) {
+  x.rs = __builtin_amdgcn_make_buffer_rsrc((void *)w.qs, 0, (int)((size_t)w.N * (w.K >> 1)), 0x00020000);
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    const int r = 8 * i + (lane >> 3);
+    const int n = min(col0 + r, (int)w.N - 1);
+    x.voff[i] = (uint32_t)n * (uint32_t)(w.K >> 1) + (uint32_t)(((lane & 7) ^ (lane >> 3)) * 16);
+  }
+  x.so = 0;
+  x.rh = __builtin_amdgcn_make_buffer_rsrc((void *)w.hdr, 0, (int)((size_t)w.N * (w.K >> 8) * 16), 0x00020000);
+  x.hoff = (uint32_t)min(col0 + (lane & 31), (int)w.N - 1) * (uint32_t)((w.K >> 8) * 16);
+  x.hso = 0;
+}
+__device__ __forceinline__ void xs_fetch(XStream &x, unsigned char *slot) {
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(x.rs, (__attribute__((address_space(3))) void *)(slot + i * 1024),
+                                             16, (int)x.voff[i], (int)x.so, 0, 0);
+  __builtin_amdgcn_raw_ptr_buffer_load_lds(x.rh, (__attribute__((address_space(3))) void *)(slot + 4096), 16,
+                                           (int)x.hoff, (int)x.hso, 0, 0);
+}
+__device__ __forceinline__ void xs_advance(XStream &x) {
+  x.so += 128;
+  x.hso += 16;
+}
+constexpr int XS_OPS = 5; /* loads one xs_fetch issues */
+
+/* One super-block: acc / accm += for the NREG accumulator registers of this lane
+ * (register r is token 8 * (r / 4) + 4g + r % 4, the lane's column n). `slot` holds
+ * the nibbles and headers (its copies have landed). */
+template <int TC, int NREG>
+__device__ __forceinline__ void xw_super_block(const unsigned char *slot, const XLds &l, int K, int sb,
+                                               int i32, int g, float (&acc)[NREG], float (&accm)[NREG]) {
+  const mv16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  const mv16f zero16f = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+  const int nsb = K >> 8;
+  /* All LDS operands of the super-block in one go: this lane's 64 bytes of nibbles
+   * (pieces 4g .. 4g+3 of row i32), the eight 16-byte row operands of its token, the
+   * token's split sub-block sums and the block scales of its NREG tokens. The
+   * compiler must not see these reads: it orders every LDS read it knows of after
+   * the direct-to-LDS copies it may alias, which would drain the ring. */
+  const int row = i32 & (TC - 1);
+  mv4i wq[4], a8[8], aminv, hdv, dv[NREG / 4];
+  {
+    auto lds = [](const void *p) { return (uint32_t)(size_t)(const __attribute__((address_space(3))) void *)p; };
+    const uint32_t rowb = lds(slot) + i32 * 128;
+    const uint32_t x7 = i32 & 7;
+    const uint32_t a0 = rowb + (((4 * g + 0) ^ x7) << 4), a1 = rowb + (((4 * g + 1) ^ x7) << 4);
+    const uint32_t a2 = rowb + (((4 * g + 2) ^ x7) << 4), a3 = rowb + (((4 * g + 3) ^ x7) << 4);
+    const uint32_t pa = lds(l.q) + row * (K + 16) + sb * 256 + g * 128;
+    const uint32_t pm = lds(l.amin) + (row * nsb + sb) * 32 + g * 16;
+    const uint32_t pd = lds(l.dA) + (sb * TC + 4 * g) * 4;
+    asm volatile("ds_read_b128 %0, %4\n\tds_read_b128 %1, %5\n\tds_read_b128 %2, %6\n\tds_read_b128 %3, %7"
+                 : "=&v"(wq[0]), "=&v"(wq[1]), "=&v"(wq[2]), "=&v"(wq[3])
+                 : "v"(a0), "v"(a1), "v"(a2), "v"(a3)
+                 : "memory");
+    asm volatile("ds_read_b128 %0, %8\n\tds_read_b128 %1, %8 offset:16\n\tds_read_b128 %2, %8 offset:32\n\t"
+                 "ds_read_b128 %3, %8 offset:48\n\tds_read_b128 %4, %8 offset:64\n\tds_read_b128 %5, %8 offset:80\n\t"
+                 "ds_read_b128 %6, %8 offset:96\n\tds_read_b128 %7, %8 offset:112"
+                 : "=&v"(a8[0]), "=&v"(a8[1]), "=&v"(a8[2]), "=&v"(a8[3]), "=&v"(a8[4]), "=&v"(a8[5]),
+                   "=&v"(a8[6]), "=&v"(a8[7])
+                 : "v"(pa)
+                 : "memory");
+    asm volatile("ds_read_b128 %0, %1" : "=&v"(aminv) : "v"(pm) : "memory");
+    asm volatile("ds_read_b128 %0, %1 offset:4096" : "=&v"(hdv) : "v"(lds(slot) + (i32 + 32 * g) * 16) : "memory");
+#pragma unroll
+    for (int q4 = 0; q4 < NREG / 4; ++q4)
+      asm volatile("ds_read_b128 %0, %1" : "=&v"(dv[q4]) : "v"(pd + q4 * 32) : "memory");
+    /* every register above is named so that nothing reads one before the wait */
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(wq[0]), "+v"(wq[1]), "+v"(wq[2]), "+v"(wq[3]), "+v"(a8[0]), "+v"(a8[1]), "+v"(a8[2]),
+                   "+v"(a8[3]), "+v"(a8[4]), "+v"(a8[5]), "+v"(a8[6]), "+v"(a8[7]), "+v"(aminv), "+v"(hdv)
+                 :
+                 : "memory");
+#pragma unroll
+    for (int q4 = 0; q4 < NREG / 4; ++q4) asm volatile("" : "+v"(dv[q4]));
+  }
+  const uint4 hd = make_uint4((uint32_t)hdv[0], (uint32_t)hdv[1], (uint32_t)hdv[2], (uint32_t)hdv[3]);
+  /* 6-bit scales of sub-blocks 4g .. 4g+3, one per byte, as two 3-bit digits */
+  const uint32_t s03 = hd.y & 0x3f3f3f3fu;
+  const uint32_t s47 = (hd.w & 0x0f0f0f0fu) | ((hd.y >> 2) & 0x30303030u);
+  const uint32_t sc = g ? s47 : s03;
+  const uint32_t slo = sc & 0x07070707u, shi = (sc >> 3) & 0x07070707u;
+  const mv8h amin = __builtin_bit_cast(mv8h, aminv);
+  mv16i Dlo = zero16, Dhi = zero16;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    /* digit of sub-block 4g + j in both 16-bit halves */
+    const uint32_t dl = __builtin_amdgcn_perm(slo, slo, 0x0c000c00u | (uint32_t)j | ((uint32_t)j << 16));
+    const uint32_t dh = __builtin_amdgcn_perm(shi, shi, 0x0c000c00u | (uint32_t)j | ((uint32_t)j << 16));
+#pragma unroll
+    for (int half = 0; half < 2; ++half) {
+      const uint32_t x0 = (uint32_t)wq[j][2 * half], x1 = (uint32_t)wq[j][2 * half + 1];
+      const uint32_t e0 = x0 & HIPQ_M4, e1 = x1 & HIPQ_M4;
+      const uint32_t o0 = (x0 >> 4) & HIPQ_M4, o1 = (x1 >> 4) & HIPQ_M4;
+      const mv4i bl = {(int)mma_pk_scale(e0, dl), (int)mma_pk_scale(e1, dl), (int)mma_pk_scale(o0, dl),
+                       (int)mma_pk_scale(o1, dl)};
+      const mv4i bh = {(int)mma_pk_scale(e0, dh), (int)mma_pk_scale(e1, dh), (int)mma_pk_scale(o0, dh),
+                       (int)mma_pk_scale(o1, dh)};
+      const mv4i a = a8[j * 2 + half];
+      Dlo = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, bl, Dlo, 0, 0, 0);
+      Dhi = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, bh, Dhi, 0, 0, 0);
+    }
+  }
+  /* mins: sum_j m_j * bsum_j, the low parts of bsum in lanes 0-31, the high parts in 32-63 */
+  const uint32_t mlo = hd.z & 0x3f3f3f3fu;
+  const uint32_t mhi = ((hd.w >> 4) & 0x0f0f0f0fu) | ((hd.z >> 2) & 0x30303030u);
+  mv8h bmin;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    bmin[j] = (_Float16)(float)((mlo >> (8 * j)) & 0xff);
+    bmin[4 + j] = (_Float16)(float)((mhi >> (8 * j)) & 0xff);
+  }
+  const mv16f Sm = __builtin_amdgcn_mfma_f32_32x32x16_f16(amin, bmin, zero16f, 0, 0, 0);
+  const float dw = hipq_h2f((uint16_t)(hd.x & 0xffff));
+  const float dmin = hipq_h2f((uint16_t)(hd.x >> 16));
+#pragma unroll
+  for (int q4 = 0; q4 < NREG / 4; ++q4) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int r = 4 * q4 + e;
+      const float dA = __int_as_float(dv[q4][e]);
+      const int I = (Dhi[r] << 3) + Dlo[r];
+      acc[r] = fmaf((float)I, dw * dA, acc[r]);
+      accm[r] = fmaf(Sm[r], dmin * dA, accm[r]);
+    }
+  }
+}
+
+/* A run of column tiles (matrix, first column) for one wavefront: the weights of
+ * the next XDEPTH - 1 super-blocks, also across tiles, are in flight while one is
+ * computed. tile_of(t, &view, &col0) names tile t; done(t, out) receives its NREG
+ * results. Loads retire in issue order, so waiting until at most the loads of the
+ * younger fetches are outstanding means the oldest fetch has landed. */
+template <int TC, int NREG, typename TileOf, typename Done>
+__device__ __forceinline__ void xw_run(int ntile, const XLds &l, int K, TileOf tile_of, Done done) {
+  static_assert(XDEPTH == 3, "the loop below is unrolled for a ring of three");
+  const int lane = threadIdx.x & 63, i32 = lane & 31, g = lane >> 5;
+  const int nsb = K >> 8;
+  const int nv = ntile * nsb;
+  XStream xs;
+  int lt = 0, lsb = 0; /* tile and super-block under the cursor */
+  int issued = 0;      /* fetches issued so far */
+  {
+    WView lw;
+    int c0;
+    tile_of(0, lw, c0);
+    xs_open(xs, lw, c0, lane);
+  }
+  /* Always issues its five loads, so that the number of loads in flight at any
+   * point of the loop is fixed; past the end of the stream it fetches the last
+   * super-block again, into a slot nobody reads any more. */
+  auto fetch = [&](unsigned char *slot) {
+    xs_fetch(xs, slot);
+    if (++issued >= nv) return; /* uniform: the cursor stays on the last super-block */
+    if (++lsb == nsb) {
+      lsb = 0;
+      ++lt;
+      WView lw;
+      int c0;
+      tile_of(lt, lw, c0);
+      xs_open(xs, lw, c0, lane);
+    } else {
+      xs_advance(xs);
+    }
+  };
+  unsigned char *const s0 = l.ring, *const s1 = l.ring + XTILE, *const s2 = l.ring + 2 * XTILE;
+  fetch(s0);
+  fetch(s1);
+  int t = 0, sb = 0, v = 0;
+  float acc[NREG], accm[NREG];
+  auto step = [&](const unsigned char *cur, unsigned char *nxt) {
+    if (sb == 0) {
+#pragma unroll
+      for (int r = 0; r < NREG; ++r) acc[r] = accm[r] = 0.f;
+    }
+    fetch(nxt); /* into the slot consumed by the previous step */
+    /* the fetch of this step has landed once only the two later ones are outstanding */
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * XS_OPS) : "memory");
+    xw_super_block<TC, NREG>(cur, l, K, sb, i32, g, acc, accm);
+    ++v;
+    if (++sb == nsb) {
+      float out[NREG];
+#pragma unroll
+      for (int r = 0; r < NREG; ++r) out[r] = acc[r] - accm[r];
+      done(t, out);
+      sb = 0;
+      ++t;
+    }
+  };
+  while (v < nv) {
+    step(s0, s2);
+    if (v < nv) step(s1, s0);
+    if (v < nv) step(s2, s1);
+  }
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); /* no copy may land after the ring is given up */
+}
+
+/* h[slot][col] = silu(x_tok . Wgate[e][col]) * (x_tok . Wup[e][col]): a workgroup
+ * serves one expert and 128 columns (32 per wavefront, the gate tile then the up
+ * tile), the expert's tokens in chunks of TC. */
+template <int TC>
+__global__ __launch_bounds__(256) void gate_up_mma_kernel(const WView *__restrict__ views, int E_,
+                                                          QView xq, const int *__restrict__ offsets,
+                                                          const int *__restrict__ slot_pair, int topk,
+                                                          int I, float *__restrict__ h) {
+  constexpr int NREG = TC / 2;
+  extern __shared__ __attribute__((aligned(16))) unsigned char xmoe_lds[];
+  const int e = blockIdx.y;
+  const int begin = offsets[e], end = offsets[e + 1];
+  if (begin == end) return; /* uniform per workgroup */
+  const WView wg = views[e], wu = views[E_ + e];
+  const int K = wg.K;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const XLds l = xlds_carve(xmoe_lds, TC, K, wave);
+  const int col0 = (blockIdx.x * 4 + wave) * 32;
+  for (int s0 = begin; s0 < end; s0 += TC) {
+    __syncthreads(); /* the previous chunk is no longer read */
+    if (threadIdx.x < TC) l.rows[threadIdx.x] = slot_pair[min(s0 + (int)threadIdx.x, end - 1)] / topk;
+    __syncthreads();
+    stage_rows<TC>(l, xq);
+    __syncthreads();
+    if (col0 >= I) continue; /* uniform per wavefront; it still takes part in the barriers */
+    float gate[NREG];
+    xw_run<TC, NREG>(
+      2, l, K,
+      [&](int t, WView &w, int &c0) {
+        w = t ? wu : wg;
+        c0 = col0;
+      },
+      [&](int t, const float(&out)[NREG]) {
+        if (t == 0) {
+#pragma unroll
+          for (int r = 0; r < NREG; ++r) gate[r] = out[r];
+        } else {
+          const int col = col0 + (lane & 31);
+#pragma unroll
+          for (int r = 0; r < NREG; ++r) {
+            const int tok = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+            if (col < I && s0 + tok < end) h[(size_t)(s0 + tok) * I + col] = silu_ref(gate[r]) * out[r];
+          }
+        }
+      });
+  }
+}
+
+/* contrib[slot][col] = (h_slot . Wdown[e][col]) * weight(pair): CT column tiles per wavefront */
+template <int TC, int CT>
+__global__ __launch_bounds__(256) void down_mma_kernel(const WView *__restrict__ views, int E_, QView hq,
+                                                       const int *__restrict__ offsets,
+                                                       const int *__restrict__ slot_pair,
+                                                       const float *__restrict__ wgt, int H,
+                                                       float *__restrict__ contrib) {
+  constexpr int NREG = TC / 2;
+  extern __shared__ __attribute__((aligned(16))) unsigned char xmoe_lds[];
+  const int e = blockIdx.y;
+  const int begin = offsets[e], end = offsets[e + 1];
+  if (begin == end) return;
+  const WView wd = views[2 * E_ + e];
+  const int K = wd.K;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const XLds l = xlds_carve(xmoe_lds, TC, K, wave);
+  const int col0 = (blockIdx.x * 4 + wave) * 32 * CT;
+  const int ntile = min(CT, (H - col0 + 31) / 32);
+  for (int s0 = begin; s0 < end; s0 += TC) {
+    __syncthreads();
+    if (threadIdx.x < TC) l.rows[threadIdx.x] = min(s0 + (int)threadIdx.x, end - 1); /* hq rows are slots */
+    __syncthreads();
+    stage_rows<TC>(l, hq);
+    __syncthreads();
+    if (ntile <= 0) continue;
+    xw_run<TC, NREG>(
+      ntile, l, K,
+      [&](int t, WView &w, int &c0) {
+        w = wd;
+        c0 = col0 + 32 * t;
+      },
+      [&](int t, const float(&out)[NREG]) {
+        const int col = col0 + 32 * t + (lane & 31);
+#pragma unroll
+        for (int r = 0; r < NREG; ++r) {
+          const int tok = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+          if (col < H && s0 + tok < end)
+            contrib[(size_t)(s0 + tok) * H + col] = out[r] * wgt[slot_pair[s0 + tok]];
+        }
+      });
+  }
+}
+
 /* y[t][c] = sum of the token's contributions, ascending expert id */
-__global__ __launch_bounds__(256) void combine_kernel(const int32_t *__restrict__ idx,
-                                                      const int *__restrict__ pair_slot, int topk,
+__global__ __launch_bounds__(256) void combine_kernel(const int *__restrict__ tok_slots, int topk,
                                                       int H, const float *__restrict__ contrib,
                                                       float *__restrict__ y) {
   const int t = blockIdx.y;
   const int c = blockIdx.x * blockDim.x + threadIdx.x;
   if (c >= H) return;
-  int ord[32];
-  for (int k = 0; k < topk; ++k) ord[k] = k;
-  for (int a = 1; a < topk; ++a) { /* insertion sort by expert id */
-    const int v = ord[a];
-    const int ev = idx[(size_t)t * topk + v];
-    int b = a - 1;
-    while (b >= 0 && idx[(size_t)t * topk + ord[b]] > ev) {
-      ord[b + 1] = ord[b];
-      --b;
-    }
-    ord[b + 1] = v;
-  }
   float acc = 0.f;
-  for (int k = 0; k < topk; ++k) {
-    const int slot = pair_slot[t * topk + ord[k]];
-    acc = acc + contrib[(size_t)slot * H + c];
+  for (int k0 = 0; k0 < topk; k0 += 8) { /* eight loads in flight, added in order */
+    float v[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+      v[k] = k0 + k < topk ? contrib[(size_t)tok_slots[t * topk + k0 + k] * H + c] : 0.f;
+#pragma unroll
+    for (int k = 0; k < 8; ++k)
+      if (k0 + k < topk) acc = acc + v[k];
   }
   y[(size_t)t * H + c] = acc;
 }
@@ -501,6 +908,41 @@ template <int DT> struct DownLauncher {
   template <int T, int KC, int G> void operator()() const { launch_down<DT, T, KC, G>(d, views, hq, b, s); }
 };
 
+/* Token chunk of the MFMA expert kernels for P pairs over E experts: the smallest
+ * of 8, 16, 32 that holds twice the mean tokens per expert (larger groups loop). */
+int mma_chunk(int64_t P, int E) {
+  const int64_t mean2 = (2 * P + E - 1) / E;
+  return mean2 <= 8 ? 8 : mean2 <= 16 ? 16 : 32;
+}
+bool use_mma(const hipq_moe_desc &d, int dt) {
+  return dt == HIPQ_Q4_K && d.hidden <= 4096 && d.intermediate <= 4096;
+}
+
+template <int TC>
+int launch_grouped_mma(const hipq::MoeArgs *a, const MoeBufs &b, const WView *views, const QAct &xq,
+                       const QAct &hq, hipStream_t s) {
+  const hipq_moe_desc &d = a->desc;
+  const int64_t P = (int64_t)d.tokens * d.topk;
+  constexpr int CT = 2;
+  const size_t lds_gu = xlds_bytes(TC, d.hidden), lds_dn = xlds_bytes(TC, d.intermediate);
+  if (lds_gu > 64 * 1024) /* beyond the default limit of a launch */
+    HIPQ_HIP(hipFuncSetAttribute((const void *)gate_up_mma_kernel<TC>,
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_gu));
+  if (lds_dn > 64 * 1024)
+    HIPQ_HIP(hipFuncSetAttribute((const void *)down_mma_kernel<TC, CT>,
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dn));
+  hipLaunchKernelGGL((gate_up_mma_kernel<TC>), dim3((d.intermediate + 127) / 128, d.experts), dim3(256), lds_gu,
+                     s, views, d.experts, qview(xq), b.offsets, b.slot_pair, d.topk, d.intermediate, b.h);
+  HIPQ_HIP(hipGetLastError());
+  int rc = hipq::launch_quantize_q8_K_rowmma(b.h, P, d.intermediate, d.intermediate, &hq, s);
+  if (rc) return rc;
+  hipLaunchKernelGGL((down_mma_kernel<TC, CT>), dim3((d.hidden + 128 * CT - 1) / (128 * CT), d.experts),
+                     dim3(256), lds_dn, s, views, d.experts, qview(hq), b.offsets, b.slot_pair, b.wgt,
+                     d.hidden, b.contrib);
+  HIPQ_HIP(hipGetLastError());
+  return HIPQ_OK;
+}
+
 template <int DT>
 int launch_grouped(const hipq::MoeArgs *a, const MoeBufs &b, const WView *views, const QAct &xq,
                    const QAct &hq, hipStream_t s) {
@@ -556,31 +998,38 @@ int launch_moe(const MoeArgs *a, void *workspace, size_t workspace_bytes, const 
   HIPQ_HIP(hipGetLastError());
   b.wgt = wgt;
   if (P <= 16384 && E <= 1024) {
-    hipLaunchKernelGGL(sort_pairs_kernel, dim3(1), dim3(1024), 0, s, idx, P, E, b.offsets, b.slot_pair,
-                       b.pair_slot);
+    hipLaunchKernelGGL(sort_pairs_kernel, dim3(1), dim3(1024), 0, s, idx, P, E, d.topk, b.offsets,
+                       b.slot_pair, b.tok_slots);
   } else {
     hipLaunchKernelGGL(fill_int_kernel, dim3((E + 255) / 256), dim3(256), 0, s, b.counts, E, 0);
     hipLaunchKernelGGL(count_kernel, dim3((P + 255) / 256), dim3(256), 0, s, idx, P, b.counts);
     hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(64), 0, s, b.counts, E, b.offsets, b.cursor);
-    hipLaunchKernelGGL(scatter_kernel, dim3((P + 255) / 256), dim3(256), 0, s, idx, P, b.offsets,
-                       b.cursor, b.slot_pair, b.pair_slot);
+    hipLaunchKernelGGL(scatter_kernel, dim3((P + 255) / 256), dim3(256), 0, s, idx, P, d.topk, b.offsets,
+                       b.cursor, b.slot_pair, b.tok_slots);
   }
   HIPQ_HIP(hipGetLastError());
 
   QAct xq = qact_carve(is_k, b.xq_mem, T, d.hidden);
   QAct hq = qact_carve(is_k, b.hq_mem, P, d.intermediate);
-  int rc = is_k ? launch_quantize_q8_K(a->x, T, d.hidden, d.hidden, 0, &xq, nullptr, s)
-                : launch_quantize_q8_0(a->x, T, d.hidden, d.hidden, &xq, nullptr, s);
+  const bool mma = use_mma(d, dt);
+  int rc = mma    ? launch_quantize_q8_K_rowmma(a->x, T, d.hidden, d.hidden, &xq, s)
+           : is_k ? launch_quantize_q8_K(a->x, T, d.hidden, d.hidden, 0, &xq, nullptr, s)
+                  : launch_quantize_q8_0(a->x, T, d.hidden, d.hidden, &xq, nullptr, s);
   if (rc) return rc;
-  if (dt == HIPQ_Q4_0)
+  if (mma) {
+    const int tc = mma_chunk(P, E);
+    rc = tc == 8    ? launch_grouped_mma<8>(a, b, views, xq, hq, s)
+         : tc == 16 ? launch_grouped_mma<16>(a, b, views, xq, hq, s)
+                    : launch_grouped_mma<32>(a, b, views, xq, hq, s);
+  } else if (dt == HIPQ_Q4_0)
     rc = launch_grouped<HIPQ_Q4_0>(a, b, views, xq, hq, s);
   else if (dt == HIPQ_Q4_K)
     rc = launch_grouped<HIPQ_Q4_K>(a, b, views, xq, hq, s);
   else
     rc = launch_grouped<HIPQ_Q6_K>(a, b, views, xq, hq, s);
   if (rc) return rc;
-  hipLaunchKernelGGL(combine_kernel, dim3((d.hidden + 255) / 256, T), dim3(256), 0, s, idx,
-                     b.pair_slot, d.topk, d.hidden, b.contrib, a->y);
+  hipLaunchKernelGGL(combine_kernel, dim3((d.hidden + 255) / 256, T), dim3(256), 0, s, b.tok_slots,
+                     d.topk, d.hidden, b.contrib, a->y);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
 }

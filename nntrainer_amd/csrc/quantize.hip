@@ -77,7 +77,7 @@ __global__ __launch_bounds__(256) void quantize_q8_0_kernel(
 }
 
 /* ---- Q8_K ---------------------------------------------------------------- */
-enum { Q8K_PLANES = 0, Q8K_CANONICAL = 1, Q8K_TILED = 2 };
+enum { Q8K_PLANES = 0, Q8K_CANONICAL = 1, Q8K_TILED = 2, Q8K_ROWMMA = 3 };
 
 /* One wavefront per (row, super-block). In the tiled mode the grid also covers
  * the padding rows M .. n_sb_total / nsb - 1, which are written as zeros. */
@@ -165,6 +165,19 @@ __global__ __launch_bounds__(256) void quantize_q8_K_kernel(
       amin_out[rb * 16 + (lane >> 3)] = __half_as_ushort(__float2half_rn((float)l6));
       amin_out[rb * 16 + 8 + (lane >> 3)] = __half_as_ushort(__float2half_rn((float)(bs - l6)));
     }
+  } else if (MODE == Q8K_ROWMMA) {
+    /* row-major, each 16-value group stored as its 8 even then its 8 odd values:
+     * this lane's four values are elements 4l .. 4l+3 of group lane / 4 */
+    int8_t *o = q_out + sb * 256 + (lane >> 2) * 16 + (lane & 3) * 2;
+    *(uint16_t *)o = (uint16_t)((q[0] & 0xff) | ((q[2] & 0xff) << 8));
+    *(uint16_t *)(o + 8) = (uint16_t)((q[1] & 0xff) | ((q[3] & 0xff) << 8));
+    if (lane == 0) d_out[sb] = d;
+    const int bs = gsum + __shfl_xor(gsum, 4, HIPQ_WAVE); /* two 16-value groups = one sub-block */
+    if ((lane & 7) == 0) {
+      const int l6 = bs & 63;
+      amin_out[sb * 16 + (lane >> 3)] = __half_as_ushort(__float2half_rn((float)l6));
+      amin_out[sb * 16 + 8 + (lane >> 3)] = __half_as_ushort(__float2half_rn((float)(bs - l6)));
+    }
   } else {
     *(int *)(q_out + sb * 256 + lane * 4) = packed;
     if (lane == 0) d_out[sb] = d;
@@ -223,6 +236,21 @@ int launch_quantize_q8_K(const float *A, int64_t M, int64_t K, int64_t lda,
     hipLaunchKernelGGL(quantize_q8_K_kernel<Q8K_PLANES>, dim3(grid), dim3(256), 0, s, A, M, total, nsb,
                        lda, mat_rows, qa->q, qa->d, qa->bsum, nullptr, nullptr, (uint16_t *)qa->ql,
                        (uint16_t *)qa->qh);
+  HIPQ_HIP(hipGetLastError());
+  return HIPQ_OK;
+}
+
+int launch_quantize_q8_K_rowmma(const float *A, int64_t M, int64_t K, int64_t lda, const QAct *qa,
+                                hipStream_t s) {
+  if (M <= 0) return HIPQ_OK;
+  if (K % 256 || lda < K) return fail(HIPQ_ERR_INVALID_ARGUMENT, "Q8_K: K=%lld must be a multiple of 256 and lda >= K", (long long)K);
+  if (((uintptr_t)A & 15) || (lda & 3))
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "activation rows must be 16-byte aligned");
+  const int nsb = (int)(K / 256);
+  const int64_t total = M * nsb;
+  const unsigned grid = (unsigned)((total + 3) / 4);
+  hipLaunchKernelGGL(quantize_q8_K_kernel<Q8K_ROWMMA>, dim3(grid), dim3(256), 0, s, A, M, total, nsb, lda,
+                     (int64_t)0, qa->q, qa->d, nullptr, nullptr, (uint16_t *)qa->bsum, nullptr, nullptr);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
 }
