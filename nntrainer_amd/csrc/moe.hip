@@ -429,12 +429,12 @@ __global__ __launch_bounds__(256) void down_long_kernel(const WView *__restrict_
  * per token group. Here a wavefront owns 32 weight rows and up to 32 tokens and
  * forms the 32 x 32 integer block sums of a super-block with
  * v_mfma_i32_32x32x32_i8: the tokens' Q8_K values are the row operand (from LDS,
- * staged once per workgroup), the weights the column operand, expanded in registers
- * from the packed nibbles into two digit planes (scale = 8 * high digit + low
- * digit, as the prefill GEMM does). Lane (n, g) holds the 64 bytes of sub-blocks
- * 4g .. 4g+3 of weight row n; a matrix step takes 16 consecutive weights per lane,
- * even ones (low nibbles) in operand bytes 0-7 and odd ones in bytes 8-15, and the
- * quantizer stores every 16-value group of the activations in that order. The mins
+ * staged once per workgroup), the weights the column operand, unpacked in registers
+ * from the nibbles. A matrix step is one sub-block: lane (n, g) supplies weights
+ * 16g .. 16g+15 of it for weight row n, even ones (low nibbles) in operand bytes
+ * 0-7 and odd ones in bytes 8-15, and the quantizer stores every 16-value group of
+ * the activations in that order; the step's sums take the sub-block's 6-bit scale
+ * in an integer multiply-add. The mins
  * go through one v_mfma_f32_32x32x16_f16 per super-block with the sub-block sums
  * split into two fp16-exact parts. Every integer is exact and the fp32 chain per
  * output is the single-row kernel's, so the results carry the same bits:
@@ -452,29 +452,28 @@ __device__ __forceinline__ uint32_t mma_pk_scale(uint32_t x, uint32_t digit2) {
 
 /* LDS of a workgroup: TC activation rows, padded so that the lanes of a 128-bit
  * read fall into different banks, then one ring of weight tiles per wavefront. */
-constexpr int XDEPTH = 3;       /* super-blocks of weights in the ring of a wavefront */
 constexpr int XTILE = 32 * 128 + 64 * 16; /* nibbles of 32 weight rows for one super-block, then their headers (twice) */
 struct XLds {
   int8_t *q;           /* [TC][K + 16] */
   uint8_t *amin;       /* [TC][nsb][32 bytes] */
   float *dA;           /* [nsb][TC] */
   int *rows;           /* [TC] source rows of the chunk */
-  unsigned char *ring; /* this wavefront's [XDEPTH][XTILE] */
+  unsigned char *ring; /* this wavefront's [XD][XTILE], XD = 2 or 3 super-blocks */
 };
 __host__ __device__ inline size_t xlds_act_bytes(int TC, int K) {
   const size_t b = (size_t)TC * (K + 16) + (size_t)TC * (K / 256) * 32 + (size_t)TC * (K / 256) * 4 + TC * 4;
   return (b + 255) & ~(size_t)255;
 }
-__host__ __device__ inline size_t xlds_bytes(int TC, int K) {
-  return xlds_act_bytes(TC, K) + 4 * XDEPTH * XTILE;
+__host__ __device__ inline size_t xlds_bytes(int TC, int K, int waves, int xd) {
+  return xlds_act_bytes(TC, K) + (size_t)waves * xd * XTILE;
 }
-__device__ __forceinline__ XLds xlds_carve(unsigned char *base, int TC, int K, int wave) {
+__device__ __forceinline__ XLds xlds_carve(unsigned char *base, int TC, int K, int wave, int xd) {
   XLds l;
   l.q = (int8_t *)base;
   l.amin = (uint8_t *)base + (size_t)TC * (K + 16);
   l.dA = (float *)(l.amin + (size_t)TC * (K / 256) * 32);
   l.rows = (int *)(l.dA + (size_t)TC * (K / 256));
-  l.ring = base + xlds_act_bytes(TC, K) + wave * (XDEPTH * XTILE);
+  l.ring = base + xlds_act_bytes(TC, K) + wave * (xd * XTILE);
   return l;
 }
 
@@ -557,80 +556,85 @@ constexpr int XS_OPS = 5; /* loads one xs_fetch issues */
 
 /* One super-block: acc / accm += for the NREG accumulator registers of this lane
  * (register r is token 8 * (r / 4) + 4g + r % 4, the lane's column n). `slot` holds
- * the nibbles and headers (its copies have landed). */
+ * the nibbles and headers (its copies have landed). One matrix step per sub-block
+ * j: lane (n, g) supplies weights 16g .. 16g+15 of it, so a step's 32 x 32 sums
+ * belong to one sub-block and take its 6-bit scale as an integer multiply-add. */
+typedef int mv2i __attribute__((ext_vector_type(2)));
 template <int TC, int NREG>
 __device__ __forceinline__ void xw_super_block(const unsigned char *slot, const XLds &l, int K, int sb,
                                                int i32, int g, float (&acc)[NREG], float (&accm)[NREG]) {
   const mv16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
   const mv16f zero16f = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
   const int nsb = K >> 8;
-  /* All LDS operands of the super-block in one go: this lane's 64 bytes of nibbles
-   * (pieces 4g .. 4g+3 of row i32), the eight 16-byte row operands of its token, the
-   * token's split sub-block sums and the block scales of its NREG tokens. The
-   * compiler must not see these reads: it orders every LDS read it knows of after
-   * the direct-to-LDS copies it may alias, which would drain the ring. */
+  /* The LDS operands: this lane's 8 bytes of every sub-block (piece j of row i32,
+   * half g), the eight 16-byte row operands of its token, the token's split
+   * sub-block sums and the block scales of its NREG tokens. The compiler must not
+   * see these reads: it orders every LDS read it knows of after the direct-to-LDS
+   * copies it may alias, which would drain the ring. */
   const int row = i32 & (TC - 1);
-  mv4i wq[4], a8[8], aminv, hdv, dv[NREG / 4];
+  mv2i wq[8];
+  mv4i a8[8], aminv, hdv, dv[NREG / 4];
+  auto lds = [](const void *p) { return (uint32_t)(size_t)(const __attribute__((address_space(3))) void *)p; };
+  const uint32_t rowb = lds(slot) + i32 * 128 + g * 8;
+  const uint32_t x7 = i32 & 7;
+  const uint32_t pa = lds(l.q) + row * (K + 16) + sb * 256 + g * 16;
+  /* in two halves (sub-blocks 0-3, 4-7) to bound the registers in use */
+  auto read_half = [&](int h2) {
+    const uint32_t w0 = rowb + (((4 * h2 + 0) ^ x7) << 4), w1 = rowb + (((4 * h2 + 1) ^ x7) << 4);
+    const uint32_t w2 = rowb + (((4 * h2 + 2) ^ x7) << 4), w3 = rowb + (((4 * h2 + 3) ^ x7) << 4);
+    const uint32_t pah = pa + h2 * 128;
+    asm volatile("ds_read_b64 %0, %8\n\tds_read_b64 %1, %9\n\tds_read_b64 %2, %10\n\tds_read_b64 %3, %11\n\t"
+                 "ds_read_b128 %4, %12\n\tds_read_b128 %5, %12 offset:32\n\tds_read_b128 %6, %12 offset:64\n\t"
+                 "ds_read_b128 %7, %12 offset:96"
+                 : "=&v"(wq[4 * h2]), "=&v"(wq[4 * h2 + 1]), "=&v"(wq[4 * h2 + 2]), "=&v"(wq[4 * h2 + 3]),
+                   "=&v"(a8[4 * h2]), "=&v"(a8[4 * h2 + 1]), "=&v"(a8[4 * h2 + 2]), "=&v"(a8[4 * h2 + 3])
+                 : "v"(w0), "v"(w1), "v"(w2), "v"(w3), "v"(pah)
+                 : "memory");
+  };
+  /* every register is named at the wait so that nothing reads one before it */
+  auto wait_half = [&](int h2) {
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(wq[4 * h2]), "+v"(wq[4 * h2 + 1]), "+v"(wq[4 * h2 + 2]), "+v"(wq[4 * h2 + 3]),
+                   "+v"(a8[4 * h2]), "+v"(a8[4 * h2 + 1]), "+v"(a8[4 * h2 + 2]), "+v"(a8[4 * h2 + 3])
+                 :
+                 : "memory");
+  };
   {
-    auto lds = [](const void *p) { return (uint32_t)(size_t)(const __attribute__((address_space(3))) void *)p; };
-    const uint32_t rowb = lds(slot) + i32 * 128;
-    const uint32_t x7 = i32 & 7;
-    const uint32_t a0 = rowb + (((4 * g + 0) ^ x7) << 4), a1 = rowb + (((4 * g + 1) ^ x7) << 4);
-    const uint32_t a2 = rowb + (((4 * g + 2) ^ x7) << 4), a3 = rowb + (((4 * g + 3) ^ x7) << 4);
-    const uint32_t pa = lds(l.q) + row * (K + 16) + sb * 256 + g * 128;
     const uint32_t pm = lds(l.amin) + (row * nsb + sb) * 32 + g * 16;
     const uint32_t pd = lds(l.dA) + (sb * TC + 4 * g) * 4;
-    asm volatile("ds_read_b128 %0, %4\n\tds_read_b128 %1, %5\n\tds_read_b128 %2, %6\n\tds_read_b128 %3, %7"
-                 : "=&v"(wq[0]), "=&v"(wq[1]), "=&v"(wq[2]), "=&v"(wq[3])
-                 : "v"(a0), "v"(a1), "v"(a2), "v"(a3)
-                 : "memory");
-    asm volatile("ds_read_b128 %0, %8\n\tds_read_b128 %1, %8 offset:16\n\tds_read_b128 %2, %8 offset:32\n\t"
-                 "ds_read_b128 %3, %8 offset:48\n\tds_read_b128 %4, %8 offset:64\n\tds_read_b128 %5, %8 offset:80\n\t"
-                 "ds_read_b128 %6, %8 offset:96\n\tds_read_b128 %7, %8 offset:112"
-                 : "=&v"(a8[0]), "=&v"(a8[1]), "=&v"(a8[2]), "=&v"(a8[3]), "=&v"(a8[4]), "=&v"(a8[5]),
-                   "=&v"(a8[6]), "=&v"(a8[7])
-                 : "v"(pa)
-                 : "memory");
-    asm volatile("ds_read_b128 %0, %1" : "=&v"(aminv) : "v"(pm) : "memory");
     asm volatile("ds_read_b128 %0, %1 offset:4096" : "=&v"(hdv) : "v"(lds(slot) + (i32 + 32 * g) * 16) : "memory");
+    read_half(0);
+    asm volatile("ds_read_b128 %0, %1" : "=&v"(aminv) : "v"(pm) : "memory");
 #pragma unroll
     for (int q4 = 0; q4 < NREG / 4; ++q4)
       asm volatile("ds_read_b128 %0, %1" : "=&v"(dv[q4]) : "v"(pd + q4 * 32) : "memory");
-    /* every register above is named so that nothing reads one before the wait */
-    asm volatile("s_waitcnt lgkmcnt(0)"
-                 : "+v"(wq[0]), "+v"(wq[1]), "+v"(wq[2]), "+v"(wq[3]), "+v"(a8[0]), "+v"(a8[1]), "+v"(a8[2]),
-                   "+v"(a8[3]), "+v"(a8[4]), "+v"(a8[5]), "+v"(a8[6]), "+v"(a8[7]), "+v"(aminv), "+v"(hdv)
-                 :
-                 : "memory");
+    read_half(1);
+    wait_half(0);
+    wait_half(1);
+    asm volatile("" : "+v"(aminv), "+v"(hdv));
 #pragma unroll
     for (int q4 = 0; q4 < NREG / 4; ++q4) asm volatile("" : "+v"(dv[q4]));
   }
   const uint4 hd = make_uint4((uint32_t)hdv[0], (uint32_t)hdv[1], (uint32_t)hdv[2], (uint32_t)hdv[3]);
-  /* 6-bit scales of sub-blocks 4g .. 4g+3, one per byte, as two 3-bit digits */
+  /* 6-bit scales of sub-blocks 0-3 and 4-7, one per byte */
   const uint32_t s03 = hd.y & 0x3f3f3f3fu;
   const uint32_t s47 = (hd.w & 0x0f0f0f0fu) | ((hd.y >> 2) & 0x30303030u);
-  const uint32_t sc = g ? s47 : s03;
-  const uint32_t slo = sc & 0x07070707u, shi = (sc >> 3) & 0x07070707u;
   const mv8h amin = __builtin_bit_cast(mv8h, aminv);
-  mv16i Dlo = zero16, Dhi = zero16;
+  int I[NREG];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    /* digit of sub-block 4g + j in both 16-bit halves */
-    const uint32_t dl = __builtin_amdgcn_perm(slo, slo, 0x0c000c00u | (uint32_t)j | ((uint32_t)j << 16));
-    const uint32_t dh = __builtin_amdgcn_perm(shi, shi, 0x0c000c00u | (uint32_t)j | ((uint32_t)j << 16));
+  for (int r = 0; r < NREG; ++r) I[r] = 0;
 #pragma unroll
-    for (int half = 0; half < 2; ++half) {
-      const uint32_t x0 = (uint32_t)wq[j][2 * half], x1 = (uint32_t)wq[j][2 * half + 1];
-      const uint32_t e0 = x0 & HIPQ_M4, e1 = x1 & HIPQ_M4;
-      const uint32_t o0 = (x0 >> 4) & HIPQ_M4, o1 = (x1 >> 4) & HIPQ_M4;
-      const mv4i bl = {(int)mma_pk_scale(e0, dl), (int)mma_pk_scale(e1, dl), (int)mma_pk_scale(o0, dl),
-                       (int)mma_pk_scale(o1, dl)};
-      const mv4i bh = {(int)mma_pk_scale(e0, dh), (int)mma_pk_scale(e1, dh), (int)mma_pk_scale(o0, dh),
-                       (int)mma_pk_scale(o1, dh)};
-      const mv4i a = a8[j * 2 + half];
-      Dlo = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, bl, Dlo, 0, 0, 0);
-      Dhi = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, bh, Dhi, 0, 0, 0);
-    }
+  for (int j = 0; j < 8; ++j) {
+    /* weight 2i / 2i+1 of the lane's 16 in the low / high nibble of byte i: the even
+     * ones become operand bytes 0-7, the odd ones bytes 8-15 (the activations'
+     * 16-value groups are stored in that order) */
+    const uint32_t x0 = (uint32_t)wq[j][0], x1 = (uint32_t)wq[j][1];
+    const mv4i b = {(int)(x0 & HIPQ_M4), (int)(x1 & HIPQ_M4), (int)((x0 >> 4) & HIPQ_M4),
+                    (int)((x1 >> 4) & HIPQ_M4)};
+    const mv16i D = __builtin_amdgcn_mfma_i32_32x32x32_i8(a8[j], b, zero16, 0, 0, 0);
+    const int scj = (int)(((j < 4 ? s03 : s47) >> (8 * (j & 3))) & 0xff);
+#pragma unroll
+    for (int r = 0; r < NREG; ++r) I[r] = __mul24(D[r], scj) + I[r];
   }
   /* mins: sum_j m_j * bsum_j, the low parts of bsum in lanes 0-31, the high parts in 32-63 */
   const uint32_t mlo = hd.z & 0x3f3f3f3fu;
@@ -650,21 +654,20 @@ __device__ __forceinline__ void xw_super_block(const unsigned char *slot, const 
     for (int e = 0; e < 4; ++e) {
       const int r = 4 * q4 + e;
       const float dA = __int_as_float(dv[q4][e]);
-      const int I = (Dhi[r] << 3) + Dlo[r];
-      acc[r] = fmaf((float)I, dw * dA, acc[r]);
+      acc[r] = fmaf((float)I[r], dw * dA, acc[r]);
       accm[r] = fmaf(Sm[r], dmin * dA, accm[r]);
     }
   }
 }
 
 /* A run of column tiles (matrix, first column) for one wavefront: the weights of
- * the next XDEPTH - 1 super-blocks, also across tiles, are in flight while one is
+ * the next XD - 1 super-blocks, also across tiles, are in flight while one is
  * computed. tile_of(t, &view, &col0) names tile t; done(t, out) receives its NREG
  * results. Loads retire in issue order, so waiting until at most the loads of the
  * younger fetches are outstanding means the oldest fetch has landed. */
-template <int TC, int NREG, typename TileOf, typename Done>
+template <int TC, int NREG, int XD, typename TileOf, typename Done>
 __device__ __forceinline__ void xw_run(int ntile, const XLds &l, int K, TileOf tile_of, Done done) {
-  static_assert(XDEPTH == 3, "the loop below is unrolled for a ring of three");
+  static_assert(XD == 2 || XD == 3, "the loop below is unrolled for a ring of two or three");
   const int lane = threadIdx.x & 63, i32 = lane & 31, g = lane >> 5;
   const int nsb = K >> 8;
   const int nv = ntile * nsb;
@@ -696,7 +699,7 @@ __device__ __forceinline__ void xw_run(int ntile, const XLds &l, int K, TileOf t
   };
   unsigned char *const s0 = l.ring, *const s1 = l.ring + XTILE, *const s2 = l.ring + 2 * XTILE;
   fetch(s0);
-  fetch(s1);
+  if (XD == 3) fetch(s1);
   int t = 0, sb = 0, v = 0;
   float acc[NREG], accm[NREG];
   auto step = [&](const unsigned char *cur, unsigned char *nxt) {
@@ -705,8 +708,8 @@ __device__ __forceinline__ void xw_run(int ntile, const XLds &l, int K, TileOf t
       for (int r = 0; r < NREG; ++r) acc[r] = accm[r] = 0.f;
     }
     fetch(nxt); /* into the slot consumed by the previous step */
-    /* the fetch of this step has landed once only the two later ones are outstanding */
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * XS_OPS) : "memory");
+    /* the fetch of this step has landed once only the XD - 1 later ones are outstanding */
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((XD - 1) * XS_OPS) : "memory");
     xw_super_block<TC, NREG>(cur, l, K, sb, i32, g, acc, accm);
     ++v;
     if (++sb == nsb) {
@@ -719,9 +722,14 @@ __device__ __forceinline__ void xw_run(int ntile, const XLds &l, int K, TileOf t
     }
   };
   while (v < nv) {
-    step(s0, s2);
-    if (v < nv) step(s1, s0);
-    if (v < nv) step(s2, s1);
+    if (XD == 3) {
+      step(s0, s2);
+      if (v < nv) step(s1, s0);
+      if (v < nv) step(s2, s1);
+    } else {
+      step(s0, s1);
+      if (v < nv) step(s1, s0);
+    }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); /* no copy may land after the ring is given up */
 }
@@ -729,8 +737,8 @@ __device__ __forceinline__ void xw_run(int ntile, const XLds &l, int K, TileOf t
 /* h[slot][col] = silu(x_tok . Wgate[e][col]) * (x_tok . Wup[e][col]): a workgroup
  * serves one expert and 128 columns (32 per wavefront, the gate tile then the up
  * tile), the expert's tokens in chunks of TC. */
-template <int TC>
-__global__ __launch_bounds__(256) void gate_up_mma_kernel(const WView *__restrict__ views, int E_,
+template <int TC, int WV, int XD>
+__global__ __launch_bounds__(64 * WV, TC <= 8 && XD == 2 ? 3 : 1) void gate_up_mma_kernel(const WView *__restrict__ views, int E_,
                                                           QView xq, const int *__restrict__ offsets,
                                                           const int *__restrict__ slot_pair, int topk,
                                                           int I, float *__restrict__ h) {
@@ -742,8 +750,8 @@ __global__ __launch_bounds__(256) void gate_up_mma_kernel(const WView *__restric
   const WView wg = views[e], wu = views[E_ + e];
   const int K = wg.K;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const XLds l = xlds_carve(xmoe_lds, TC, K, wave);
-  const int col0 = (blockIdx.x * 4 + wave) * 32;
+  const XLds l = xlds_carve(xmoe_lds, TC, K, wave, XD);
+  const int col0 = (blockIdx.x * WV + wave) * 32;
   for (int s0 = begin; s0 < end; s0 += TC) {
     __syncthreads(); /* the previous chunk is no longer read */
     if (threadIdx.x < TC) l.rows[threadIdx.x] = slot_pair[min(s0 + (int)threadIdx.x, end - 1)] / topk;
@@ -752,7 +760,7 @@ __global__ __launch_bounds__(256) void gate_up_mma_kernel(const WView *__restric
     __syncthreads();
     if (col0 >= I) continue; /* uniform per wavefront; it still takes part in the barriers */
     float gate[NREG];
-    xw_run<TC, NREG>(
+    xw_run<TC, NREG, XD>(
       2, l, K,
       [&](int t, WView &w, int &c0) {
         w = t ? wu : wg;
@@ -775,8 +783,8 @@ __global__ __launch_bounds__(256) void gate_up_mma_kernel(const WView *__restric
 }
 
 /* contrib[slot][col] = (h_slot . Wdown[e][col]) * weight(pair): CT column tiles per wavefront */
-template <int TC, int CT>
-__global__ __launch_bounds__(256) void down_mma_kernel(const WView *__restrict__ views, int E_, QView hq,
+template <int TC, int CT, int XD>
+__global__ __launch_bounds__(256, TC <= 8 && XD == 2 ? 3 : 1) void down_mma_kernel(const WView *__restrict__ views, int E_, QView hq,
                                                        const int *__restrict__ offsets,
                                                        const int *__restrict__ slot_pair,
                                                        const float *__restrict__ wgt, int H,
@@ -789,7 +797,7 @@ __global__ __launch_bounds__(256) void down_mma_kernel(const WView *__restrict__
   const WView wd = views[2 * E_ + e];
   const int K = wd.K;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const XLds l = xlds_carve(xmoe_lds, TC, K, wave);
+  const XLds l = xlds_carve(xmoe_lds, TC, K, wave, XD);
   const int col0 = (blockIdx.x * 4 + wave) * 32 * CT;
   const int ntile = min(CT, (H - col0 + 31) / 32);
   for (int s0 = begin; s0 < end; s0 += TC) {
@@ -799,7 +807,7 @@ __global__ __launch_bounds__(256) void down_mma_kernel(const WView *__restrict__
     stage_rows<TC>(l, hq);
     __syncthreads();
     if (ntile <= 0) continue;
-    xw_run<TC, NREG>(
+    xw_run<TC, NREG, XD>(
       ntile, l, K,
       [&](int t, WView &w, int &c0) {
         w = wd;
@@ -908,39 +916,64 @@ template <int DT> struct DownLauncher {
   template <int T, int KC, int G> void operator()() const { launch_down<DT, T, KC, G>(d, views, hq, b, s); }
 };
 
-/* Token chunk of the MFMA expert kernels for P pairs over E experts: the smallest
- * of 8, 16, 32 that holds twice the mean tokens per expert (larger groups loop). */
-int mma_chunk(int64_t P, int E) {
-  const int64_t mean2 = (2 * P + E - 1) / E;
-  return mean2 <= 8 ? 8 : mean2 <= 16 ? 16 : 32;
+template <int TC, int WV, int XD>
+int launch_gate_up_mma(const hipq_moe_desc &d, const MoeBufs &b, const WView *views, const QAct &xq,
+                       hipStream_t s) {
+  const size_t lds = xlds_bytes(TC, d.hidden, WV, XD);
+  if (lds > 64 * 1024) /* beyond the default limit of a launch */
+    HIPQ_HIP(hipFuncSetAttribute((const void *)gate_up_mma_kernel<TC, WV, XD>,
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  hipLaunchKernelGGL((gate_up_mma_kernel<TC, WV, XD>), dim3((d.intermediate + 32 * WV - 1) / (32 * WV), d.experts),
+                     dim3(64 * WV), lds, s, views, d.experts, qview(xq), b.offsets, b.slot_pair, d.topk,
+                     d.intermediate, b.h);
+  HIPQ_HIP(hipGetLastError());
+  return HIPQ_OK;
 }
-bool use_mma(const hipq_moe_desc &d, int dt) {
-  return dt == HIPQ_Q4_K && d.hidden <= 4096 && d.intermediate <= 4096;
+template <int TC, int CT, int XD>
+int launch_down_mma(const hipq_moe_desc &d, const MoeBufs &b, const WView *views, const QAct &hq,
+                    hipStream_t s) {
+  const size_t lds = xlds_bytes(TC, d.intermediate, 4, XD);
+  if (lds > 64 * 1024)
+    HIPQ_HIP(hipFuncSetAttribute((const void *)down_mma_kernel<TC, CT, XD>,
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+  hipLaunchKernelGGL((down_mma_kernel<TC, CT, XD>), dim3((d.hidden + 128 * CT - 1) / (128 * CT), d.experts),
+                     dim3(256), lds, s, views, d.experts, qview(hq), b.offsets, b.slot_pair, b.wgt, d.hidden,
+                     b.contrib);
+  HIPQ_HIP(hipGetLastError());
+  return HIPQ_OK;
 }
+
+constexpr size_t XLDS_MAX = 160 * 1024; /* LDS of a CU */
 
 template <int TC>
 int launch_grouped_mma(const hipq::MoeArgs *a, const MoeBufs &b, const WView *views, const QAct &xq,
                        const QAct &hq, hipStream_t s) {
   const hipq_moe_desc &d = a->desc;
   const int64_t P = (int64_t)d.tokens * d.topk;
-  constexpr int CT = 2;
-  const size_t lds_gu = xlds_bytes(TC, d.hidden), lds_dn = xlds_bytes(TC, d.intermediate);
-  if (lds_gu > 64 * 1024) /* beyond the default limit of a launch */
-    HIPQ_HIP(hipFuncSetAttribute((const void *)gate_up_mma_kernel<TC>,
-                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_gu));
-  if (lds_dn > 64 * 1024)
-    HIPQ_HIP(hipFuncSetAttribute((const void *)down_mma_kernel<TC, CT>,
-                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_dn));
-  hipLaunchKernelGGL((gate_up_mma_kernel<TC>), dim3((d.intermediate + 127) / 128, d.experts), dim3(256), lds_gu,
-                     s, views, d.experts, qview(xq), b.offsets, b.slot_pair, d.topk, d.intermediate, b.h);
-  HIPQ_HIP(hipGetLastError());
-  int rc = hipq::launch_quantize_q8_K_rowmma(b.h, P, d.intermediate, d.intermediate, &hq, s);
+  /* gate/up: four wavefronts with a ring of three super-blocks each where that fits;
+   * down: one column tile per wavefront and a ring of two (rows are short, more
+   * workgroups per CU pay more than a deeper ring) */
+  int rc = xlds_bytes(TC, d.hidden, 4, 3) <= XLDS_MAX ? launch_gate_up_mma<TC, 4, 3>(d, b, views, xq, s)
+                                                       : launch_gate_up_mma<TC, 4, 2>(d, b, views, xq, s);
   if (rc) return rc;
-  hipLaunchKernelGGL((down_mma_kernel<TC, CT>), dim3((d.hidden + 128 * CT - 1) / (128 * CT), d.experts),
-                     dim3(256), lds_dn, s, views, d.experts, qview(hq), b.offsets, b.slot_pair, b.wgt,
-                     d.hidden, b.contrib);
-  HIPQ_HIP(hipGetLastError());
-  return HIPQ_OK;
+  rc = hipq::launch_quantize_q8_K_rowmma(b.h, P, d.intermediate, d.intermediate, &hq, s);
+  if (rc) return rc;
+  return launch_down_mma<TC, 1, 2>(d, b, views, hq, s);
+}
+
+/* Token chunk of the MFMA expert kernels for P pairs over E experts: the smallest
+ * of 8, 16, 32 that holds twice the mean tokens per expert (larger groups loop),
+ * reduced until the activation rows and the weight rings fit the LDS. */
+int mma_chunk(const hipq_moe_desc &d, int64_t P, int E) {
+  const int64_t mean2 = (2 * P + E - 1) / E;
+  int tc = mean2 <= 8 ? 8 : mean2 <= 16 ? 16 : 32;
+  const int kmax = d.hidden > d.intermediate ? d.hidden : d.intermediate;
+  while (tc > 8 && xlds_bytes(tc, kmax, 4, 2) > XLDS_MAX) tc >>= 1;
+  return tc;
+}
+bool use_mma(const hipq_moe_desc &d, int dt) {
+  const int kmax = d.hidden > d.intermediate ? d.hidden : d.intermediate;
+  return dt == HIPQ_Q4_K && xlds_bytes(8, kmax, 4, 2) <= XLDS_MAX;
 }
 
 template <int DT>
@@ -1017,7 +1050,7 @@ int launch_moe(const MoeArgs *a, void *workspace, size_t workspace_bytes, const 
                   : launch_quantize_q8_0(a->x, T, d.hidden, d.hidden, &xq, nullptr, s);
   if (rc) return rc;
   if (mma) {
-    const int tc = mma_chunk(P, E);
+    const int tc = mma_chunk(d, P, E);
     rc = tc == 8    ? launch_grouped_mma<8>(a, b, views, xq, hq, s)
          : tc == 16 ? launch_grouped_mma<16>(a, b, views, xq, hq, s)
                     : launch_grouped_mma<32>(a, b, views, xq, hq, s);

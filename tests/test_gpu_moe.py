@@ -17,7 +17,13 @@ def _experts(cr, e, i, h, seed):
     return gate, up, down
 
 
-@pytest.mark.parametrize("t,h,i,e,k", [(8, 256, 256, 8, 2), (64, 512, 256, 16, 4), (5, 2048, 768, 8, 8)])
+# the later shapes reach the kernels' other paths: 16- and 32-token chunks with
+# experts that hold more tokens than a chunk (48 tokens x 4 of 4 experts), rows long
+# enough that the weight ring drops to two super-blocks (hidden 3072 at 32 tokens),
+# and rows beyond what the matrix-core kernels stage in LDS (hidden 8192)
+@pytest.mark.parametrize("t,h,i,e,k", [(8, 256, 256, 8, 2), (64, 512, 256, 16, 4), (5, 2048, 768, 8, 8),
+                                       (40, 512, 256, 8, 2), (48, 256, 512, 4, 4), (72, 3072, 256, 4, 2),
+                                       (3, 8192, 256, 4, 2)])
 def test_moe_matches_oracle(hipq, cr, t, h, i, e, k):
     import gpu_util as gu
     import torch
