@@ -20,12 +20,14 @@
  * reference's M = 1 matmuls do.
  *
  * Launch plan (all on one stream, no host synchronisation; grids do not depend
- * on device data): router logits (optional) -> route -> count -> scan ->
- * scatter (pairs sorted by expert) -> quantize x -> grouped gate+up GEMV with
- * fused SwiGLU over (column tiles x experts) -> quantize h -> grouped down GEMV
- * scaled by the routing weight -> combine. Within an expert the weight rows are
- * streamed once per group of four tokens. Each single-row product is computed by
- * the same engine as the decode GEMV, so it carries the reference's bits.
+ * on device data): router logits (optional) -> route -> sort of the pairs by
+ * expert (one workgroup; count / scan / scatter kernels for very long chunks) ->
+ * quantize x -> grouped gate+up product with fused SwiGLU over (column tiles x
+ * experts) -> quantize h -> grouped down product scaled by the routing weight ->
+ * combine. Q4_K experts whose rows fit the LDS run on the matrix cores, 8 to 32
+ * tokens of an expert per pass over its weights; the other formats and longer rows
+ * use the decode GEMV's engine, four tokens per pass. Both carry the reference's
+ * bits for every single-row product.
  */
 #include "gemv_device.h"
 
@@ -667,7 +669,6 @@ __device__ __forceinline__ void xw_super_block(const unsigned char *slot, const 
  * younger fetches are outstanding means the oldest fetch has landed. */
 template <int TC, int NREG, int XD, typename TileOf, typename Done>
 __device__ __forceinline__ void xw_run(int ntile, const XLds &l, int K, TileOf tile_of, Done done) {
-  static_assert(XD == 2 || XD == 3, "the loop below is unrolled for a ring of two or three");
   const int lane = threadIdx.x & 63, i32 = lane & 31, g = lane >> 5;
   const int nsb = K >> 8;
   const int nv = ntile * nsb;
@@ -697,21 +698,27 @@ __device__ __forceinline__ void xw_run(int ntile, const XLds &l, int K, TileOf t
       xs_advance(xs);
     }
   };
-  unsigned char *const s0 = l.ring, *const s1 = l.ring + XTILE, *const s2 = l.ring + 2 * XTILE;
-  fetch(s0);
-  if (XD == 3) fetch(s1);
-  int t = 0, sb = 0, v = 0;
+  /* ring slots by fetch number modulo XD; the loop keeps XD - 1 fetches ahead */
+  int fslot = 0; /* slot of the next fetch */
+  auto fetch_next = [&]() {
+    fetch(l.ring + fslot * XTILE);
+    fslot = fslot + 1 == XD ? 0 : fslot + 1;
+  };
+#pragma unroll
+  for (int i = 0; i < XD - 1; ++i) fetch_next();
+  int cslot = 0; /* slot of the super-block computed next */
+  int t = 0, sb = 0;
   float acc[NREG], accm[NREG];
-  auto step = [&](const unsigned char *cur, unsigned char *nxt) {
+  for (int v = 0; v < nv; ++v) {
     if (sb == 0) {
 #pragma unroll
       for (int r = 0; r < NREG; ++r) acc[r] = accm[r] = 0.f;
     }
-    fetch(nxt); /* into the slot consumed by the previous step */
+    fetch_next(); /* into the slot consumed by the previous step */
     /* the fetch of this step has landed once only the XD - 1 later ones are outstanding */
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"((XD - 1) * XS_OPS) : "memory");
-    xw_super_block<TC, NREG>(cur, l, K, sb, i32, g, acc, accm);
-    ++v;
+    xw_super_block<TC, NREG>(l.ring + cslot * XTILE, l, K, sb, i32, g, acc, accm);
+    cslot = cslot + 1 == XD ? 0 : cslot + 1;
     if (++sb == nsb) {
       float out[NREG];
 #pragma unroll
@@ -719,16 +726,6 @@ __device__ __forceinline__ void xw_run(int ntile, const XLds &l, int K, TileOf t
       done(t, out);
       sb = 0;
       ++t;
-    }
-  };
-  while (v < nv) {
-    if (XD == 3) {
-      step(s0, s2);
-      if (v < nv) step(s1, s0);
-      if (v < nv) step(s2, s1);
-    } else {
-      step(s0, s1);
-      if (v < nv) step(s1, s0);
     }
   }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); /* no copy may land after the ring is given up */
