@@ -970,7 +970,9 @@ int mma_chunk(const hipq_moe_desc &d, int64_t P, int E) {
 }
 bool use_mma(const hipq_moe_desc &d, int dt) {
   const int kmax = d.hidden > d.intermediate ? d.hidden : d.intermediate;
-  return dt == HIPQ_Q4_K && xlds_bytes(8, kmax, 4, 2) <= XLDS_MAX;
+  /* the copies address an expert's plane with 32-bit offsets */
+  const bool small = (uint64_t)d.hidden * (uint64_t)d.intermediate / 2 < (1ull << 32);
+  return dt == HIPQ_Q4_K && small && xlds_bytes(8, kmax, 4, 2) <= XLDS_MAX;
 }
 
 template <int DT>
