@@ -102,12 +102,12 @@ template <bool PW> struct GemvRec<HIPQ_Q4_0, PW> {
   static constexpr int LANES_PER_OUT = 1;
 };
 template <> struct GemvRec<HIPQ_Q4_K, false> {
-  static constexpr int UNIT = 64;
+  static constexpr int UNIT = 32;
   static constexpr int PER_CHUNK = (HIPQ_KCHUNK / 256) * 4 + 4; /* {fI, sd, fIm, sm} per super-block */
   static constexpr int LANES_PER_OUT = 1;
 };
 template <> struct GemvRec<HIPQ_Q4_K, true> {
-  static constexpr int UNIT = 64;
+  static constexpr int UNIT = 32;
   static constexpr int PER_CHUNK = (HIPQ_KCHUNK / 256) * 10 + 2; /* {I[4], Im[4], sd, sm} per super-block */
   static constexpr int LANES_PER_OUT = 1;
 };
@@ -118,7 +118,7 @@ template <bool PW> struct GemvRec<HIPQ_Q6_K, PW> {
 };
 
 /* Units a lane handles per chunk of KC weights: 64 lanes cover a 4096-weight chunk
- * in 2 (Q4_0) or 1 (Q4_K, Q6_K) steps. Kernels for short rows (MoE experts) pick
+ * in 2 (Q4_0, Q4_K) or 1 (Q6_K) steps. Kernels for short rows (MoE experts) pick
  * fewer lanes per row and a smaller chunk so that no lane and no register idles. */
 template <int DT, int T, int KC> struct GemvUnits {
   static constexpr int MAXU = (KC / GemvRec<DT, false>::UNIT + T - 1) / T;
@@ -195,106 +195,97 @@ template <int T, int R, bool PW, int KC> struct GemvQ40 {
 };
 
 /* ---- Q4_K ----------------------------------------------------------------------- */
-/* A unit is one sub-block pair: 16 bytes of sub-block 2c then 16 bytes of
- * sub-block 2c+1 of a super-block (eight weights per dword); 4 consecutive lanes
- * hold one super-block, so its integer sums meet in two quad-permute DPP steps. */
+/* A unit is one sub-block: its 16 bytes (eight weights per dword). Consecutive lanes
+ * take consecutive sub-blocks, so one load instruction of a wavefront covers 1 KB of
+ * consecutive bytes (lanes 32 bytes apart, each taking a sub-block pair with two
+ * loads, stream measurably slower). 8 consecutive lanes hold one super-block; its
+ * integer sums meet in three DPP steps. */
 template <int T, int R, bool PW, int KC> struct GemvQ4K {
+  static_assert(T % 8 == 0, "a super-block's eight sub-blocks sit in eight consecutive lanes");
   static constexpr int MAXU = GemvUnits<HIPQ_Q4_K, T, KC>::MAXU;
   static constexpr int PER = GemvRec<HIPQ_Q4_K, PW>::PER_CHUNK;
   struct Act {
-    /* digits of the activations of sub-blocks 2c (l0, h0) and 2c+1 (l1, h1) */
-    uint4 l0[MAXU][R], l1[MAXU][R], h0[MAXU][R], h1[MAXU][R];
-    int bs0[MAXU][R], bs1[MAXU][R]; /* sums of the activations of sub-blocks 2c, 2c+1 */
+    uint4 l[MAXU][R], h[MAXU][R]; /* digits of the sub-block's activations */
+    int bs[MAXU][R];              /* their sum */
     float dA[MAXU][R];
   };
   struct Wt {
-    uint4 q0[MAXU], q1[MAXU];
+    uint4 q[MAXU];
     uint4 hd[MAXU];
   };
   __device__ static __forceinline__ void load_act(Act &A, const QView &qa, const int (&arow)[R],
                                                   int tl, int k0, int kc) {
-    const int nsb = qa.K >> 8, un = kc >> 6, b0 = k0 >> 8;
+    const int nsb = qa.K >> 8, un = kc >> 5, b0 = k0 >> 8;
 #pragma unroll
     for (int i = 0; i < MAXU; ++i) {
       if (i * T >= un) break;
       const int u = min(tl + i * T, un - 1);
-      const int b = u >> 2, c = u & 3;
+      const int b = u >> 3, j = u & 7;
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        const size_t off = (size_t)arow[r] * (qa.K >> 1) + (size_t)(b0 + b) * 128 + c * 32;
-        const uint4 *al = (const uint4 *)(qa.ql + off), *ah = (const uint4 *)(qa.qh + off);
-        A.l0[i][r] = al[0];
-        A.l1[i][r] = al[1];
-        A.h0[i][r] = ah[0];
-        A.h1[i][r] = ah[1];
-        const int2 bsw = *(const int2 *)(qa.bsum + (size_t)arow[r] * (qa.K >> 4) +
-                                         (b0 + b) * 16 + 4 * c);
-        A.bs0[i][r] = (int)(int16_t)(bsw.x & 0xffff) + (bsw.x >> 16);
-        A.bs1[i][r] = (int)(int16_t)(bsw.y & 0xffff) + (bsw.y >> 16);
+        const size_t off = (size_t)arow[r] * (qa.K >> 1) + (size_t)(b0 + b) * 128 + j * 16;
+        A.l[i][r] = *(const uint4 *)(qa.ql + off);
+        A.h[i][r] = *(const uint4 *)(qa.qh + off);
+        const int bsw = *(const int *)(qa.bsum + (size_t)arow[r] * (qa.K >> 4) + (b0 + b) * 16 + 2 * j);
+        A.bs[i][r] = (int)(int16_t)(bsw & 0xffff) + (bsw >> 16);
         A.dA[i][r] = qa.d[(size_t)arow[r] * nsb + b0 + b];
       }
     }
   }
   __device__ static __forceinline__ void load_w(Wt &W, const WView &w, int row, int tl, int k0,
                                                 int kc) {
-    const int nsb = w.K >> 8, un = kc >> 6, b0 = k0 >> 8;
+    const int nsb = w.K >> 8, un = kc >> 5, b0 = k0 >> 8;
     const uint4 *qs = (const uint4 *)(w.qs + (size_t)row * (w.K >> 1) + (size_t)b0 * 128);
     const uint4 *hdr = (const uint4 *)w.hdr + (size_t)row * nsb + b0;
 #pragma unroll
     for (int i = 0; i < MAXU; ++i) {
       if (i * T >= un) break;
       const int u = min(tl + i * T, un - 1);
-      W.q0[i] = hipq_ld_stream(qs + 2 * u);
-      W.q1[i] = hipq_ld_stream(qs + 2 * u + 1);
-      W.hd[i] = hipq_ld_global(hdr + (u >> 2));
+      W.q[i] = hipq_ld_stream(qs + u);
+      W.hd[i] = hipq_ld_global(hdr + (u >> 3));
     }
   }
   __device__ static __forceinline__ void compute(const Wt &W, const Act &A, int tl, int kc,
                                                  uint32_t *rec) {
-    const int un = kc >> 6;
+    const int un = kc >> 5;
 #pragma unroll
     for (int i = 0; i < MAXU; ++i) {
       if (i * T >= un) break;
       const int u = tl + i * T;
       const bool on = u < un;
       const int uc = on ? u : un - 1;
-      const int b = uc >> 2, c = uc & 3;
-      const uint4 q0 = W.q0[i], q1 = W.q1[i];
+      const int b = uc >> 3, j = uc & 7;
       const uint4 hd = W.hd[i];
-      /* 6-bit scales / mins of sub-blocks 2c, 2c+1: two adjacent bytes */
-      const int sh = 16 * (c & 1);
+      /* 6-bit scale / min of sub-block j: byte j of y / z for j < 4, else the low /
+       * high nibble of byte j-4 of w with bits 6-7 of byte j-4 of y / z on top */
+      const int sh = 8 * (j & 3);
       const uint32_t y = hd.y >> sh, z = hd.z >> sh, ww = hd.w >> sh;
-      const uint32_t sc_hi = (ww & 0x0f0fu) | (((y >> 6) & 0x0303u) << 4);
-      const uint32_t mn_hi = ((ww >> 4) & 0x0f0fu) | (((z >> 6) & 0x0303u) << 4);
-      const uint32_t scw = c < 2 ? (y & 0x3f3fu) : sc_hi;
-      const uint32_t mnw = c < 2 ? (z & 0x3f3fu) : mn_hi;
-      const int sc0 = (int)(scw & 0xff), sc1 = (int)(scw >> 8);
-      const int mn0 = (int)(mnw & 0xff), mn1 = (int)(mnw >> 8);
+      const int sc = (int)(j < 4 ? (y & 0x3fu) : ((ww & 0x0fu) | ((y >> 2) & 0x30u)));
+      const int mn = (int)(j < 4 ? (z & 0x3fu) : (((ww >> 4) & 0x0fu) | ((z >> 2) & 0x30u)));
       const float dw = hipq_h2f((uint16_t)(hd.x & 0xffff));
       const float dmin = hipq_h2f((uint16_t)(hd.x >> 16));
 #pragma unroll
       for (int r = 0; r < R; ++r) {
-        /* q0 / q1: the 32 weights of sub-block 2c / 2c+1 */
-        const int dlo = hipq_dot32_u4(q0, A.l0[i][r], A.h0[i][r]);
-        const int dhi = hipq_dot32_u4(q1, A.l1[i][r], A.h1[i][r]);
-        int I = __mul24(sc0, dlo) + __mul24(sc1, dhi);
-        int Im = __mul24(mn0, A.bs0[i][r]) + __mul24(mn1, A.bs1[i][r]);
+        int I = __mul24(sc, hipq_dot32_u4(W.q[i], A.l[i][r], A.h[i][r]));
+        int Im = __mul24(mn, A.bs[i][r]);
+        I += hipq_dpp_i<HIPQ_DPP_XOR1>(I); /* the sub-block pair */
+        Im += hipq_dpp_i<HIPQ_DPP_XOR1>(Im);
         if (PW) {
-          if (on) {
+          if (on && (j & 1) == 0) {
             uint32_t *o = rec + r * PER + b * 10;
-            o[c] = (uint32_t)I;
-            o[4 + c] = (uint32_t)Im;
-            if (c == 0) {
+            o[j >> 1] = (uint32_t)I;
+            o[4 + (j >> 1)] = (uint32_t)Im;
+            if (j == 0) {
               o[8] = __float_as_uint(dw * A.dA[i][r]);
               o[9] = __float_as_uint(dmin * A.dA[i][r]);
             }
           }
         } else {
-          I += hipq_dpp_i<HIPQ_DPP_XOR1>(I); /* the four pairs of the super-block */
-          Im += hipq_dpp_i<HIPQ_DPP_XOR1>(Im);
-          I += hipq_dpp_i<HIPQ_DPP_XOR2>(I);
+          I += hipq_dpp_i<HIPQ_DPP_XOR2>(I); /* the four pairs of the super-block */
           Im += hipq_dpp_i<HIPQ_DPP_XOR2>(Im);
-          if (on && c == 0) {
+          I += hipq_dpp_i<HIPQ_DPP_HALF_MIRROR>(I);
+          Im += hipq_dpp_i<HIPQ_DPP_HALF_MIRROR>(Im);
+          if (on && j == 0) {
             float4 v;
             v.x = (float)I;
             v.y = dw * A.dA[i][r];
