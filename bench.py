@@ -101,7 +101,7 @@ def main():
     blocks = torch.empty(capi.weight_nbytes("q4_K", N, K), dtype=torch.uint8, device="cuda")
     capi.quantize_weights("q4_K", w32, N, K, blocks, stream=stream)
     torch.cuda.synchronize()
-    n_copies = 12  # 12 x 28.3 MB = 340 MB of distinct weights, more than the 256 MB last-level cache
+    n_copies = 20  # 20 x 28.3 MB = 566 MB of distinct weights, twice the 256 MB last-level cache
     weights = [capi.Weight("q4_K", N, K, blocks, mem=capi.MEM_DEVICE) for _ in range(n_copies)]
     del w32
     c = torch.empty((M, N), device="cuda", dtype=torch.float32)
@@ -149,6 +149,47 @@ def main():
     big_gbs = big_bytes / (big_ms * 1e-3) / 1e9
     for w in big:
         w.destroy()
+
+    # ---- the other GEMV configurations: C1 (Q4_0, 4096 x 4096) and C3 (Q6_K lm_head) ----
+    def gemv_case(kind, n, k, copies, bytes_per_weight_num, bytes_per_weight_den):
+        w32_ = torch.randn((n, k), generator=gen, device="cuda", dtype=torch.float32) * 0.02
+        b_ = torch.empty(capi.weight_nbytes(kind, n, k), dtype=torch.uint8, device="cuda")
+        capi.quantize_weights(kind, w32_, n, k, b_, stream=stream)
+        torch.cuda.synchronize()
+        del w32_
+        ws_ = [capi.Weight(kind, n, k, b_, mem=capi.MEM_DEVICE) for _ in range(copies)]
+        a_ = torch.randn((1, k), generator=gen, device="cuda")
+        c_ = torch.empty((1, n), device="cuda")
+        capi.time_matmul(ws_, a_, 1, c_, 2 * copies, phase=1, stream=stream)
+        ms_ = capi.time_matmul(ws_, a_, 1, c_, max(60, 4 * copies), phase=1, stream=stream)
+        all_ms_ = capi.time_matmul(ws_, a_, 1, c_, max(60, 4 * copies), phase=0, stream=stream)
+        for w_ in ws_:
+            w_.destroy()
+        by_ = n * k * bytes_per_weight_num // bytes_per_weight_den + 4 * k + 4 * n
+        return ms_, all_ms_, by_
+
+    c1_ms, c1_all_ms, c1_bytes = gemv_case("q4_0", 4096, 4096, 60, 18, 32)
+    c3_ms, c3_all_ms, c3_bytes = gemv_case("q6_K", 151936, 4096, 2, 210, 256)
+
+    # ---- the FC stack of one decoder layer of C5 (Qwen3-0.6B shapes, Q4_0), quantizer included ----
+    def fc_stack(rows):
+        shapes = [(2048, 1024), (1024, 1024), (1024, 1024), (1024, 2048), (3072, 1024), (3072, 1024), (1024, 3072)]
+        total = 0.0
+        for n_, k_ in shapes:
+            w32_ = torch.randn((n_, k_), generator=gen, device="cuda", dtype=torch.float32) * 0.02
+            b_ = torch.empty(capi.weight_nbytes("q4_0", n_, k_), dtype=torch.uint8, device="cuda")
+            capi.quantize_weights("q4_0", w32_, n_, k_, b_, stream=stream)
+            torch.cuda.synchronize()
+            ws_ = [capi.Weight("q4_0", n_, k_, b_, mem=capi.MEM_DEVICE) for _ in range(8)]
+            a_ = torch.randn((rows, k_), generator=gen, device="cuda")
+            c_ = torch.empty((rows, n_), device="cuda")
+            capi.time_matmul(ws_, a_, rows, c_, 16, phase=0, stream=stream)
+            total += capi.time_matmul(ws_, a_, rows, c_, 80, phase=0, stream=stream)
+            for w_ in ws_:
+                w_.destroy()
+        return total
+
+    c5_prefill_ms, c5_decode_ms = fc_stack(512), fc_stack(1)
 
     # ---- the MoE block of configs[3]: 64 tokens, 128 experts, top-8, Q4_K ----------
     mt, mh, me, mi, mk = 64, 2048, 128, 768, 8
@@ -225,6 +266,22 @@ def main():
                          "achieved": round(big_gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(big_gbs / HBM_PEAK_GBS, 5), "kernel_ms": round(big_ms, 5),
                          "traffic": TRAFFIC_GEMV_LM_HEAD, "algorithmic_bytes_per_launch": big_bytes}},
+        "c1_q4_0_gemv": {
+            "workload": "Q4_0 GEMV M=1 K=4096 N=4096 (BASELINE configs[0]), 60 weight copies rotated (566 MB)",
+            "ms_per_call": round(c1_all_ms, 5),
+            "roofline": {"bound": "hbm", "achieved": round(c1_bytes / (c1_ms * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBS,
+                         "unit": "GB/s", "frac": round(c1_bytes / (c1_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 5),
+                         "kernel_ms": round(c1_ms, 5), "traffic": None, "algorithmic_bytes_per_launch": c1_bytes}},
+        "c3_q6_K_lm_head_gemv": {
+            "workload": "Q6_K GEMV M=1 K=4096 N=151936 (BASELINE configs[2]), 2 weight copies rotated (1 GB)",
+            "ms_per_call": round(c3_all_ms, 5),
+            "roofline": {"bound": "hbm", "achieved": round(c3_bytes / (c3_ms * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBS,
+                         "unit": "GB/s", "frac": round(c3_bytes / (c3_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 5),
+                         "kernel_ms": round(c3_ms, 5), "traffic": None, "algorithmic_bytes_per_launch": c3_bytes}},
+        "c5_fc_stack_per_layer": {
+            "workload": "the seven Q4_0 FCs of one Qwen3-0.6B-shaped decoder layer (BASELINE configs[4]) through "
+                        "hipq_matmul, quantizers included, 8 weight copies rotated per FC",
+            "prefill_512_rows_ms": round(c5_prefill_ms, 5), "decode_1_row_ms": round(c5_decode_ms, 5)},
         "moe_block": {
             "workload": "MoE FFN block (BASELINE configs[3]): 64 tokens, hidden 2048, 128 experts x "
                         "(gate/up 2048->768, down 768->2048) Q4_K, top-8; router, sort, experts, combine; "
