@@ -91,9 +91,11 @@ QAct qact_carve(int dtype_is_k, void *mem, int64_t M, int64_t K);
 /* Q8_K activations in the form the Q4_K prefill GEMM copies straight from    */
 /* HBM into LDS, tiled by 128 rows (mt = m / 128, rows padded to 128):         */
 /*   qt   [mt][K/128][16384]: one 128-row x 128-deep stage, laid out as        */
-/*        [m%128/32][k%128/32][k%2][m%32][k%32/2], i.e. 16-byte operands in the  */
-/*        order the lanes of the 32x32x32 int8 matrix instruction take them,    */
-/*        even k in lanes 0-31 and odd k in lanes 32-63 (as the weights' nibbles) */
+/*        [m%128/32][step 4][g 2][m%32][16 bytes]: the 16-byte operands in the  */
+/*        order the lanes of the 32x32x32 int8 matrix instruction take them.    */
+/*        Lane group g covers sub-blocks 4g .. 4g+3 of the super-block, two     */
+/*        steps each (first, second 16 values); an operand holds its 16 values   */
+/*        as the 8 even then the 8 odd ones (as the weights' nibbles unpack)     */
 /*   amin [mt][K/256][128][16] fp16: per row and super-block the eight         */
 /*        sub-block sums (bsum[2j] + bsum[2j+1]) split into a part in 0..63    */
 /*        (first 8) and a multiple of 64 (last 8), both exact in fp16          */

@@ -148,15 +148,18 @@ __global__ __launch_bounds__(256) void quantize_q8_K_kernel(
   } else if (MODE == Q8K_TILED) {
     const int64_t mt = m >> 7;
     const int r = (int)(m & 127);
-    /* lane holds elements 4*lane .. 4*lane+3 of the super-block */
-    const int stage = b * 2 + (lane >> 5);
-    const int kk = (lane * 4) & 127;
-    const int64_t tile = (mt * (2 * nsb) + stage) * 16384;
-    /* element k of a 32-deep step goes to half k % 2, byte k / 2: this lane's four
-     * values are two even and two odd elements */
-    const int off = ((r >> 5) * 4 + (kk >> 5)) * 1024 + (r & 31) * 16 + ((kk & 31) >> 1);
+    /* lane holds elements 4*lane .. 4*lane+3 of the super-block: sub-block lane / 8,
+     * whose 16-value half (lane / 4) % 2 is one 16-byte operand. The GEMM's lane
+     * (row, g) takes sub-blocks 4g .. 4g+3, two 32-deep steps each, so the operand
+     * belongs to step s = 2 * (sub-block % 4) + half of lane group g = sub-block / 4;
+     * within the operand the 8 even values come first, then the 8 odd ones (the
+     * order in which the weights' nibble bytes unpack). */
+    const int jb = lane >> 3, g = jb >> 2;
+    const int st = 2 * (jb & 3) + ((lane >> 2) & 1);
+    const int64_t tile = (mt * (2 * nsb) + b * 2 + (st >> 2)) * 16384;
+    const int off = ((r >> 5) * 4 + (st & 3)) * 1024 + (g * 32 + (r & 31)) * 16 + (lane & 3) * 2;
     *(uint16_t *)(q_out + tile + off) = (uint16_t)((q[0] & 0xff) | ((q[2] & 0xff) << 8));
-    *(uint16_t *)(q_out + tile + off + 512) = (uint16_t)((q[1] & 0xff) | ((q[3] & 0xff) << 8));
+    *(uint16_t *)(q_out + tile + off + 8) = (uint16_t)((q[1] & 0xff) | ((q[3] & 0xff) << 8));
     const int64_t rb = (mt * nsb + b) * 128 + r;
     if (lane == 0) d_out[rb] = d;
     const int bs = gsum + __shfl_xor(gsum, 4, HIPQ_WAVE); /* two 16-value groups = one sub-block */
