@@ -55,19 +55,20 @@ typedef _Float16 v8h __attribute__((ext_vector_type(8)));
 typedef unsigned short v2us __attribute__((ext_vector_type(2)));
 typedef __amdgpu_buffer_rsrc_t rsrc_t;
 
-constexpr int BM = 64, BN = 128;
-constexpr int TM = BM / 32; /* MFMA row tiles per wavefront */
-constexpr int NT = 256;          /* 4 wavefronts, 64 x 32 outputs each */
-constexpr int ASTAGE = BM * 128; /* bytes of one 128-deep activation stage of the tile */
+constexpr int BN = 128;
+constexpr int NT = 256;           /* 4 wavefronts side by side, 32 columns each */
 constexpr int QSTAGE = 128 * 128; /* bytes of one stage as the quantizer writes it (128 rows) */
 
-/* LDS of a workgroup */
-struct Smem {
+/* LDS of a workgroup whose wavefronts hold TM row tiles of 32 (tile height 32 * TM) */
+template <int TM> struct Smem {
+  static constexpr int BM = 32 * TM;
+  static constexpr int ASTAGE = BM * 128; /* bytes of one 128-deep activation stage of the tile */
   int8_t a[3][ASTAGE];       /* ring of stages, each [row/32][step 4][lane 64][16] */
   _Float16 amin[2][BM * 16]; /* per super-block: per row 8 low parts, 8 high parts of bsum32_j */
   float dA[2][BM];
 };
-static_assert(sizeof(Smem) * 3 <= 160 * 1024, "three workgroups per CU must fit the 160 KB LDS");
+static_assert(sizeof(Smem<2>) * 3 <= 160 * 1024 && sizeof(Smem<4>) * 2 <= 160 * 1024,
+              "three workgroups of 64 rows or two of 128 rows per CU must fit the 160 KB LDS");
 
 __device__ __forceinline__ uint32_t pk_scale(uint32_t x, uint32_t digit2) {
   const v2us r = __builtin_bit_cast(v2us, x) * __builtin_bit_cast(v2us, digit2);
@@ -101,24 +102,36 @@ __device__ __forceinline__ void load_wh(WHalf &W, const Src &sr, int sb, int h) 
   W.q[0] = hipq_ld_global(sr.wq + sb * 8 + 2 * h);
   W.q[1] = hipq_ld_global(sr.wq + sb * 8 + 2 * h + 1);
 }
-/* stage (128 deep) -> ring slot: wavefront w copies the 4 KB of rows 32w .. 32w+31 */
-__device__ __forceinline__ void dma_a(const Src &sr, Smem &sm, int stage, int slot) {
-  const uint32_t so = (uint32_t)stage * QSTAGE + sr.wave * 2048;
-  int8_t *l = sm.a[slot] + sr.wave * 2048;
+/* stage (128 deep) -> ring slot: each wavefront copies a quarter of the tile's stage, TM KB */
+template <int TM>
+__device__ __forceinline__ void dma_a(const Src &sr, Smem<TM> &sm, int stage, int slot) {
+  const uint32_t so = (uint32_t)stage * QSTAGE + sr.wave * (TM * 1024);
+  int8_t *l = sm.a[slot] + sr.wave * (TM * 1024);
 #pragma unroll
-  for (int i = 0; i < 2; ++i) dma16(sr.qt, sr.lane * 16, so + i * 1024, l + i * 1024);
+  for (int i = 0; i < TM; ++i) dma16(sr.qt, sr.lane * 16, so + i * 1024, l + i * 1024);
 }
-__device__ __forceinline__ void dma_rows(const Src &sr, Smem &sm, int sb, int buf) {
-  if (sr.wave < 2) dma16(sr.amin, sr.lane * 16, (uint32_t)sb * (128 * 32) + sr.wave * 1024, (char *)sm.amin[buf] + sr.wave * 1024);
-  if (sr.wave == 2) dma4(sr.dAt, sr.lane * 4, (uint32_t)sb * (128 * 4), sm.dA[buf]);
+/* per-row data of a super-block: 32 bytes of bsum parts and one scale per row */
+template <int TM>
+__device__ __forceinline__ void dma_rows(const Src &sr, Smem<TM> &sm, int sb, int buf) {
+  if (sr.wave < TM) /* uniform per wavefront */
+    dma16(sr.amin, sr.lane * 16, (uint32_t)sb * (128 * 32) + sr.wave * 1024, (char *)sm.amin[buf] + sr.wave * 1024);
+  if (TM == 2 ? sr.wave == 2 : sr.wave < 2)
+    dma4(sr.dAt, sr.lane * 4, (uint32_t)sb * (128 * 4) + (TM == 2 ? 0 : sr.wave * 256),
+         sm.dA[buf] + (TM == 2 ? 0 : sr.wave * 64));
 }
+/* Loads a wavefront issues at least per stage (some wavefronts copy no per-row
+ * data): what may stay in flight at the stage's barrier. First / second half. */
+template <int TM> struct InFlight {
+  static constexpr int FIRST = TM + (TM == 2 ? 0 : 1) + 2; /* copies of the ring, row data, two nibble loads */
+  static constexpr int SECOND = TM + 3;                    /* copies of the ring, two nibble loads, the header */
+};
 
 /* four 32-deep steps of one 128-deep stage: H = which half of the super-block */
-template <int H>
-__device__ __forceinline__ void stage_mma(const Smem &sm, int slot, const WHalf &W, uint32_t slo, uint32_t shi,
+template <int H, int TM>
+__device__ __forceinline__ void stage_mma(const Smem<TM> &sm, int slot, const WHalf &W, uint32_t slo, uint32_t shi,
                                           int lane, v16i (&Dlo)[TM], v16i (&Dhi)[TM]) {
   const v16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-  const int8_t *pa = sm.a[0] + slot * ASTAGE + lane * 16;
+  const int8_t *pa = sm.a[0] + slot * Smem<TM>::ASTAGE + lane * 16;
   v4i a[2][TM];
 #pragma unroll
   for (int tm = 0; tm < TM; ++tm) a[0][tm] = *(const v4i *)(pa + (tm * 4) * 1024);
@@ -144,7 +157,8 @@ __device__ __forceinline__ void stage_mma(const Smem &sm, int slot, const WHalf 
   }
 }
 
-__device__ __forceinline__ void epilogue(const Smem &sm, int buf, const uint4 &hd, int lane, const v16i (&Dlo)[TM],
+template <int TM>
+__device__ __forceinline__ void epilogue(const Smem<TM> &sm, int buf, const uint4 &hd, int lane, const v16i (&Dlo)[TM],
                                          const v16i (&Dhi)[TM], float (&acc)[TM][16]) {
   const v16f zero16f = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
   const int i32 = lane & 31, g = lane >> 5;
@@ -181,12 +195,14 @@ __device__ __forceinline__ void epilogue(const Smem &sm, int buf, const uint4 &h
   }
 }
 
-__global__ __launch_bounds__(NT, 3) void gemm_q4k_kernel(WView w, const int8_t *__restrict__ qt,
+template <int TM>
+__global__ __launch_bounds__(NT, TM == 2 ? 3 : 2) void gemm_q4k_kernel(WView w, const int8_t *__restrict__ qt,
                                                          const uint16_t *__restrict__ amin,
                                                          const float *__restrict__ dAt, int M, int mtiles,
                                                          int ntiles, float *__restrict__ C, int64_t ldc) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-  Smem &sm = *reinterpret_cast<Smem *>(smem_raw);
+  Smem<TM> &sm = *reinterpret_cast<Smem<TM> *>(smem_raw);
+  constexpr int BM = 32 * TM;
   const int id = blockIdx.x;
   const int xcd = id & 7, qd = id >> 3;
   const int mt = qd % mtiles, nt = (qd / mtiles) * 8 + xcd;
@@ -198,8 +214,8 @@ __global__ __launch_bounds__(NT, 3) void gemm_q4k_kernel(WView w, const int8_t *
   const int i32 = lane & 31, g = lane >> 5;
 
   Src sr;
-  /* the quantizer tiles by 128 rows: this 64-row tile is half mt & 1 of quantizer tile mt / 2 */
-  const int qt128 = mt >> 1, hrow = mt & 1;
+  /* the quantizer tiles by 128 rows: a 64-row tile is half mt & 1 of quantizer tile mt / 2 */
+  const int qt128 = TM == 2 ? mt >> 1 : mt, hrow = TM == 2 ? mt & 1 : 0;
   sr.qt = make_rsrc(qt + (size_t)qt128 * (2 * nsb) * QSTAGE + hrow * 8192, (uint32_t)(2 * nsb) * QSTAGE);
   sr.amin = make_rsrc(amin + ((size_t)qt128 * nsb * 128 + hrow * 64) * 16, (uint32_t)nsb * 128 * 32);
   sr.dAt = make_rsrc(dAt + (size_t)qt128 * nsb * 128 + hrow * 64, (uint32_t)nsb * 128 * 4);
@@ -240,7 +256,7 @@ __global__ __launch_bounds__(NT, 3) void gemm_q4k_kernel(WView w, const int8_t *
       load_wh(Wb, sr, sb, 1);
       stage_mma<0>(sm, slot, Wa, slo, shi, lane, Dlo, Dhi);
       slot = slot == 2 ? 0 : slot + 1;
-      sync_lds<4>();
+      sync_lds<InFlight<TM>::FIRST>();
     }
     {
       const int s2 = slot >= 1 ? slot - 1 : 2;
@@ -251,7 +267,7 @@ __global__ __launch_bounds__(NT, 3) void gemm_q4k_kernel(WView w, const int8_t *
       slot = slot == 2 ? 0 : slot + 1;
     }
     epilogue(sm, eb, hd, lane, Dlo, Dhi, acc);
-    sync_lds<5>();
+    sync_lds<InFlight<TM>::SECOND>();
   };
   int sb = 0;
   for (; sb + 1 < nsb; sb += 2) {
@@ -275,17 +291,29 @@ __global__ __launch_bounds__(NT, 3) void gemm_q4k_kernel(WView w, const int8_t *
 
 namespace hipq {
 
-int launch_gemm_q4k(const hipq_weight *w, const QActTiled *qa, int M, float *C, int64_t ldc, hipStream_t s) {
-  const int mtiles = (M + BM - 1) / BM;
-  if ((M + 127) / 128 != qa->mtiles || qa->K != w->K)
-    return fail(HIPQ_ERR_INVALID_ARGUMENT, "tiled activations do not match the matmul shape");
+template <int TM>
+int launch_tiles(const hipq_weight *w, const QActTiled *qa, int M, float *C, int64_t ldc, hipStream_t s) {
+  const int mtiles = (M + 32 * TM - 1) / (32 * TM);
   const int ntiles = (int)((w->N + BN - 1) / BN);
   const int ngroups = (ntiles + 7) / 8;
   const unsigned grid = (unsigned)(mtiles * ngroups * 8);
-  hipLaunchKernelGGL(gemm_q4k_kernel, dim3(grid), dim3(NT), sizeof(Smem), s, wview(w), qa->qt, qa->amin, qa->dAt, M,
-                     mtiles, ntiles, C, ldc);
+  hipLaunchKernelGGL(gemm_q4k_kernel<TM>, dim3(grid), dim3(NT), sizeof(Smem<TM>), s, wview(w), qa->qt, qa->amin,
+                     qa->dAt, M, mtiles, ntiles, C, ldc);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
+}
+
+int launch_gemm_q4k(const hipq_weight *w, const QActTiled *qa, int M, float *C, int64_t ldc, hipStream_t s) {
+  if ((M + 127) / 128 != qa->mtiles || qa->K != w->K)
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "tiled activations do not match the matmul shape");
+  /* 128-row tiles do a fifth more work per CU and time (the weight expansion is
+   * shared by twice the rows) but only two workgroups fit a CU: 512 tiles per round
+   * against 768 of the 64-row kind. Pick by the number of rounds. */
+  const int64_t nt = (w->N + BN - 1) / BN;
+  const int64_t rounds64 = (((int64_t)(M + 63) / 64) * nt + 767) / 768;
+  const int64_t rounds128 = (((int64_t)(M + 127) / 128) * nt + 511) / 512;
+  if (rounds128 * 6 < rounds64 * 5) return launch_tiles<4>(w, qa, M, C, ldc, s);
+  return launch_tiles<2>(w, qa, M, C, ldc, s);
 }
 
 } // namespace hipq

@@ -73,6 +73,21 @@ def test_gemm_matches_oracle(hipq, cr, kind, m, n, k):
     assert gu.rel_err(got, ref) <= gu.TOL, gu.rel_err(got, ref)
 
 
+def test_q4_K_gemm_tall_tiles(hipq, cr):
+    """A shape for which the Q4_K GEMM picks its 128-row tiles (two rounds of 64-row
+    tiles against one of 128-row tiles), with M not a multiple of the tile height."""
+    import gpu_util as gu
+    m, n, k = 1000, 8192, 512
+    blocks = _weights(cr, "q4_K", n, k, seed=47)
+    a = synth.normal(447, (m, k))
+    ref = cr.gemm(cr.oracle(), "q4_K", a, blocks, n)
+    w = capi.Weight("q4_K", n, k, blocks)
+    got = gu.gpu_matmul(w, a)
+    w.destroy()
+    assert not np.isnan(got).any()
+    assert gu.rel_err(got, ref) <= gu.TOL, gu.rel_err(got, ref)
+
+
 @pytest.mark.parametrize("kind", ["q4_0", "q4_K"])
 def test_x8_layout_equals_canonical(hipq, cr, kind):
     """Weights handed over in NNTrainer's 8-row interleave give the same outputs."""
