@@ -24,9 +24,9 @@ HBM_PEAK_GBS = 8000.0    # MI355X HBM3E peak, GB/s
 # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs of this script, scaled by
 # what the same counters read for its 256 MiB device copy (profiles/gemm_q4k_prefill_m512_k4096_n12288.txt,
 # profiles/gemv_q4k_decode_m1_k4096.txt, profiles/moe_block_q4k_64tok_128experts.txt). Measured once, not live: counters need the profiler attached.
-TRAFFIC_GEMM_C2 = 72.98e6 + 25.17e6
-TRAFFIC_GEMV_C2 = 28.42e6 + 0.05e6
-TRAFFIC_GEMV_LM_HEAD = 354.13e6 + 0.61e6
+TRAFFIC_GEMM_C2 = 48.68e6 + 25.17e6
+TRAFFIC_GEMV_C2 = 28.45e6 + 0.05e6
+TRAFFIC_GEMV_LM_HEAD = 350.25e6 + 0.62e6
 METRIC = "Q4 GEMV effective GB/s (%HBM peak); prefill GEMM int8 TOPS (%MFMA peak)"
 
 
@@ -246,7 +246,7 @@ def main():
         "config": {"workload": "Q4_K x Q8_K prefill GEMM, M=512 K=4096 N=12288 (BASELINE configs[1]); "
                                "step = activation quantizer + block-dot GEMM on HBM-resident inputs",
                    "M": M, "K": K, "N": N, "weight_copies_rotated": n_copies},
-        "roofline": {"bound": "mfma", "kernel": "gemm_q4k_kernel", "achieved": round(gemm_tops, 3),
+        "roofline": {"bound": "mfma", "kernel": "gemm_q4k_kernel<2>", "achieved": round(gemm_tops, 3),
                      "peak": INT8_PEAK_TOPS, "unit": "TOP/s", "frac": round(gemm_tops / INT8_PEAK_TOPS, 5),
                      "kernel_ms": round(gemm_ms, 5), "traffic": TRAFFIC_GEMM_C2,
                      "algorithmic_ops_per_launch": ops},
@@ -289,7 +289,7 @@ def main():
             "ms_per_block": round(moe_ms, 5), "active_experts": active,
             "roofline": {"bound": "hbm", "achieved": round(moe_gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(moe_gbs / HBM_PEAK_GBS, 5), "algorithmic_bytes_per_block": moe_bytes,
-                         "traffic": 234.0e6 + 117.1e6 + 7.9e6}},
+                         "traffic": 233.2e6 + 117.1e6 + 7.9e6}},
     }
     if not args.no_cpu:
         capi.matmul(weights[0], a, M, c, stream=stream)

@@ -22,11 +22,14 @@
  * result is exact (< 2^24). Per super-block and output the ALU does
  *       acc += dA * (d * float(Dlo + 8*Dhi) - dmin * Im).
  *
- * Tiling. A workgroup (4 wavefronts side by side) owns a 64 x 128 tile of C, each
- * wavefront 64 rows x 32 columns (2 MFMA row tiles x 2 digit chains). K is walked
- * in stages of 128. Three workgroups share a CU (29 KB of LDS and at most 168
- * registers each), so one's matrix phase overlaps the others' vector work, and
- * the 768 tiles of the 512 x 12288 reference shape are all resident at once.
+ * Tiling. A workgroup (4 wavefronts side by side) owns a 64 x 128 or 128 x 128 tile
+ * of C, each wavefront all its rows x 32 columns (2 or 4 MFMA row tiles x 2 digit
+ * chains). K is walked in stages of 128. Three workgroups of the 64-row kind share
+ * a CU (29 KB of LDS, at most 168 registers), so one's matrix phase overlaps the
+ * others' vector work and the 768 tiles of the 512 x 12288 reference shape are all
+ * resident at once; of the 128-row kind two fit (57 KB, 256 registers), which do a
+ * fifth more work per unit of time because the weight expansion is shared by twice
+ * the rows. The launcher picks by the number of rounds the grid takes.
  *  - Weights never pass through LDS: a wavefront owns its 32 columns for the whole
  *    of K, lane (n, g) reads the 64 bytes of sub-blocks 4g .. 4g+3 of column n one
  *    stage ahead (ordinary loads: two lanes share a 128-byte line) and expands 16
