@@ -137,6 +137,28 @@ def test_matmul_multi_shares_quantization(hipq, cr):
         w.destroy()
 
 
+@pytest.mark.parametrize("kind,m", [("q4_K", 1), ("q4_K", 40), ("q6_K", 3)])
+def test_matmul_multi_other_formats_and_prefill(hipq, cr, kind, m):
+    """The multi-weight entry with the Q8_K formats, one row and a prefill chunk (the
+    Q4_K prefill goes through the tiled activations and the matrix-core GEMM)."""
+    import gpu_util as gu
+    import torch
+    k = 512
+    ns = [384, 128, 256]
+    blocks = [_weights(cr, kind, n, k, seed=80 + i) for i, n in enumerate(ns)]
+    ws = [capi.Weight(kind, n, k, b) for n, b in zip(ns, blocks)]
+    a = synth.normal(83, (m, k))
+    outs = [torch.full((m, n), float("nan"), device="cuda") for n in ns]
+    capi.matmul_multi(ws, gu.dev(a), m, outs, stream=gu.stream())
+    torch.cuda.synchronize()
+    for n, b, o in zip(ns, blocks, outs):
+        got = o.cpu().numpy()
+        assert not np.isnan(got).any()
+        assert gu.rel_err(got, cr.gemm(cr.oracle(), kind, a, b, n)) <= gu.TOL
+    for w in ws:
+        w.destroy()
+
+
 def test_bad_arguments_are_reported(hipq):
     with pytest.raises(capi.HipqError) as e:
         capi.weight_nbytes("q4_K", 16, 100)  # K not a multiple of 256 (q4_k_tensor.cpp:23-27)
