@@ -300,8 +300,8 @@ template <int T, int R, bool PW, int KC> struct GemvQ4K {
 };
 
 /* ---- Q6_K ----------------------------------------------------------------------- */
-/* A unit is 64 weights = 2 x 16 B of ql + 16 B of qh, unit uu = half*2 + hl of a
- * super-block. Dword t of the unit belongs to partial l = hl*4 + t; lanes uu and
+/* A unit is 64 weights = 16 B of each ql plane + 16 B of qh, unit uu = half*2 + hl of
+ * a super-block. Dword t of the unit belongs to partial l = hl*4 + t; lanes uu and
  * uu^2 hold the two 128-element halves. */
 template <int T, int R, bool PW, int KC> struct GemvQ6K {
   static constexpr int MAXU = GemvUnits<HIPQ_Q6_K, T, KC>::MAXU;
@@ -336,7 +336,9 @@ template <int T, int R, bool PW, int KC> struct GemvQ6K {
   __device__ static __forceinline__ void load_w(Wt &W, const WView &w, int row, int tl, int k0,
                                                 int kc) {
     const int nsb = w.K >> 8, b0 = k0 >> 8, un = kc >> 6;
-    const uint8_t *qlrow = w.qs + (size_t)row * (w.K >> 1) + (size_t)b0 * 128;
+    /* two ql planes of N * K / 4 bytes each: a unit's first and second 16 bytes */
+    const uint8_t *qlrow = w.qs + (size_t)row * (w.K >> 2) + (size_t)b0 * 64;
+    const uint8_t *qlrow2 = qlrow + (size_t)w.N * (w.K >> 2);
     const uint8_t *qhrow = w.qh + (size_t)row * (w.K >> 2) + (size_t)b0 * 64;
     const int8_t *scrow = w.sc + (size_t)row * (w.K >> 4) + (size_t)b0 * 16;
     const uint16_t *drow = w.d + (size_t)row * nsb + b0;
@@ -344,12 +346,12 @@ template <int T, int R, bool PW, int KC> struct GemvQ6K {
     for (int i = 0; i < MAXU; ++i) {
       if (i * T >= un) break;
       const int u = min(tl + i * T, un - 1);
-      const int b = u >> 2, uu = u & 3, half = uu >> 1, hl = uu & 1;
-      const uint8_t *ql = qlrow + b * 128 + half * 64 + hl * 16;
-      W.qa[i] = hipq_ld_stream((const uint4 *)ql);
-      W.qb[i] = hipq_ld_stream((const uint4 *)(ql + 32));
-      W.qh[i] = hipq_ld_stream((const uint4 *)(qhrow + b * 64 + half * 32 + hl * 16));
-      W.scw[i] = hipq_ld_global((const int *)(scrow + b * 16 + uu * 4));
+      const int b = u >> 2;
+      /* consecutive lanes take consecutive 16-byte pieces of every plane */
+      W.qa[i] = hipq_ld_stream((const uint4 *)(qlrow + u * 16));
+      W.qb[i] = hipq_ld_stream((const uint4 *)(qlrow2 + u * 16));
+      W.qh[i] = hipq_ld_stream((const uint4 *)(qhrow + u * 16));
+      W.scw[i] = hipq_ld_global((const int *)(scrow + u * 4));
       W.d[i] = hipq_ld_global(drow + b);
     }
   }

@@ -25,7 +25,10 @@
 /*   Q4_K: qs [N][K/2]  (128 B per super-block: sub-block j = bytes 16j..16j+15, */
 /*                      weight 2i low / 2i+1 high nibble of byte i)             */
 /*         hdr[N][K/256][16] = {fp16 d, fp16 dmin, scales[12]}                */
-/*   Q6_K: qs [N][K/2]  (ql, 128 B per super-block, byte order of block_q6_K) */
+/*   Q6_K: qs [2][N][K/4] (ql in two planes, 64 B per super-block each: unit  */
+/*                      uu = half*2 + hl holds bytes half*64 + hl*16 .. +15 of  */
+/*                      block_q6_K::ql in the first and those 32 further on in   */
+/*                      the second)                                              */
 /*         qh [N][K/4]  (64 B per super-block, same byte order)               */
 /*         sc [N][K/16] int8, regrouped per super-block as [unit u][group g]  */
 /*                      = scales[(u>>1)*8 + g*2 + (u&1)]                      */

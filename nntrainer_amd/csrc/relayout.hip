@@ -103,7 +103,17 @@ __global__ void relayout_q6_K(const uint8_t *__restrict__ src, int64_t total,
   const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (i >= total) return;
   const uint8_t *blk = src + i * 210;
-  for (int k = 0; k < 128; ++k) ql[i * 128 + k] = blk[k];
+  /* ql in two planes: unit uu = half * 2 + hl takes bytes half*64 + hl*16 .. +15 (low
+   * nibbles: elements l, high: l + 64) from the first and the 16 bytes 32 further on
+   * (elements l + 32, l + 96) from the second, so that the units of a row are
+   * consecutive 16-byte pieces in both */
+  uint8_t *qlb = ql + total * 64;
+  for (int uu = 0; uu < 4; ++uu)
+    for (int t = 0; t < 16; ++t) {
+      const int o = (uu >> 1) * 64 + (uu & 1) * 16 + t;
+      ql[i * 64 + uu * 16 + t] = blk[o];
+      qlb[i * 64 + uu * 16 + t] = blk[o + 32];
+    }
   for (int k = 0; k < 64; ++k) qh[i * 64 + k] = blk[128 + k];
   for (int u = 0; u < 4; ++u)
     for (int g = 0; g < 4; ++g)
