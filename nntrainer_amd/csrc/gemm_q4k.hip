@@ -209,7 +209,7 @@ __global__ __launch_bounds__(NT, TM == 2 ? 3 : 2) void gemm_q4k_kernel(WView w, 
   const int id = blockIdx.x;
   const int xcd = id & 7, qd = id >> 3;
   const int mt = qd % mtiles, nt = (qd / mtiles) * 8 + xcd;
-  if (nt >= ntiles) return;
+  if (nt >= ntiles) return; /* uniform per workgroup */
   const int m0 = mt * BM, n0 = nt * BN;
   const int nsb = w.K >> 8;
   const int lane = threadIdx.x & 63;
@@ -245,6 +245,12 @@ __global__ __launch_bounds__(NT, TM == 2 ? 3 : 2) void gemm_q4k_kernel(WView w, 
   sync_lds<0>();
   int slot = 0; /* ring slot of the current stage */
   const int nstage = 2 * nsb;
+  /* One super-block = two 128-deep stages. Each stage first issues what later
+   * stages need (the copy of the stage after next into the ring slot read last,
+   * the other half's nibbles, once per super-block the next one's row data and
+   * header), then runs its four matrix steps; the barrier at its end waits for the
+   * loads issued BEFORE this stage (they retire in order) and leaves this stage's in
+   * flight. hd / hdn and Wa / Wb alternate between consecutive super-blocks. */
   auto super_block = [&](int sb, const uint4 &hd, uint4 &hdn, int eb) {
     /* 6-bit scales of sub-blocks 4g .. 4g+3, one per byte, as two 3-bit digits */
     const uint32_t s03 = hd.y & 0x3f3f3f3fu;
