@@ -21,13 +21,14 @@
  *
  * Launch plan (all on one stream, no host synchronisation; grids do not depend
  * on device data): router logits (optional) -> route -> sort of the pairs by
- * expert (one workgroup; count / scan / scatter kernels for very long chunks) ->
- * quantize x -> grouped gate+up product with fused SwiGLU over (column tiles x
- * experts) -> quantize h -> grouped down product scaled by the routing weight ->
- * combine. Q4_K experts whose rows fit the LDS run on the matrix cores, 8 to 32
- * tokens of an expert per pass over its weights; the other formats and longer rows
- * use the decode GEMV's engine, four tokens per pass. Both carry the reference's
- * bits for every single-row product.
+ * expert (one workgroup; count / scan / scatter kernels for very long chunks),
+ * which also lists the work items (expert, chunk of its slots) -> quantize x ->
+ * grouped gate+up product with fused SwiGLU over (column tiles x work items) ->
+ * quantize h -> grouped down product scaled by the routing weight -> combine.
+ * Q4_K experts whose rows fit the LDS run on the matrix cores, 8 to 32 tokens of
+ * an expert per work item; the other formats and longer rows use the decode
+ * GEMV's engine, four tokens per pass over an expert's weights. Both carry the
+ * reference's bits for every single-row product.
  */
 #include "gemv_device.h"
 
@@ -42,6 +43,7 @@ struct MoeBufs {
   int *counts, *offsets, *cursor;
   int *slot_pair; /* pair (token * topk + k) of each slot */
   int *tok_slots; /* [T][topk]: a token's slots in ascending expert id */
+  int *items;     /* [0] = number of work items, then (expert, first slot) per item */
   float *h;       /* [P][I] by slot */
   float *contrib; /* [P][H] by slot */
   void *xq_mem, *hq_mem;
@@ -74,6 +76,8 @@ size_t carve(const hipq_moe_desc &d, int is_k, uint8_t *base, MoeBufs *b) {
   if (b) b->slot_pair = (int *)p;
   p = take(P * 4);
   if (b) b->tok_slots = (int *)p;
+  p = take((2 * (E + P) + 2) * 4);
+  if (b) b->items = (int *)p;
   p = take(P * I * 4);
   if (b) b->h = (float *)p;
   p = take(P * H * 4);
@@ -197,11 +201,14 @@ __global__ __launch_bounds__(1024) void sort_pairs_kernel(const int32_t *__restr
                                                           int E, int topk,
                                                           int *__restrict__ offsets,
                                                           int *__restrict__ slot_pair,
-                                                          int *__restrict__ tok_slots) {
+                                                          int *__restrict__ tok_slots, int chunk,
+                                                          int *__restrict__ items) {
   __shared__ int cnt[1024];
   __shared__ int off[1024];
+  __shared__ int nitems;
   const int t = threadIdx.x;
   cnt[t] = 0;
+  if (t == 0) nitems = 0;
   __syncthreads();
   for (int i = t; i < P; i += 1024) atomicAdd(&cnt[idx[i]], 1);
   __syncthreads();
@@ -218,7 +225,17 @@ __global__ __launch_bounds__(1024) void sort_pairs_kernel(const int32_t *__restr
   const int excl = off[t] - own;
   if (t < E) offsets[t] = excl;
   if (t == E - 1) offsets[E] = off[t];
+  /* work items of the expert kernels: an expert's slots in chunks (any order) */
+  if (chunk > 0 && t < E && own > 0) {
+    const int nch = (own + chunk - 1) / chunk;
+    const int at = atomicAdd(&nitems, nch);
+    for (int c = 0; c < nch; ++c) {
+      items[2 + 2 * (at + c)] = t;
+      items[3 + 2 * (at + c)] = excl + c * chunk;
+    }
+  }
   __syncthreads();
+  if (t == 0) items[0] = nitems;
   off[t] = excl;
   cnt[t] = 0;
   __syncthreads();
@@ -241,15 +258,22 @@ __global__ void count_kernel(const int32_t *__restrict__ idx, int P, int *__rest
 }
 
 __global__ void scan_kernel(const int *__restrict__ counts, int E, int *__restrict__ offsets,
-                            int *__restrict__ cursor) {
+                            int *__restrict__ cursor, int chunk, int *__restrict__ items) {
   if (threadIdx.x == 0 && blockIdx.x == 0) {
-    int acc = 0;
+    int acc = 0, n = 0;
     for (int e = 0; e < E; ++e) {
       offsets[e] = acc;
+      if (chunk > 0)
+        for (int c = 0; c < counts[e]; c += chunk) {
+          items[2 + 2 * n] = e;
+          items[3 + 2 * n] = acc + c;
+          ++n;
+        }
       acc += counts[e];
       cursor[e] = 0;
     }
     offsets[E] = acc;
+    items[0] = n;
   }
 }
 
@@ -436,46 +460,40 @@ __global__ __launch_bounds__(256) void down_long_kernel(const WView *__restrict_
  * 16g .. 16g+15 of it for weight row n, even ones (low nibbles) in operand bytes
  * 0-7 and odd ones in bytes 8-15, and the quantizer stores every 16-value group of
  * the activations in that order; the step's sums take the sub-block's 6-bit scale
- * in an integer multiply-add. The mins
- * go through one v_mfma_f32_32x32x16_f16 per super-block with the sub-block sums
- * split into two fp16-exact parts. Every integer is exact and the fp32 chain per
- * output is the single-row kernel's, so the results carry the same bits:
- *   acc = fma(float(I), d * dA, acc); accm = fma(float(Im), dmin * dA, accm). */
+ * in an integer multiply-add. The mins go through one v_mfma_f32_32x32x16_f16 per
+ * super-block with the sub-block sums split into two fp16-exact parts. Every
+ * integer is exact and the fp32 chain per output is the single-row kernel's, so the
+ * results carry the same bits:
+ *   acc = fma(float(I), d * dA, acc); accm = fma(float(Im), dmin * dA, accm).
+ *
+ * The unit of work is an item of the list the pair sort writes: up to TC slots of
+ * one expert. A workgroup takes one item and 128 (gate/up) or 256 (down) columns,
+ * so an expert with more than TC tokens is served by several workgroups side by
+ * side instead of one that walks its weights several times. */
+typedef int mv2i __attribute__((ext_vector_type(2)));
 typedef int mv4i __attribute__((ext_vector_type(4)));
 typedef int mv16i __attribute__((ext_vector_type(16)));
 typedef float mv16f __attribute__((ext_vector_type(16)));
 typedef _Float16 mv8h __attribute__((ext_vector_type(8)));
-typedef unsigned short mv2us __attribute__((ext_vector_type(2)));
 
-__device__ __forceinline__ uint32_t mma_pk_scale(uint32_t x, uint32_t digit2) {
-  const mv2us r = __builtin_bit_cast(mv2us, x) * __builtin_bit_cast(mv2us, digit2);
-  return __builtin_bit_cast(uint32_t, r);
-}
-
-/* LDS of a workgroup: TC activation rows, padded so that the lanes of a 128-bit
- * read fall into different banks, then one ring of weight tiles per wavefront. */
-constexpr int XTILE = 32 * 128 + 64 * 16; /* nibbles of 32 weight rows for one super-block, then their headers (twice) */
+/* LDS of a workgroup: the item's TC activation rows, padded so that the lanes of a
+ * 128-bit read fall into different banks. */
 struct XLds {
-  int8_t *q;           /* [TC][K + 16] */
-  uint8_t *amin;       /* [TC][nsb][32 bytes] */
-  float *dA;           /* [nsb][TC] */
-  int *rows;           /* [TC] source rows of the chunk */
-  unsigned char *ring; /* this wavefront's [XD][XTILE], XD = 2 or 3 super-blocks */
+  int8_t *q;     /* [TC][K + 16] */
+  uint8_t *amin; /* [TC][nsb][32 bytes] */
+  float *dA;     /* [nsb][TC] */
+  int *rows;     /* [TC] source rows of the item */
 };
-__host__ __device__ inline size_t xlds_act_bytes(int TC, int K) {
+__host__ __device__ inline size_t xlds_bytes(int TC, int K) {
   const size_t b = (size_t)TC * (K + 16) + (size_t)TC * (K / 256) * 32 + (size_t)TC * (K / 256) * 4 + TC * 4;
   return (b + 255) & ~(size_t)255;
 }
-__host__ __device__ inline size_t xlds_bytes(int TC, int K, int waves, int xd) {
-  return xlds_act_bytes(TC, K) + (size_t)waves * xd * XTILE;
-}
-__device__ __forceinline__ XLds xlds_carve(unsigned char *base, int TC, int K, int wave, int xd) {
+__device__ __forceinline__ XLds xlds_carve(unsigned char *base, int TC, int K) {
   XLds l;
   l.q = (int8_t *)base;
   l.amin = (uint8_t *)base + (size_t)TC * (K + 16);
   l.dA = (float *)(l.amin + (size_t)TC * (K / 256) * 32);
   l.rows = (int *)(l.dA + (size_t)TC * (K / 256));
-  l.ring = base + xlds_act_bytes(TC, K) + wave * (xd * XTILE);
   return l;
 }
 
@@ -512,133 +530,70 @@ __device__ __forceinline__ void stage_rows(const XLds &l, const QView &a) {
   }
 }
 
-/* The weight stream of a wavefront. A super-block of a tile's 32 rows is 32 lines of
- * 128 bytes; four direct-to-LDS copies fetch 8 whole lines each (8 lanes per line:
- * fully coalesced) into the next ring slot, so no registers hold weights in flight
- * and the ring can run several super-blocks ahead. Lane L of copy i fetches piece
- * (L % 8) ^ (L / 8) of row 8i + L / 8 and the hardware stores it at slot byte
- * 1024 i + 16 L: row r of the slot holds its eight 16-byte pieces XOR-swizzled by
- * r % 8, which spreads the later 128-bit reads of a column of pieces over the banks.
- * A fifth copy brings each lane the 16-byte header of its row. */
-typedef __amdgpu_buffer_rsrc_t xrsrc_t;
-struct XStream {
-  xrsrc_t rs;       /* the tile's nibble plane */
-  uint32_t voff[4]; /* this lane's byte offset for each of the four copies, super-block 0 */
-  uint32_t so;      /* + byte offset of the super-block under the cursor */
-  xrsrc_t rh;       /* the tile's header plane */
-  uint32_t hoff;    /* this lane's row (lane % 32) in it, super-block 0 */
-  uint32_t hso;     /* + byte offset of the super-block under the cursor */
+/* The weight stream. Lane (n, g) of a wavefront loads 16-byte piece 2i + g of weight row n for i = 0..3
+ * (four 128-bit loads cover the row's super-block between its two lanes) and its
+ * header. Piece p holds the 32 weights of sub-block p; a matrix step wants weights
+ * 0-15 of one sub-block from lane (n, 0) and 16-31 from lane (n, 1), so the two
+ * lanes exchange one half each with v_permlane32_swap: afterwards both hold their
+ * halves of sub-blocks 2i and 2i + 1. The loads of the next super-block(s) are in
+ * flight during the arithmetic of the current one; nothing but the activations
+ * occupies LDS, so the number of resident wavefronts is bounded by registers (three
+ * or four per SIMD for TC = 8) and one launch holds all work items of a prefill
+ * chunk at once. */
+constexpr int XPD = 1; /* super-blocks the loads run ahead of the arithmetic */
+struct XRegs {
+  mv4i q[4];
+  mv4i hd;
 };
-__device__ __forceinline__ void xs_open(XStream &x, const WView &w, int col0, int lane) {
-  x.rs = __builtin_amdgcn_make_buffer_rsrc((void *)w.qs, 0, (int)((size_t)w.N * (w.K >> 1)), 0x00020000);
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    const int r = 8 * i + (lane >> 3);
-    const int n = min(col0 + r, (int)w.N - 1);
-    x.voff[i] = (uint32_t)n * (uint32_t)(w.K >> 1) + (uint32_t)(((lane & 7) ^ (lane >> 3)) * 16);
-  }
-  x.so = 0;
-  x.rh = __builtin_amdgcn_make_buffer_rsrc((void *)w.hdr, 0, (int)((size_t)w.N * (w.K >> 8) * 16), 0x00020000);
-  x.hoff = (uint32_t)min(col0 + (lane & 31), (int)w.N - 1) * (uint32_t)((w.K >> 8) * 16);
-  x.hso = 0;
-}
-__device__ __forceinline__ void xs_fetch(XStream &x, unsigned char *slot) {
-#pragma unroll
-  for (int i = 0; i < 4; ++i)
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(x.rs, (__attribute__((address_space(3))) void *)(slot + i * 1024),
-                                             16, (int)x.voff[i], (int)x.so, 0, 0);
-  __builtin_amdgcn_raw_ptr_buffer_load_lds(x.rh, (__attribute__((address_space(3))) void *)(slot + 4096), 16,
-                                           (int)x.hoff, (int)x.hso, 0, 0);
-}
-__device__ __forceinline__ void xs_advance(XStream &x) {
-  x.so += 128;
-  x.hso += 16;
-}
-constexpr int XS_OPS = 5; /* loads one xs_fetch issues */
 
-/* One super-block: acc / accm += for the NREG accumulator registers of this lane
- * (register r is token 8 * (r / 4) + 4g + r % 4, the lane's column n). `slot` holds
- * the nibbles and headers (its copies have landed). One matrix step per sub-block
- * j: lane (n, g) supplies weights 16g .. 16g+15 of it, so a step's 32 x 32 sums
- * belong to one sub-block and take its 6-bit scale as an integer multiply-add. */
-typedef int mv2i __attribute__((ext_vector_type(2)));
 template <int TC, int NREG>
-__device__ __forceinline__ void xw_super_block(const unsigned char *slot, const XLds &l, int K, int sb,
-                                               int i32, int g, float (&acc)[NREG], float (&accm)[NREG]) {
+__device__ __forceinline__ void xr_super_block(const XRegs &W, const XLds &l, int K, int sb, int i32, int g,
+                                               float (&acc)[NREG], float (&accm)[NREG]) {
   const mv16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
   const mv16f zero16f = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
   const int nsb = K >> 8;
-  /* The LDS operands: this lane's 8 bytes of every sub-block (piece j of row i32,
-   * half g), the eight 16-byte row operands of its token, the token's split
-   * sub-block sums and the block scales of its NREG tokens. The compiler must not
-   * see these reads: it orders every LDS read it knows of after the direct-to-LDS
-   * copies it may alias, which would drain the ring. */
   const int row = i32 & (TC - 1);
+  const int8_t *pa = l.q + row * (K + 16) + sb * 256 + g * 16;
+  const mv8h amin = *(const mv8h *)(l.amin + (row * nsb + sb) * 32 + g * 16);
+  mv4i dv[NREG / 4];
+#pragma unroll
+  for (int q4 = 0; q4 < NREG / 4; ++q4) dv[q4] = *(const mv4i *)(l.dA + sb * TC + 4 * g + q4 * 8);
   mv2i wq[8];
-  mv4i a8[8], aminv, hdv, dv[NREG / 4];
-  auto lds = [](const void *p) { return (uint32_t)(size_t)(const __attribute__((address_space(3))) void *)p; };
-  const uint32_t rowb = lds(slot) + i32 * 128 + g * 8;
-  const uint32_t x7 = i32 & 7;
-  const uint32_t pa = lds(l.q) + row * (K + 16) + sb * 256 + g * 16;
-  /* in two halves (sub-blocks 0-3, 4-7) to bound the registers in use */
-  auto read_half = [&](int h2) {
-    const uint32_t w0 = rowb + (((4 * h2 + 0) ^ x7) << 4), w1 = rowb + (((4 * h2 + 1) ^ x7) << 4);
-    const uint32_t w2 = rowb + (((4 * h2 + 2) ^ x7) << 4), w3 = rowb + (((4 * h2 + 3) ^ x7) << 4);
-    const uint32_t pah = pa + h2 * 128;
-    asm volatile("ds_read_b64 %0, %8\n\tds_read_b64 %1, %9\n\tds_read_b64 %2, %10\n\tds_read_b64 %3, %11\n\t"
-                 "ds_read_b128 %4, %12\n\tds_read_b128 %5, %12 offset:32\n\tds_read_b128 %6, %12 offset:64\n\t"
-                 "ds_read_b128 %7, %12 offset:96"
-                 : "=&v"(wq[4 * h2]), "=&v"(wq[4 * h2 + 1]), "=&v"(wq[4 * h2 + 2]), "=&v"(wq[4 * h2 + 3]),
-                   "=&v"(a8[4 * h2]), "=&v"(a8[4 * h2 + 1]), "=&v"(a8[4 * h2 + 2]), "=&v"(a8[4 * h2 + 3])
-                 : "v"(w0), "v"(w1), "v"(w2), "v"(w3), "v"(pah)
-                 : "memory");
-  };
-  /* every register is named at the wait so that nothing reads one before it */
-  auto wait_half = [&](int h2) {
-    asm volatile("s_waitcnt lgkmcnt(0)"
-                 : "+v"(wq[4 * h2]), "+v"(wq[4 * h2 + 1]), "+v"(wq[4 * h2 + 2]), "+v"(wq[4 * h2 + 3]),
-                   "+v"(a8[4 * h2]), "+v"(a8[4 * h2 + 1]), "+v"(a8[4 * h2 + 2]), "+v"(a8[4 * h2 + 3])
-                 :
-                 : "memory");
-  };
-  {
-    const uint32_t pm = lds(l.amin) + (row * nsb + sb) * 32 + g * 16;
-    const uint32_t pd = lds(l.dA) + (sb * TC + 4 * g) * 4;
-    asm volatile("ds_read_b128 %0, %1 offset:4096" : "=&v"(hdv) : "v"(lds(slot) + (i32 + 32 * g) * 16) : "memory");
-    read_half(0);
-    asm volatile("ds_read_b128 %0, %1" : "=&v"(aminv) : "v"(pm) : "memory");
 #pragma unroll
-    for (int q4 = 0; q4 < NREG / 4; ++q4)
-      asm volatile("ds_read_b128 %0, %1" : "=&v"(dv[q4]) : "v"(pd + q4 * 32) : "memory");
-    read_half(1);
-    wait_half(0);
-    wait_half(1);
-    asm volatile("" : "+v"(aminv), "+v"(hdv));
-#pragma unroll
-    for (int q4 = 0; q4 < NREG / 4; ++q4) asm volatile("" : "+v"(dv[q4]));
+  for (int i = 0; i < 4; ++i) {
+    const auto r0 = __builtin_amdgcn_permlane32_swap((unsigned)W.q[i][0], (unsigned)W.q[i][2], false, false);
+    const auto r1 = __builtin_amdgcn_permlane32_swap((unsigned)W.q[i][1], (unsigned)W.q[i][3], false, false);
+    wq[2 * i] = mv2i{(int)r0[0], (int)r1[0]};
+    wq[2 * i + 1] = mv2i{(int)r0[1], (int)r1[1]};
   }
-  const uint4 hd = make_uint4((uint32_t)hdv[0], (uint32_t)hdv[1], (uint32_t)hdv[2], (uint32_t)hdv[3]);
-  /* 6-bit scales of sub-blocks 0-3 and 4-7, one per byte */
+  const uint4 hd = make_uint4((uint32_t)W.hd[0], (uint32_t)W.hd[1], (uint32_t)W.hd[2], (uint32_t)W.hd[3]);
   const uint32_t s03 = hd.y & 0x3f3f3f3fu;
   const uint32_t s47 = (hd.w & 0x0f0f0f0fu) | ((hd.y >> 2) & 0x30303030u);
-  const mv8h amin = __builtin_bit_cast(mv8h, aminv);
   int I[NREG];
 #pragma unroll
   for (int r = 0; r < NREG; ++r) I[r] = 0;
-#pragma unroll
-  for (int j = 0; j < 8; ++j) {
-    /* weight 2i / 2i+1 of the lane's 16 in the low / high nibble of byte i: the even
-     * ones become operand bytes 0-7, the odd ones bytes 8-15 (the activations'
-     * 16-value groups are stored in that order) */
+  mv16i D[2];
+  auto step = [&](int j) {
     const uint32_t x0 = (uint32_t)wq[j][0], x1 = (uint32_t)wq[j][1];
     const mv4i b = {(int)(x0 & HIPQ_M4), (int)(x1 & HIPQ_M4), (int)((x0 >> 4) & HIPQ_M4),
                     (int)((x1 >> 4) & HIPQ_M4)};
-    const mv16i D = __builtin_amdgcn_mfma_i32_32x32x32_i8(a8[j], b, zero16, 0, 0, 0);
+    const mv4i a8 = *(const mv4i *)(pa + j * 32);
+    D[j & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a8, b, zero16, 0, 0, 0);
+  };
+  auto scale = [&](int j) {
     const int scj = (int)(((j < 4 ? s03 : s47) >> (8 * (j & 3))) & 0xff);
 #pragma unroll
-    for (int r = 0; r < NREG; ++r) I[r] = __mul24(D[r], scj) + I[r];
+    for (int r = 0; r < NREG; ++r) I[r] = __mul24(D[j & 1][r], scj) + I[r];
+  };
+  step(0);
+#pragma unroll
+  for (int j = 1; j < 8; ++j) {
+    step(j);
+    __builtin_amdgcn_sched_barrier(0);
+    scale(j - 1);
   }
-  /* mins: sum_j m_j * bsum_j, the low parts of bsum in lanes 0-31, the high parts in 32-63 */
+  __builtin_amdgcn_sched_barrier(0);
+  scale(7);
   const uint32_t mlo = hd.z & 0x3f3f3f3fu;
   const uint32_t mhi = ((hd.w >> 4) & 0x0f0f0f0fu) | ((hd.z >> 2) & 0x30303030u);
   mv8h bmin;
@@ -662,164 +617,164 @@ __device__ __forceinline__ void xw_super_block(const unsigned char *slot, const 
   }
 }
 
-/* A run of column tiles (matrix, first column) for one wavefront: the weights of
- * the next XD - 1 super-blocks, also across tiles, are in flight while one is
- * computed. tile_of(t, &view, &col0) names tile t; done(t, out) receives its NREG
- * results. Loads retire in issue order, so waiting until at most the loads of the
- * younger fetches are outstanding means the oldest fetch has landed. */
-template <int TC, int NREG, int XD, typename TileOf, typename Done>
-__device__ __forceinline__ void xw_run(int ntile, const XLds &l, int K, TileOf tile_of, Done done) {
+/* A run of column tiles for one wavefront, the loads PD super-blocks ahead of the
+ * arithmetic, also across tiles. tile_of(t, &view, &col0) names tile t; done(t, out)
+ * receives its NREG results. */
+template <int TC, int NREG, int PD, typename TileOf, typename Done, typename Pre>
+__device__ __forceinline__ void xr_run(int ntile, const XLds &l, int K, TileOf tile_of, Done done, Pre pre) {
+  constexpr int NB = PD + 1;
   const int lane = threadIdx.x & 63, i32 = lane & 31, g = lane >> 5;
   const int nsb = K >> 8;
   const int nv = ntile * nsb;
-  XStream xs;
-  int lt = 0, lsb = 0; /* tile and super-block under the cursor */
-  int issued = 0;      /* fetches issued so far */
-  {
-    WView lw;
+  const uint8_t *qrow, *hrow;
+  int lt = 0, lsb = 0, issued = 0;
+  auto open = [&](int t) {
+    WView w;
     int c0;
-    tile_of(0, lw, c0);
-    xs_open(xs, lw, c0, lane);
-  }
-  /* Always issues its five loads, so that the number of loads in flight at any
-   * point of the loop is fixed; past the end of the stream it fetches the last
-   * super-block again, into a slot nobody reads any more. */
-  auto fetch = [&](unsigned char *slot) {
-    xs_fetch(xs, slot);
+    tile_of(t, w, c0);
+    const int n = min(c0 + i32, (int)w.N - 1);
+    qrow = w.qs + (size_t)n * (size_t)(K >> 1) + g * 16;
+    hrow = w.hdr + (size_t)n * (size_t)(nsb * 16);
+  };
+  open(0);
+  auto load = [&](XRegs &r) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) r.q[i] = hipq_ld_global((const mv4i *)(qrow + lsb * 128 + i * 32));
+    r.hd = hipq_ld_global((const mv4i *)(hrow + lsb * 16));
     if (++issued >= nv) return; /* uniform: the cursor stays on the last super-block */
     if (++lsb == nsb) {
       lsb = 0;
-      ++lt;
-      WView lw;
-      int c0;
-      tile_of(lt, lw, c0);
-      xs_open(xs, lw, c0, lane);
-    } else {
-      xs_advance(xs);
+      open(++lt);
     }
   };
-  /* ring slots by fetch number modulo XD; the loop keeps XD - 1 fetches ahead */
-  int fslot = 0; /* slot of the next fetch */
-  auto fetch_next = [&]() {
-    fetch(l.ring + fslot * XTILE);
-    fslot = fslot + 1 == XD ? 0 : fslot + 1;
-  };
+  /* Every step issues its loads, past the end of the stream those of the last
+   * super-block again: a fixed number of loads is then in flight at each wait. */
+  XRegs buf[NB];
 #pragma unroll
-  for (int i = 0; i < XD - 1; ++i) fetch_next();
-  int cslot = 0; /* slot of the super-block computed next */
+  for (int p = 0; p < PD; ++p) load(buf[p]);
+  pre(); /* the activations are staged while the first weights are on their way */
   int t = 0, sb = 0;
   float acc[NREG], accm[NREG];
-  for (int v = 0; v < nv; ++v) {
-    if (sb == 0) {
+  for (int v0 = 0; v0 < nv; v0 += NB) {
 #pragma unroll
-      for (int r = 0; r < NREG; ++r) acc[r] = accm[r] = 0.f;
-    }
-    fetch_next(); /* into the slot consumed by the previous step */
-    /* the fetch of this step has landed once only the XD - 1 later ones are outstanding */
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((XD - 1) * XS_OPS) : "memory");
-    xw_super_block<TC, NREG>(l.ring + cslot * XTILE, l, K, sb, i32, g, acc, accm);
-    cslot = cslot + 1 == XD ? 0 : cslot + 1;
-    if (++sb == nsb) {
-      float out[NREG];
+    for (int u = 0; u < NB; ++u) {
+      const int v = v0 + u;
+      if (v < nv) {
+        load(buf[(u + PD) % NB]);
+        if (sb == 0) {
 #pragma unroll
-      for (int r = 0; r < NREG; ++r) out[r] = acc[r] - accm[r];
-      done(t, out);
-      sb = 0;
-      ++t;
+          for (int r = 0; r < NREG; ++r) acc[r] = accm[r] = 0.f;
+        }
+        xr_super_block<TC, NREG>(buf[u], l, K, sb, i32, g, acc, accm);
+        if (++sb == nsb) {
+          float out[NREG];
+#pragma unroll
+          for (int r = 0; r < NREG; ++r) out[r] = acc[r] - accm[r];
+          done(t, out);
+          sb = 0;
+          ++t;
+        }
+      }
     }
   }
-  asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); /* no copy may land after the ring is given up */
 }
 
-/* h[slot][col] = silu(x_tok . Wgate[e][col]) * (x_tok . Wup[e][col]): a workgroup
- * serves one expert and 128 columns (32 per wavefront, the gate tile then the up
- * tile), the expert's tokens in chunks of TC. */
-template <int TC, int WV, int XD>
-__global__ __launch_bounds__(64 * WV, TC <= 8 && XD == 2 ? 3 : 1) void gate_up_mma_kernel(const WView *__restrict__ views, int E_,
-                                                          QView xq, const int *__restrict__ offsets,
-                                                          const int *__restrict__ slot_pair, int topk,
-                                                          int I, float *__restrict__ h) {
+template <int TC>
+__global__ __launch_bounds__(256, TC <= 8 ? 3 : TC <= 16 ? 2 : 1) void gate_up_mma_kernel(
+  const WView *__restrict__ views, int E_, QView xq, const int *__restrict__ offsets,
+  const int *__restrict__ items, const int *__restrict__ slot_pair, int topk, int I, float *__restrict__ h) {
   constexpr int NREG = TC / 2;
   extern __shared__ __attribute__((aligned(16))) unsigned char xmoe_lds[];
-  const int e = blockIdx.y;
-  const int begin = offsets[e], end = offsets[e + 1];
-  if (begin == end) return; /* uniform per workgroup */
+  const int item = blockIdx.y;
+  if (item >= items[0]) return; /* uniform per workgroup */
+  const int e = items[2 + 2 * item], s0 = items[3 + 2 * item];
+  const int end = min(s0 + TC, offsets[e + 1]);
   const WView wg = views[e], wu = views[E_ + e];
   const int K = wg.K;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const XLds l = xlds_carve(xmoe_lds, TC, K, wave, XD);
-  const int col0 = (blockIdx.x * WV + wave) * 32;
-  for (int s0 = begin; s0 < end; s0 += TC) {
-    __syncthreads(); /* the previous chunk is no longer read */
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
+  const XLds l = xlds_carve(xmoe_lds, TC, K);
+  const int col0 = (blockIdx.x * 4 + wave) * 32;
+  const uint64_t dqs = (uint64_t)wu.qs - (uint64_t)wg.qs, dhdr = (uint64_t)wu.hdr - (uint64_t)wg.hdr;
+  auto stage = [&]() {
     if (threadIdx.x < TC) l.rows[threadIdx.x] = slot_pair[min(s0 + (int)threadIdx.x, end - 1)] / topk;
     __syncthreads();
     stage_rows<TC>(l, xq);
     __syncthreads();
-    if (col0 >= I) continue; /* uniform per wavefront; it still takes part in the barriers */
-    float gate[NREG];
-    xw_run<TC, NREG, XD>(
-      2, l, K,
-      [&](int t, WView &w, int &c0) {
-        w = t ? wu : wg;
-        c0 = col0;
-      },
-      [&](int t, const float(&out)[NREG]) {
-        if (t == 0) {
-#pragma unroll
-          for (int r = 0; r < NREG; ++r) gate[r] = out[r];
-        } else {
-          const int col = col0 + (lane & 31);
-#pragma unroll
-          for (int r = 0; r < NREG; ++r) {
-            const int tok = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-            if (col < I && s0 + tok < end) h[(size_t)(s0 + tok) * I + col] = silu_ref(gate[r]) * out[r];
-          }
-        }
-      });
+  };
+  if (col0 >= I) { /* uniform per wavefront; it still takes part in the barriers */
+    stage();
+    return;
   }
+  float gate[NREG];
+  xr_run<TC, NREG, XPD>(
+    2, l, K,
+    [&](int t, WView &w, int &c0) {
+      const uint64_t up = (uint64_t)0 - (uint64_t)(t & 1);
+      w.qs = (const uint8_t *)((uint64_t)wg.qs + (up & dqs));
+      w.hdr = (const uint8_t *)((uint64_t)wg.hdr + (up & dhdr));
+      w.N = wg.N;
+      w.K = wg.K;
+      c0 = col0;
+    },
+    [&](int t, const float(&out)[NREG]) {
+      if (t == 0) {
+#pragma unroll
+        for (int r = 0; r < NREG; ++r) gate[r] = out[r];
+      } else {
+        const int col = col0 + (lane & 31);
+#pragma unroll
+        for (int r = 0; r < NREG; ++r) {
+          const int tok = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+          if (col < I && s0 + tok < end) h[(size_t)(s0 + tok) * I + col] = silu_ref(gate[r]) * out[r];
+        }
+      }
+    },
+    stage);
 }
 
-/* contrib[slot][col] = (h_slot . Wdown[e][col]) * weight(pair): CT column tiles per wavefront */
-template <int TC, int CT, int XD>
-__global__ __launch_bounds__(256, TC <= 8 && XD == 2 ? 3 : 1) void down_mma_kernel(const WView *__restrict__ views, int E_, QView hq,
-                                                       const int *__restrict__ offsets,
-                                                       const int *__restrict__ slot_pair,
-                                                       const float *__restrict__ wgt, int H,
-                                                       float *__restrict__ contrib) {
+template <int TC, int CT>
+__global__ __launch_bounds__(256, TC <= 8 ? 4 : TC <= 16 ? 2 : 1) void down_mma_kernel(
+  const WView *__restrict__ views, int E_, QView hq, const int *__restrict__ offsets,
+  const int *__restrict__ items, const int *__restrict__ slot_pair, const float *__restrict__ wgt, int H,
+  float *__restrict__ contrib) {
   constexpr int NREG = TC / 2;
   extern __shared__ __attribute__((aligned(16))) unsigned char xmoe_lds[];
-  const int e = blockIdx.y;
-  const int begin = offsets[e], end = offsets[e + 1];
-  if (begin == end) return;
+  const int item = blockIdx.y;
+  if (item >= items[0]) return;
+  const int e = items[2 + 2 * item], s0 = items[3 + 2 * item];
+  const int end = min(s0 + TC, offsets[e + 1]);
   const WView wd = views[2 * E_ + e];
   const int K = wd.K;
-  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-  const XLds l = xlds_carve(xmoe_lds, TC, K, wave, XD);
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
+  const XLds l = xlds_carve(xmoe_lds, TC, K);
   const int col0 = (blockIdx.x * 4 + wave) * 32 * CT;
   const int ntile = min(CT, (H - col0 + 31) / 32);
-  for (int s0 = begin; s0 < end; s0 += TC) {
-    __syncthreads();
+  auto stage = [&]() {
     if (threadIdx.x < TC) l.rows[threadIdx.x] = min(s0 + (int)threadIdx.x, end - 1); /* hq rows are slots */
     __syncthreads();
     stage_rows<TC>(l, hq);
     __syncthreads();
-    if (ntile <= 0) continue;
-    xw_run<TC, NREG, XD>(
-      ntile, l, K,
-      [&](int t, WView &w, int &c0) {
-        w = wd;
-        c0 = col0 + 32 * t;
-      },
-      [&](int t, const float(&out)[NREG]) {
-        const int col = col0 + 32 * t + (lane & 31);
-#pragma unroll
-        for (int r = 0; r < NREG; ++r) {
-          const int tok = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-          if (col < H && s0 + tok < end)
-            contrib[(size_t)(s0 + tok) * H + col] = out[r] * wgt[slot_pair[s0 + tok]];
-        }
-      });
+  };
+  if (ntile <= 0) {
+    stage();
+    return;
   }
+  xr_run<TC, NREG, XPD>(
+    ntile, l, K,
+    [&](int t, WView &w, int &c0) {
+      w = wd;
+      c0 = col0 + 32 * t;
+    },
+    [&](int t, const float(&out)[NREG]) {
+      const int col = col0 + 32 * t + (lane & 31);
+#pragma unroll
+      for (int r = 0; r < NREG; ++r) {
+        const int tok = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        if (col < H && s0 + tok < end)
+          contrib[(size_t)(s0 + tok) * H + col] = out[r] * wgt[slot_pair[s0 + tok]];
+      }
+    },
+    stage);
 }
 
 /* y[t][c] = sum of the token's contributions, ascending expert id */
@@ -913,33 +868,6 @@ template <int DT> struct DownLauncher {
   template <int T, int KC, int G> void operator()() const { launch_down<DT, T, KC, G>(d, views, hq, b, s); }
 };
 
-template <int TC, int WV, int XD>
-int launch_gate_up_mma(const hipq_moe_desc &d, const MoeBufs &b, const WView *views, const QAct &xq,
-                       hipStream_t s) {
-  const size_t lds = xlds_bytes(TC, d.hidden, WV, XD);
-  if (lds > 64 * 1024) /* beyond the default limit of a launch */
-    HIPQ_HIP(hipFuncSetAttribute((const void *)gate_up_mma_kernel<TC, WV, XD>,
-                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-  hipLaunchKernelGGL((gate_up_mma_kernel<TC, WV, XD>), dim3((d.intermediate + 32 * WV - 1) / (32 * WV), d.experts),
-                     dim3(64 * WV), lds, s, views, d.experts, qview(xq), b.offsets, b.slot_pair, d.topk,
-                     d.intermediate, b.h);
-  HIPQ_HIP(hipGetLastError());
-  return HIPQ_OK;
-}
-template <int TC, int CT, int XD>
-int launch_down_mma(const hipq_moe_desc &d, const MoeBufs &b, const WView *views, const QAct &hq,
-                    hipStream_t s) {
-  const size_t lds = xlds_bytes(TC, d.intermediate, 4, XD);
-  if (lds > 64 * 1024)
-    HIPQ_HIP(hipFuncSetAttribute((const void *)down_mma_kernel<TC, CT, XD>,
-                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
-  hipLaunchKernelGGL((down_mma_kernel<TC, CT, XD>), dim3((d.hidden + 128 * CT - 1) / (128 * CT), d.experts),
-                     dim3(256), lds, s, views, d.experts, qview(hq), b.offsets, b.slot_pair, b.wgt, d.hidden,
-                     b.contrib);
-  HIPQ_HIP(hipGetLastError());
-  return HIPQ_OK;
-}
-
 constexpr size_t XLDS_MAX = 160 * 1024; /* LDS of a CU */
 
 template <int TC>
@@ -947,32 +875,41 @@ int launch_grouped_mma(const hipq::MoeArgs *a, const MoeBufs &b, const WView *vi
                        const QAct &hq, hipStream_t s) {
   const hipq_moe_desc &d = a->desc;
   const int64_t P = (int64_t)d.tokens * d.topk;
-  /* gate/up: four wavefronts with a ring of three super-blocks each where that fits;
-   * down: one column tile per wavefront and a ring of two (rows are short, more
-   * workgroups per CU pay more than a deeper ring) */
-  int rc = xlds_bytes(TC, d.hidden, 4, 3) <= XLDS_MAX ? launch_gate_up_mma<TC, 4, 3>(d, b, views, xq, s)
-                                                       : launch_gate_up_mma<TC, 4, 2>(d, b, views, xq, s);
+  constexpr int CT = 2; /* column tiles per wavefront of the down product: its rows are short */
+  const size_t lds_g = xlds_bytes(TC, d.hidden), lds_d = xlds_bytes(TC, d.intermediate);
+  if (lds_g > 64 * 1024) /* beyond the default limit of a launch */
+    HIPQ_HIP(hipFuncSetAttribute((const void *)gate_up_mma_kernel<TC>,
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_g));
+  /* an upper bound of the work items: one per active expert and one per full chunk */
+  const int max_items = (int)((P < d.experts ? P : d.experts) + P / TC);
+  hipLaunchKernelGGL((gate_up_mma_kernel<TC>), dim3((d.intermediate + 127) / 128, max_items), dim3(256), lds_g, s,
+                     views, d.experts, qview(xq), b.offsets, b.items, b.slot_pair, d.topk, d.intermediate, b.h);
+  HIPQ_HIP(hipGetLastError());
+  int rc = hipq::launch_quantize_q8_K_rowmma(b.h, P, d.intermediate, d.intermediate, &hq, s);
   if (rc) return rc;
-  rc = hipq::launch_quantize_q8_K_rowmma(b.h, P, d.intermediate, d.intermediate, &hq, s);
-  if (rc) return rc;
-  return launch_down_mma<TC, 1, 2>(d, b, views, hq, s);
+  if (lds_d > 64 * 1024)
+    HIPQ_HIP(hipFuncSetAttribute((const void *)down_mma_kernel<TC, CT>,
+                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_d));
+  hipLaunchKernelGGL((down_mma_kernel<TC, CT>), dim3((d.hidden + 128 * CT - 1) / (128 * CT), max_items), dim3(256),
+                     lds_d, s, views, d.experts, qview(hq), b.offsets, b.items, b.slot_pair, b.wgt, d.hidden,
+                     b.contrib);
+  HIPQ_HIP(hipGetLastError());
+  return HIPQ_OK;
 }
 
-/* Token chunk of the MFMA expert kernels for P pairs over E experts: the smallest
- * of 8, 16, 32 that holds twice the mean tokens per expert (larger groups loop),
- * reduced until the activation rows and the weight rings fit the LDS. */
+/* Token chunk of the matrix-core expert kernels for P pairs over E experts: the
+ * smallest of 8, 16, 32 that holds twice the mean tokens per expert (an expert with
+ * more becomes several work items), reduced until the activation rows fit the LDS. */
 int mma_chunk(const hipq_moe_desc &d, int64_t P, int E) {
   const int64_t mean2 = (2 * P + E - 1) / E;
   int tc = mean2 <= 8 ? 8 : mean2 <= 16 ? 16 : 32;
   const int kmax = d.hidden > d.intermediate ? d.hidden : d.intermediate;
-  while (tc > 8 && xlds_bytes(tc, kmax, 4, 2) > XLDS_MAX) tc >>= 1;
+  while (tc > 8 && xlds_bytes(tc, kmax) > XLDS_MAX) tc >>= 1;
   return tc;
 }
 bool use_mma(const hipq_moe_desc &d, int dt) {
   const int kmax = d.hidden > d.intermediate ? d.hidden : d.intermediate;
-  /* the copies address an expert's plane with 32-bit offsets */
-  const bool small = (uint64_t)d.hidden * (uint64_t)d.intermediate / 2 < (1ull << 32);
-  return dt == HIPQ_Q4_K && small && xlds_bytes(8, kmax, 4, 2) <= XLDS_MAX;
+  return dt == HIPQ_Q4_K && xlds_bytes(8, kmax) <= XLDS_MAX;
 }
 
 template <int DT>
@@ -1023,6 +960,8 @@ int launch_moe(const MoeArgs *a, void *workspace, size_t workspace_bytes, const 
     HIPQ_HIP(hipGetLastError());
     logits = b.logits;
   }
+  const bool mma = use_mma(d, dt);
+  const int chunk = mma ? mma_chunk(d, P, E) : 0; /* tokens of an expert per work item of the matrix-core kernels */
   int32_t *idx = a->topk_idx ? a->topk_idx : b.idx;
   float *wgt = a->topk_w ? a->topk_w : b.wgt;
   hipLaunchKernelGGL(route_kernel, dim3((T + 3) / 4), dim3(256), 0, s, logits, T, E, d.topk,
@@ -1031,11 +970,11 @@ int launch_moe(const MoeArgs *a, void *workspace, size_t workspace_bytes, const 
   b.wgt = wgt;
   if (P <= 16384 && E <= 1024) {
     hipLaunchKernelGGL(sort_pairs_kernel, dim3(1), dim3(1024), 0, s, idx, P, E, d.topk, b.offsets,
-                       b.slot_pair, b.tok_slots);
+                       b.slot_pair, b.tok_slots, chunk, b.items);
   } else {
     hipLaunchKernelGGL(fill_int_kernel, dim3((E + 255) / 256), dim3(256), 0, s, b.counts, E, 0);
     hipLaunchKernelGGL(count_kernel, dim3((P + 255) / 256), dim3(256), 0, s, idx, P, b.counts);
-    hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(64), 0, s, b.counts, E, b.offsets, b.cursor);
+    hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(64), 0, s, b.counts, E, b.offsets, b.cursor, chunk, b.items);
     hipLaunchKernelGGL(scatter_kernel, dim3((P + 255) / 256), dim3(256), 0, s, idx, P, d.topk, b.offsets,
                        b.cursor, b.slot_pair, b.tok_slots);
   }
@@ -1043,13 +982,12 @@ int launch_moe(const MoeArgs *a, void *workspace, size_t workspace_bytes, const 
 
   QAct xq = qact_carve(is_k, b.xq_mem, T, d.hidden);
   QAct hq = qact_carve(is_k, b.hq_mem, P, d.intermediate);
-  const bool mma = use_mma(d, dt);
   int rc = mma    ? launch_quantize_q8_K_rowmma(a->x, T, d.hidden, d.hidden, &xq, s)
            : is_k ? launch_quantize_q8_K(a->x, T, d.hidden, d.hidden, 0, &xq, nullptr, s)
                   : launch_quantize_q8_0(a->x, T, d.hidden, d.hidden, &xq, nullptr, s);
   if (rc) return rc;
   if (mma) {
-    const int tc = mma_chunk(d, P, E);
+    const int tc = chunk;
     rc = tc == 8    ? launch_grouped_mma<8>(a, b, views, xq, hq, s)
          : tc == 16 ? launch_grouped_mma<16>(a, b, views, xq, hq, s)
                     : launch_grouped_mma<32>(a, b, views, xq, hq, s);
