@@ -202,30 +202,37 @@ def main():
         return capi.Weight("q4_K", n, k, eb, mem=capi.MEM_DEVICE)
 
     # two sets of experts (2 x 340 MB) so that consecutive calls do not hit the last-level cache
-    sets = [([mk_expert(mi, mh) for _ in range(me)], [mk_expert(mi, mh) for _ in range(me)],
-             [mk_expert(mh, mi) for _ in range(me)]) for _ in range(2)]
+    sets = [capi.Experts([mk_expert(mi, mh) for _ in range(me)], [mk_expert(mi, mh) for _ in range(me)],
+                         [mk_expert(mh, mi) for _ in range(me)]) for _ in range(2)]
     mx = torch.randn((mt, mh), generator=gen, device="cuda")
     ml = torch.randn((mt, me), generator=gen, device="cuda")
     my = torch.empty((mt, mh), device="cuda")
     midx = torch.zeros((mt, mk), dtype=torch.int32, device="cuda")
-    for i in range(4):
-        g_, u_, d_ = sets[i % 2]
-        capi.moe_forward(mt, mh, mi, me, mk, g_, u_, d_, mx, my, router_logits=ml, topk_idx=midx, stream=stream)
-    torch.cuda.synchronize()
-    active = int(torch.unique(midx).numel())
-    ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    reps = 40
-    ev0.record()
-    for i in range(reps):
-        g_, u_, d_ = sets[i % 2]
-        capi.moe_forward(mt, mh, mi, me, mk, g_, u_, d_, mx, my, router_logits=ml, stream=stream)
-    ev1.record()
-    torch.cuda.synchronize()
-    moe_ms = ev0.elapsed_time(ev1) / reps
+
+    def moe_time(tokens, reps=40):
+        """Milliseconds per block of `tokens` tokens, and the number of experts they reach."""
+        x_, l_, y_, i_ = mx[:tokens], ml[:tokens], my[:tokens], midx[:tokens]
+        for i in range(4):
+            capi.moe_forward(tokens, mh, mi, me, mk, sets[i % 2], None, None, x_, y_, router_logits=l_,
+                             topk_idx=i_, stream=stream)
+        torch.cuda.synchronize()
+        n_active = int(torch.unique(i_).numel())
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record()
+        for i in range(reps):
+            capi.moe_forward(tokens, mh, mi, me, mk, sets[i % 2], None, None, x_, y_, router_logits=l_,
+                             stream=stream)
+        ev1.record()
+        torch.cuda.synchronize()
+        return ev0.elapsed_time(ev1) / reps, n_active
+
+    moe_ms, active = moe_time(mt)
+    moe_decode_ms, decode_active = moe_time(1)
     moe_bytes = active * 3 * (mi * mh * 144 // 256) + 2 * mt * mh * 4
     moe_gbs = moe_bytes / (moe_ms * 1e-3) / 1e9
+    moe_decode_bytes = decode_active * 3 * (mi * mh * 144 // 256) + 2 * mh * 4
     for st_ in sets:
-        for lst in st_:
+        for lst in st_.weights:
             for w_ in lst:
                 w_.destroy()
 
@@ -289,7 +296,9 @@ def main():
             "ms_per_block": round(moe_ms, 5), "active_experts": active,
             "roofline": {"bound": "hbm", "achieved": round(moe_gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(moe_gbs / HBM_PEAK_GBS, 5), "algorithmic_bytes_per_block": moe_bytes,
-                         "traffic": 233.2e6 + 117.1e6 + 7.9e6}},
+                         "traffic": 233.2e6 + 117.1e6 + 7.9e6},
+            "decode_token": {"ms_per_block": round(moe_decode_ms, 5), "active_experts": decode_active,
+                             "gbs": round(moe_decode_bytes / (moe_decode_ms * 1e-3) / 1e9, 2)}},
     }
     if not args.no_cpu:
         capi.matmul(weights[0], a, M, c, stream=stream)

@@ -158,12 +158,23 @@ def quantize_weights(dtype, w, n, k, out, mem=MEM_DEVICE, stream=None):
     check(lib().hipq_quantize_weights(DTYPES.get(dtype, dtype), _addr(w), n, k, _addr(out), mem, stream))
 
 
+class Experts:
+    """The handle arrays of a block's expert weights, built once: a decode step is a few
+    tens of microseconds, less than marshalling 3 x E handles per call would cost."""
+
+    def __init__(self, gate, up, down):
+        arr = lambda ws: (C.c_void_p * len(ws))(*[w.handle.value for w in ws])
+        self.weights = (list(gate), list(up), list(down))  # keeps the handles alive
+        self.gate, self.up, self.down = arr(gate), arr(up), arr(down)
+
+
 def moe_forward(tokens, hidden, inter, experts, topk, gate, up, down, x, y, router_logits=None,
                 router_weight=None, topk_idx=None, topk_w=None, renormalize=True, mem=MEM_DEVICE,
                 stream=None):
+    """gate / up / down: lists of E weights each, or gate = Experts(...) and up = down = None."""
     d = MoeDesc(tokens, hidden, inter, experts, topk, 1 if renormalize else 0)
-    arr = lambda ws: (C.c_void_p * experts)(*[w.handle.value for w in ws])
-    check(lib().hipq_moe_forward(C.byref(d), arr(gate), arr(up), arr(down), _addr(x),
+    ex = gate if isinstance(gate, Experts) else Experts(gate, up, down)
+    check(lib().hipq_moe_forward(C.byref(d), ex.gate, ex.up, ex.down, _addr(x),
                                  _addr(router_logits), _addr(router_weight), _addr(y),
                                  _addr(topk_idx), _addr(topk_w), mem, stream))
 

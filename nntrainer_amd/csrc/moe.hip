@@ -679,7 +679,13 @@ __device__ __forceinline__ void xr_run(int ntile, const XLds &l, int K, TileOf t
   }
 }
 
-template <int TC>
+/* h[slot][col] = silu(x_tok . Wgate[e][col]) * (x_tok . Wup[e][col]) for one work
+ * item. A wavefront forms the gate tile and then the up tile of its 32 columns
+ * (128 columns per workgroup). With few items (decode, short chunks) that leaves
+ * most of the chip idle, so the PAIRED form halves the stream per wavefront:
+ * wavefronts 0-1 form the gate tiles and 2-3 the up tiles of 64 columns, and the
+ * gate values cross through LDS. */
+template <int TC, bool PAIRED>
 __global__ __launch_bounds__(256, TC <= 8 ? 3 : TC <= 16 ? 2 : 1) void gate_up_mma_kernel(
   const WView *__restrict__ views, int E_, QView xq, const int *__restrict__ offsets,
   const int *__restrict__ items, const int *__restrict__ slot_pair, int topk, int I, float *__restrict__ h) {
@@ -693,7 +699,9 @@ __global__ __launch_bounds__(256, TC <= 8 ? 3 : TC <= 16 ? 2 : 1) void gate_up_m
   const int K = wg.K;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
   const XLds l = xlds_carve(xmoe_lds, TC, K);
-  const int col0 = (blockIdx.x * 4 + wave) * 32;
+  float *xch = (float *)(xmoe_lds + xlds_bytes(TC, K)); /* PAIRED: [2 tiles][NREG][64 lanes] */
+  const int col0 = PAIRED ? (blockIdx.x * 2 + (wave & 1)) * 32 : (blockIdx.x * 4 + wave) * 32;
+  const int first = PAIRED ? wave >> 1 : 0; /* 0: gate, 1: up */
   const uint64_t dqs = (uint64_t)wu.qs - (uint64_t)wg.qs, dhdr = (uint64_t)wu.hdr - (uint64_t)wg.hdr;
   auto stage = [&]() {
     if (threadIdx.x < TC) l.rows[threadIdx.x] = slot_pair[min(s0 + (int)threadIdx.x, end - 1)] / topk;
@@ -701,42 +709,61 @@ __global__ __launch_bounds__(256, TC <= 8 ? 3 : TC <= 16 ? 2 : 1) void gate_up_m
     stage_rows<TC>(l, xq);
     __syncthreads();
   };
+  float gate[NREG], up[NREG];
+  auto store = [&]() {
+    const int col = col0 + (lane & 31);
+#pragma unroll
+    for (int r = 0; r < NREG; ++r) {
+      const int tok = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+      if (col < I && s0 + tok < end) h[(size_t)(s0 + tok) * I + col] = silu_ref(gate[r]) * up[r];
+    }
+  };
   if (col0 >= I) { /* uniform per wavefront; it still takes part in the barriers */
     stage();
+    if (PAIRED) __syncthreads();
     return;
   }
-  float gate[NREG];
   xr_run<TC, NREG, XPD>(
-    2, l, K,
+    PAIRED ? 1 : 2, l, K,
     [&](int t, WView &w, int &c0) {
-      const uint64_t up = (uint64_t)0 - (uint64_t)(t & 1);
-      w.qs = (const uint8_t *)((uint64_t)wg.qs + (up & dqs));
-      w.hdr = (const uint8_t *)((uint64_t)wg.hdr + (up & dhdr));
+      const uint64_t isup = (uint64_t)0 - (uint64_t)((t + first) & 1);
+      w.qs = (const uint8_t *)((uint64_t)wg.qs + (isup & dqs));
+      w.hdr = (const uint8_t *)((uint64_t)wg.hdr + (isup & dhdr));
       w.N = wg.N;
       w.K = wg.K;
       c0 = col0;
     },
     [&](int t, const float(&out)[NREG]) {
-      if (t == 0) {
+      if (t + first == 0) {
 #pragma unroll
         for (int r = 0; r < NREG; ++r) gate[r] = out[r];
       } else {
-        const int col = col0 + (lane & 31);
 #pragma unroll
-        for (int r = 0; r < NREG; ++r) {
-          const int tok = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-          if (col < I && s0 + tok < end) h[(size_t)(s0 + tok) * I + col] = silu_ref(gate[r]) * out[r];
-        }
+        for (int r = 0; r < NREG; ++r) up[r] = out[r];
+        if (!PAIRED) store();
       }
     },
     stage);
+  if (PAIRED) {
+    float *mine = xch + (wave & 1) * (NREG * 64) + lane;
+    if (first == 0) {
+#pragma unroll
+      for (int r = 0; r < NREG; ++r) mine[r * 64] = gate[r];
+    }
+    __syncthreads();
+    if (first == 1) {
+#pragma unroll
+      for (int r = 0; r < NREG; ++r) gate[r] = mine[r * 64];
+      store();
+    }
+  }
 }
 
-template <int TC, int CT>
+template <int TC>
 __global__ __launch_bounds__(256, TC <= 8 ? 4 : TC <= 16 ? 2 : 1) void down_mma_kernel(
   const WView *__restrict__ views, int E_, QView hq, const int *__restrict__ offsets,
   const int *__restrict__ items, const int *__restrict__ slot_pair, const float *__restrict__ wgt, int H,
-  float *__restrict__ contrib) {
+  float *__restrict__ contrib, int ct) {
   constexpr int NREG = TC / 2;
   extern __shared__ __attribute__((aligned(16))) unsigned char xmoe_lds[];
   const int item = blockIdx.y;
@@ -747,8 +774,8 @@ __global__ __launch_bounds__(256, TC <= 8 ? 4 : TC <= 16 ? 2 : 1) void down_mma_
   const int K = wd.K;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
   const XLds l = xlds_carve(xmoe_lds, TC, K);
-  const int col0 = (blockIdx.x * 4 + wave) * 32 * CT;
-  const int ntile = min(CT, (H - col0 + 31) / 32);
+  const int col0 = (blockIdx.x * 4 + wave) * 32 * ct;
+  const int ntile = min(ct, (H - col0 + 31) / 32);
   auto stage = [&]() {
     if (threadIdx.x < TC) l.rows[threadIdx.x] = min(s0 + (int)threadIdx.x, end - 1); /* hq rows are slots */
     __syncthreads();
@@ -875,24 +902,35 @@ int launch_grouped_mma(const hipq::MoeArgs *a, const MoeBufs &b, const WView *vi
                        const QAct &hq, hipStream_t s) {
   const hipq_moe_desc &d = a->desc;
   const int64_t P = (int64_t)d.tokens * d.topk;
-  constexpr int CT = 2; /* column tiles per wavefront of the down product: its rows are short */
-  const size_t lds_g = xlds_bytes(TC, d.hidden), lds_d = xlds_bytes(TC, d.intermediate);
-  if (lds_g > 64 * 1024) /* beyond the default limit of a launch */
-    HIPQ_HIP(hipFuncSetAttribute((const void *)gate_up_mma_kernel<TC>,
-                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_g));
   /* an upper bound of the work items: one per active expert and one per full chunk */
   const int max_items = (int)((P < d.experts ? P : d.experts) + P / TC);
-  hipLaunchKernelGGL((gate_up_mma_kernel<TC>), dim3((d.intermediate + 127) / 128, max_items), dim3(256), lds_g, s,
-                     views, d.experts, qview(xq), b.offsets, b.items, b.slot_pair, d.topk, d.intermediate, b.h);
+  /* Few work items: halve the gate/up stream of a wavefront and give the down product
+   * one column tile per wavefront instead of two (its rows are short), so that more
+   * wavefronts share the weights' bytes. */
+  const bool few = (int64_t)max_items * ((d.intermediate + 127) / 128) * 4 <= 2048;
+  const size_t lds_g = xlds_bytes(TC, d.hidden) + (few ? TC * 256 : 0);
+  const size_t lds_d = xlds_bytes(TC, d.intermediate);
+  const void *kg = few ? (const void *)gate_up_mma_kernel<TC, true> : (const void *)gate_up_mma_kernel<TC, false>;
+  if (lds_g > 64 * 1024) /* beyond the default limit of a launch */
+    HIPQ_HIP(hipFuncSetAttribute(kg, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_g));
+  if (few)
+    hipLaunchKernelGGL((gate_up_mma_kernel<TC, true>), dim3((d.intermediate + 63) / 64, max_items), dim3(256), lds_g,
+                       s, views, d.experts, qview(xq), b.offsets, b.items, b.slot_pair, d.topk, d.intermediate,
+                       b.h);
+  else
+    hipLaunchKernelGGL((gate_up_mma_kernel<TC, false>), dim3((d.intermediate + 127) / 128, max_items), dim3(256),
+                       lds_g, s, views, d.experts, qview(xq), b.offsets, b.items, b.slot_pair, d.topk,
+                       d.intermediate, b.h);
   HIPQ_HIP(hipGetLastError());
   int rc = hipq::launch_quantize_q8_K_rowmma(b.h, P, d.intermediate, d.intermediate, &hq, s);
   if (rc) return rc;
   if (lds_d > 64 * 1024)
-    HIPQ_HIP(hipFuncSetAttribute((const void *)down_mma_kernel<TC, CT>,
-                                 hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_d));
-  hipLaunchKernelGGL((down_mma_kernel<TC, CT>), dim3((d.hidden + 128 * CT - 1) / (128 * CT), max_items), dim3(256),
+    HIPQ_HIP(hipFuncSetAttribute((const void *)down_mma_kernel<TC>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                 (int)lds_d));
+  const int ct = few ? 1 : 2;
+  hipLaunchKernelGGL((down_mma_kernel<TC>), dim3((d.hidden + 128 * ct - 1) / (128 * ct), max_items), dim3(256),
                      lds_d, s, views, d.experts, qview(hq), b.offsets, b.items, b.slot_pair, b.wgt, d.hidden,
-                     b.contrib);
+                     b.contrib, ct);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
 }
@@ -904,12 +942,12 @@ int mma_chunk(const hipq_moe_desc &d, int64_t P, int E) {
   const int64_t mean2 = (2 * P + E - 1) / E;
   int tc = mean2 <= 8 ? 8 : mean2 <= 16 ? 16 : 32;
   const int kmax = d.hidden > d.intermediate ? d.hidden : d.intermediate;
-  while (tc > 8 && xlds_bytes(tc, kmax) > XLDS_MAX) tc >>= 1;
+  while (tc > 8 && xlds_bytes(tc, kmax) + tc * 256 > XLDS_MAX) tc >>= 1; /* + the paired form's exchange area */
   return tc;
 }
 bool use_mma(const hipq_moe_desc &d, int dt) {
   const int kmax = d.hidden > d.intermediate ? d.hidden : d.intermediate;
-  return dt == HIPQ_Q4_K && xlds_bytes(8, kmax) <= XLDS_MAX;
+  return dt == HIPQ_Q4_K && xlds_bytes(8, kmax) + 8 * 256 <= XLDS_MAX;
 }
 
 template <int DT>
