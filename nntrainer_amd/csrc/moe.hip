@@ -102,14 +102,10 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const float *__restr
   }
 }
 
-/* One wavefront per token: softmax, top-k, optional renormalisation. */
-__global__ __launch_bounds__(256) void route_kernel(const float *__restrict__ logits, int T, int E,
-                                                    int topk, int renorm,
-                                                    int32_t *__restrict__ idx,
-                                                    float *__restrict__ wgt) {
+/* Routing of token t by one wavefront: softmax, top-k, optional renormalisation. */
+__device__ __forceinline__ void route_token(const float *__restrict__ logits, int t, int E, int topk,
+                                            int renorm, int32_t *idx, float *wgt) {
   const int lane = threadIdx.x & 63;
-  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
-  if (t >= T) return; /* uniform per wavefront */
   constexpr int MAXV = 16; /* E <= 1024 */
   float p[MAXV];
   const float *lg = logits + (size_t)t * E;
@@ -184,9 +180,17 @@ __global__ __launch_bounds__(256) void route_kernel(const float *__restrict__ lo
   }
 }
 
+__global__ __launch_bounds__(256) void route_kernel(const float *__restrict__ logits, int T, int E,
+                                                    int topk, int renorm, int32_t *__restrict__ idx,
+                                                    float *__restrict__ wgt) {
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= T) return; /* uniform per wavefront */
+  route_token(logits, t, E, topk, renorm, idx, wgt);
+}
+
 /* Where the slot of pair i goes in tok_slots: a token's slots in ascending expert
  * id, the order in which its contributions are added. */
-__device__ __forceinline__ int rank_in_token(const int32_t *__restrict__ idx, int i, int topk) {
+__device__ __forceinline__ int rank_in_token(const int32_t *idx, int i, int topk) {
   const int t = i / topk;
   const int e = idx[i];
   int r = 0;
@@ -194,15 +198,12 @@ __device__ __forceinline__ int rank_in_token(const int32_t *__restrict__ idx, in
   return t * topk + r;
 }
 
-/* Count, scan and scatter of the (token, k) pairs by expert in one workgroup:
- * the sort of a decode step or a short prefill chunk is a few thousand pairs, and
- * four tiny launches would cost more than the work. E <= 1024. */
-__global__ __launch_bounds__(1024) void sort_pairs_kernel(const int32_t *__restrict__ idx, int P,
-                                                          int E, int topk,
-                                                          int *__restrict__ offsets,
-                                                          int *__restrict__ slot_pair,
-                                                          int *__restrict__ tok_slots, int chunk,
-                                                          int *__restrict__ items) {
+/* Count, scan and scatter of the (token, k) pairs by expert in one workgroup of
+ * 1024 threads: the sort of a decode step or a short prefill chunk is a few thousand
+ * pairs, and four tiny launches would cost more than the work. E <= 1024. */
+__device__ __forceinline__ void sort_pairs(const int32_t *idx, int P, int E, int topk, int *__restrict__ offsets,
+                                           int *__restrict__ slot_pair, int *__restrict__ tok_slots, int chunk,
+                                           int *__restrict__ items) {
   __shared__ int cnt[1024];
   __shared__ int off[1024];
   __shared__ int nitems;
@@ -225,17 +226,28 @@ __global__ __launch_bounds__(1024) void sort_pairs_kernel(const int32_t *__restr
   const int excl = off[t] - own;
   if (t < E) offsets[t] = excl;
   if (t == E - 1) offsets[E] = off[t];
-  /* work items of the expert kernels: an expert's slots in chunks (any order) */
-  if (chunk > 0 && t < E && own > 0) {
-    const int nch = (own + chunk - 1) / chunk;
-    const int at = atomicAdd(&nitems, nch);
+  /* work items of the expert kernels: an expert's slots in chunks. A wavefront
+   * numbers its experts' chunks with a prefix sum and takes its range of the list
+   * with one atomic (the order of the wavefronts' ranges does not matter). */
+  if (chunk > 0) {
+    const int nch = t < E ? (own + chunk - 1) / chunk : 0;
+    int incl = nch;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+      const int v = __shfl_up(incl, d, 64);
+      if ((t & 63) >= d) incl += v;
+    }
+    int base = 0;
+    if ((t & 63) == 63 && incl > 0) base = atomicAdd(&nitems, incl);
+    base = __shfl(base, 63, 64);
+    const int at = base + incl - nch;
     for (int c = 0; c < nch; ++c) {
       items[2 + 2 * (at + c)] = t;
       items[3 + 2 * (at + c)] = excl + c * chunk;
     }
+    __syncthreads();
+    if (t == 0) items[0] = nitems;
   }
-  __syncthreads();
-  if (t == 0) items[0] = nitems;
   off[t] = excl;
   cnt[t] = 0;
   __syncthreads();
@@ -245,6 +257,26 @@ __global__ __launch_bounds__(1024) void sort_pairs_kernel(const int32_t *__restr
     slot_pair[slot] = i;
     tok_slots[rank_in_token(idx, i, topk)] = slot;
   }
+}
+
+__global__ __launch_bounds__(1024) void sort_pairs_kernel(const int32_t *__restrict__ idx, int P, int E, int topk,
+                                                          int *__restrict__ offsets, int *__restrict__ slot_pair,
+                                                          int *__restrict__ tok_slots, int chunk,
+                                                          int *__restrict__ items) {
+  sort_pairs(idx, P, E, topk, offsets, slot_pair, tok_slots, chunk, items);
+}
+
+/* Routing and sort of up to 16 tokens (a decode step) in one launch: a wavefront
+ * routes each token, then the workgroup sorts the pairs it has just written. */
+__global__ __launch_bounds__(1024) void route_sort_kernel(const float *__restrict__ logits, int T, int E, int topk,
+                                                          int renorm, int32_t *idx, float *wgt,
+                                                          int *__restrict__ offsets, int *__restrict__ slot_pair,
+                                                          int *__restrict__ tok_slots, int chunk,
+                                                          int *__restrict__ items) {
+  const int t = threadIdx.x >> 6;
+  if (t < T) route_token(logits, t, E, topk, renorm, idx, wgt);
+  __syncthreads(); /* orders the routing's stores before the sort's loads */
+  sort_pairs(idx, T * topk, E, topk, offsets, slot_pair, tok_slots, chunk, items);
 }
 
 __global__ void fill_int_kernel(int *p, int n, int v) {
@@ -1002,11 +1034,19 @@ int launch_moe(const MoeArgs *a, void *workspace, size_t workspace_bytes, const 
   const int chunk = mma ? mma_chunk(d, P, E) : 0; /* tokens of an expert per work item of the matrix-core kernels */
   int32_t *idx = a->topk_idx ? a->topk_idx : b.idx;
   float *wgt = a->topk_w ? a->topk_w : b.wgt;
-  hipLaunchKernelGGL(route_kernel, dim3((T + 3) / 4), dim3(256), 0, s, logits, T, E, d.topk,
-                     d.renormalize, idx, wgt);
-  HIPQ_HIP(hipGetLastError());
   b.wgt = wgt;
-  if (P <= 16384 && E <= 1024) {
+  if (T <= 16 && E <= 1024) {
+    hipLaunchKernelGGL(route_sort_kernel, dim3(1), dim3(1024), 0, s, logits, T, E, d.topk, d.renormalize, idx,
+                       wgt, b.offsets, b.slot_pair, b.tok_slots, chunk, b.items);
+    HIPQ_HIP(hipGetLastError());
+  } else {
+    hipLaunchKernelGGL(route_kernel, dim3((T + 3) / 4), dim3(256), 0, s, logits, T, E, d.topk, d.renormalize,
+                       idx, wgt);
+    HIPQ_HIP(hipGetLastError());
+  }
+  if (T <= 16 && E <= 1024) {
+    /* routed and sorted above */
+  } else if (P <= 16384 && E <= 1024) {
     hipLaunchKernelGGL(sort_pairs_kernel, dim3(1), dim3(1024), 0, s, idx, P, E, d.topk, b.offsets,
                        b.slot_pair, b.tok_slots, chunk, b.items);
   } else {
