@@ -17,13 +17,14 @@ def _experts(cr, e, i, h, seed):
     return gate, up, down
 
 
-# the later shapes reach the kernels' other paths: 16- and 32-token chunks with
-# experts that hold more tokens than a chunk (48 tokens x 4 of 4 experts), rows long
-# enough that the weight ring drops to two super-blocks (hidden 3072 at 32 tokens),
-# and rows beyond what the matrix-core kernels stage in LDS (hidden 8192)
+# the later shapes reach the kernels' other paths: 16- and 32-token work items with
+# experts that hold more tokens than one item (48 tokens x 4 of 4 experts), long rows
+# (hidden 3072 at 32 tokens), rows beyond what the matrix-core kernels stage in LDS
+# (hidden 8192), and a block with enough work items for the plain (unpaired) gate/up
+# form (64 tokens over 128 experts, 768 columns)
 @pytest.mark.parametrize("t,h,i,e,k", [(8, 256, 256, 8, 2), (64, 512, 256, 16, 4), (5, 2048, 768, 8, 8),
                                        (40, 512, 256, 8, 2), (48, 256, 512, 4, 4), (72, 3072, 256, 4, 2),
-                                       (3, 8192, 256, 4, 2)])
+                                       (3, 8192, 256, 4, 2), (64, 256, 768, 128, 8)])
 def test_moe_matches_oracle(hipq, cr, t, h, i, e, k):
     import gpu_util as gu
     import torch
@@ -53,6 +54,34 @@ def test_moe_matches_oracle(hipq, cr, t, h, i, e, k):
     capi.moe_forward(t, h, i, e, k, wg, wu, wd, dx, y2, router_logits=dl, stream=gu.stream())
     torch.cuda.synchronize()
     assert torch.equal(y, y2)
+    for w in wg + wu + wd:
+        w.destroy()
+
+
+@pytest.mark.parametrize("t,h,i,e,k", [(64, 512, 256, 32, 2), (64, 256, 256, 16, 2), (96, 256, 256, 8, 2)])
+def test_moe_skewed_routing(hipq, cr, t, h, i, e, k):
+    """Every token chooses expert 0: it holds far more slots than a work item (8, 16 or
+    32 of them), so several workgroups serve it side by side."""
+    import gpu_util as gu
+    import torch
+    gate, up, down = _experts(cr, e, i, h, seed=5000)
+    x = synth.normal(5100, (t, h))
+    logits = synth.normal(5101, (t, e))
+    logits[:, 0] += 8.0
+    ref_y, ref_idx, ref_w = cr.moe_forward(x, logits, gate, up, down, k)
+    assert (ref_idx == 0).any(axis=1).all()
+    wg = [capi.Weight("q4_K", i, h, b) for b in gate]
+    wu = [capi.Weight("q4_K", i, h, b) for b in up]
+    wd = [capi.Weight("q4_K", h, i, b) for b in down]
+    y = torch.full((t, h), float("nan"), device="cuda")
+    idx = torch.zeros((t, k), dtype=torch.int32, device="cuda")
+    capi.moe_forward(t, h, i, e, k, wg, wu, wd, gu.dev(x), y, router_logits=gu.dev(logits), topk_idx=idx,
+                     stream=gu.stream())
+    torch.cuda.synchronize()
+    assert np.array_equal(idx.cpu().numpy(), ref_idx)
+    got = y.cpu().numpy()
+    assert not np.isnan(got).any()
+    assert gu.rel_err(got, ref_y) <= 2e-6, gu.rel_err(got, ref_y)
     for w in wg + wu + wd:
         w.destroy()
 
