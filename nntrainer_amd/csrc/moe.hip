@@ -604,28 +604,22 @@ __device__ __forceinline__ void xr_super_block(const XRegs &W, const XLds &l, in
   int I[NREG];
 #pragma unroll
   for (int r = 0; r < NREG; ++r) I[r] = 0;
-  mv16i D[2];
-  auto step = [&](int j) {
+#pragma unroll
+  for (int j = 0; j < 8; ++j) {
+    /* weight 2i / 2i+1 of the lane's 16 in the low / high nibble of byte i: the even
+     * ones become operand bytes 0-7, the odd ones bytes 8-15 (the activations'
+     * 16-value groups are stored in that order) */
     const uint32_t x0 = (uint32_t)wq[j][0], x1 = (uint32_t)wq[j][1];
     const mv4i b = {(int)(x0 & HIPQ_M4), (int)(x1 & HIPQ_M4), (int)((x0 >> 4) & HIPQ_M4),
                     (int)((x1 >> 4) & HIPQ_M4)};
     const mv4i a8 = *(const mv4i *)(pa + j * 32);
-    D[j & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a8, b, zero16, 0, 0, 0);
-  };
-  auto scale = [&](int j) {
+    /* one result register for all steps: four wavefronts per SIMD hide the matrix
+     * core's latency better than a second register (and a third wavefront) did */
+    const mv16i D = __builtin_amdgcn_mfma_i32_32x32x32_i8(a8, b, zero16, 0, 0, 0);
     const int scj = (int)(((j < 4 ? s03 : s47) >> (8 * (j & 3))) & 0xff);
 #pragma unroll
-    for (int r = 0; r < NREG; ++r) I[r] = __mul24(D[j & 1][r], scj) + I[r];
-  };
-  step(0);
-#pragma unroll
-  for (int j = 1; j < 8; ++j) {
-    step(j);
-    __builtin_amdgcn_sched_barrier(0);
-    scale(j - 1);
+    for (int r = 0; r < NREG; ++r) I[r] = __mul24(D[r], scj) + I[r];
   }
-  __builtin_amdgcn_sched_barrier(0);
-  scale(7);
   const uint32_t mlo = hd.z & 0x3f3f3f3fu;
   const uint32_t mhi = ((hd.w >> 4) & 0x0f0f0f0fu) | ((hd.z >> 2) & 0x30303030u);
   mv8h bmin;
@@ -718,7 +712,7 @@ __device__ __forceinline__ void xr_run(int ntile, const XLds &l, int K, TileOf t
  * wavefronts 0-1 form the gate tiles and 2-3 the up tiles of 64 columns, and the
  * gate values cross through LDS. */
 template <int TC, bool PAIRED>
-__global__ __launch_bounds__(256, TC <= 8 ? 3 : TC <= 16 ? 2 : 1) void gate_up_mma_kernel(
+__global__ __launch_bounds__(256, TC <= 8 ? 4 : TC <= 16 ? 2 : 1) void gate_up_mma_kernel(
   const WView *__restrict__ views, int E_, QView xq, const int *__restrict__ offsets,
   const int *__restrict__ items, const int *__restrict__ slot_pair, int topk, int I, float *__restrict__ h) {
   constexpr int NREG = TC / 2;
@@ -772,10 +766,12 @@ __global__ __launch_bounds__(256, TC <= 8 ? 3 : TC <= 16 ? 2 : 1) void gate_up_m
       } else {
 #pragma unroll
         for (int r = 0; r < NREG; ++r) up[r] = out[r];
-        if (!PAIRED) store();
       }
     },
     stage);
+  /* the SwiGLU (a double-precision exponential) comes after the stream, when no
+   * weights are held in registers any more */
+  if (!PAIRED) store();
   if (PAIRED) {
     float *mine = xch + (wave & 1) * (NREG * 64) + lane;
     if (first == 0) {
