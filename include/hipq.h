@@ -143,7 +143,12 @@ typedef struct hipq_moe_desc {
  *  [T x E] (logits already computed) and `router_weight` [H x E] fp32 (the
  *  layer's "gate" weight; logits = x . router_weight) must be non-NULL.
  *  y [T x H]. topk_idx [T x topk] int32 and topk_w [T x topk] fp32 are optional
- *  outputs of the routing. */
+ *  outputs of the routing.
+ *  The first call with a set of Q4_K experts re-stores them on the device in the
+ *  order the expert kernels read (a one-time pass, synchronous); from then on
+ *  these handles serve hipq_moe_forward only and hipq_matmul refuses them. In
+ *  the reference an expert's weight tensors belong to its MoE layer alone
+ *  (qwen_moe_layer.cpp:50-159). */
 HIPQ_API int hipq_moe_forward(const hipq_moe_desc *desc, const hipq_weight_t *gate,
                               const hipq_weight_t *up, const hipq_weight_t *down,
                               const float *x, const float *router_logits,

@@ -154,6 +154,9 @@ int multiply(const hipq_weight *w, const QAct &qa, int64_t M, float *C, int64_t 
 int check_matmul_args(hipq_weight_t w, const float *A, int64_t M, int64_t lda, const float *C,
                       int64_t ldc) {
   if (!w || !A || !C) return fail(HIPQ_ERR_INVALID_ARGUMENT, "null weight, activation or output");
+  if (w->expert_tiles)
+    return fail(HIPQ_ERR_INVALID_ARGUMENT,
+                "the weight has been an expert of hipq_moe_forward and is stored for that use only");
   if (M < 0) return fail(HIPQ_ERR_INVALID_ARGUMENT, "M = %lld", (long long)M);
   if (lda < w->K) return fail(HIPQ_ERR_INVALID_ARGUMENT, "lda %lld < K %lld", (long long)lda, (long long)w->K);
   if (ldc < w->N) return fail(HIPQ_ERR_INVALID_ARGUMENT, "ldc %lld < N %lld", (long long)ldc, (long long)w->N);
@@ -280,6 +283,7 @@ int hipq_weight_create(int dtype, int layout, int64_t N, int64_t K, const void *
   if (!w) return fail(HIPQ_ERR_OUT_OF_MEMORY, "host allocation failed");
   w->dtype = dtype;
   w->device = g.device;
+  w->expert_tiles = 0;
   w->N = N;
   w->K = K;
   /* planes, each 256-byte aligned */
@@ -576,6 +580,10 @@ int hipq_moe_forward(const hipq_moe_desc *desc, const hipq_weight_t *gate, const
     for (int e = 0; e < d.experts; ++e) key.push_back(up[e]);
     for (int e = 0; e < d.experts; ++e) key.push_back(down[e]);
     if (t.key != key || !t.dev) {
+      /* experts that run on the matrix cores are stored by 32-row tiles from here on */
+      if (hipq::moe_wants_tiles(&d, dt))
+        for (const hipq_weight *w : key)
+          if (!w->expert_tiles && (rc = hipq::tile_expert_weight(const_cast<hipq_weight *>(w)))) return rc;
       std::vector<WView> host(key.size());
       for (size_t i = 0; i < key.size(); ++i) host[i] = wview(key[i]);
       if (t.dev) {

@@ -34,10 +34,19 @@
 /*                      = scales[(u>>1)*8 + g*2 + (u&1)]                      */
 /*         d  [N][K/256] fp16                                                 */
 /* The total size equals the packed ggml size; nothing is expanded in HBM.    */
+/*                                                                             */
+/* Q4_K expert weights of a mixture-of-experts block that runs on the matrix   */
+/* cores are re-laid out once more, by tiles of 32 rows (rows padded to 32):    */
+/*   qs  [N/32][K/256][4][64][16 B]: for load i of lane (n, g) the two 8-byte    */
+/*       halves g of sub-blocks 2i and 2i+1 of row n -- the 16 bytes the lane    */
+/*       feeds into two matrix steps, consecutive lanes consecutive in memory    */
+/*   hdr [N/32][K/256][32][16 B]                                                */
+/* Such a weight serves the expert kernels only.                               */
 /* ------------------------------------------------------------------------- */
 struct hipq_weight {
   int dtype;
   int device;
+  int expert_tiles; /* Q4_K only: re-laid out for the matrix-core expert kernels (see below) */
   int64_t N, K;
   uint8_t *base;   /* one allocation holding all planes */
   size_t bytes;
@@ -174,6 +183,7 @@ struct MoeArgs {
   float *topk_w;              /* device or null */
 };
 size_t moe_workspace_bytes(const hipq_moe_desc *d);
+bool moe_wants_tiles(const hipq_moe_desc *d, int dtype); /* the block's experts run on the matrix cores */
 int launch_moe(const MoeArgs *a, void *workspace, size_t workspace_bytes,
                const WView *dev_views /* [3*E] gate|up|down, device */,
                hipStream_t s);
@@ -183,6 +193,7 @@ int launch_quantize_weights(int dtype, const float *W, int64_t N, int64_t K,
                             void *out_blocks, hipStream_t s);
 
 /* relayout.hip ------------------------------------------------------------ */
+int tile_expert_weight(hipq_weight *w); /* planes -> 32-row tiles, in a new allocation; synchronous */
 int launch_relayout(hipq_weight *w, int layout, const uint8_t *src_dev,
                     hipStream_t s);
 

@@ -562,16 +562,15 @@ __device__ __forceinline__ void stage_rows(const XLds &l, const QView &a) {
   }
 }
 
-/* The weight stream. Lane (n, g) of a wavefront loads 16-byte piece 2i + g of weight row n for i = 0..3
- * (four 128-bit loads cover the row's super-block between its two lanes) and its
- * header. Piece p holds the 32 weights of sub-block p; a matrix step wants weights
- * 0-15 of one sub-block from lane (n, 0) and 16-31 from lane (n, 1), so the two
- * lanes exchange one half each with v_permlane32_swap: afterwards both hold their
- * halves of sub-blocks 2i and 2i + 1. The loads of the next super-block(s) are in
- * flight during the arithmetic of the current one; nothing but the activations
- * occupies LDS, so the number of resident wavefronts is bounded by registers (three
- * or four per SIMD for TC = 8) and one launch holds all work items of a prefill
- * chunk at once. */
+/* The weight stream. The experts' weights are stored by tiles of 32 rows: per tile
+ * and super-block four 1 KB groups, group i holding for lane (n, g) the halves g
+ * (weights 16g .. 16g+15) of sub-blocks 2i and 2i+1 of row n, then the 32 headers.
+ * A wavefront's 128-bit load i therefore reads 1 KB of consecutive memory (whole
+ * cache lines, marked non-temporal) and every lane receives exactly the bytes of its
+ * two matrix steps. The loads of the next super-block are in flight during the
+ * arithmetic of the current one, also across tiles; nothing but the activations
+ * occupies LDS, so the number of resident wavefronts is bounded by registers (four
+ * per SIMD for TC = 8) and one launch holds all work items of a prefill chunk. */
 constexpr int XPD = 1; /* super-blocks the loads run ahead of the arithmetic */
 struct XRegs {
   mv4i q[4];
@@ -593,10 +592,8 @@ __device__ __forceinline__ void xr_super_block(const XRegs &W, const XLds &l, in
   mv2i wq[8];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    const auto r0 = __builtin_amdgcn_permlane32_swap((unsigned)W.q[i][0], (unsigned)W.q[i][2], false, false);
-    const auto r1 = __builtin_amdgcn_permlane32_swap((unsigned)W.q[i][1], (unsigned)W.q[i][3], false, false);
-    wq[2 * i] = mv2i{(int)r0[0], (int)r1[0]};
-    wq[2 * i + 1] = mv2i{(int)r0[1], (int)r1[1]};
+    wq[2 * i] = mv2i{W.q[i][0], W.q[i][1]};
+    wq[2 * i + 1] = mv2i{W.q[i][2], W.q[i][3]};
   }
   const uint4 hd = make_uint4((uint32_t)W.hd[0], (uint32_t)W.hd[1], (uint32_t)W.hd[2], (uint32_t)W.hd[3]);
   const uint32_t s03 = hd.y & 0x3f3f3f3fu;
@@ -658,15 +655,16 @@ __device__ __forceinline__ void xr_run(int ntile, const XLds &l, int K, TileOf t
     WView w;
     int c0;
     tile_of(t, w, c0);
-    const int n = min(c0 + i32, (int)w.N - 1);
-    qrow = w.qs + (size_t)n * (size_t)(K >> 1) + g * 16;
-    hrow = w.hdr + (size_t)n * (size_t)(nsb * 16);
+    const int tile = c0 >> 5; /* c0 < N: rows past N are zero padding of the last tile */
+    qrow = w.qs + (size_t)tile * (size_t)(16 * K) + lane * 16;
+    hrow = w.hdr + (size_t)tile * (size_t)(nsb * 512) + i32 * 16;
   };
   open(0);
   auto load = [&](XRegs &r) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) r.q[i] = hipq_ld_global((const mv4i *)(qrow + lsb * 128 + i * 32));
-    r.hd = hipq_ld_global((const mv4i *)(hrow + lsb * 16));
+    for (int i = 0; i < 4; ++i)
+      r.q[i] = __builtin_bit_cast(mv4i, hipq_ld_stream((const uint4 *)(qrow + lsb * 4096 + i * 1024)));
+    r.hd = hipq_ld_global((const mv4i *)(hrow + lsb * 512));
     if (++issued >= nv) return; /* uniform: the cursor stays on the last super-block */
     if (++lsb == nsb) {
       lsb = 0;
@@ -999,6 +997,8 @@ int launch_grouped(const hipq::MoeArgs *a, const MoeBufs &b, const WView *views,
 } // namespace
 
 namespace hipq {
+
+bool moe_wants_tiles(const hipq_moe_desc *d, int dtype) { return use_mma(*d, dtype); }
 
 size_t moe_workspace_bytes(const hipq_moe_desc *d) {
   /* sized for the larger (Q8_K) activation form */

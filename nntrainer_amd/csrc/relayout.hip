@@ -121,9 +121,60 @@ __global__ void relayout_q6_K(const uint8_t *__restrict__ src, int64_t total,
   d[i] = (uint16_t)(blk[208] | (blk[209] << 8));
 }
 
+/* planes -> tiles of 32 rows for the expert kernels: thread = one 16-byte piece */
+__global__ void tile_q4_K(const uint8_t *__restrict__ qs, const uint8_t *__restrict__ hdr, int N, int nsb,
+                          int64_t pieces, uint8_t *__restrict__ tq, uint8_t *__restrict__ th) {
+  const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= pieces) return;
+  const int lane = (int)(p & 63), i = (int)((p >> 6) & 3);
+  const int64_t ts = p >> 8; /* tile * nsb + sb */
+  const int sb = (int)(ts % nsb);
+  const int64_t tile = ts / nsb;
+  const int64_t n = tile * 32 + (lane & 31);
+  const int g = lane >> 5;
+  uint2 a = make_uint2(0, 0), b = make_uint2(0, 0);
+  if (n < N) {
+    const uint8_t *src = qs + (n * nsb + sb) * 128 + g * 8;
+    a = *(const uint2 *)(src + (2 * i) * 16);
+    b = *(const uint2 *)(src + (2 * i + 1) * 16);
+  }
+  *(uint4 *)(tq + p * 16) = make_uint4(a.x, a.y, b.x, b.y);
+  if (i == 0 && g == 0)
+    *(uint4 *)(th + (ts * 32 + (lane & 31)) * 16) =
+      n < N ? *(const uint4 *)(hdr + (n * nsb + sb) * 16) : make_uint4(0, 0, 0, 0);
+}
+
 } // namespace
 
 namespace hipq {
+
+int tile_expert_weight(hipq_weight *w) {
+  if (w->dtype != HIPQ_Q4_K) return fail(HIPQ_ERR_INVALID_ARGUMENT, "only Q4_K weights have an expert layout");
+  if (w->expert_tiles) return HIPQ_OK;
+  const int nsb = (int)(w->K / 256);
+  const int64_t tiles = (w->N + 31) / 32;
+  const size_t q_bytes = (size_t)tiles * nsb * 4096, h_bytes = (size_t)tiles * nsb * 512;
+  const size_t o_hdr = (q_bytes + 255) & ~(size_t)255;
+  uint8_t *nb = nullptr;
+  hipError_t e = hipMalloc((void **)&nb, o_hdr + h_bytes);
+  if (e != hipSuccess) return fail(HIPQ_ERR_OUT_OF_MEMORY, "expert tiles of %zu bytes: %s", o_hdr + h_bytes, hipGetErrorString(e));
+  const int64_t pieces = tiles * nsb * 256;
+  hipLaunchKernelGGL(tile_q4_K, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, nullptr, w->qs, w->hdr,
+                     (int)w->N, nsb, pieces, nb, nb + o_hdr);
+  e = hipGetLastError();
+  if (e == hipSuccess) e = hipDeviceSynchronize(); /* nothing may still read the planes that are freed next */
+  if (e != hipSuccess) {
+    (void)hipFree(nb);
+    return fail(HIPQ_ERR_RUNTIME, "expert tiling: %s", hipGetErrorString(e));
+  }
+  (void)hipFree(w->base);
+  w->base = nb;
+  w->bytes = o_hdr + h_bytes;
+  w->qs = nb;
+  w->hdr = nb + o_hdr;
+  w->expert_tiles = 1;
+  return HIPQ_OK;
+}
 
 int launch_relayout(hipq_weight *w, int layout, const uint8_t *src, hipStream_t s) {
   const int x8 = layout == HIPQ_LAYOUT_X8;

@@ -86,6 +86,32 @@ def test_moe_skewed_routing(hipq, cr, t, h, i, e, k):
         w.destroy()
 
 
+def test_expert_weights_serve_the_moe_block_only(hipq, cr):
+    """Q4_K experts are re-stored for the expert kernels at the first block; a plain
+    matmul on such a handle is refused, the block keeps giving the same bits."""
+    import gpu_util as gu
+    import torch
+    t, h, i, e, k = 4, 256, 256, 4, 2
+    gate, up, down = _experts(cr, e, i, h, seed=7000)
+    wg = [capi.Weight("q4_K", i, h, b) for b in gate]
+    wu = [capi.Weight("q4_K", i, h, b) for b in up]
+    wd = [capi.Weight("q4_K", h, i, b) for b in down]
+    x = gu.dev(synth.normal(7100, (t, h)))
+    logits = gu.dev(synth.normal(7101, (t, e)))
+    a = gu.dev(synth.normal(7102, (1, h)))
+    c = torch.empty((1, i), device="cuda")
+    capi.matmul(wg[0], a, 1, c, stream=gu.stream())  # fine before the first block
+    y1, y2 = torch.empty((t, h), device="cuda"), torch.empty((t, h), device="cuda")
+    capi.moe_forward(t, h, i, e, k, wg, wu, wd, x, y1, router_logits=logits, stream=gu.stream())
+    with pytest.raises(capi.HipqError):
+        capi.matmul(wg[0], a, 1, c, stream=gu.stream())
+    capi.moe_forward(t, h, i, e, k, wg, wu, wd, x, y2, router_logits=logits, stream=gu.stream())
+    torch.cuda.synchronize()
+    assert torch.equal(y1, y2)
+    for w in wg + wu + wd:
+        w.destroy()
+
+
 def test_moe_router_weight_path(hipq, cr):
     """Logits computed on the device from the fp32 router weight."""
     import gpu_util as gu
