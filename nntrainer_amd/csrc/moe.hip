@@ -31,6 +31,7 @@
  * reference's bits for every single-row product.
  */
 #include "gemv_device.h"
+#include "quantize_device.h"
 
 namespace {
 
@@ -103,10 +104,10 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const float *__restr
 }
 
 /* Routing of token t by one wavefront: softmax, top-k, optional renormalisation. */
+template <int MAXV> /* logits per lane: E <= 64 * MAXV */
 __device__ __forceinline__ void route_token(const float *__restrict__ logits, int t, int E, int topk,
                                             int renorm, int32_t *idx, float *wgt) {
   const int lane = threadIdx.x & 63;
-  constexpr int MAXV = 16; /* E <= 1024 */
   float p[MAXV];
   const float *lg = logits + (size_t)t * E;
   float mx = -INFINITY;
@@ -180,12 +181,13 @@ __device__ __forceinline__ void route_token(const float *__restrict__ logits, in
   }
 }
 
+template <int MAXV>
 __global__ __launch_bounds__(256) void route_kernel(const float *__restrict__ logits, int T, int E,
                                                     int topk, int renorm, int32_t *__restrict__ idx,
                                                     float *__restrict__ wgt) {
   const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (t >= T) return; /* uniform per wavefront */
-  route_token(logits, t, E, topk, renorm, idx, wgt);
+  route_token<MAXV>(logits, t, E, topk, renorm, idx, wgt);
 }
 
 /* Where the slot of pair i goes in tok_slots: a token's slots in ascending expert
@@ -206,6 +208,7 @@ __device__ __forceinline__ void sort_pairs(const int32_t *idx, int P, int E, int
                                            int *__restrict__ items) {
   __shared__ int cnt[1024];
   __shared__ int off[1024];
+  __shared__ int wsum[16];
   __shared__ int nitems;
   const int t = threadIdx.x;
   cnt[t] = 0;
@@ -213,19 +216,23 @@ __device__ __forceinline__ void sort_pairs(const int32_t *idx, int P, int E, int
   __syncthreads();
   for (int i = t; i < P; i += 1024) atomicAdd(&cnt[idx[i]], 1);
   __syncthreads();
-  /* inclusive scan over the 1024 slots (Hillis-Steele), exclusive = inclusive - own */
+  /* exclusive scan over the 1024 slots: prefix sums inside each wavefront, then the
+   * sixteen wavefront totals */
   const int own = cnt[t];
-  off[t] = own;
-  __syncthreads();
-  for (int d = 1; d < 1024; d <<= 1) {
-    const int v = t >= d ? off[t - d] : 0;
-    __syncthreads();
-    off[t] += v;
-    __syncthreads();
+  int winc = own;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int v = __shfl_up(winc, d, 64);
+    if ((t & 63) >= d) winc += v;
   }
-  const int excl = off[t] - own;
+  if ((t & 63) == 63) wsum[t >> 6] = winc;
+  __syncthreads();
+  int wbase = 0;
+#pragma unroll
+  for (int w = 0; w < 16; ++w) wbase += w < (t >> 6) ? wsum[w] : 0;
+  const int excl = wbase + winc - own;
   if (t < E) offsets[t] = excl;
-  if (t == E - 1) offsets[E] = off[t];
+  if (t == E - 1) offsets[E] = excl + own;
   /* work items of the expert kernels: an expert's slots in chunks. A wavefront
    * numbers its experts' chunks with a prefix sum and takes its range of the list
    * with one atomic (the order of the wavefronts' ranges does not matter). */
@@ -268,13 +275,62 @@ __global__ __launch_bounds__(1024) void sort_pairs_kernel(const int32_t *__restr
 
 /* Routing and sort of up to 16 tokens (a decode step) in one launch: a wavefront
  * routes each token, then the workgroup sorts the pairs it has just written. */
+template <int MAXV>
 __global__ __launch_bounds__(1024) void route_sort_kernel(const float *__restrict__ logits, int T, int E, int topk,
                                                           int renorm, int32_t *idx, float *wgt,
                                                           int *__restrict__ offsets, int *__restrict__ slot_pair,
                                                           int *__restrict__ tok_slots, int chunk,
                                                           int *__restrict__ items) {
   const int t = threadIdx.x >> 6;
-  if (t < T) route_token(logits, t, E, topk, renorm, idx, wgt);
+  if (t < T) route_token<MAXV>(logits, t, E, topk, renorm, idx, wgt);
+  __syncthreads(); /* orders the routing's stores before the sort's loads */
+  sort_pairs(idx, T * topk, E, topk, offsets, slot_pair, tok_slots, chunk, items);
+}
+
+/* The rows of x quantized for the matrix-core expert kernels, in the same launch as
+ * the routing (neither needs the other): workgroups 0 .. route_blocks - 1 route (or
+ * route and sort, with 1024 threads), the others quantize one super-block per
+ * wavefront. */
+struct XQuant {
+  const float *x;
+  int64_t n_sb; /* T * H / 256 */
+  int nsb;
+  int8_t *q;
+  float *d;
+  uint16_t *amin;
+};
+__device__ __forceinline__ void quantize_x(const XQuant &xq, int T, int block) {
+  const int64_t sb = (int64_t)block * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (sb >= xq.n_sb) return; /* uniform per wavefront */
+  hipq_quantize_q8_K_wave<Q8K_ROWMMA>(xq.x, T, sb, xq.nsb, (int64_t)xq.nsb * 256, 0, xq.q, xq.d, nullptr, nullptr,
+                                      xq.amin, nullptr, nullptr);
+}
+
+template <int MAXV>
+__global__ __launch_bounds__(256) void route_quantize_kernel(const float *__restrict__ logits, int T, int E,
+                                                             int topk, int renorm, int32_t *__restrict__ idx,
+                                                             float *__restrict__ wgt, int route_blocks,
+                                                             XQuant xq) {
+  if ((int)blockIdx.x >= route_blocks) {
+    quantize_x(xq, T, blockIdx.x - route_blocks);
+    return;
+  }
+  const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (t >= T) return; /* uniform per wavefront */
+  route_token<MAXV>(logits, t, E, topk, renorm, idx, wgt);
+}
+
+template <int MAXV>
+__global__ __launch_bounds__(1024) void route_sort_quantize_kernel(
+  const float *__restrict__ logits, int T, int E, int topk, int renorm, int32_t *idx, float *wgt,
+  int *__restrict__ offsets, int *__restrict__ slot_pair, int *__restrict__ tok_slots, int chunk,
+  int *__restrict__ items, XQuant xq) {
+  if (blockIdx.x > 0) {
+    quantize_x(xq, T, blockIdx.x - 1);
+    return;
+  }
+  const int t = threadIdx.x >> 6;
+  if (t < T) route_token<MAXV>(logits, t, E, topk, renorm, idx, wgt);
   __syncthreads(); /* orders the routing's stores before the sort's loads */
   sort_pairs(idx, T * topk, E, topk, offsets, slot_pair, tok_slots, chunk, items);
 }
@@ -1031,13 +1087,41 @@ int launch_moe(const MoeArgs *a, void *workspace, size_t workspace_bytes, const 
   int32_t *idx = a->topk_idx ? a->topk_idx : b.idx;
   float *wgt = a->topk_w ? a->topk_w : b.wgt;
   b.wgt = wgt;
+  /* the router is instantiated for 2, 4 and 16 logits per lane (E <= 128, 256, 1024):
+   * a short kernel whose code is mostly fetched cold, so its length is its time.
+   * For the matrix-core expert kernels the same launch quantizes x. */
+  QAct xq = qact_carve(is_k, b.xq_mem, T, d.hidden);
+  QAct hq = qact_carve(is_k, b.hq_mem, P, d.intermediate);
+  const XQuant xqa = {a->x, (int64_t)T * (d.hidden / 256), d.hidden / 256, xq.q, xq.d, (uint16_t *)xq.bsum};
+  if (mma && (((uintptr_t)a->x & 15) != 0))
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "activation rows must be 16-byte aligned");
   if (T <= 16 && E <= 1024) {
-    hipLaunchKernelGGL(route_sort_kernel, dim3(1), dim3(1024), 0, s, logits, T, E, d.topk, d.renormalize, idx,
-                       wgt, b.offsets, b.slot_pair, b.tok_slots, chunk, b.items);
+    const unsigned qblocks = mma ? (unsigned)((xqa.n_sb + 15) / 16) : 0;
+    auto launch = [&](auto fused, auto plain) {
+      if (mma)
+        hipLaunchKernelGGL(fused, dim3(1 + qblocks), dim3(1024), 0, s, logits, T, E, d.topk, d.renormalize, idx,
+                           wgt, b.offsets, b.slot_pair, b.tok_slots, chunk, b.items, xqa);
+      else
+        hipLaunchKernelGGL(plain, dim3(1), dim3(1024), 0, s, logits, T, E, d.topk, d.renormalize, idx, wgt,
+                           b.offsets, b.slot_pair, b.tok_slots, chunk, b.items);
+    };
+    if (E <= 128) launch(route_sort_quantize_kernel<2>, route_sort_kernel<2>);
+    else if (E <= 256) launch(route_sort_quantize_kernel<4>, route_sort_kernel<4>);
+    else launch(route_sort_quantize_kernel<16>, route_sort_kernel<16>);
     HIPQ_HIP(hipGetLastError());
   } else {
-    hipLaunchKernelGGL(route_kernel, dim3((T + 3) / 4), dim3(256), 0, s, logits, T, E, d.topk, d.renormalize,
-                       idx, wgt);
+    const int rblocks = (T + 3) / 4;
+    const unsigned qblocks = mma ? (unsigned)((xqa.n_sb + 3) / 4) : 0;
+    auto launch = [&](auto fused, auto plain) {
+      if (mma)
+        hipLaunchKernelGGL(fused, dim3(rblocks + qblocks), dim3(256), 0, s, logits, T, E, d.topk, d.renormalize,
+                           idx, wgt, rblocks, xqa);
+      else
+        hipLaunchKernelGGL(plain, dim3(rblocks), dim3(256), 0, s, logits, T, E, d.topk, d.renormalize, idx, wgt);
+    };
+    if (E <= 128) launch(route_quantize_kernel<2>, route_kernel<2>);
+    else if (E <= 256) launch(route_quantize_kernel<4>, route_kernel<4>);
+    else launch(route_quantize_kernel<16>, route_kernel<16>);
     HIPQ_HIP(hipGetLastError());
   }
   if (T <= 16 && E <= 1024) {
@@ -1054,9 +1138,7 @@ int launch_moe(const MoeArgs *a, void *workspace, size_t workspace_bytes, const 
   }
   HIPQ_HIP(hipGetLastError());
 
-  QAct xq = qact_carve(is_k, b.xq_mem, T, d.hidden);
-  QAct hq = qact_carve(is_k, b.hq_mem, P, d.intermediate);
-  int rc = mma    ? launch_quantize_q8_K_rowmma(a->x, T, d.hidden, d.hidden, &xq, s)
+  int rc = mma    ? HIPQ_OK /* quantized with the routing */
            : is_k ? launch_quantize_q8_K(a->x, T, d.hidden, d.hidden, 0, &xq, nullptr, s)
                   : launch_quantize_q8_0(a->x, T, d.hidden, d.hidden, &xq, nullptr, s);
   if (rc) return rc;

@@ -1,0 +1,149 @@
+// SPDX-License-Identifier: Apache-2.0
+/**
+ * @file   quantize_device.h
+ * @brief  The Q8_K activation quantizer of one wavefront (one 256-value
+ *         super-block), shared by the quantizer kernels and by kernels that
+ *         quantize rows as part of another launch.
+ *
+ * Bit-exact with the reference CPU quantizers in an x86 AVX2 GCC build
+ * (IMPL = nntrainer/tensor/cpu_backend/ggml_interface/nntr_ggml_impl):
+ *   ROW  IMPL/nntr_ggml_impl_quant.cpp:1334-1374, where the compiler fuses
+ *        iscale*x + 1.5*2^23 into a single rounding
+ *   MAT  IMPL/nntr_ggml_impl.cpp:7504-7737 (product rounded to fp32, then to
+ *        the nearest-even integer; scale negative iff some x == +amax)
+ */
+#ifndef HIPQ_QUANTIZE_DEVICE_H
+#define HIPQ_QUANTIZE_DEVICE_H
+#include "hipq_internal.h"
+
+static constexpr float kRoundMagic = 12582912.f; /* 1.5 * 2^23 */
+
+__device__ __forceinline__ int magic_to_int(float biased) {
+  return (int)(__float_as_uint(biased) & 0x007fffffu) - 0x00400000;
+}
+
+__device__ __forceinline__ int pack4(int a, int b, int c, int d) {
+  return (a & 0xff) | ((b & 0xff) << 8) | ((c & 0xff) << 16) | ((d & 0xff) << 24);
+}
+
+/* output forms of the Q8_K quantizer */
+enum { Q8K_PLANES = 0, Q8K_CANONICAL = 1, Q8K_TILED = 2, Q8K_ROWMMA = 3 };
+
+/* Super-block sb = (row m, block b) of A by the calling wavefront (all 64 lanes).
+ * In the tiled mode rows M and beyond are padding and are written as zeros. Rows
+ * below mat_rows take the 4-row quantizer's semantics, the others the row
+ * quantizer's. */
+template <int MODE>
+__device__ __forceinline__ void hipq_quantize_q8_K_wave(
+  const float *__restrict__ A, int64_t M, int64_t sb, int nsb, int64_t lda, int64_t mat_rows,
+  int8_t *__restrict__ q_out, float *__restrict__ d_out, int16_t *__restrict__ bsum_out,
+  uint8_t *__restrict__ canon_out, uint16_t *__restrict__ amin_out, uint16_t *__restrict__ ql_out,
+  uint16_t *__restrict__ qh_out) {
+  const int lane = threadIdx.x & 63;
+  const int64_t m = sb / nsb;
+  const int b = (int)(sb - m * nsb);
+  float4 xv = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (m < M) xv = *(const float4 *)(A + m * lda + (int64_t)b * 256 + lane * 4);
+  const float x[4] = {xv.x, xv.y, xv.z, xv.w};
+
+  float amax = fmaxf(fmaxf(fabsf(x[0]), fabsf(x[1])), fmaxf(fabsf(x[2]), fabsf(x[3])));
+  amax = hipq_group_max<64>(amax);
+
+  int q[4];
+  float d;
+  if (amax == 0.0f) {
+    q[0] = q[1] = q[2] = q[3] = 0;
+    d = 0.f;
+  } else if (m < mat_rows) {
+    /* 4-row quantizer semantics */
+    const bool hit = (x[0] == amax) | (x[1] == amax) | (x[2] == amax) | (x[3] == amax);
+    const bool pos_hit = __ballot(hit) != 0ull;
+    const float iscale = pos_hit ? __fdiv_rn(-127.f, amax) : __fdiv_rn(127.f, amax);
+    d = __fdiv_rn(1.f, iscale);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int v = (int)rintf(__fmul_rn(x[i], iscale));
+      q[i] = max(-128, min(127, v));
+    }
+  } else {
+    /* row quantizer semantics: sign of the FIRST element of maximal magnitude */
+    float cand = 0.f;
+    bool has = false;
+#pragma unroll
+    for (int i = 3; i >= 0; --i)
+      if (fabsf(x[i]) == amax) {
+        cand = x[i];
+        has = true;
+      }
+    const unsigned long long mask = __ballot(has);
+    const int first = __ffsll((long long)mask) - 1;
+    const float vmax = __shfl(cand, first, HIPQ_WAVE);
+    const float iscale = __fdiv_rn(-127.f, vmax);
+    d = __fdiv_rn(1.f, iscale);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      q[i] = min(127, magic_to_int(__fmaf_rn(iscale, x[i], kRoundMagic)));
+  }
+
+  const int packed = pack4(q[0], q[1], q[2], q[3]);
+  int gsum = q[0] + q[1] + q[2] + q[3];
+  gsum = hipq_group_sum_i<4>(gsum); /* 4 lanes = one 16-value group */
+
+  if (MODE == Q8K_CANONICAL) {
+    uint8_t *o = canon_out + sb * 292;
+    if (lane == 0) *(float *)o = d;
+    *(int *)(o + 4 + lane * 4) = packed;
+    if ((lane & 3) == 0) *(int16_t *)(o + 260 + (lane >> 2) * 2) = (int16_t)gsum;
+  } else if (MODE == Q8K_TILED) {
+    const int64_t mt = m >> 7;
+    const int r = (int)(m & 127);
+    /* lane holds elements 4*lane .. 4*lane+3 of the super-block: sub-block lane / 8,
+     * whose 16-value half (lane / 4) % 2 is one 16-byte operand. The GEMM's lane
+     * (row, g) takes sub-blocks 4g .. 4g+3, two 32-deep steps each, so the operand
+     * belongs to step s = 2 * (sub-block % 4) + half of lane group g = sub-block / 4;
+     * within the operand the 8 even values come first, then the 8 odd ones (the
+     * order in which the weights' nibble bytes unpack). */
+    const int jb = lane >> 3, g = jb >> 2;
+    const int st = 2 * (jb & 3) + ((lane >> 2) & 1);
+    const int64_t tile = (mt * (2 * nsb) + b * 2 + (st >> 2)) * 16384;
+    const int off = ((r >> 5) * 4 + (st & 3)) * 1024 + (g * 32 + (r & 31)) * 16 + (lane & 3) * 2;
+    *(uint16_t *)(q_out + tile + off) = (uint16_t)((q[0] & 0xff) | ((q[2] & 0xff) << 8));
+    *(uint16_t *)(q_out + tile + off + 8) = (uint16_t)((q[1] & 0xff) | ((q[3] & 0xff) << 8));
+    const int64_t rb = (mt * nsb + b) * 128 + r;
+    if (lane == 0) d_out[rb] = d;
+    const int bs = gsum + __shfl_xor(gsum, 4, HIPQ_WAVE); /* two 16-value groups = one sub-block */
+    if ((lane & 7) == 0) {
+      const int l6 = bs & 63;
+      amin_out[rb * 16 + (lane >> 3)] = __half_as_ushort(__float2half_rn((float)l6));
+      amin_out[rb * 16 + 8 + (lane >> 3)] = __half_as_ushort(__float2half_rn((float)(bs - l6)));
+    }
+  } else if (MODE == Q8K_ROWMMA) {
+    /* row-major, each 16-value group stored as its 8 even then its 8 odd values:
+     * this lane's four values are elements 4l .. 4l+3 of group lane / 4 */
+    int8_t *o = q_out + sb * 256 + (lane >> 2) * 16 + (lane & 3) * 2;
+    *(uint16_t *)o = (uint16_t)((q[0] & 0xff) | ((q[2] & 0xff) << 8));
+    *(uint16_t *)(o + 8) = (uint16_t)((q[1] & 0xff) | ((q[3] & 0xff) << 8));
+    if (lane == 0) d_out[sb] = d;
+    const int bs = gsum + __shfl_xor(gsum, 4, HIPQ_WAVE); /* two 16-value groups = one sub-block */
+    if ((lane & 7) == 0) {
+      const int l6 = bs & 63;
+      amin_out[sb * 16 + (lane >> 3)] = __half_as_ushort(__float2half_rn((float)l6));
+      amin_out[sb * 16 + 8 + (lane >> 3)] = __half_as_ushort(__float2half_rn((float)(bs - l6)));
+    }
+  } else {
+    *(int *)(q_out + sb * 256 + lane * 4) = packed;
+    if (lane == 0) d_out[sb] = d;
+    if ((lane & 3) == 0) bsum_out[sb * 16 + (lane >> 2)] = (int16_t)gsum;
+    /* 4-bit digits for the v_dot8_u32_u4 kernels: q = 16 * (qh - 8) + ql */
+    uint32_t lo = 0, hi = 0;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      lo |= (uint32_t)(q[i] & 15) << (4 * i);
+      hi |= (uint32_t)(((q[i] >> 4) + 8) & 15) << (4 * i);
+    }
+    ql_out[sb * 64 + lane] = (uint16_t)lo;
+    qh_out[sb * 64 + lane] = (uint16_t)hi;
+  }
+}
+
+#endif /* HIPQ_QUANTIZE_DEVICE_H */
