@@ -296,7 +296,7 @@ def main():
             "ms_per_block": round(moe_ms, 5), "active_experts": active,
             "roofline": {"bound": "hbm", "achieved": round(moe_gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(moe_gbs / HBM_PEAK_GBS, 5), "algorithmic_bytes_per_block": moe_bytes,
-                         "traffic": 251.1e6 + 127.1e6 + 7.9e6},
+                         "traffic": 236.4e6 + 124.9e6 + 13.0e6},
             "decode_token": {"ms_per_block": round(moe_decode_ms, 5), "active_experts": decode_active,
                              "gbs": round(moe_decode_bytes / (moe_decode_ms * 1e-3) / 1e9, 2)}},
     }
