@@ -86,6 +86,32 @@ def test_moe_skewed_routing(hipq, cr, t, h, i, e, k):
         w.destroy()
 
 
+def test_moe_long_chunk_uses_the_multi_kernel_sort(hipq, cr):
+    """More than 16384 (token, expert) pairs: the pairs are counted, scanned and
+    scattered by separate kernels, which also list the work items."""
+    import gpu_util as gu
+    import torch
+    t, h, i, e, k = 2112, 256, 256, 8, 8
+    gate, up, down = _experts(cr, e, i, h, seed=9000)
+    x = synth.normal(9100, (t, h))
+    logits = synth.normal(9101, (t, e))
+    ref_y, ref_idx, _ = cr.moe_forward(x, logits, gate, up, down, k)
+    wg = [capi.Weight("q4_K", i, h, b) for b in gate]
+    wu = [capi.Weight("q4_K", i, h, b) for b in up]
+    wd = [capi.Weight("q4_K", h, i, b) for b in down]
+    y = torch.full((t, h), float("nan"), device="cuda")
+    idx = torch.zeros((t, k), dtype=torch.int32, device="cuda")
+    capi.moe_forward(t, h, i, e, k, wg, wu, wd, gu.dev(x), y, router_logits=gu.dev(logits), topk_idx=idx,
+                     stream=gu.stream())
+    torch.cuda.synchronize()
+    assert np.array_equal(np.sort(idx.cpu().numpy(), axis=1), np.sort(ref_idx, axis=1))
+    got = y.cpu().numpy()
+    assert not np.isnan(got).any()
+    assert gu.rel_err(got, ref_y) <= 2e-6, gu.rel_err(got, ref_y)
+    for w in wg + wu + wd:
+        w.destroy()
+
+
 def test_expert_weights_serve_the_moe_block_only(hipq, cr):
     """Q4_K experts are re-stored for the expert kernels at the first block; a plain
     matmul on such a handle is refused, the block keeps giving the same bits."""
