@@ -50,10 +50,10 @@ __global__ __launch_bounds__(256) void gemv_stream_kernel(WView w, QView qa,
   if (first >= w.N) return; /* uniform per wavefront; all syncs below are wavefront-local */
   const int K = w.K;
   const int arow[1] = {0};
+  typename E::Wts W[2];
+  E::load_w(W[0], w, first, 0, K); /* before the activations, whose loads are followed by arithmetic */
   typename E::Act A;
   E::load_act(A, qa, arow, 0, K);
-  typename E::Wts W[2];
-  E::load_w(W[0], w, first, 0, K);
 #pragma unroll
   for (int i = 0; i < GPW; ++i) {
     const int row0 = first + i * G;

@@ -126,17 +126,26 @@ template <int DT, int T, int KC> struct GemvUnits {
 };
 
 /* ---- Q4_0 ----------------------------------------------------------------------- */
+/* A zero the compiler cannot see through, produced where the call stands: a value
+ * combined with it cannot be computed before that point. */
+__device__ __forceinline__ uint32_t hipq_late_zero() {
+  uint32_t z;
+  asm volatile("v_mov_b32 %0, 0" : "=v"(z) : : "memory");
+  return z;
+}
+
 template <int T, int R, bool PW, int KC> struct GemvQ40 {
   static constexpr int MAXU = GemvUnits<HIPQ_Q4_0, T, KC>::MAXU;
   static constexpr int PER = GemvRec<HIPQ_Q4_0, PW>::PER_CHUNK;
   struct Act {
     int4 a0[MAXU][R], a1[MAXU][R];
-    float da[MAXU][R];
-    int bsum[MAXU][R];
+    uint32_t meta[MAXU][R]; /* fp16 d | int16 block sum << 16, decoded where it is used: arithmetic on a
+                               loaded value here would make the loads behind it wait for it */
   };
   struct Wt {
     uint4 q[MAXU];
-    uint16_t d[MAXU];
+    uint32_t d[MAXU]; /* the fp16 scale in a register of its own: two 16-bit loads into the halves of
+                         one register would have to wait for each other */
   };
   __device__ static __forceinline__ void load_act(Act &A, const QView &qa, const int (&arow)[R],
                                                   int tl, int k0, int kc) {
@@ -150,9 +159,7 @@ template <int T, int R, bool PW, int KC> struct GemvQ40 {
         const int4 *a = (const int4 *)(qa.q + (size_t)arow[r] * qa.K + (size_t)(u0 + u) * 32);
         A.a0[i][r] = a[0];
         A.a1[i][r] = a[1];
-        const uint32_t meta = qa.meta[(size_t)arow[r] * units + u0 + u];
-        A.da[i][r] = hipq_h2f((uint16_t)(meta & 0xffff));
-        A.bsum[i][r] = (int)(int16_t)(meta >> 16);
+        A.meta[i][r] = qa.meta[(size_t)arow[r] * units + u0 + u];
       }
     }
   }
@@ -177,17 +184,20 @@ template <int T, int R, bool PW, int KC> struct GemvQ40 {
       if (i * T >= un) break;
       const int u = tl + i * T;
       const uint4 q = W.q[i];
-      const float d = hipq_h2f(W.d[i]);
+      /* the zero is produced here, behind the loads: without it the compiler converts
+       * each scale right behind its load, and the loads after that one wait for it */
+      const float d = hipq_h2f((uint16_t)(W.d[i] | hipq_late_zero()));
       const uint32_t lo[4] = {q.x & HIPQ_M4, q.y & HIPQ_M4, q.z & HIPQ_M4, q.w & HIPQ_M4};
       const uint32_t hi[4] = {(q.x >> 4) & HIPQ_M4, (q.y >> 4) & HIPQ_M4, (q.z >> 4) & HIPQ_M4,
                               (q.w >> 4) & HIPQ_M4};
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         /* weights are nibble - 8 */
-        const int isum = hipq_dot16(lo, A.a0[i][r]) + hipq_dot16(hi, A.a1[i][r]) - 8 * A.bsum[i][r];
+        const int bsum = (int)(int16_t)(A.meta[i][r] >> 16);
+        const int isum = hipq_dot16(lo, A.a0[i][r]) + hipq_dot16(hi, A.a1[i][r]) - 8 * bsum;
         float2 v;
         v.x = (float)isum;
-        v.y = d * A.da[i][r];
+        v.y = d * hipq_h2f((uint16_t)(A.meta[i][r] & 0xffff));
         if (u < un) *(float2 *)(rec + r * PER + 2 * u) = v;
       }
     }
@@ -206,7 +216,7 @@ template <int T, int R, bool PW, int KC> struct GemvQ4K {
   static constexpr int PER = GemvRec<HIPQ_Q4_K, PW>::PER_CHUNK;
   struct Act {
     uint4 l[MAXU][R], h[MAXU][R]; /* digits of the sub-block's activations */
-    int bs[MAXU][R];              /* their sum */
+    int bs[MAXU][R];              /* the two int16 sums of its halves, as loaded */
     float dA[MAXU][R];
   };
   struct Wt {
@@ -227,7 +237,7 @@ template <int T, int R, bool PW, int KC> struct GemvQ4K {
         A.l[i][r] = *(const uint4 *)(qa.ql + off);
         A.h[i][r] = *(const uint4 *)(qa.qh + off);
         const int bsw = *(const int *)(qa.bsum + (size_t)arow[r] * (qa.K >> 4) + (b0 + b) * 16 + 2 * j);
-        A.bs[i][r] = (int)(int16_t)(bsw & 0xffff) + (bsw >> 16);
+        A.bs[i][r] = bsw;
         A.dA[i][r] = qa.d[(size_t)arow[r] * nsb + b0 + b];
       }
     }
@@ -267,7 +277,7 @@ template <int T, int R, bool PW, int KC> struct GemvQ4K {
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         int I = __mul24(sc, hipq_dot32_u4(W.q[i], A.l[i][r], A.h[i][r]));
-        int Im = __mul24(mn, A.bs[i][r]);
+        int Im = __mul24(mn, (int)(int16_t)(A.bs[i][r] & 0xffff) + (A.bs[i][r] >> 16));
         I += hipq_dpp_i<HIPQ_DPP_XOR1>(I); /* the sub-block pair */
         Im += hipq_dpp_i<HIPQ_DPP_XOR1>(Im);
         if (PW) {
@@ -587,16 +597,26 @@ __device__ __forceinline__ GemvOut gemv_engine(const WView &w, int row0, const Q
                                                uint32_t *lds) {
   typedef GemvCore<DT, T, R, G, PW, KC> E;
   typename E::Chain c = E::begin(arow, pair_rows);
-  for (int k0 = 0; k0 < w.K; k0 += KC) {
-    const int kc = min(KC, w.K - k0);
-    typename E::Act A;
-    E::load_act(A, qa, arow, k0, kc);
+  auto chunk = [&](int k0, int kc) {
+    /* the weights first: the activations' loads are followed by arithmetic on what
+     * they return, and in the other order the weight loads would be issued only
+     * after that round trip */
     typename E::Wts W;
     E::load_w(W, w, row0, k0, kc);
+    typename E::Act A;
+    E::load_act(A, qa, arow, k0, kc);
     E::compute(W, A, kc, lds);
     hipq_wave_lds_sync();
     E::chain(c, kc, lds);
     hipq_wave_lds_sync();
+  };
+  /* Rows of one chunk (the usual case) run outside the loop: inside it the compiler
+   * guards every load's destination registers against the loads of the previous
+   * iteration, which serialises the loads of the first one as well. */
+  if (w.K <= KC) {
+    chunk(0, w.K);
+  } else {
+    for (int k0 = 0; k0 < w.K; k0 += KC) chunk(k0, min(KC, w.K - k0));
   }
   return E::finish(c);
 }
