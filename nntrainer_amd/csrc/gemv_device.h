@@ -178,26 +178,28 @@ template <int T, int R, bool PW, int KC> struct GemvQ40 {
   }
   __device__ static __forceinline__ void compute(const Wt &W, const Act &A, int tl, int kc,
                                                  uint32_t *rec) {
+    /* the zero is produced here, behind the loads: without it the compiler decodes each
+     * 16-bit value right behind its load, and the loads after that one wait for it */
+    const uint32_t late = hipq_late_zero();
     const int un = kc >> 5;
 #pragma unroll
     for (int i = 0; i < MAXU; ++i) {
       if (i * T >= un) break;
       const int u = tl + i * T;
       const uint4 q = W.q[i];
-      /* the zero is produced here, behind the loads: without it the compiler converts
-       * each scale right behind its load, and the loads after that one wait for it */
-      const float d = hipq_h2f((uint16_t)(W.d[i] | hipq_late_zero()));
+      const float d = hipq_h2f((uint16_t)(W.d[i] | late));
       const uint32_t lo[4] = {q.x & HIPQ_M4, q.y & HIPQ_M4, q.z & HIPQ_M4, q.w & HIPQ_M4};
       const uint32_t hi[4] = {(q.x >> 4) & HIPQ_M4, (q.y >> 4) & HIPQ_M4, (q.z >> 4) & HIPQ_M4,
                               (q.w >> 4) & HIPQ_M4};
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         /* weights are nibble - 8 */
-        const int bsum = (int)(int16_t)(A.meta[i][r] >> 16);
+        const uint32_t meta = A.meta[i][r] | late;
+        const int bsum = (int)(int16_t)(meta >> 16);
         const int isum = hipq_dot16(lo, A.a0[i][r]) + hipq_dot16(hi, A.a1[i][r]) - 8 * bsum;
         float2 v;
         v.x = (float)isum;
-        v.y = d * hipq_h2f((uint16_t)(A.meta[i][r] & 0xffff));
+        v.y = d * hipq_h2f((uint16_t)(meta & 0xffff));
         if (u < un) *(float2 *)(rec + r * PER + 2 * u) = v;
       }
     }
