@@ -167,8 +167,8 @@ __device__ __forceinline__ void epilogue(const Smem<TM> &sm, int buf, const uint
   const int i32 = lane & 31, g = lane >> 5;
   const float dcol = hipq_h2f((uint16_t)(hd.x & 0xffff));
   const float ndmin = -hipq_h2f((uint16_t)(hd.x >> 16));
-  const uint32_t mlo = hd.z & 0x3f3f3f3fu;
-  const uint32_t mhi = ((hd.w >> 4) & 0x0f0f0f0fu) | (((hd.z >> 6) & 0x03030303u) << 4);
+  const uint32_t mlo = (hd.w & 0x0f0f0f0fu) | ((hd.y >> 2) & 0x30303030u);
+  const uint32_t mhi = ((hd.w >> 4) & 0x0f0f0f0fu) | ((hd.z >> 2) & 0x30303030u);
   v8h bmin;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
@@ -253,9 +253,7 @@ __global__ __launch_bounds__(NT, TM == 2 ? 3 : 2) void gemm_q4k_kernel(WView w, 
    * flight. hd / hdn and Wa / Wb alternate between consecutive super-blocks. */
   auto super_block = [&](int sb, const uint4 &hd, uint4 &hdn, int eb) {
     /* 6-bit scales of sub-blocks 4g .. 4g+3, one per byte, as two 3-bit digits */
-    const uint32_t s03 = hd.y & 0x3f3f3f3fu;
-    const uint32_t s47 = (hd.w & 0x0f0f0f0fu) | ((hd.y >> 2) & 0x30303030u);
-    const uint32_t sc = g ? s47 : s03;
+    const uint32_t sc = (g ? hd.z : hd.y) & 0x3f3f3f3fu;
     const uint32_t slo = sc & 0x07070707u, shi = (sc >> 3) & 0x07070707u;
     const int sbn = min(sb + 1, nsb - 1);
     {

@@ -268,12 +268,11 @@ template <int T, int R, bool PW, int KC> struct GemvQ4K {
       const int uc = on ? u : un - 1;
       const int b = uc >> 3, j = uc & 7;
       const uint4 hd = W.hd[i];
-      /* 6-bit scale / min of sub-block j: byte j of y / z for j < 4, else the low /
-       * high nibble of byte j-4 of w with bits 6-7 of byte j-4 of y / z on top */
-      const int sh = 8 * (j & 3);
-      const uint32_t y = hd.y >> sh, z = hd.z >> sh, ww = hd.w >> sh;
-      const int sc = (int)(j < 4 ? (y & 0x3fu) : ((ww & 0x0fu) | ((y >> 2) & 0x30u)));
-      const int mn = (int)(j < 4 ? (z & 0x3fu) : (((ww >> 4) & 0x0fu) | ((z >> 2) & 0x30u)));
+      /* scale and min of sub-block j: byte j of (y, z) holds sc_j and, in its top two
+       * bits, m_j >> 4; byte j & 3 of w holds m_j & 15 in its low (j < 4) or high nibble */
+      const uint32_t yz = (j < 4 ? hd.y : hd.z) >> (8 * (j & 3));
+      const int sc = (int)(yz & 0x3fu);
+      const int mn = (int)(((hd.w >> (8 * (j & 3) + (j & 4))) & 0x0fu) | ((yz >> 2) & 0x30u));
       const float dw = hipq_h2f((uint16_t)(hd.x & 0xffff));
       const float dmin = hipq_h2f((uint16_t)(hd.x >> 16));
 #pragma unroll

@@ -24,7 +24,12 @@
 /*         d  [N][K/32] fp16                                                  */
 /*   Q4_K: qs [N][K/2]  (128 B per super-block: sub-block j = bytes 16j..16j+15, */
 /*                      weight 2i low / 2i+1 high nibble of byte i)             */
-/*         hdr[N][K/256][16] = {fp16 d, fp16 dmin, scales[12]}                */
+/*         hdr[N][K/256][16] = {fp16 d, fp16 dmin, sm[8], ml[4]}: the 6-bit     */
+/*                      scales sc_j and mins m_j of block_q4_K regrouped so that */
+/*                      byte sm[j] = sc_j | (m_j >> 4) << 6 and byte ml[k] =     */
+/*                      (m_k & 15) | (m_(k+4) & 15) << 4. A GEMV lane takes the  */
+/*                      scale and min of ONE sub-block with three shifts; the    */
+/*                      matrix kernels take all eight as bytes of two words      */
 /*   Q6_K: qs [2][N][K/4] (ql in two planes, 64 B per super-block each: unit  */
 /*                      uu = half*2 + hl holds bytes half*64 + hl*16 .. +15 of  */
 /*                      block_q6_K::ql in the first and those 32 further on in   */

@@ -653,7 +653,7 @@ __device__ __forceinline__ void xr_super_block(const XRegs &W, const XLds &l, in
   }
   const uint4 hd = make_uint4((uint32_t)W.hd[0], (uint32_t)W.hd[1], (uint32_t)W.hd[2], (uint32_t)W.hd[3]);
   const uint32_t s03 = hd.y & 0x3f3f3f3fu;
-  const uint32_t s47 = (hd.w & 0x0f0f0f0fu) | ((hd.y >> 2) & 0x30303030u);
+  const uint32_t s47 = hd.z & 0x3f3f3f3fu;
   int I[NREG];
 #pragma unroll
   for (int r = 0; r < NREG; ++r) I[r] = 0;
@@ -673,7 +673,7 @@ __device__ __forceinline__ void xr_super_block(const XRegs &W, const XLds &l, in
 #pragma unroll
     for (int r = 0; r < NREG; ++r) I[r] = __mul24(D[r], scj) + I[r];
   }
-  const uint32_t mlo = hd.z & 0x3f3f3f3fu;
+  const uint32_t mlo = (hd.w & 0x0f0f0f0fu) | ((hd.y >> 2) & 0x30303030u);
   const uint32_t mhi = ((hd.w >> 4) & 0x0f0f0f0fu) | ((hd.z >> 2) & 0x30303030u);
   mv8h bmin;
 #pragma unroll

@@ -54,10 +54,18 @@ __global__ void relayout_q4_K(const uint8_t *__restrict__ src, int x8, int64_t N
   const int b = (int)(i - n * nb);
   uint8_t *oq = qs + i * 128;
   uint8_t *oh = hdr + i * 16;
+  uint8_t sc[8], mn[8]; /* the super-block's 6-bit scales and mins */
   uint8_t cq[128]; /* the super-block's qs in the byte order of block_q4_K */
   if (!x8) {
     const uint8_t *blk = src + i * 144;
-    for (int k = 0; k < 16; ++k) oh[k] = blk[k];
+    for (int k = 0; k < 4; ++k) oh[k] = blk[k];
+    const uint8_t *s = blk + 4; /* the 12 packed bytes of block_q4_K */
+    for (int j = 0; j < 4; ++j) {
+      sc[j] = s[j] & 63;
+      mn[j] = s[j + 4] & 63;
+      sc[j + 4] = (uint8_t)((s[j + 8] & 0x0f) | ((s[j] >> 6) << 4));
+      mn[j + 4] = (uint8_t)((s[j + 8] >> 4) | ((s[j + 4] >> 6) << 4));
+    }
     for (int k = 0; k < 128; ++k) cq[k] = blk[16 + k];
   } else {
     const int r = (int)(n & 7);
@@ -67,24 +75,19 @@ __global__ void relayout_q4_K(const uint8_t *__restrict__ src, int x8, int64_t N
     oh[2] = grp[16 + 2 * r];
     oh[3] = grp[16 + 2 * r + 1];
     /* group g of the interleaved scales holds sub-block g of all 8 rows,
-     * indexed by row; rebuild this row's 12 bytes indexed by sub-block */
-    uint8_t s[12];
-    for (int k = 0; k < 12; ++k) s[k] = 0;
+     * indexed by row */
     for (int g = 0; g < 8; ++g) {
-      int sc, mn;
-      scale_min(r, grp + 32 + 12 * g, sc, mn);
-      if (g < 4) {
-        s[g] |= (uint8_t)sc;
-        s[g + 4] |= (uint8_t)mn;
-      } else {
-        s[g + 4] = (uint8_t)((sc & 0x0f) | ((mn & 0x0f) << 4));
-        s[g - 4] |= (uint8_t)((sc >> 4) << 6);
-        s[g] |= (uint8_t)((mn >> 4) << 6);
-      }
+      int s1, m1;
+      scale_min(r, grp + 32 + 12 * g, s1, m1);
+      sc[g] = (uint8_t)s1;
+      mn[g] = (uint8_t)m1;
     }
-    for (int k = 0; k < 12; ++k) oh[4 + k] = s[k];
     for (int k = 0; k < 128; ++k) cq[k] = grp[128 + (k >> 3) * 64 + r * 8 + (k & 7)];
   }
+  /* each sub-block's scale in a byte of its own with the top two bits of its min
+   * above it, then the low four bits of the mins of sub-blocks k and k + 4 per byte */
+  for (int j = 0; j < 8; ++j) oh[4 + j] = (uint8_t)(sc[j] | ((mn[j] >> 4) << 6));
+  for (int k = 0; k < 4; ++k) oh[12 + k] = (uint8_t)((mn[k] & 15) | ((mn[k + 4] & 15) << 4));
   /* block_q4_K keeps sub-blocks 2c / 2c+1 in the low / high nibbles of 32 bytes.
    * The device plane stores each sub-block's 32 weights as 16 consecutive bytes,
    * weight 2i in the low and 2i+1 in the high nibble of byte i, so that one
