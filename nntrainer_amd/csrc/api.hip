@@ -179,6 +179,7 @@ int matmul_device(hipq_weight_t w, const float *A, int64_t M, int64_t lda, float
                   hipStream_t s) {
   if (M == 0) return HIPQ_OK;
   if (wants_tiled(w, M)) return matmul_tiled(w, A, M, lda, C, ldc, s, 0);
+  if (M == 1 && hipq::gemv_fuses_quantizer(w, A)) return hipq::launch_gemv_fused(w, A, C, s);
   const int is_k = w->dtype != HIPQ_Q4_0;
   void *mem = nullptr;
   int rc = workspace(s, qact_bytes(is_k, M, w->K), &mem);
@@ -523,6 +524,10 @@ int hipq_time_matmul(int n_weights, const hipq_weight_t *w, const float *A, int6
     const hipq_weight *wi = w[it % n_weights];
     if (tiled) {
       rc = matmul_tiled(wi, A, M, lda, C, ldc, s, phase);
+      continue;
+    }
+    if (phase == 0 && M == 1 && hipq::gemv_fuses_quantizer(wi, A)) {
+      rc = hipq::launch_gemv_fused(wi, A, C, s);
       continue;
     }
     if (phase == 0 || phase == 2) rc = quantize_for(wi, A, M, lda, qa, s);

@@ -18,6 +18,7 @@
  * 16 bytes per lane per load, all loads of a group in flight together.
  */
 #include "gemv_device.h"
+#include "quantize_device.h"
 
 namespace {
 
@@ -67,6 +68,108 @@ __global__ __launch_bounds__(256) void gemv_stream_kernel(WView w, QView qa,
     const GemvOut o = E::finish(c);
     if (o.valid && row0 + o.g < w.N) C[row0 + o.g] = o.v;
   }
+}
+
+/* Decode GEMV on the fp32 activation row itself: the workgroup quantizes the row
+ * into LDS (the arithmetic of the quantizer kernels, so the blocks are the same
+ * bits) while its weight loads are in flight, and the engine reads the activations
+ * from there. Saves the quantizer's launch, which costs more than the redundant
+ * quantization as long as the matrix is small. One chunk only (K <= 4096). */
+template <int DT> __host__ __device__ constexpr int fused_act_bytes(int K) {
+  /* Q8_0: q [K], meta [K/32] u32; Q8_K: q [K], ql [K/2], qh [K/2], bsum [K/16] i16, d [K/256] f32 */
+  return ((DT == HIPQ_Q4_0 ? K + K / 8 : 2 * K + K / 8 + K / 64) + 15) & ~15;
+}
+
+template <int DT, int T, int G>
+__global__ __launch_bounds__(256) void gemv_fused_kernel(WView w, const float *__restrict__ x,
+                                                         float *__restrict__ C) {
+  typedef GemvCore<DT, T, 1, G, false> E;
+  extern __shared__ __attribute__((aligned(16))) uint32_t gemv_lds[];
+  const int K = w.K;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  uint8_t *ap = (uint8_t *)gemv_lds;
+  uint32_t *lds = gemv_lds + fused_act_bytes<DT>(K) / 4 + wave * GemvLds<DT, 1, G, false>::DWORDS;
+  const int row0 = (blockIdx.x * 4 + wave) * G;
+  const int arow[1] = {0};
+
+  /* the row first (it comes from the cache), then the weights: the wait for the row
+   * leaves the weight loads in flight. Positions beyond the row re-read its end. */
+  float4 xs[4];
+  if (DT == HIPQ_Q4_0) {
+    const int nb = K >> 5;
+#pragma unroll
+    for (int p = 0; p < 4; ++p)
+      xs[p] = *(const float4 *)(x + min((int)(threadIdx.x >> 3) + 32 * p, nb - 1) * 32 + (threadIdx.x & 7) * 4);
+  } else {
+    const int nsb = K >> 8;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) xs[p] = *(const float4 *)(x + min(wave + 4 * p, nsb - 1) * 256 + lane * 4);
+  }
+  typename E::Wts W;
+  E::load_w(W, w, row0, 0, K);
+
+  QView qa;
+  qa.K = K;
+  qa.q = (const int8_t *)ap;
+  if (DT == HIPQ_Q4_0) {
+    int8_t *q = (int8_t *)ap;
+    uint32_t *meta = (uint32_t *)(ap + K);
+    qa.meta = meta;
+    qa.d = nullptr;
+    qa.bsum = nullptr;
+    qa.ql = qa.qh = nullptr;
+    const int nb = K >> 5, sub = threadIdx.x & 7;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      if (32 * p >= nb) break; /* uniform */
+      const int blk = (int)(threadIdx.x >> 3) + 32 * p;
+      uint16_t dh;
+      int qsum;
+      const int packed = hipq_quantize_q8_0_lane(xs[p], dh, qsum);
+      const int bsum = hipq_group_sum_i<8>(qsum);
+      if (blk < nb) {
+        *(int *)(q + blk * 32 + sub * 4) = packed;
+        if (sub == 0) meta[blk] = (uint32_t)dh | ((uint32_t)(bsum & 0xffff) << 16);
+      }
+    }
+  } else {
+    int8_t *q = (int8_t *)ap;
+    uint16_t *ql = (uint16_t *)(ap + K), *qh = (uint16_t *)(ap + K + (K >> 1));
+    int16_t *bsum = (int16_t *)(ap + 2 * K);
+    float *d = (float *)(ap + 2 * K + (K >> 3));
+    qa.meta = nullptr;
+    qa.d = d;
+    qa.bsum = bsum;
+    qa.ql = (const uint8_t *)ql;
+    qa.qh = (const uint8_t *)qh;
+    const int nsb = K >> 8;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+      const int sb = wave + 4 * p;
+      if (sb >= nsb) break; /* uniform per wavefront */
+      hipq_quantize_q8_K_values<Q8K_PLANES>(xs[p], 0, sb, sb, nsb, 0, q, d, bsum, nullptr, nullptr, ql, qh);
+    }
+  }
+  __syncthreads();
+
+  typename E::Act A;
+  E::load_act(A, qa, arow, 0, K);
+  typename E::Chain c = E::begin(arow, 0);
+  E::compute(W, A, K, lds);
+  hipq_wave_lds_sync();
+  E::chain(c, K, lds);
+  hipq_wave_lds_sync();
+  const GemvOut o = E::finish(c);
+  if (o.valid && row0 + o.g < w.N) C[row0 + o.g] = o.v;
+}
+
+template <int DT, int T, int G>
+int launch_fused_one(const hipq_weight *w, const float *x, float *C, hipStream_t s) {
+  const unsigned grid = (unsigned)((w->N + 4 * G - 1) / (4 * G));
+  const size_t lds = fused_act_bytes<DT>((int)w->K) + 4 * GemvLds<DT, 1, G, false>::DWORDS * sizeof(uint32_t);
+  hipLaunchKernelGGL((gemv_fused_kernel<DT, T, G>), dim3(grid), dim3(256), lds, s, wview(w), x, C);
+  HIPQ_HIP(hipGetLastError());
+  return HIPQ_OK;
 }
 
 template <int DT, int G, int GPW>
@@ -126,6 +229,26 @@ int launch_m1(const hipq_weight *w, const QAct *qa, float *C, int64_t ldc, hipSt
   }
 }
 
+/* The shapes of launch_m1 below its streaming case, on the fp32 row. */
+template <int DT> int launch_fused(const hipq_weight *w, const float *x, float *C, hipStream_t s) {
+  const int64_t units = w->K / GemvRec<DT, false>::UNIT;
+  if (units < 64) {
+    if (pick_group(w->N, 8) == 8) return launch_fused_one<DT, 16, 8>(w, x, C, s);
+    return launch_fused_one<DT, 16, 4>(w, x, C, s);
+  }
+  switch (pick_group(w->N, 8)) {
+  case 8:
+    return launch_fused_one<DT, 64, 8>(w, x, C, s);
+  case 4:
+    return launch_fused_one<DT, 64, 4>(w, x, C, s);
+  case 2:
+    return launch_fused_one<DT, 64, 2>(w, x, C, s);
+  default:
+    if (DT == HIPQ_Q4_0) return launch_fused_one<DT, 64, 2>(w, x, C, s);
+    return launch_fused_one<DT, 64, 1>(w, x, C, s);
+  }
+}
+
 /* 2..8 activation rows in one pass (small prefill chunks, leftover rows). */
 template <int DT>
 int launch_mr(const hipq_weight *w, const QAct *qa, int M, int pair_rows, float *C, int64_t ldc,
@@ -154,6 +277,26 @@ int launch_gemv(const hipq_weight *w, const QAct *qa, int M, int pair_rows, floa
   case HIPQ_Q6_K:
     return M == 1 ? launch_m1<HIPQ_Q6_K>(w, qa, C, ldc, s)
                   : launch_mr<HIPQ_Q6_K>(w, qa, M, pair_rows, C, ldc, s);
+  }
+  return fail(HIPQ_ERR_INVALID_ARGUMENT, "unknown weight dtype %d", w->dtype);
+}
+
+/* Matrices up to 128 MB of weights: beyond that the quantizer's launch is a few
+ * per cent of the GEMV and every workgroup quantizing the row costs as much. */
+bool gemv_fuses_quantizer(const hipq_weight *w, const float *x) {
+  return w->K <= HIPQ_KCHUNK && w->N < 32768 && ((uintptr_t)x & 15) == 0;
+}
+
+int launch_gemv_fused(const hipq_weight *w, const float *x, float *C, hipStream_t s) {
+  if (!gemv_fuses_quantizer(w, x))
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "this matrix does not take the GEMV that quantizes its own row");
+  switch (w->dtype) {
+  case HIPQ_Q4_0:
+    return launch_fused<HIPQ_Q4_0>(w, x, C, s);
+  case HIPQ_Q4_K:
+    return launch_fused<HIPQ_Q4_K>(w, x, C, s);
+  case HIPQ_Q6_K:
+    return launch_fused<HIPQ_Q6_K>(w, x, C, s);
   }
   return fail(HIPQ_ERR_INVALID_ARGUMENT, "unknown weight dtype %d", w->dtype);
 }

@@ -164,6 +164,9 @@ int launch_quantize_q8_K_tiled(const float *A, int64_t M, int64_t K, int64_t lda
 /* gemv.hip ---------------------------------------------------------------- */
 /* C[m][n] for m < M <= 8: one pass over the weights, M activation rows.
  * Rows below pair_rows use the reference GEMM kernel's fp32 order (Q4_K). */
+/* one fp32 activation row, quantized inside the GEMV's workgroups (small matrices) */
+bool gemv_fuses_quantizer(const hipq_weight *w, const float *x);
+int launch_gemv_fused(const hipq_weight *w, const float *x, float *C, hipStream_t s);
 int launch_gemv(const hipq_weight *w, const QAct *qa, int M, int pair_rows,
                 float *C, int64_t ldc, hipStream_t s);
 

@@ -39,17 +39,9 @@ __global__ __launch_bounds__(256) void quantize_q8_0_kernel(
   const int b = (int)(blk - m * nb);
   const float4 x = *(const float4 *)(A + m * lda + (int64_t)b * 32 + sub * 4);
 
-  float amax = fmaxf(fmaxf(fabsf(x.x), fabsf(x.y)), fmaxf(fabsf(x.z), fabsf(x.w)));
-  amax = hipq_group_max<8>(amax);
-
-  const float d = __fdiv_rn(amax, 127.f);
-  const float id = (amax != 0.0f) ? __fdiv_rn(127.f, amax) : 0.0f;
-  const int q0 = (int)rintf(__fmul_rn(x.x, id));
-  const int q1 = (int)rintf(__fmul_rn(x.y, id));
-  const int q2 = (int)rintf(__fmul_rn(x.z, id));
-  const int q3 = (int)rintf(__fmul_rn(x.w, id));
-  const int packed = pack4(q0, q1, q2, q3);
-  const uint16_t dh = hipq_f2h(d);
+  uint16_t dh;
+  int qsum;
+  const int packed = hipq_quantize_q8_0_lane(x, dh, qsum);
 
   if (CANONICAL) {
     if (!live) return;
@@ -59,7 +51,7 @@ __global__ __launch_bounds__(256) void quantize_q8_0_kernel(
     qs[0] = (uint16_t)(packed & 0xffff);
     qs[1] = (uint16_t)((unsigned)packed >> 16);
   } else {
-    int bsum = hipq_group_sum_i<8>(q0 + q1 + q2 + q3);
+    int bsum = hipq_group_sum_i<8>(qsum);
     if (!live) return;
     *(int *)(q_out + (m * nb + b) * 32 + sub * 4) = packed;
     if (sub == 0) meta_out[m * nb + b] = (uint32_t)dh | ((uint32_t)(bsum & 0xffff) << 16);

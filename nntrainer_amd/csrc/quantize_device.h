@@ -2,11 +2,14 @@
 /**
  * @file   quantize_device.h
  * @brief  The Q8_K activation quantizer of one wavefront (one 256-value
- *         super-block), shared by the quantizer kernels and by kernels that
- *         quantize rows as part of another launch.
+ *         super-block) and the Q8_0 quantizer of eight lanes (one 32-value
+ *         block), shared by the quantizer kernels and by kernels that quantize
+ *         rows as part of another launch.
  *
  * Bit-exact with the reference CPU quantizers in an x86 AVX2 GCC build
  * (IMPL = nntrainer/tensor/cpu_backend/ggml_interface/nntr_ggml_impl):
+ *   Q8_0 IMPL/nntr_ggml_impl_quant.cpp:613-701 and the per-row content of
+ *        IMPL/nntr_ggml_impl.cpp:7879-7980
  *   ROW  IMPL/nntr_ggml_impl_quant.cpp:1334-1374, where the compiler fuses
  *        iscale*x + 1.5*2^23 into a single rounding
  *   MAT  IMPL/nntr_ggml_impl.cpp:7504-7737 (product rounded to fp32, then to
@@ -26,24 +29,35 @@ __device__ __forceinline__ int pack4(int a, int b, int c, int d) {
   return (a & 0xff) | ((b & 0xff) << 8) | ((c & 0xff) << 16) | ((d & 0xff) << 24);
 }
 
+/* Q8_0: the calling lane holds four consecutive values of a 32-value block, the
+ * eight lanes of the block are consecutive. Returns the lane's four int8 values
+ * packed; dh = the block's fp16 scale. */
+__device__ __forceinline__ int hipq_quantize_q8_0_lane(const float4 &x, uint16_t &dh, int &qsum) {
+  float amax = fmaxf(fmaxf(fabsf(x.x), fabsf(x.y)), fmaxf(fabsf(x.z), fabsf(x.w)));
+  amax = hipq_group_max<8>(amax);
+  const float d = __fdiv_rn(amax, 127.f);
+  const float id = (amax != 0.0f) ? __fdiv_rn(127.f, amax) : 0.0f;
+  const int q0 = (int)rintf(__fmul_rn(x.x, id));
+  const int q1 = (int)rintf(__fmul_rn(x.y, id));
+  const int q2 = (int)rintf(__fmul_rn(x.z, id));
+  const int q3 = (int)rintf(__fmul_rn(x.w, id));
+  dh = hipq_f2h(d);
+  qsum = q0 + q1 + q2 + q3;
+  return pack4(q0, q1, q2, q3);
+}
+
 /* output forms of the Q8_K quantizer */
 enum { Q8K_PLANES = 0, Q8K_CANONICAL = 1, Q8K_TILED = 2, Q8K_ROWMMA = 3 };
 
-/* Super-block sb = (row m, block b) of A by the calling wavefront (all 64 lanes).
- * In the tiled mode rows M and beyond are padding and are written as zeros. Rows
- * below mat_rows take the 4-row quantizer's semantics, the others the row
- * quantizer's. */
+/* Super-block sb = (row m, block b) by the calling wavefront (all 64 lanes), lane l
+ * holding its values 4l .. 4l+3 in xv. Rows below mat_rows take the 4-row
+ * quantizer's semantics, the others the row quantizer's. */
 template <int MODE>
-__device__ __forceinline__ void hipq_quantize_q8_K_wave(
-  const float *__restrict__ A, int64_t M, int64_t sb, int nsb, int64_t lda, int64_t mat_rows,
-  int8_t *__restrict__ q_out, float *__restrict__ d_out, int16_t *__restrict__ bsum_out,
-  uint8_t *__restrict__ canon_out, uint16_t *__restrict__ amin_out, uint16_t *__restrict__ ql_out,
-  uint16_t *__restrict__ qh_out) {
+__device__ __forceinline__ void hipq_quantize_q8_K_values(
+  const float4 &xv, int64_t m, int b, int64_t sb, int nsb, int64_t mat_rows, int8_t *__restrict__ q_out,
+  float *__restrict__ d_out, int16_t *__restrict__ bsum_out, uint8_t *__restrict__ canon_out,
+  uint16_t *__restrict__ amin_out, uint16_t *__restrict__ ql_out, uint16_t *__restrict__ qh_out) {
   const int lane = threadIdx.x & 63;
-  const int64_t m = sb / nsb;
-  const int b = (int)(sb - m * nsb);
-  float4 xv = make_float4(0.f, 0.f, 0.f, 0.f);
-  if (m < M) xv = *(const float4 *)(A + m * lda + (int64_t)b * 256 + lane * 4);
   const float x[4] = {xv.x, xv.y, xv.z, xv.w};
 
   float amax = fmaxf(fmaxf(fabsf(x[0]), fabsf(x[1])), fmaxf(fabsf(x[2]), fabsf(x[3])));
@@ -144,6 +158,23 @@ __device__ __forceinline__ void hipq_quantize_q8_K_wave(
     ql_out[sb * 64 + lane] = (uint16_t)lo;
     qh_out[sb * 64 + lane] = (uint16_t)hi;
   }
+}
+
+/* The same with the values read from row m of A. In the tiled mode rows M and
+ * beyond are padding and are written as zeros. */
+template <int MODE>
+__device__ __forceinline__ void hipq_quantize_q8_K_wave(
+  const float *__restrict__ A, int64_t M, int64_t sb, int nsb, int64_t lda, int64_t mat_rows,
+  int8_t *__restrict__ q_out, float *__restrict__ d_out, int16_t *__restrict__ bsum_out,
+  uint8_t *__restrict__ canon_out, uint16_t *__restrict__ amin_out, uint16_t *__restrict__ ql_out,
+  uint16_t *__restrict__ qh_out) {
+  const int lane = threadIdx.x & 63;
+  const int64_t m = sb / nsb;
+  const int b = (int)(sb - m * nsb);
+  float4 xv = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (m < M) xv = *(const float4 *)(A + m * lda + (int64_t)b * 256 + lane * 4);
+  hipq_quantize_q8_K_values<MODE>(xv, m, b, sb, nsb, mat_rows, q_out, d_out, bsum_out, canon_out, amin_out,
+                                  ql_out, qh_out);
 }
 
 #endif /* HIPQ_QUANTIZE_DEVICE_H */

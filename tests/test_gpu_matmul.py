@@ -137,6 +137,32 @@ def test_matmul_multi_shares_quantization(hipq, cr):
         w.destroy()
 
 
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("n,k", [(8, 256), (37, 256), (1000, 768), (1024, 1024), (3072, 1024), (2050, 2048),
+                                 (4096, 4096), (8200, 3072), (12288, 4096)])
+def test_decode_row_quantized_in_the_gemv_equals_the_two_launches(hipq, cr, kind, n, k):
+    """hipq_matmul with one row on a small matrix runs one kernel whose workgroups
+    quantize the row themselves; the multi-weight entry keeps the quantizer kernel and
+    the GEMV on its blocks. Same arithmetic, so the outputs are the same bits; the
+    oracle pins both."""
+    import gpu_util as gu
+    import torch
+    blocks = _weights(cr, kind, n, k, seed=500 + n)
+    a = synth.normal(600 + k, (1, k))
+    a[0, 5] = 0.0
+    if k >= 512:
+        a[0, 256:512] = 0.0   # an all-zero block: scale 0
+    w = capi.Weight(kind, n, k, blocks)
+    one = gu.gpu_matmul(w, a)
+    two = torch.full((1, n), float("nan"), device="cuda")
+    capi.matmul_multi([w], gu.dev(a), 1, [two], stream=gu.stream())
+    torch.cuda.synchronize()
+    w.destroy()
+    assert np.array_equal(one, two.cpu().numpy())
+    ref = cr.gemm(cr.oracle(), kind, a, blocks, n)
+    assert gu.rel_err(one, ref) <= gu.TOL
+
+
 @pytest.mark.parametrize("kind,m", [("q4_K", 1), ("q4_K", 40), ("q6_K", 3)])
 def test_matmul_multi_other_formats_and_prefill(hipq, cr, kind, m):
     """The multi-weight entry with the Q8_K formats, one row and a prefill chunk (the
