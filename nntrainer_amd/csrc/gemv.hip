@@ -147,7 +147,8 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(WView w, const float *_
     for (int p = 0; p < 4; ++p) {
       const int sb = wave + 4 * p;
       if (sb >= nsb) break; /* uniform per wavefront */
-      hipq_quantize_q8_K_values<Q8K_PLANES>(xs[p], 0, sb, sb, nsb, 0, q, d, bsum, nullptr, nullptr, ql, qh);
+      hipq_quantize_q8_K_values < DT == HIPQ_Q4_K ? Q8K_DIGITS : Q8K_BYTES > (xs[p], 0, sb, sb, nsb, 0, q, d, bsum,
+                                                                             nullptr, nullptr, ql, qh);
     }
   }
   __syncthreads();

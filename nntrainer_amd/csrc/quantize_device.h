@@ -47,7 +47,14 @@ __device__ __forceinline__ int hipq_quantize_q8_0_lane(const float4 &x, uint16_t
 }
 
 /* output forms of the Q8_K quantizer */
-enum { Q8K_PLANES = 0, Q8K_CANONICAL = 1, Q8K_TILED = 2, Q8K_ROWMMA = 3 };
+enum {
+  Q8K_PLANES = 0,
+  Q8K_CANONICAL = 1,
+  Q8K_TILED = 2,
+  Q8K_ROWMMA = 3,
+  Q8K_DIGITS = 4, /* of the planes only what the Q4_K GEMV reads: ql, qh, bsum, d */
+  Q8K_BYTES = 5   /* of the planes only what the Q6_K GEMV reads: q, d */
+};
 
 /* Super-block sb = (row m, block b) by the calling wavefront (all 64 lanes), lane l
  * holding its values 4l .. 4l+3 in xv. Rows below mat_rows take the 4-row
@@ -145,18 +152,20 @@ __device__ __forceinline__ void hipq_quantize_q8_K_values(
       amin_out[sb * 16 + 8 + (lane >> 3)] = __half_as_ushort(__float2half_rn((float)(bs - l6)));
     }
   } else {
-    *(int *)(q_out + sb * 256 + lane * 4) = packed;
+    if (MODE != Q8K_DIGITS) *(int *)(q_out + sb * 256 + lane * 4) = packed;
     if (lane == 0) d_out[sb] = d;
-    if ((lane & 3) == 0) bsum_out[sb * 16 + (lane >> 2)] = (int16_t)gsum;
-    /* 4-bit digits for the v_dot8_u32_u4 kernels: q = 16 * (qh - 8) + ql */
-    uint32_t lo = 0, hi = 0;
+    if (MODE != Q8K_BYTES) {
+      if ((lane & 3) == 0) bsum_out[sb * 16 + (lane >> 2)] = (int16_t)gsum;
+      /* 4-bit digits for the v_dot8_u32_u4 kernels: q = 16 * (qh - 8) + ql */
+      uint32_t lo = 0, hi = 0;
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      lo |= (uint32_t)(q[i] & 15) << (4 * i);
-      hi |= (uint32_t)(((q[i] >> 4) + 8) & 15) << (4 * i);
+      for (int i = 0; i < 4; ++i) {
+        lo |= (uint32_t)(q[i] & 15) << (4 * i);
+        hi |= (uint32_t)(((q[i] >> 4) + 8) & 15) << (4 * i);
+      }
+      ql_out[sb * 64 + lane] = (uint16_t)lo;
+      qh_out[sb * 64 + lane] = (uint16_t)hi;
     }
-    ql_out[sb * 64 + lane] = (uint16_t)lo;
-    qh_out[sb * 64 + lane] = (uint16_t)hi;
   }
 }
 
