@@ -191,6 +191,63 @@ def main():
 
     c5_prefill_ms, c5_decode_ms = fc_stack(512), fc_stack(1)
 
+    def decode_layer_graph(grouped):
+        """One decode step's FCs of 8 layers (8 weight copies) captured in a graph and
+        replayed: milliseconds per layer without the host's launch cost. grouped: Q, K, V
+        and gate, up each as one hipq_matmul_multi call (4 launches per layer, not 7)."""
+        shapes = [(2048, 1024), (1024, 1024), (1024, 1024), (1024, 2048), (3072, 1024), (3072, 1024), (1024, 3072)]
+        layers = []
+        for _ in range(8):
+            ws_ = []
+            for n_, k_ in shapes:
+                w32_ = torch.randn((n_, k_), generator=gen, device="cuda", dtype=torch.float32) * 0.02
+                b_ = torch.empty(capi.weight_nbytes("q4_0", n_, k_), dtype=torch.uint8, device="cuda")
+                capi.quantize_weights("q4_0", w32_, n_, k_, b_, stream=stream)
+                torch.cuda.synchronize()
+                ws_.append(capi.Weight("q4_0", n_, k_, b_, mem=capi.MEM_DEVICE))
+            layers.append(ws_)
+        xs_ = {k_: torch.randn((1, k_), generator=gen, device="cuda") for k_ in (1024, 2048, 3072)}
+        cs_ = [torch.empty((1, n_), device="cuda") for n_, _ in shapes]
+
+        def step(st):
+            for ws_ in layers:
+                if grouped:
+                    capi.matmul_multi(ws_[0:3], xs_[1024], 1, cs_[0:3], stream=st)
+                    capi.matmul(ws_[3], xs_[2048], 1, cs_[3], stream=st)
+                    capi.matmul_multi(ws_[4:6], xs_[1024], 1, cs_[4:6], stream=st)
+                    capi.matmul(ws_[6], xs_[3072], 1, cs_[6], stream=st)
+                else:
+                    for w_, (n_, k_), c_ in zip(ws_, shapes, cs_):
+                        capi.matmul(w_, xs_[k_], 1, c_, stream=st)
+
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step(side.cuda_stream)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            step(side.cuda_stream)
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        reps = 20
+        e0.record()
+        for _ in range(reps):
+            graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / (reps * len(layers))
+        del graph
+        for ws_ in layers:
+            for w_ in ws_:
+                w_.destroy()
+        return ms
+
+    c5_graph_ms, c5_graph_grouped_ms = decode_layer_graph(False), decode_layer_graph(True)
+
     # ---- the MoE block of configs[3]: 64 tokens, 128 experts, top-8, Q4_K ----------
     mt, mh, me, mi, mk = 64, 2048, 128, 768, 8
 
@@ -288,7 +345,9 @@ def main():
         "c5_fc_stack_per_layer": {
             "workload": "the seven Q4_0 FCs of one Qwen3-0.6B-shaped decoder layer (BASELINE configs[4]) through "
                         "hipq_matmul, quantizers included, 8 weight copies rotated per FC",
-            "prefill_512_rows_ms": round(c5_prefill_ms, 5), "decode_1_row_ms": round(c5_decode_ms, 5)},
+            "prefill_512_rows_ms": round(c5_prefill_ms, 5), "decode_1_row_ms": round(c5_decode_ms, 5),
+            "decode_1_row_in_a_graph_ms": round(c5_graph_ms, 5),
+            "decode_1_row_in_a_graph_qkv_and_gate_up_as_one_launch_each_ms": round(c5_graph_grouped_ms, 5)},
         "moe_block": {
             "workload": "MoE FFN block (BASELINE configs[3]): 64 tokens, hidden 2048, 128 experts x "
                         "(gate/up 2048->768, down 768->2048) Q4_K, top-8; router, sort, experts, combine; "

@@ -112,12 +112,16 @@ HIPQ_API int hipq_quantize_q8_K(const float *A, int64_t M, int64_t K, int64_t ld
  *  form of gemm_q4_0 / gemm_q4_K / gemm_q6_K (x86_compute_backend.cpp:301-341)
  *  as reached from FloatTensor::dotQnK (float_tensor.cpp:923-969). M == 1 runs
  *  the decode GEMV kernels, M > 1 the prefill GEMM kernels. lda >= K and
- *  ldc >= N are row strides in elements. */
+ *  ldc >= N are row strides in elements. With M == 1, K <= 4096, N < 32768 and
+ *  device memory the call is a single kernel launch (the GEMV quantizes the row
+ *  itself) and uses no workspace. */
 HIPQ_API int hipq_matmul(hipq_weight_t w, const float *A, int64_t M, int64_t lda,
                          float *C, int64_t ldc, int mem, void *stream);
 
 /** One fp32 activation against several weights sharing K (the QKV layer's
- *  vector dot, float_tensor.cpp:724-798): quantizes A once. */
+ *  vector dot, float_tensor.cpp:724-798): quantizes A once. One row against up to
+ *  four weights of one format (K <= 4096, fewer than 32768 rows together, device
+ *  memory) is a single kernel launch for all of them. */
 HIPQ_API int hipq_matmul_multi(int count, const hipq_weight_t *w, const float *A,
                                int64_t M, int64_t lda, float *const *C,
                                const int64_t *ldc, int mem, void *stream);

@@ -456,6 +456,8 @@ int hipq_matmul_multi(int count, const hipq_weight_t *w, const float *A, int64_t
   }
   if (M == 0) return HIPQ_OK;
   hipStream_t s = (hipStream_t)stream;
+  if (M == 1 && hipq::gemv_fuses_quantizer_multi(count, w, A))
+    return hipq::launch_gemv_fused_multi(count, w, A, C, s);
   /* one quantization per distinct activation format among the weights */
   auto klass = [&](const hipq_weight *x) {
     if (x->dtype == HIPQ_Q4_0) return 0;

@@ -81,15 +81,15 @@ template <int DT> __host__ __device__ constexpr int fused_act_bytes(int K) {
 }
 
 template <int DT, int T, int G>
-__global__ __launch_bounds__(256) void gemv_fused_kernel(WView w, const float *__restrict__ x,
-                                                         float *__restrict__ C) {
+__device__ __forceinline__ void gemv_fused_body(const WView &w, const float *__restrict__ x,
+                                                float *__restrict__ C, int block) {
   typedef GemvCore<DT, T, 1, G, false> E;
   extern __shared__ __attribute__((aligned(16))) uint32_t gemv_lds[];
   const int K = w.K;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   uint8_t *ap = (uint8_t *)gemv_lds;
   uint32_t *lds = gemv_lds + fused_act_bytes<DT>(K) / 4 + wave * GemvLds<DT, 1, G, false>::DWORDS;
-  const int row0 = (blockIdx.x * 4 + wave) * G;
+  const int row0 = (block * 4 + wave) * G;
   const int arow[1] = {0};
 
   /* the row first (it comes from the cache), then the weights: the wait for the row
@@ -162,6 +162,47 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(WView w, const float *_
   hipq_wave_lds_sync();
   const GemvOut o = E::finish(c);
   if (o.valid && row0 + o.g < w.N) C[row0 + o.g] = o.v;
+}
+
+template <int DT, int T, int G>
+__global__ __launch_bounds__(256) void gemv_fused_kernel(WView w, const float *__restrict__ x,
+                                                         float *__restrict__ C) {
+  gemv_fused_body<DT, T, G>(w, x, C, (int)blockIdx.x);
+}
+
+/* Up to four weights of one format and K on the same row, one launch: the
+ * workgroups of weight i are blocks end[i-1] .. end[i]-1 of the grid. */
+constexpr int FUSED_MAXW = 4;
+struct FusedMulti {
+  WView w[FUSED_MAXW];
+  float *C[FUSED_MAXW];
+  int end[FUSED_MAXW];
+};
+template <int DT, int T, int G>
+__global__ __launch_bounds__(256) void gemv_fused_multi_kernel(FusedMulti mw, const float *__restrict__ x) {
+  const int b = (int)blockIdx.x;
+  int i = 0;
+#pragma unroll
+  for (int k = 0; k + 1 < FUSED_MAXW; ++k) i += b >= mw.end[k];
+  const int first = i ? mw.end[i - 1] : 0;
+  gemv_fused_body<DT, T, G>(mw.w[i], x, mw.C[i], b - first);
+}
+
+template <int DT, int T, int G>
+int launch_fused_many(int count, const hipq_weight *const *w, const float *x, float *const *C, hipStream_t s) {
+  FusedMulti mw;
+  int blocks = 0;
+  for (int i = 0; i < FUSED_MAXW; ++i) {
+    const int j = i < count ? i : count - 1;
+    mw.w[i] = wview(w[j]);
+    mw.C[i] = C[j];
+    if (i < count) blocks += (int)((w[i]->N + 4 * G - 1) / (4 * G));
+    mw.end[i] = blocks;
+  }
+  const size_t lds = fused_act_bytes<DT>((int)w[0]->K) + 4 * GemvLds<DT, 1, G, false>::DWORDS * sizeof(uint32_t);
+  hipLaunchKernelGGL((gemv_fused_multi_kernel<DT, T, G>), dim3((unsigned)blocks), dim3(256), lds, s, mw, x);
+  HIPQ_HIP(hipGetLastError());
+  return HIPQ_OK;
 }
 
 template <int DT, int T, int G>
@@ -250,6 +291,22 @@ template <int DT> int launch_fused(const hipq_weight *w, const float *x, float *
   }
 }
 
+template <int DT>
+int launch_fused_multi(int count, const hipq_weight *const *w, const float *x, float *const *C, hipStream_t s) {
+  int64_t n = 0;
+  for (int i = 0; i < count; ++i) n += w[i]->N;
+  const int64_t units = w[0]->K / GemvRec<DT, false>::UNIT;
+  const int g = pick_group(n, 8);
+  if (units < 64) {
+    if (g == 8) return launch_fused_many<DT, 16, 8>(count, w, x, C, s);
+    return launch_fused_many<DT, 16, 4>(count, w, x, C, s);
+  }
+  if (g == 8) return launch_fused_many<DT, 64, 8>(count, w, x, C, s);
+  if (g == 4) return launch_fused_many<DT, 64, 4>(count, w, x, C, s);
+  if (g == 2 || DT == HIPQ_Q4_0) return launch_fused_many<DT, 64, 2>(count, w, x, C, s);
+  return launch_fused_many<DT, 64, 1>(count, w, x, C, s);
+}
+
 /* 2..8 activation rows in one pass (small prefill chunks, leftover rows). */
 template <int DT>
 int launch_mr(const hipq_weight *w, const QAct *qa, int M, int pair_rows, float *C, int64_t ldc,
@@ -286,6 +343,31 @@ int launch_gemv(const hipq_weight *w, const QAct *qa, int M, int pair_rows, floa
  * per cent of the GEMV and every workgroup quantizing the row costs as much. */
 bool gemv_fuses_quantizer(const hipq_weight *w, const float *x) {
   return w->K <= HIPQ_KCHUNK && w->N < 32768 && ((uintptr_t)x & 15) == 0;
+}
+
+bool gemv_fuses_quantizer_multi(int count, const hipq_weight *const *w, const float *x) {
+  if (count < 1 || count > FUSED_MAXW) return false;
+  int64_t n = 0;
+  for (int i = 0; i < count; ++i) {
+    if (w[i]->dtype != w[0]->dtype || w[i]->K != w[0]->K || !gemv_fuses_quantizer(w[i], x)) return false;
+    n += w[i]->N;
+  }
+  return n < 32768;
+}
+
+int launch_gemv_fused_multi(int count, const hipq_weight *const *w, const float *x, float *const *C,
+                            hipStream_t s) {
+  if (!gemv_fuses_quantizer_multi(count, w, x))
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "these matrices do not take the GEMV that quantizes its own row");
+  switch (w[0]->dtype) {
+  case HIPQ_Q4_0:
+    return launch_fused_multi<HIPQ_Q4_0>(count, w, x, C, s);
+  case HIPQ_Q4_K:
+    return launch_fused_multi<HIPQ_Q4_K>(count, w, x, C, s);
+  case HIPQ_Q6_K:
+    return launch_fused_multi<HIPQ_Q6_K>(count, w, x, C, s);
+  }
+  return fail(HIPQ_ERR_INVALID_ARGUMENT, "unknown weight dtype %d", w[0]->dtype);
 }
 
 int launch_gemv_fused(const hipq_weight *w, const float *x, float *C, hipStream_t s) {

@@ -167,6 +167,10 @@ int launch_quantize_q8_K_tiled(const float *A, int64_t M, int64_t K, int64_t lda
 /* one fp32 activation row, quantized inside the GEMV's workgroups (small matrices) */
 bool gemv_fuses_quantizer(const hipq_weight *w, const float *x);
 int launch_gemv_fused(const hipq_weight *w, const float *x, float *C, hipStream_t s);
+/* the same for up to four weights of one format and K, one launch */
+bool gemv_fuses_quantizer_multi(int count, const hipq_weight *const *w, const float *x);
+int launch_gemv_fused_multi(int count, const hipq_weight *const *w, const float *x, float *const *C,
+                            hipStream_t s);
 int launch_gemv(const hipq_weight *w, const QAct *qa, int M, int pair_rows,
                 float *C, int64_t ldc, hipStream_t s);
 

@@ -142,9 +142,9 @@ def test_matmul_multi_shares_quantization(hipq, cr):
                                  (4096, 4096), (8200, 3072), (12288, 4096)])
 def test_decode_row_quantized_in_the_gemv_equals_the_two_launches(hipq, cr, kind, n, k):
     """hipq_matmul with one row on a small matrix runs one kernel whose workgroups
-    quantize the row themselves; the multi-weight entry keeps the quantizer kernel and
-    the GEMV on its blocks. Same arithmetic, so the outputs are the same bits; the
-    oracle pins both."""
+    quantize the row themselves; the multi-weight entry with more than four weights
+    keeps the quantizer kernel and the GEMV on its blocks. Same arithmetic, so the
+    outputs are the same bits; the oracle pins both."""
     import gpu_util as gu
     import torch
     blocks = _weights(cr, kind, n, k, seed=500 + n)
@@ -154,13 +154,78 @@ def test_decode_row_quantized_in_the_gemv_equals_the_two_launches(hipq, cr, kind
         a[0, 256:512] = 0.0   # an all-zero block: scale 0
     w = capi.Weight(kind, n, k, blocks)
     one = gu.gpu_matmul(w, a)
-    two = torch.full((1, n), float("nan"), device="cuda")
-    capi.matmul_multi([w], gu.dev(a), 1, [two], stream=gu.stream())
+    two = [torch.full((1, n), float("nan"), device="cuda") for _ in range(5)]
+    capi.matmul_multi([w] * 5, gu.dev(a), 1, two, stream=gu.stream())
     torch.cuda.synchronize()
     w.destroy()
-    assert np.array_equal(one, two.cpu().numpy())
+    for t in two:
+        assert np.array_equal(one, t.cpu().numpy())
     ref = cr.gemm(cr.oracle(), kind, a, blocks, n)
     assert gu.rel_err(one, ref) <= gu.TOL
+
+
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("k,ns", [(1024, [2048, 1024, 1024]), (1024, [3072, 3072]), (256, [8, 37, 4, 130]),
+                                  (4096, [4096]), (2048, [1000, 6150])])
+def test_decode_row_on_several_weights_is_one_launch_with_the_same_bits(hipq, cr, kind, k, ns):
+    """Up to four weights of one format and K on one row go out as a single launch
+    (Q, K and V, or gate and up, of a decoder layer); the outputs are those of
+    hipq_matmul on each weight."""
+    import gpu_util as gu
+    import torch
+    blocks = [_weights(cr, kind, n, k, seed=700 + n + i) for i, n in enumerate(ns)]
+    ws = [capi.Weight(kind, n, k, b) for n, b in zip(ns, blocks)]
+    a = synth.normal(710 + k, (1, k))
+    outs = [torch.full((1, n), float("nan"), device="cuda") for n in ns]
+    capi.matmul_multi(ws, gu.dev(a), 1, outs, stream=gu.stream())
+    torch.cuda.synchronize()
+    for w, b, n, o in zip(ws, blocks, ns, outs):
+        assert np.array_equal(o.cpu().numpy(), gu.gpu_matmul(w, a))
+        assert gu.rel_err(o.cpu().numpy(), cr.gemm(cr.oracle(), kind, a, b, n)) <= gu.TOL
+    for w in ws:
+        w.destroy()
+
+
+def test_decode_calls_replay_from_a_captured_graph(hipq, cr):
+    """The one-row calls are single kernel launches without allocations, so a caller
+    can capture a decoder layer's FCs in a graph. Every replay, with other work on
+    the device in between, gives the bits of the direct calls."""
+    import gpu_util as gu
+    import torch
+    k, ns = 1024, [2048, 1024, 1024]
+    blocks = [_weights(cr, "q4_0", n, k, seed=800 + i) for i, n in enumerate(ns)]
+    ws = [capi.Weight("q4_0", n, k, b) for n, b in zip(ns, blocks)]
+    wo = capi.Weight("q4_0", k, 2048, _weights(cr, "q4_0", k, 2048, seed=810))
+    x = torch.zeros((1, k), device="cuda")
+    qkv = [torch.zeros((1, n), device="cuda") for n in ns]
+    y = torch.zeros((1, k), device="cuda")
+
+    def layer(stream):
+        capi.matmul_multi(ws, x, 1, qkv, stream=stream)
+        capi.matmul(wo, qkv[0], 1, y, stream=stream)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        layer(side.cuda_stream)          # first calls outside the capture
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        layer(side.cuda_stream)
+    for it in range(4):
+        x.copy_(gu.dev(synth.normal(820 + it, (1, k))))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = [t.clone() for t in qkv] + [y.clone()]
+        scratch = torch.randn(1 << 20, device="cuda").sum()   # other work between the replays
+        layer(torch.cuda.current_stream().cuda_stream)
+        torch.cuda.synchronize()
+        for g, e in zip(got, qkv + [y]):
+            assert torch.equal(g, e), "replay %d differs from the direct calls" % it
+        assert torch.isfinite(scratch)
+    for w in ws + [wo]:
+        w.destroy()
 
 
 @pytest.mark.parametrize("kind,m", [("q4_K", 1), ("q4_K", 40), ("q6_K", 3)])
