@@ -97,6 +97,34 @@ HIPQ_API int hipq_weight_create(int dtype, int layout, int64_t N, int64_t K,
 HIPQ_API int hipq_weight_destroy(hipq_weight_t w);
 HIPQ_API int hipq_weight_dims(hipq_weight_t w, int *dtype, int64_t *N, int64_t *K);
 
+/** One tensor of a weight file in NNTrainer's MODEL_FORMAT_BIN: the file is the
+ *  tensors of the model's graph one after the other with no directory, so the
+ *  caller lists them in graph order (NeuralNetwork::load,
+ *  models/neuralnet.cpp:679-712). dtype HIPQ_Q4_0 / HIPQ_Q4_K / HIPQ_Q6_K: an
+ *  N x K weight this library takes (its size follows from the dims; a Q4_K
+ *  tensor is preceded by its 16-bit quantization scheme, Q4_0 and Q6_K tensors
+ *  are not, neuralnet.cpp:696-703). dtype HIPQ_FILE_SKIP: `bytes` bytes of
+ *  something else (fp32 norms, embeddings, biases). */
+#define HIPQ_FILE_SKIP (-1)
+typedef struct hipq_file_tensor {
+  int dtype;
+  int layout; /* hipq_layout of a weight; NNTrainer writes Q4_0 and Q4_K as X8 */
+  int64_t N, K;
+  int64_t bytes; /* HIPQ_FILE_SKIP only */
+} hipq_file_tensor;
+/** Where each listed tensor's data starts (after a Q4_K tensor's scheme word)
+ *  when the first one starts at `offset`, and where the list ends. Host
+ *  arithmetic only: usable without a device. data_offsets may be NULL. */
+HIPQ_API int hipq_file_layout(int count, const hipq_file_tensor *tensors, int64_t offset,
+                              int64_t *data_offsets, int64_t *end_offset);
+/** Reads the listed tensors from `path` starting at `offset` and creates a
+ *  weight handle for each quantized one (out[i] = NULL for skipped tensors).
+ *  On an error no handle is left behind. A Q4_K tensor whose scheme word says
+ *  Q4_Kx8 (quantizer.h:37) must be listed with HIPQ_LAYOUT_X8. */
+HIPQ_API int hipq_weights_from_file(const char *path, int64_t offset, int count,
+                                    const hipq_file_tensor *tensors, hipq_weight_t *out,
+                                    int64_t *end_offset);
+
 /** Activation quantizer fp32 -> Q8_0, canonical block_q8_0 output (34 B per 32
  *  values), M rows of K values (K % 32 == 0). Replaces nntr_quantize_row_q8_0 /
  *  nntr_quantize_mat_q8_0_4x8 (nntr_ggml_impl_quant.cpp:532-875,

@@ -21,7 +21,7 @@ SYMBOLS = [
     "hipq_init", "hipq_shutdown", "hipq_last_error", "hipq_version", "hipq_weight_nbytes",
     "hipq_weight_create", "hipq_weight_destroy", "hipq_weight_dims", "hipq_quantize_q8_0",
     "hipq_quantize_q8_K", "hipq_matmul", "hipq_matmul_multi", "hipq_moe_forward",
-    "hipq_quantize_weights", "hipq_time_matmul",
+    "hipq_quantize_weights", "hipq_time_matmul", "hipq_file_layout", "hipq_weights_from_file",
 ]
 
 
@@ -29,6 +29,14 @@ class HipqError(RuntimeError):
     def __init__(self, code, msg):
         super().__init__("hipq error %d: %s" % (code, msg))
         self.code = code
+
+
+class FileTensor(C.Structure):
+    _fields_ = [("dtype", C.c_int32), ("layout", C.c_int32), ("N", C.c_int64), ("K", C.c_int64),
+                ("bytes", C.c_int64)]
+
+
+FILE_SKIP = -1
 
 
 class MoeDesc(C.Structure):
@@ -63,6 +71,9 @@ def lib():
         L.hipq_weight_nbytes.argtypes = [i32, i64, i64]
         L.hipq_weight_create.argtypes = [i32, i32, i64, i64, vp, i32, C.POINTER(vp)]
         L.hipq_weight_destroy.argtypes = [vp]
+        L.hipq_file_layout.argtypes = [i32, C.POINTER(FileTensor), i64, C.POINTER(i64), C.POINTER(i64)]
+        L.hipq_weights_from_file.argtypes = [C.c_char_p, i64, i32, C.POINTER(FileTensor), C.POINTER(vp),
+                                             C.POINTER(i64)]
         L.hipq_weight_dims.argtypes = [vp, C.POINTER(i32), C.POINTER(i64), C.POINTER(i64)]
         L.hipq_quantize_q8_0.argtypes = [vp, i64, i64, i64, vp, i32, vp]
         L.hipq_quantize_q8_K.argtypes = [vp, i64, i64, i64, i32, vp, i32, vp]
@@ -125,6 +136,44 @@ class Weight:
             self.destroy()
         except Exception:
             pass
+
+
+def _file_tensors(tensors):
+    """tensors: ("skip", nbytes) or (dtype, n, k[, layout]) in the file's order."""
+    arr = (FileTensor * len(tensors))()
+    for i, t in enumerate(tensors):
+        if t[0] == "skip":
+            arr[i] = FileTensor(FILE_SKIP, 0, 0, 0, t[1])
+        else:
+            arr[i] = FileTensor(DTYPES.get(t[0], t[0]), t[3] if len(t) > 3 else LAYOUT_CANONICAL, t[1], t[2], 0)
+    return arr
+
+
+def file_layout(tensors, offset=0):
+    """Data offset of every listed tensor of a MODEL_FORMAT_BIN file and the end offset."""
+    arr = _file_tensors(tensors)
+    offs = (C.c_int64 * len(tensors))()
+    end = C.c_int64()
+    check(lib().hipq_file_layout(len(tensors), arr, offset, offs, C.byref(end)))
+    return list(offs), end.value
+
+
+def weights_from_file(path, tensors, offset=0):
+    """Weight objects (None for skipped tensors) read from a MODEL_FORMAT_BIN file, and the
+    offset behind the last listed tensor."""
+    arr = _file_tensors(tensors)
+    hs = (C.c_void_p * len(tensors))()
+    end = C.c_int64()
+    check(lib().hipq_weights_from_file(str(path).encode(), offset, len(tensors), arr, hs, C.byref(end)))
+    out = []
+    for t, h in zip(tensors, hs):
+        if t[0] == "skip":
+            out.append(None)
+            continue
+        w = Weight.__new__(Weight)
+        w.dtype, w.n, w.k, w._h = DTYPES.get(t[0], t[0]), t[1], t[2], C.c_void_p(h)
+        out.append(w)
+    return out, end.value
 
 
 def weight_nbytes(dtype, n, k):

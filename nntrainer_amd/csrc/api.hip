@@ -347,6 +347,72 @@ int hipq_weight_create(int dtype, int layout, int64_t N, int64_t K, const void *
   return HIPQ_OK;
 }
 
+int hipq_file_layout(int count, const hipq_file_tensor *tensors, int64_t offset, int64_t *data_offsets,
+                     int64_t *end_offset) {
+  if (count < 0 || (count && !tensors) || offset < 0)
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "bad tensor list");
+  int64_t at = offset;
+  for (int i = 0; i < count; ++i) {
+    const hipq_file_tensor &t = tensors[i];
+    int64_t size;
+    if (t.dtype == HIPQ_FILE_SKIP) {
+      if (t.bytes < 0) return fail(HIPQ_ERR_INVALID_ARGUMENT, "tensor %d: negative size", i);
+      size = t.bytes;
+    } else {
+      size = hipq_weight_nbytes(t.dtype, t.N, t.K);
+      if (size < 0) return (int)size;
+      if (t.dtype == HIPQ_Q4_K) at += 2; /* the scheme word comes first */
+    }
+    if (data_offsets) data_offsets[i] = at;
+    at += size;
+  }
+  if (end_offset) *end_offset = at;
+  return HIPQ_OK;
+}
+
+int hipq_weights_from_file(const char *path, int64_t offset, int count, const hipq_file_tensor *tensors,
+                           hipq_weight_t *out, int64_t *end_offset) {
+  int rc = require_ready();
+  if (rc) return rc;
+  if (!path || !out) return fail(HIPQ_ERR_INVALID_ARGUMENT, "null argument");
+  std::vector<int64_t> at((size_t)(count > 0 ? count : 0));
+  int64_t end = 0;
+  if ((rc = hipq_file_layout(count, tensors, offset, at.data(), &end))) return rc;
+  for (int i = 0; i < count; ++i) out[i] = nullptr;
+  FILE *f = fopen(path, "rb");
+  if (!f) return fail(HIPQ_ERR_INVALID_ARGUMENT, "cannot open %s", path);
+  std::vector<unsigned char> buf;
+  for (int i = 0; i < count && !rc; ++i) {
+    const hipq_file_tensor &t = tensors[i];
+    if (t.dtype == HIPQ_FILE_SKIP) continue;
+    const int64_t size = hipq_weight_nbytes(t.dtype, t.N, t.K);
+    if (t.dtype == HIPQ_Q4_K) {
+      uint16_t scheme = 0;
+      if (fseeko(f, (off_t)(at[i] - 2), SEEK_SET) || fread(&scheme, 2, 1, f) != 1)
+        rc = fail(HIPQ_ERR_INVALID_ARGUMENT, "%s ends before tensor %d", path, i);
+      else if (scheme == 0x03 && t.layout != HIPQ_LAYOUT_X8)
+        rc = fail(HIPQ_ERR_INVALID_ARGUMENT, "tensor %d is stored as Q4_Kx8 but listed as canonical", i);
+      if (rc) break;
+    }
+    buf.resize((size_t)size);
+    if (fseeko(f, (off_t)at[i], SEEK_SET) || fread(buf.data(), 1, (size_t)size, f) != (size_t)size) {
+      rc = fail(HIPQ_ERR_INVALID_ARGUMENT, "%s ends before the end of tensor %d", path, i);
+      break;
+    }
+    rc = hipq_weight_create(t.dtype, t.layout, t.N, t.K, buf.data(), HIPQ_MEM_HOST, &out[i]);
+  }
+  fclose(f);
+  if (rc) {
+    for (int i = 0; i < count; ++i) {
+      if (out[i]) (void)hipq_weight_destroy(out[i]);
+      out[i] = nullptr;
+    }
+    return rc;
+  }
+  if (end_offset) *end_offset = end;
+  return HIPQ_OK;
+}
+
 int hipq_weight_destroy(hipq_weight_t w) {
   if (!w) return HIPQ_OK;
   int rc = require_ready();

@@ -34,6 +34,35 @@ def test_weight_size_rules():
         assert e.value.code == -1
 
 
+def test_model_file_offsets_follow_the_reference_rule():
+    """MODEL_FORMAT_BIN is the graph's tensors back to back; only tensors with
+    quantization parameters other than Q4_0 / Q6_K carry a 16-bit scheme word in front
+    (models/neuralnet.cpp:696-703). Host arithmetic: no device needed."""
+    tensors = [("skip", 151936 * 1024 * 4),            # fp32 embedding
+               ("skip", 1024 * 4),                     # a norm's gamma
+               ("q4_0", 2048, 1024, capi.LAYOUT_X8),
+               ("q4_K", 3072, 1024, capi.LAYOUT_X8),
+               ("q4_K", 1024, 3072, capi.LAYOUT_X8),
+               ("q6_K", 151936, 1024)]
+    offs, end = capi.file_layout(tensors, offset=16)
+    want, at = [], 16
+    for t in tensors:
+        if t[0] == "skip":
+            want.append(at)
+            at += t[1]
+            continue
+        if t[0] == "q4_K":
+            at += 2
+        want.append(at)
+        at += capi.weight_nbytes(t[0], t[1], t[2])
+    assert offs == want and end == at
+    assert capi.file_layout([], offset=5) == ([], 5)
+    with pytest.raises(capi.HipqError):
+        capi.file_layout([("q4_K", 8, 100)])
+    with pytest.raises(capi.HipqError):
+        capi.file_layout([("skip", -1)])
+
+
 def test_no_gpu_means_loud_failure():
     import torch
     if torch.cuda.is_available():
@@ -45,6 +74,9 @@ def test_no_gpu_means_loud_failure():
     with pytest.raises(capi.HipqError) as e:
         capi.Weight("q4_0", 8, 32, blocks)
     assert e.value.code == -2  # HIPQ_ERR_NOT_INITIALIZED: nothing computes without the device
+    with pytest.raises(capi.HipqError) as e:
+        capi.weights_from_file("/nonexistent", [("q4_0", 8, 32)])
+    assert e.value.code == -2
 
 
 def test_product_never_imports_the_oracle():

@@ -228,6 +228,42 @@ def test_decode_calls_replay_from_a_captured_graph(hipq, cr):
         w.destroy()
 
 
+def test_weights_read_from_a_model_file(hipq, cr, tmp_path):
+    """A file laid out as NNTrainer writes MODEL_FORMAT_BIN (tensors back to back, Q4_0 and
+    Q4_K in the 8-row interleave, a scheme word in front of Q4_K only): the handles read
+    from it multiply like handles made from the same bytes."""
+    import gpu_util as gu
+    specs = [("q4_0", 512, 1024), ("q4_K", 256, 512), ("q6_K", 384, 256), ("q4_K", 128, 256)]
+    blocks = [_weights(cr, kind, n, k, seed=900 + i) for i, (kind, n, k) in enumerate(specs)]
+    stored = [cr.repack_x8(cr.oracle(), kind, b, n, k) if kind != "q6_K" else b
+              for (kind, n, k), b in zip(specs, blocks)]
+    path = tmp_path / "model.bin"
+    listing = [("skip", 4096)]
+    with open(path, "wb") as f:
+        f.write(b"\0" * 7)                            # the caller's start offset
+        f.write(np.arange(1024, dtype=np.float32).tobytes())
+        for (kind, n, k), b in zip(specs, stored):
+            if kind == "q4_K":
+                f.write(np.uint16(3).tobytes())       # QScheme::Q4_Kx8
+            f.write(np.ascontiguousarray(b).tobytes())
+            listing.append((kind, n, k, capi.LAYOUT_X8 if kind != "q6_K" else capi.LAYOUT_CANONICAL))
+        f.write(b"tail")
+    ws, end = capi.weights_from_file(path, listing, offset=7)
+    assert ws[0] is None and end == path.stat().st_size - 4
+    for w, (kind, n, k), b in zip(ws[1:], specs, blocks):
+        a = synth.normal(910 + n, (3, k))
+        ref = capi.Weight(kind, n, k, b)
+        assert np.array_equal(gu.gpu_matmul(w, a), gu.gpu_matmul(ref, a))
+        ref.destroy()
+        w.destroy()
+    # a Q4_Kx8 tensor listed as canonical, and a file that ends early, leave no handle behind
+    with pytest.raises(capi.HipqError):
+        capi.weights_from_file(path, [("skip", 4096), ("q4_0", 512, 1024, capi.LAYOUT_X8), ("q4_K", 256, 512)],
+                               offset=7)
+    with pytest.raises(capi.HipqError):
+        capi.weights_from_file(path, listing + [("q6_K", 4096, 4096)], offset=7)
+
+
 @pytest.mark.parametrize("kind,m", [("q4_K", 1), ("q4_K", 40), ("q6_K", 3)])
 def test_matmul_multi_other_formats_and_prefill(hipq, cr, kind, m):
     """The multi-weight entry with the Q8_K formats, one row and a prefill chunk (the
