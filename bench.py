@@ -283,8 +283,37 @@ def main():
         torch.cuda.synchronize()
         return ev0.elapsed_time(ev1) / reps, n_active
 
+    def moe_graph_time(tokens, reps=20):
+        """The same from a captured graph of one call per expert set: the device's time
+        without the host's share of the launches."""
+        x_, l_, y_ = mx[:tokens], ml[:tokens], my[:tokens]
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):   # the first call on a stream allocates its workspace
+            capi.moe_forward(tokens, mh, mi, me, mk, sets[0], None, None, x_, y_, router_logits=l_,
+                             stream=side.cuda_stream)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            for st_ in sets:
+                capi.moe_forward(tokens, mh, mi, me, mk, st_, None, None, x_, y_, router_logits=l_,
+                                 stream=side.cuda_stream)
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record()
+        for _ in range(reps):
+            graph.replay()
+        ev1.record()
+        torch.cuda.synchronize()
+        return ev0.elapsed_time(ev1) / (reps * len(sets))
+
     moe_ms, active = moe_time(mt)
+    moe_graph_ms = moe_graph_time(mt)
     moe_decode_ms, decode_active = moe_time(1)
+    moe_decode_graph_ms = moe_graph_time(1)
     moe_bytes = active * 3 * (mi * mh * 144 // 256) + 2 * mt * mh * 4
     moe_gbs = moe_bytes / (moe_ms * 1e-3) / 1e9
     moe_decode_bytes = decode_active * 3 * (mi * mh * 144 // 256) + 2 * mh * 4
@@ -352,11 +381,14 @@ def main():
             "workload": "MoE FFN block (BASELINE configs[3]): 64 tokens, hidden 2048, 128 experts x "
                         "(gate/up 2048->768, down 768->2048) Q4_K, top-8; router, sort, experts, combine; "
                         "two expert sets alternated; whole call incl. launches",
-            "ms_per_block": round(moe_ms, 5), "active_experts": active,
+            "ms_per_block": round(moe_ms, 5), "ms_per_block_in_a_graph": round(moe_graph_ms, 5),
+            "active_experts": active,
             "roofline": {"bound": "hbm", "achieved": round(moe_gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(moe_gbs / HBM_PEAK_GBS, 5), "algorithmic_bytes_per_block": moe_bytes,
                          "traffic": 236.4e6 + 124.9e6 + 13.0e6},
-            "decode_token": {"ms_per_block": round(moe_decode_ms, 5), "active_experts": decode_active,
+            "decode_token": {"ms_per_block": round(moe_decode_ms, 5),
+                             "ms_per_block_in_a_graph": round(moe_decode_graph_ms, 5),
+                             "active_experts": decode_active,
                              "gbs": round(moe_decode_bytes / (moe_decode_ms * 1e-3) / 1e9, 2)}},
     }
     if not args.no_cpu:

@@ -138,6 +138,47 @@ def test_expert_weights_serve_the_moe_block_only(hipq, cr):
         w.destroy()
 
 
+@pytest.mark.parametrize("t", [1, 24])
+def test_moe_block_replays_from_a_captured_graph(hipq, cr, t):
+    """After a first call (which builds the expert table and the workspace) the block is
+    kernel launches only: a caller can capture it. Every replay, with new inputs and
+    other work in between, gives the bits of a direct call."""
+    import gpu_util as gu
+    import torch
+    h, i, e, k = 512, 256, 16, 4
+    gate, up, down = _experts(cr, e, i, h, seed=1500)
+    ex = capi.Experts([capi.Weight("q4_K", i, h, b) for b in gate], [capi.Weight("q4_K", i, h, b) for b in up],
+                      [capi.Weight("q4_K", h, i, b) for b in down])
+    x = torch.zeros((t, h), device="cuda")
+    logits = torch.zeros((t, e), device="cuda")
+    y = torch.zeros((t, h), device="cuda")
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        capi.moe_forward(t, h, i, e, k, ex, None, None, x, y, router_logits=logits, stream=side.cuda_stream)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        capi.moe_forward(t, h, i, e, k, ex, None, None, x, y, router_logits=logits, stream=side.cuda_stream)
+    for it in range(4):
+        x.copy_(gu.dev(synth.normal(1510 + it, (t, h))))
+        logits.copy_(gu.dev(synth.normal(1520 + it, (t, e))))
+        graph.replay()
+        torch.cuda.synchronize()
+        got = y.clone()
+        other = torch.randn(1 << 20, device="cuda").sum()
+        y.fill_(float("nan"))
+        capi.moe_forward(t, h, i, e, k, ex, None, None, x, y, router_logits=logits, stream=gu.stream())
+        torch.cuda.synchronize()
+        assert torch.equal(got, y), "replay %d differs from the direct call" % it
+        assert torch.isfinite(other)
+    del graph
+    for ws in ex.weights:
+        for w in ws:
+            w.destroy()
+
+
 def test_moe_router_weight_path(hipq, cr):
     """Logits computed on the device from the fp32 router weight."""
     import gpu_util as gu
