@@ -841,11 +841,15 @@ __global__ __launch_bounds__(256, TC <= 8 ? 4 : TC <= 16 ? 2 : 1) void gate_up_m
   }
 }
 
-template <int TC>
+/* QH: the rows of h come as fp32 (hf) and the workgroup quantizes those of its item
+ * itself while its first weights are on their way, with the quantizer kernel's
+ * arithmetic. Every column workgroup of an item repeats that, which pays with few
+ * items (a decode step: one launch less), not with many. */
+template <int TC, bool QH>
 __global__ __launch_bounds__(256, TC <= 8 ? 4 : TC <= 16 ? 2 : 1) void down_mma_kernel(
-  const WView *__restrict__ views, int E_, QView hq, const int *__restrict__ offsets,
-  const int *__restrict__ items, const int *__restrict__ slot_pair, const float *__restrict__ wgt, int H,
-  float *__restrict__ contrib, int ct) {
+  const WView *__restrict__ views, int E_, QView hq, const float *__restrict__ hf,
+  const int *__restrict__ offsets, const int *__restrict__ items, const int *__restrict__ slot_pair,
+  const float *__restrict__ wgt, int H, float *__restrict__ contrib, int ct) {
   constexpr int NREG = TC / 2;
   extern __shared__ __attribute__((aligned(16))) unsigned char xmoe_lds[];
   const int item = blockIdx.y;
@@ -859,6 +863,20 @@ __global__ __launch_bounds__(256, TC <= 8 ? 4 : TC <= 16 ? 2 : 1) void down_mma_
   const int col0 = (blockIdx.x * 4 + wave) * 32 * ct;
   const int ntile = min(ct, (H - col0 + 31) / 32);
   auto stage = [&]() {
+    if (QH) {
+      /* rows past the item's end stay as they are: a row of the matrix product
+       * depends on its own activations only, and those rows are not stored */
+      const int nsb = K >> 8;
+      for (int u = wave; u < (end - s0) * nsb; u += 4) { /* uniform per wavefront */
+        const int r = u / nsb, b = u - r * nsb;
+        const float4 xv = *(const float4 *)(hf + (size_t)(s0 + r) * K + b * 256 + lane * 4);
+        hipq_quantize_q8_K_values<Q8K_ROWMMA>(xv, 0, b, b, nsb, 0, l.q + (size_t)r * (K + 16), l.dA + r, nullptr,
+                                              nullptr, (uint16_t *)(l.amin + (size_t)r * nsb * 32), nullptr,
+                                              nullptr, TC);
+      }
+      __syncthreads();
+      return;
+    }
     if (threadIdx.x < TC) l.rows[threadIdx.x] = min(s0 + (int)threadIdx.x, end - 1); /* hq rows are slots */
     __syncthreads();
     stage_rows<TC>(l, hq);
@@ -1004,15 +1022,21 @@ int launch_grouped_mma(const hipq::MoeArgs *a, const MoeBufs &b, const WView *vi
                        lds_g, s, views, d.experts, qview(xq), b.offsets, b.items, b.slot_pair, d.topk,
                        d.intermediate, b.h);
   HIPQ_HIP(hipGetLastError());
-  int rc = hipq::launch_quantize_q8_K_rowmma(b.h, P, d.intermediate, d.intermediate, &hq, s);
-  if (rc) return rc;
+  if (!few) {
+    int rc = hipq::launch_quantize_q8_K_rowmma(b.h, P, d.intermediate, d.intermediate, &hq, s);
+    if (rc) return rc;
+  }
+  const void *kd = few ? (const void *)down_mma_kernel<TC, true> : (const void *)down_mma_kernel<TC, false>;
   if (lds_d > 64 * 1024)
-    HIPQ_HIP(hipFuncSetAttribute((const void *)down_mma_kernel<TC>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                 (int)lds_d));
+    HIPQ_HIP(hipFuncSetAttribute(kd, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_d));
   const int ct = few ? 1 : 2;
-  hipLaunchKernelGGL((down_mma_kernel<TC>), dim3((d.hidden + 128 * ct - 1) / (128 * ct), max_items), dim3(256),
-                     lds_d, s, views, d.experts, qview(hq), b.offsets, b.items, b.slot_pair, b.wgt, d.hidden,
-                     b.contrib, ct);
+  const dim3 gd((d.hidden + 128 * ct - 1) / (128 * ct), max_items);
+  if (few)
+    hipLaunchKernelGGL((down_mma_kernel<TC, true>), gd, dim3(256), lds_d, s, views, d.experts, qview(hq), b.h,
+                       b.offsets, b.items, b.slot_pair, b.wgt, d.hidden, b.contrib, ct);
+  else
+    hipLaunchKernelGGL((down_mma_kernel<TC, false>), gd, dim3(256), lds_d, s, views, d.experts, qview(hq), b.h,
+                       b.offsets, b.items, b.slot_pair, b.wgt, d.hidden, b.contrib, ct);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
 }

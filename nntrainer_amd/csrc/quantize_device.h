@@ -58,12 +58,14 @@ enum {
 
 /* Super-block sb = (row m, block b) by the calling wavefront (all 64 lanes), lane l
  * holding its values 4l .. 4l+3 in xv. Rows below mat_rows take the 4-row
- * quantizer's semantics, the others the row quantizer's. */
+ * quantizer's semantics, the others the row quantizer's. d_stride: distance of
+ * consecutive super-blocks' scales in d_out (the row form only). */
 template <int MODE>
 __device__ __forceinline__ void hipq_quantize_q8_K_values(
   const float4 &xv, int64_t m, int b, int64_t sb, int nsb, int64_t mat_rows, int8_t *__restrict__ q_out,
   float *__restrict__ d_out, int16_t *__restrict__ bsum_out, uint8_t *__restrict__ canon_out,
-  uint16_t *__restrict__ amin_out, uint16_t *__restrict__ ql_out, uint16_t *__restrict__ qh_out) {
+  uint16_t *__restrict__ amin_out, uint16_t *__restrict__ ql_out, uint16_t *__restrict__ qh_out,
+  int d_stride = 1) {
   const int lane = threadIdx.x & 63;
   const float x[4] = {xv.x, xv.y, xv.z, xv.w};
 
@@ -144,7 +146,7 @@ __device__ __forceinline__ void hipq_quantize_q8_K_values(
     int8_t *o = q_out + sb * 256 + (lane >> 2) * 16 + (lane & 3) * 2;
     *(uint16_t *)o = (uint16_t)((q[0] & 0xff) | ((q[2] & 0xff) << 8));
     *(uint16_t *)(o + 8) = (uint16_t)((q[1] & 0xff) | ((q[3] & 0xff) << 8));
-    if (lane == 0) d_out[sb] = d;
+    if (lane == 0) d_out[sb * d_stride] = d;
     const int bs = gsum + __shfl_xor(gsum, 4, HIPQ_WAVE); /* two 16-value groups = one sub-block */
     if ((lane & 7) == 0) {
       const int l6 = bs & 63;
