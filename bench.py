@@ -385,7 +385,7 @@ def main():
             "active_experts": active,
             "roofline": {"bound": "hbm", "achieved": round(moe_gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(moe_gbs / HBM_PEAK_GBS, 5), "algorithmic_bytes_per_block": moe_bytes,
-                         "traffic": 236.4e6 + 124.9e6 + 13.0e6},
+                         "traffic": 236.2e6 + 123.4e6 + 13.0e6},
             "decode_token": {"ms_per_block": round(moe_decode_ms, 5),
                              "ms_per_block_in_a_graph": round(moe_decode_graph_ms, 5),
                              "active_experts": decode_active,
