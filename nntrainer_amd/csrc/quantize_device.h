@@ -29,6 +29,17 @@ __device__ __forceinline__ int pack4(int a, int b, int c, int d) {
   return (a & 0xff) | ((b & 0xff) << 8) | ((c & 0xff) << 16) | ((d & 0xff) << 24);
 }
 
+/* The 16-byte matrix operand of a 16-value group, from the four lanes of a quad that
+ * hold its values 4i .. 4i+3 each (q[0..3] of lane i): the 8 even values first, then
+ * the 8 odd ones. Every lane of the quad returns the whole operand. */
+__device__ __forceinline__ uint4 hipq_quad_operand(const int (&q)[4]) {
+  const int mine = (q[0] & 0xff) | ((q[2] & 0xff) << 8) | ((q[1] & 0xff) << 16) | ((q[3] & 0xff) << 24);
+  const uint32_t d0 = (uint32_t)hipq_dpp_i<0x00>(mine), d1 = (uint32_t)hipq_dpp_i<0x55>(mine);
+  const uint32_t d2 = (uint32_t)hipq_dpp_i<0xAA>(mine), d3 = (uint32_t)hipq_dpp_i<0xFF>(mine);
+  return make_uint4((d0 & 0xffffu) | (d1 << 16), (d2 & 0xffffu) | (d3 << 16), (d0 >> 16) | (d1 & 0xffff0000u),
+                    (d2 >> 16) | (d3 & 0xffff0000u));
+}
+
 /* Q8_0: the calling lane holds four consecutive values of a 32-value block, the
  * eight lanes of the block are consecutive. Returns the lane's four int8 values
  * packed; dh = the block's fp16 scale. */
@@ -129,9 +140,9 @@ __device__ __forceinline__ void hipq_quantize_q8_K_values(
     const int jb = lane >> 3, g = jb >> 2;
     const int st = 2 * (jb & 3) + ((lane >> 2) & 1);
     const int64_t tile = (mt * (2 * nsb) + b * 2 + (st >> 2)) * 16384;
-    const int off = ((r >> 5) * 4 + (st & 3)) * 1024 + (g * 32 + (r & 31)) * 16 + (lane & 3) * 2;
-    *(uint16_t *)(q_out + tile + off) = (uint16_t)((q[0] & 0xff) | ((q[2] & 0xff) << 8));
-    *(uint16_t *)(q_out + tile + off + 8) = (uint16_t)((q[1] & 0xff) | ((q[3] & 0xff) << 8));
+    const int off = ((r >> 5) * 4 + (st & 3)) * 1024 + (g * 32 + (r & 31)) * 16;
+    const uint4 op = hipq_quad_operand(q); /* one 16-byte store per quad instead of eight of 2 bytes */
+    if ((lane & 3) == 0) *(uint4 *)(q_out + tile + off) = op;
     const int64_t rb = (mt * nsb + b) * 128 + r;
     if (lane == 0) d_out[rb] = d;
     const int bs = gsum + __shfl_xor(gsum, 4, HIPQ_WAVE); /* two 16-value groups = one sub-block */
@@ -143,9 +154,8 @@ __device__ __forceinline__ void hipq_quantize_q8_K_values(
   } else if (MODE == Q8K_ROWMMA) {
     /* row-major, each 16-value group stored as its 8 even then its 8 odd values:
      * this lane's four values are elements 4l .. 4l+3 of group lane / 4 */
-    int8_t *o = q_out + sb * 256 + (lane >> 2) * 16 + (lane & 3) * 2;
-    *(uint16_t *)o = (uint16_t)((q[0] & 0xff) | ((q[2] & 0xff) << 8));
-    *(uint16_t *)(o + 8) = (uint16_t)((q[1] & 0xff) | ((q[3] & 0xff) << 8));
+    const uint4 op = hipq_quad_operand(q);
+    if ((lane & 3) == 0) *(uint4 *)(q_out + sb * 256 + (lane >> 2) * 16) = op;
     if (lane == 0) d_out[sb * d_stride] = d;
     const int bs = gsum + __shfl_xor(gsum, 4, HIPQ_WAVE); /* two 16-value groups = one sub-block */
     if ((lane & 7) == 0) {
