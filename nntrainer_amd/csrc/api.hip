@@ -31,6 +31,10 @@ thread_local char tl_error[768] = "";
 struct Workspace {
   void *ptr = nullptr;
   size_t bytes = 0;
+  /* held while a call enqueues its launches: two threads that name the same stream
+   * must not interleave their kernels (the second would quantize into the scratch
+   * the first one's product has not read yet) */
+  std::recursive_mutex enqueue;
 };
 
 struct MoeTable {
@@ -97,6 +101,12 @@ int workspace(hipStream_t s, size_t bytes, void **out) {
   *out = w.ptr;
   return HIPQ_OK;
 }
+
+std::recursive_mutex &enqueue_lock(hipStream_t s) {
+  std::lock_guard<std::mutex> lk(g.mu);
+  return g.ws[s].enqueue; /* nodes of the map do not move */
+}
+typedef std::lock_guard<std::recursive_mutex> EnqueueGuard;
 
 bool dtype_ok(int dt) { return dt == HIPQ_Q4_0 || dt == HIPQ_Q4_K || dt == HIPQ_Q6_K; }
 int64_t block_elems(int dt) { return dt == HIPQ_Q4_0 ? 32 : 256; }
@@ -490,6 +500,7 @@ int hipq_matmul(hipq_weight_t w, const float *A, int64_t M, int64_t lda, float *
   if (rc) return rc;
   if ((rc = check_matmul_args(w, A, M, lda, C, ldc))) return rc;
   hipStream_t s = (hipStream_t)stream;
+  EnqueueGuard eg(enqueue_lock(s));
   if (mem == HIPQ_MEM_DEVICE) return matmul_device(w, A, M, lda, C, ldc, s);
   if (mem != HIPQ_MEM_HOST) return fail(HIPQ_ERR_INVALID_ARGUMENT, "unknown mem kind %d", mem);
   if (M == 0) return HIPQ_OK;
@@ -522,6 +533,7 @@ int hipq_matmul_multi(int count, const hipq_weight_t *w, const float *A, int64_t
   }
   if (M == 0) return HIPQ_OK;
   hipStream_t s = (hipStream_t)stream;
+  EnqueueGuard eg(enqueue_lock(s));
   if (M == 1 && hipq::gemv_fuses_quantizer_multi(count, w, A))
     return hipq::launch_gemv_fused_multi(count, w, A, C, s);
   /* one quantization per distinct activation format among the weights */
@@ -571,6 +583,7 @@ int hipq_time_matmul(int n_weights, const hipq_weight_t *w, const float *A, int6
       return fail(HIPQ_ERR_INVALID_ARGUMENT, "timed weights must share dtype and K");
   }
   hipStream_t s = (hipStream_t)stream;
+  EnqueueGuard eg(enqueue_lock(s));
   const int is_k = w[0]->dtype != HIPQ_Q4_0;
   bool tiled = true;
   for (int i = 0; i < n_weights; ++i) tiled = tiled && wants_tiled(w[i], M);
@@ -641,6 +654,7 @@ int hipq_moe_forward(const hipq_moe_desc *desc, const hipq_weight_t *gate, const
   }
   if (d.tokens == 0) return HIPQ_OK;
   hipStream_t s = (hipStream_t)stream;
+  EnqueueGuard eg(enqueue_lock(s));
 
   /* device table of the 3E weight views, rebuilt only when the handles change */
   WView *dev_views = nullptr;

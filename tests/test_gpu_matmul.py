@@ -234,6 +234,53 @@ def test_decode_calls_replay_from_a_captured_graph(hipq, cr):
         w.destroy()
 
 
+@pytest.mark.parametrize("own_streams", [False, True])
+def test_calls_from_several_threads(hipq, cr, own_streams):
+    """The entry points are called from several threads (the reference's expert loop
+    runs Tensor::dot inside an OpenMP loop, qwen_moe_layer.cpp:478-490; model load uses a
+    thread per node). Calls that name the same stream share its scratch: their launches
+    must not interleave. Every result equals the one a single thread gets."""
+    import threading
+    import gpu_util as gu
+    import torch
+    n, k = 384, 512
+    ws = {kind: capi.Weight(kind, n, k, _weights(cr, kind, n, k, seed=950)) for kind in ("q4_0", "q4_K")}
+    cases = [(kind, m) for kind in ws for m in (1, 5, 40)]
+    acts = {m: gu.dev(synth.normal(960 + m, (m, k))) for m in (1, 5, 40)}
+    want = {}
+    for kind, m in cases:
+        c = torch.empty((m, n), device="cuda")
+        capi.matmul(ws[kind], acts[m], m, c, stream=gu.stream())
+        torch.cuda.synchronize()
+        want[(kind, m)] = c.clone()
+    errors = []
+
+    def work(tid):
+        try:
+            st = torch.cuda.Stream() if own_streams else torch.cuda.current_stream()
+            outs = {cs: torch.empty((cs[1], n), device="cuda") for cs in cases}
+            for it in range(25):
+                for kind, m in cases[tid % 2:] + cases[:tid % 2]:
+                    capi.matmul(ws[kind], acts[m], m, outs[(kind, m)], stream=st.cuda_stream)
+                st.synchronize()
+                for cs in cases:
+                    if not torch.equal(outs[cs], want[cs]):
+                        errors.append((tid, it, cs))
+                        return
+        except Exception as e:  # noqa: BLE001 - reported below
+            errors.append((tid, repr(e)))
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(4)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    torch.cuda.synchronize()
+    for w in ws.values():
+        w.destroy()
+    assert not errors, errors[:3]
+
+
 def test_weights_read_from_a_model_file(hipq, cr, tmp_path):
     """A file laid out as NNTrainer writes MODEL_FORMAT_BIN (tensors back to back, Q4_0 and
     Q4_K in the 8-row interleave, a scheme word in front of Q4_K only): the handles read
