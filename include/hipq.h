@@ -146,6 +146,20 @@ HIPQ_API int hipq_quantize_q8_K(const float *A, int64_t M, int64_t K, int64_t ld
 HIPQ_API int hipq_matmul(hipq_weight_t w, const float *A, int64_t M, int64_t lda,
                          float *C, int64_t ldc, int mem, void *stream);
 
+/** hipq_matmul on device buffers for callers that cannot allocate device memory:
+ *  code under HIP graph capture, tight serving loops, harnesses that forbid it.
+ *  It has no counterpart in the reference. The quantized activations of the call
+ *  live in a fixed array of 16 MiB inside the library's device code (each GPU the
+ *  library runs on holds one until the process ends) instead of the per-stream
+ *  workspace that hipq_matmul grows on demand; a call that needs more
+ *  (M * K beyond about 7.8 million values for Q6_K weights, 14 million for Q4_0
+ *  and Q4_K) returns HIPQ_ERR_NOT_SUPPORTED. The call performs no device
+ *  allocation and no free and enqueues the same kernels as hipq_matmul, so
+ *  results are the same bits. All calls on a GPU share that one array: calls
+ *  whose kernels may overlap on the device (different streams) race on it. */
+HIPQ_API int hipq_matmul_noalloc(hipq_weight_t w, const float *A, int64_t M, int64_t lda,
+                                 float *C, int64_t ldc, void *stream);
+
 /** One fp32 activation against several weights sharing K (the QKV layer's
  *  vector dot, float_tensor.cpp:724-798): quantizes A once. One row against up to
  *  four weights of one format (K <= 4096, fewer than 32768 rows together, device

@@ -24,6 +24,14 @@
 
 #include "hipq_internal.h"
 
+/* Scratch of hipq_matmul_noalloc: quantized activations of one call. Every GPU the
+ * library runs on holds its own copy of the array at its own address until the
+ * process ends; in host code the array's name is only a stand-in, the address
+ * comes from hipGetSymbolAddress with that device current (hipq_init). */
+constexpr size_t NOALLOC_SCRATCH_BYTES = (size_t)16 << 20;
+constexpr int MAX_DEVICES = 64;
+static __device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];
+
 namespace {
 
 thread_local char tl_error[768] = "";
@@ -46,6 +54,8 @@ struct State {
   std::mutex mu;
   bool ready = false;
   int device = -1;
+  void *scratch_ptr[MAX_DEVICES] = {}; /* device address of `scratch`, per device */
+  std::recursive_mutex noalloc_enqueue; /* calls that share the scratch submit one at a time */
   std::unordered_map<hipStream_t, Workspace> ws;
   /* one table of expert weight views per MoE layer, found by its first gate weight */
   std::unordered_map<const hipq_weight *, MoeTable> moe_tables;
@@ -133,8 +143,25 @@ bool wants_tiled(const hipq_weight *w, int64_t M) {
   return w->dtype == HIPQ_Q4_K && M > 8 && w->N * (w->K / 2) < (int64_t(1) << 32);
 }
 
+/* Where a call's quantized activations go: the per-stream workspace (grown on
+ * demand) or, for the entry point that may not allocate, the static scratch. */
+struct Scratch {
+  bool fixed;
+  hipStream_t s;
+  int get(size_t bytes, void **out) const {
+    if (!fixed) return workspace(s, bytes, out);
+    if (bytes > NOALLOC_SCRATCH_BYTES)
+      return fail(HIPQ_ERR_NOT_SUPPORTED,
+                  "this matmul needs %zu bytes of scratch for its quantized activations; the "
+                  "allocation-free entry point holds %zu",
+                  bytes, NOALLOC_SCRATCH_BYTES);
+    *out = g.scratch_ptr[g.device];
+    return HIPQ_OK;
+  }
+};
+
 int matmul_tiled(const hipq_weight *w, const float *A, int64_t M, int64_t lda, float *C, int64_t ldc,
-                 hipStream_t s, int phase);
+                 hipStream_t s, int phase, const Scratch &sc);
 
 /* Quantize the activations the way the reference does for this weight type. */
 int quantize_for(const hipq_weight *w, const float *A, int64_t M, int64_t lda, const QAct &qa,
@@ -175,9 +202,9 @@ int check_matmul_args(hipq_weight_t w, const float *A, int64_t M, int64_t lda, c
 
 /* phase: 0 quantizer + GEMM, 1 GEMM only (activations from the previous call), 2 quantizer only */
 int matmul_tiled(const hipq_weight *w, const float *A, int64_t M, int64_t lda, float *C, int64_t ldc,
-                 hipStream_t s, int phase) {
+                 hipStream_t s, int phase, const Scratch &sc) {
   void *mem = nullptr;
-  int rc = workspace(s, qact_tiled_bytes(M, w->K), &mem);
+  int rc = sc.get(qact_tiled_bytes(M, w->K), &mem);
   if (rc) return rc;
   QActTiled qa = qact_tiled_carve(mem, M, w->K);
   if (phase != 1) rc = hipq::launch_quantize_q8_K_tiled(A, M, w->K, lda, (M / 4) * 4, &qa, s);
@@ -186,13 +213,13 @@ int matmul_tiled(const hipq_weight *w, const float *A, int64_t M, int64_t lda, f
 }
 
 int matmul_device(hipq_weight_t w, const float *A, int64_t M, int64_t lda, float *C, int64_t ldc,
-                  hipStream_t s) {
+                  hipStream_t s, const Scratch &sc) {
   if (M == 0) return HIPQ_OK;
-  if (wants_tiled(w, M)) return matmul_tiled(w, A, M, lda, C, ldc, s, 0);
+  if (wants_tiled(w, M)) return matmul_tiled(w, A, M, lda, C, ldc, s, 0, sc);
   if (M == 1 && hipq::gemv_fuses_quantizer(w, A)) return hipq::launch_gemv_fused(w, A, C, s);
   const int is_k = w->dtype != HIPQ_Q4_0;
   void *mem = nullptr;
-  int rc = workspace(s, qact_bytes(is_k, M, w->K), &mem);
+  int rc = sc.get(qact_bytes(is_k, M, w->K), &mem);
   if (rc) return rc;
   QAct qa = qact_carve(is_k, mem, M, w->K);
   rc = quantize_for(w, A, M, lda, qa, s);
@@ -240,6 +267,12 @@ int hipq_init(int device) {
     return fail(HIPQ_ERR_NOT_SUPPORTED, "device %d is %s; this library is built for gfx950 only",
                 device, prop.gcnArchName);
   HIPQ_HIP(hipSetDevice(device));
+  if (device >= MAX_DEVICES) return fail(HIPQ_ERR_NOT_SUPPORTED, "device index %d is beyond %d", device, MAX_DEVICES - 1);
+  if (!g.scratch_ptr[device]) {
+    void *p = nullptr;
+    HIPQ_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+    g.scratch_ptr[device] = p;
+  }
   g.device = device;
   g.ready = true;
   return HIPQ_OK;
@@ -501,7 +534,8 @@ int hipq_matmul(hipq_weight_t w, const float *A, int64_t M, int64_t lda, float *
   if ((rc = check_matmul_args(w, A, M, lda, C, ldc))) return rc;
   hipStream_t s = (hipStream_t)stream;
   EnqueueGuard eg(enqueue_lock(s));
-  if (mem == HIPQ_MEM_DEVICE) return matmul_device(w, A, M, lda, C, ldc, s);
+  const Scratch sc{false, s};
+  if (mem == HIPQ_MEM_DEVICE) return matmul_device(w, A, M, lda, C, ldc, s, sc);
   if (mem != HIPQ_MEM_HOST) return fail(HIPQ_ERR_INVALID_ARGUMENT, "unknown mem kind %d", mem);
   if (M == 0) return HIPQ_OK;
   DevBuf dA, dC;
@@ -509,12 +543,24 @@ int hipq_matmul(hipq_weight_t w, const float *A, int64_t M, int64_t lda, float *
   if ((rc = dC.alloc((size_t)M * w->N * 4))) return rc;
   HIPQ_HIP(hipMemcpy2D(dA.p, (size_t)w->K * 4, A, (size_t)lda * 4, (size_t)w->K * 4, (size_t)M,
                        hipMemcpyHostToDevice));
-  rc = matmul_device(w, (const float *)dA.p, M, w->K, (float *)dC.p, w->N, s);
+  rc = matmul_device(w, (const float *)dA.p, M, w->K, (float *)dC.p, w->N, s, sc);
   if (rc) return rc;
   HIPQ_HIP(hipStreamSynchronize(s));
   HIPQ_HIP(hipMemcpy2D(C, (size_t)ldc * 4, dC.p, (size_t)w->N * 4, (size_t)w->N * 4, (size_t)M,
                        hipMemcpyDeviceToHost));
   return HIPQ_OK;
+}
+
+int hipq_matmul_noalloc(hipq_weight_t w, const float *A, int64_t M, int64_t lda, float *C,
+                        int64_t ldc, void *stream) {
+  int rc = require_ready();
+  if (rc) return rc;
+  if ((rc = check_matmul_args(w, A, M, lda, C, ldc))) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  /* one scratch per GPU: calls submit one at a time; the kernels of two calls on
+   * different streams would still race on it, which is the caller's to avoid */
+  EnqueueGuard eg(g.noalloc_enqueue);
+  return matmul_device(w, A, M, lda, C, ldc, s, Scratch{true, s});
 }
 
 int hipq_matmul_multi(int count, const hipq_weight_t *w, const float *A, int64_t M, int64_t lda,
@@ -546,7 +592,7 @@ int hipq_matmul_multi(int count, const hipq_weight_t *w, const float *A, int64_t
     bool first = true;
     for (int i = 0; i < count; ++i)
       if (klass(w[i]) == 3) {
-        if ((rc = matmul_tiled(w[i], A, M, lda, C[i], ldc[i], s, first ? 0 : 1))) return rc;
+        if ((rc = matmul_tiled(w[i], A, M, lda, C[i], ldc[i], s, first ? 0 : 1, Scratch{false, s}))) return rc;
         first = false;
       }
   }
@@ -590,7 +636,7 @@ int hipq_time_matmul(int n_weights, const hipq_weight_t *w, const float *A, int6
   void *memp = nullptr;
   QAct qa{};
   if (tiled) {
-    if ((rc = matmul_tiled(w[0], A, M, lda, C, ldc, s, 2))) return rc;
+    if ((rc = matmul_tiled(w[0], A, M, lda, C, ldc, s, 2, Scratch{false, s}))) return rc;
   } else {
     if ((rc = workspace(s, qact_bytes(is_k, M, w[0]->K), &memp))) return rc;
     qa = qact_carve(is_k, memp, M, w[0]->K);
@@ -604,7 +650,7 @@ int hipq_time_matmul(int n_weights, const hipq_weight_t *w, const float *A, int6
   for (int it = 0; it < iters && !rc; ++it) {
     const hipq_weight *wi = w[it % n_weights];
     if (tiled) {
-      rc = matmul_tiled(wi, A, M, lda, C, ldc, s, phase);
+      rc = matmul_tiled(wi, A, M, lda, C, ldc, s, phase, Scratch{false, s});
       continue;
     }
     if (phase == 0 && M == 1 && hipq::gemv_fuses_quantizer(wi, A)) {

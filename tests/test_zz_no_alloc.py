@@ -1,0 +1,65 @@
+"""hipq_matmul_noalloc (quantized activations in the library's fixed scratch array, no
+device allocation inside the call) against hipq_matmul on the same inputs, through the
+C ABI. Both enqueue the same kernels, so the outputs must be the same bits. Every case
+makes two calls in a row, the second with a smaller input: the scratch keeps the first
+call's contents and nothing of it may leak into the second result."""
+import numpy as np
+import pytest
+
+from nntrainer_amd import capi, synth
+
+pytestmark = pytest.mark.gpu
+
+
+def _pair(hipq, cr, kind, n, k, m_big, m_small):
+    import torch
+    import gpu_util as gu
+
+    blocks = cr.quantize_weights(cr.oracle(), kind, synth.normal(900 + n, (n, k), 0.02))
+    w = capi.Weight(kind, n, k, blocks)
+    try:
+        for call, m in enumerate((m_big, m_small)):
+            a = synth.normal(910 + 7 * call + m, (m, k))
+            da = gu.dev(a)
+            want = torch.full((m, n), float("nan"), device="cuda", dtype=torch.float32)
+            got = torch.full((m, n), float("nan"), device="cuda", dtype=torch.float32)
+            capi.matmul(w, da, m, want, stream=gu.stream())
+            torch.cuda.synchronize()
+            free_before = torch.cuda.mem_get_info()[0]
+            capi.matmul_noalloc(w, da, m, got, stream=gu.stream())
+            torch.cuda.synchronize()
+            assert torch.cuda.mem_get_info()[0] == free_before, "the call changed the device's free memory"
+            g, r = got.cpu().numpy(), want.cpu().numpy()
+            assert not np.isnan(g).any()
+            assert np.array_equal(g.view(np.uint32), r.view(np.uint32)), (kind, m, gu.rel_err(g, r))
+            if call == 1:
+                ref = cr.gemm(cr.oracle(), kind, a, blocks, n)
+                assert gu.rel_err(g, ref) <= gu.TOL
+    finally:
+        w.destroy()
+
+
+@pytest.mark.parametrize("kind", ["q4_0", "q4_K", "q6_K"])
+@pytest.mark.parametrize("m_big,m_small", [(256, 37), (64, 5), (6, 1)])
+def test_noalloc_matches_matmul_twice(hipq, cr, kind, m_big, m_small):
+    _pair(hipq, cr, kind, 640, 1024, m_big, m_small)
+
+
+def test_noalloc_large_row_count_then_one_row(hipq, cr):
+    """A vocabulary-sized matrix (two launches even for one row: the row's blocks pass
+    through the scratch) after a prefill-sized call."""
+    _pair(hipq, cr, "q4_K", 40000, 512, 512, 1)
+
+
+def test_noalloc_rejects_what_does_not_fit(hipq, cr):
+    import torch
+    n, k = 256, 4096
+    blocks = cr.quantize_weights(cr.oracle(), "q6_K", synth.normal(5, (n, k), 0.02))
+    w = capi.Weight("q6_K", n, k, blocks)
+    m = 4096  # 16.8 million values: beyond the scratch
+    a = torch.zeros((m, k), device="cuda")
+    c = torch.zeros((m, n), device="cuda")
+    with pytest.raises(capi.HipqError) as e:
+        capi.matmul_noalloc(w, a, m, c)
+    assert e.value.code == -4 and "scratch" in str(e.value)
+    w.destroy()
