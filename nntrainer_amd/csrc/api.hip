@@ -208,8 +208,11 @@ int matmul_tiled(const hipq_weight *w, const float *A, int64_t M, int64_t lda, f
   if (rc) return rc;
   QActTiled qa = qact_tiled_carve(mem, M, w->K);
   if (phase != 1) rc = hipq::launch_quantize_q8_K_tiled(A, M, w->K, lda, (M / 4) * 4, &qa, s);
-  if (!rc && phase != 2) rc = hipq::launch_gemm_q4k(w, &qa, (int)M, C, ldc, s);
-  return rc;
+  if (rc || phase == 2) return rc;
+  /* The GEMM reads a tile copy of the weights (coalesced loads), made at the weight's first
+   * prefill product; the entry point that may not allocate reads the planes until it exists. */
+  if (!w->gt_base && !sc.fixed && (rc = hipq::ensure_gemm_tiles(const_cast<hipq_weight *>(w)))) return rc;
+  return hipq::launch_gemm_q4k(w, &qa, (int)M, C, ldc, s);
 }
 
 int matmul_device(hipq_weight_t w, const float *A, int64_t M, int64_t lda, float *C, int64_t ldc,
@@ -328,6 +331,8 @@ int hipq_weight_create(int dtype, int layout, int64_t N, int64_t K, const void *
   w->dtype = dtype;
   w->device = g.device;
   w->expert_tiles = 0;
+  w->gt_base = nullptr;
+  w->gt_qs = w->gt_hdr = nullptr;
   w->N = N;
   w->K = K;
   /* planes, each 256-byte aligned */
@@ -462,6 +467,7 @@ int hipq_weight_destroy(hipq_weight_t w) {
   if (rc) return rc;
   (void)hipDeviceSynchronize();
   (void)hipFree(w->base);
+  if (w->gt_base) (void)hipFree(w->gt_base);
   {
     std::lock_guard<std::mutex> lk(g.mu);
     g.live_weights--;

@@ -101,9 +101,17 @@ struct Src {
 struct WHalf { /* this lane's two sub-blocks of one 128-deep stage */
   uint4 q[2];
 };
-__device__ __forceinline__ void load_wh(WHalf &W, const Src &sr, int sb, int h) {
-  W.q[0] = hipq_ld_global(sr.wq + sb * 8 + 2 * h);
-  W.q[1] = hipq_ld_global(sr.wq + sb * 8 + 2 * h + 1);
+/* TILES: the weights come from the tile copy (hipq_internal.h, gt_qs): piece i of lane
+ * (n, g) is sub-block 4g + i, 64 lanes x 16 bytes consecutive per piece, so a load
+ * instruction covers 1 KB of memory instead of 32 separate lines. */
+template <bool TILES> __device__ __forceinline__ void load_wh(WHalf &W, const Src &sr, int sb, int h) {
+  if (TILES) {
+    W.q[0] = hipq_ld_global(sr.wq + (sb * 4 + 2 * h) * 64);
+    W.q[1] = hipq_ld_global(sr.wq + (sb * 4 + 2 * h + 1) * 64);
+  } else {
+    W.q[0] = hipq_ld_global(sr.wq + sb * 8 + 2 * h);
+    W.q[1] = hipq_ld_global(sr.wq + sb * 8 + 2 * h + 1);
+  }
 }
 /* stage (128 deep) -> ring slot: each wavefront copies a quarter of the tile's stage, TM KB */
 template <int TM>
@@ -198,7 +206,7 @@ __device__ __forceinline__ void epilogue(const Smem<TM> &sm, int buf, const uint
   }
 }
 
-template <int TM>
+template <int TM, bool TILES>
 __global__ __launch_bounds__(NT, TM == 2 ? 3 : 2) void gemm_q4k_kernel(WView w, const int8_t *__restrict__ qt,
                                                          const uint16_t *__restrict__ amin,
                                                          const float *__restrict__ dAt, int M, int mtiles,
@@ -223,8 +231,16 @@ __global__ __launch_bounds__(NT, TM == 2 ? 3 : 2) void gemm_q4k_kernel(WView w, 
   sr.amin = make_rsrc(amin + ((size_t)qt128 * nsb * 128 + hrow * 64) * 16, (uint32_t)nsb * 128 * 32);
   sr.dAt = make_rsrc(dAt + (size_t)qt128 * nsb * 128 + hrow * 64, (uint32_t)nsb * 128 * 4);
   const int n = min(n0 + wave * 32 + i32, (int)w.N - 1);
-  sr.wq = (const uint4 *)(w.qs + (size_t)n * (w.K >> 1) + g * 64);
-  sr.whd = (const uint4 *)w.hdr + (size_t)n * nsb;
+  constexpr int HSTRIDE = TILES ? 32 : 1; /* uint4 between a column's consecutive super-block headers */
+  if (TILES) {
+    /* the copy pads N to 32 rows: a wavefront whose columns start below N has its tile */
+    const size_t wt = (size_t)(min(n0 + wave * 32, (int)w.N - 1) >> 5);
+    sr.wq = (const uint4 *)(w.qs + wt * nsb * 4096) + lane;
+    sr.whd = (const uint4 *)(w.hdr + wt * nsb * 512) + i32;
+  } else {
+    sr.wq = (const uint4 *)(w.qs + (size_t)n * (w.K >> 1) + g * 64);
+    sr.whd = (const uint4 *)w.hdr + (size_t)n * nsb;
+  }
   sr.wave = wave;
   sr.lane = lane;
 
@@ -237,7 +253,7 @@ __global__ __launch_bounds__(NT, TM == 2 ? 3 : 2) void gemm_q4k_kernel(WView w, 
 
   WHalf Wa, Wb; /* first / second half of a super-block */
   uint4 hd0, hd1;
-  load_wh(Wa, sr, 0, 0);
+  load_wh<TILES>(Wa, sr, 0, 0);
   hd0 = hipq_ld_global(sr.whd);
   dma_rows(sr, sm, 0, 0);
   dma_a(sr, sm, 0, 0);
@@ -260,7 +276,7 @@ __global__ __launch_bounds__(NT, TM == 2 ? 3 : 2) void gemm_q4k_kernel(WView w, 
       const int s2 = slot >= 1 ? slot - 1 : 2; /* the slot read last stage */
       dma_a(sr, sm, min(2 * sb + 2, nstage - 1), s2);
       dma_rows(sr, sm, sbn, eb ^ 1);
-      load_wh(Wb, sr, sb, 1);
+      load_wh<TILES>(Wb, sr, sb, 1);
       stage_mma<0>(sm, slot, Wa, slo, shi, lane, Dlo, Dhi);
       slot = slot == 2 ? 0 : slot + 1;
       sync_lds<InFlight<TM>::FIRST>();
@@ -268,8 +284,8 @@ __global__ __launch_bounds__(NT, TM == 2 ? 3 : 2) void gemm_q4k_kernel(WView w, 
     {
       const int s2 = slot >= 1 ? slot - 1 : 2;
       dma_a(sr, sm, min(2 * sb + 3, nstage - 1), s2);
-      load_wh(Wa, sr, sbn, 0);
-      hdn = hipq_ld_global(sr.whd + sbn);
+      load_wh<TILES>(Wa, sr, sbn, 0);
+      hdn = hipq_ld_global(sr.whd + sbn * HSTRIDE);
       stage_mma<1>(sm, slot, Wb, slo, shi, lane, Dlo, Dhi);
       slot = slot == 2 ? 0 : slot + 1;
     }
@@ -304,7 +320,14 @@ int launch_tiles(const hipq_weight *w, const QActTiled *qa, int M, float *C, int
   const int ntiles = (int)((w->N + BN - 1) / BN);
   const int ngroups = (ntiles + 7) / 8;
   const unsigned grid = (unsigned)(mtiles * ngroups * 8);
-  hipLaunchKernelGGL(gemm_q4k_kernel<TM>, dim3(grid), dim3(NT), sizeof(Smem<TM>), s, wview(w), qa->qt, qa->amin,
+  WView v = wview(w);
+  if (w->gt_base) { /* the tile copy, where the weight has one */
+    v.qs = w->gt_qs;
+    v.hdr = w->gt_hdr;
+    hipLaunchKernelGGL((gemm_q4k_kernel<TM, true>), dim3(grid), dim3(NT), sizeof(Smem<TM>), s, v, qa->qt, qa->amin,
+                       qa->dAt, M, mtiles, ntiles, C, ldc);
+  } else
+    hipLaunchKernelGGL((gemm_q4k_kernel<TM, false>), dim3(grid), dim3(NT), sizeof(Smem<TM>), s, v, qa->qt, qa->amin,
                      qa->dAt, M, mtiles, ntiles, C, ldc);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;

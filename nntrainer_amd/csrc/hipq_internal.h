@@ -60,6 +60,14 @@ struct hipq_weight {
   const uint8_t *hdr;
   const int8_t *sc;
   const uint16_t *d;
+  /* Q4_K only, built by the first prefill product of the weight (ensure_gemm_tiles): a
+   * second copy of the nibbles and headers by tiles of 32 rows, in the order the
+   * wavefronts of the prefill GEMM load them, so that each of their 128-bit load
+   * instructions covers 1 KB of consecutive memory:
+   *   gt_qs  [N/32][K/256][4][64][16 B]: load i of lane (n, g) = sub-block 4g + i of row n
+   *   gt_hdr [N/32][K/256][32][16 B] */
+  uint8_t *gt_base;
+  const uint8_t *gt_qs, *gt_hdr;
 };
 
 /* Plain-data view of a weight passed to kernels by value. */
@@ -206,6 +214,7 @@ int launch_quantize_weights(int dtype, const float *W, int64_t N, int64_t K,
 
 /* relayout.hip ------------------------------------------------------------ */
 int tile_expert_weight(hipq_weight *w); /* planes -> 32-row tiles, in a new allocation; synchronous */
+int ensure_gemm_tiles(hipq_weight *w);  /* adds the prefill GEMM's tile copy (allocates once; synchronous) */
 int launch_relayout(hipq_weight *w, int layout, const uint8_t *src_dev,
                     hipStream_t s);
 

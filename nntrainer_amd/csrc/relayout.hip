@@ -11,6 +11,8 @@
  * with the array-of-structs -> planes split. Pure byte movement; runs once per
  * weight at load time, one thread per source block.
  */
+#include <mutex>
+
 #include "hipq_internal.h"
 
 namespace {
@@ -147,9 +149,57 @@ __global__ void tile_q4_K(const uint8_t *__restrict__ qs, const uint8_t *__restr
       n < N ? *(const uint4 *)(hdr + (n * nsb + sb) * 16) : make_uint4(0, 0, 0, 0);
 }
 
+/* planes -> tiles of 32 rows for the prefill GEMM: thread = one 16-byte piece,
+ * piece (i, lane (n, g)) = sub-block 4g + i of row n */
+__global__ void gemm_tile_q4_K(const uint8_t *__restrict__ qs, const uint8_t *__restrict__ hdr, int N, int nsb,
+                               int64_t pieces, uint8_t *__restrict__ tq, uint8_t *__restrict__ th) {
+  const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= pieces) return;
+  const int lane = (int)(p & 63), i = (int)((p >> 6) & 3);
+  const int64_t ts = p >> 8; /* tile * nsb + sb */
+  const int sb = (int)(ts % nsb);
+  const int64_t n = (ts / nsb) * 32 + (lane & 31);
+  const int g = lane >> 5;
+  uint4 v = make_uint4(0, 0, 0, 0);
+  if (n < N) v = *(const uint4 *)(qs + (n * nsb + sb) * 128 + (4 * g + i) * 16);
+  *(uint4 *)(tq + p * 16) = v;
+  if (i == 0 && g == 0)
+    *(uint4 *)(th + (ts * 32 + (lane & 31)) * 16) =
+      n < N ? *(const uint4 *)(hdr + (n * nsb + sb) * 16) : make_uint4(0, 0, 0, 0);
+}
+
 } // namespace
 
 namespace hipq {
+
+int ensure_gemm_tiles(hipq_weight *w) {
+  static std::mutex mu; /* two threads may run their first prefill product on one weight */
+  std::lock_guard<std::mutex> lk(mu);
+  if (w->gt_base) return HIPQ_OK;
+  if (w->dtype != HIPQ_Q4_K || w->expert_tiles)
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "only Q4_K weights in the plane layout have a GEMM tile copy");
+  const int nsb = (int)(w->K / 256);
+  const int64_t tiles = (w->N + 31) / 32;
+  const size_t q_bytes = (size_t)tiles * nsb * 4096, h_bytes = (size_t)tiles * nsb * 512;
+  const size_t o_hdr = (q_bytes + 255) & ~(size_t)255;
+  uint8_t *nb = nullptr;
+  hipError_t e = hipMalloc((void **)&nb, o_hdr + h_bytes);
+  if (e != hipSuccess)
+    return fail(HIPQ_ERR_OUT_OF_MEMORY, "GEMM tiles of %zu bytes: %s", o_hdr + h_bytes, hipGetErrorString(e));
+  const int64_t pieces = tiles * nsb * 256;
+  hipLaunchKernelGGL(gemm_tile_q4_K, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, nullptr, w->qs, w->hdr,
+                     (int)w->N, nsb, pieces, nb, nb + o_hdr);
+  e = hipGetLastError();
+  if (e == hipSuccess) e = hipStreamSynchronize(nullptr); /* the caller's stream may be another one */
+  if (e != hipSuccess) {
+    (void)hipFree(nb);
+    return fail(HIPQ_ERR_RUNTIME, "GEMM tiling: %s", hipGetErrorString(e));
+  }
+  w->gt_qs = nb;
+  w->gt_hdr = nb + o_hdr;
+  w->gt_base = nb; /* last: readers test this field */
+  return HIPQ_OK;
+}
 
 int tile_expert_weight(hipq_weight *w) {
   if (w->dtype != HIPQ_Q4_K) return fail(HIPQ_ERR_INVALID_ARGUMENT, "only Q4_K weights have an expert layout");
