@@ -94,6 +94,9 @@ HIPQ_API int64_t hipq_weight_nbytes(int dtype, int64_t N, int64_t K);
  *  FullyConnectedLayer's weight tensor becomes on this back-end. */
 HIPQ_API int hipq_weight_create(int dtype, int layout, int64_t N, int64_t K,
                                 const void *bytes, int mem, hipq_weight_t *out);
+/** Waits for the device, then frees the weight. A HIP graph captured from a call that named
+ *  the weight (a matmul on it, an MoE block it is an expert of) must not be replayed
+ *  afterwards. */
 HIPQ_API int hipq_weight_destroy(hipq_weight_t w);
 HIPQ_API int hipq_weight_dims(hipq_weight_t w, int *dtype, int64_t *N, int64_t *K);
 

@@ -471,10 +471,17 @@ int hipq_weight_destroy(hipq_weight_t w) {
   {
     std::lock_guard<std::mutex> lk(g.mu);
     g.live_weights--;
-    /* tables may name w: drop them (the device was synchronized above) */
-    for (auto &kv : g.moe_tables)
-      if (kv.second.dev) (void)hipFree(kv.second.dev);
-    g.moe_tables.clear();
+    /* drop the expert tables that name w, and only those (the device was synchronized
+     * above): the tables of other layers stay valid, also for graphs captured with them */
+    for (auto it = g.moe_tables.begin(); it != g.moe_tables.end();) {
+      bool names = false;
+      for (const hipq_weight *k : it->second.key) names = names || k == w;
+      if (names) {
+        if (it->second.dev) (void)hipFree(it->second.dev);
+        it = g.moe_tables.erase(it);
+      } else
+        ++it;
+    }
   }
   delete w;
   return HIPQ_OK;

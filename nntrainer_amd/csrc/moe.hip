@@ -137,6 +137,11 @@ __device__ __forceinline__ void route_token(const float *__restrict__ logits, in
   for (int i = 0; i < MAXV; ++i) {
     const int e = lane + 64 * i;
     p[i] = (64 * i < E && e < E) ? __fdiv_rn(p[i], sum) : -1.f; /* -1: never selected */
+    /* A NaN among the logits makes every probability NaN, which no comparison below
+     * would ever select: the stored index would lie outside [0, E) and the kernels
+     * behind index tables with it. Such values count as 0, so the selection still
+     * returns topk distinct experts (the reference's partial_sort always does). */
+    if (!(p[i] == p[i])) p[i] = 0.f;
   }
   float ksum = 0.f;
   float myw = 0.f; /* lane kk keeps the kk-th weight */

@@ -140,10 +140,16 @@ void FullyConnectedLayerHip::incremental_forwarding(RunLayerContext &context, un
   hidden_step_dim.batch(1);
   hidden_step_dim.height(to - from);
 
-  /* rows [0, to - from) of every batch entry, as fc_layer.cpp:271-296 */
+  /* Rows [0, to - from) of every batch entry, as fc_layer.cpp:266-296. The reference takes
+   * the INPUT of entry b at b times the feature length of the OUTPUT (fc_layer.cpp:268-270);
+   * for batch 1, every LLM call, that is offset 0 either way. The same rule here, so that a
+   * graph that runs on both engines sees the same numbers; where it would leave the input
+   * tensor (the reference then reads past its end) the call is refused instead. */
   for (unsigned int b = 0; b < hidden_.batch(); ++b) {
-    Tensor input_step =
-      input_.getSharedDataTensor(input_step_dim, b * input_dim.getFeatureLen(), true);
+    const size_t in_off = (size_t)b * hidden_dim.getFeatureLen();
+    NNTR_THROW_IF(in_off + (size_t)(to - from) * input_dim.width() > input_.size(), std::invalid_argument)
+      << "incremental_forwarding: batch entry " << b << " of the input lies outside the tensor";
+    Tensor input_step = input_.getSharedDataTensor(input_step_dim, in_off, true);
     Tensor hidden_step =
       hidden_.getSharedDataTensor(hidden_step_dim, b * hidden_dim.getFeatureLen(), true);
 
@@ -162,6 +168,27 @@ void FullyConnectedLayerHip::calcDerivative(RunLayerContext &) {
 
 void FullyConnectedLayerHip::calcGradient(RunLayerContext &) {
   throw exception::not_supported("FullyConnectedLayerHip does not support backwarding");
+}
+
+static void drop_device_copies(RunLayerContext &run_context) {
+  for (unsigned int i = 0; i < run_context.getNumWeights(); ++i)
+    hipq_host::global_cache().invalidate(run_context.getWeight(i).getData<uint8_t>());
+}
+
+void FullyConnectedLayerHip::read(std::ifstream &file, RunLayerContext &run_context, bool opt_var,
+                   ml::train::ExecutionMode mode, bool trainable, TensorDim::DataType defineWeightDataType,
+                   bool fsu, size_t start_offset, bool read_from_offset, int file_fd) {
+  Layer::read(file, run_context, opt_var, mode, trainable, defineWeightDataType, fsu, start_offset,
+              read_from_offset, file_fd);
+  drop_device_copies(run_context);
+}
+
+void FullyConnectedLayerHip::read(ReadSource src, RunLayerContext &run_context, bool opt_var, ml::train::ExecutionMode mode,
+                   bool trainable, TensorDim::DataType defineWeightDataType, bool fsu, size_t start_offset,
+                   bool read_from_offset) {
+  Layer::read(src, run_context, opt_var, mode, trainable, defineWeightDataType, fsu, start_offset,
+              read_from_offset);
+  drop_device_copies(run_context);
 }
 
 } // namespace nntrainer

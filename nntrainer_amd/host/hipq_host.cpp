@@ -7,6 +7,7 @@
 #include "hipq_host.h"
 
 #include <atomic>
+#include <cstring>
 #include <sstream>
 
 namespace hipq_host {
@@ -49,23 +50,45 @@ bool runtime_available(int device) noexcept {
 
 WeightCache::~WeightCache() { clear(); }
 
+/* Eight 8-byte words of the buffer (both ends and six in between) folded into one:
+ * cheap enough for every forward call, and a rewritten weight differs in them. */
+static uint64_t sample_tag(const void *bytes, int64_t n) {
+  const unsigned char *p = static_cast<const unsigned char *>(bytes);
+  uint64_t tag = 0x9e3779b97f4a7c15ull ^ (uint64_t)n;
+  if (n < 8)
+    return tag;
+  const int64_t last = n - 8;
+  for (int i = 0; i < 8; ++i) {
+    uint64_t v;
+    std::memcpy(&v, p + (last * i / 7), 8);
+    tag = (tag ^ v) * 0xff51afd7ed558ccdull;
+    tag ^= tag >> 29;
+  }
+  return tag;
+}
+
 hipq_weight_t WeightCache::get(const void *host_bytes, const WeightSpec &spec) {
   if (!host_bytes)
     throw std::invalid_argument("[hipq] weight tensor has no data");
+  const int64_t nbytes = hipq_weight_nbytes(spec.dtype, spec.N, spec.K);
+  if (nbytes < 0)
+    check((int)nbytes, "hipq_weight_nbytes");
+  const uint64_t tag = sample_tag(host_bytes, nbytes);
   std::lock_guard<std::mutex> lock(mtx);
   auto it = map.find(host_bytes);
   if (it != map.end()) {
     const WeightSpec &o = it->second.spec;
-    if (o.dtype == spec.dtype && o.layout == spec.layout && o.N == spec.N && o.K == spec.K)
+    if (o.dtype == spec.dtype && o.layout == spec.layout && o.N == spec.N && o.K == spec.K &&
+        it->second.tag == tag)
       return it->second.w;
-    /* the allocator handed the address to another tensor: replace */
+    /* the allocator handed the address to another tensor, or the bytes were rewritten: replace */
     hipq_weight_destroy(it->second.w);
     map.erase(it);
   }
   hipq_weight_t w = nullptr;
   check(hipq_weight_create(spec.dtype, spec.layout, spec.N, spec.K, host_bytes, HIPQ_MEM_HOST, &w),
         "hipq_weight_create");
-  map.emplace(host_bytes, Entry{w, spec});
+  map.emplace(host_bytes, Entry{w, spec, tag});
   return w;
 }
 

@@ -74,9 +74,12 @@ public:
   WeightCache(const WeightCache &) = delete;
   WeightCache &operator=(const WeightCache &) = delete;
 
-  /** the device weight for these host bytes; uploads on first use */
+  /** the device weight for these host bytes; uploads on first use, and again when a
+   *  sample of the bytes (first, last and six words in between) no longer matches the
+   *  one taken at the upload: a buffer rewritten in place behind the layers' backs */
   hipq_weight_t get(const void *host_bytes, const WeightSpec &spec);
-  /** forget (and free) the device copy of a host buffer whose content changed */
+  /** forget (and free) the device copy of a host buffer whose content changed; the layers
+   *  call it for their weights after the framework has read them from a file */
   void invalidate(const void *host_bytes);
   void clear();
   size_t size() const;
@@ -85,6 +88,7 @@ private:
   struct Entry {
     hipq_weight_t w;
     WeightSpec spec;
+    uint64_t tag; /* sample of the host bytes at upload time */
   };
   mutable std::mutex mtx;
   std::unordered_map<const void *, Entry> map;

@@ -13,6 +13,10 @@
  *                            fills its tensors from the files, runs forwarding
  *                            (from == to == 0) or incremental_forwarding and
  *                            writes the output tensor
+ *   fcreload <dtype> <K> <N> <height> <weightA> <weightB> <input> <read|poke> <outA> <outB>
+ *                            forwarding with weight A, then the weight tensor's bytes are replaced
+ *                            by B in place -- through Layer::read as the model loader does it, or
+ *                            behind the layer's back -- and forwarding runs again
  *   moe <dtype> <T> <H> <I> <E> <k> <incremental> <router> <experts> <input> <out>
  *                            the same for qwen_moe; <experts> holds up_e, gate_e,
  *                            down_e for e = 0.. in the order the layer requests them
@@ -218,6 +222,32 @@ static int run_fc(Context *ctx, char **a) {
   return 0;
 }
 
+static int run_fc_reload(Context *ctx, char **a) {
+  const std::string dt = a[0];
+  const unsigned K = std::atoi(a[1]), N = std::atoi(a[2]), height = std::atoi(a[3]);
+  const std::string wa = a[4], wb = a[5], ipath = a[6], how = a[7], oa = a[8], ob = a[9];
+  auto layer = ctx->createLayerObject("fully_connected", {"unit=" + std::to_string(N), "disable_bias=true"});
+  InitLayerContext ic({TensorDim(1, 1, height, K)}, "fc", Tformat::NCHW, dtype_of(dt), Tdatatype::FP32);
+  layer->finalize(ic);
+  RunLayerContext rc(ic);
+  const size_t wbytes = mirror_tensor_bytes(rc.getWeight(0).getDim());
+  read_into(wa, rc.getWeight(0).getData<uint8_t>(), wbytes);
+  read_into(ipath, rc.getInput(0).getData<float>(), (size_t)height * K * 4);
+  float *out = rc.getOutput(0).getData<float>();
+  layer->forwarding(rc, false);
+  write_from(oa, out, (size_t)height * N * 4);
+  if (how == "read") {
+    std::ifstream f(wb, std::ios::binary);
+    layer->read(f, rc, false, ml::train::ExecutionMode::INFERENCE, false, dtype_of(dt), false);
+  } else {
+    read_into(wb, rc.getWeight(0).getData<uint8_t>(), wbytes);
+  }
+  layer->forwarding(rc, false);
+  write_from(ob, out, (size_t)height * N * 4);
+  std::printf("FC RELOAD DONE\n");
+  return 0;
+}
+
 static int run_moe(Context *ctx, char **a) {
   const std::string dt = a[0];
   const unsigned T = std::atoi(a[1]), H = std::atoi(a[2]), I = std::atoi(a[3]), E = std::atoi(a[4]),
@@ -265,6 +295,8 @@ int main(int argc, char **argv) {
       return run_fc(ctx, argv + 3);
     if (mode == "moe" && argc == 14)
       return run_moe(ctx, argv + 3);
+    if (mode == "fcreload" && argc == 13)
+      return run_fc_reload(ctx, argv + 3);
     std::printf("bad arguments for mode %s (argc %d)\n", mode.c_str(), argc);
     return 2;
   } catch (const std::exception &e) {

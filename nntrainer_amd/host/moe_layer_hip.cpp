@@ -183,4 +183,25 @@ void MoELayerHip::calcGradient(RunLayerContext &) {
   throw exception::not_supported("MoELayerHip does not support backwarding");
 }
 
+static void drop_device_copies(RunLayerContext &run_context) {
+  for (unsigned int i = 0; i < run_context.getNumWeights(); ++i)
+    hipq_host::global_cache().invalidate(run_context.getWeight(i).getData<uint8_t>());
+}
+
+void MoELayerHip::read(std::ifstream &file, RunLayerContext &run_context, bool opt_var,
+                   ml::train::ExecutionMode mode, bool trainable, TensorDim::DataType defineWeightDataType,
+                   bool fsu, size_t start_offset, bool read_from_offset, int file_fd) {
+  Layer::read(file, run_context, opt_var, mode, trainable, defineWeightDataType, fsu, start_offset,
+              read_from_offset, file_fd);
+  drop_device_copies(run_context);
+}
+
+void MoELayerHip::read(ReadSource src, RunLayerContext &run_context, bool opt_var, ml::train::ExecutionMode mode,
+                   bool trainable, TensorDim::DataType defineWeightDataType, bool fsu, size_t start_offset,
+                   bool read_from_offset) {
+  Layer::read(src, run_context, opt_var, mode, trainable, defineWeightDataType, fsu, start_offset,
+              read_from_offset);
+  drop_device_copies(run_context);
+}
+
 } // namespace nntrainer

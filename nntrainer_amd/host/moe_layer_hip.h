@@ -34,6 +34,15 @@ public:
   void calcDerivative(RunLayerContext &context) override;
   void calcGradient(RunLayerContext &context) override;
   void setProperty(const std::vector<std::string> &values) override;
+  /** The framework reads the weights into the tensors it owns; the device copies made from
+   *  their earlier content (a first forward before the load, a reload, a buffer that a
+   *  swapped-in weight shares) are dropped, so the next forward uploads the new bytes. */
+  void read(std::ifstream &file, RunLayerContext &run_context, bool opt_var, ml::train::ExecutionMode mode,
+            bool trainable, TensorDim::DataType defineWeightDataType, bool fsu, size_t start_offset = 0,
+            bool read_from_offset = false, int file_fd = -1) override;
+  void read(ReadSource src, RunLayerContext &run_context, bool opt_var, ml::train::ExecutionMode mode,
+            bool trainable, TensorDim::DataType defineWeightDataType, bool fsu, size_t start_offset = 0,
+            bool read_from_offset = false) override;
   const std::string getType() const override { return MoELayerHip::type; }
   bool supportBackwarding() const override { return false; }
 

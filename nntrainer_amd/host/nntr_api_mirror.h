@@ -32,6 +32,7 @@
 #include <string>
 #include <tuple>
 #include <unordered_map>
+#include <variant>
 #include <vector>
 
 namespace ml {
@@ -41,6 +42,7 @@ namespace train {
 enum LayerType { LAYER_FC = 1 };
 
 enum class ExportMethods { METHOD_STRINGVECTOR = 0 };
+enum class ExecutionMode { TRAIN = 0, INFERENCE = 1 };
 
 class TensorDim {
 public:
@@ -143,9 +145,24 @@ inline size_t mirror_tensor_bytes(const TensorDim &d) {
   }
 }
 
+/** where a layer's weights are read from (nntrainer/utils/util_func.h:43) */
+using ReadSource = std::variant<std::ifstream *, const char *>;
+
 /** Host tensor: a view (offset + dims) into shared storage. */
 class Tensor {
 public:
+  /** the tensor's bytes from a model file, in place (tensor.h:1646-1655) */
+  void read(std::ifstream &file, size_t start_offset = 0, bool read_from_offset = false, int /*file_fd*/ = -1) {
+    if (read_from_offset)
+      file.seekg((std::streamoff)start_offset);
+    file.read(getData<char>(), (std::streamsize)mirror_tensor_bytes(dim));
+    NNTR_THROW_IF(file.fail(), std::runtime_error) << "short read of a tensor";
+  }
+  void read(ReadSource src, size_t start_offset = 0, bool read_from_offset = false) {
+    NNTR_THROW_IF(!std::holds_alternative<std::ifstream *>(src), std::invalid_argument) << "file sources only";
+    read(*std::get<std::ifstream *>(src), start_offset, read_from_offset);
+  }
+
   Tensor() = default;
   explicit Tensor(const TensorDim &d) : dim(d), store(std::make_shared<std::vector<uint8_t>>(mirror_tensor_bytes(d))) {}
   Tensor(size_t b, size_t c, size_t h, size_t w, TensorDim::TensorType t = TensorDim::TensorType()) :
@@ -304,6 +321,19 @@ public:
   virtual void calcGradient(RunLayerContext &) {}
   virtual void setProperty(const std::vector<std::string> &values) = 0;
   virtual void exportTo(Exporter &, const ml::train::ExportMethods &) const {}
+  /** weights from a model file (layer_devel.h:391-470, the inference branch) */
+  virtual void read(std::ifstream &file, RunLayerContext &run_context, bool /*opt_var*/,
+                    ml::train::ExecutionMode /*mode*/, bool /*trainable*/, TensorDim::DataType /*defineWeightDataType*/,
+                    bool /*fsu*/, size_t start_offset = 0, bool read_from_offset = false, int file_fd = -1) {
+    for (unsigned int i = 0; i < run_context.getNumWeights(); ++i)
+      run_context.getWeight(i).read(file, start_offset, read_from_offset, file_fd);
+  }
+  virtual void read(ReadSource src, RunLayerContext &run_context, bool /*opt_var*/, ml::train::ExecutionMode /*mode*/,
+                    bool /*trainable*/, TensorDim::DataType /*defineWeightDataType*/, bool /*fsu*/,
+                    size_t start_offset = 0, bool read_from_offset = false) {
+    for (unsigned int i = 0; i < run_context.getNumWeights(); ++i)
+      run_context.getWeight(i).read(src, start_offset, read_from_offset);
+  }
   virtual void setBatch(RunLayerContext &, unsigned int) {}
   virtual bool supportBackwarding() const = 0;
 };

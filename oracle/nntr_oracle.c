@@ -824,27 +824,41 @@ void orc_gemm_q6_K(int M, int N, int K, const float *A, const void *W, float *C)
 /* mixture of experts                                                         */
 /* ------------------------------------------------------------------------- */
 
-/* M == 1 Q4_K matmul into a caller buffer, serial (called from a parallel loop). */
-static void gemv_q4_K_serial(int N, int K, const float *a, const uint8_t *w, float *c,
-                             uint8_t *qa) {
+/* M == 1 matmul of one weight format into a caller buffer, serial (called from a
+ * parallel loop): the row quantizer and the dot kernel the reference's wrappers use for
+ * a single row (GI/ggml_interface_omp.cpp:303-330, 404-431, 500-566).
+ * kind: 2 Q4_0, 12 Q4_K, 14 Q6_K (the ggml type ids). */
+static size_t moe_row_bytes(int kind, int K) {
+  return kind == 2 ? (size_t)(K / 32) * ORC_Q4_0_BYTES
+                   : (size_t)(K / ORC_QK_K) * (kind == 12 ? ORC_Q4_K_BYTES : ORC_Q6_K_BYTES);
+}
+static void gemv_serial(int kind, int N, int K, const float *a, const uint8_t *w, float *c, uint8_t *qa) {
+  const size_t rb = moe_row_bytes(kind, K);
+  if (kind == 2) {
+    const int nb = K / 32;
+    orc_quantize_row_q8_0(a, qa, K);
+    for (int n = 0; n < N; ++n) c[n] = dot_q4_0_q8_0(w + (size_t)n * rb, qa, nb);
+    return;
+  }
   const int nb = K / ORC_QK_K;
   memset(qa, 0, (size_t)nb * ORC_Q8_K_BYTES);
   orc_quantize_row_q8_K(a, qa, K);
   for (int n = 0; n < N; ++n)
-    c[n] = dot_q4_K_q8_K(w + (size_t)n * nb * ORC_Q4_K_BYTES, qa, nb, 0);
+    c[n] = kind == 12 ? dot_q4_K_q8_K(w + (size_t)n * rb, qa, nb, 0) : dot_q6_K_q8_K(w + (size_t)n * rb, qa, nb);
 }
 
-/* Applications/CausalLM/layers/qwen_moe_layer.cpp:394-503 with :332-392.
+/* Applications/CausalLM/layers/qwen_moe_layer.cpp:394-503 with :332-392 (renormalize
+ * = 1, the incremental path) and :161-259 (renormalize = 0, the forwarding path, which
+ * uses the softmax values of the selected experts as they are).
  * Routing: softmax over the E logits (subtract row max, exp, divide by the row
- * sum), top-k by descending probability, weights divided by their sum.
+ * sum), top-k by descending probability, weights divided by their sum if renormalize.
  * Expert e, token t (one at a time, M = 1): g = x.Wgate, u = x.Wup,
- * h = (sigmoid(g) * g) * u with sigmoid evaluated in double and cast,
- * o = h.Wdown, contribution = o * weight. Contributions are added into y in
- * ascending expert order. */
-void orc_moe_forward_q4_K(int T, int H, int I, int E, int topk, const float *x,
-                          const float *logits, const void *const *gate,
-                          const void *const *up, const void *const *down,
-                          float *y, int32_t *topk_idx, float *topk_w) {
+ * h = (sigmoid(g) * g) * u with sigmoid evaluated in double and cast
+ * (nntrainer/layers/acti_func.h:286-288, 400-405), o = h.Wdown, contribution =
+ * o * weight. Contributions are added into y in ascending expert order. */
+void orc_moe_forward(int kind, int renormalize, int T, int H, int I, int E, int topk, const float *x,
+                     const float *logits, const void *const *gate, const void *const *up,
+                     const void *const *down, float *y, int32_t *topk_idx, float *topk_w) {
   int32_t *idx = (int32_t *)malloc(sizeof(int32_t) * (size_t)T * topk);
   float *wt = (float *)malloc(sizeof(float) * (size_t)T * topk);
   float *p = (float *)malloc(sizeof(float) * (size_t)E);
@@ -871,7 +885,8 @@ void orc_moe_forward_q4_K(int T, int H, int I, int E, int topk, const float *x,
       wt[t * topk + k] = p[best];
       ksum += p[best];
     }
-    for (int k = 0; k < topk; ++k) wt[t * topk + k] = wt[t * topk + k] / ksum;
+    if (renormalize)
+      for (int k = 0; k < topk; ++k) wt[t * topk + k] = wt[t * topk + k] / ksum;
   }
   free(p);
   free(taken);
@@ -885,7 +900,7 @@ void orc_moe_forward_q4_K(int T, int H, int I, int E, int topk, const float *x,
 #pragma omp parallel
   {
     const int kmax = H > I ? H : I;
-    uint8_t *qa = (uint8_t *)malloc((size_t)(kmax / ORC_QK_K) * ORC_Q8_K_BYTES);
+    uint8_t *qa = (uint8_t *)malloc((size_t)(kmax / 32) * ORC_Q8_0_BYTES + (size_t)(kmax / ORC_QK_K + 1) * ORC_Q8_K_BYTES);
     float *g = (float *)malloc(sizeof(float) * (size_t)I);
     float *u = (float *)malloc(sizeof(float) * (size_t)I);
     float *h = (float *)malloc(sizeof(float) * (size_t)I);
@@ -894,14 +909,14 @@ void orc_moe_forward_q4_K(int T, int H, int I, int E, int topk, const float *x,
       const int t = pr / topk, e = idx[pr];
       const float *xt = x + (size_t)t * H;
       float *o = contrib + (size_t)pr * H;
-      gemv_q4_K_serial(I, H, xt, (const uint8_t *)gate[e], g, qa);
-      gemv_q4_K_serial(I, H, xt, (const uint8_t *)up[e], u, qa);
+      gemv_serial(kind, I, H, xt, (const uint8_t *)gate[e], g, qa);
+      gemv_serial(kind, I, H, xt, (const uint8_t *)up[e], u, qa);
       for (int i = 0; i < I; ++i) {
         const float en = (float)exp((double)(-g[i]));
         const float sig = (float)(1.0 / (1.0 + (double)en));
         h[i] = (sig * g[i]) * u[i];
       }
-      gemv_q4_K_serial(H, I, h, (const uint8_t *)down[e], o, qa);
+      gemv_serial(kind, H, I, h, (const uint8_t *)down[e], o, qa);
       for (int c = 0; c < H; ++c) o[c] = o[c] * wt[pr];
     }
     free(qa);
@@ -923,6 +938,13 @@ void orc_moe_forward_q4_K(int T, int H, int I, int E, int topk, const float *x,
   free(contrib);
   free(idx);
   free(wt);
+}
+
+void orc_moe_forward_q4_K(int T, int H, int I, int E, int topk, const float *x,
+                          const float *logits, const void *const *gate,
+                          const void *const *up, const void *const *down,
+                          float *y, int32_t *topk_idx, float *topk_w) {
+  orc_moe_forward(12, 1, T, H, I, E, topk, x, logits, gate, up, down, y, topk_idx, topk_w);
 }
 
 void orc_set_threads(int n) {

@@ -98,6 +98,11 @@ void orc_gemm_q6_K(int M, int N, int K, const float *A, const void *W, float *C)
  *   x [T x H] fp32; logits [T x E] fp32 router logits (already x . gate);
  *   gate/up: E arrays of Q4_K blocks of [I x H]; down: E arrays of [H x I];
  *   y [T x H] fp32. topk_idx/topk_w (may be NULL) receive the routing. */
+void orc_moe_forward(int kind /* 2 Q4_0, 12 Q4_K, 14 Q6_K */, int renormalize /* 0: the forwarding
+                     path, qwen_moe_layer.cpp:161-259 */, int T, int H, int I, int E, int topk,
+                     const float *x, const float *logits, const void *const *gate,
+                     const void *const *up, const void *const *down, float *y, int32_t *topk_idx,
+                     float *topk_w);
 void orc_moe_forward_q4_K(int T, int H, int I, int E, int topk, const float *x,
                           const float *logits, const void *const *gate,
                           const void *const *up, const void *const *down,

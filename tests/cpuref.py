@@ -193,18 +193,20 @@ def gemm_prepacked(lib, kind, a, packed, n):
     return c
 
 
-def moe_forward(x, logits, gate, up, down, topk):
-    """Oracle MoE block. gate/up/down: lists (len E) of canonical Q4_K block arrays."""
+def moe_forward(x, logits, gate, up, down, topk, kind="q4_K", renormalize=True):
+    """Oracle MoE block. gate/up/down: lists (len E) of canonical block arrays of `kind`."""
     lib = oracle()
     x = np.ascontiguousarray(x, np.float32)
     logits = np.ascontiguousarray(logits, np.float32)
     t, h = x.shape
     e = logits.shape[1]
-    i = gate[0].size // ((h // 256) * 144)
+    nbytes, blk = BLOCK_BYTES[kind]
+    i = gate[0].size // ((h // blk) * nbytes)
     arr = lambda lst: (_c.c_void_p * e)(*[w.ctypes.data for w in lst])
     y = np.zeros((t, h), np.float32)
     idx = np.zeros((t, topk), np.int32)
     wt = np.zeros((t, topk), np.float32)
-    lib.orc_moe_forward_q4_K(_i32(t), _i32(h), _i32(i), _i32(e), _i32(topk), _ptr(x), _ptr(logits),
-                             arr(gate), arr(up), arr(down), _ptr(y), _ptr(idx), _ptr(wt))
+    lib.orc_moe_forward(_i32({"q4_0": 2, "q4_K": 12, "q6_K": 14}[kind]), _i32(1 if renormalize else 0), _i32(t),
+                        _i32(h), _i32(i), _i32(e), _i32(topk), _ptr(x), _ptr(logits), arr(gate), arr(up),
+                        arr(down), _ptr(y), _ptr(idx), _ptr(wt))
     return y, idx, wt

@@ -1,0 +1,100 @@
+"""GPU parity of product branches the other files do not reach: the MoE block with the
+softmax values used as they are (renormalize = 0, the reference's forwarding path,
+qwen_moe_layer.cpp:161-259), MoE blocks whose experts are Q4_0 or Q6_K (MoELayer accepts
+any weight dtype of the model, qwen_moe_layer.cpp:50-159), and Q4_0 matmuls whose K is a
+multiple of 32 but not of 256 (legal per q4_0_tensor.cpp:25-28). All against the oracle,
+through the C ABI."""
+import numpy as np
+import pytest
+
+from nntrainer_amd import capi, synth
+
+pytestmark = pytest.mark.gpu
+
+
+def _experts(cr, kind, e, i, h, seed):
+    q = lambda s, shape: cr.quantize_weights(cr.oracle(), kind, synth.normal(s, shape, 0.02))
+    return ([q(seed + 3 * x, (i, h)) for x in range(e)], [q(seed + 3 * x + 1, (i, h)) for x in range(e)],
+            [q(seed + 3 * x + 2, (h, i)) for x in range(e)])
+
+
+def _run_moe(cr, kind, t, h, i, e, k, renormalize, seed):
+    import gpu_util as gu
+    import torch
+    gate, up, down = _experts(cr, kind, e, i, h, seed)
+    x = synth.normal(seed + 500, (t, h))
+    logits = synth.normal(seed + 501, (t, e))
+    ref_y, ref_idx, ref_w = cr.moe_forward(x, logits, gate, up, down, k, kind=kind, renormalize=renormalize)
+    wg = [capi.Weight(kind, i, h, b) for b in gate]
+    wu = [capi.Weight(kind, i, h, b) for b in up]
+    wd = [capi.Weight(kind, h, i, b) for b in down]
+    y = torch.full((t, h), float("nan"), device="cuda")
+    idx = torch.zeros((t, k), dtype=torch.int32, device="cuda")
+    wt = torch.zeros((t, k), device="cuda")
+    capi.moe_forward(t, h, i, e, k, wg, wu, wd, gu.dev(x), y, router_logits=gu.dev(logits), topk_idx=idx,
+                     topk_w=wt, renormalize=renormalize, stream=gu.stream())
+    torch.cuda.synchronize()
+    for w in wg + wu + wd:
+        w.destroy()
+    assert np.array_equal(idx.cpu().numpy(), ref_idx)
+    assert np.abs(wt.cpu().numpy() - ref_w).max() <= 1e-6
+    if not renormalize:
+        assert (ref_w.sum(1) < 0.999).all(), "the case must tell the two weightings apart"
+    got = y.cpu().numpy()
+    assert not np.isnan(got).any()
+    # every single-row product carries the reference's bits; only the softmax row sum
+    # (order unspecified in the reference) may move the last bits of the routing weights
+    assert gu.rel_err(got, ref_y) <= 2e-6, gu.rel_err(got, ref_y)
+
+
+@pytest.mark.parametrize("t,h,i,e,k", [(8, 256, 256, 8, 2), (64, 512, 256, 16, 4), (1, 2048, 768, 16, 8)])
+def test_moe_without_renormalization(hipq, cr, t, h, i, e, k):
+    _run_moe(cr, "q4_K", t, h, i, e, k, False, seed=7000)
+
+
+@pytest.mark.parametrize("kind", ["q4_0", "q6_K"])
+@pytest.mark.parametrize("t,h,i,e,k,renorm", [(6, 256, 256, 8, 2, True), (33, 512, 256, 8, 4, True),
+                                              (1, 1024, 512, 4, 2, True), (12, 256, 512, 8, 3, False)])
+def test_moe_with_q4_0_and_q6_K_experts(hipq, cr, kind, t, h, i, e, k, renorm):
+    _run_moe(cr, kind, t, h, i, e, k, renorm, seed=7100)
+
+
+@pytest.mark.parametrize("k", [32, 96, 1056])
+@pytest.mark.parametrize("m", [1, 5, 64])
+def test_q4_0_with_k_not_a_multiple_of_256(hipq, cr, k, m):
+    import gpu_util as gu
+    n = 320
+    blocks = cr.quantize_weights(cr.oracle(), "q4_0", synth.normal(7200 + k, (n, k), 0.02))
+    a = synth.normal(7300 + m, (m, k))
+    ref = cr.gemm(cr.oracle(), "q4_0", a, blocks, n)
+    w = capi.Weight("q4_0", n, k, blocks)
+    got = gu.gpu_matmul(w, a)
+    w.destroy()
+    assert not np.isnan(got).any()
+    assert gu.rel_err(got, ref) <= gu.TOL
+    assert np.array_equal(got.view(np.uint32), ref.view(np.uint32))
+
+
+def test_router_with_nan_logits_stays_in_range(hipq, cr):
+    """A NaN among the router logits must still give expert indices below E (the reference's
+    partial_sort always does): the expert kernels index tables with them."""
+    import gpu_util as gu
+    import torch
+    t, h, i, e, k = 4, 256, 256, 8, 2
+    gate, up, down = _experts(cr, "q4_K", e, i, h, 7400)
+    wg = [capi.Weight("q4_K", i, h, b) for b in gate]
+    wu = [capi.Weight("q4_K", i, h, b) for b in up]
+    wd = [capi.Weight("q4_K", h, i, b) for b in down]
+    logits = synth.normal(7401, (t, e))
+    logits[1, :] = np.nan
+    logits[2, 3] = np.nan
+    y = torch.zeros((t, h), device="cuda")
+    idx = torch.full((t, k), -1, dtype=torch.int32, device="cuda")
+    capi.moe_forward(t, h, i, e, k, wg, wu, wd, gu.dev(synth.normal(7402, (t, h))), y, router_logits=gu.dev(logits),
+                     topk_idx=idx, stream=gu.stream())
+    torch.cuda.synchronize()
+    got = idx.cpu().numpy()
+    for w in wg + wu + wd:
+        w.destroy()
+    assert ((got >= 0) & (got < e)).all(), got
+    assert all(len(set(r)) == k for r in got.tolist())

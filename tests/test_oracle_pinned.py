@@ -51,8 +51,22 @@ def test_fp16_conversions_match_reference():
 @pytest.mark.parametrize("kind", KINDS)
 @pytest.mark.parametrize("sigma", [0.02, 1.0])
 def test_weight_quantizer_bytes_match_reference(kind, sigma):
-    w = _w(3, 256, 2048, sigma)
+    """4.2 million weights per format and scale (16 384 super-blocks of 256): the searches
+    are order-sensitive fp32 code and every configuration's weights come out of them."""
+    w = _w(3, 1024, 4096, sigma)
     assert np.array_equal(cr.quantize_weights(cr.oracle(), kind, w), cr.quantize_weights(cr.ref(), kind, w))
+
+
+@needs_ref
+@pytest.mark.parametrize("kind", KINDS)
+def test_weight_quantizer_bytes_match_reference_uniform(kind):
+    """The inputs of the reference's own quantizer tests: uniform in (-1, 1)
+    (unittest_nntrainer_cpu_backend.cpp:35-48), plus rows with exact zeros and ties."""
+    u = np.random.default_rng(9).uniform(-1.0, 1.0, (512, 2048)).astype(np.float32)
+    u[0, :256] = 0.0
+    u[1, :64] = 0.25
+    u[2, ::2] = -u[2, 1::2]
+    assert np.array_equal(cr.quantize_weights(cr.oracle(), kind, u), cr.quantize_weights(cr.ref(), kind, u))
 
 
 @needs_ref
@@ -188,6 +202,7 @@ def test_moe_equals_dense_per_token_evaluation():
     x = synth.normal(200, (t, h))
     logits = synth.normal(201, (t, e))
     y, idx, wt = cr.moe_forward(x, logits, gate, up, down, k)
+    f32 = np.float32
     want = np.zeros((t, h), np.float64)
     for tt in range(t):
         order = np.argsort(-logits[tt], kind="stable")[:k]
@@ -195,12 +210,24 @@ def test_moe_equals_dense_per_token_evaluation():
         lw = np.exp(logits[tt, order].astype(np.float64) - logits[tt, order].max())
         lw /= lw.sum()  # renormalised softmax == softmax over the selected logits
         for ee, ww in zip(order, lw):
-            g = cr.gemm(o, "q4_K", x[tt:tt + 1], gate[ee], i)[0].astype(np.float64)
-            u = cr.gemm(o, "q4_K", x[tt:tt + 1], up[ee], i)[0].astype(np.float64)
-            hh = (g / (1 + np.exp(-g)) * u).astype(np.float32)
-            want[tt] += ww * cr.gemm(o, "q4_K", hh[None], down[ee], h)[0]
-    assert np.abs(y - want).max() / np.abs(want).max() < 2e-3  # h re-rounded to fp32 / requantized
+            g = cr.gemm(o, "q4_K", x[tt:tt + 1], gate[ee], i)[0]
+            u = cr.gemm(o, "q4_K", x[tt:tt + 1], up[ee], i)[0]
+            # acti_func.h:286-288, 400-405 taken literally: sigmoid = (float)(1.0 / (1.0 + exp(-x)))
+            # with exp returning float, then two fp32 multiplies
+            en = np.exp(-g.astype(np.float64)).astype(f32)
+            sig = (1.0 / (1.0 + en.astype(np.float64))).astype(f32)
+            hh = (sig * g).astype(f32) * u
+            want[tt] += ww * cr.gemm(o, "q4_K", hh[None], down[ee], h)[0].astype(np.float64)
+    assert np.abs(y - want).max() / np.abs(want).max() < 1e-5
     assert np.abs(wt.sum(1) - 1).max() < 1e-6
+    # the forwarding path (qwen_moe_layer.cpp:161-259) keeps the softmax values as they are
+    y0, idx0, wt0 = cr.moe_forward(x, logits, gate, up, down, k, renormalize=False)
+    assert np.array_equal(idx0, idx)
+    full = np.exp(logits.astype(np.float64) - logits.max(1, keepdims=True))
+    full /= full.sum(1, keepdims=True)
+    assert np.abs(wt0 - np.take_along_axis(full, idx0.astype(np.int64), 1)).max() < 1e-6
+    scale = wt0.astype(np.float64).sum(1, keepdims=True)  # y0 = y * (sum of the kept softmax values)
+    assert np.abs(y0 - want * scale).max() / np.abs(want).max() < 1e-5
 
 
 # ------------------------------------------------------------------ 3. golden digests
