@@ -212,17 +212,6 @@ HIPQ_API int hipq_moe_forward(const hipq_moe_desc *desc, const hipq_weight_t *ga
 HIPQ_API int hipq_quantize_weights(int dtype, const float *W, int64_t N, int64_t K,
                                    void *out_blocks, int mem, void *stream);
 
-/** Timing helper for benchmarks: runs the matmul `iters` times on device
- *  buffers, rotating over `n_weights` handles (distinct copies defeat the
- *  last-level cache), brackets the launches with HIP events recorded on
- *  `stream` and returns the average milliseconds per call.
- *  phase 0: whole call (activation quantizer + block-dot kernel);
- *  phase 1: block-dot kernel only, on activations quantized once beforehand;
- *  phase 2: activation quantizer only. */
-HIPQ_API int hipq_time_matmul(int n_weights, const hipq_weight_t *w, const float *A,
-                              int64_t M, int64_t lda, float *C, int64_t ldc,
-                              int iters, int phase, void *stream, float *ms_per_call);
-
 #ifdef __cplusplus
 }
 #endif

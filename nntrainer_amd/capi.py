@@ -21,8 +21,10 @@ SYMBOLS = [
     "hipq_init", "hipq_shutdown", "hipq_last_error", "hipq_version", "hipq_weight_nbytes",
     "hipq_weight_create", "hipq_weight_destroy", "hipq_weight_dims", "hipq_quantize_q8_0",
     "hipq_quantize_q8_K", "hipq_matmul", "hipq_matmul_noalloc", "hipq_matmul_multi", "hipq_moe_forward",
-    "hipq_quantize_weights", "hipq_time_matmul", "hipq_file_layout", "hipq_weights_from_file",
+    "hipq_quantize_weights", "hipq_file_layout", "hipq_weights_from_file",
 ]
+# measurement helpers of csrc/hipq_bench.h: exported for bench.py, not part of the product ABI
+BENCH_SYMBOLS = ["hipq_time_matmul", "hipq_bench_matmul_steps", "hipq_bench_mfma_ceiling"]
 
 
 class HipqError(RuntimeError):
@@ -86,6 +88,9 @@ def lib():
         L.hipq_quantize_weights.argtypes = [i32, vp, i64, i64, vp, i32, vp]
         L.hipq_time_matmul.argtypes = [i32, C.POINTER(vp), vp, i64, i64, vp, i64, i32, i32, vp,
                                        C.POINTER(C.c_float)]
+        fp = C.POINTER(C.c_float)
+        L.hipq_bench_matmul_steps.argtypes = [i32, C.POINTER(vp), vp, i64, i64, vp, i64, i32, vp, fp, fp, fp]
+        L.hipq_bench_mfma_ceiling.argtypes = [C.c_float, vp, fp, fp]
         _lib = L
     return _lib
 
@@ -243,3 +248,21 @@ def time_matmul(ws, a, m, c, iters, phase=0, stream=None):
     check(lib().hipq_time_matmul(n, hs, _addr(a), m, ws[0].k, _addr(c), ws[0].n, iters, phase,
                                  stream, C.byref(ms)))
     return ms.value
+
+
+def bench_matmul_steps(ws, a, m, c, steps, stream=None):
+    """(total, quantizer, product) milliseconds per step of `steps` whole matmuls, all three
+    from the same launches (events on `stream` between the kernels)."""
+    n = len(ws)
+    hs = (C.c_void_p * n)(*[w.handle.value for w in ws])
+    t, q, p = C.c_float(), C.c_float(), C.c_float()
+    check(lib().hipq_bench_matmul_steps(n, hs, _addr(a), m, ws[0].k, _addr(c), ws[0].n, steps, stream,
+                                        C.byref(t), C.byref(q), C.byref(p)))
+    return t.value / steps, q.value / steps, p.value / steps
+
+
+def bench_mfma_ceiling(target_ms=2.0, stream=None):
+    """(TOP/s, GHz) of a kernel that issues nothing but the int8 matrix instruction."""
+    tops, ghz = C.c_float(), C.c_float()
+    check(lib().hipq_bench_mfma_ceiling(target_ms, stream, C.byref(tops), C.byref(ghz)))
+    return tops.value, ghz.value

@@ -22,6 +22,7 @@
 #include <unordered_map>
 #include <vector>
 
+#include "hipq_bench.h"
 #include "hipq_internal.h"
 
 /* Scratch of hipq_matmul_noalloc: quantized activations of one call. Every GPU the
@@ -682,6 +683,56 @@ int hipq_time_matmul(int n_weights, const hipq_weight_t *w, const float *A, int6
   if (rc) return rc;
   if (er != hipSuccess) return fail(HIPQ_ERR_RUNTIME, "timing: %s", hipGetErrorString(er));
   *ms_per_call = ms / (float)iters;
+  return HIPQ_OK;
+}
+
+int hipq_bench_matmul_steps(int n_weights, const hipq_weight_t *w, const float *A, int64_t M, int64_t lda,
+                            float *C, int64_t ldc, int steps, void *stream, float *total_ms,
+                            float *quantizer_ms, float *product_ms) {
+  int rc = require_ready();
+  if (rc) return rc;
+  if (n_weights <= 0 || !w || steps <= 0 || steps > 100000 || !total_ms || !quantizer_ms || !product_ms)
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "bad timing arguments");
+  for (int i = 0; i < n_weights; ++i) {
+    if ((rc = check_matmul_args(w[i], A, M, lda, C, ldc))) return rc;
+    if (!wants_tiled(w[i], M))
+      return fail(HIPQ_ERR_NOT_SUPPORTED, "the step timer covers the tiled Q4_K prefill product");
+  }
+  hipStream_t s = (hipStream_t)stream;
+  EnqueueGuard eg(enqueue_lock(s));
+  const Scratch sc{false, s};
+  /* one untimed call first: workspace and tile copies exist before the events */
+  for (int i = 0; i < n_weights; ++i)
+    if ((rc = matmul_tiled(w[i], A, M, lda, C, ldc, s, 0, sc))) return rc;
+  std::vector<hipEvent_t> ev((size_t)2 * steps + 1);
+  for (auto &e : ev) HIPQ_HIP(hipEventCreate(&e));
+  HIPQ_HIP(hipStreamSynchronize(s));
+  hipError_t er = hipSuccess;
+  for (int it = 0; it < steps && !rc && er == hipSuccess; ++it) {
+    const hipq_weight *wi = w[it % n_weights];
+    er = hipEventRecord(ev[2 * it], s);
+    rc = matmul_tiled(wi, A, M, lda, C, ldc, s, 2, sc);
+    if (!rc && er == hipSuccess) er = hipEventRecord(ev[2 * it + 1], s);
+    if (!rc) rc = matmul_tiled(wi, A, M, lda, C, ldc, s, 1, sc);
+  }
+  if (er == hipSuccess) er = hipEventRecord(ev[2 * steps], s);
+  if (er == hipSuccess) er = hipEventSynchronize(ev[2 * steps]);
+  double q = 0.0, p = 0.0;
+  float total = 0.f;
+  for (int it = 0; it < steps && !rc && er == hipSuccess; ++it) {
+    float a = 0.f, b = 0.f;
+    er = hipEventElapsedTime(&a, ev[2 * it], ev[2 * it + 1]);
+    if (er == hipSuccess) er = hipEventElapsedTime(&b, ev[2 * it + 1], ev[2 * it + 2]);
+    q += a;
+    p += b;
+  }
+  if (!rc && er == hipSuccess) er = hipEventElapsedTime(&total, ev[0], ev[2 * steps]);
+  for (auto &e : ev) (void)hipEventDestroy(e);
+  if (rc) return rc;
+  if (er != hipSuccess) return fail(HIPQ_ERR_RUNTIME, "timing: %s", hipGetErrorString(er));
+  *total_ms = total;
+  *quantizer_ms = (float)q;
+  *product_ms = (float)p;
   return HIPQ_OK;
 }
 

@@ -1,0 +1,78 @@
+// SPDX-License-Identifier: Apache-2.0
+/**
+ * @file   bench_kernels.hip
+ * @brief  The matrix-core ceiling kernel of hipq_bench.h: what the int8 matrix
+ *         instruction sustains on this device when nothing else is issued.
+ */
+#include "hipq_bench.h"
+#include "hipq_internal.h"
+
+namespace {
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+__global__ __launch_bounds__(256) void mfma_ceiling_kernel(int iters, int *sink, long long *clocks) {
+  const int lane = threadIdx.x & 63;
+  v16i d0 = {0}, d1 = {0}, d2 = {0}, d3 = {0};
+  const v4i a = {lane, 1, 2, 3}, b = {3, 2, 1, lane};
+  const long long c0 = __builtin_readcyclecounter(), r0 = wall_clock64();
+  for (int i = 0; i < iters; ++i) {
+    d0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, d0, 0, 0, 0);
+    d1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, d1, 0, 0, 0);
+    d2 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, d2, 0, 0, 0);
+    d3 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, d3, 0, 0, 0);
+  }
+  const long long c1 = __builtin_readcyclecounter(), r1 = wall_clock64();
+  const int res = d0[0] + d1[1] + d2[2] + d3[3];
+  if (res == 0x7fffffff) sink[threadIdx.x] = res; /* keeps the results alive */
+  if (blockIdx.x == 0 && threadIdx.x == 0) {
+    clocks[0] = c1 - c0; /* shader clocks */
+    clocks[1] = r1 - r0; /* 100 MHz ticks */
+  }
+}
+
+} // namespace
+
+extern "C" int hipq_bench_mfma_ceiling(float target_ms, void *stream, float *tops, float *ghz) {
+  using hipq::fail;
+  if (!tops || !ghz || !(target_ms > 0.f)) return fail(HIPQ_ERR_INVALID_ARGUMENT, "bad ceiling arguments");
+  hipStream_t s = (hipStream_t)stream;
+  int dev = 0, cus = 0;
+  HIPQ_HIP(hipGetDevice(&dev));
+  HIPQ_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+  int *sink = nullptr;
+  long long *clocks = nullptr;
+  HIPQ_HIP(hipMalloc((void **)&sink, 256 * sizeof(int)));
+  HIPQ_HIP(hipMalloc((void **)&clocks, 2 * sizeof(long long)));
+  hipEvent_t e0, e1;
+  HIPQ_HIP(hipEventCreate(&e0));
+  HIPQ_HIP(hipEventCreate(&e1));
+  const int wg = cus * 3; /* three workgroups of four wavefronts per CU: three per SIMD */
+  /* 4 instructions of 32 clocks per iteration and wavefront, three wavefronts per SIMD, ~2.4 GHz */
+  int iters = (int)(target_ms * 1e-3 * 2.4e9 / (4 * 32 * 3));
+  if (iters < 1000) iters = 1000;
+  float ms = 0.f;
+  int rc = HIPQ_OK;
+  for (int pass = 0; pass < 2 && !rc; ++pass) { /* the first pass warms the clocks up */
+    hipError_t e = hipEventRecord(e0, s);
+    hipLaunchKernelGGL(mfma_ceiling_kernel, dim3(wg), dim3(256), 0, s, iters, sink, clocks);
+    if (e == hipSuccess) e = hipGetLastError();
+    if (e == hipSuccess) e = hipEventRecord(e1, s);
+    if (e == hipSuccess) e = hipEventSynchronize(e1);
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+    if (e != hipSuccess) rc = fail(HIPQ_ERR_RUNTIME, "ceiling kernel: %s", hipGetErrorString(e));
+  }
+  long long h[2] = {0, 1};
+  if (!rc && hipMemcpy(h, clocks, sizeof(h), hipMemcpyDeviceToHost) != hipSuccess)
+    rc = fail(HIPQ_ERR_RUNTIME, "ceiling kernel: copy failed");
+  (void)hipEventDestroy(e0);
+  (void)hipEventDestroy(e1);
+  (void)hipFree(sink);
+  (void)hipFree(clocks);
+  if (rc) return rc;
+  const double ops = 2.0 * 32 * 32 * 32 * 4.0 * (double)iters * 4.0 * wg; /* per instruction x wavefronts */
+  *tops = (float)(ops / (ms * 1e-3) / 1e12);
+  *ghz = (float)((double)h[0] * 0.1 / (double)h[1]); /* clocks per 10 ns tick */
+  return HIPQ_OK;
+}

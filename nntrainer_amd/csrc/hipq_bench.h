@@ -1,0 +1,43 @@
+/* SPDX-License-Identifier: Apache-2.0 */
+/**
+ * @file   hipq_bench.h
+ * @brief  Measurement helpers exported by libhipq.so for bench.py only. They are not
+ *         part of the product's C ABI (include/hipq.h) and replace nothing in the
+ *         reference: event-timed launch loops and a matrix-core ceiling kernel.
+ */
+#ifndef HIPQ_BENCH_H
+#define HIPQ_BENCH_H
+
+#include "hipq.h"
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/** Runs the matmul `iters` times on device buffers, rotating over `n_weights` handles
+ *  (distinct copies defeat the last-level cache), brackets the launches with HIP events
+ *  recorded on `stream` and returns the average milliseconds per call.
+ *  phase 0: whole call (activation quantizer + block-dot kernel);
+ *  phase 1: block-dot kernel only, on activations quantized once beforehand;
+ *  phase 2: activation quantizer only. */
+HIPQ_API int hipq_time_matmul(int n_weights, const hipq_weight_t *w, const float *A, int64_t M,
+                              int64_t lda, float *C, int64_t ldc, int iters, int phase, void *stream,
+                              float *ms_per_call);
+
+/** `steps` whole matmuls (activation quantizer, then block-dot kernel) as hipq_matmul
+ *  enqueues them, with one event before each quantizer, one between the two kernels and
+ *  one behind the last product, all on `stream`: the three figures come from the same
+ *  launches and add up (total = quantizer + product). Milliseconds, sums over the steps. */
+HIPQ_API int hipq_bench_matmul_steps(int n_weights, const hipq_weight_t *w, const float *A, int64_t M,
+                                     int64_t lda, float *C, int64_t ldc, int steps, void *stream,
+                                     float *total_ms, float *quantizer_ms, float *product_ms);
+
+/** Nothing but v_mfma_i32_32x32x32_i8 on every SIMD of the device (three wavefronts each,
+ *  four independent accumulators) for about `target_ms`: the int8 rate the matrix cores
+ *  sustain here, in TOP/s, and the shader clock during the run in GHz. */
+HIPQ_API int hipq_bench_mfma_ceiling(float target_ms, void *stream, float *tops, float *ghz);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* HIPQ_BENCH_H */
