@@ -205,6 +205,34 @@ HIPQ_API int hipq_moe_forward(const hipq_moe_desc *desc, const hipq_weight_t *ga
                               int32_t *topk_idx, float *topk_w, int mem,
                               void *stream);
 
+/** Variants of the block for the other MoE layers of the LLM application. All pointers
+ *  live where `mem` says, like x.
+ *  - HIPQ_MOE_QWEN (or ext == NULL): hipq_moe_forward as above. It also serves the cached
+ *    layer (CachedSlimMoELayer::incremental_forwarding, qwen_moe_layer_cached.cpp:266-470):
+ *    that layer differs in where expert weights live between calls (paged in on demand, 32 kept;
+ *    here all experts stay in HBM) and in running one batched product per expert, which is how
+ *    this library runs every MoE; routing, expert arithmetic and the ascending-expert sum are
+ *    the same.
+ *  - HIPQ_MOE_GPT_OSS: GptOssMoELayer (gpt_oss_moe_layer.cpp:372-449, 452-568): the router
+ *    logits take router_bias [E]; per expert g = gate(x) + gate_bias[e], u = up(x) + up_bias[e],
+ *    h = (g / (1 + exp(-alpha g))) * (u + 1), y_e = down(h) + down_bias[e]; no clamping (the
+ *    reference has it commented out); top-k weights renormalised per desc->renormalize. */
+enum { HIPQ_MOE_QWEN = 0, HIPQ_MOE_GPT_OSS = 1 };
+typedef struct hipq_moe_ext {
+  int32_t variant;          /* HIPQ_MOE_*                                    */
+  float alpha;              /* gpt_oss: 1.702 (gpt_oss_moe_layer.h:126)      */
+  const float *router_bias; /* [E] or NULL; needs router_weight              */
+  const float *gate_bias;   /* [E x I], gpt_oss                              */
+  const float *up_bias;     /* [E x I], gpt_oss                              */
+  const float *down_bias;   /* [E x H], gpt_oss                              */
+} hipq_moe_ext;
+HIPQ_API int hipq_moe_forward_ext(const hipq_moe_desc *desc, const hipq_moe_ext *ext,
+                                  const hipq_weight_t *gate, const hipq_weight_t *up,
+                                  const hipq_weight_t *down, const float *x,
+                                  const float *router_logits, const float *router_weight,
+                                  float *y, int32_t *topk_idx, float *topk_w, int mem,
+                                  void *stream);
+
 /** Offline weight quantizers fp32 [N x K] -> canonical blocks, on the GPU.
  *  Replace quantize_q4_0 / quantize_q4_K / quantize_q6_K
  *  (x86_compute_backend.cpp:343-370 -> nntr_ggml_impl_quant.cpp:452-467,

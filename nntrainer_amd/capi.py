@@ -21,6 +21,7 @@ SYMBOLS = [
     "hipq_init", "hipq_shutdown", "hipq_last_error", "hipq_version", "hipq_weight_nbytes",
     "hipq_weight_create", "hipq_weight_destroy", "hipq_weight_dims", "hipq_quantize_q8_0",
     "hipq_quantize_q8_K", "hipq_matmul", "hipq_matmul_noalloc", "hipq_matmul_multi", "hipq_moe_forward",
+    "hipq_moe_forward_ext",
     "hipq_quantize_weights", "hipq_file_layout", "hipq_weights_from_file",
 ]
 # measurement helpers of csrc/hipq_bench.h: exported for bench.py, not part of the product ABI
@@ -44,6 +45,14 @@ FILE_SKIP = -1
 class MoeDesc(C.Structure):
     _fields_ = [("tokens", C.c_int32), ("hidden", C.c_int32), ("intermediate", C.c_int32),
                 ("experts", C.c_int32), ("topk", C.c_int32), ("renormalize", C.c_int32)]
+
+
+class MoeExt(C.Structure):
+    _fields_ = [("variant", C.c_int32), ("alpha", C.c_float), ("router_bias", C.c_void_p),
+                ("gate_bias", C.c_void_p), ("up_bias", C.c_void_p), ("down_bias", C.c_void_p)]
+
+
+MOE_QWEN, MOE_GPT_OSS = 0, 1
 
 
 def build(force=False):
@@ -85,6 +94,8 @@ def lib():
                                         C.POINTER(i64), i32, vp]
         L.hipq_moe_forward.argtypes = [C.POINTER(MoeDesc), C.POINTER(vp), C.POINTER(vp),
                                        C.POINTER(vp), vp, vp, vp, vp, vp, vp, i32, vp]
+        L.hipq_moe_forward_ext.argtypes = [C.POINTER(MoeDesc), C.POINTER(MoeExt), C.POINTER(vp), C.POINTER(vp),
+                                           C.POINTER(vp), vp, vp, vp, vp, vp, vp, i32, vp]
         L.hipq_quantize_weights.argtypes = [i32, vp, i64, i64, vp, i32, vp]
         L.hipq_time_matmul.argtypes = [i32, C.POINTER(vp), vp, i64, i64, vp, i64, i32, i32, vp,
                                        C.POINTER(C.c_float)]
@@ -238,6 +249,18 @@ def moe_forward(tokens, hidden, inter, experts, topk, gate, up, down, x, y, rout
     check(lib().hipq_moe_forward(C.byref(d), ex.gate, ex.up, ex.down, _addr(x),
                                  _addr(router_logits), _addr(router_weight), _addr(y),
                                  _addr(topk_idx), _addr(topk_w), mem, stream))
+
+
+def moe_forward_gpt_oss(tokens, hidden, inter, experts, topk, gate, up, down, x, y, gate_bias, up_bias,
+                        down_bias, alpha=1.702, router_logits=None, router_weight=None, router_bias=None,
+                        topk_idx=None, topk_w=None, renormalize=True, mem=MEM_DEVICE, stream=None):
+    """The GPT-OSS block: biased router and projections, (g / (1 + exp(-alpha g))) * (u + 1)."""
+    d = MoeDesc(tokens, hidden, inter, experts, topk, 1 if renormalize else 0)
+    ext = MoeExt(MOE_GPT_OSS, alpha, _addr(router_bias), _addr(gate_bias), _addr(up_bias), _addr(down_bias))
+    ex = gate if isinstance(gate, Experts) else Experts(gate, up, down)
+    check(lib().hipq_moe_forward_ext(C.byref(d), C.byref(ext), ex.gate, ex.up, ex.down, _addr(x),
+                                     _addr(router_logits), _addr(router_weight), _addr(y),
+                                     _addr(topk_idx), _addr(topk_w), mem, stream))
 
 
 def time_matmul(ws, a, m, c, iters, phase=0, stream=None):

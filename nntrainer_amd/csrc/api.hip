@@ -742,11 +742,27 @@ int hipq_moe_forward(const hipq_moe_desc *desc, const hipq_weight_t *gate, const
                      const hipq_weight_t *down, const float *x, const float *router_logits,
                      const float *router_weight, float *y, int32_t *topk_idx, float *topk_w,
                      int mem, void *stream) {
+  return hipq_moe_forward_ext(desc, nullptr, gate, up, down, x, router_logits, router_weight, y, topk_idx,
+                              topk_w, mem, stream);
+}
+
+int hipq_moe_forward_ext(const hipq_moe_desc *desc, const hipq_moe_ext *ext, const hipq_weight_t *gate,
+                         const hipq_weight_t *up, const hipq_weight_t *down, const float *x,
+                         const float *router_logits, const float *router_weight, float *y,
+                         int32_t *topk_idx, float *topk_w, int mem, void *stream) {
   int rc = require_ready();
   if (rc) return rc;
   if (!desc || !gate || !up || !down || !x || !y)
     return fail(HIPQ_ERR_INVALID_ARGUMENT, "null argument");
   const hipq_moe_desc d = *desc;
+  hipq_moe_ext x_ = {};
+  if (ext) x_ = *ext;
+  if (x_.variant != HIPQ_MOE_QWEN && x_.variant != HIPQ_MOE_GPT_OSS)
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "unknown MoE variant %d", x_.variant);
+  if (x_.variant == HIPQ_MOE_GPT_OSS && (!x_.gate_bias || !x_.up_bias || !x_.down_bias))
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "the gpt_oss variant needs gate_bias, up_bias and down_bias");
+  if (x_.router_bias && router_logits)
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "router_bias applies to logits formed from router_weight only");
   if (d.tokens < 0 || d.hidden <= 0 || d.intermediate <= 0 || d.experts <= 0 || d.topk <= 0 ||
       d.topk > d.experts || d.topk > 32 || d.experts > 1024)
     return fail(HIPQ_ERR_INVALID_ARGUMENT, "bad MoE shape T=%d H=%d I=%d E=%d k=%d", d.tokens,
@@ -804,7 +820,14 @@ int hipq_moe_forward(const hipq_moe_desc *desc, const hipq_weight_t *gate, const
   a.gate = gate;
   a.up = up;
   a.down = down;
+  a.epi.kind = x_.variant;
+  a.epi.alpha = x_.alpha;
+  a.epi.gate_bias = x_.gate_bias;
+  a.epi.up_bias = x_.up_bias;
+  a.epi.down_bias = x_.down_bias;
+  a.router_bias = x_.router_bias;
   const size_t T = (size_t)d.tokens, H = (size_t)d.hidden, E = (size_t)d.experts, k = (size_t)d.topk;
+  const size_t I = (size_t)d.intermediate;
   if (mem == HIPQ_MEM_DEVICE) {
     a.x = x;
     a.router_logits = router_logits;
@@ -815,7 +838,20 @@ int hipq_moe_forward(const hipq_moe_desc *desc, const hipq_weight_t *gate, const
     return hipq::launch_moe(&a, ws, ws_bytes, dev_views, s);
   }
   if (mem != HIPQ_MEM_HOST) return fail(HIPQ_ERR_INVALID_ARGUMENT, "unknown mem kind %d", mem);
-  DevBuf dx, dr, dy, di, dw;
+  DevBuf dx, dr, dy, di, dw, dbr, dbg, dbu, dbd;
+  auto to_device = [&](DevBuf &b, const float *src, size_t n, const float **dst) -> int {
+    if (!src) return HIPQ_OK;
+    if (int r = b.alloc(n * 4)) return r;
+    HIPQ_HIP(hipMemcpy(b.p, src, n * 4, hipMemcpyHostToDevice));
+    *dst = (const float *)b.p;
+    return HIPQ_OK;
+  };
+  if ((rc = to_device(dbr, x_.router_bias, E, &a.router_bias))) return rc;
+  if (x_.variant == HIPQ_MOE_GPT_OSS) {
+    if ((rc = to_device(dbg, x_.gate_bias, E * I, &a.epi.gate_bias))) return rc;
+    if ((rc = to_device(dbu, x_.up_bias, E * I, &a.epi.up_bias))) return rc;
+    if ((rc = to_device(dbd, x_.down_bias, E * H, &a.epi.down_bias))) return rc;
+  }
   if ((rc = dx.alloc(T * H * 4))) return rc;
   if ((rc = dr.alloc((router_logits ? T * E : H * E) * 4))) return rc;
   if ((rc = dy.alloc(T * H * 4))) return rc;

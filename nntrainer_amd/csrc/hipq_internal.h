@@ -190,8 +190,18 @@ int launch_gemm_q4k(const hipq_weight *w, const QActTiled *qa, int M, float *C,
                     int64_t ldc, hipStream_t s);
 
 /* moe.hip ----------------------------------------------------------------- */
+/* Variant of the expert MLP. kind 0: h = silu(g) * u, y = down(h) (qwen_moe_layer.cpp:332-392).
+ * kind 1: g and u take a bias, h = (g / (1 + exp(-alpha g))) * (u + 1), y = down(h) + bias
+ * (gpt_oss_moe_layer.cpp:372-449). Biases are device pointers, [E][I], [E][I], [E][H]. */
+struct MoeEpi {
+  const float *gate_bias, *up_bias, *down_bias;
+  float alpha;
+  int kind;
+};
 struct MoeArgs {
   hipq_moe_desc desc;
+  MoeEpi epi;
+  const float *router_bias; /* device [E] or null; applies to logits formed from router_weight */
   const hipq_weight *const *gate;
   const hipq_weight *const *up;
   const hipq_weight *const *down;

@@ -90,16 +90,18 @@ size_t carve(const hipq_moe_desc &d, int is_k, uint8_t *base, MoeBufs *b) {
   return o;
 }
 
-/* logits[t][e] = sum_h x[t][h] * Wr[h][e] */
+/* logits[t][e] = sum_h x[t][h] * Wr[h][e] (+ bias[e], added after the sum as the reference
+ * adds it to the finished product, gpt_oss_moe_layer.cpp:500-503) */
 __global__ __launch_bounds__(256) void router_logits_kernel(const float *__restrict__ x,
                                                             const float *__restrict__ wr, int H,
-                                                            int E, float *__restrict__ logits) {
+                                                            int E, const float *__restrict__ bias,
+                                                            float *__restrict__ logits) {
   const int t = blockIdx.x;
   const float *xt = x + (size_t)t * H;
   for (int e = threadIdx.x; e < E; e += blockDim.x) {
     float acc = 0.f;
     for (int h = 0; h < H; ++h) acc = fmaf(xt[h], wr[(size_t)h * E + e], acc);
-    logits[(size_t)t * E + e] = acc;
+    logits[(size_t)t * E + e] = bias ? acc + bias[e] : acc;
   }
 }
 
@@ -388,6 +390,22 @@ __device__ __forceinline__ float silu_ref(float g) {
   return sig * g;
 }
 
+/* The activation between the projections and the bias of the down projection, by expert
+ * variant (hipq_internal.h, MoeEpi). For the biased variant the value of column col of expert
+ * e is (g / (1 + exp(-alpha g))) * (u + 1) with g and u the biased products, in fp32
+ * (gpt_oss_moe_layer.cpp:406-437; swiglu with alpha, fallback_internal.cpp:425-432). */
+__device__ __forceinline__ float moe_act(const hipq::MoeEpi &ep, int e, int I, int col, float g, float u) {
+  if (ep.kind == 0) return silu_ref(g) * u;
+  g = g + ep.gate_bias[(size_t)e * I + col];
+  u = u + ep.up_bias[(size_t)e * I + col];
+  u = u + 1.f;
+  return (g / (1.f + expf(-ep.alpha * g))) * u;
+}
+__device__ __forceinline__ float moe_out(const hipq::MoeEpi &ep, int e, int H, int col, float o, float w) {
+  if (ep.kind != 0) o = o + ep.down_bias[(size_t)e * H + col];
+  return o * w;
+}
+
 /* One group of G weight rows against the cached activations: phase 1 into the
  * wavefront's LDS records, phase 2 fp32 chains, result of this lane's chain. */
 template <typename E>
@@ -412,7 +430,7 @@ template <int DT, int T, int KC, int G, int CPW>
 __global__ __launch_bounds__(256) void gate_up_kernel(const WView *__restrict__ views, int E_,
                                                       QView xq, const int *__restrict__ offsets,
                                                       const int *__restrict__ slot_pair, int topk,
-                                                      int I, float *__restrict__ h) {
+                                                      int I, float *__restrict__ h, hipq::MoeEpi ep) {
   typedef GemvCore<DT, T, RTOK, G, false, KC> E;
   extern __shared__ uint32_t moe_lds[];
   const int e = blockIdx.y;
@@ -444,7 +462,7 @@ __global__ __launch_bounds__(256) void gate_up_kernel(const WView *__restrict__ 
       if (cg + 1 < CPW && col0 + G < I) E::load_w(Wg, wg, col0 + G, 0, K);
       const GemvOut u = run_group<E>(Wu, A, arow, K, lds);
       if (g.valid && col0 + g.g < I && s0 + g.r < end)
-        h[(size_t)(s0 + g.r) * I + col0 + g.g] = silu_ref(g.v) * u.v;
+        h[(size_t)(s0 + g.r) * I + col0 + g.g] = moe_act(ep, e, I, col0 + g.g, g.v, u.v);
     }
   }
 }
@@ -455,7 +473,7 @@ __global__ __launch_bounds__(256) void down_kernel(const WView *__restrict__ vie
                                                    const int *__restrict__ offsets,
                                                    const int *__restrict__ slot_pair,
                                                    const float *__restrict__ wgt, int H,
-                                                   float *__restrict__ contrib) {
+                                                   float *__restrict__ contrib, hipq::MoeEpi ep) {
   typedef GemvCore<DT, T, RTOK, G, false, KC> E;
   extern __shared__ uint32_t moe_lds[];
   const int e = blockIdx.y;
@@ -482,7 +500,7 @@ __global__ __launch_bounds__(256) void down_kernel(const WView *__restrict__ vie
       if (cg + 1 < CPW && col0 + G < H) E::load_w(W[(cg + 1) & 1], wd, col0 + G, 0, K);
       const GemvOut o = run_group<E>(W[cg & 1], A, arow, K, lds);
       if (o.valid && col0 + o.g < H && s0 + o.r < end)
-        contrib[(size_t)(s0 + o.r) * H + col0 + o.g] = o.v * wgt[slot_pair[s0 + o.r]];
+        contrib[(size_t)(s0 + o.r) * H + col0 + o.g] = moe_out(ep, e, H, col0 + o.g, o.v, wgt[slot_pair[s0 + o.r]]);
     }
   }
 }
@@ -493,7 +511,8 @@ template <int DT>
 __global__ __launch_bounds__(256) void gate_up_long_kernel(const WView *__restrict__ views, int E_,
                                                            QView xq, const int *__restrict__ offsets,
                                                            const int *__restrict__ slot_pair,
-                                                           int topk, int I, float *__restrict__ h) {
+                                                           int topk, int I, float *__restrict__ h,
+                                                           hipq::MoeEpi ep) {
   constexpr int G = 2;
   extern __shared__ uint32_t moe_lds[];
   const int e = blockIdx.y;
@@ -513,7 +532,7 @@ __global__ __launch_bounds__(256) void gate_up_long_kernel(const WView *__restri
     const GemvOut g = gemv_engine<DT, 64, RTOK, G, false>(wg, col0, xq, arow, 0, lds);
     const GemvOut u = gemv_engine<DT, 64, RTOK, G, false>(wu, col0, xq, arow, 0, lds);
     if (g.valid && col0 + g.g < I && s0 + g.r < end)
-      h[(size_t)(s0 + g.r) * I + col0 + g.g] = silu_ref(g.v) * u.v;
+      h[(size_t)(s0 + g.r) * I + col0 + g.g] = moe_act(ep, e, I, col0 + g.g, g.v, u.v);
   }
 }
 
@@ -522,7 +541,7 @@ __global__ __launch_bounds__(256) void down_long_kernel(const WView *__restrict_
                                                         QView hq, const int *__restrict__ offsets,
                                                         const int *__restrict__ slot_pair,
                                                         const float *__restrict__ wgt, int H,
-                                                        float *__restrict__ contrib) {
+                                                        float *__restrict__ contrib, hipq::MoeEpi ep) {
   constexpr int G = 2;
   extern __shared__ uint32_t moe_lds[];
   const int e = blockIdx.y;
@@ -538,7 +557,7 @@ __global__ __launch_bounds__(256) void down_long_kernel(const WView *__restrict_
     for (int r = 0; r < RTOK; ++r) arow[r] = min(s0 + r, end - 1);
     const GemvOut o = gemv_engine<DT, 64, RTOK, G, false>(wd, col0, hq, arow, 0, lds);
     if (o.valid && col0 + o.g < H && s0 + o.r < end)
-      contrib[(size_t)(s0 + o.r) * H + col0 + o.g] = o.v * wgt[slot_pair[s0 + o.r]];
+      contrib[(size_t)(s0 + o.r) * H + col0 + o.g] = moe_out(ep, e, H, col0 + o.g, o.v, wgt[slot_pair[s0 + o.r]]);
   }
 }
 
@@ -773,7 +792,8 @@ __device__ __forceinline__ void xr_run(int ntile, const XLds &l, int K, TileOf t
 template <int TC, bool PAIRED>
 __global__ __launch_bounds__(256, TC <= 8 ? 4 : TC <= 16 ? 2 : 1) void gate_up_mma_kernel(
   const WView *__restrict__ views, int E_, QView xq, const int *__restrict__ offsets,
-  const int *__restrict__ items, const int *__restrict__ slot_pair, int topk, int I, float *__restrict__ h) {
+  const int *__restrict__ items, const int *__restrict__ slot_pair, int topk, int I, float *__restrict__ h,
+  hipq::MoeEpi ep) {
   constexpr int NREG = TC / 2;
   extern __shared__ __attribute__((aligned(16))) unsigned char xmoe_lds[];
   const int item = blockIdx.y;
@@ -800,7 +820,7 @@ __global__ __launch_bounds__(256, TC <= 8 ? 4 : TC <= 16 ? 2 : 1) void gate_up_m
 #pragma unroll
     for (int r = 0; r < NREG; ++r) {
       const int tok = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-      if (col < I && s0 + tok < end) h[(size_t)(s0 + tok) * I + col] = silu_ref(gate[r]) * up[r];
+      if (col < I && s0 + tok < end) h[(size_t)(s0 + tok) * I + col] = moe_act(ep, e, I, col, gate[r], up[r]);
     }
   };
   if (col0 >= I) { /* uniform per wavefront; it still takes part in the barriers */
@@ -854,7 +874,7 @@ template <int TC, bool QH>
 __global__ __launch_bounds__(256, TC <= 8 ? 4 : TC <= 16 ? 2 : 1) void down_mma_kernel(
   const WView *__restrict__ views, int E_, QView hq, const float *__restrict__ hf,
   const int *__restrict__ offsets, const int *__restrict__ items, const int *__restrict__ slot_pair,
-  const float *__restrict__ wgt, int H, float *__restrict__ contrib, int ct) {
+  const float *__restrict__ wgt, int H, float *__restrict__ contrib, int ct, hipq::MoeEpi ep) {
   constexpr int NREG = TC / 2;
   extern __shared__ __attribute__((aligned(16))) unsigned char xmoe_lds[];
   const int item = blockIdx.y;
@@ -903,7 +923,7 @@ __global__ __launch_bounds__(256, TC <= 8 ? 4 : TC <= 16 ? 2 : 1) void down_mma_
       for (int r = 0; r < NREG; ++r) {
         const int tok = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
         if (col < H && s0 + tok < end)
-          contrib[(size_t)(s0 + tok) * H + col] = out[r] * wgt[slot_pair[s0 + tok]];
+          contrib[(size_t)(s0 + tok) * H + col] = moe_out(ep, e, H, col, out[r], wgt[slot_pair[s0 + tok]]);
       }
     },
     stage);
@@ -937,34 +957,34 @@ __global__ __launch_bounds__(256) void combine_kernel(const int *__restrict__ to
 constexpr int CPW = 4; /* column groups per wavefront */
 
 template <int DT, int T, int KC, int G>
-void launch_gate_up(const hipq_moe_desc &d, const WView *views, const QAct &xq, const MoeBufs &b,
-                    hipStream_t s) {
+void launch_gate_up(const hipq_moe_desc &d, const hipq::MoeEpi &ep, const WView *views, const QAct &xq,
+                    const MoeBufs &b, hipStream_t s) {
   const size_t lds = 4 * GemvLds<DT, RTOK, G, false>::DWORDS * sizeof(uint32_t);
   if (d.hidden > KC) {
     const dim3 grid((d.intermediate + 7) / 8, d.experts);
     const size_t lds_long = 4 * GemvLds<DT, RTOK, 2, false>::DWORDS * sizeof(uint32_t);
     hipLaunchKernelGGL((gate_up_long_kernel<DT>), grid, dim3(256), lds_long, s, views, d.experts,
-                       qview(xq), b.offsets, b.slot_pair, d.topk, d.intermediate, b.h);
+                       qview(xq), b.offsets, b.slot_pair, d.topk, d.intermediate, b.h, ep);
     return;
   }
   const dim3 grid((d.intermediate + 4 * G * CPW - 1) / (4 * G * CPW), d.experts);
   hipLaunchKernelGGL((gate_up_kernel<DT, T, KC, G, CPW>), grid, dim3(256), lds, s, views, d.experts,
-                     qview(xq), b.offsets, b.slot_pair, d.topk, d.intermediate, b.h);
+                     qview(xq), b.offsets, b.slot_pair, d.topk, d.intermediate, b.h, ep);
 }
 template <int DT, int T, int KC, int G>
-void launch_down(const hipq_moe_desc &d, const WView *views, const QAct &hq, const MoeBufs &b,
-                 hipStream_t s) {
+void launch_down(const hipq_moe_desc &d, const hipq::MoeEpi &ep, const WView *views, const QAct &hq,
+                 const MoeBufs &b, hipStream_t s) {
   const size_t lds = 4 * GemvLds<DT, RTOK, G, false>::DWORDS * sizeof(uint32_t);
   if (d.intermediate > KC) {
     const dim3 grid((d.hidden + 7) / 8, d.experts);
     const size_t lds_long = 4 * GemvLds<DT, RTOK, 2, false>::DWORDS * sizeof(uint32_t);
     hipLaunchKernelGGL((down_long_kernel<DT>), grid, dim3(256), lds_long, s, views, d.experts,
-                       qview(hq), b.offsets, b.slot_pair, b.wgt, d.hidden, b.contrib);
+                       qview(hq), b.offsets, b.slot_pair, b.wgt, d.hidden, b.contrib, ep);
     return;
   }
   const dim3 grid((d.hidden + 4 * G * CPW - 1) / (4 * G * CPW), d.experts);
   hipLaunchKernelGGL((down_kernel<DT, T, KC, G, CPW>), grid, dim3(256), lds, s, views, d.experts,
-                     qview(hq), b.offsets, b.slot_pair, b.wgt, d.hidden, b.contrib);
+                     qview(hq), b.offsets, b.slot_pair, b.wgt, d.hidden, b.contrib, ep);
 }
 
 /* calls f.template operator()<T, KC, G>() for the shape class of K */
@@ -985,19 +1005,21 @@ template <int DT, typename F> void for_row_length(int64_t K, F f) {
 
 template <int DT> struct GateUpLauncher {
   const hipq_moe_desc &d;
+  const hipq::MoeEpi &ep;
   const WView *views;
   const QAct &xq;
   const MoeBufs &b;
   hipStream_t s;
-  template <int T, int KC, int G> void operator()() const { launch_gate_up<DT, T, KC, G>(d, views, xq, b, s); }
+  template <int T, int KC, int G> void operator()() const { launch_gate_up<DT, T, KC, G>(d, ep, views, xq, b, s); }
 };
 template <int DT> struct DownLauncher {
   const hipq_moe_desc &d;
+  const hipq::MoeEpi &ep;
   const WView *views;
   const QAct &hq;
   const MoeBufs &b;
   hipStream_t s;
-  template <int T, int KC, int G> void operator()() const { launch_down<DT, T, KC, G>(d, views, hq, b, s); }
+  template <int T, int KC, int G> void operator()() const { launch_down<DT, T, KC, G>(d, ep, views, hq, b, s); }
 };
 
 constexpr size_t XLDS_MAX = 160 * 1024; /* LDS of a CU */
@@ -1021,11 +1043,11 @@ int launch_grouped_mma(const hipq::MoeArgs *a, const MoeBufs &b, const WView *vi
   if (few)
     hipLaunchKernelGGL((gate_up_mma_kernel<TC, true>), dim3((d.intermediate + 63) / 64, max_items), dim3(256), lds_g,
                        s, views, d.experts, qview(xq), b.offsets, b.items, b.slot_pair, d.topk, d.intermediate,
-                       b.h);
+                       b.h, a->epi);
   else
     hipLaunchKernelGGL((gate_up_mma_kernel<TC, false>), dim3((d.intermediate + 127) / 128, max_items), dim3(256),
                        lds_g, s, views, d.experts, qview(xq), b.offsets, b.items, b.slot_pair, d.topk,
-                       d.intermediate, b.h);
+                       d.intermediate, b.h, a->epi);
   HIPQ_HIP(hipGetLastError());
   if (!few) {
     int rc = hipq::launch_quantize_q8_K_rowmma(b.h, P, d.intermediate, d.intermediate, &hq, s);
@@ -1038,10 +1060,10 @@ int launch_grouped_mma(const hipq::MoeArgs *a, const MoeBufs &b, const WView *vi
   const dim3 gd((d.hidden + 128 * ct - 1) / (128 * ct), max_items);
   if (few)
     hipLaunchKernelGGL((down_mma_kernel<TC, true>), gd, dim3(256), lds_d, s, views, d.experts, qview(hq), b.h,
-                       b.offsets, b.items, b.slot_pair, b.wgt, d.hidden, b.contrib, ct);
+                       b.offsets, b.items, b.slot_pair, b.wgt, d.hidden, b.contrib, ct, a->epi);
   else
     hipLaunchKernelGGL((down_mma_kernel<TC, false>), gd, dim3(256), lds_d, s, views, d.experts, qview(hq), b.h,
-                       b.offsets, b.items, b.slot_pair, b.wgt, d.hidden, b.contrib, ct);
+                       b.offsets, b.items, b.slot_pair, b.wgt, d.hidden, b.contrib, ct, a->epi);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
 }
@@ -1067,14 +1089,14 @@ int launch_grouped(const hipq::MoeArgs *a, const MoeBufs &b, const WView *views,
   const hipq_moe_desc &d = a->desc;
   const int64_t P = (int64_t)d.tokens * d.topk;
   int rc;
-  for_row_length<DT>(d.hidden, GateUpLauncher<DT>{d, views, xq, b, s});
+  for_row_length<DT>(d.hidden, GateUpLauncher<DT>{d, a->epi, views, xq, b, s});
   HIPQ_HIP(hipGetLastError());
   if (DT == HIPQ_Q4_0)
     rc = hipq::launch_quantize_q8_0(b.h, P, d.intermediate, d.intermediate, &hq, nullptr, s);
   else
     rc = hipq::launch_quantize_q8_K(b.h, P, d.intermediate, d.intermediate, 0, &hq, nullptr, s);
   if (rc) return rc;
-  for_row_length<DT>(d.intermediate, DownLauncher<DT>{d, views, hq, b, s});
+  for_row_length<DT>(d.intermediate, DownLauncher<DT>{d, a->epi, views, hq, b, s});
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
 }
@@ -1107,7 +1129,7 @@ int launch_moe(const MoeArgs *a, void *workspace, size_t workspace_bytes, const 
   const float *logits = a->router_logits;
   if (!logits) {
     hipLaunchKernelGGL(router_logits_kernel, dim3(T), dim3(256), 0, s, a->x, a->router_weight,
-                       d.hidden, E, b.logits);
+                       d.hidden, E, a->router_bias, b.logits);
     HIPQ_HIP(hipGetLastError());
     logits = b.logits;
   }

@@ -5,25 +5,12 @@
  */
 #include "fc_layer_hip.h"
 
-#include "hipq_host.h"
+#include "layer_common.h"
 #include "layer_props.h"
 
 namespace nntrainer {
 
 static constexpr unsigned int SINGLE_INOUT_IDX = 0;
-
-static int hipq_dtype_of(Tdatatype t) {
-  switch (t) {
-  case Tdatatype::Q4_0:
-    return HIPQ_Q4_0;
-  case Tdatatype::Q4_K:
-    return HIPQ_Q4_K;
-  case Tdatatype::Q6_K:
-    return HIPQ_Q6_K;
-  default:
-    return -1;
-  }
-}
 
 void FullyConnectedLayerHip::setProperty(const std::vector<std::string> &values) {
   for (const auto &kv : hipq_host::split_properties(values)) {
@@ -168,11 +155,6 @@ void FullyConnectedLayerHip::calcDerivative(RunLayerContext &) {
 
 void FullyConnectedLayerHip::calcGradient(RunLayerContext &) {
   throw exception::not_supported("FullyConnectedLayerHip does not support backwarding");
-}
-
-static void drop_device_copies(RunLayerContext &run_context) {
-  for (unsigned int i = 0; i < run_context.getNumWeights(); ++i)
-    hipq_host::global_cache().invalidate(run_context.getWeight(i).getData<uint8_t>());
 }
 
 void FullyConnectedLayerHip::read(std::ifstream &file, RunLayerContext &run_context, bool opt_var,

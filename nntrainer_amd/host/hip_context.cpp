@@ -13,6 +13,8 @@
 #include "fc_layer_hip.h"
 #include "hipq_host.h"
 #include "moe_layer_hip.h"
+#include "qkv_layer_hip.h"
+#include "tie_word_embedding_hip.h"
 
 namespace nntrainer {
 
@@ -50,6 +52,14 @@ void HipContext::add_default_object() {
   /* an application layer: it has no integer key in the framework either
    * (Applications/CausalLM/layers/qwen_moe_layer.h:107) */
   registerFactory(nntrainer::createLayer<MoELayerHip>, MoELayerHip::type, -1);
+  /* the application's other layers on this path, under their own type keys
+   * (qkv_layer.h:143, tie_word_embedding.h:140, qwen_moe_layer_cached.h:114-115,
+   * gpt_oss_moe_layer.h:102, gpt_oss_moe_layer_cached.h:105-106) */
+  registerFactory(nntrainer::createLayer<QKVLayerHip>, QKVLayerHip::type, -1);
+  registerFactory(nntrainer::createLayer<TieWordEmbeddingHip>, TieWordEmbeddingHip::type, -1);
+  registerFactory(nntrainer::createLayer<CachedSlimMoELayerHip>, CachedSlimMoELayerHip::type, -1);
+  registerFactory(nntrainer::createLayer<GptOssMoELayerHip>, GptOssMoELayerHip::type, -1);
+  registerFactory(nntrainer::createLayer<CachedSlimGptOssMoELayerHip>, CachedSlimGptOssMoELayerHip::type, -1);
 }
 
 int HipContext::registerFactory(const FactoryType<Layer> factory, const std::string &key,

@@ -149,11 +149,49 @@ void matmul_multi(WeightCache &cache, const std::vector<const void *> &weight_by
         "hipq_matmul_multi");
 }
 
+hipq_weight_t upload(const void *host_bytes, const WeightSpec &spec) {
+  require_runtime();
+  if (!host_bytes)
+    throw std::invalid_argument("[hipq] upload: the weight has no bytes (a virtual tensor that is not active?)");
+  hipq_weight_t w = nullptr;
+  check(hipq_weight_create(spec.dtype, spec.layout, spec.N, spec.K, host_bytes, HIPQ_MEM_HOST, &w),
+        "hipq_weight_create");
+  return w;
+}
+
+void release(hipq_weight_t w) noexcept {
+  if (w)
+    hipq_weight_destroy(w);
+}
+
+void moe_forward_resident(const MoeShape &shape, const hipq_weight_t *gate, const hipq_weight_t *up,
+                          const hipq_weight_t *down, const float *x, const float *router_weight, float *y,
+                          const MoeExtras *extras) {
+  require_runtime();
+  hipq_moe_desc desc;
+  desc.tokens = shape.tokens;
+  desc.hidden = shape.hidden;
+  desc.intermediate = shape.intermediate;
+  desc.experts = shape.experts;
+  desc.topk = shape.topk;
+  desc.renormalize = shape.renormalize ? 1 : 0;
+  hipq_moe_ext ext;
+  ext.variant = extras && extras->gpt_oss ? HIPQ_MOE_GPT_OSS : HIPQ_MOE_QWEN;
+  ext.alpha = extras ? extras->alpha : 0.f;
+  ext.router_bias = extras ? extras->router_bias : nullptr;
+  ext.gate_bias = extras ? extras->gate_bias : nullptr;
+  ext.up_bias = extras ? extras->up_bias : nullptr;
+  ext.down_bias = extras ? extras->down_bias : nullptr;
+  check(hipq_moe_forward_ext(&desc, &ext, gate, up, down, x, nullptr, router_weight, y, nullptr, nullptr,
+                             HIPQ_MEM_HOST, nullptr),
+        "hipq_moe_forward");
+}
+
 void moe_forward(WeightCache &cache, const MoeShape &shape, int dtype,
                  const std::vector<const void *> &gate_bytes,
                  const std::vector<const void *> &up_bytes,
                  const std::vector<const void *> &down_bytes, const float *x,
-                 const float *router_weight, float *y) {
+                 const float *router_weight, float *y, const MoeExtras *extras) {
   require_runtime();
   const size_t E = (size_t)shape.experts;
   if (gate_bytes.size() != E || up_bytes.size() != E || down_bytes.size() != E)
@@ -167,16 +205,7 @@ void moe_forward(WeightCache &cache, const MoeShape &shape, int dtype,
     u[e] = cache.get(up_bytes[e], gu);
     d[e] = cache.get(down_bytes[e], dn);
   }
-  hipq_moe_desc desc;
-  desc.tokens = shape.tokens;
-  desc.hidden = shape.hidden;
-  desc.intermediate = shape.intermediate;
-  desc.experts = shape.experts;
-  desc.topk = shape.topk;
-  desc.renormalize = shape.renormalize ? 1 : 0;
-  check(hipq_moe_forward(&desc, g.data(), u.data(), d.data(), x, nullptr, router_weight, y, nullptr,
-                         nullptr, HIPQ_MEM_HOST, nullptr),
-        "hipq_moe_forward");
+  moe_forward_resident(shape, g.data(), u.data(), d.data(), x, router_weight, y, extras);
 }
 
 } // namespace hipq_host

@@ -117,6 +117,20 @@ struct MoeShape {
   bool renormalize;
 };
 
+/** What the GPT-OSS block adds to the Qwen block (hipq_moe_ext of include/hipq.h): host pointers,
+ *  biases as [experts x intermediate], [experts x intermediate], [experts x hidden]. */
+struct MoeExtras {
+  bool gpt_oss = false;
+  float alpha = 1.702f;
+  const float *router_bias = nullptr;
+  const float *gate_bias = nullptr, *up_bias = nullptr, *down_bias = nullptr;
+};
+
+/** A device copy that the caller owns (not entered into a cache): for weights whose host bytes
+ *  come and go (virtual tensors), where an address is no identity. */
+hipq_weight_t upload(const void *host_bytes, const WeightSpec &spec);
+void release(hipq_weight_t w) noexcept;
+
 /**
  * The MoE block of qwen_moe_layer.cpp:394-503 on host pointers: router matmul
  * with the fp32 gate weight [hidden x experts], softmax, top-k, renormalise,
@@ -126,7 +140,12 @@ void moe_forward(WeightCache &cache, const MoeShape &shape, int dtype,
                  const std::vector<const void *> &gate_bytes,
                  const std::vector<const void *> &up_bytes,
                  const std::vector<const void *> &down_bytes, const float *x,
-                 const float *router_weight, float *y);
+                 const float *router_weight, float *y, const MoeExtras *extras = nullptr);
+
+/** the same block on device copies the caller already holds (experts entries each) */
+void moe_forward_resident(const MoeShape &shape, const hipq_weight_t *gate, const hipq_weight_t *up,
+                          const hipq_weight_t *down, const float *x, const float *router_weight, float *y,
+                          const MoeExtras *extras = nullptr);
 
 } // namespace hipq_host
 

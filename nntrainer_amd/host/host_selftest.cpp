@@ -20,6 +20,16 @@
  *   moe <dtype> <T> <H> <I> <E> <k> <incremental> <router> <experts> <input> <out>
  *                            the same for qwen_moe; <experts> holds up_e, gate_e,
  *                            down_e for e = 0.. in the order the layer requests them
+ *   moex <type> <dtype> <T> <H> <I> <E> <k> <incremental> <weights> <input> <out>
+ *                            any of the MoE layer types; <weights> holds every weight in the order
+ *                            the layer requests them and is loaded through Layer::read (which is how
+ *                            virtual tensors get their bytes)
+ *   qkv <dtype> <K> <Nq> <Nk> <Nv> <height> <from> <to> <weights> <input> <out>
+ *                            qkv_layer; <weights> holds q, k, v; <out> the three outputs one after
+ *                            the other
+ *   lmhead <dtype> <K> <unit> <batch> <height> <from> <to> <table> <input> <out>
+ *   embed <dtype> <in_dim> <out_dim> <batch> <width> <from> <to> <table> <ids> <out>
+ *                            tie_word_embeddings in its two modes
  * The test suite compares the written outputs with expected values it computes itself.
  */
 #include <dlfcn.h>
@@ -28,6 +38,7 @@
 #include <cstdlib>
 #include <fstream>
 #include <iostream>
+#include <memory>
 #include <string>
 #include <vector>
 
@@ -84,6 +95,8 @@ static Tdatatype dtype_of(const std::string &s) {
     return Tdatatype::Q4_K;
   if (s == "q6_K")
     return Tdatatype::Q6_K;
+  if (s == "fp32")
+    return Tdatatype::FP32;
   std::printf("unknown dtype %s\n", s.c_str());
   std::exit(2);
 }
@@ -183,6 +196,71 @@ static int run_api(Context *ctx) {
       "qwen_moe", {"num_experts=2", "num_experts_per_token=3", "unit=256", "moe_activation=swish"});
     EXPECT_THROW(k->finalize(ic), std::invalid_argument);
   }
+  /* qkv_layer: three weights in q, k, v order, three outputs (qkv_layer.cpp:43-110) */
+  {
+    auto qkv = ctx->createLayerObject("qkv_layer", {"q_unit=512", "k_unit=256", "v_unit=128"});
+    EXPECT(qkv && qkv->getType() == "qkv_layer");
+    InitLayerContext ic({TensorDim(1, 1, 9, 1024)}, "l0_qkv", Tformat::NCHW, Tdatatype::Q4_0, Tdatatype::FP32);
+    qkv->finalize(ic);
+    const auto &w = ic.getWeightRequests();
+    EXPECT(w.size() == 3);
+    EXPECT(w[0].name == "l0_qkv:qweight" && w[0].dim == TensorDim(1, 1, 1024, 512));
+    EXPECT(w[1].name == "l0_qkv:kweight" && w[1].dim == TensorDim(1, 1, 1024, 256));
+    EXPECT(w[2].name == "l0_qkv:vweight" && w[2].dim == TensorDim(1, 1, 1024, 128));
+    EXPECT(w[2].dim.getDataType() == Tdatatype::Q4_0);
+    EXPECT(ic.getOutputDimensions().size() == 3);
+    EXPECT(ic.getOutputDimensions()[0] == TensorDim(1, 1, 9, 512));
+    EXPECT(ic.getOutputDimensions()[2] == TensorDim(1, 1, 9, 128));
+    EXPECT_THROW(ctx->createLayerObject("qkv_layer", {"q_unit=8", "k_unit=8"})->finalize(ic), std::invalid_argument);
+    EXPECT_THROW(ctx->createLayerObject("qkv_layer", {"unit=8"}), std::invalid_argument);
+  }
+  /* tie_word_embeddings: the mode follows from the properties (tie_word_embedding.cpp:43-51) */
+  {
+    auto head = ctx->createLayerObject("tie_word_embeddings", {"unit=4096", "disable_bias=true"});
+    EXPECT(head && head->getType() == "tie_word_embeddings");
+    InitLayerContext ic({TensorDim(1, 1, 5, 1024)}, "out", Tformat::NCHW, Tdatatype::Q6_K, Tdatatype::FP32);
+    head->finalize(ic);
+    EXPECT(ic.getWeightRequests().size() == 1);
+    EXPECT(ic.getWeightRequests()[0].name == "out:Embedding");
+    EXPECT(ic.getWeightRequests()[0].dim == TensorDim(1, 1, 4096, 1024)); /* the table: unit rows */
+    EXPECT(ic.getOutputDimensions()[0] == TensorDim(1, 1, 5, 4096));
+    auto emb = ctx->createLayerObject("tie_word_embeddings", {"in_dim=4096", "out_dim=1024"});
+    InitLayerContext ie({TensorDim(1, 1, 1, 7)}, "emb", Tformat::NCHW, Tdatatype::Q6_K, Tdatatype::FP32);
+    emb->finalize(ie);
+    EXPECT(ie.getWeightRequests()[0].dim == TensorDim(1, 1, 4096, 1024));
+    EXPECT(ie.getOutputDimensions()[0] == TensorDim(1, 1, 7, 1024));
+    auto biased = ctx->createLayerObject("tie_word_embeddings", {"unit=4096"});
+    EXPECT_THROW(biased->finalize(ic), exception::not_supported);
+  }
+  /* the other MoE layers: request order and virtual tensors */
+  {
+    auto cached = ctx->createLayerObject(
+      "moe_cached_slim", {"num_experts=4", "num_experts_per_token=2", "unit=256", "moe_activation=swish"});
+    EXPECT(cached && cached->getType() == "moe_cached_slim");
+    InitLayerContext ic({TensorDim(1, 1, 5, 512)}, "m", Tformat::NCHW, Tdatatype::Q4_K, Tdatatype::FP32);
+    cached->finalize(ic);
+    EXPECT(ic.getWeightRequests().size() == 13);
+    EXPECT(!ic.getWeightRequests()[0].is_virtual && ic.getWeightRequests()[1].is_virtual &&
+           ic.getWeightRequests()[12].is_virtual);
+    auto oss = ctx->createLayerObject("gpt_oss_moe", {"num_experts=4", "num_experts_per_token=2", "unit=256"});
+    EXPECT(oss && oss->getType() == "gpt_oss_moe");
+    InitLayerContext io({TensorDim(1, 1, 5, 512)}, "g", Tformat::NCHW, Tdatatype::Q4_K, Tdatatype::FP32);
+    oss->finalize(io);
+    const auto &w = io.getWeightRequests();
+    EXPECT(w.size() == 2 + 6 * 4);
+    EXPECT(w[0].name == "g:gate" && w[1].name == "g:gate_bias" && w[1].dim == TensorDim(1, 1, 1, 4));
+    EXPECT(w[2].name == "g:expert_up_0" && w[3].name == "g:expert_up_bias_0" && w[3].dim == TensorDim(1, 1, 1, 256));
+    EXPECT(w[4].name == "g:expert_gate_0" && w[5].name == "g:expert_gate_bias_0");
+    EXPECT(w[6].name == "g:expert_down_0" && w[7].name == "g:expert_down_bias_0" &&
+           w[7].dim == TensorDim(1, 1, 1, 512) && w[7].dim.getDataType() == Tdatatype::FP32);
+    EXPECT(!w[2].is_virtual);
+    auto both = ctx->createLayerObject("gpt_oss_moe_slim_cached",
+                                       {"num_experts=4", "num_experts_per_token=2", "unit=256"});
+    InitLayerContext ib({TensorDim(1, 1, 5, 512)}, "b", Tformat::NCHW, Tdatatype::Q4_K, Tdatatype::FP32);
+    both->finalize(ib);
+    EXPECT(ib.getWeightRequests().size() == 26 && ib.getWeightRequests()[3].is_virtual &&
+           !ib.getWeightRequests()[1].is_virtual);
+  }
   /* inference only */
   {
     RunLayerContext rc;
@@ -281,6 +359,103 @@ static int run_moe(Context *ctx, char **a) {
   return 0;
 }
 
+static int run_moex(Context *ctx, char **a) {
+  const std::string type = a[0], dt = a[1];
+  const unsigned T = std::atoi(a[2]), H = std::atoi(a[3]), I = std::atoi(a[4]), E = std::atoi(a[5]),
+                 k = std::atoi(a[6]), incremental = std::atoi(a[7]);
+  const std::string wpath = a[8], ipath = a[9], opath = a[10];
+  std::vector<std::string> props = {"num_experts=" + std::to_string(E), "num_experts_per_token=" + std::to_string(k),
+                                    "unit=" + std::to_string(I)};
+  if (type.find("gpt_oss") == std::string::npos)
+    props.push_back("moe_activation=swish");
+  auto layer = ctx->createLayerObject(type, props);
+  InitLayerContext ic({TensorDim(1, 1, T, H)}, "moe", Tformat::NCHW, dtype_of(dt), Tdatatype::FP32);
+  layer->finalize(ic);
+  RunLayerContext rc(ic);
+  {
+    std::ifstream f(wpath, std::ios::binary);
+    layer->read(f, rc, false, ml::train::ExecutionMode::INFERENCE, false, dtype_of(dt), false);
+  }
+  read_into(ipath, rc.getInput(0).getData<float>(), (size_t)T * H * 4);
+  float *out = rc.getOutput(0).getData<float>();
+  for (size_t i = 0; i < (size_t)T * H; ++i)
+    out[i] = -12345.f;
+  for (int rep = 0; rep < 2; ++rep) { /* the second run finds cached experts resident */
+    if (incremental)
+      layer->incremental_forwarding(rc, 0, T, false);
+    else
+      layer->forwarding(rc, false);
+  }
+  write_from(opath, out, (size_t)T * H * 4);
+  /* a cached layer leaves its virtual expert tensors deactivated */
+  unsigned active_virtual = 0;
+  for (unsigned i = 0; i < rc.getNumWeights(); ++i)
+    if (ic.getWeightRequests()[i].is_virtual && rc.getWeight(i).getData<uint8_t>() != nullptr)
+      ++active_virtual;
+  std::printf("MOEX DONE active_virtual=%u\n", active_virtual);
+  return 0;
+}
+
+static int run_qkv(Context *ctx, char **a) {
+  const std::string dt = a[0];
+  const unsigned K = std::atoi(a[1]), Nq = std::atoi(a[2]), Nk = std::atoi(a[3]), Nv = std::atoi(a[4]),
+                 height = std::atoi(a[5]), from = std::atoi(a[6]), to = std::atoi(a[7]);
+  const std::string wpath = a[8], ipath = a[9], opath = a[10];
+  auto layer = ctx->createLayerObject("qkv_layer", {"q_unit=" + std::to_string(Nq), "k_unit=" + std::to_string(Nk),
+                                                     "v_unit=" + std::to_string(Nv)});
+  InitLayerContext ic({TensorDim(1, 1, height, K)}, "qkv", Tformat::NCHW, dtype_of(dt), Tdatatype::FP32);
+  layer->finalize(ic);
+  RunLayerContext rc(ic);
+  {
+    std::ifstream f(wpath, std::ios::binary);
+    layer->read(f, rc, false, ml::train::ExecutionMode::INFERENCE, false, dtype_of(dt), false);
+  }
+  read_into(ipath, rc.getInput(0).getData<float>(), (size_t)height * K * 4);
+  const unsigned N[3] = {Nq, Nk, Nv};
+  for (int o = 0; o < 3; ++o) {
+    float *out = rc.getOutput(o).getData<float>();
+    for (size_t i = 0; i < (size_t)height * N[o]; ++i)
+      out[i] = -12345.f; /* rows a step does not write keep this value */
+  }
+  layer->forwarding(rc, false); /* a no-op in this layer */
+  layer->incremental_forwarding(rc, from, to, false);
+  std::ofstream f(opath, std::ios::binary);
+  for (int o = 0; o < 3; ++o)
+    f.write(rc.getOutput(o).getData<char>(), (size_t)height * N[o] * 4);
+  std::printf("QKV DONE\n");
+  return 0;
+}
+
+static int run_tie(Context *ctx, bool lmhead, char **a) {
+  const std::string dt = a[0];
+  const unsigned d0 = std::atoi(a[1]), d1 = std::atoi(a[2]), batch = std::atoi(a[3]), len = std::atoi(a[4]),
+                 from = std::atoi(a[5]), to = std::atoi(a[6]);
+  const std::string tpath = a[7], ipath = a[8], opath = a[9];
+  std::unique_ptr<Layer> layer;
+  std::vector<TensorDim> in;
+  if (lmhead) { /* d0 = K, d1 = unit, len = height */
+    layer = ctx->createLayerObject("tie_word_embeddings", {"unit=" + std::to_string(d1), "disable_bias=true"});
+    in = {TensorDim(batch, 1, len, d0)};
+  } else { /* d0 = in_dim, d1 = out_dim, len = ids per batch entry */
+    layer = ctx->createLayerObject("tie_word_embeddings",
+                                   {"in_dim=" + std::to_string(d0), "out_dim=" + std::to_string(d1)});
+    in = {TensorDim(batch, 1, 1, len)};
+  }
+  InitLayerContext ic(in, "tie", Tformat::NCHW, dtype_of(dt), Tdatatype::FP32);
+  layer->finalize(ic);
+  RunLayerContext rc(ic);
+  read_into(tpath, rc.getWeight(0).getData<uint8_t>(), mirror_tensor_bytes(rc.getWeight(0).getDim()));
+  read_into(ipath, rc.getInput(0).getData<float>(), rc.getInput(0).size() * 4);
+  float *out = rc.getOutput(0).getData<float>();
+  const size_t n_out = rc.getOutput(0).size();
+  for (size_t i = 0; i < n_out; ++i)
+    out[i] = -12345.f;
+  layer->incremental_forwarding(rc, from, to, false);
+  write_from(opath, out, n_out * 4);
+  std::printf("TIE DONE\n");
+  return 0;
+}
+
 int main(int argc, char **argv) {
   if (argc < 3) {
     std::printf("usage: %s <plugin.so> api | fc ... | moe ...\n", argv[0]);
@@ -297,6 +472,12 @@ int main(int argc, char **argv) {
       return run_moe(ctx, argv + 3);
     if (mode == "fcreload" && argc == 13)
       return run_fc_reload(ctx, argv + 3);
+    if (mode == "moex" && argc == 14)
+      return run_moex(ctx, argv + 3);
+    if (mode == "qkv" && argc == 14)
+      return run_qkv(ctx, argv + 3);
+    if ((mode == "lmhead" || mode == "embed") && argc == 13)
+      return run_tie(ctx, mode == "lmhead", argv + 3);
     std::printf("bad arguments for mode %s (argc %d)\n", mode.c_str(), argc);
     return 2;
   } catch (const std::exception &e) {

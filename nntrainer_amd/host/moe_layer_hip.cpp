@@ -5,12 +5,19 @@
  */
 #include "moe_layer_hip.h"
 
-#include "hipq_host.h"
+#include <cstring>
+
+#include "layer_common.h"
 #include "layer_props.h"
 
 namespace nntrainer {
 
 static constexpr unsigned int SINGLE_INOUT_IDX = 0;
+
+MoELayerHip::~MoELayerHip() {
+  for (hipq_weight_t w : resident)
+    hipq_host::release(w);
+}
 
 void MoELayerHip::setProperty(const std::vector<std::string> &values) {
   for (const auto &kv : hipq_host::split_properties(values)) {
@@ -76,11 +83,17 @@ void MoELayerHip::finalize(InitLayerContext &context) {
     << "hidden " << hidden << " and unit " << intermediate << " must be multiples of the quantization block "
     << block;
 
-  /* 1. router weight, always fp32 */
+  /* 1. router weight, always fp32 (and its bias: gpt_oss_moe_layer.cpp:94-101) */
   TensorDim gate_dim(1, 1, hidden, num_experts,
                      TensorDim::TensorType(context.getFormat(), Tdatatype::FP32), 0b0011);
   gate_idx = context.requestWeight(gate_dim, Initializer::NONE, WeightRegularizer::NONE, 1.0f, 0.0f,
                                    "gate", true);
+  if (gpt_oss) {
+    TensorDim gate_bias_dim(1, 1, 1, num_experts,
+                            TensorDim::TensorType(context.getFormat(), context.getActivationDataType()));
+    gate_bias_idx = context.requestWeight(gate_bias_dim, Initializer::NONE, WeightRegularizer::NONE, 1.0f, 0.0f,
+                                          "gate_bias", false);
+  }
 
   /* 2. experts, in the order the model file stores them: up, gate, down */
   expert_gate_proj_indices.clear();
@@ -96,16 +109,30 @@ void MoELayerHip::finalize(InitLayerContext &context) {
   TensorDim expert_down_dim(1, 1, intermediate, hidden,
                             TensorDim::TensorType(context.getFormat(), context.getWeightDataType()),
                             0b0011);
+  /* the cached layers request their expert tensors as virtual ones
+   * (qwen_moe_layer_cached.cpp:134-152, gpt_oss_moe_layer_cached.cpp:140-173); the gpt_oss
+   * layers put each projection's bias right behind it (gpt_oss_moe_layer.cpp:136-169) */
+  expert_gate_bias_indices.clear();
+  expert_up_bias_indices.clear();
+  expert_down_bias_indices.clear();
+  const TensorDim::TensorType act_type(context.getFormat(), context.getActivationDataType());
+  TensorDim expert_gate_bias_dim(1, 1, 1, intermediate, act_type, 0b0011);
+  TensorDim expert_down_bias_dim(1, 1, 1, hidden, act_type, 0b0011);
+  auto request = [&](const TensorDim &dim, const std::string &name) {
+    return context.requestWeight(dim, Initializer::NONE, WeightRegularizer::NONE, 1.0f, 0.0f, name, false,
+                                 cached);
+  };
   for (unsigned int i = 0; i < num_experts; ++i) {
-    expert_up_proj_indices.push_back(
-      context.requestWeight(expert_gate_dim, Initializer::NONE, WeightRegularizer::NONE, 1.0f, 0.0f,
-                            "expert_up_" + std::to_string(i), false));
-    expert_gate_proj_indices.push_back(
-      context.requestWeight(expert_gate_dim, Initializer::NONE, WeightRegularizer::NONE, 1.0f, 0.0f,
-                            "expert_gate_" + std::to_string(i), false));
-    expert_down_proj_indices.push_back(
-      context.requestWeight(expert_down_dim, Initializer::NONE, WeightRegularizer::NONE, 1.0f, 0.0f,
-                            "expert_down_" + std::to_string(i), false));
+    const std::string n = std::to_string(i);
+    expert_up_proj_indices.push_back(request(expert_gate_dim, "expert_up_" + n));
+    if (gpt_oss)
+      expert_up_bias_indices.push_back(request(expert_gate_bias_dim, "expert_up_bias_" + n));
+    expert_gate_proj_indices.push_back(request(expert_gate_dim, "expert_gate_" + n));
+    if (gpt_oss)
+      expert_gate_bias_indices.push_back(request(expert_gate_bias_dim, "expert_gate_bias_" + n));
+    expert_down_proj_indices.push_back(request(expert_down_dim, "expert_down_" + n));
+    if (gpt_oss)
+      expert_down_bias_indices.push_back(request(expert_down_bias_dim, "expert_down_bias_" + n));
   }
 
   /* 3. the scratch tensors of the CPU layer, kept so that tensor indices and
@@ -120,32 +147,93 @@ void MoELayerHip::finalize(InitLayerContext &context) {
 }
 
 void MoELayerHip::run(RunLayerContext &context, const float *x, float *y, unsigned int tokens,
-                      bool renormalize) const {
-  std::vector<const void *> g(num_experts), u(num_experts), d(num_experts);
-  for (unsigned int e = 0; e < num_experts; ++e) {
-    g[e] = context.getWeight(expert_gate_proj_indices[e]).getData<uint8_t>();
-    u[e] = context.getWeight(expert_up_proj_indices[e]).getData<uint8_t>();
-    d[e] = context.getWeight(expert_down_proj_indices[e]).getData<uint8_t>();
-  }
-  const float *router = context.getWeight(gate_idx).getData<float>();
+                      bool renormalize, bool with_router_bias) {
+  const unsigned int E = num_experts;
   hipq_host::MoeShape shape;
   shape.tokens = (int)tokens;
   shape.hidden = (int)hidden;
   shape.intermediate = (int)intermediate;
-  shape.experts = (int)num_experts;
+  shape.experts = (int)E;
   shape.topk = (int)topk;
   shape.renormalize = renormalize;
-  hipq_host::moe_forward(hipq_host::global_cache(), shape, weight_dtype, g, u, d, x, router, y);
+  const float *router = context.getWeight(gate_idx).getData<float>();
+
+  /* a virtual tensor has bytes only between activate() and deactivate() */
+  auto with_bytes = [&](unsigned int idx, auto use) {
+    Tensor &t = context.getWeight(idx);
+    if (cached)
+      t.activate();
+    use(t);
+    if (cached)
+      t.deactivate();
+  };
+
+  hipq_host::MoeExtras extras;
+  if (gpt_oss) {
+    bias_gate.resize((size_t)E * intermediate);
+    bias_up.resize((size_t)E * intermediate);
+    bias_down.resize((size_t)E * hidden);
+    for (unsigned int e = 0; e < E; ++e) {
+      with_bytes(expert_gate_bias_indices[e], [&](Tensor &t) {
+        std::memcpy(&bias_gate[(size_t)e * intermediate], t.getData<float>(), (size_t)intermediate * 4);
+      });
+      with_bytes(expert_up_bias_indices[e], [&](Tensor &t) {
+        std::memcpy(&bias_up[(size_t)e * intermediate], t.getData<float>(), (size_t)intermediate * 4);
+      });
+      with_bytes(expert_down_bias_indices[e], [&](Tensor &t) {
+        std::memcpy(&bias_down[(size_t)e * hidden], t.getData<float>(), (size_t)hidden * 4);
+      });
+    }
+    extras.gpt_oss = true;
+    extras.alpha = 1.702f; /* gpt_oss_moe_layer.h:126 */
+    extras.gate_bias = bias_gate.data();
+    extras.up_bias = bias_up.data();
+    extras.down_bias = bias_down.data();
+    extras.router_bias = with_router_bias ? context.getWeight(gate_bias_idx).getData<float>() : nullptr;
+  }
+
+  if (cached) {
+    /* every expert once into HBM, where it stays: the reference's 32-entry LRU over host
+     * memory (qwen_moe_layer_cached.cpp:376-454) has nothing to manage here */
+    if (resident.empty()) {
+      resident.assign(3 * (size_t)E, nullptr);
+      const int layout = hipq_host::framework_layout(weight_dtype);
+      const hipq_host::WeightSpec gu{weight_dtype, layout, (int64_t)intermediate, (int64_t)hidden};
+      const hipq_host::WeightSpec dn{weight_dtype, layout, (int64_t)hidden, (int64_t)intermediate};
+      for (unsigned int e = 0; e < E; ++e) {
+        with_bytes(expert_gate_proj_indices[e],
+                   [&](Tensor &t) { resident[e] = hipq_host::upload(t.getData<uint8_t>(), gu); });
+        with_bytes(expert_up_proj_indices[e],
+                   [&](Tensor &t) { resident[E + e] = hipq_host::upload(t.getData<uint8_t>(), gu); });
+        with_bytes(expert_down_proj_indices[e],
+                   [&](Tensor &t) { resident[2 * (size_t)E + e] = hipq_host::upload(t.getData<uint8_t>(), dn); });
+      }
+    }
+    hipq_host::moe_forward_resident(shape, resident.data(), resident.data() + E, resident.data() + 2 * (size_t)E,
+                                    x, router, y, &extras);
+    return;
+  }
+
+  std::vector<const void *> g(E), u(E), d(E);
+  for (unsigned int e = 0; e < E; ++e) {
+    g[e] = context.getWeight(expert_gate_proj_indices[e]).getData<uint8_t>();
+    u[e] = context.getWeight(expert_up_proj_indices[e]).getData<uint8_t>();
+    d[e] = context.getWeight(expert_down_proj_indices[e]).getData<uint8_t>();
+  }
+  hipq_host::moe_forward(hipq_host::global_cache(), shape, weight_dtype, g, u, d, x, router, y, &extras);
 }
 
 void MoELayerHip::forwarding(RunLayerContext &context, bool training) {
   NNTR_THROW_IF(training, exception::not_supported) << "MoELayerHip is an inference layer";
+  if (cached) /* the cached layers run by steps only (qwen_moe_layer_cached.cpp:173-174) */
+    return;
   Tensor &input_ = context.getInput(SINGLE_INOUT_IDX);
   Tensor &output_ = context.getOutput(SINGLE_INOUT_IDX);
   const unsigned int total_tokens = input_.batch() * input_.height();
-  /* the whole-tensor path keeps the softmax weights as they are
-   * (qwen_moe_layer.cpp:161-259 does not renormalise) */
-  run(context, input_.getData<float>(), output_.getData<float>(), total_tokens, false);
+  /* the whole-tensor path keeps the softmax weights as they are (qwen_moe_layer.cpp:161-259
+   * does not renormalise) and, in the gpt_oss layer, leaves the router bias out
+   * (gpt_oss_moe_layer.cpp:209-212) */
+  run(context, input_.getData<float>(), output_.getData<float>(), total_tokens, false, false);
 }
 
 void MoELayerHip::incremental_forwarding(RunLayerContext &context, unsigned int from,
@@ -171,7 +259,9 @@ void MoELayerHip::incremental_forwarding(RunLayerContext &context, unsigned int 
       input_.getSharedDataTensor(input_step_dim, b * input_.getDim().getFeatureLen(), true);
     Tensor output =
       output_.getSharedDataTensor(output_step_dim, b * output_.getDim().getFeatureLen(), true);
-    run(context, input.getData<float>(), output.getData<float>(), to - from, true);
+    /* of the two gpt_oss layers only the uncached one adds the router bias
+     * (gpt_oss_moe_layer.cpp:500-504 against gpt_oss_moe_layer_cached.cpp:243-246) */
+    run(context, input.getData<float>(), output.getData<float>(), to - from, true, gpt_oss && !cached);
   }
 }
 
@@ -183,10 +273,13 @@ void MoELayerHip::calcGradient(RunLayerContext &) {
   throw exception::not_supported("MoELayerHip does not support backwarding");
 }
 
-static void drop_device_copies(RunLayerContext &run_context) {
-  for (unsigned int i = 0; i < run_context.getNumWeights(); ++i)
-    hipq_host::global_cache().invalidate(run_context.getWeight(i).getData<uint8_t>());
-}
+/* of a cached layer also the copies it holds itself: the next step uploads again */
+#define HIPQ_MOE_DROP_RESIDENT()                                                                    \
+  do {                                                                                              \
+    for (hipq_weight_t w : resident)                                                                \
+      hipq_host::release(w);                                                                        \
+    resident.clear();                                                                               \
+  } while (0)
 
 void MoELayerHip::read(std::ifstream &file, RunLayerContext &run_context, bool opt_var,
                    ml::train::ExecutionMode mode, bool trainable, TensorDim::DataType defineWeightDataType,
@@ -194,6 +287,7 @@ void MoELayerHip::read(std::ifstream &file, RunLayerContext &run_context, bool o
   Layer::read(file, run_context, opt_var, mode, trainable, defineWeightDataType, fsu, start_offset,
               read_from_offset, file_fd);
   drop_device_copies(run_context);
+  HIPQ_MOE_DROP_RESIDENT();
 }
 
 void MoELayerHip::read(ReadSource src, RunLayerContext &run_context, bool opt_var, ml::train::ExecutionMode mode,
@@ -202,6 +296,7 @@ void MoELayerHip::read(ReadSource src, RunLayerContext &run_context, bool opt_va
   Layer::read(src, run_context, opt_var, mode, trainable, defineWeightDataType, fsu, start_offset,
               read_from_offset);
   drop_device_copies(run_context);
+  HIPQ_MOE_DROP_RESIDENT();
 }
 
 } // namespace nntrainer

@@ -155,7 +155,9 @@ public:
   void read(std::ifstream &file, size_t start_offset = 0, bool read_from_offset = false, int /*file_fd*/ = -1) {
     if (read_from_offset)
       file.seekg((std::streamoff)start_offset);
-    file.read(getData<char>(), (std::streamsize)mirror_tensor_bytes(dim));
+    /* a virtual tensor only notes where its bytes are (tensor.cpp, read of a virtual tensor) */
+    char *dst = is_virtual ? reinterpret_cast<char *>(this->file->data()) : getData<char>();
+    file.read(dst, (std::streamsize)mirror_tensor_bytes(dim));
     NNTR_THROW_IF(file.fail(), std::runtime_error) << "short read of a tensor";
   }
   void read(ReadSource src, size_t start_offset = 0, bool read_from_offset = false) {
@@ -165,6 +167,25 @@ public:
 
   Tensor() = default;
   explicit Tensor(const TensorDim &d) : dim(d), store(std::make_shared<std::vector<uint8_t>>(mirror_tensor_bytes(d))) {}
+  /** a virtual tensor (requestWeight(..., is_virtual = true)): its bytes live in the model file
+   *  until activate() maps them in and are gone again after deactivate() (tensor.h:1979-1993).
+   *  Here the "file" is a second buffer that a test fills through mirror_file_bytes(). */
+  static Tensor make_virtual(const TensorDim &d) {
+    Tensor t;
+    t.dim = d;
+    t.is_virtual = true;
+    t.file = std::make_shared<std::vector<uint8_t>>(mirror_tensor_bytes(d));
+    return t;
+  }
+  void activate() {
+    if (is_virtual && !store)
+      store = std::make_shared<std::vector<uint8_t>>(*file);
+  }
+  void deactivate() {
+    if (is_virtual)
+      store.reset();
+  }
+  uint8_t *mirror_file_bytes() { return file ? file->data() : nullptr; }
   Tensor(size_t b, size_t c, size_t h, size_t w, TensorDim::TensorType t = TensorDim::TensorType()) :
     Tensor(TensorDim(b, c, h, w, t)) {}
 
@@ -222,6 +243,8 @@ private:
   TensorDim dim;
   std::shared_ptr<std::vector<uint8_t>> store;
   size_t offset_bytes = 0;
+  bool is_virtual = false;
+  std::shared_ptr<std::vector<uint8_t>> file;
 };
 
 /** What a layer declares in finalize(): weights and scratch tensors by spec. */
@@ -231,6 +254,7 @@ public:
     TensorDim dim;
     std::string name;
     bool trainable;
+    bool is_virtual;
   };
   struct TensorRequest {
     TensorDim dim;
@@ -254,8 +278,8 @@ public:
 
   unsigned int requestWeight(const TensorDim &dim, const Initializer, const WeightRegularizer,
                              const float, const float, const std::string &name, bool trainable = true,
-                             bool = false, unsigned int = 3) {
-    weights.push_back({dim, prefix + ":" + name, trainable});
+                             bool is_virtual = false, unsigned int = 3) {
+    weights.push_back({dim, prefix + ":" + name, trainable, is_virtual});
     return weights.size() - 1;
   }
   unsigned int requestTensor(const TensorDim &dim, const std::string &name,
@@ -288,7 +312,7 @@ public:
     for (auto &d : init.getOutputDimensions())
       outputs.emplace_back(d);
     for (auto &w : init.getWeightRequests())
-      weights.emplace_back(w.dim);
+      weights.push_back(w.is_virtual ? Tensor::make_virtual(w.dim) : Tensor(w.dim));
     for (auto &t : init.getTensorRequests())
       tensors.emplace_back(t.dim);
   }

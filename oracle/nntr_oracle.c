@@ -856,9 +856,11 @@ static void gemv_serial(int kind, int N, int K, const float *a, const uint8_t *w
  * h = (sigmoid(g) * g) * u with sigmoid evaluated in double and cast
  * (nntrainer/layers/acti_func.h:286-288, 400-405), o = h.Wdown, contribution =
  * o * weight. Contributions are added into y in ascending expert order. */
-void orc_moe_forward(int kind, int renormalize, int T, int H, int I, int E, int topk, const float *x,
-                     const float *logits, const void *const *gate, const void *const *up,
-                     const void *const *down, float *y, int32_t *topk_idx, float *topk_w) {
+static void moe_forward_impl(int kind, int renormalize, int T, int H, int I, int E, int topk, const float *x,
+                             const float *logits, const void *const *gate, const void *const *up,
+                             const void *const *down, const float *gate_bias, const float *up_bias,
+                             const float *down_bias, int gpt_oss, float alpha, float *y, int32_t *topk_idx,
+                             float *topk_w) {
   int32_t *idx = (int32_t *)malloc(sizeof(int32_t) * (size_t)T * topk);
   float *wt = (float *)malloc(sizeof(float) * (size_t)T * topk);
   float *p = (float *)malloc(sizeof(float) * (size_t)E);
@@ -911,12 +913,26 @@ void orc_moe_forward(int kind, int renormalize, int T, int H, int I, int E, int 
       float *o = contrib + (size_t)pr * H;
       gemv_serial(kind, I, H, xt, (const uint8_t *)gate[e], g, qa);
       gemv_serial(kind, I, H, xt, (const uint8_t *)up[e], u, qa);
-      for (int i = 0; i < I; ++i) {
-        const float en = (float)exp((double)(-g[i]));
-        const float sig = (float)(1.0 / (1.0 + (double)en));
-        h[i] = (sig * g[i]) * u[i];
+      if (gpt_oss) {
+        /* gpt_oss_moe_layer.cpp:406-437: biases added to the finished products, one added to
+         * up, then swiglu with alpha = (Y / (1 + exp(-alpha Y))) * Z in fp32
+         * (fallback_internal.cpp:425-432), Y = gate, Z = up + 1 */
+        for (int i = 0; i < I; ++i) {
+          const float gi = g[i] + gate_bias[(size_t)e * I + i];
+          float ui = u[i] + up_bias[(size_t)e * I + i];
+          ui = ui + 1.f;
+          h[i] = (gi / (1.f + expf(-alpha * gi))) * ui;
+        }
+      } else {
+        for (int i = 0; i < I; ++i) {
+          const float en = (float)exp((double)(-g[i]));
+          const float sig = (float)(1.0 / (1.0 + (double)en));
+          h[i] = (sig * g[i]) * u[i];
+        }
       }
       gemv_serial(kind, H, I, h, (const uint8_t *)down[e], o, qa);
+      if (gpt_oss) /* gpt_oss_moe_layer.cpp:441: token_expert_output.add_i(down_bias), then the weight */
+        for (int c = 0; c < H; ++c) o[c] = o[c] + down_bias[(size_t)e * H + c];
       for (int c = 0; c < H; ++c) o[c] = o[c] * wt[pr];
     }
     free(qa);
@@ -938,6 +954,27 @@ void orc_moe_forward(int kind, int renormalize, int T, int H, int I, int E, int 
   free(contrib);
   free(idx);
   free(wt);
+}
+
+void orc_moe_forward(int kind, int renormalize, int T, int H, int I, int E, int topk, const float *x,
+                     const float *logits, const void *const *gate, const void *const *up,
+                     const void *const *down, float *y, int32_t *topk_idx, float *topk_w) {
+  moe_forward_impl(kind, renormalize, T, H, I, E, topk, x, logits, gate, up, down, NULL, NULL, NULL, 0, 0.f, y,
+                   topk_idx, topk_w);
+}
+
+/* GptOssMoELayer::incremental_forwarding (gpt_oss_moe_layer.cpp:452-568) with the expert of
+ * compute_expert_forward_no_critical (:372-449). logits already hold the router bias.
+ * gate_bias, up_bias [E][I]; down_bias [E][H]. The reference accumulates weight * expert output
+ * per expert and then adds the experts in ascending order, which for one token is the ascending
+ * sum of its pairs, as above. */
+void orc_moe_forward_gpt_oss(int kind, int renormalize, int T, int H, int I, int E, int topk, const float *x,
+                             const float *logits, const void *const *gate, const void *const *up,
+                             const void *const *down, const float *gate_bias, const float *up_bias,
+                             const float *down_bias, float alpha, float *y, int32_t *topk_idx,
+                             float *topk_w) {
+  moe_forward_impl(kind, renormalize, T, H, I, E, topk, x, logits, gate, up, down, gate_bias, up_bias, down_bias,
+                   1, alpha, y, topk_idx, topk_w);
 }
 
 void orc_moe_forward_q4_K(int T, int H, int I, int E, int topk, const float *x,

@@ -103,6 +103,11 @@ void orc_moe_forward(int kind /* 2 Q4_0, 12 Q4_K, 14 Q6_K */, int renormalize /*
                      const float *x, const float *logits, const void *const *gate,
                      const void *const *up, const void *const *down, float *y, int32_t *topk_idx,
                      float *topk_w);
+void orc_moe_forward_gpt_oss(int kind, int renormalize, int T, int H, int I, int E, int topk, const float *x,
+                             const float *logits, const void *const *gate, const void *const *up,
+                             const void *const *down, const float *gate_bias, const float *up_bias,
+                             const float *down_bias, float alpha, float *y, int32_t *topk_idx,
+                             float *topk_w);
 void orc_moe_forward_q4_K(int T, int H, int I, int E, int topk, const float *x,
                           const float *logits, const void *const *gate,
                           const void *const *up, const void *const *down,

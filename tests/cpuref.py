@@ -210,3 +210,25 @@ def moe_forward(x, logits, gate, up, down, topk, kind="q4_K", renormalize=True):
                         _i32(h), _i32(i), _i32(e), _i32(topk), _ptr(x), _ptr(logits), arr(gate), arr(up),
                         arr(down), _ptr(y), _ptr(idx), _ptr(wt))
     return y, idx, wt
+
+
+def moe_forward_gpt_oss(x, logits, gate, up, down, gate_bias, up_bias, down_bias, topk, alpha=1.702, kind="q4_K",
+                        renormalize=True):
+    """Oracle GPT-OSS MoE block; logits already hold the router bias. Biases [E, I], [E, I], [E, H]."""
+    lib = oracle()
+    x = np.ascontiguousarray(x, np.float32)
+    logits = np.ascontiguousarray(logits, np.float32)
+    gb, ub, db = (np.ascontiguousarray(b, np.float32) for b in (gate_bias, up_bias, down_bias))
+    t, h = x.shape
+    e = logits.shape[1]
+    nbytes, blk = BLOCK_BYTES[kind]
+    i = gate[0].size // ((h // blk) * nbytes)
+    arr = lambda lst: (_c.c_void_p * e)(*[w.ctypes.data for w in lst])
+    y = np.zeros((t, h), np.float32)
+    idx = np.zeros((t, topk), np.int32)
+    wt = np.zeros((t, topk), np.float32)
+    lib.orc_moe_forward_gpt_oss(_i32({"q4_0": 2, "q4_K": 12, "q6_K": 14}[kind]), _i32(1 if renormalize else 0),
+                                _i32(t), _i32(h), _i32(i), _i32(e), _i32(topk), _ptr(x), _ptr(logits), arr(gate),
+                                arr(up), arr(down), _ptr(gb), _ptr(ub), _ptr(db), _c.c_float(alpha), _ptr(y),
+                                _ptr(idx), _ptr(wt))
+    return y, idx, wt

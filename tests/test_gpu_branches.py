@@ -98,3 +98,72 @@ def test_router_with_nan_logits_stays_in_range(hipq, cr):
         w.destroy()
     assert ((got >= 0) & (got < e)).all(), got
     assert all(len(set(r)) == k for r in got.tolist())
+
+
+def _gpt_oss_case(cr, kind, t, h, i, e, k, seed):
+    gate, up, down = _experts(cr, kind, e, i, h, seed)
+    x = synth.normal(seed + 500, (t, h))
+    gb = synth.normal(seed + 502, (e, i), 0.3)
+    ub = synth.normal(seed + 503, (e, i), 0.3)
+    db = synth.normal(seed + 504, (e, h), 0.3)
+    return gate, up, down, x, gb, ub, db
+
+
+@pytest.mark.parametrize("kind,t,h,i,e,k", [("q4_K", 8, 256, 256, 8, 2), ("q4_K", 64, 512, 256, 16, 4),
+                                            ("q4_K", 1, 2048, 768, 16, 4), ("q4_0", 9, 256, 512, 8, 4),
+                                            ("q6_K", 5, 512, 256, 4, 2)])
+def test_gpt_oss_moe_matches_oracle(hipq, cr, kind, t, h, i, e, k):
+    """hipq_moe_forward_ext, GPT-OSS variant (gpt_oss_moe_layer.cpp:372-449, 452-568): biased
+    projections, swiglu with alpha on (gate, up + 1), biased down projection. The integer and
+    fp32 chains of the three products carry the reference's bits; the exponential is the device's
+    expf against the host's, so the bar is the fp32 tolerance, not bit identity."""
+    import gpu_util as gu
+    import torch
+    gate, up, down, x, gb, ub, db = _gpt_oss_case(cr, kind, t, h, i, e, k, 7600)
+    logits = synth.normal(7601, (t, e))
+    ref_y, ref_idx, ref_w = cr.moe_forward_gpt_oss(x, logits, gate, up, down, gb, ub, db, k, kind=kind)
+    wg = [capi.Weight(kind, i, h, b) for b in gate]
+    wu = [capi.Weight(kind, i, h, b) for b in up]
+    wd = [capi.Weight(kind, h, i, b) for b in down]
+    y = torch.full((t, h), float("nan"), device="cuda")
+    idx = torch.zeros((t, k), dtype=torch.int32, device="cuda")
+    capi.moe_forward_gpt_oss(t, h, i, e, k, wg, wu, wd, gu.dev(x), y, gu.dev(gb), gu.dev(ub), gu.dev(db),
+                             router_logits=gu.dev(logits), topk_idx=idx, stream=gu.stream())
+    torch.cuda.synchronize()
+    got = y.cpu().numpy()
+    assert np.array_equal(idx.cpu().numpy(), ref_idx)
+    assert not np.isnan(got).any()
+    assert gu.rel_err(got, ref_y) <= gu.TOL, gu.rel_err(got, ref_y)
+    # the biases and the + 1 matter at this size: without them the result is far off
+    plain, _, _ = cr.moe_forward(x, logits, gate, up, down, k, kind=kind)
+    assert gu.rel_err(plain, ref_y) > 0.05
+    for w in wg + wu + wd:
+        w.destroy()
+
+
+def test_gpt_oss_moe_router_bias_and_host_memory(hipq, cr):
+    """Router logits formed on the device from the fp32 router weight plus its bias
+    (gpt_oss_moe_layer.cpp:500-503), all operands in host memory."""
+    import gpu_util as gu
+    kind, t, h, i, e, k = "q4_K", 6, 256, 256, 8, 2
+    gate, up, down, x, gb, ub, db = _gpt_oss_case(cr, kind, t, h, i, e, k, 7700)
+    wr = synth.normal(7701, (h, e), 0.1)
+    rb = synth.normal(7702, (e,), 2.0)  # large enough to change the routing
+    logits = ((x.astype(np.float64) @ wr.astype(np.float64)).astype(np.float32) + rb).astype(np.float32)
+    ref_y, ref_idx, _ = cr.moe_forward_gpt_oss(x, logits, gate, up, down, gb, ub, db, k, kind=kind)
+    _, idx_without, _ = cr.moe_forward_gpt_oss(x, logits - rb, gate, up, down, gb, ub, db, k, kind=kind)
+    assert not np.array_equal(ref_idx, idx_without), "the bias must change the routing of the case"
+    wg = [capi.Weight(kind, i, h, b) for b in gate]
+    wu = [capi.Weight(kind, i, h, b) for b in up]
+    wd = [capi.Weight(kind, h, i, b) for b in down]
+    y = np.full((t, h), np.nan, np.float32)
+    idx = np.zeros((t, k), np.int32)
+    capi.moe_forward_gpt_oss(t, h, i, e, k, wg, wu, wd, x, y, gb, ub, db, router_weight=wr, router_bias=rb,
+                             topk_idx=idx, mem=capi.MEM_HOST)
+    assert np.array_equal(idx, ref_idx)
+    assert gu.rel_err(y, ref_y) <= 2e-4  # logits differ in the last bits
+    with pytest.raises(capi.HipqError):  # a bias for logits the caller computed is refused
+        capi.moe_forward_gpt_oss(t, h, i, e, k, wg, wu, wd, x, y, gb, ub, db, router_logits=logits, router_bias=rb,
+                                 mem=capi.MEM_HOST)
+    for w in wg + wu + wd:
+        w.destroy()

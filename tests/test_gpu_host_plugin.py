@@ -171,3 +171,156 @@ def test_moe_forwarding_keeps_softmax_values(cr, tmp_path):
     got = np.fromfile(tmp_path / "y.bin", np.float32).reshape(t, h)
     err = np.abs(got - ref_y).max() / np.abs(ref_y).max()
     assert err <= 2e-4, err  # router logits computed on the device differ in the last bits
+
+
+@pytest.mark.parametrize("kind,k,nq,nk,nv,height,frm,to", [
+    ("q4_0", 1024, 2048, 1024, 1024, 1, 7, 8),    # a decode step of the Qwen3-0.6B shape: one launch
+    ("q4_K", 1024, 512, 256, 256, 1, 0, 1),
+    ("q6_K", 512, 256, 256, 128, 1, 3, 4),
+    ("q4_0", 1024, 512, 256, 256, 24, 0, 17),    # prefill: rows [0, 17) of 24
+])
+def test_qkv_layer_matches_oracle_bit_for_bit(cr, tmp_path, kind, k, nq, nk, nv, height, frm, to):
+    """qkv_layer created through the context: three quantized products of one activation
+    (qkv_layer.cpp:132-181). Decode rows and Q4_0 prefill rows follow the reference's evaluation
+    order, so the outputs carry the oracle's bits."""
+    ws, fws = [], []
+    for j, n in enumerate((nq, nk, nv)):
+        blocks, fw = _framework_bytes(cr, kind, synth.normal(8000 + j, (n, k), 0.02), n, k)
+        ws.append(blocks)
+        fws.append(fw)
+    x = synth.normal(8010 + height, (height, k))
+    with open(tmp_path / "w.bin", "wb") as f:
+        for fw in fws:
+            f.write(fw.tobytes())
+    x.tofile(tmp_path / "x.bin")
+    out = _run(["qkv", kind, k, nq, nk, nv, height, frm, to, tmp_path / "w.bin", tmp_path / "x.bin",
+                tmp_path / "y.bin"])
+    assert "QKV DONE" in out
+    got = np.fromfile(tmp_path / "y.bin", np.float32)
+    rows, off = to - frm, 0
+    for blocks, n in zip(ws, (nq, nk, nv)):
+        y = got[off:off + height * n].reshape(height, n)
+        off += height * n
+        ref = cr.gemm(cr.oracle(), kind, x[:rows], blocks, n)
+        assert np.array_equal(y[:rows].view(np.uint32), ref.view(np.uint32))
+        assert np.all(y[rows:] == -12345.0)
+
+
+@pytest.mark.parametrize("batch,height,frm,to", [(1, 1, 11, 12), (1, 9, 0, 9), (2, 6, 0, 4)])
+def test_tied_lm_head_matches_oracle(cr, tmp_path, batch, height, frm, to):
+    """tie_word_embeddings with `unit`: hidden = input . table^T for one row per batch entry, row 0
+    of a one-token step, else the step's last row (tie_word_embedding.cpp:252-303); the table is
+    the Q6_K embedding matrix, unit rows of K values."""
+    kind, k, unit = "q6_K", 512, 1000
+    table = cr.quantize_weights(cr.oracle(), kind, synth.normal(8100, (unit, k), 0.02))
+    x = synth.normal(8101 + height, (batch, height, k))
+    table.tofile(tmp_path / "t.bin")
+    x.tofile(tmp_path / "x.bin")
+    _run(["lmhead", kind, k, unit, batch, height, frm, to, tmp_path / "t.bin", tmp_path / "x.bin",
+          tmp_path / "y.bin"])
+    got = np.fromfile(tmp_path / "y.bin", np.float32).reshape(batch, height, unit)
+    row = 0 if to - frm == 1 else to - 1
+    for b in range(batch):
+        ref = cr.gemm(cr.oracle(), kind, x[b, row:row + 1], table, unit)
+        assert np.array_equal(got[b, row].view(np.uint32), ref[0].view(np.uint32))
+        rest = np.delete(got[b], row, axis=0)
+        assert np.all(rest == -12345.0)
+
+
+@pytest.mark.parametrize("kind", ["q6_K", "fp32"])
+def test_tied_embedding_rows(cr, tmp_path, kind):
+    """tie_word_embeddings without `unit`: row `id` of the table per input id, dequantized for
+    Q6_K (tie_word_embedding.cpp:183-250). Host work; here because the same layer object type
+    serves both ends of the model."""
+    in_dim, out_dim, batch, width = 300, 512, 2, 5
+    w32 = synth.normal(8200, (in_dim, out_dim), 0.02)
+    if kind == "q6_K":
+        table = cr.quantize_weights(cr.oracle(), kind, w32)
+        rows = cr.dequantize(cr.oracle(), kind, table, in_dim * out_dim).reshape(in_dim, out_dim)
+    else:
+        table, rows = w32, w32
+    ids = np.array([[0, 299, 17, 5, 17], [1, 2, 3, 4, 250]], np.float32)
+    table.tofile(tmp_path / "t.bin")
+    ids.tofile(tmp_path / "i.bin")
+    _run(["embed", kind, in_dim, out_dim, batch, width, 0, 3, tmp_path / "t.bin", tmp_path / "i.bin",
+          tmp_path / "y.bin"])
+    got = np.fromfile(tmp_path / "y.bin", np.float32).reshape(batch, width, out_dim)
+    for b in range(batch):
+        for i in range(3):
+            assert np.array_equal(got[b, i].view(np.uint32), rows[int(ids[b, i])].view(np.uint32))
+        assert np.all(got[b, 3:] == -12345.0)
+
+
+def _moe_file(cr, path, kind, e, i, h, wr, experts, gate_bias=None, biases=None):
+    """every weight of an MoE layer in the order it requests them"""
+    gate, up, down = experts
+    with open(path, "wb") as f:
+        f.write(wr.tobytes())
+        if gate_bias is not None:
+            f.write(gate_bias.tobytes())
+        for x in range(e):
+            f.write(cr.repack_x8(cr.oracle(), kind, up[x], i, h).tobytes())
+            if biases:
+                f.write(biases[1][x].tobytes())
+            f.write(cr.repack_x8(cr.oracle(), kind, gate[x], i, h).tobytes())
+            if biases:
+                f.write(biases[0][x].tobytes())
+            f.write(cr.repack_x8(cr.oracle(), kind, down[x], h, i).tobytes())
+            if biases:
+                f.write(biases[2][x].tobytes())
+
+
+def _moe_case(cr, seed, t, h, i, e):
+    q = lambda s, shape: cr.quantize_weights(cr.oracle(), "q4_K", synth.normal(s, shape, 0.02))
+    experts = ([q(seed + 3 * x, (i, h)) for x in range(e)], [q(seed + 3 * x + 1, (i, h)) for x in range(e)],
+               [q(seed + 3 * x + 2, (h, i)) for x in range(e)])
+    xin = synth.normal(seed + 100, (t, h))
+    wr = synth.normal(seed + 101, (h, e), 0.1)
+    logits = (xin.astype(np.float64) @ wr.astype(np.float64)).astype(np.float32)
+    return experts, xin, wr, logits
+
+
+def test_cached_moe_layer(cr, tmp_path):
+    """moe_cached_slim (qwen_moe_layer_cached.cpp:266-470): virtual expert tensors, loaded through
+    Layer::read, activated once, kept in HBM and left deactivated; the result is the Qwen block's."""
+    t, h, i, e, k = 12, 512, 256, 8, 2
+    experts, xin, wr, logits = _moe_case(cr, 8300, t, h, i, e)
+    ref_y, _, _ = cr.moe_forward(xin, logits, *experts, k)
+    _moe_file(cr, tmp_path / "w.bin", "q4_K", e, i, h, wr, experts)
+    xin.tofile(tmp_path / "x.bin")
+    out = _run(["moex", "moe_cached_slim", "q4_K", t, h, i, e, k, 1, tmp_path / "w.bin", tmp_path / "x.bin",
+                tmp_path / "y.bin"])
+    assert "active_virtual=0" in out
+    got = np.fromfile(tmp_path / "y.bin", np.float32).reshape(t, h)
+    assert np.abs(got - ref_y).max() / np.abs(ref_y).max() <= 2e-4
+    # forwarding() of the cached layer is a no-op, as in the reference
+    _run(["moex", "moe_cached_slim", "q4_K", t, h, i, e, k, 0, tmp_path / "w.bin", tmp_path / "x.bin",
+          tmp_path / "y0.bin"])
+    assert np.all(np.fromfile(tmp_path / "y0.bin", np.float32) == -12345.0)
+
+
+@pytest.mark.parametrize("layer,incremental", [("gpt_oss_moe", 1), ("gpt_oss_moe", 0),
+                                               ("gpt_oss_moe_slim_cached", 1)])
+def test_gpt_oss_moe_layers(cr, tmp_path, layer, incremental):
+    """gpt_oss_moe and its cached twin through the context. The router bias enters only in the
+    uncached layer's incremental_forwarding (gpt_oss_moe_layer.cpp:500-504; not :209-212, not
+    gpt_oss_moe_layer_cached.cpp:243-246), and forwarding() keeps the softmax values as they are."""
+    t, h, i, e, k = 9, 256, 256, 8, 2
+    experts, xin, wr, logits = _moe_case(cr, 8400, t, h, i, e)
+    rb = synth.normal(8450, (e,), 2.0)
+    gb = synth.normal(8451, (e, i), 0.3)
+    ub = synth.normal(8452, (e, i), 0.3)
+    db = synth.normal(8453, (e, h), 0.3)
+    with_bias = layer == "gpt_oss_moe" and incremental == 1
+    lg = (logits + rb).astype(np.float32) if with_bias else logits
+    ref_y, ref_idx, _ = cr.moe_forward_gpt_oss(xin, lg, *experts, gb, ub, db, k, renormalize=bool(incremental))
+    other, other_idx, _ = cr.moe_forward_gpt_oss(xin, logits if with_bias else (logits + rb).astype(np.float32),
+                                                 *experts, gb, ub, db, k, renormalize=bool(incremental))
+    assert not np.array_equal(ref_idx, other_idx), "the router bias must matter in this case"
+    _moe_file(cr, tmp_path / "w.bin", "q4_K", e, i, h, wr, experts, gate_bias=rb, biases=(gb, ub, db))
+    xin.tofile(tmp_path / "x.bin")
+    out = _run(["moex", layer, "q4_K", t, h, i, e, k, incremental, tmp_path / "w.bin", tmp_path / "x.bin",
+                tmp_path / "y.bin"])
+    assert "active_virtual=0" in out
+    got = np.fromfile(tmp_path / "y.bin", np.float32).reshape(t, h)
+    assert np.abs(got - ref_y).max() / np.abs(ref_y).max() <= 2e-4

@@ -230,6 +230,48 @@ def test_moe_equals_dense_per_token_evaluation():
     assert np.abs(y0 - want * scale).max() / np.abs(want).max() < 1e-5
 
 
+def test_gpt_oss_moe_reduces_to_known_cases():
+    """The GPT-OSS block of the oracle (gpt_oss_moe_layer.cpp:372-449), pinned three ways.
+    (1) With up_bias = -1, the other biases 0 and alpha = 1 its activation is silu(g) * u: the
+    block must then equal the Qwen block, whose own pins are above (float against double
+    exponential: 1e-6). (2) alpha = 0 makes the sigmoid 1/2 whatever g is: h = g/2 * (u + 1),
+    evaluated here from the oracle's single-row products with nonzero biases; a dropped bias, a
+    missing + 1 or a bias on the wrong side of the activation fails it. (3) The down bias enters
+    after the product and before the routing weight: y(db) - y(0) = sum_k w_k db[e_k]."""
+    o = cr.oracle()
+    t, h, i, e, k = 5, 256, 256, 6, 2
+    gate = [cr.quantize_weights(o, "q4_K", synth.normal(300 + 3 * x, (i, h), 0.02)) for x in range(e)]
+    up = [cr.quantize_weights(o, "q4_K", synth.normal(301 + 3 * x, (i, h), 0.02)) for x in range(e)]
+    down = [cr.quantize_weights(o, "q4_K", synth.normal(302 + 3 * x, (h, i), 0.02)) for x in range(e)]
+    x = synth.normal(400, (t, h))
+    logits = synth.normal(401, (t, e))
+    zi, zh = np.zeros((e, i), np.float32), np.zeros((e, h), np.float32)
+    # (1)
+    y_q, idx_q, wt_q = cr.moe_forward(x, logits, gate, up, down, k)
+    y1, idx1, wt1 = cr.moe_forward_gpt_oss(x, logits, gate, up, down, zi, zi - 1, zh, k, alpha=1.0)
+    assert np.array_equal(idx1, idx_q) and np.array_equal(wt1, wt_q)
+    assert np.abs(y1 - y_q).max() / np.abs(y_q).max() < 1e-6
+    # (2)
+    gb, ub, db = synth.normal(402, (e, i), 0.3), synth.normal(403, (e, i), 0.3), synth.normal(404, (e, h), 0.3)
+    y2, idx2, wt2 = cr.moe_forward_gpt_oss(x, logits, gate, up, down, gb, ub, db, k, alpha=0.0)
+    want = np.zeros((t, h), np.float64)
+    for tt in range(t):
+        for ee, ww in sorted(zip(idx2[tt], wt2[tt])):
+            g = cr.gemm(o, "q4_K", x[tt:tt + 1], gate[ee], i)[0] + gb[ee]
+            u = cr.gemm(o, "q4_K", x[tt:tt + 1], up[ee], i)[0] + ub[ee]
+            hh = ((g / np.float32(2)) * (u + np.float32(1))).astype(np.float32)
+            want[tt] += np.float64(ww) * (cr.gemm(o, "q4_K", hh[None], down[ee], h)[0].astype(np.float64) + db[ee])
+    assert np.abs(y2 - want).max() / np.abs(want).max() < 1e-5
+    # (3)
+    ya, idx3, wt3 = cr.moe_forward_gpt_oss(x, logits, gate, up, down, gb, ub, db, k)
+    yb, _, _ = cr.moe_forward_gpt_oss(x, logits, gate, up, down, gb, ub, zh, k)
+    shift = np.einsum("tk,tkh->th", wt3.astype(np.float64), db[idx3.astype(np.int64)].astype(np.float64))
+    assert np.abs((ya.astype(np.float64) - yb) - shift).max() < 2e-5
+    # and alpha is the sigmoid's slope: the default differs from alpha = 1 at this size
+    yc, _, _ = cr.moe_forward_gpt_oss(x, logits, gate, up, down, gb, ub, db, k, alpha=1.0)
+    assert np.abs(ya - yc).max() / np.abs(ya).max() > 1e-2
+
+
 # ------------------------------------------------------------------ 3. golden digests
 def _digest_cases():
     o = cr.oracle()
