@@ -161,6 +161,30 @@ def main():
     # what the int8 matrix instruction sustains on this device with nothing else issued
     ceiling_tops, ceiling_ghz = capi.bench_mfma_ceiling(2.0, stream=stream)
 
+    # ---- the same step with operands in host memory (what the Layer API hands over) --------
+    # Not `value`: the PCIe-inclusive rate of the whole call, activations in and outputs back
+    # (8 MB + 25 MB), from pageable memory (through the library's pinned ring) and from memory of
+    # the context's allocator (page-locked, by DMA as it is). Synchronous calls, wall clock.
+    import ctypes
+    a_host = a.cpu().numpy()
+    c_host = np.empty((M, N), np.float32)
+    pa, pc = capi.host_alloc(M * K * 4), capi.host_alloc(M * N * 4)
+    a_pin = np.ctypeslib.as_array(ctypes.cast(pa, ctypes.POINTER(ctypes.c_float)), (M, K))
+    a_pin[:] = a_host
+
+    def host_call_ms(src, dst, reps=7):
+        ts = []
+        for i in range(reps + 2):
+            t0 = time.perf_counter()
+            capi.matmul(weights[i % n_copies], src, M, dst, mem=capi.MEM_HOST)
+            ts.append((time.perf_counter() - t0) * 1e3)
+        return sorted(ts[2:])[reps // 2]
+
+    pageable_ms = host_call_ms(a_host, c_host)
+    pinned_ms = host_call_ms(pa, pc)
+    capi.host_free(pa)
+    capi.host_free(pc)
+
     # ---- decode GEMV over the same matrix, weights rotating through HBM ----
     a1 = a[:1].contiguous()
     c1 = torch.empty((1, N), device="cuda", dtype=torch.float32)
@@ -387,6 +411,12 @@ def main():
                      "mfma_ceiling_tops": round(ceiling_tops, 1), "mfma_ceiling_clock_ghz": round(ceiling_ghz, 3),
                      "frac_of_measured_ceiling": round(gemm_tops / ceiling_tops, 5)},
         "quantizer_ms": round(quant_ms, 5),
+        "pcie_inclusive": {"workload": "the same step through hipq_matmul with HIPQ_MEM_HOST operands: 8.4 MB of "
+                                       "activations in, 25.2 MB of outputs back, synchronous call, median of 7",
+                           "pageable_ms_per_step": round(pageable_ms, 4),
+                           "pageable_tops": round(ops / (pageable_ms * 1e-3) / 1e12, 2),
+                           "page_locked_ms_per_step": round(pinned_ms, 4),
+                           "page_locked_tops": round(ops / (pinned_ms * 1e-3) / 1e12, 2)},
         "timing": {"method": "median of 5 blocks of `steps` hipq_matmul calls; HIP events on the launch stream "
                              "before the quantizer, between the two kernels and behind the GEMM of every step: "
                              "ms_per_step = quantizer_ms + roofline.kernel_ms from the same launches",

@@ -233,6 +233,20 @@ HIPQ_API int hipq_moe_forward_ext(const hipq_moe_desc *desc, const hipq_moe_ext 
                                   float *y, int32_t *topk_idx, float *topk_w, int mem,
                                   void *stream);
 
+/** Page-locked host memory, zero-filled: what a context's MemAllocator hands the framework's
+ *  memory pool (MemAllocator::alloc / free, nntrainer/mem_allocator.cpp:22-30; set by the
+ *  context, cl_context.cpp:83). Tensors that live in it cross to the GPU by DMA as they are;
+ *  any other host memory passed with HIPQ_MEM_HOST goes through a pinned staging ring inside
+ *  the library (8 MiB), at the speed of a host memcpy. */
+HIPQ_API int hipq_host_alloc(void **ptr, size_t bytes);
+HIPQ_API int hipq_host_free(void *ptr);
+
+/** Frees the scratch the library keeps for a stream (it grows on demand with the calls made on
+ *  the stream and is otherwise kept until hipq_shutdown). Call it before destroying a stream
+ *  that calls were made on; waits for the stream. No counterpart in the reference, whose OpenCL
+ *  back-end has one queue (opencl_command_queue_manager.cpp). */
+HIPQ_API int hipq_stream_release(void *stream);
+
 /** Offline weight quantizers fp32 [N x K] -> canonical blocks, on the GPU.
  *  Replace quantize_q4_0 / quantize_q4_K / quantize_q6_K
  *  (x86_compute_backend.cpp:343-370 -> nntr_ggml_impl_quant.cpp:452-467,

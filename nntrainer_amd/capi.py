@@ -21,7 +21,7 @@ SYMBOLS = [
     "hipq_init", "hipq_shutdown", "hipq_last_error", "hipq_version", "hipq_weight_nbytes",
     "hipq_weight_create", "hipq_weight_destroy", "hipq_weight_dims", "hipq_quantize_q8_0",
     "hipq_quantize_q8_K", "hipq_matmul", "hipq_matmul_noalloc", "hipq_matmul_multi", "hipq_moe_forward",
-    "hipq_moe_forward_ext",
+    "hipq_moe_forward_ext", "hipq_host_alloc", "hipq_host_free", "hipq_stream_release",
     "hipq_quantize_weights", "hipq_file_layout", "hipq_weights_from_file",
 ]
 # measurement helpers of csrc/hipq_bench.h: exported for bench.py, not part of the product ABI
@@ -97,6 +97,9 @@ def lib():
         L.hipq_moe_forward_ext.argtypes = [C.POINTER(MoeDesc), C.POINTER(MoeExt), C.POINTER(vp), C.POINTER(vp),
                                            C.POINTER(vp), vp, vp, vp, vp, vp, vp, i32, vp]
         L.hipq_quantize_weights.argtypes = [i32, vp, i64, i64, vp, i32, vp]
+        L.hipq_host_alloc.argtypes = [C.POINTER(vp), C.c_size_t]
+        L.hipq_host_free.argtypes = [vp]
+        L.hipq_stream_release.argtypes = [vp]
         L.hipq_time_matmul.argtypes = [i32, C.POINTER(vp), vp, i64, i64, vp, i64, i32, i32, vp,
                                        C.POINTER(C.c_float)]
         fp = C.POINTER(C.c_float)
@@ -261,6 +264,21 @@ def moe_forward_gpt_oss(tokens, hidden, inter, experts, topk, gate, up, down, x,
     check(lib().hipq_moe_forward_ext(C.byref(d), C.byref(ext), ex.gate, ex.up, ex.down, _addr(x),
                                      _addr(router_logits), _addr(router_weight), _addr(y),
                                      _addr(topk_idx), _addr(topk_w), mem, stream))
+
+
+def host_alloc(nbytes):
+    """Address of `nbytes` of zero-filled page-locked host memory (hipq_host_free releases it)."""
+    p = C.c_void_p()
+    check(lib().hipq_host_alloc(C.byref(p), nbytes))
+    return p.value
+
+
+def host_free(addr):
+    check(lib().hipq_host_free(addr))
+
+
+def stream_release(stream=None):
+    check(lib().hipq_stream_release(stream))
 
 
 def time_matmul(ws, a, m, c, iters, phase=0, stream=None):

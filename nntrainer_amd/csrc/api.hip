@@ -40,6 +40,9 @@ thread_local char tl_error[768] = "";
 struct Workspace {
   void *ptr = nullptr;
   size_t bytes = 0;
+  /* device copies of a host-memory call's operands (the kernels' own scratch is ptr) */
+  void *io = nullptr;
+  size_t io_bytes = 0;
   /* held while a call enqueues its launches: two threads that name the same stream
    * must not interleave their kernels (the second would quantize into the scratch
    * the first one's product has not read yet) */
@@ -110,6 +113,158 @@ int workspace(hipStream_t s, size_t bytes, void **out) {
     w.bytes = want;
   }
   *out = w.ptr;
+  return HIPQ_OK;
+}
+
+int io_buffer(hipStream_t s, size_t bytes, void **out) {
+  std::lock_guard<std::mutex> lk(g.mu);
+  Workspace &w = g.ws[s];
+  if (w.io_bytes < bytes) {
+    if (w.io) {
+      HIPQ_HIP(hipStreamSynchronize(s));
+      HIPQ_HIP(hipFree(w.io));
+      w.io = nullptr;
+      w.io_bytes = 0;
+    }
+    size_t want = (bytes + ((size_t)1 << 20) - 1) & ~(((size_t)1 << 20) - 1);
+    hipError_t e = hipMalloc(&w.io, want);
+    if (e != hipSuccess) {
+      w.io = nullptr;
+      return fail(HIPQ_ERR_OUT_OF_MEMORY, "operand buffer of %zu bytes: %s", want, hipGetErrorString(e));
+    }
+    w.io_bytes = want;
+  }
+  *out = w.io;
+  return HIPQ_OK;
+}
+
+/* Host memory the framework hands over is pageable: a copy from it goes through the runtime's
+ * own small staging and reaches a few GB/s. This ring of pinned slots takes its place: the
+ * caller's thread copies a slice into a slot while the DMA engine moves the slice before it, so
+ * a transfer runs at the speed of a host memcpy. Memory that is pinned already (the allocator of
+ * hipq_host_alloc, or any hipHostMalloc) is handed to the DMA engine as it is. One ring per
+ * process, one transfer at a time; a slot is reused once the event recorded behind its last
+ * copy has passed, whichever stream that copy was on. */
+struct StageRing {
+  static constexpr int SLOTS = 4;
+  static constexpr size_t SLOT_BYTES = (size_t)2 << 20;
+  std::mutex mu;
+  char *base = nullptr;
+  hipEvent_t ev[SLOTS];
+  bool busy[SLOTS] = {false, false, false, false}; /* ev[k] was recorded after the slot's last use */
+  size_t pos = 0;                                  /* slots are taken round robin across transfers */
+  /* the slot is free again: the copy that read or wrote it last has completed */
+  int wait_free(int k) {
+    if (busy[k]) {
+      HIPQ_HIP(hipEventSynchronize(ev[k]));
+      busy[k] = false;
+    }
+    return HIPQ_OK;
+  }
+  int ensure() {
+    if (base) return HIPQ_OK;
+    HIPQ_HIP(hipHostMalloc((void **)&base, SLOTS * SLOT_BYTES, hipHostMallocDefault));
+    for (int i = 0; i < SLOTS; ++i) HIPQ_HIP(hipEventCreateWithFlags(&ev[i], hipEventDisableTiming));
+    return HIPQ_OK;
+  }
+};
+StageRing g_ring;
+
+bool is_pinned(const void *p) {
+  hipPointerAttribute_t at;
+  if (hipPointerGetAttributes(&at, p) != hipSuccess) {
+    (void)hipGetLastError(); /* an ordinary host pointer: not an error of ours */
+    return false;
+  }
+  return at.type == hipMemoryTypeHost;
+}
+
+/* rows x width bytes between host (pitch hpitch) and a dense device buffer, in order on s.
+ * to_device: the copy is queued when this returns (the host bytes have been read). Otherwise
+ * the host bytes are written when this returns. */
+int stage_copy(bool to_device, void *dev, void *host, size_t hpitch, size_t width, size_t rows, hipStream_t s) {
+  if (!rows || !width) return HIPQ_OK;
+  if (is_pinned(host)) {
+    if (to_device) {
+      HIPQ_HIP(hipMemcpy2DAsync(dev, width, host, hpitch, width, rows, hipMemcpyHostToDevice, s));
+    } else {
+      HIPQ_HIP(hipMemcpy2DAsync(host, hpitch, dev, width, width, rows, hipMemcpyDeviceToHost, s));
+      HIPQ_HIP(hipStreamSynchronize(s));
+    }
+    return HIPQ_OK;
+  }
+  std::lock_guard<std::mutex> lk(g_ring.mu);
+  int rc = g_ring.ensure();
+  if (rc) return rc;
+  constexpr int SLOTS = StageRing::SLOTS;
+  /* a slice = as many whole rows as fit a slot, or a piece of one long row */
+  const size_t rows_per = width <= StageRing::SLOT_BYTES ? StageRing::SLOT_BYTES / width : 0;
+  struct Slice {
+    size_t row, off, nrows, bytes; /* nrows rows from `row`, or `bytes` of row `row` from byte `off` */
+  };
+  auto slice_at = [&](size_t i, Slice &sl) -> bool {
+    if (rows_per) {
+      sl.row = i * rows_per;
+      if (sl.row >= rows) return false;
+      sl.off = 0;
+      sl.nrows = rows - sl.row < rows_per ? rows - sl.row : rows_per;
+      sl.bytes = sl.nrows * width;
+      return true;
+    }
+    const size_t per_row = (width + StageRing::SLOT_BYTES - 1) / StageRing::SLOT_BYTES;
+    sl.row = i / per_row;
+    if (sl.row >= rows) return false;
+    sl.off = (i % per_row) * StageRing::SLOT_BYTES;
+    sl.nrows = 1;
+    sl.bytes = width - sl.off < StageRing::SLOT_BYTES ? width - sl.off : StageRing::SLOT_BYTES;
+    return true;
+  };
+  auto host_rows = [&](const Slice &sl, char *slot, bool into_slot) {
+    if (hpitch == width || sl.nrows == 1) {
+      char *h = (char *)host + sl.row * hpitch + sl.off;
+      if (into_slot) memcpy(slot, h, sl.bytes); else memcpy(h, slot, sl.bytes);
+      return;
+    }
+    for (size_t r = 0; r < sl.nrows; ++r) {
+      char *h = (char *)host + (sl.row + r) * hpitch;
+      if (into_slot) memcpy(slot + r * width, h, width); else memcpy(h, slot + r * width, width);
+    }
+  };
+  Slice sl;
+  const size_t p0 = g_ring.pos; /* slice i uses slot (p0 + i) % SLOTS */
+  if (to_device) {
+    size_t i = 0;
+    for (; slice_at(i, sl); ++i) {
+      const int k = (int)((p0 + i) % SLOTS);
+      if ((rc = g_ring.wait_free(k))) return rc; /* also a slot an earlier transfer left in flight */
+      host_rows(sl, g_ring.base + k * StageRing::SLOT_BYTES, true);
+      HIPQ_HIP(hipMemcpyAsync((char *)dev + sl.row * width + sl.off, g_ring.base + k * StageRing::SLOT_BYTES, sl.bytes,
+                              hipMemcpyHostToDevice, s));
+      HIPQ_HIP(hipEventRecord(g_ring.ev[k], s));
+      g_ring.busy[k] = true;
+    }
+    g_ring.pos = p0 + i;
+    return HIPQ_OK;
+  }
+  size_t issued = 0, done = 0;
+  for (;;) {
+    while (issued < done + SLOTS && slice_at(issued, sl)) {
+      const int k = (int)((p0 + issued) % SLOTS);
+      if ((rc = g_ring.wait_free(k))) return rc;
+      HIPQ_HIP(hipMemcpyAsync(g_ring.base + k * StageRing::SLOT_BYTES, (char *)dev + sl.row * width + sl.off, sl.bytes,
+                              hipMemcpyDeviceToHost, s));
+      HIPQ_HIP(hipEventRecord(g_ring.ev[k], s));
+      g_ring.busy[k] = true;
+      ++issued;
+    }
+    if (done == issued) break;
+    const int k = (int)((p0 + done) % SLOTS);
+    if ((rc = g_ring.wait_free(k))) return rc;
+    slice_at(done, sl);
+    host_rows(sl, g_ring.base + k * StageRing::SLOT_BYTES, false);
+    ++done;
+  }
+  g_ring.pos = p0 + issued;
   return HIPQ_OK;
 }
 
@@ -289,14 +444,65 @@ int hipq_shutdown(void) {
     return fail(HIPQ_ERR_INVALID_ARGUMENT, "%lld weights still alive", (long long)g.live_weights);
   (void)hipSetDevice(g.device);
   (void)hipDeviceSynchronize();
-  for (auto &kv : g.ws)
+  for (auto &kv : g.ws) {
     if (kv.second.ptr) (void)hipFree(kv.second.ptr);
+    if (kv.second.io) (void)hipFree(kv.second.io);
+  }
   g.ws.clear();
+  {
+    std::lock_guard<std::mutex> rl(g_ring.mu);
+    if (g_ring.base) {
+      for (int i = 0; i < StageRing::SLOTS; ++i) (void)hipEventDestroy(g_ring.ev[i]);
+      (void)hipHostFree(g_ring.base);
+      g_ring.base = nullptr;
+    }
+  }
   for (auto &kv : g.moe_tables)
     if (kv.second.dev) (void)hipFree(kv.second.dev);
   g.moe_tables.clear();
   g.ready = false;
   g.device = -1;
+  return HIPQ_OK;
+}
+
+int hipq_stream_release(void *stream) {
+  int rc = require_ready();
+  if (rc) return rc;
+  hipStream_t s = (hipStream_t)stream;
+  std::lock_guard<std::mutex> lk(g.mu);
+  auto it = g.ws.find(s);
+  if (it == g.ws.end()) return HIPQ_OK;
+  /* a caller that still enqueues on the stream from another thread holds the lock: refuse */
+  std::unique_lock<std::recursive_mutex> el(it->second.enqueue, std::try_to_lock);
+  if (!el.owns_lock()) return fail(HIPQ_ERR_INVALID_ARGUMENT, "the stream is in use by another call");
+  HIPQ_HIP(hipStreamSynchronize(s));
+  if (it->second.ptr) (void)hipFree(it->second.ptr);
+  if (it->second.io) (void)hipFree(it->second.io);
+  el.unlock();
+  el.release();
+  g.ws.erase(it);
+  return HIPQ_OK;
+}
+
+int hipq_host_alloc(void **ptr, size_t bytes) {
+  int rc = require_ready();
+  if (rc) return rc;
+  if (!ptr) return fail(HIPQ_ERR_INVALID_ARGUMENT, "null argument");
+  *ptr = nullptr;
+  hipError_t e = hipHostMalloc(ptr, bytes ? bytes : 16, hipHostMallocDefault);
+  if (e != hipSuccess) {
+    *ptr = nullptr;
+    return fail(HIPQ_ERR_OUT_OF_MEMORY, "hipHostMalloc(%zu): %s", bytes, hipGetErrorString(e));
+  }
+  memset(*ptr, 0, bytes); /* as the framework's default allocator (calloc, mem_allocator.cpp:22-27) */
+  return HIPQ_OK;
+}
+
+int hipq_host_free(void *ptr) {
+  if (!ptr) return HIPQ_OK;
+  int rc = require_ready();
+  if (rc) return rc;
+  HIPQ_HIP(hipHostFree(ptr));
   return HIPQ_OK;
 }
 
@@ -552,17 +758,15 @@ int hipq_matmul(hipq_weight_t w, const float *A, int64_t M, int64_t lda, float *
   if (mem == HIPQ_MEM_DEVICE) return matmul_device(w, A, M, lda, C, ldc, s, sc);
   if (mem != HIPQ_MEM_HOST) return fail(HIPQ_ERR_INVALID_ARGUMENT, "unknown mem kind %d", mem);
   if (M == 0) return HIPQ_OK;
-  DevBuf dA, dC;
-  if ((rc = dA.alloc((size_t)M * w->K * 4))) return rc;
-  if ((rc = dC.alloc((size_t)M * w->N * 4))) return rc;
-  HIPQ_HIP(hipMemcpy2D(dA.p, (size_t)w->K * 4, A, (size_t)lda * 4, (size_t)w->K * 4, (size_t)M,
-                       hipMemcpyHostToDevice));
-  rc = matmul_device(w, (const float *)dA.p, M, w->K, (float *)dC.p, w->N, s, sc);
-  if (rc) return rc;
-  HIPQ_HIP(hipStreamSynchronize(s));
-  HIPQ_HIP(hipMemcpy2D(C, (size_t)ldc * 4, dC.p, (size_t)w->N * 4, (size_t)w->N * 4, (size_t)M,
-                       hipMemcpyDeviceToHost));
-  return HIPQ_OK;
+  /* host operands: device copies in the stream's operand buffer (grown on demand, no
+   * allocation per call), moved through the pinned ring */
+  const size_t a_bytes = ((size_t)M * w->K * 4 + 255) & ~(size_t)255, c_bytes = (size_t)M * w->N * 4;
+  void *io = nullptr;
+  if ((rc = io_buffer(s, a_bytes + c_bytes, &io))) return rc;
+  float *dA = (float *)io, *dC = (float *)((char *)io + a_bytes);
+  if ((rc = stage_copy(true, dA, (void *)A, (size_t)lda * 4, (size_t)w->K * 4, (size_t)M, s))) return rc;
+  if ((rc = matmul_device(w, dA, M, w->K, dC, w->N, s, sc))) return rc;
+  return stage_copy(false, dC, C, (size_t)ldc * 4, (size_t)w->N * 4, (size_t)M, s);
 }
 
 int hipq_matmul_noalloc(hipq_weight_t w, const float *A, int64_t M, int64_t lda, float *C,
@@ -586,14 +790,35 @@ int hipq_matmul_multi(int count, const hipq_weight_t *w, const float *A, int64_t
     if ((rc = check_matmul_args(w[i], A, M, lda, C[i], ldc[i]))) return rc;
     if (w[i]->K != w[0]->K) return fail(HIPQ_ERR_INVALID_ARGUMENT, "weights disagree on K");
   }
-  if (mem != HIPQ_MEM_DEVICE) {
-    for (int i = 0; i < count; ++i)
-      if ((rc = hipq_matmul(w[i], A, M, lda, C[i], ldc[i], mem, stream))) return rc;
-    return HIPQ_OK;
-  }
+  if (mem != HIPQ_MEM_DEVICE && mem != HIPQ_MEM_HOST)
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "unknown mem kind %d", mem);
   if (M == 0) return HIPQ_OK;
   hipStream_t s = (hipStream_t)stream;
   EnqueueGuard eg(enqueue_lock(s));
+  if (mem == HIPQ_MEM_HOST) {
+    /* the activation crosses once, the products run as for device memory, the outputs return */
+    const int64_t Kh = w[0]->K;
+    size_t total = ((size_t)M * Kh * 4 + 255) & ~(size_t)255;
+    std::vector<size_t> off(count);
+    for (int i = 0; i < count; ++i) {
+      off[i] = total;
+      total += ((size_t)M * w[i]->N * 4 + 255) & ~(size_t)255;
+    }
+    void *io = nullptr;
+    if ((rc = io_buffer(s, total, &io))) return rc;
+    if ((rc = stage_copy(true, io, (void *)A, (size_t)lda * 4, (size_t)Kh * 4, (size_t)M, s))) return rc;
+    std::vector<float *> dC(count);
+    std::vector<int64_t> dld(count);
+    for (int i = 0; i < count; ++i) {
+      dC[i] = (float *)((char *)io + off[i]);
+      dld[i] = w[i]->N;
+    }
+    if ((rc = hipq_matmul_multi(count, w, (const float *)io, M, Kh, dC.data(), dld.data(), HIPQ_MEM_DEVICE, stream)))
+      return rc;
+    for (int i = 0; i < count; ++i)
+      if ((rc = stage_copy(false, dC[i], C[i], (size_t)ldc[i] * 4, (size_t)w[i]->N * 4, (size_t)M, s))) return rc;
+    return HIPQ_OK;
+  }
   if (M == 1 && hipq::gemv_fuses_quantizer_multi(count, w, A))
     return hipq::launch_gemv_fused_multi(count, w, A, C, s);
   /* one quantization per distinct activation format among the weights */
@@ -857,7 +1082,7 @@ int hipq_moe_forward_ext(const hipq_moe_desc *desc, const hipq_moe_ext *ext, con
   if ((rc = dy.alloc(T * H * 4))) return rc;
   if ((rc = di.alloc(T * k * 4))) return rc;
   if ((rc = dw.alloc(T * k * 4))) return rc;
-  HIPQ_HIP(hipMemcpy(dx.p, x, T * H * 4, hipMemcpyHostToDevice));
+  if ((rc = stage_copy(true, dx.p, (void *)x, H * 4, H * 4, T, s))) return rc;
   HIPQ_HIP(hipMemcpy(dr.p, router_logits ? router_logits : router_weight,
                      (router_logits ? T * E : H * E) * 4, hipMemcpyHostToDevice));
   a.x = (const float *)dx.p;
@@ -867,8 +1092,7 @@ int hipq_moe_forward_ext(const hipq_moe_desc *desc, const hipq_moe_ext *ext, con
   a.topk_idx = (int32_t *)di.p;
   a.topk_w = (float *)dw.p;
   if ((rc = hipq::launch_moe(&a, ws, ws_bytes, dev_views, s))) return rc;
-  HIPQ_HIP(hipStreamSynchronize(s));
-  HIPQ_HIP(hipMemcpy(y, dy.p, T * H * 4, hipMemcpyDeviceToHost));
+  if ((rc = stage_copy(false, dy.p, y, H * 4, H * 4, T, s))) return rc;
   if (topk_idx) HIPQ_HIP(hipMemcpy(topk_idx, di.p, T * k * 4, hipMemcpyDeviceToHost));
   if (topk_w) HIPQ_HIP(hipMemcpy(topk_w, dw.p, T * k * 4, hipMemcpyDeviceToHost));
   return HIPQ_OK;

@@ -11,6 +11,7 @@
 #include <sstream>
 
 #include "fc_layer_hip.h"
+#include "hip_mem_allocator.h"
 #include "hipq_host.h"
 #include "moe_layer_hip.h"
 #include "qkv_layer_hip.h"
@@ -38,6 +39,9 @@ void HipContext::initialize() noexcept {
         std::fprintf(stderr, "[HipContext] no usable HIP device (%s); layers will fail at forward time\n",
                      hipq_last_error());
       add_default_object();
+      /* the pool that holds a model's tensors allocates through the context's allocator
+       * (cl_context.cpp:83 sets the default one): page-locked memory here */
+      getContextData()->setMemAllocator(std::make_shared<HipMemAllocator>());
     });
   } catch (const std::exception &e) {
     std::fprintf(stderr, "[HipContext] initialize failed: %s\n", e.what());

@@ -118,6 +118,23 @@ static void write_from(const std::string &path, const void *src, size_t bytes) {
 static int run_api(Context *ctx) {
   EXPECT(ctx->getName() == "gpu");
   EXPECT(ctx->getContextData() != nullptr);
+  /* the context publishes an allocator (cl_context.cpp:83); it works without a device too */
+  {
+    auto ma = ctx->getContextData()->getMemAllocator();
+    EXPECT(ma != nullptr);
+    if (ma) {
+      EXPECT(ma->getName() == "gpu");
+      void *p = nullptr;
+      ma->alloc(&p, 4096, 64);
+      EXPECT(p != nullptr);
+      bool zero = p != nullptr;
+      for (int i = 0; zero && i < 4096; ++i)
+        zero = static_cast<unsigned char *>(p)[i] == 0;
+      EXPECT(zero);
+      ma->free(p);
+      ma->free(nullptr);
+    }
+  }
 
   /* factory keys: string (case-insensitive) and integer */
   auto fc = ctx->createLayerObject("fully_connected", {"unit=512", "disable_bias=true"});

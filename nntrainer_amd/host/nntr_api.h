@@ -15,6 +15,7 @@
 #include <layer.h>
 #include <layer_context.h>
 #include <layer_devel.h>
+#include <mem_allocator.h>
 #include <nntrainer_error.h>
 #include <tensor.h>
 #include <tensor_dim.h>

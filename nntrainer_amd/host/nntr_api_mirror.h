@@ -23,6 +23,7 @@
 #include <array>
 #include <bitset>
 #include <cstdint>
+#include <cstdlib>
 #include <cstring>
 #include <fstream>
 #include <functional>
@@ -369,9 +370,13 @@ std::unique_ptr<Layer> createLayer(const std::vector<std::string> &props = {}) {
   return ptr;
 }
 
+/** nntrainer/mem_allocator.h:24-33, mem_allocator.cpp:22-30 */
 class MemAllocator {
 public:
+  MemAllocator() = default;
   virtual ~MemAllocator() = default;
+  virtual void alloc(void **ptr, size_t size, size_t /*alignment*/) { *ptr = std::calloc(size, 1); }
+  virtual void free(void *ptr) { std::free(ptr); }
   virtual std::string getName() { return "cpu"; }
 };
 

@@ -1,0 +1,99 @@
+"""Host-memory operands of the C ABI (HIPQ_MEM_HOST): pageable memory goes through the library's
+pinned staging ring, page-locked memory (hipq_host_alloc, what the context's MemAllocator hands
+the framework, cl_context.cpp:83) by DMA as it is. Both must give the bits of the device-memory
+call. Also: the multi-weight call on host memory, and releasing a stream's scratch."""
+import ctypes
+
+import numpy as np
+import pytest
+
+from nntrainer_amd import capi, synth
+
+pytestmark = pytest.mark.gpu
+
+
+def _device_result(w, a):
+    import gpu_util as gu
+    return gu.gpu_matmul(w, a)
+
+
+@pytest.mark.parametrize("kind,m,k,n,lda_pad,ldc_pad", [
+    ("q4_0", 700, 1024, 3000, 0, 0),     # A 2.8 MB, C 8.4 MB: several slices of the ring each way
+    ("q4_0", 700, 1024, 3000, 32, 8),    # strided rows on both sides
+    ("q4_K", 37, 2048, 1024, 0, 0),
+    ("q6_K", 1, 1024, 5000, 0, 0),       # decode row
+    ("q4_0", 1, 32, 600000, 0, 0),       # one output row longer than a ring slot (2.4 MB)
+])
+def test_pageable_operands_give_the_device_bits(hipq, cr, kind, m, k, n, lda_pad, ldc_pad):
+    blocks = cr.quantize_weights(cr.oracle(), kind, synth.normal(9000 + n % 97, (n, k), 0.02))
+    w = capi.Weight(kind, n, k, blocks)
+    a = synth.normal(9001 + m, (m, k))
+    want = _device_result(w, a)
+    lda, ldc = k + lda_pad, n + ldc_pad
+    a_host = np.full((m, lda), np.float32(7e9))
+    a_host[:, :k] = a
+    c_host = np.full((m, ldc), np.float32(-3.5))
+    for _ in range(2):  # the second call finds ring slots and operand buffers in use before
+        c_host[:, :n] = np.nan
+        capi.matmul(w, a_host, m, c_host, lda=lda, ldc=ldc, mem=capi.MEM_HOST)
+        assert np.array_equal(c_host[:, :n].view(np.uint32), want.view(np.uint32))
+        assert np.all(c_host[:, n:] == np.float32(-3.5)), "the padding of the output rows was written"
+    w.destroy()
+
+
+def test_page_locked_operands(hipq, cr):
+    kind, m, k, n = "q4_K", 64, 1024, 768
+    blocks = cr.quantize_weights(cr.oracle(), kind, synth.normal(9100, (n, k), 0.02))
+    w = capi.Weight(kind, n, k, blocks)
+    a = synth.normal(9101, (m, k))
+    want = _device_result(w, a)
+    pa, pc = capi.host_alloc(m * k * 4), capi.host_alloc(m * n * 4)
+    try:
+        a_pin = np.ctypeslib.as_array(ctypes.cast(pa, ctypes.POINTER(ctypes.c_float)), (m, k))
+        c_pin = np.ctypeslib.as_array(ctypes.cast(pc, ctypes.POINTER(ctypes.c_float)), (m, n))
+        assert not a_pin.any() and not c_pin.any(), "the allocator hands out zero-filled memory"
+        a_pin[:] = a
+        capi.matmul(w, pa, m, pc, mem=capi.MEM_HOST)
+        assert np.array_equal(c_pin.view(np.uint32), want.view(np.uint32))
+    finally:
+        capi.host_free(pa)
+        capi.host_free(pc)
+        capi.host_free(None)
+    w.destroy()
+
+
+@pytest.mark.parametrize("kind,m", [("q4_0", 1), ("q4_0", 19), ("q4_K", 1), ("q6_K", 3)])
+def test_multi_weight_call_on_host_memory(hipq, cr, kind, m):
+    """hipq_matmul_multi with host operands: the activation crosses once and the products run as
+    for device memory; same bits as one hipq_matmul per weight."""
+    k, ns = 1024, (512, 256, 384)
+    ws = [capi.Weight(kind, n, k, cr.quantize_weights(cr.oracle(), kind, synth.normal(9200 + n, (n, k), 0.02)))
+          for n in ns]
+    a = synth.normal(9201 + m, (m, k))
+    cs = [np.full((m, n), np.nan, np.float32) for n in ns]
+    capi.matmul_multi(ws, a, m, cs, mem=capi.MEM_HOST)
+    for w, c in zip(ws, cs):
+        assert np.array_equal(c.view(np.uint32), _device_result(w, a).view(np.uint32))
+        w.destroy()
+
+
+def test_stream_release(hipq, cr):
+    """A stream's scratch can be given back and comes again with the next call."""
+    import gpu_util as gu
+    import torch
+    kind, m, k, n = "q4_K", 16, 1024, 512
+    w = capi.Weight(kind, n, k, cr.quantize_weights(cr.oracle(), kind, synth.normal(9300, (n, k), 0.02)))
+    a = synth.normal(9301, (m, k))
+    want = _device_result(w, a)
+    st = torch.cuda.Stream()
+    da = gu.dev(a)
+    torch.cuda.synchronize()
+    for _ in range(2):
+        dc = torch.full((m, n), float("nan"), device="cuda")
+        torch.cuda.synchronize()
+        capi.matmul(w, da, m, dc, stream=st.cuda_stream)
+        st.synchronize()
+        assert np.array_equal(dc.cpu().numpy().view(np.uint32), want.view(np.uint32))
+        capi.stream_release(st.cuda_stream)
+    capi.stream_release(st.cuda_stream)  # nothing kept: a no-op
+    w.destroy()
