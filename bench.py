@@ -257,8 +257,10 @@ def main():
 
     def decode_layer_graph(grouped):
         """One decode step's FCs of 8 layers (8 weight copies) captured in a graph and
-        replayed: milliseconds per layer without the host's launch cost. grouped: Q, K, V
-        and gate, up each as one hipq_matmul_multi call (4 launches per layer, not 7)."""
+        replayed: milliseconds per layer without the host's launch cost. grouped = 1: Q, K, V
+        and gate, up each as one hipq_matmul_multi call (4 launches per layer, not 7).
+        grouped = 2: Q, K, V as one call and up, gate and the SwiGLU between them and the down
+        projection as one hipq_mlp_swiglu call (the qkv_layer and mlp_swiglu layers of the context)."""
         shapes = [(2048, 1024), (1024, 1024), (1024, 1024), (1024, 2048), (3072, 1024), (3072, 1024), (1024, 3072)]
         layers = []
         for _ in range(8):
@@ -275,7 +277,12 @@ def main():
 
         def step(st):
             for ws_ in layers:
-                if grouped:
+                if grouped == 2:
+                    capi.matmul_multi(ws_[0:3], xs_[1024], 1, cs_[0:3], stream=st)
+                    capi.matmul(ws_[3], xs_[2048], 1, cs_[3], stream=st)
+                    capi.mlp_swiglu(ws_[4], ws_[5], xs_[1024], 1, cs_[4], stream=st)
+                    capi.matmul(ws_[6], xs_[3072], 1, cs_[6], stream=st)
+                elif grouped:
                     capi.matmul_multi(ws_[0:3], xs_[1024], 1, cs_[0:3], stream=st)
                     capi.matmul(ws_[3], xs_[2048], 1, cs_[3], stream=st)
                     capi.matmul_multi(ws_[4:6], xs_[1024], 1, cs_[4:6], stream=st)
@@ -310,7 +317,8 @@ def main():
                 w_.destroy()
         return ms
 
-    c5_graph_ms, c5_graph_grouped_ms = decode_layer_graph(False), decode_layer_graph(True)
+    c5_graph_ms, c5_graph_grouped_ms = decode_layer_graph(0), decode_layer_graph(1)
+    c5_graph_fused_ms = decode_layer_graph(2)
 
     # ---- the MoE block of configs[3]: 64 tokens, 128 experts, top-8, Q4_K ----------
     mt, mh, me, mi, mk = 64, 2048, 128, 768, 8
@@ -454,7 +462,8 @@ def main():
                         "hipq_matmul, quantizers included, 8 weight copies rotated per FC",
             "prefill_512_rows_ms": round(c5_prefill_ms, 5), "decode_1_row_ms": round(c5_decode_ms, 5),
             "decode_1_row_in_a_graph_ms": round(c5_graph_ms, 5),
-            "decode_1_row_in_a_graph_qkv_and_gate_up_as_one_launch_each_ms": round(c5_graph_grouped_ms, 5)},
+            "decode_1_row_in_a_graph_qkv_and_gate_up_as_one_launch_each_ms": round(c5_graph_grouped_ms, 5),
+            "decode_1_row_in_a_graph_qkv_one_launch_up_gate_swiglu_one_launch_ms": round(c5_graph_fused_ms, 5)},
         "moe_block": {
             "workload": "MoE FFN block (BASELINE configs[3]): 64 tokens, hidden 2048, 128 experts x "
                         "(gate/up 2048->768, down 768->2048) Q4_K, top-8; router, sort, experts, combine; "

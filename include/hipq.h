@@ -171,6 +171,17 @@ HIPQ_API int hipq_matmul_multi(int count, const hipq_weight_t *w, const float *A
                                int64_t M, int64_t lda, float *const *C,
                                const int64_t *ldc, int mem, void *stream);
 
+/** The first half of a gated MLP: out[M x N] = swiglu(A . W_act^T, A . W_mul^T) with the
+ *  framework's swiglu, X = (Y / (1 + exp(-Y))) * Z in fp32 (nntrainer::swiglu,
+ *  fallback_internal.cpp:417-423). In the LLM application these are three layers, the FCs
+ *  "ffn_up" (Y) and "ffn_gate" (Z) and the SwiGLULayer on their outputs
+ *  (Applications/CausalLM/layers/swiglu.cpp:40-62, causal_lm.cpp:672-695); here one call that
+ *  quantizes A once, and for one row (K <= 4096, 2 N < 32768, device memory) one kernel launch
+ *  in which the two products never leave the registers. The products are those of hipq_matmul
+ *  bit for bit; the exponential is the device's expf. */
+HIPQ_API int hipq_mlp_swiglu(hipq_weight_t w_act, hipq_weight_t w_mul, const float *A, int64_t M,
+                             int64_t lda, float *out, int64_t ldo, int mem, void *stream);
+
 /** Mixture-of-experts feed-forward block (MoELayer::incremental_forwarding,
  *  qwen_moe_layer.cpp:394-503): softmax over E router logits, top-k, weights
  *  renormalised to sum 1, per (token, expert) SwiGLU MLP

@@ -21,7 +21,7 @@ SYMBOLS = [
     "hipq_init", "hipq_shutdown", "hipq_last_error", "hipq_version", "hipq_weight_nbytes",
     "hipq_weight_create", "hipq_weight_destroy", "hipq_weight_dims", "hipq_quantize_q8_0",
     "hipq_quantize_q8_K", "hipq_matmul", "hipq_matmul_noalloc", "hipq_matmul_multi", "hipq_moe_forward",
-    "hipq_moe_forward_ext", "hipq_host_alloc", "hipq_host_free", "hipq_stream_release",
+    "hipq_moe_forward_ext", "hipq_mlp_swiglu", "hipq_host_alloc", "hipq_host_free", "hipq_stream_release",
     "hipq_quantize_weights", "hipq_file_layout", "hipq_weights_from_file",
 ]
 # measurement helpers of csrc/hipq_bench.h: exported for bench.py, not part of the product ABI
@@ -97,6 +97,7 @@ def lib():
         L.hipq_moe_forward_ext.argtypes = [C.POINTER(MoeDesc), C.POINTER(MoeExt), C.POINTER(vp), C.POINTER(vp),
                                            C.POINTER(vp), vp, vp, vp, vp, vp, vp, i32, vp]
         L.hipq_quantize_weights.argtypes = [i32, vp, i64, i64, vp, i32, vp]
+        L.hipq_mlp_swiglu.argtypes = [vp, vp, vp, i64, i64, vp, i64, i32, vp]
         L.hipq_host_alloc.argtypes = [C.POINTER(vp), C.c_size_t]
         L.hipq_host_free.argtypes = [vp]
         L.hipq_stream_release.argtypes = [vp]
@@ -227,6 +228,12 @@ def matmul_multi(ws, a, m, cs, mem=MEM_DEVICE, stream=None):
     cp = (C.c_void_p * n)(*[_addr(c) for c in cs])
     ld = (C.c_int64 * n)(*[w.n for w in ws])
     check(lib().hipq_matmul_multi(n, hs, _addr(a), m, ws[0].k, cp, ld, mem, stream))
+
+
+def mlp_swiglu(w_act, w_mul, a, m, out, lda=None, ldo=None, mem=MEM_DEVICE, stream=None):
+    """out = swiglu(a . w_act^T, a . w_mul^T): the gated half of a dense MLP in one call."""
+    check(lib().hipq_mlp_swiglu(w_act.handle, w_mul.handle, _addr(a), m, lda or w_act.k, _addr(out),
+                                ldo or w_act.n, mem, stream))
 
 
 def quantize_weights(dtype, w, n, k, out, mem=MEM_DEVICE, stream=None):

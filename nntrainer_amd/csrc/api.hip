@@ -781,6 +781,49 @@ int hipq_matmul_noalloc(hipq_weight_t w, const float *A, int64_t M, int64_t lda,
   return matmul_device(w, A, M, lda, C, ldc, s, Scratch{true, s});
 }
 
+int hipq_mlp_swiglu(hipq_weight_t w_act, hipq_weight_t w_mul, const float *A, int64_t M, int64_t lda,
+                    float *out, int64_t ldo, int mem, void *stream) {
+  int rc = require_ready();
+  if (rc) return rc;
+  if ((rc = check_matmul_args(w_act, A, M, lda, out, ldo))) return rc;
+  if ((rc = check_matmul_args(w_mul, A, M, lda, out, ldo))) return rc;
+  if (w_act->K != w_mul->K || w_act->N != w_mul->N)
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "the two projections differ in shape");
+  if (mem != HIPQ_MEM_DEVICE && mem != HIPQ_MEM_HOST)
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "unknown mem kind %d", mem);
+  if (M == 0) return HIPQ_OK;
+  hipStream_t s = (hipStream_t)stream;
+  EnqueueGuard eg(enqueue_lock(s));
+  const int64_t N = w_act->N, K = w_act->K;
+  const size_t a_bytes = ((size_t)M * K * 4 + 255) & ~(size_t)255, o_bytes = ((size_t)M * N * 4 + 255) & ~(size_t)255;
+  if (mem == HIPQ_MEM_DEVICE && M == 1 && hipq::gemv_fuses_swiglu(w_act, w_mul, A))
+    return hipq::launch_gemv_fused_swiglu(w_act, w_mul, A, out, s);
+  /* otherwise: both products from one quantization into the stream's operand buffer, then the
+   * activation; host operands cross through the same buffer */
+  void *io = nullptr;
+  if ((rc = io_buffer(s, a_bytes + 3 * o_bytes, &io))) return rc;
+  float *dA = (float *)io, *dY = (float *)((char *)io + a_bytes), *dZ = (float *)((char *)dY + o_bytes),
+        *dO = (float *)((char *)dZ + o_bytes);
+  const float *a_dev = A;
+  int64_t a_ld = lda;
+  if (mem == HIPQ_MEM_HOST) {
+    if ((rc = stage_copy(true, dA, (void *)A, (size_t)lda * 4, (size_t)K * 4, (size_t)M, s))) return rc;
+    a_dev = dA;
+    a_ld = K;
+    if (M == 1 && hipq::gemv_fuses_swiglu(w_act, w_mul, dA)) {
+      if ((rc = hipq::launch_gemv_fused_swiglu(w_act, w_mul, dA, dO, s))) return rc;
+      return stage_copy(false, dO, out, (size_t)ldo * 4, (size_t)N * 4, 1, s);
+    }
+  }
+  const hipq_weight_t ws[2] = {w_act, w_mul};
+  float *const cs[2] = {dY, dZ};
+  const int64_t lds[2] = {N, N};
+  if ((rc = hipq_matmul_multi(2, ws, a_dev, M, a_ld, cs, lds, HIPQ_MEM_DEVICE, stream))) return rc;
+  if (mem == HIPQ_MEM_DEVICE) return hipq::launch_swiglu_rows(dY, dZ, M, N, out, ldo, s);
+  if ((rc = hipq::launch_swiglu_rows(dY, dZ, M, N, dO, N, s))) return rc;
+  return stage_copy(false, dO, out, (size_t)ldo * 4, (size_t)N * 4, (size_t)M, s);
+}
+
 int hipq_matmul_multi(int count, const hipq_weight_t *w, const float *A, int64_t M, int64_t lda,
                       float *const *C, const int64_t *ldc, int mem, void *stream) {
   int rc = require_ready();

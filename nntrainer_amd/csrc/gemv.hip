@@ -80,10 +80,11 @@ template <int DT> __host__ __device__ constexpr int fused_act_bytes(int K) {
   return ((DT == HIPQ_Q4_0 ? K + K / 8 : 2 * K + K / 8 + K / 64) + 15) & ~15;
 }
 
-template <int DT, int T, int G>
-__device__ __forceinline__ void gemv_fused_body(const WView &w, const float *__restrict__ x,
-                                                float *__restrict__ C, int block) {
+template <int DT, int T, int G, int NW, typename Store>
+__device__ __forceinline__ void gemv_fused_rows(const WView (&wv)[NW], const float *__restrict__ x, int block,
+                                                Store store) {
   typedef GemvCore<DT, T, 1, G, false> E;
+  const WView &w = wv[0];
   extern __shared__ __attribute__((aligned(16))) uint32_t gemv_lds[];
   const int K = w.K;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -105,8 +106,9 @@ __device__ __forceinline__ void gemv_fused_body(const WView &w, const float *__r
 #pragma unroll
     for (int p = 0; p < 4; ++p) xs[p] = *(const float4 *)(x + min(wave + 4 * p, nsb - 1) * 256 + lane * 4);
   }
-  typename E::Wts W;
-  E::load_w(W, w, row0, 0, K);
+  typename E::Wts W[NW];
+#pragma unroll
+  for (int i = 0; i < NW; ++i) E::load_w(W[i], wv[i], row0, 0, K);
 
   QView qa;
   qa.K = K;
@@ -155,13 +157,43 @@ __device__ __forceinline__ void gemv_fused_body(const WView &w, const float *__r
 
   typename E::Act A;
   E::load_act(A, qa, arow, 0, K);
-  typename E::Chain c = E::begin(arow, 0);
-  E::compute(W, A, K, lds);
-  hipq_wave_lds_sync();
-  E::chain(c, K, lds);
-  hipq_wave_lds_sync();
-  const GemvOut o = E::finish(c);
-  if (o.valid && row0 + o.g < w.N) C[row0 + o.g] = o.v;
+  GemvOut o[NW];
+#pragma unroll
+  for (int i = 0; i < NW; ++i) {
+    typename E::Chain c = E::begin(arow, 0);
+    E::compute(W[i], A, K, lds);
+    hipq_wave_lds_sync();
+    E::chain(c, K, lds);
+    hipq_wave_lds_sync();
+    o[i] = E::finish(c);
+  }
+  /* the results of the NW weights' row row0 + o[0].g sit in the same lane */
+  if (o[0].valid && row0 + o[0].g < w.N) store(row0 + o[0].g, o);
+}
+
+template <int DT, int T, int G>
+__device__ __forceinline__ void gemv_fused_body(const WView &w, const float *__restrict__ x,
+                                                float *__restrict__ C, int block) {
+  const WView wv[1] = {w};
+  gemv_fused_rows<DT, T, G, 1>(wv, x, block, [&](int row, const GemvOut(&o)[1]) { C[row] = o[0].v; });
+}
+
+/* out[n] = silu(x . Wact[n]) * (x . Wmul[n]): the two projections of a gated MLP and the
+ * SwiGLU between them and the down projection as one launch. A wavefront forms the same G
+ * rows of both matrices (their loads in flight together) and the lane that ends up with
+ * row n of the one also holds row n of the other. The activation is the framework's swiglu
+ * (X = (Y / (1 + exp(-Y))) * Z in fp32, fallback_internal.cpp:417-423), applied by
+ * SwiGLULayer::incremental_forwarding to the outputs of ffn_up (Y) and ffn_gate (Z)
+ * (Applications/CausalLM/layers/swiglu.cpp:40-62, causal_lm.cpp:690-695). */
+template <int DT, int T, int G>
+__global__ __launch_bounds__(256) void gemv_fused_swiglu_kernel(WView wact, WView wmul,
+                                                                const float *__restrict__ x,
+                                                                float *__restrict__ out) {
+  const WView wv[2] = {wact, wmul};
+  gemv_fused_rows<DT, T, G, 2>(wv, x, (int)blockIdx.x, [&](int row, const GemvOut(&o)[2]) {
+    const float y = o[0].v, z = o[1].v;
+    out[row] = (y / (1.f + expf(-y))) * z;
+  });
 }
 
 template <int DT, int T, int G>
@@ -242,6 +274,29 @@ int pick_group(int64_t N, int gmax) {
    * lm_head; smaller matrices want more, shorter wavefronts */
   int g = N >= 8192 ? 4 : (N >= 2048 ? 2 : 1);
   return g < gmax ? g : gmax;
+}
+
+template <int DT, int T, int G>
+int launch_fused_swiglu_one(const hipq_weight *wa, const hipq_weight *wm, const float *x, float *out,
+                            hipStream_t s) {
+  const unsigned grid = (unsigned)((wa->N + 4 * G - 1) / (4 * G));
+  const size_t lds = fused_act_bytes<DT>((int)wa->K) + 4 * GemvLds<DT, 1, G, false>::DWORDS * sizeof(uint32_t);
+  hipLaunchKernelGGL((gemv_fused_swiglu_kernel<DT, T, G>), dim3(grid), dim3(256), lds, s, wview(wa), wview(wm), x,
+                     out);
+  HIPQ_HIP(hipGetLastError());
+  return HIPQ_OK;
+}
+
+/* the shapes of launch_fused for twice the rows (two matrices a wavefront) */
+template <int DT>
+int launch_fused_swiglu(const hipq_weight *wa, const hipq_weight *wm, const float *x, float *out, hipStream_t s) {
+  const int64_t units = wa->K / GemvRec<DT, false>::UNIT;
+  /* a wavefront forms G rows of each matrix: half the group of a single matrix with as many rows */
+  const int g = pick_group(2 * wa->N, 8) / 2;
+  if (units < 64) return launch_fused_swiglu_one<DT, 16, 4>(wa, wm, x, out, s);
+  if (g >= 4) return launch_fused_swiglu_one<DT, 64, 4>(wa, wm, x, out, s);
+  if (g == 2) return launch_fused_swiglu_one<DT, 64, 2>(wa, wm, x, out, s);
+  return launch_fused_swiglu_one<DT, 64, 1>(wa, wm, x, out, s);
 }
 
 /* One activation row: the decode shape, tuned for parallelism. */
@@ -370,6 +425,43 @@ int launch_gemv_fused_multi(int count, const hipq_weight *const *w, const float 
     return launch_fused_multi<HIPQ_Q6_K>(count, w, x, C, s);
   }
   return fail(HIPQ_ERR_INVALID_ARGUMENT, "unknown weight dtype %d", w[0]->dtype);
+}
+
+bool gemv_fuses_swiglu(const hipq_weight *wa, const hipq_weight *wm, const float *x) {
+  return wa->dtype == wm->dtype && wa->K == wm->K && wa->N == wm->N && gemv_fuses_quantizer(wa, x) &&
+         2 * wa->N < 32768;
+}
+
+int launch_gemv_fused_swiglu(const hipq_weight *wa, const hipq_weight *wm, const float *x, float *out,
+                             hipStream_t s) {
+  if (!gemv_fuses_swiglu(wa, wm, x))
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "these matrices do not take the fused gated-MLP GEMV");
+  switch (wa->dtype) {
+  case HIPQ_Q4_0:
+    return launch_fused_swiglu<HIPQ_Q4_0>(wa, wm, x, out, s);
+  case HIPQ_Q4_K:
+    return launch_fused_swiglu<HIPQ_Q4_K>(wa, wm, x, out, s);
+  case HIPQ_Q6_K:
+    return launch_fused_swiglu<HIPQ_Q6_K>(wa, wm, x, out, s);
+  }
+  return fail(HIPQ_ERR_INVALID_ARGUMENT, "unknown weight dtype %d", wa->dtype);
+}
+
+/* out[m][n] = (y / (1 + exp(-y))) * z, elementwise (the same activation for M > 1 rows) */
+__global__ __launch_bounds__(256) void swiglu_rows_kernel(const float *__restrict__ y, const float *__restrict__ z,
+                                                          int64_t n_total, int64_t N, int64_t ldo,
+                                                          float *__restrict__ out) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n_total) return;
+  const float yv = y[i], zv = z[i];
+  out[(i / N) * ldo + i % N] = (yv / (1.f + expf(-yv))) * zv;
+}
+
+int launch_swiglu_rows(const float *y, const float *z, int64_t M, int64_t N, float *out, int64_t ldo, hipStream_t s) {
+  const int64_t n = M * N;
+  hipLaunchKernelGGL(swiglu_rows_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, y, z, n, N, ldo, out);
+  HIPQ_HIP(hipGetLastError());
+  return HIPQ_OK;
 }
 
 int launch_gemv_fused(const hipq_weight *w, const float *x, float *C, hipStream_t s) {

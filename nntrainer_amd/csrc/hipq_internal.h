@@ -179,6 +179,11 @@ int launch_gemv_fused(const hipq_weight *w, const float *x, float *C, hipStream_
 bool gemv_fuses_quantizer_multi(int count, const hipq_weight *const *w, const float *x);
 int launch_gemv_fused_multi(int count, const hipq_weight *const *w, const float *x, float *const *C,
                             hipStream_t s);
+/* out = swiglu(x . Wact, x . Wmul), one row, one launch; and the activation alone for M rows */
+bool gemv_fuses_swiglu(const hipq_weight *wa, const hipq_weight *wm, const float *x);
+int launch_gemv_fused_swiglu(const hipq_weight *wa, const hipq_weight *wm, const float *x, float *out,
+                             hipStream_t s);
+int launch_swiglu_rows(const float *y, const float *z, int64_t M, int64_t N, float *out, int64_t ldo, hipStream_t s);
 int launch_gemv(const hipq_weight *w, const QAct *qa, int M, int pair_rows,
                 float *C, int64_t ldc, hipStream_t s);
 

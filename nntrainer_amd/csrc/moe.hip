@@ -1049,16 +1049,21 @@ int launch_grouped_mma(const hipq::MoeArgs *a, const MoeBufs &b, const WView *vi
                        lds_g, s, views, d.experts, qview(xq), b.offsets, b.items, b.slot_pair, d.topk,
                        d.intermediate, b.h, a->epi);
   HIPQ_HIP(hipGetLastError());
-  if (!few) {
+  /* the down kernel quantizes its item's rows of h itself (QH): one launch less. With many items
+   * every column workgroup of an item repeats the rows, which costs less than the launch did
+   * (92.6 -> 90.3 us at 64 tokens). The launch-a-quantizer form stays for rows too long to be
+   * quantized inside a workgroup's start-up. */
+  const bool qh = true;
+  if (!qh) {
     int rc = hipq::launch_quantize_q8_K_rowmma(b.h, P, d.intermediate, d.intermediate, &hq, s);
     if (rc) return rc;
   }
-  const void *kd = few ? (const void *)down_mma_kernel<TC, true> : (const void *)down_mma_kernel<TC, false>;
+  const void *kd = qh ? (const void *)down_mma_kernel<TC, true> : (const void *)down_mma_kernel<TC, false>;
   if (lds_d > 64 * 1024)
     HIPQ_HIP(hipFuncSetAttribute(kd, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_d));
   const int ct = few ? 1 : 2;
   const dim3 gd((d.hidden + 128 * ct - 1) / (128 * ct), max_items);
-  if (few)
+  if (qh)
     hipLaunchKernelGGL((down_mma_kernel<TC, true>), gd, dim3(256), lds_d, s, views, d.experts, qview(hq), b.h,
                        b.offsets, b.items, b.slot_pair, b.wgt, d.hidden, b.contrib, ct, a->epi);
   else

@@ -13,6 +13,7 @@
 #include "fc_layer_hip.h"
 #include "hip_mem_allocator.h"
 #include "hipq_host.h"
+#include "mlp_swiglu_layer_hip.h"
 #include "moe_layer_hip.h"
 #include "qkv_layer_hip.h"
 #include "tie_word_embedding_hip.h"
@@ -64,6 +65,9 @@ void HipContext::add_default_object() {
   registerFactory(nntrainer::createLayer<CachedSlimMoELayerHip>, CachedSlimMoELayerHip::type, -1);
   registerFactory(nntrainer::createLayer<GptOssMoELayerHip>, GptOssMoELayerHip::type, -1);
   registerFactory(nntrainer::createLayer<CachedSlimGptOssMoELayerHip>, CachedSlimGptOssMoELayerHip::type, -1);
+  /* ffn_up + ffn_gate + swiglu of the application's MLP as one layer (no counterpart in the
+   * framework: a graph opts in by creating it) */
+  registerFactory(nntrainer::createLayer<MlpSwiGLULayerHip>, MlpSwiGLULayerHip::type, -1);
 }
 
 int HipContext::registerFactory(const FactoryType<Layer> factory, const std::string &key,

@@ -149,6 +149,13 @@ void matmul_multi(WeightCache &cache, const std::vector<const void *> &weight_by
         "hipq_matmul_multi");
 }
 
+void mlp_swiglu(WeightCache &cache, const void *act_bytes, const void *mul_bytes, const WeightSpec &spec,
+                const float *A, int64_t M, int64_t lda, float *out, int64_t ldo) {
+  require_runtime();
+  hipq_weight_t wa = cache.get(act_bytes, spec), wm = cache.get(mul_bytes, spec);
+  check(hipq_mlp_swiglu(wa, wm, A, M, lda, out, ldo, HIPQ_MEM_HOST, nullptr), "hipq_mlp_swiglu");
+}
+
 hipq_weight_t upload(const void *host_bytes, const WeightSpec &spec) {
   require_runtime();
   if (!host_bytes)

@@ -112,6 +112,10 @@ void matmul_multi(WeightCache &cache, const std::vector<const void *> &weight_by
                   const std::vector<WeightSpec> &specs, const float *A, int64_t M,
                   int64_t lda, const std::vector<float *> &C);
 
+/** out[M x N] = swiglu(A . Wact^T, A . Wmul^T), both weights of one spec (hipq_mlp_swiglu) */
+void mlp_swiglu(WeightCache &cache, const void *act_bytes, const void *mul_bytes, const WeightSpec &spec,
+                const float *A, int64_t M, int64_t lda, float *out, int64_t ldo);
+
 struct MoeShape {
   int tokens, hidden, intermediate, experts, topk;
   bool renormalize;

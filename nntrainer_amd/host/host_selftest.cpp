@@ -27,6 +27,8 @@
  *   qkv <dtype> <K> <Nq> <Nk> <Nv> <height> <from> <to> <weights> <input> <out>
  *                            qkv_layer; <weights> holds q, k, v; <out> the three outputs one after
  *                            the other
+ *   mlp <dtype> <K> <unit> <batch> <height> <from> <to> <weights> <input> <out>
+ *                            mlp_swiglu; <weights> holds the up then the gate matrix
  *   lmhead <dtype> <K> <unit> <batch> <height> <from> <to> <table> <input> <out>
  *   embed <dtype> <in_dim> <out_dim> <batch> <width> <from> <to> <table> <ids> <out>
  *                            tie_word_embeddings in its two modes
@@ -278,6 +280,18 @@ static int run_api(Context *ctx) {
     EXPECT(ib.getWeightRequests().size() == 26 && ib.getWeightRequests()[3].is_virtual &&
            !ib.getWeightRequests()[1].is_virtual);
   }
+  /* mlp_swiglu: up then gate, the order of the two FCs' weights in a model file */
+  {
+    auto mlp = ctx->createLayerObject("mlp_swiglu", {"unit=3072", "disable_bias=true"});
+    EXPECT(mlp && mlp->getType() == "mlp_swiglu");
+    InitLayerContext ic({TensorDim(1, 1, 4, 1024)}, "l0_ffn", Tformat::NCHW, Tdatatype::Q4_0, Tdatatype::FP32);
+    mlp->finalize(ic);
+    EXPECT(ic.getWeightRequests().size() == 2);
+    EXPECT(ic.getWeightRequests()[0].name == "l0_ffn:up_weight" && ic.getWeightRequests()[1].name == "l0_ffn:gate_weight");
+    EXPECT(ic.getWeightRequests()[1].dim == TensorDim(1, 1, 1024, 3072));
+    EXPECT(ic.getOutputDimensions()[0] == TensorDim(1, 1, 4, 3072));
+    EXPECT_THROW(ctx->createLayerObject("mlp_swiglu", {"unit=8", "disable_bias=false"}), exception::not_supported);
+  }
   /* inference only */
   {
     RunLayerContext rc;
@@ -443,6 +457,32 @@ static int run_qkv(Context *ctx, char **a) {
   return 0;
 }
 
+static int run_mlp(Context *ctx, char **a) {
+  const std::string dt = a[0];
+  const unsigned K = std::atoi(a[1]), N = std::atoi(a[2]), batch = std::atoi(a[3]), height = std::atoi(a[4]),
+                 from = std::atoi(a[5]), to = std::atoi(a[6]);
+  const std::string wpath = a[7], ipath = a[8], opath = a[9];
+  auto layer = ctx->createLayerObject("mlp_swiglu", {"unit=" + std::to_string(N), "disable_bias=true"});
+  InitLayerContext ic({TensorDim(batch, 1, height, K)}, "mlp", Tformat::NCHW, dtype_of(dt), Tdatatype::FP32);
+  layer->finalize(ic);
+  RunLayerContext rc(ic);
+  {
+    std::ifstream f(wpath, std::ios::binary);
+    layer->read(f, rc, false, ml::train::ExecutionMode::INFERENCE, false, dtype_of(dt), false);
+  }
+  read_into(ipath, rc.getInput(0).getData<float>(), (size_t)batch * height * K * 4);
+  float *out = rc.getOutput(0).getData<float>();
+  for (size_t i = 0; i < (size_t)batch * height * N; ++i)
+    out[i] = -12345.f;
+  if (from == 0 && to == 0)
+    layer->forwarding(rc, false);
+  else
+    layer->incremental_forwarding(rc, from, to, false);
+  write_from(opath, out, (size_t)batch * height * N * 4);
+  std::printf("MLP DONE\n");
+  return 0;
+}
+
 static int run_tie(Context *ctx, bool lmhead, char **a) {
   const std::string dt = a[0];
   const unsigned d0 = std::atoi(a[1]), d1 = std::atoi(a[2]), batch = std::atoi(a[3]), len = std::atoi(a[4]),
@@ -493,6 +533,8 @@ int main(int argc, char **argv) {
       return run_moex(ctx, argv + 3);
     if (mode == "qkv" && argc == 14)
       return run_qkv(ctx, argv + 3);
+    if (mode == "mlp" && argc == 13)
+      return run_mlp(ctx, argv + 3);
     if ((mode == "lmhead" || mode == "embed") && argc == 13)
       return run_tie(ctx, mode == "lmhead", argv + 3);
     std::printf("bad arguments for mode %s (argc %d)\n", mode.c_str(), argc);

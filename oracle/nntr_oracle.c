@@ -984,6 +984,13 @@ void orc_moe_forward_q4_K(int T, int H, int I, int E, int topk, const float *x,
   orc_moe_forward(12, 1, T, H, I, E, topk, x, logits, gate, up, down, y, topk_idx, topk_w);
 }
 
+/* nntrainer::swiglu(N, X, Y, Z): X = (Y / (1 + exp(-Y))) * Z, fp32 with the float exponential
+ * (fallback_internal.cpp:417-423; the AVX2 build evaluates the same expression with a polynomial
+ * exponential, avx2_impl.cpp:304-311, within the path's tolerance of this one). */
+void orc_swiglu(int64_t n, float *x, const float *y, const float *z) {
+  for (int64_t i = 0; i < n; ++i) x[i] = (y[i] / (1.f + expf(-y[i]))) * z[i];
+}
+
 void orc_set_threads(int n) {
 #ifdef _OPENMP
   omp_set_num_threads(n);

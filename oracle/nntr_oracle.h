@@ -113,6 +113,7 @@ void orc_moe_forward_q4_K(int T, int H, int I, int E, int topk, const float *x,
                           const void *const *up, const void *const *down,
                           float *y, int32_t *topk_idx, float *topk_w);
 
+void orc_swiglu(int64_t n, float *x, const float *y, const float *z);
 void orc_set_threads(int n);
 
 #ifdef __cplusplus

@@ -232,3 +232,13 @@ def moe_forward_gpt_oss(x, logits, gate, up, down, gate_bias, up_bias, down_bias
                                 arr(up), arr(down), _ptr(gb), _ptr(ub), _ptr(db), _c.c_float(alpha), _ptr(y),
                                 _ptr(idx), _ptr(wt))
     return y, idx, wt
+
+
+def swiglu(y, z):
+    """Oracle of nntrainer::swiglu: (y / (1 + exp(-y))) * z in fp32."""
+    lib = oracle()
+    y = np.ascontiguousarray(y, np.float32)
+    z = np.ascontiguousarray(z, np.float32)
+    x = np.empty_like(y)
+    lib.orc_swiglu(_c.c_int64(y.size), _ptr(x), _ptr(y), _ptr(z))
+    return x

@@ -167,3 +167,38 @@ def test_gpt_oss_moe_router_bias_and_host_memory(hipq, cr):
                                  mem=capi.MEM_HOST)
     for w in wg + wu + wd:
         w.destroy()
+
+
+@pytest.mark.parametrize("kind,m,k,n", [("q4_0", 1, 1024, 3072), ("q4_K", 1, 2048, 768), ("q6_K", 1, 1024, 512),
+                                        ("q4_0", 1, 96, 320),      # K below one chunk unit: not fused
+                                        ("q4_0", 24, 1024, 3072), ("q4_K", 5, 1024, 512)])
+@pytest.mark.parametrize("mem", ["device", "host"])
+def test_mlp_swiglu_matches_oracle(hipq, cr, kind, m, k, n, mem):
+    """hipq_mlp_swiglu: out = swiglu(a . Wact^T, a . Wmul^T) (swiglu.cpp:40-62 on the outputs of
+    ffn_up and ffn_gate, causal_lm.cpp:672-695). The products carry the bits of hipq_matmul; the
+    exponential is the device's, so the result is held to the fp32 tolerance."""
+    import gpu_util as gu
+    import torch
+    wa = cr.quantize_weights(cr.oracle(), kind, synth.normal(7800 + n, (n, k), 0.05))
+    wm = cr.quantize_weights(cr.oracle(), kind, synth.normal(7801 + n, (n, k), 0.05))
+    a = synth.normal(7802 + m, (m, k))
+    y = cr.gemm(cr.oracle(), kind, a, wa, n)
+    z = cr.gemm(cr.oracle(), kind, a, wm, n)
+    ref = cr.swiglu(y, z)
+    assert np.abs(ref - y * z).max() > 0.05 * np.abs(ref).max(), "the activation must matter in this case"
+    ha, hm = capi.Weight(kind, n, k, wa), capi.Weight(kind, n, k, wm)
+    if mem == "device":
+        out = torch.full((m, n), float("nan"), device="cuda")
+        capi.mlp_swiglu(ha, hm, gu.dev(a), m, out, stream=gu.stream())
+        torch.cuda.synchronize()
+        got = out.cpu().numpy()
+    else:
+        got = np.full((m, n), np.nan, np.float32)
+        capi.mlp_swiglu(ha, hm, a, m, got, mem=capi.MEM_HOST)
+    assert not np.isnan(got).any()
+    assert gu.rel_err(got, ref) <= gu.TOL, gu.rel_err(got, ref)
+    # and it is the activation of the library's own products, element by element
+    yg, zg = gu.gpu_matmul(ha, a), gu.gpu_matmul(hm, a)
+    assert np.abs(got - cr.swiglu(yg, zg)).max() <= 1e-6 * np.abs(ref).max()
+    ha.destroy()
+    hm.destroy()

@@ -324,3 +324,28 @@ def test_gpt_oss_moe_layers(cr, tmp_path, layer, incremental):
     assert "active_virtual=0" in out
     got = np.fromfile(tmp_path / "y.bin", np.float32).reshape(t, h)
     assert np.abs(got - ref_y).max() / np.abs(ref_y).max() <= 2e-4
+
+
+@pytest.mark.parametrize("kind,k,n,batch,height,frm,to", [("q4_0", 1024, 3072, 1, 1, 5, 6),   # decode: one launch
+                                                          ("q4_K", 1024, 768, 1, 20, 0, 0),    # forwarding
+                                                          ("q4_0", 512, 256, 2, 8, 0, 5)])     # prefill step, batch 2
+def test_mlp_swiglu_layer(cr, tmp_path, kind, k, n, batch, height, frm, to):
+    """mlp_swiglu through the context: ffn_up, ffn_gate and the SwiGLU between them
+    (causal_lm.cpp:672-695) as one layer; weights in the file order of the two FCs."""
+    up, fup = _framework_bytes(cr, kind, synth.normal(8500, (n, k), 0.05), n, k)
+    gate, fgate = _framework_bytes(cr, kind, synth.normal(8501, (n, k), 0.05), n, k)
+    x = synth.normal(8502 + height, (batch, height, k))
+    with open(tmp_path / "w.bin", "wb") as f:
+        f.write(fup.tobytes())
+        f.write(fgate.tobytes())
+    x.tofile(tmp_path / "x.bin")
+    out = _run(["mlp", kind, k, n, batch, height, frm, to, tmp_path / "w.bin", tmp_path / "x.bin", tmp_path / "y.bin"])
+    assert "MLP DONE" in out
+    got = np.fromfile(tmp_path / "y.bin", np.float32).reshape(batch, height, n)
+    rows = height if to == 0 else to - frm
+    for b in range(batch):
+        y = cr.gemm(cr.oracle(), kind, x[b, :rows], up, n)
+        z = cr.gemm(cr.oracle(), kind, x[b, :rows], gate, n)
+        ref = cr.swiglu(y, z)
+        assert np.abs(got[b, :rows] - ref).max() / np.abs(ref).max() <= TOL
+        assert np.all(got[b, rows:] == -12345.0)

@@ -56,7 +56,7 @@ def test_forward_without_device_raises(tmp_path):
 
 
 ADAPTERS = ["hip_context.cpp", "hip_mem_allocator.cpp", "fc_layer_hip.cpp", "moe_layer_hip.cpp",
-            "qkv_layer_hip.cpp", "tie_word_embedding_hip.cpp", "hipq_host.cpp"]
+            "qkv_layer_hip.cpp", "tie_word_embedding_hip.cpp", "mlp_swiglu_layer_hip.cpp", "hipq_host.cpp"]
 
 
 @pytest.mark.skipif(not os.path.isdir(REFERENCE), reason="reference checkout not present")

@@ -298,3 +298,18 @@ def test_golden_digests():
     got = _digest_cases()
     assert got["input_w"] == want["input_w"], "input generator drifted, not the oracle"
     assert got == want
+
+
+def test_swiglu_oracle_is_silu_times_gate():
+    """orc_swiglu against what the mathematics fixes: y * sigmoid(y) * z in float64, its values at
+    0 and for large |y| (z y and 0), and its antisymmetry in z."""
+    rng = np.random.default_rng(11)
+    y = rng.normal(0, 3, 4096).astype(np.float32)
+    z = rng.normal(0, 2, 4096).astype(np.float32)
+    got = cr.swiglu(y, z)
+    want = y.astype(np.float64) / (1.0 + np.exp(-y.astype(np.float64))) * z.astype(np.float64)
+    assert np.abs(got - want).max() <= 4e-7 * np.abs(want).max()
+    assert np.array_equal(cr.swiglu(np.zeros(4, np.float32), z[:4]), np.zeros(4, np.float32))
+    big = np.array([40.0, -40.0, 100.0, -100.0], np.float32)
+    assert np.allclose(cr.swiglu(big, np.full(4, 2.0, np.float32)), [80.0, 0.0, 200.0, 0.0], atol=1e-12)
+    assert np.array_equal(cr.swiglu(y, -z), -got)
