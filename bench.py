@@ -24,7 +24,7 @@ HBM_PEAK_GBS = 8000.0    # MI355X HBM3E peak, GB/s
 # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs of this script, scaled by
 # what the same counters read for its 256 MiB device copy (profiles/gemm_q4k_prefill_m512_k4096_n12288.txt,
 # profiles/gemv_q4k_decode_m1_k4096.txt, profiles/moe_block_q4k_64tok_128experts.txt). Measured once, not live: counters need the profiler attached.
-TRAFFIC_GEMM_C2 = 48.68e6 + 25.17e6
+TRAFFIC_GEMM_C2 = 48.23e6 + 25.17e6
 TRAFFIC_GEMV_C2 = 28.45e6 + 0.05e6
 TRAFFIC_GEMV_LM_HEAD = 350.25e6 + 0.62e6
 METRIC = "Q4 GEMV effective GB/s (%HBM peak); prefill GEMM int8 TOPS (%MFMA peak)"
@@ -411,7 +411,7 @@ def main():
         "config": {"workload": "Q4_K x Q8_K prefill GEMM, M=512 K=4096 N=12288 (BASELINE configs[1]); "
                                "step = activation quantizer + block-dot GEMM on HBM-resident inputs",
                    "M": M, "K": K, "N": N, "weight_copies_rotated": n_copies},
-        "roofline": {"bound": "mfma", "kernel": "gemm_q4k_kernel<2>", "achieved": round(gemm_tops, 3),
+        "roofline": {"bound": "mfma", "kernel": "gemm_q4k_kernel<2, true>", "achieved": round(gemm_tops, 3),
                      "peak": INT8_PEAK_TOPS, "unit": "TOP/s", "frac": round(gemm_tops / INT8_PEAK_TOPS, 5),
                      "kernel_ms": round(gemm_ms, 5), "traffic": TRAFFIC_GEMM_C2,
                      "traffic_from": "profiles/gemm_q4k_prefill_m512_k4096_n12288.txt (counter runs; not live)",
@@ -472,7 +472,7 @@ def main():
             "active_experts": active,
             "roofline": {"bound": "hbm", "achieved": round(moe_gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(moe_gbs / HBM_PEAK_GBS, 5), "algorithmic_bytes_per_block": moe_bytes,
-                         "traffic": 236.2e6 + 123.4e6 + 13.0e6},
+                         "traffic": 238.2e6 + 134.7e6 + 12.0e6},
             "decode_token": {"ms_per_block": round(moe_decode_ms, 5),
                              "ms_per_block_in_a_graph": round(moe_decode_graph_ms, 5),
                              "active_experts": decode_active,
