@@ -63,6 +63,9 @@ struct State {
   std::unordered_map<hipStream_t, Workspace> ws;
   /* one table of expert weight views per MoE layer, found by its first gate weight */
   std::unordered_map<const hipq_weight *, MoeTable> moe_tables;
+  /* held from the look-up of an expert table until the launches that read it are enqueued,
+   * and by whoever frees a table: taken before mu, never the other way round */
+  std::mutex moe_mu;
   int64_t live_weights = 0;
 };
 State g;
@@ -70,6 +73,7 @@ State g;
 } // namespace
 
 namespace hipq {
+thread_local const LaunchTimer *launch_timer = nullptr;
 
 int fail(int code, const char *fmt, ...) {
   va_list ap;
@@ -672,14 +676,17 @@ int hipq_weight_destroy(hipq_weight_t w) {
   if (!w) return HIPQ_OK;
   int rc = require_ready();
   if (rc) return rc;
-  (void)hipDeviceSynchronize();
-  (void)hipFree(w->base);
-  if (w->gt_base) (void)hipFree(w->gt_base);
   {
+    /* no MoE call is between its table look-up and its launches while moe_mu is held, so
+     * after the synchronization nothing on the device reads w or a table that names it */
+    std::lock_guard<std::mutex> ml(g.moe_mu);
+    (void)hipDeviceSynchronize();
+    (void)hipFree(w->base);
+    if (w->gt_base) (void)hipFree(w->gt_base);
     std::lock_guard<std::mutex> lk(g.mu);
     g.live_weights--;
-    /* drop the expert tables that name w, and only those (the device was synchronized
-     * above): the tables of other layers stay valid, also for graphs captured with them */
+    /* drop the expert tables that name w, and only those: the tables of other layers stay
+     * valid, also for graphs captured with them */
     for (auto it = g.moe_tables.begin(); it != g.moe_tables.end();) {
       bool names = false;
       for (const hipq_weight *k : it->second.key) names = names || k == w;
@@ -972,29 +979,34 @@ int hipq_bench_matmul_steps(int n_weights, const hipq_weight_t *w, const float *
   /* one untimed call first: workspace and tile copies exist before the events */
   for (int i = 0; i < n_weights; ++i)
     if ((rc = matmul_tiled(w[i], A, M, lda, C, ldc, s, 0, sc))) return rc;
-  std::vector<hipEvent_t> ev((size_t)2 * steps + 1);
+  /* Two events before and behind the block give the steps' total; every launch carries a
+   * start and a stop event of its own (hipq_internal.h, LaunchTimer), which hold the kernel's
+   * own time without putting marker packets between the kernels. */
+  std::vector<hipEvent_t> ev((size_t)4 * steps + 2);
   for (auto &e : ev) HIPQ_HIP(hipEventCreate(&e));
   HIPQ_HIP(hipStreamSynchronize(s));
-  hipError_t er = hipSuccess;
+  hipError_t er = hipEventRecord(ev[4 * steps], s);
   for (int it = 0; it < steps && !rc && er == hipSuccess; ++it) {
     const hipq_weight *wi = w[it % n_weights];
-    er = hipEventRecord(ev[2 * it], s);
+    const hipq::LaunchTimer tq{ev[4 * it], ev[4 * it + 1]}, tp{ev[4 * it + 2], ev[4 * it + 3]};
+    hipq::launch_timer = &tq;
     rc = matmul_tiled(wi, A, M, lda, C, ldc, s, 2, sc);
-    if (!rc && er == hipSuccess) er = hipEventRecord(ev[2 * it + 1], s);
+    hipq::launch_timer = &tp;
     if (!rc) rc = matmul_tiled(wi, A, M, lda, C, ldc, s, 1, sc);
+    hipq::launch_timer = nullptr;
   }
-  if (er == hipSuccess) er = hipEventRecord(ev[2 * steps], s);
-  if (er == hipSuccess) er = hipEventSynchronize(ev[2 * steps]);
+  if (er == hipSuccess) er = hipEventRecord(ev[4 * steps + 1], s);
+  if (er == hipSuccess) er = hipEventSynchronize(ev[4 * steps + 1]);
   double q = 0.0, p = 0.0;
   float total = 0.f;
   for (int it = 0; it < steps && !rc && er == hipSuccess; ++it) {
     float a = 0.f, b = 0.f;
-    er = hipEventElapsedTime(&a, ev[2 * it], ev[2 * it + 1]);
-    if (er == hipSuccess) er = hipEventElapsedTime(&b, ev[2 * it + 1], ev[2 * it + 2]);
+    er = hipEventElapsedTime(&a, ev[4 * it], ev[4 * it + 1]);
+    if (er == hipSuccess) er = hipEventElapsedTime(&b, ev[4 * it + 2], ev[4 * it + 3]);
     q += a;
     p += b;
   }
-  if (!rc && er == hipSuccess) er = hipEventElapsedTime(&total, ev[0], ev[2 * steps]);
+  if (!rc && er == hipSuccess) er = hipEventElapsedTime(&total, ev[4 * steps], ev[4 * steps + 1]);
   for (auto &e : ev) (void)hipEventDestroy(e);
   if (rc) return rc;
   if (er != hipSuccess) return fail(HIPQ_ERR_RUNTIME, "timing: %s", hipGetErrorString(er));
@@ -1050,8 +1062,11 @@ int hipq_moe_forward_ext(const hipq_moe_desc *desc, const hipq_moe_ext *ext, con
   hipStream_t s = (hipStream_t)stream;
   EnqueueGuard eg(enqueue_lock(s));
 
-  /* device table of the 3E weight views, rebuilt only when the handles change */
+  /* device table of the 3E weight views, rebuilt only when the handles change; moe_mu keeps
+   * the table from being rebuilt or freed by another thread before the launches below are in
+   * the stream (whoever frees one synchronizes the device first, under the same lock) */
   WView *dev_views = nullptr;
+  std::lock_guard<std::mutex> ml(g.moe_mu);
   {
     std::lock_guard<std::mutex> lk(g.mu);
     MoeTable &t = g.moe_tables[gate[0]];

@@ -324,11 +324,11 @@ int launch_tiles(const hipq_weight *w, const QActTiled *qa, int M, float *C, int
   if (w->gt_base) { /* the tile copy, where the weight has one */
     v.qs = w->gt_qs;
     v.hdr = w->gt_hdr;
-    hipLaunchKernelGGL((gemm_q4k_kernel<TM, true>), dim3(grid), dim3(NT), sizeof(Smem<TM>), s, v, qa->qt, qa->amin,
-                       qa->dAt, M, mtiles, ntiles, C, ldc);
+    launch_kernel(gemm_q4k_kernel<TM, true>, dim3(grid), dim3(NT), sizeof(Smem<TM>), s, v, (const int8_t *)qa->qt,
+                  (const uint16_t *)qa->amin, (const float *)qa->dAt, M, mtiles, ntiles, C, ldc);
   } else
-    hipLaunchKernelGGL((gemm_q4k_kernel<TM, false>), dim3(grid), dim3(NT), sizeof(Smem<TM>), s, v, qa->qt, qa->amin,
-                     qa->dAt, M, mtiles, ntiles, C, ldc);
+    launch_kernel(gemm_q4k_kernel<TM, false>, dim3(grid), dim3(NT), sizeof(Smem<TM>), s, v, (const int8_t *)qa->qt,
+                  (const uint16_t *)qa->amin, (const float *)qa->dAt, M, mtiles, ntiles, C, ldc);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
 }

@@ -25,9 +25,12 @@ HIPQ_API int hipq_time_matmul(int n_weights, const hipq_weight_t *w, const float
                               float *ms_per_call);
 
 /** `steps` whole matmuls (activation quantizer, then block-dot kernel) as hipq_matmul
- *  enqueues them, with one event before each quantizer, one between the two kernels and
- *  one behind the last product, all on `stream`: the three figures come from the same
- *  launches and add up (total = quantizer + product). Milliseconds, sums over the steps. */
+ *  enqueues them on `stream`. total_ms: between one event recorded before the first
+ *  quantizer and one behind the last product (nothing else is put into the stream, so the
+ *  kernels follow each other as they do in a caller's loop). quantizer_ms, product_ms: sums
+ *  of the kernels' own durations, taken from a start and a stop event attached to each of
+ *  the same launches (hipExtLaunchKernelGGL): what a kernel trace reports for them.
+ *  total >= quantizer + product; the difference is the time between the kernels. */
 HIPQ_API int hipq_bench_matmul_steps(int n_weights, const hipq_weight_t *w, const float *A, int64_t M,
                                      int64_t lda, float *C, int64_t ldc, int steps, void *stream,
                                      float *total_ms, float *quantizer_ms, float *product_ms);

@@ -207,7 +207,12 @@ __device__ __forceinline__ int rank_in_token(const int32_t *idx, int i, int topk
   return t * topk + r;
 }
 
-/* Count, scan and scatter of the (token, k) pairs by expert in one workgroup of
+/* The kernels below index tables of E entries with the expert ids that route_token wrote in
+ * the same call: it always stores topk distinct ids in [0, E) (topk <= E is checked at the
+ * boundary; a NaN probability counts as 0 and is still selectable), so the ids need no
+ * further range check here.
+ *
+ * Count, scan and scatter of the (token, k) pairs by expert in one workgroup of
  * 1024 threads: the sort of a decode step or a short prefill chunk is a few thousand
  * pairs, and four tiny launches would cost more than the work. E <= 1024. */
 __device__ __forceinline__ void sort_pairs(const int32_t *idx, int P, int E, int topk, int *__restrict__ offsets,

@@ -144,8 +144,9 @@ int launch_quantize_q8_K_tiled(const float *A, int64_t M, int64_t K, int64_t lda
   const int nsb = (int)(K / 256);
   const int64_t total = (int64_t)qa->mtiles * 128 * nsb;
   const unsigned grid = (unsigned)((total + 3) / 4);
-  hipLaunchKernelGGL(quantize_q8_K_kernel<Q8K_TILED>, dim3(grid), dim3(256), 0, s, A, M, total, nsb, lda,
-                     mat_rows, qa->qt, qa->dAt, nullptr, nullptr, qa->amin, nullptr, nullptr);
+  launch_kernel(quantize_q8_K_kernel<Q8K_TILED>, dim3(grid), dim3(256), 0, s, A, M, total, (int)nsb, lda, mat_rows,
+                qa->qt, qa->dAt, (int16_t *)nullptr, (uint8_t *)nullptr, qa->amin, (uint16_t *)nullptr,
+                (uint16_t *)nullptr);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
 }
