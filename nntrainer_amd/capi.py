@@ -25,7 +25,8 @@ SYMBOLS = [
     "hipq_quantize_weights", "hipq_file_layout", "hipq_weights_from_file",
 ]
 # measurement helpers of csrc/hipq_bench.h: exported for bench.py, not part of the product ABI
-BENCH_SYMBOLS = ["hipq_time_matmul", "hipq_bench_matmul_steps", "hipq_bench_mfma_ceiling"]
+BENCH_SYMBOLS = ["hipq_time_matmul", "hipq_bench_matmul_steps", "hipq_bench_mfma_ceiling",
+                 "hipq_bench_tiled_bytes", "hipq_bench_quantize_tiled"]
 
 
 class HipqError(RuntimeError):
@@ -106,6 +107,9 @@ def lib():
         fp = C.POINTER(C.c_float)
         L.hipq_bench_matmul_steps.argtypes = [i32, C.POINTER(vp), vp, i64, i64, vp, i64, i32, vp, fp, fp, fp]
         L.hipq_bench_mfma_ceiling.argtypes = [C.c_float, vp, fp, fp]
+        L.hipq_bench_tiled_bytes.argtypes = [i64, i64]
+        L.hipq_bench_tiled_bytes.restype = i64
+        L.hipq_bench_quantize_tiled.argtypes = [vp, i64, i64, i64, vp, vp]
         _lib = L
     return _lib
 
@@ -307,6 +311,18 @@ def bench_matmul_steps(ws, a, m, c, steps, stream=None):
     check(lib().hipq_bench_matmul_steps(n, hs, _addr(a), m, ws[0].k, _addr(c), ws[0].n, steps, stream,
                                         C.byref(t), C.byref(q), C.byref(p)))
     return t.value / steps, q.value / steps, p.value / steps
+
+
+def bench_tiled_bytes(m, k):
+    n = lib().hipq_bench_tiled_bytes(m, k)
+    if n < 0:
+        raise HipqError(int(n), "bad shape")
+    return int(n)
+
+
+def bench_quantize_tiled(a, m, k, out, lda=None, stream=None):
+    """The tiled Q8_K form of device rows `a` into the device buffer `out` (bench_tiled_bytes)."""
+    check(lib().hipq_bench_quantize_tiled(_addr(a), m, k, lda if lda is not None else k, _addr(out), stream))
 
 
 def bench_mfma_ceiling(target_ms=2.0, stream=None):

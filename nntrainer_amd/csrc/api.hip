@@ -1016,6 +1016,19 @@ int hipq_bench_matmul_steps(int n_weights, const hipq_weight_t *w, const float *
   return HIPQ_OK;
 }
 
+int64_t hipq_bench_tiled_bytes(int64_t M, int64_t K) {
+  if (M <= 0 || K <= 0 || K % 256) return HIPQ_ERR_INVALID_ARGUMENT;
+  return (int64_t)qact_tiled_bytes(M, K);
+}
+
+int hipq_bench_quantize_tiled(const float *A, int64_t M, int64_t K, int64_t lda, void *out, void *stream) {
+  int rc = require_ready();
+  if (rc) return rc;
+  if (!A || !out || M <= 0 || K <= 0) return fail(HIPQ_ERR_INVALID_ARGUMENT, "bad argument");
+  const QActTiled qa = qact_tiled_carve(out, M, K);
+  return hipq::launch_quantize_q8_K_tiled(A, M, K, lda, (M / 4) * 4, &qa, (hipStream_t)stream);
+}
+
 /* ---- mixture of experts ---------------------------------------------------- */
 
 int hipq_moe_forward(const hipq_moe_desc *desc, const hipq_weight_t *gate, const hipq_weight_t *up,

@@ -1,9 +1,10 @@
 /* SPDX-License-Identifier: Apache-2.0 */
 /**
  * @file   hipq_bench.h
- * @brief  Measurement helpers exported by libhipq.so for bench.py only. They are not
- *         part of the product's C ABI (include/hipq.h) and replace nothing in the
- *         reference: event-timed launch loops and a matrix-core ceiling kernel.
+ * @brief  Measurement and test helpers exported by libhipq.so for bench.py and the GPU
+ *         tests only. They are not part of the product's C ABI (include/hipq.h) and
+ *         replace nothing in the reference: event-timed launch loops, a matrix-core
+ *         ceiling kernel, and a view of an internal buffer layout for its parity test.
  */
 #ifndef HIPQ_BENCH_H
 #define HIPQ_BENCH_H
@@ -39,6 +40,14 @@ HIPQ_API int hipq_bench_matmul_steps(int n_weights, const hipq_weight_t *w, cons
  *  four independent accumulators) for about `target_ms`: the int8 rate the matrix cores
  *  sustain here, in TOP/s, and the shader clock during the run in GHz. */
 HIPQ_API int hipq_bench_mfma_ceiling(float target_ms, void *stream, float *tops, float *ghz);
+
+/** The Q8_K activation quantizer in the form the Q4_K prefill product reads (rows tiled by
+ *  128, 16-byte matrix operands; csrc/hipq_internal.h, QActTiled), written into ONE device
+ *  buffer `out` of hipq_bench_tiled_bytes(M, K) bytes: the int8 tiles, then the fp16 parts of
+ *  the sub-block sums, then the scales. For the test that compares it, value by value, with
+ *  the canonical blocks of hipq_quantize_q8_K. A, out: device memory. */
+HIPQ_API int64_t hipq_bench_tiled_bytes(int64_t M, int64_t K);
+HIPQ_API int hipq_bench_quantize_tiled(const float *A, int64_t M, int64_t K, int64_t lda, void *out, void *stream);
 
 #ifdef __cplusplus
 }

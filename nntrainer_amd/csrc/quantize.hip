@@ -60,8 +60,7 @@ __global__ __launch_bounds__(256) void quantize_q8_0_kernel(
 
 /* ---- Q8_K ---------------------------------------------------------------- */
 
-/* One wavefront per (row, super-block). In the tiled mode the grid also covers
- * the padding rows M .. n_sb_total / nsb - 1, which are written as zeros. */
+/* One wavefront per (row, super-block). */
 template <int MODE>
 __global__ __launch_bounds__(256) void quantize_q8_K_kernel(
   const float *__restrict__ A, int64_t M, int64_t n_sb_total, int nsb, int64_t lda,
@@ -72,6 +71,114 @@ __global__ __launch_bounds__(256) void quantize_q8_K_kernel(
   if (sb >= n_sb_total) return; /* uniform per wavefront */
   hipq_quantize_q8_K_wave<MODE>(A, M, sb, nsb, lda, mat_rows, q_out, d_out, bsum_out, canon_out, amin_out,
                                 ql_out, qh_out);
+}
+
+/* The tiled form for the Q4_K prefill GEMM. A wavefront takes super-block b of four
+ * consecutive rows (a 4-aligned quad, so that all four follow the same quantizer's
+ * semantics): sixteen lanes per row, sixteen values per lane in four 16-byte loads, lane
+ * l of a row holding values 64 i + 4 l .. + 3 of the super-block from load i. That is the
+ * arithmetic of hipq_quantize_q8_K_values value by value; the reductions stay inside a
+ * 16-lane row (four DPP steps) and the scale's two divisions serve sixteen values per
+ * lane instead of four. Rows M and beyond of the last 128-row tile are written as zeros. */
+__global__ __launch_bounds__(256) void quantize_q8_K_tiled_kernel(
+  const float *__restrict__ A, int64_t M, int64_t n_units, int nsb, int64_t lda, int64_t mat_rows,
+  int8_t *__restrict__ q_out, float *__restrict__ d_out, uint16_t *__restrict__ amin_out) {
+  const int64_t unit = (int64_t)blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (unit >= n_units) return; /* uniform per wavefront */
+  const int lane = threadIdx.x & 63, l16 = lane & 15;
+  const int64_t mq = unit / nsb;
+  const int b = (int)(unit - mq * nsb);
+  const int64_t m = mq * 4 + (lane >> 4);
+  float x[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+    if (m < M) v = *(const float4 *)(A + m * lda + (int64_t)b * 256 + 64 * i + 4 * l16);
+    x[i][0] = v.x, x[i][1] = v.y, x[i][2] = v.z, x[i][3] = v.w;
+  }
+  float amax = 0.f;
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int c = 0; c < 4; ++c) amax = fmaxf(amax, fabsf(x[i][c]));
+  amax = hipq_group_max<16>(amax);
+  const bool zero = amax == 0.0f;
+  const float amax1 = zero ? 1.f : amax; /* keeps the arithmetic below finite; the results are dropped */
+  int q[4][4];
+  float d;
+  if (mq * 4 < mat_rows) { /* uniform: the 4-row quantizer's semantics */
+    bool hit = false;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int c = 0; c < 4; ++c) hit = hit | (x[i][c] == amax);
+    const unsigned row_hits = (unsigned)(__ballot(hit) >> (lane & 48)) & 0xffffu;
+    const float iscale = row_hits ? __fdiv_rn(-127.f, amax1) : __fdiv_rn(127.f, amax1);
+    d = __fdiv_rn(1.f, iscale);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int c = 0; c < 4; ++c) {
+        const int v = (int)rintf(__fmul_rn(x[i][c], iscale));
+        q[i][c] = max(-128, min(127, v));
+      }
+  } else { /* the row quantizer's: sign of the FIRST value of maximal magnitude */
+    float cand = 0.f;
+    int key = 1024;
+#pragma unroll
+    for (int i = 3; i >= 0; --i)
+#pragma unroll
+      for (int c = 3; c >= 0; --c)
+        if (fabsf(x[i][c]) == amax) {
+          cand = x[i][c];
+          key = 64 * i + 4 * l16 + c;
+        }
+    int kmin = key;
+    kmin = min(kmin, hipq_dpp_i<HIPQ_DPP_XOR1>(kmin));
+    kmin = min(kmin, hipq_dpp_i<HIPQ_DPP_XOR2>(kmin));
+    kmin = min(kmin, hipq_dpp_i<HIPQ_DPP_HALF_MIRROR>(kmin));
+    kmin = min(kmin, hipq_dpp_i<HIPQ_DPP_MIRROR>(kmin));
+    const unsigned owners = (unsigned)(__ballot(key == kmin) >> (lane & 48)) & 0xffffu;
+    const int src = (lane & 48) + __ffs((int)owners) - 1; /* keys are distinct: one owner, or all when none has one */
+    const float vmax = __shfl(cand, src, HIPQ_WAVE);
+    const float iscale = __fdiv_rn(-127.f, zero ? 1.f : vmax);
+    d = __fdiv_rn(1.f, iscale);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+      for (int c = 0; c < 4; ++c) q[i][c] = min(127, magic_to_int(__fmaf_rn(iscale, x[i][c], kRoundMagic)));
+  }
+  if (zero) {
+    d = 0.f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) q[i][0] = q[i][1] = q[i][2] = q[i][3] = 0;
+  }
+
+  const int64_t mt = m >> 7;
+  const int r = (int)(m & 127);
+  const int64_t rb = (mt * nsb + b) * 128 + r;
+  if (l16 == 0) d_out[rb] = d;
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    /* the quad of lanes 4k .. 4k+3 holds the 16-value group 4 i + k: half (k & 1) of
+     * sub-block jb = 2 i + (k >> 1). The GEMM's lane (row, g) takes sub-blocks 4g .. 4g+3,
+     * two 32-deep steps each: the group is the operand of step st of lane group g. */
+    const int jb = 2 * i + (l16 >> 3), g = i >> 1;
+    const int st = 2 * (jb & 3) + ((l16 >> 2) & 1);
+    const int64_t tile = (mt * (2 * nsb) + b * 2 + (st >> 2)) * 16384;
+    const int off = ((r >> 5) * 4 + (st & 3)) * 1024 + (g * 32 + (r & 31)) * 16;
+    const uint4 op = hipq_quad_operand(q[i]);
+    if ((lane & 3) == 0) *(uint4 *)(q_out + tile + off) = op;
+    int bs = q[i][0] + q[i][1] + q[i][2] + q[i][3];
+    bs += hipq_dpp_i<HIPQ_DPP_XOR1>(bs);
+    bs += hipq_dpp_i<HIPQ_DPP_XOR2>(bs);
+    bs += hipq_dpp_i<HIPQ_DPP_HALF_MIRROR>(bs); /* the eight lanes of the sub-block */
+    if ((lane & 7) == 0) {
+      const int l6 = bs & 63;
+      amin_out[rb * 16 + jb] = __half_as_ushort(__float2half_rn((float)l6));
+      amin_out[rb * 16 + 8 + jb] = __half_as_ushort(__float2half_rn((float)(bs - l6)));
+    }
+  }
 }
 
 } // namespace
@@ -142,11 +249,10 @@ int launch_quantize_q8_K_tiled(const float *A, int64_t M, int64_t K, int64_t lda
   if (((uintptr_t)A & 15) || (lda & 3))
     return fail(HIPQ_ERR_INVALID_ARGUMENT, "activation rows must be 16-byte aligned");
   const int nsb = (int)(K / 256);
-  const int64_t total = (int64_t)qa->mtiles * 128 * nsb;
-  const unsigned grid = (unsigned)((total + 3) / 4);
-  launch_kernel(quantize_q8_K_kernel<Q8K_TILED>, dim3(grid), dim3(256), 0, s, A, M, total, (int)nsb, lda, mat_rows,
-                qa->qt, qa->dAt, (int16_t *)nullptr, (uint8_t *)nullptr, qa->amin, (uint16_t *)nullptr,
-                (uint16_t *)nullptr);
+  const int64_t units = (int64_t)qa->mtiles * 32 * nsb; /* (row quad, super-block) pairs, padding rows included */
+  const unsigned grid = (unsigned)((units + 3) / 4);
+  launch_kernel(quantize_q8_K_tiled_kernel, dim3(grid), dim3(256), 0, s, A, M, units, (int)nsb, lda, mat_rows, qa->qt,
+                qa->dAt, qa->amin);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
 }

@@ -61,7 +61,6 @@ __device__ __forceinline__ int hipq_quantize_q8_0_lane(const float4 &x, uint16_t
 enum {
   Q8K_PLANES = 0,
   Q8K_CANONICAL = 1,
-  Q8K_TILED = 2,
   Q8K_ROWMMA = 3,
   Q8K_DIGITS = 4, /* of the planes only what the Q4_K GEMV reads: ql, qh, bsum, d */
   Q8K_BYTES = 5   /* of the planes only what the Q6_K GEMV reads: q, d */
@@ -128,29 +127,6 @@ __device__ __forceinline__ void hipq_quantize_q8_K_values(
     if (lane == 0) *(float *)o = d;
     *(int *)(o + 4 + lane * 4) = packed;
     if ((lane & 3) == 0) *(int16_t *)(o + 260 + (lane >> 2) * 2) = (int16_t)gsum;
-  } else if (MODE == Q8K_TILED) {
-    const int64_t mt = m >> 7;
-    const int r = (int)(m & 127);
-    /* lane holds elements 4*lane .. 4*lane+3 of the super-block: sub-block lane / 8,
-     * whose 16-value half (lane / 4) % 2 is one 16-byte operand. The GEMM's lane
-     * (row, g) takes sub-blocks 4g .. 4g+3, two 32-deep steps each, so the operand
-     * belongs to step s = 2 * (sub-block % 4) + half of lane group g = sub-block / 4;
-     * within the operand the 8 even values come first, then the 8 odd ones (the
-     * order in which the weights' nibble bytes unpack). */
-    const int jb = lane >> 3, g = jb >> 2;
-    const int st = 2 * (jb & 3) + ((lane >> 2) & 1);
-    const int64_t tile = (mt * (2 * nsb) + b * 2 + (st >> 2)) * 16384;
-    const int off = ((r >> 5) * 4 + (st & 3)) * 1024 + (g * 32 + (r & 31)) * 16;
-    const uint4 op = hipq_quad_operand(q); /* one 16-byte store per quad instead of eight of 2 bytes */
-    if ((lane & 3) == 0) *(uint4 *)(q_out + tile + off) = op;
-    const int64_t rb = (mt * nsb + b) * 128 + r;
-    if (lane == 0) d_out[rb] = d;
-    const int bs = gsum + __shfl_xor(gsum, 4, HIPQ_WAVE); /* two 16-value groups = one sub-block */
-    if ((lane & 7) == 0) {
-      const int l6 = bs & 63;
-      amin_out[rb * 16 + (lane >> 3)] = __half_as_ushort(__float2half_rn((float)l6));
-      amin_out[rb * 16 + 8 + (lane >> 3)] = __half_as_ushort(__float2half_rn((float)(bs - l6)));
-    }
   } else if (MODE == Q8K_ROWMMA) {
     /* row-major, each 16-value group stored as its 8 even then its 8 odd values:
      * this lane's four values are elements 4l .. 4l+3 of group lane / 4 */
@@ -181,8 +157,7 @@ __device__ __forceinline__ void hipq_quantize_q8_K_values(
   }
 }
 
-/* The same with the values read from row m of A. In the tiled mode rows M and
- * beyond are padding and are written as zeros. */
+/* The same with the values read from row m of A (rows M and beyond read as zeros). */
 template <int MODE>
 __device__ __forceinline__ void hipq_quantize_q8_K_wave(
   const float *__restrict__ A, int64_t M, int64_t sb, int nsb, int64_t lda, int64_t mat_rows,
