@@ -75,6 +75,30 @@ def cpu_baseline(blocks_host, a_host, gpu_out, budget_s=12.0):
             "gpu_vs_cpu_max_rel_err": err}
 
 
+def cpu_port_all_threads(kind, m, n, k, a_host, blocks_host, work, unit, budget_s=4.0):
+    """The second thread policy of the reference: every hardware thread over a column partition,
+    what its default `mixed` back-end does (BS::thread_pool(hardware_concurrency()),
+    bs_thread_pool_manager.hpp:41). That back-end's pool is not part of the library built from
+    the reference's sources here, so this figure times this repository's C restatement of the
+    same kernels (kind "port") with all threads of the box's CPU share."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import cpuref as cr
+    lib = cr.oracle()
+    threads = max(1, min(os.cpu_count() or 1, int(os.environ.get("OMP_THREAD_LIMIT", "16"))))
+    lib.orc_set_threads(threads)
+    cr.gemm(lib, kind, a_host, blocks_host, n)
+    t0, reps = time.perf_counter(), 0
+    while True:
+        cr.gemm(lib, kind, a_host, blocks_host, n)
+        reps += 1
+        el = time.perf_counter() - t0
+        if el > budget_s or reps >= 500:
+            break
+    return {"value": round(work / (el / reps) / (1e12 if unit == "TOPS" else 1e9), 4), "unit": unit,
+            "threads": threads, "kind": "port", "ms_per_call": round(el / reps * 1e3, 4),
+            "sample": "%d calls, M=%d K=%d N=%d" % (reps, m, k, n)}
+
+
 def cpu_gemv_baseline(kind, n, k, host, nbytes, budget_s=4.0):
     """One-row matmul of the reference library (its OpenMP wrapper asks for 4 threads on this
     path, ggml_interface_omp.cpp:309, 410) on the GPU leg's weights and row: effective GB/s
@@ -496,6 +520,13 @@ def main():
         out["cpu_baseline_gemv"] = {
             "c1_q4_0_m1_k4096_n4096": cpu_gemv_baseline("q4_0", 4096, 4096, c1_host, c1_bytes),
             "c3_q6_K_m1_k4096_n151936": cpu_gemv_baseline("q6_K", 151936, 4096, c3_host, c3_bytes)}
+        out["cpu_baseline_all_threads"] = {
+            "c2_q4_K_m512_k4096_n12288": cpu_port_all_threads("q4_K", M, N, K, a.cpu().numpy(), blocks.cpu().numpy(),
+                                                              2.0 * M * N * K, "TOPS", budget_s=6.0),
+            "c1_q4_0_m1_k4096_n4096": cpu_port_all_threads("q4_0", 1, 4096, 4096, c1_host[1], c1_host[0],
+                                                           c1_bytes, "GB/s", budget_s=2.0),
+            "c3_q6_K_m1_k4096_n151936": cpu_port_all_threads("q6_K", 1, 151936, 4096, c3_host[1], c3_host[0],
+                                                             c3_bytes, "GB/s", budget_s=3.0)}
     for w in weights:
         w.destroy()
     print(json.dumps(out))
