@@ -297,9 +297,14 @@ QAct qact_rows(const QAct &a, int is_k, int64_t r0, int64_t rows) {
   return v;
 }
 
-/* The Q4_K prefill GEMM takes its activations in the tiled form and addresses
- * the weight planes with 32-bit byte offsets. */
-bool wants_tiled(const hipq_weight *w, int64_t M) {
+/* The prefill GEMMs of the K-formats take their activations in the tiled form. The Q4_K one
+ * addresses the weight planes with 32-bit byte offsets where it has no tile copy; the Q6_K
+ * one reads the tile copy only, which the entry point that may not allocate cannot build
+ * (such a call then walks the rows eight at a time through the GEMV engine, as every call with
+ * up to 16 rows does: two or three passes over the weights cost what a 64-row tile does, and
+ * keep the reference's bits). */
+bool wants_tiled(const hipq_weight *w, int64_t M, bool may_allocate = true) {
+  if (w->dtype == HIPQ_Q6_K) return M > 16 && (w->gt_base || may_allocate);
   return w->dtype == HIPQ_Q4_K && M > 8 && w->N * (w->K / 2) < (int64_t(1) << 32);
 }
 
@@ -367,18 +372,22 @@ int matmul_tiled(const hipq_weight *w, const float *A, int64_t M, int64_t lda, f
   int rc = sc.get(qact_tiled_bytes(M, w->K), &mem);
   if (rc) return rc;
   QActTiled qa = qact_tiled_carve(mem, M, w->K);
-  if (phase != 1) rc = hipq::launch_quantize_q8_K_tiled(A, M, w->K, lda, (M / 4) * 4, &qa, s);
+  /* rows below the last multiple of four follow the 4-row quantizer for Q4_K (what the
+   * reference's GEMM wrapper calls for them); its Q6_K path quantizes row by row */
+  const int64_t mat_rows = w->dtype == HIPQ_Q4_K ? (M / 4) * 4 : 0;
+  if (phase != 1) rc = hipq::launch_quantize_q8_K_tiled(A, M, w->K, lda, mat_rows, &qa, s);
   if (rc || phase == 2) return rc;
   /* The GEMM reads a tile copy of the weights (coalesced loads), made at the weight's first
    * prefill product; the entry point that may not allocate reads the planes until it exists. */
   if (!w->gt_base && !sc.fixed && (rc = hipq::ensure_gemm_tiles(const_cast<hipq_weight *>(w)))) return rc;
+  if (w->dtype == HIPQ_Q6_K) return hipq::launch_gemm_q6k(w, &qa, (int)M, C, ldc, s);
   return hipq::launch_gemm_q4k(w, &qa, (int)M, C, ldc, s);
 }
 
 int matmul_device(hipq_weight_t w, const float *A, int64_t M, int64_t lda, float *C, int64_t ldc,
                   hipStream_t s, const Scratch &sc) {
   if (M == 0) return HIPQ_OK;
-  if (wants_tiled(w, M)) return matmul_tiled(w, A, M, lda, C, ldc, s, 0, sc);
+  if (wants_tiled(w, M, !sc.fixed)) return matmul_tiled(w, A, M, lda, C, ldc, s, 0, sc);
   if (M == 1 && hipq::gemv_fuses_quantizer(w, A)) return hipq::launch_gemv_fused(w, A, C, s);
   const int is_k = w->dtype != HIPQ_Q4_0;
   void *mem = nullptr;
@@ -543,7 +552,7 @@ int hipq_weight_create(int dtype, int layout, int64_t N, int64_t K, const void *
   w->device = g.device;
   w->expert_tiles = 0;
   w->gt_base = nullptr;
-  w->gt_qs = w->gt_hdr = nullptr;
+  w->gt_qs = w->gt_qh = w->gt_hdr = nullptr;
   w->N = N;
   w->K = K;
   /* planes, each 256-byte aligned */
@@ -874,13 +883,13 @@ int hipq_matmul_multi(int count, const hipq_weight_t *w, const float *A, int64_t
   /* one quantization per distinct activation format among the weights */
   auto klass = [&](const hipq_weight *x) {
     if (x->dtype == HIPQ_Q4_0) return 0;
-    if (wants_tiled(x, M)) return 3;
+    if (wants_tiled(x, M)) return x->dtype == HIPQ_Q4_K ? 3 : 4; /* the two tiled forms differ in their rows' quantizer */
     return (x->dtype == HIPQ_Q4_K && M > 1) ? 1 : 2;
   };
-  {
+  for (int k = 3; k <= 4; ++k) {
     bool first = true;
     for (int i = 0; i < count; ++i)
-      if (klass(w[i]) == 3) {
+      if (klass(w[i]) == k) {
         if ((rc = matmul_tiled(w[i], A, M, lda, C[i], ldc[i], s, first ? 0 : 1, Scratch{false, s}))) return rc;
         first = false;
       }

@@ -61,14 +61,21 @@ struct hipq_weight {
   const uint8_t *hdr;
   const int8_t *sc;
   const uint16_t *d;
-  /* Q4_K only, built by the first prefill product of the weight (ensure_gemm_tiles): a
-   * second copy of the nibbles and headers by tiles of 32 rows, in the order the
-   * wavefronts of the prefill GEMM load them, so that each of their 128-bit load
-   * instructions covers 1 KB of consecutive memory:
+  /* Built by the first prefill product of the weight (ensure_gemm_tiles): a second copy by
+   * tiles of 32 rows, in the order the wavefronts of the prefill GEMM load it, so that each
+   * of their 128-bit load instructions covers 1 KB of consecutive memory.
+   * Q4_K:
    *   gt_qs  [N/32][K/256][4][64][16 B]: load i of lane (n, g) = sub-block 4g + i of row n
-   *   gt_hdr [N/32][K/256][32][16 B] */
+   *   gt_hdr [N/32][K/256][32][16 B]
+   * Q6_K: lane (n, g) owns half g (128 weights) of row n's super-block, eight steps of 16
+   *   weights with one scale each:
+   *   gt_qs  [N/32][K/256][4][64][16 B]: load i = steps 2i, 2i+1; per step 8 bytes, weight
+   *          2k / 2k+1 of the step's 16 in the low / high nibble of byte k (low four bits)
+   *   gt_qh  [N/32][K/256][2][64][16 B]: load i = steps 4i .. 4i+3; per step 4 bytes, byte k =
+   *          bits 4-5 of weights 2k, 2k+8, 2k+1, 2k+9 (two bits each, in that order)
+   *   gt_hdr [N/32][K/256][64][16 B]: the lane's eight int8 scales, then the fp16 d */
   uint8_t *gt_base;
-  const uint8_t *gt_qs, *gt_hdr;
+  const uint8_t *gt_qs, *gt_qh, *gt_hdr;
 };
 
 /* Plain-data view of a weight passed to kernels by value. */
@@ -209,6 +216,7 @@ int launch_gemv(const hipq_weight *w, const QAct *qa, int M, int pair_rows,
 int launch_gemm(const hipq_weight *w, const QAct *qa, int M, float *C,
                 int64_t ldc, hipStream_t s);
 /* gemm_q4k.hip: Q4_K with the sub-block scales folded into two int8 digit planes */
+int launch_gemm_q6k(const hipq_weight *w, const QActTiled *qa, int M, float *C, int64_t ldc, hipStream_t s);
 int launch_gemm_q4k(const hipq_weight *w, const QActTiled *qa, int M, float *C,
                     int64_t ldc, hipStream_t s);
 

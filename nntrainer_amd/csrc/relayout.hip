@@ -168,6 +168,60 @@ __global__ void gemm_tile_q4_K(const uint8_t *__restrict__ qs, const uint8_t *__
       n < N ? *(const uint4 *)(hdr + (n * nsb + sb) * 16) : make_uint4(0, 0, 0, 0);
 }
 
+/* Q6_K planes -> tiles of 32 rows for the prefill GEMM (hipq_internal.h, gt_qs / gt_qh / gt_hdr
+ * of a Q6_K weight): thread = lane (n, g) of one (tile, super-block), which owns half g of
+ * row n's super-block. In block_q6_K order the half's 128 weights are four quarters of 32:
+ * quarter c takes its low four bits from the low (c < 2) or high nibbles of ql bytes
+ * 64 g + 32 (c & 1) .. + 31 and its bits 4-5 from bits 2c, 2c+1 of qh bytes 32 g .. + 31
+ * (dequantize_row_q6_K, nntr_ggml_impl_quant.cpp:1291-1325). Step s of the lane = weights
+ * 16 s .. 16 s + 15 of the half = bytes 16 (s & 1) .. + 15 of quarter s >> 1. The planes
+ * hold ql bytes 64 g + 16 u + t (u = 0, 1) at unit 2g + u of the first plane and the bytes
+ * 32 further on at the same place of the second (relayout_q6_K above). */
+__global__ void gemm_tile_q6_K(const uint8_t *__restrict__ ql, const uint8_t *__restrict__ qh,
+                               const int8_t *__restrict__ sc, const uint16_t *__restrict__ d, int N, int nsb,
+                               int64_t total_sb, int64_t lanes, uint8_t *__restrict__ tq, uint8_t *__restrict__ th,
+                               uint8_t *__restrict__ thd) {
+  const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (p >= lanes) return;
+  const int lane = (int)(p & 63);
+  const int64_t ts = p >> 6; /* tile * nsb + sb */
+  const int sb = (int)(ts % nsb);
+  const int64_t n = (ts / nsb) * 32 + (lane & 31);
+  const int g = lane >> 5;
+  uint32_t x[8][2], hb[8];
+  uint32_t hdr[4] = {0, 0, 0, 0};
+  for (int s = 0; s < 8; ++s) x[s][0] = x[s][1] = hb[s] = 0;
+  if (n < N) {
+    const int64_t i = n * nsb + sb;
+    const uint8_t *qlb = ql + total_sb * 64;
+    for (int s = 0; s < 8; ++s) {
+      const int c = s >> 1;
+      const uint8_t *nib = ((c & 1) ? qlb : ql) + i * 64 + (2 * g + (s & 1)) * 16;
+      const uint8_t *hi = qh + i * 64 + 32 * g + 16 * (s & 1);
+      uint32_t w4[16], w2[16];
+      for (int k = 0; k < 16; ++k) {
+        w4[k] = (c < 2) ? (nib[k] & 15u) : (uint32_t)(nib[k] >> 4);
+        w2[k] = (hi[k] >> (2 * c)) & 3u;
+      }
+      for (int k = 0; k < 4; ++k) {
+        x[s][0] |= (w4[2 * k] | (w4[2 * k + 1] << 4)) << (8 * k);
+        x[s][1] |= (w4[8 + 2 * k] | (w4[8 + 2 * k + 1] << 4)) << (8 * k);
+        hb[s] |= (w2[2 * k] | (w2[2 * k + 8] << 2) | (w2[2 * k + 1] << 4) | (w2[2 * k + 9] << 6)) << (8 * k);
+      }
+      /* the scale of weights 128 g + 16 s .. + 15 is scales[8 g + s]; the plane keeps scale j of
+       * half h at (2 h + (j & 1)) * 4 + ((j & 7) >> 1) */
+      const uint32_t sv = (uint8_t)sc[i * 16 + (2 * g + (s & 1)) * 4 + (s >> 1)];
+      hdr[s >> 2] |= sv << (8 * (s & 3));
+    }
+    hdr[2] = d[i];
+  }
+  for (int q = 0; q < 4; ++q)
+    *(uint4 *)(tq + ((ts * 4 + q) * 64 + lane) * 16) = make_uint4(x[2 * q][0], x[2 * q][1], x[2 * q + 1][0], x[2 * q + 1][1]);
+  for (int q = 0; q < 2; ++q)
+    *(uint4 *)(th + ((ts * 2 + q) * 64 + lane) * 16) = make_uint4(hb[4 * q], hb[4 * q + 1], hb[4 * q + 2], hb[4 * q + 3]);
+  *(uint4 *)(thd + (ts * 64 + lane) * 16) = make_uint4(hdr[0], hdr[1], hdr[2], hdr[3]);
+}
+
 } // namespace
 
 namespace hipq {
@@ -176,19 +230,27 @@ int ensure_gemm_tiles(hipq_weight *w) {
   static std::mutex mu; /* two threads may run their first prefill product on one weight */
   std::lock_guard<std::mutex> lk(mu);
   if (w->gt_base) return HIPQ_OK;
-  if (w->dtype != HIPQ_Q4_K || w->expert_tiles)
-    return fail(HIPQ_ERR_INVALID_ARGUMENT, "only Q4_K weights in the plane layout have a GEMM tile copy");
+  if ((w->dtype != HIPQ_Q4_K && w->dtype != HIPQ_Q6_K) || w->expert_tiles)
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "only Q4_K and Q6_K weights in the plane layout have a GEMM tile copy");
   const int nsb = (int)(w->K / 256);
   const int64_t tiles = (w->N + 31) / 32;
-  const size_t q_bytes = (size_t)tiles * nsb * 4096, h_bytes = (size_t)tiles * nsb * 512;
-  const size_t o_hdr = (q_bytes + 255) & ~(size_t)255;
+  const bool q6 = w->dtype == HIPQ_Q6_K;
+  /* Q4_K: nibbles, headers. Q6_K: nibbles, high bits, scales (every part a multiple of 256 bytes) */
+  const size_t q_bytes = (size_t)tiles * nsb * 4096, x_bytes = q6 ? (size_t)tiles * nsb * 2048 : 0,
+               h_bytes = (size_t)tiles * nsb * (q6 ? 1024 : 512);
   uint8_t *nb = nullptr;
-  hipError_t e = hipMalloc((void **)&nb, o_hdr + h_bytes);
+  hipError_t e = hipMalloc((void **)&nb, q_bytes + x_bytes + h_bytes);
   if (e != hipSuccess)
-    return fail(HIPQ_ERR_OUT_OF_MEMORY, "GEMM tiles of %zu bytes: %s", o_hdr + h_bytes, hipGetErrorString(e));
-  const int64_t pieces = tiles * nsb * 256;
-  hipLaunchKernelGGL(gemm_tile_q4_K, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, nullptr, w->qs, w->hdr,
-                     (int)w->N, nsb, pieces, nb, nb + o_hdr);
+    return fail(HIPQ_ERR_OUT_OF_MEMORY, "GEMM tiles of %zu bytes: %s", q_bytes + x_bytes + h_bytes, hipGetErrorString(e));
+  if (q6) {
+    const int64_t lanes = tiles * nsb * 64;
+    hipLaunchKernelGGL(gemm_tile_q6_K, dim3((unsigned)((lanes + 255) / 256)), dim3(256), 0, nullptr, w->qs, w->qh, w->sc,
+                       w->d, (int)w->N, nsb, (int64_t)w->N * nsb, lanes, nb, nb + q_bytes, nb + q_bytes + x_bytes);
+  } else {
+    const int64_t pieces = tiles * nsb * 256;
+    hipLaunchKernelGGL(gemm_tile_q4_K, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, nullptr, w->qs, w->hdr,
+                       (int)w->N, nsb, pieces, nb, nb + q_bytes);
+  }
   e = hipGetLastError();
   if (e == hipSuccess) e = hipStreamSynchronize(nullptr); /* the caller's stream may be another one */
   if (e != hipSuccess) {
@@ -196,7 +258,8 @@ int ensure_gemm_tiles(hipq_weight *w) {
     return fail(HIPQ_ERR_RUNTIME, "GEMM tiling: %s", hipGetErrorString(e));
   }
   w->gt_qs = nb;
-  w->gt_hdr = nb + o_hdr;
+  w->gt_qh = q6 ? nb + q_bytes : nullptr;
+  w->gt_hdr = nb + q_bytes + x_bytes;
   w->gt_base = nb; /* last: readers test this field */
   return HIPQ_OK;
 }

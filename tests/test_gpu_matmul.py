@@ -71,12 +71,40 @@ def test_gemm_matches_oracle(hipq, cr, kind, m, n, k):
     w.destroy()
     assert not np.isnan(got).any()
     assert gu.rel_err(got, ref) <= gu.TOL, gu.rel_err(got, ref)
-    if kind != "q4_K":
-        # Q4_0 (one fma per 32-block, in block order) and Q6_K (rows through the GEMV
-        # engine) reproduce the reference's fp32 order: same bits, so a decoder's prefill
-        # cannot drift from the CPU leg. The Q4_K matrix-core GEMM does not claim that.
+    if kind == "q4_0":
+        # Q4_0 (one fma per 32-block, in block order) reproduces the reference's fp32 order:
+        # same bits, so a decoder's prefill cannot drift from the CPU leg. The matrix-core
+        # GEMMs of the K-formats (two int8 planes per product) do not claim that.
         assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), \
             "%d of %d outputs differ in bits" % ((got.view(np.uint32) != ref.view(np.uint32)).sum(), got.size)
+
+
+@pytest.mark.parametrize("m,n,k", [(17, 128, 256), (33, 200, 768), (64, 96, 1024), (100, 1000, 512),
+                                   (512, 4096, 4096), (1100, 8192, 512)])
+def test_q6_K_gemm_matches_oracle(hipq, cr, m, n, k):
+    """The Q6_K prefill product on the matrix cores (M > 8): one and three super-blocks per row,
+    N not a multiple of the 32-row weight tiles or of the 128-column workgroup tiles, M not a
+    multiple of the tile heights, a shape that takes the 128-row tiles, and the size of a
+    Q6_K FC of a 4096-wide model. Rows up to eight keep the GEMV engine and the reference's bits."""
+    import gpu_util as gu
+    blocks = _weights(cr, "q6_K", n, k, seed=61 + m)
+    a = synth.normal(600 + m, (m, k))
+    a[0, :] = 0.0                      # a row of zero scales
+    a[m - 1, 3] = 40.0                 # a row whose scale is set by one value
+    ref = cr.gemm(cr.oracle(), "q6_K", a, blocks, n)
+    w = capi.Weight("q6_K", n, k, blocks)
+    got = gu.gpu_matmul(w, a)
+    again = gu.gpu_matmul(w, a)        # the weight's tile copy exists now
+    few = gu.gpu_matmul(w, a[:8])
+    w.destroy()
+    assert not np.isnan(got).any()
+    assert gu.rel_err(got, ref) <= gu.TOL, gu.rel_err(got, ref)
+    assert np.array_equal(got, again)
+    assert np.array_equal(few.view(np.uint32), ref[:8].view(np.uint32))
+    # per row as well: a row of small outputs must not hide behind the matrix maximum
+    scale = np.abs(ref).max(axis=1)
+    rows = scale > 0
+    assert (np.abs(got - ref).max(axis=1)[rows] / scale[rows]).max() <= 2e-4
 
 
 def test_q4_K_gemm_tall_tiles(hipq, cr):
