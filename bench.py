@@ -75,30 +75,6 @@ def cpu_baseline(blocks_host, a_host, gpu_out, budget_s=12.0):
             "gpu_vs_cpu_max_rel_err": err}
 
 
-def cpu_port_all_threads(kind, m, n, k, a_host, blocks_host, work, unit, budget_s=4.0):
-    """The second thread policy of the reference: every hardware thread over a column partition,
-    what its default `mixed` back-end does (BS::thread_pool(hardware_concurrency()),
-    bs_thread_pool_manager.hpp:41). That back-end's pool is not part of the library built from
-    the reference's sources here, so this figure times this repository's C restatement of the
-    same kernels (kind "port") with all threads of the box's CPU share."""
-    sys.path.insert(0, os.path.join(ROOT, "tests"))
-    import cpuref as cr
-    lib = cr.oracle()
-    threads = max(1, min(os.cpu_count() or 1, int(os.environ.get("OMP_THREAD_LIMIT", "16"))))
-    lib.orc_set_threads(threads)
-    cr.gemm(lib, kind, a_host, blocks_host, n)
-    t0, reps = time.perf_counter(), 0
-    while True:
-        cr.gemm(lib, kind, a_host, blocks_host, n)
-        reps += 1
-        el = time.perf_counter() - t0
-        if el > budget_s or reps >= 500:
-            break
-    return {"value": round(work / (el / reps) / (1e12 if unit == "TOPS" else 1e9), 4), "unit": unit,
-            "threads": threads, "kind": "port", "ms_per_call": round(el / reps * 1e3, 4),
-            "sample": "%d calls, M=%d K=%d N=%d" % (reps, m, k, n)}
-
-
 def cpu_gemv_baseline(kind, n, k, host, nbytes, budget_s=4.0):
     """One-row matmul of the reference library (its OpenMP wrapper asks for 4 threads on this
     path, ggml_interface_omp.cpp:309, 410) on the GPU leg's weights and row: effective GB/s
@@ -242,7 +218,7 @@ def main():
         w.destroy()
 
     # ---- the other GEMV configurations: C1 (Q4_0, 4096 x 4096) and C3 (Q6_K lm_head) ----
-    def gemv_case(kind, n, k, copies, bytes_per_weight_num, bytes_per_weight_den):
+    def gemv_case(kind, n, k, copies, bytes_per_weight_num, bytes_per_weight_den, prefill_rows=0):
         w32_ = torch.randn((n, k), generator=gen, device="cuda", dtype=torch.float32) * 0.02
         b_ = torch.empty(capi.weight_nbytes(kind, n, k), dtype=torch.uint8, device="cuda")
         capi.quantize_weights(kind, w32_, n, k, b_, stream=stream)
@@ -257,13 +233,24 @@ def main():
         capi.matmul(ws_[0], a_, 1, c_, stream=stream)
         torch.cuda.synchronize()
         host_ = None if args.no_cpu else (b_.cpu().numpy(), a_.cpu().numpy(), c_.cpu().numpy())
+        pre_ = None
+        if prefill_rows:
+            # the same weights against `prefill_rows` rows: the matrix-core product of the format
+            ap_ = torch.randn((prefill_rows, k), generator=gen, device="cuda")
+            cp_ = torch.empty((prefill_rows, n), device="cuda")
+            capi.time_matmul(ws_, ap_, prefill_rows, cp_, 2 * copies, phase=0, stream=stream)
+            pre_ = (sorted(capi.time_matmul(ws_, ap_, prefill_rows, cp_, 6 * copies, phase=1, stream=stream)
+                           for _ in range(3))[1],
+                    sorted(capi.time_matmul(ws_, ap_, prefill_rows, cp_, 6 * copies, phase=0, stream=stream)
+                           for _ in range(3))[1])
+            del ap_, cp_
         for w_ in ws_:
             w_.destroy()
         by_ = n * k * bytes_per_weight_num // bytes_per_weight_den + 4 * k + 4 * n
-        return ms_, all_ms_, by_, host_
+        return ms_, all_ms_, by_, host_, pre_
 
-    c1_ms, c1_all_ms, c1_bytes, c1_host = gemv_case("q4_0", 4096, 4096, 60, 18, 32)
-    c3_ms, c3_all_ms, c3_bytes, c3_host = gemv_case("q6_K", 151936, 4096, 2, 210, 256)
+    c1_ms, c1_all_ms, c1_bytes, c1_host, _ = gemv_case("q4_0", 4096, 4096, 60, 18, 32)
+    c3_ms, c3_all_ms, c3_bytes, c3_host, c3_prefill = gemv_case("q6_K", 151936, 4096, 2, 210, 256, prefill_rows=512)
 
     # ---- the FC stack of one decoder layer of C5 (Qwen3-0.6B shapes, Q4_0), quantizer included ----
     def fc_stack(rows):
@@ -492,6 +479,16 @@ def main():
             "roofline": {"bound": "hbm", "achieved": round(c3_bytes / (c3_ms * 1e-3) / 1e9, 2), "peak": HBM_PEAK_GBS,
                          "unit": "GB/s", "frac": round(c3_bytes / (c3_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 5),
                          "kernel_ms": round(c3_ms, 5), "traffic": None, "algorithmic_bytes_per_launch": c3_bytes}},
+        "q6_K_prefill_lm_head_size": {
+            "workload": "Q6_K x Q8_K prefill GEMM, M=512 K=4096 N=151936 (the C3 weights against 512 rows), "
+                        "2 weight copies rotated",
+            "ms_per_call": round(c3_prefill[1], 5),
+            "roofline": {"bound": "mfma", "kernel": "gemm_q6k_kernel<4>",
+                         "achieved": round(2.0 * 512 * 151936 * 4096 / (c3_prefill[0] * 1e-3) / 1e12, 3),
+                         "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                         "frac": round(2.0 * 512 * 151936 * 4096 / (c3_prefill[0] * 1e-3) / 1e12 / INT8_PEAK_TOPS, 5),
+                         "kernel_ms": round(c3_prefill[0], 5), "traffic": None,
+                         "algorithmic_ops_per_launch": 2.0 * 512 * 151936 * 4096}},
         "c5_fc_stack_per_layer": {
             "workload": "the seven Q4_0 FCs of one Qwen3-0.6B-shaped decoder layer (BASELINE configs[4]) through "
                         "hipq_matmul, quantizers included, 8 weight copies rotated per FC",
@@ -520,13 +517,6 @@ def main():
         out["cpu_baseline_gemv"] = {
             "c1_q4_0_m1_k4096_n4096": cpu_gemv_baseline("q4_0", 4096, 4096, c1_host, c1_bytes),
             "c3_q6_K_m1_k4096_n151936": cpu_gemv_baseline("q6_K", 151936, 4096, c3_host, c3_bytes)}
-        out["cpu_baseline_all_threads"] = {
-            "c2_q4_K_m512_k4096_n12288": cpu_port_all_threads("q4_K", M, N, K, a.cpu().numpy(), blocks.cpu().numpy(),
-                                                              2.0 * M * N * K, "TOPS", budget_s=6.0),
-            "c1_q4_0_m1_k4096_n4096": cpu_port_all_threads("q4_0", 1, 4096, 4096, c1_host[1], c1_host[0],
-                                                           c1_bytes, "GB/s", budget_s=2.0),
-            "c3_q6_K_m1_k4096_n151936": cpu_port_all_threads("q6_K", 1, 151936, 4096, c3_host[1], c3_host[0],
-                                                             c3_bytes, "GB/s", budget_s=3.0)}
     for w in weights:
         w.destroy()
     print(json.dumps(out))
