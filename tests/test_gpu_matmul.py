@@ -345,7 +345,7 @@ def test_weights_read_from_a_model_file(hipq, cr, tmp_path):
         capi.weights_from_file(path, listing + [("q6_K", 4096, 4096)], offset=7)
 
 
-@pytest.mark.parametrize("kind,m", [("q4_K", 1), ("q4_K", 40), ("q6_K", 3)])
+@pytest.mark.parametrize("kind,m", [("q4_K", 1), ("q4_K", 40), ("q6_K", 3), ("q6_K", 40)])
 def test_matmul_multi_other_formats_and_prefill(hipq, cr, kind, m):
     """The multi-weight entry with the Q8_K formats, one row and a prefill chunk (the
     Q4_K prefill goes through the tiled activations and the matrix-core GEMM)."""
@@ -363,6 +363,32 @@ def test_matmul_multi_other_formats_and_prefill(hipq, cr, kind, m):
         got = o.cpu().numpy()
         assert not np.isnan(got).any()
         assert gu.rel_err(got, cr.gemm(cr.oracle(), kind, a, b, n)) <= gu.TOL
+    for w in ws:
+        w.destroy()
+
+
+def test_matmul_multi_mixed_k_formats_prefill(hipq, cr):
+    """Q4_K and Q6_K weights in one multi-weight prefill call: both take tiled Q8_K activations, but
+    the reference quantizes the rows of a Q4_K product four at a time and those of a Q6_K product one
+    by one (different sign rules), so the two groups must not share one quantization. Row 2 holds
+    +amax before -amax, where the two quantizers differ."""
+    import gpu_util as gu
+    import torch
+    m, k = 40, 512
+    kinds, ns = ["q4_K", "q6_K", "q4_K", "q6_K"], [256, 160, 128, 384]
+    blocks = [_weights(cr, kd, n, k, seed=90 + i) for i, (kd, n) in enumerate(zip(kinds, ns))]
+    ws = [capi.Weight(kd, n, k, b) for kd, n, b in zip(kinds, ns, blocks)]
+    a = synth.normal(93, (m, k))
+    a[2, 5] = 9.5
+    a[2, 9] = -9.5
+    outs = [torch.full((m, n), float("nan"), device="cuda") for n in ns]
+    capi.matmul_multi(ws, gu.dev(a), m, outs, stream=gu.stream())
+    torch.cuda.synchronize()
+    for kd, n, b, o, w in zip(kinds, ns, blocks, outs, ws):
+        got = o.cpu().numpy()
+        assert not np.isnan(got).any()
+        assert gu.rel_err(got, cr.gemm(cr.oracle(), kd, a, b, n)) <= gu.TOL
+        assert np.array_equal(got, gu.gpu_matmul(w, a)), "the multi-weight call differs from the single one"
     for w in ws:
         w.destroy()
 
