@@ -95,9 +95,17 @@ __device__ __forceinline__ int acc_row(int r, int lane) { return 8 * (r >> 2) + 
 
 struct Src {
   rsrc_t qt, amin, dAt;
-  const uint4 *wq, *whd; /* this lane's 64 bytes of nibbles / header of super-block 0 */
+  const uint4 *wq, *whd; /* plane layout: this lane's 64 bytes of nibbles / header of super-block 0 */
+  rsrc_t rq, rh;         /* tile copy: the wavefront's tile, nibbles / headers; the descriptors sit in scalar
+                            registers and a load names a lane offset and a scalar offset (no per-lane
+                            64-bit pointers to keep or to add to) */
   int wave, lane;
 };
+typedef unsigned int u4v __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ uint4 ld16(rsrc_t r, uint32_t voff, uint32_t soff) {
+  const u4v v = __builtin_amdgcn_raw_buffer_load_b128(r, (int)voff, (int)soff, 0);
+  return make_uint4(v[0], v[1], v[2], v[3]);
+}
 struct WHalf { /* this lane's two sub-blocks of one 128-deep stage */
   uint4 q[2];
 };
@@ -106,8 +114,8 @@ struct WHalf { /* this lane's two sub-blocks of one 128-deep stage */
  * instruction covers 1 KB of memory instead of 32 separate lines. */
 template <bool TILES> __device__ __forceinline__ void load_wh(WHalf &W, const Src &sr, int sb, int h) {
   if (TILES) {
-    W.q[0] = hipq_ld_global(sr.wq + (sb * 4 + 2 * h) * 64);
-    W.q[1] = hipq_ld_global(sr.wq + (sb * 4 + 2 * h + 1) * 64);
+    W.q[0] = ld16(sr.rq, sr.lane * 16, (uint32_t)(sb * 4 + 2 * h) * 1024);
+    W.q[1] = ld16(sr.rq, sr.lane * 16, (uint32_t)(sb * 4 + 2 * h + 1) * 1024);
   } else {
     W.q[0] = hipq_ld_global(sr.wq + sb * 8 + 2 * h);
     W.q[1] = hipq_ld_global(sr.wq + sb * 8 + 2 * h + 1);
@@ -235,8 +243,10 @@ __global__ __launch_bounds__(NT, TM == 2 ? 3 : 2) void gemm_q4k_kernel(WView w, 
   if (TILES) {
     /* the copy pads N to 32 rows: a wavefront whose columns start below N has its tile */
     const size_t wt = (size_t)(min(n0 + wave * 32, (int)w.N - 1) >> 5);
-    sr.wq = (const uint4 *)(w.qs + wt * nsb * 4096) + lane;
-    sr.whd = (const uint4 *)(w.hdr + wt * nsb * 512) + i32;
+    sr.rq = make_rsrc(w.qs + wt * nsb * 4096, (uint32_t)nsb * 4096);
+    sr.rh = make_rsrc(w.hdr + wt * nsb * 512, (uint32_t)nsb * 512);
+    sr.wq = nullptr;
+    sr.whd = nullptr;
   } else {
     sr.wq = (const uint4 *)(w.qs + (size_t)n * (w.K >> 1) + g * 64);
     sr.whd = (const uint4 *)w.hdr + (size_t)n * nsb;
@@ -254,7 +264,7 @@ __global__ __launch_bounds__(NT, TM == 2 ? 3 : 2) void gemm_q4k_kernel(WView w, 
   WHalf Wa, Wb; /* first / second half of a super-block */
   uint4 hd0, hd1;
   load_wh<TILES>(Wa, sr, 0, 0);
-  hd0 = hipq_ld_global(sr.whd);
+  hd0 = TILES ? ld16(sr.rh, i32 * 16, 0) : hipq_ld_global(sr.whd);
   dma_rows(sr, sm, 0, 0);
   dma_a(sr, sm, 0, 0);
   dma_a(sr, sm, 1, 1);
@@ -285,7 +295,7 @@ __global__ __launch_bounds__(NT, TM == 2 ? 3 : 2) void gemm_q4k_kernel(WView w, 
       const int s2 = slot >= 1 ? slot - 1 : 2;
       dma_a(sr, sm, min(2 * sb + 3, nstage - 1), s2);
       load_wh<TILES>(Wa, sr, sbn, 0);
-      hdn = hipq_ld_global(sr.whd + sbn * HSTRIDE);
+      hdn = TILES ? ld16(sr.rh, i32 * 16, (uint32_t)sbn * 512) : hipq_ld_global(sr.whd + sbn * HSTRIDE);
       stage_mma<1>(sm, slot, Wb, slo, shi, lane, Dlo, Dhi);
       slot = slot == 2 ? 0 : slot + 1;
     }
