@@ -145,7 +145,13 @@ HIPQ_API int hipq_quantize_q8_K(const float *A, int64_t M, int64_t K, int64_t ld
  *  the decode GEMV kernels, M > 1 the prefill GEMM kernels. lda >= K and
  *  ldc >= N are row strides in elements. With M == 1, K <= 4096, N < 32768 and
  *  device memory the call is a single kernel launch (the GEMV quantizes the row
- *  itself) and uses no workspace. */
+ *  itself) and uses no workspace.
+ *  Outputs carry the bits of the reference's AVX2 kernels for every Q4_0 product and for
+ *  Q4_K with up to 8 and Q6_K with up to 16 rows; with more rows the K-formats run on the
+ *  int8 matrix cores and agree with the reference to 1e-4 of the output's maximum (same
+ *  quantized activations, another order of the fp32 sums). The first such product of a
+ *  weight adds a copy of it in the kernels' load order (allocates; 0.56 bytes per weight
+ *  for Q4_K, 0.875 for Q6_K), kept until hipq_weight_destroy. */
 HIPQ_API int hipq_matmul(hipq_weight_t w, const float *A, int64_t M, int64_t lda,
                          float *C, int64_t ldc, int mem, void *stream);
 
