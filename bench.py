@@ -272,8 +272,8 @@ def main():
 
     c5_prefill_ms, c5_decode_ms = fc_stack(512), fc_stack(1)
 
-    def decode_layer_graph(grouped):
-        """One decode step's FCs of 8 layers (8 weight copies) captured in a graph and
+    def decode_layer_graph(grouped, rows=1):
+        """One step's FCs of 8 layers (8 weight copies) against `rows` rows captured in a graph and
         replayed: milliseconds per layer without the host's launch cost. grouped = 1: Q, K, V
         and gate, up each as one hipq_matmul_multi call (4 launches per layer, not 7).
         grouped = 2: Q, K, V as one call and up, gate and the SwiGLU between them and the down
@@ -289,24 +289,24 @@ def main():
                 torch.cuda.synchronize()
                 ws_.append(capi.Weight("q4_0", n_, k_, b_, mem=capi.MEM_DEVICE))
             layers.append(ws_)
-        xs_ = {k_: torch.randn((1, k_), generator=gen, device="cuda") for k_ in (1024, 2048, 3072)}
-        cs_ = [torch.empty((1, n_), device="cuda") for n_, _ in shapes]
+        xs_ = {k_: torch.randn((rows, k_), generator=gen, device="cuda") for k_ in (1024, 2048, 3072)}
+        cs_ = [torch.empty((rows, n_), device="cuda") for n_, _ in shapes]
 
         def step(st):
             for ws_ in layers:
                 if grouped == 2:
-                    capi.matmul_multi(ws_[0:3], xs_[1024], 1, cs_[0:3], stream=st)
-                    capi.matmul(ws_[3], xs_[2048], 1, cs_[3], stream=st)
-                    capi.mlp_swiglu(ws_[4], ws_[5], xs_[1024], 1, cs_[4], stream=st)
-                    capi.matmul(ws_[6], xs_[3072], 1, cs_[6], stream=st)
+                    capi.matmul_multi(ws_[0:3], xs_[1024], rows, cs_[0:3], stream=st)
+                    capi.matmul(ws_[3], xs_[2048], rows, cs_[3], stream=st)
+                    capi.mlp_swiglu(ws_[4], ws_[5], xs_[1024], rows, cs_[4], stream=st)
+                    capi.matmul(ws_[6], xs_[3072], rows, cs_[6], stream=st)
                 elif grouped:
-                    capi.matmul_multi(ws_[0:3], xs_[1024], 1, cs_[0:3], stream=st)
-                    capi.matmul(ws_[3], xs_[2048], 1, cs_[3], stream=st)
-                    capi.matmul_multi(ws_[4:6], xs_[1024], 1, cs_[4:6], stream=st)
-                    capi.matmul(ws_[6], xs_[3072], 1, cs_[6], stream=st)
+                    capi.matmul_multi(ws_[0:3], xs_[1024], rows, cs_[0:3], stream=st)
+                    capi.matmul(ws_[3], xs_[2048], rows, cs_[3], stream=st)
+                    capi.matmul_multi(ws_[4:6], xs_[1024], rows, cs_[4:6], stream=st)
+                    capi.matmul(ws_[6], xs_[3072], rows, cs_[6], stream=st)
                 else:
                     for w_, (n_, k_), c_ in zip(ws_, shapes, cs_):
-                        capi.matmul(w_, xs_[k_], 1, c_, stream=st)
+                        capi.matmul(w_, xs_[k_], rows, c_, stream=st)
 
         side = torch.cuda.Stream()
         side.wait_stream(torch.cuda.current_stream())
@@ -336,6 +336,7 @@ def main():
 
     c5_graph_ms, c5_graph_grouped_ms = decode_layer_graph(0), decode_layer_graph(1)
     c5_graph_fused_ms = decode_layer_graph(2)
+    c5_prefill_graph_ms, c5_prefill_grouped_ms = decode_layer_graph(0, 512), decode_layer_graph(1, 512)
 
     # ---- the MoE block of configs[3]: 64 tokens, 128 experts, top-8, Q4_K ----------
     mt, mh, me, mi, mk = 64, 2048, 128, 768, 8
@@ -492,7 +493,10 @@ def main():
         "c5_fc_stack_per_layer": {
             "workload": "the seven Q4_0 FCs of one Qwen3-0.6B-shaped decoder layer (BASELINE configs[4]) through "
                         "hipq_matmul, quantizers included, 8 weight copies rotated per FC",
-            "prefill_512_rows_ms": round(c5_prefill_ms, 5), "decode_1_row_ms": round(c5_decode_ms, 5),
+            "prefill_512_rows_ms": round(c5_prefill_ms, 5),
+            "prefill_512_rows_in_a_graph_ms": round(c5_prefill_graph_ms, 5),
+            "prefill_512_rows_in_a_graph_qkv_and_gate_up_as_one_call_each_ms": round(c5_prefill_grouped_ms, 5),
+            "decode_1_row_ms": round(c5_decode_ms, 5),
             "decode_1_row_in_a_graph_ms": round(c5_graph_ms, 5),
             "decode_1_row_in_a_graph_qkv_and_gate_up_as_one_launch_each_ms": round(c5_graph_grouped_ms, 5),
             "decode_1_row_in_a_graph_qkv_one_launch_up_gate_swiglu_one_launch_ms": round(c5_graph_fused_ms, 5)},

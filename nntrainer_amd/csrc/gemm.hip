@@ -248,13 +248,32 @@ __device__ __forceinline__ void compute_second_half(const Half &hf, float2 dar, 
   pin(acc);
 }
 
+/* Up to four weights of one K against the same activations as ONE launch: the grid's columns are
+ * the concatenation of the weights' column tiles (Q, K, V or gate, up of a layer: three or two
+ * small grids become one that fills the chip, and two launches fewer). */
+struct MultiQ40 {
+  WView w[4];
+  float *C[4];
+  int64_t ldc[4];
+  int tile_end[4]; /* running sum of the weights' column tiles */
+};
+
 __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void gemm_q40_kernel(
-  WView w, QView qa, int M, float *__restrict__ C, int64_t ldc) {
+  MultiQ40 mw, QView qa, int M) {
   __shared__ SmemQ40 smb[2];
+  /* which weight this workgroup's column tile belongs to (uniform) */
+  int bx = blockIdx.x, wi = 0;
+  if (bx >= mw.tile_end[0]) wi = 1;
+  if (bx >= mw.tile_end[1]) wi = 2;
+  if (bx >= mw.tile_end[2]) wi = 3;
+  if (wi) bx -= mw.tile_end[wi - 1];
+  const WView w = wi == 0 ? mw.w[0] : wi == 1 ? mw.w[1] : wi == 2 ? mw.w[2] : mw.w[3];
+  float *__restrict__ C = wi == 0 ? mw.C[0] : wi == 1 ? mw.C[1] : wi == 2 ? mw.C[2] : mw.C[3];
+  const int64_t ldc = wi == 0 ? mw.ldc[0] : wi == 1 ? mw.ldc[1] : wi == 2 ? mw.ldc[2] : mw.ldc[3];
   const int lane = threadIdx.x & 63;
   const int wave = threadIdx.x >> 6;
   const int wm = wave >> 1, wn = wave & 1; /* 4 x 2 wavefronts, 16 x 16 each */
-  const int n0 = blockIdx.x * BN, m0 = blockIdx.y * BM;
+  const int n0 = bx * BN, m0 = blockIdx.y * BM;
   const int i16 = lane & 15, g = lane >> 4;
   const int nchunks = w.K / KC;
   const int nb = w.K >> 5;
@@ -336,16 +355,40 @@ __global__ __launch_bounds__(NT) __attribute__((amdgpu_waves_per_eu(4, 4))) void
 
 namespace hipq {
 
-int launch_gemm(const hipq_weight *w, const QAct *qa, int M, float *C, int64_t ldc,
-                hipStream_t s) {
+static int check_gemm_weight(const hipq_weight *w) {
   if (w->K % KC) return fail(HIPQ_ERR_NOT_SUPPORTED, "gemm needs K %% 256 == 0, got %lld", (long long)w->K);
   if (w->dtype != HIPQ_Q4_0) return fail(HIPQ_ERR_NOT_SUPPORTED, "gemm: dtype %d has no MFMA path here", w->dtype);
   if ((int64_t)BM * w->K >= (int64_t)1 << 31)
     return fail(HIPQ_ERR_NOT_SUPPORTED, "gemm: K = %lld is beyond the kernel's 32-bit tile offsets", (long long)w->K);
-  const dim3 grid((unsigned)((w->N + BN - 1) / BN), (unsigned)((M + BM - 1) / BM));
-  hipLaunchKernelGGL(gemm_q40_kernel, grid, dim3(NT), 0, s, wview(w), qview(*qa), M, C, ldc);
+  return HIPQ_OK;
+}
+
+int launch_gemm_multi(int count, const hipq_weight *const *w, const QAct *qa, int M, float *const *C,
+                      const int64_t *ldc, hipStream_t s) {
+  if (count < 1 || count > 4) return fail(HIPQ_ERR_INVALID_ARGUMENT, "gemm: 1 to 4 weights per launch, got %d", count);
+  MultiQ40 mw;
+  int tiles = 0;
+  for (int i = 0; i < 4; ++i) {
+    const hipq_weight *wi = w[i < count ? i : count - 1];
+    if (i < count) {
+      if (int rc = check_gemm_weight(wi)) return rc;
+      if (wi->K != w[0]->K) return fail(HIPQ_ERR_INVALID_ARGUMENT, "gemm: the weights of one launch share K");
+      tiles += (int)((wi->N + BN - 1) / BN);
+    }
+    mw.w[i] = wview(wi);
+    mw.C[i] = C[i < count ? i : count - 1];
+    mw.ldc[i] = ldc[i < count ? i : count - 1];
+    mw.tile_end[i] = tiles; /* unused entries repeat the total: no workgroup lands in them */
+  }
+  const dim3 grid((unsigned)tiles, (unsigned)((M + BM - 1) / BM));
+  hipLaunchKernelGGL(gemm_q40_kernel, grid, dim3(NT), 0, s, mw, qview(*qa), M);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
+}
+
+int launch_gemm(const hipq_weight *w, const QAct *qa, int M, float *C, int64_t ldc,
+                hipStream_t s) {
+  return launch_gemm_multi(1, &w, qa, M, &C, &ldc, s);
 }
 
 } // namespace hipq
