@@ -887,6 +887,31 @@ int hipq_matmul_multi(int count, const hipq_weight_t *w, const float *A, int64_t
     return (x->dtype == HIPQ_Q4_K && M > 1) ? 1 : 2;
   };
   for (int k = 3; k <= 4; ++k) {
+    int members = 0;
+    for (int i = 0; i < count; ++i) members += klass(w[i]) == k;
+    if (k == 3 && members > 1) {
+      /* Q4_K: one quantization, then the products four weights a launch (the grids of K and V of
+       * a layer with grouped-query attention would be an eighth of the chip each) */
+      void *mem = nullptr;
+      if ((rc = workspace(s, qact_tiled_bytes(M, w[0]->K), &mem))) return rc;
+      const QActTiled qa = qact_tiled_carve(mem, M, w[0]->K);
+      if ((rc = hipq::launch_quantize_q8_K_tiled(A, M, w[0]->K, lda, (M / 4) * 4, &qa, s))) return rc;
+      const hipq_weight *gw[4];
+      float *gc[4];
+      int64_t gl[4];
+      int ng = 0;
+      for (int i = 0; i < count; ++i) {
+        if (klass(w[i]) != k) continue;
+        if (!w[i]->gt_base && (rc = hipq::ensure_gemm_tiles(const_cast<hipq_weight *>(w[i])))) return rc;
+        gw[ng] = w[i], gc[ng] = C[i], gl[ng] = ldc[i];
+        if (++ng == 4) {
+          if ((rc = hipq::launch_gemm_q4k_multi(ng, gw, &qa, (int)M, gc, gl, s))) return rc;
+          ng = 0;
+        }
+      }
+      if (ng && (rc = hipq::launch_gemm_q4k_multi(ng, gw, &qa, (int)M, gc, gl, s))) return rc;
+      continue;
+    }
     bool first = true;
     for (int i = 0; i < count; ++i)
       if (klass(w[i]) == k) {

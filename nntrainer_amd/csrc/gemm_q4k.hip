@@ -214,18 +214,14 @@ __device__ __forceinline__ void epilogue(const Smem<TM> &sm, int buf, const uint
   }
 }
 
+/* the tile (mt, nt) of one weight's product */
 template <int TM, bool TILES>
-__global__ __launch_bounds__(NT, TM == 2 ? 3 : 2) void gemm_q4k_kernel(WView w, const int8_t *__restrict__ qt,
-                                                         const uint16_t *__restrict__ amin,
-                                                         const float *__restrict__ dAt, int M, int mtiles,
-                                                         int ntiles, float *__restrict__ C, int64_t ldc) {
+__device__ __forceinline__ void gemm_q4k_tile(const WView &w, const int8_t *__restrict__ qt,
+                                              const uint16_t *__restrict__ amin, const float *__restrict__ dAt, int M,
+                                              int mt, int nt, float *__restrict__ C, int64_t ldc) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   Smem<TM> &sm = *reinterpret_cast<Smem<TM> *>(smem_raw);
   constexpr int BM = 32 * TM;
-  const int id = blockIdx.x;
-  const int xcd = id & 7, qd = id >> 3;
-  const int mt = qd % mtiles, nt = (qd / mtiles) * 8 + xcd;
-  if (nt >= ntiles) return; /* uniform per workgroup */
   const int m0 = mt * BM, n0 = nt * BN;
   const int nsb = w.K >> 8;
   const int lane = threadIdx.x & 63;
@@ -320,6 +316,47 @@ __global__ __launch_bounds__(NT, TM == 2 ? 3 : 2) void gemm_q4k_kernel(WView w, 
     }
 }
 
+template <int TM, bool TILES>
+__global__ __launch_bounds__(NT, TM == 2 ? 3 : 2) void gemm_q4k_kernel(WView w, const int8_t *__restrict__ qt,
+                                                         const uint16_t *__restrict__ amin,
+                                                         const float *__restrict__ dAt, int M, int mtiles,
+                                                         int ntiles, float *__restrict__ C, int64_t ldc) {
+  const int id = blockIdx.x;
+  const int xcd = id & 7, qd = id >> 3;
+  const int mt = qd % mtiles, nt = (qd / mtiles) * 8 + xcd;
+  if (nt >= ntiles) return; /* uniform per workgroup */
+  gemm_q4k_tile<TM, TILES>(w, qt, amin, dAt, M, mt, nt, C, ldc);
+}
+
+/* Up to four weights of one K (each with its tile copy) against the same activations as ONE
+ * launch: the column tiles of the weights follow each other in the grid (Q, K, V of a layer with
+ * grouped-query attention: two of the three grids would be an eighth of the chip each). */
+struct MultiQ4K {
+  WView w[4];
+  float *C[4];
+  int64_t ldc[4];
+  int tile_end[4]; /* running sum of the weights' column tiles */
+};
+template <int TM>
+__global__ __launch_bounds__(NT, TM == 2 ? 3 : 2) void gemm_q4k_multi_kernel(MultiQ4K mw, const int8_t *__restrict__ qt,
+                                                               const uint16_t *__restrict__ amin,
+                                                               const float *__restrict__ dAt, int M, int mtiles) {
+  const int id = blockIdx.x;
+  const int xcd = id & 7, qd = id >> 3;
+  const int mt = qd % mtiles;
+  int nt = (qd / mtiles) * 8 + xcd;
+  if (nt >= mw.tile_end[3]) return; /* uniform per workgroup */
+  int wi = 0;
+  if (nt >= mw.tile_end[0]) wi = 1;
+  if (nt >= mw.tile_end[1]) wi = 2;
+  if (nt >= mw.tile_end[2]) wi = 3;
+  if (wi) nt -= mw.tile_end[wi - 1];
+  const WView w = wi == 0 ? mw.w[0] : wi == 1 ? mw.w[1] : wi == 2 ? mw.w[2] : mw.w[3];
+  float *C = wi == 0 ? mw.C[0] : wi == 1 ? mw.C[1] : wi == 2 ? mw.C[2] : mw.C[3];
+  const int64_t ldc = wi == 0 ? mw.ldc[0] : wi == 1 ? mw.ldc[1] : wi == 2 ? mw.ldc[2] : mw.ldc[3];
+  gemm_q4k_tile<TM, true>(w, qt, amin, dAt, M, mt, nt, C, ldc);
+}
+
 } // namespace
 
 namespace hipq {
@@ -339,6 +376,43 @@ int launch_tiles(const hipq_weight *w, const QActTiled *qa, int M, float *C, int
   } else
     launch_kernel(gemm_q4k_kernel<TM, false>, dim3(grid), dim3(NT), sizeof(Smem<TM>), s, v, (const int8_t *)qa->qt,
                   (const uint16_t *)qa->amin, (const float *)qa->dAt, M, mtiles, ntiles, C, ldc);
+  HIPQ_HIP(hipGetLastError());
+  return HIPQ_OK;
+}
+
+/* count weights (2 to 4) of one K, every one with its tile copy, as one launch */
+int launch_gemm_q4k_multi(int count, const hipq_weight *const *w, const QActTiled *qa, int M, float *const *C,
+                          const int64_t *ldc, hipStream_t s) {
+  if (count < 1 || count > 4) return fail(HIPQ_ERR_INVALID_ARGUMENT, "1 to 4 weights per launch, got %d", count);
+  if ((M + 127) / 128 != qa->mtiles) return fail(HIPQ_ERR_INVALID_ARGUMENT, "tiled activations do not match the matmul shape");
+  MultiQ4K mw;
+  int tiles = 0;
+  for (int i = 0; i < 4; ++i) {
+    const hipq_weight *wi = w[i < count ? i : count - 1];
+    if (i < count) {
+      if (wi->dtype != HIPQ_Q4_K || !wi->gt_base || wi->K != qa->K)
+        return fail(HIPQ_ERR_INVALID_ARGUMENT, "the weights of one launch are Q4_K with a tile copy and share K");
+      tiles += (int)((wi->N + BN - 1) / BN);
+    }
+    mw.w[i] = wview(wi);
+    mw.w[i].qs = wi->gt_qs;
+    mw.w[i].hdr = wi->gt_hdr;
+    mw.C[i] = C[i < count ? i : count - 1];
+    mw.ldc[i] = ldc[i < count ? i : count - 1];
+    mw.tile_end[i] = tiles;
+  }
+  const int64_t rounds64 = (((int64_t)(M + 63) / 64) * tiles + 767) / 768;
+  const int64_t rounds128 = (((int64_t)(M + 127) / 128) * tiles + 511) / 512;
+  const int ngroups = (tiles + 7) / 8;
+  if (rounds128 * 6 < rounds64 * 5) {
+    const int mtiles = (M + 127) / 128;
+    hipLaunchKernelGGL(gemm_q4k_multi_kernel<4>, dim3((unsigned)(mtiles * ngroups * 8)), dim3(NT), sizeof(Smem<4>), s, mw,
+                       (const int8_t *)qa->qt, (const uint16_t *)qa->amin, (const float *)qa->dAt, M, mtiles);
+  } else {
+    const int mtiles = (M + 63) / 64;
+    hipLaunchKernelGGL(gemm_q4k_multi_kernel<2>, dim3((unsigned)(mtiles * ngroups * 8)), dim3(NT), sizeof(Smem<2>), s, mw,
+                       (const int8_t *)qa->qt, (const uint16_t *)qa->amin, (const float *)qa->dAt, M, mtiles);
+  }
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
 }

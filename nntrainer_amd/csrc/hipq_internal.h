@@ -219,6 +219,8 @@ int launch_gemm(const hipq_weight *w, const QAct *qa, int M, float *C,
 int launch_gemm_multi(int count, const hipq_weight *const *w, const QAct *qa, int M, float *const *C,
                       const int64_t *ldc, hipStream_t s);
 /* gemm_q4k.hip: Q4_K with the sub-block scales folded into two int8 digit planes */
+int launch_gemm_q4k_multi(int count, const hipq_weight *const *w, const QActTiled *qa, int M, float *const *C,
+                          const int64_t *ldc, hipStream_t s);
 int launch_gemm_q6k(const hipq_weight *w, const QActTiled *qa, int M, float *C, int64_t ldc, hipStream_t s);
 int launch_gemm_q4k(const hipq_weight *w, const QActTiled *qa, int M, float *C,
                     int64_t ldc, hipStream_t s);

@@ -393,6 +393,30 @@ def test_matmul_multi_mixed_k_formats_prefill(hipq, cr):
         w.destroy()
 
 
+@pytest.mark.parametrize("kind", ["q4_K", "q4_0"])
+def test_matmul_multi_prefill_five_weights_one_launch_per_four(hipq, cr, kind):
+    """Prefill products of several weights go out up to four a launch (column tiles of the weights
+    side by side in one grid): five weights make a launch of four and one of one; widths that are
+    no multiple of the workgroup's column tile; every output equals the single-weight call's."""
+    import gpu_util as gu
+    import torch
+    m, k = 300, 1024
+    ns = [512, 96, 200, 1024, 136]
+    blocks = [_weights(cr, kind, n, k, seed=110 + i) for i, n in enumerate(ns)]
+    ws = [capi.Weight(kind, n, k, b) for n, b in zip(ns, blocks)]
+    a = synth.normal(113, (m, k))
+    outs = [torch.full((m, n), float("nan"), device="cuda") for n in ns]
+    capi.matmul_multi(ws, gu.dev(a), m, outs, stream=gu.stream())
+    torch.cuda.synchronize()
+    for n, b, o, w in zip(ns, blocks, outs, ws):
+        got = o.cpu().numpy()
+        assert not np.isnan(got).any()
+        assert gu.rel_err(got, cr.gemm(cr.oracle(), kind, a, b, n)) <= gu.TOL
+        assert np.array_equal(got, gu.gpu_matmul(w, a)), "the multi-weight call differs from the single one"
+    for w in ws:
+        w.destroy()
+
+
 def test_bad_arguments_are_reported(hipq):
     with pytest.raises(capi.HipqError) as e:
         capi.weight_nbytes("q4_K", 16, 100)  # K not a multiple of 256 (q4_k_tensor.cpp:23-27)
