@@ -614,34 +614,37 @@ __device__ __forceinline__ XLds xlds_carve(unsigned char *base, int TC, int K) {
   return l;
 }
 
-/* Copy the chunk's activation rows (l.rows, already in LDS) from the planes of a.
- * Loads are issued four at a time before their stores so that their latencies overlap. */
+/* Copy the item's nrows activation rows (l.rows, already in LDS) from the planes of a; the
+ * other rows of the matrix operand keep whatever the LDS held: a row of the product depends on
+ * its own activations only, and those rows are not stored. Loads are issued four at a time
+ * before their stores so that their latencies overlap. */
 template <int TC>
-__device__ __forceinline__ void stage_rows(const XLds &l, const QView &a) {
+__device__ __forceinline__ void stage_rows(const XLds &l, const QView &a, int nrows) {
   const int K = a.K, nsb = K >> 8;
   const int cpr = K >> 4; /* 16-byte pieces per row */
   const int nt = blockDim.x;
-  for (int c0 = threadIdx.x; c0 < TC * cpr; c0 += 4 * nt) {
+  const int np = nrows * cpr;
+  for (int c0 = threadIdx.x; c0 < np; c0 += 4 * nt) {
     mv4i v0, v1, v2, v3;
     int d0, d1, d2, d3;
     auto ld = [&](int u, mv4i &v, int &dst) {
-      const int c = min(c0 + u * nt, TC * cpr - 1);
+      const int c = min(c0 + u * nt, np - 1);
       const int r = c / cpr, o = c - r * cpr;
       v = *(const mv4i *)(a.q + (size_t)l.rows[r] * K + o * 16);
       dst = r * (K + 16) + o * 16;
     };
     ld(0, v0, d0), ld(1, v1, d1), ld(2, v2, d2), ld(3, v3, d3);
     *(mv4i *)(l.q + d0) = v0;
-    if (c0 + nt < TC * cpr) *(mv4i *)(l.q + d1) = v1;
-    if (c0 + 2 * nt < TC * cpr) *(mv4i *)(l.q + d2) = v2;
-    if (c0 + 3 * nt < TC * cpr) *(mv4i *)(l.q + d3) = v3;
+    if (c0 + nt < np) *(mv4i *)(l.q + d1) = v1;
+    if (c0 + 2 * nt < np) *(mv4i *)(l.q + d2) = v2;
+    if (c0 + 3 * nt < np) *(mv4i *)(l.q + d3) = v3;
   }
-  for (int c = threadIdx.x; c < TC * nsb * 2; c += nt) {
+  for (int c = threadIdx.x; c < nrows * nsb * 2; c += nt) {
     const int r = c / (nsb * 2), o = c - r * (nsb * 2);
     const mv4i v = *(const mv4i *)((const uint8_t *)a.bsum + ((size_t)l.rows[r] * nsb) * 32 + o * 16);
     *(mv4i *)(l.amin + ((size_t)r * nsb) * 32 + o * 16) = v;
   }
-  for (int c = threadIdx.x; c < TC * nsb; c += nt) {
+  for (int c = threadIdx.x; c < nrows * nsb; c += nt) {
     const int r = c / nsb, b = c - r * nsb;
     l.dA[b * TC + r] = a.d[(size_t)l.rows[r] * nsb + b];
   }
@@ -657,6 +660,7 @@ __device__ __forceinline__ void stage_rows(const XLds &l, const QView &a) {
  * occupies LDS, so the number of resident wavefronts is bounded by registers (four
  * per SIMD for TC = 8) and one launch holds all work items of a prefill chunk. */
 constexpr int XPD = 1; /* super-blocks the loads run ahead of the arithmetic */
+typedef __amdgpu_buffer_rsrc_t xrsrc_t;
 struct XRegs {
   mv4i q[4];
   mv4i hd;
@@ -734,22 +738,24 @@ __device__ __forceinline__ void xr_run(int ntile, const XLds &l, int K, TileOf t
   const int lane = threadIdx.x & 63, i32 = lane & 31, g = lane >> 5;
   const int nsb = K >> 8;
   const int nv = ntile * nsb;
-  const uint8_t *qrow, *hrow;
+  /* the current tile's nibbles and headers as buffer descriptors in scalar registers: a load
+   * names the lane's offset and a scalar offset, so no lane keeps or adds 64-bit addresses */
+  xrsrc_t rq, rh;
   int lt = 0, lsb = 0, issued = 0;
   auto open = [&](int t) {
     WView w;
     int c0;
     tile_of(t, w, c0);
     const int tile = c0 >> 5; /* c0 < N: rows past N are zero padding of the last tile */
-    qrow = w.qs + (size_t)tile * (size_t)(16 * K) + lane * 16;
-    hrow = w.hdr + (size_t)tile * (size_t)(nsb * 512) + i32 * 16;
+    rq = __builtin_amdgcn_make_buffer_rsrc((void *)(w.qs + (size_t)tile * (size_t)(16 * K)), 0, 16 * K, 0x00020000);
+    rh = __builtin_amdgcn_make_buffer_rsrc((void *)(w.hdr + (size_t)tile * (size_t)(nsb * 512)), 0, nsb * 512, 0x00020000);
   };
   open(0);
   auto load = [&](XRegs &r) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      r.q[i] = __builtin_bit_cast(mv4i, hipq_ld_stream((const uint4 *)(qrow + lsb * 4096 + i * 1024)));
-    r.hd = hipq_ld_global((const mv4i *)(hrow + lsb * 512));
+    for (int i = 0; i < 4; ++i) /* non-temporal: every load instruction covers whole cache lines */
+      r.q[i] = __builtin_bit_cast(mv4i, __builtin_amdgcn_raw_buffer_load_b128(rq, lane * 16, lsb * 4096 + i * 1024, 2));
+    r.hd = __builtin_bit_cast(mv4i, __builtin_amdgcn_raw_buffer_load_b128(rh, i32 * 16, lsb * 512, 0));
     if (++issued >= nv) return; /* uniform: the cursor stays on the last super-block */
     if (++lsb == nsb) {
       lsb = 0;
@@ -816,7 +822,7 @@ __global__ __launch_bounds__(256, TC <= 8 ? 4 : TC <= 16 ? 2 : 1) void gate_up_m
   auto stage = [&]() {
     if (threadIdx.x < TC) l.rows[threadIdx.x] = slot_pair[min(s0 + (int)threadIdx.x, end - 1)] / topk;
     __syncthreads();
-    stage_rows<TC>(l, xq);
+    stage_rows<TC>(l, xq, end - s0);
     __syncthreads();
   };
   float gate[NREG], up[NREG];
@@ -909,7 +915,7 @@ __global__ __launch_bounds__(256, TC <= 8 ? 4 : TC <= 16 ? 2 : 1) void down_mma_
     }
     if (threadIdx.x < TC) l.rows[threadIdx.x] = min(s0 + (int)threadIdx.x, end - 1); /* hq rows are slots */
     __syncthreads();
-    stage_rows<TC>(l, hq);
+    stage_rows<TC>(l, hq, end - s0);
     __syncthreads();
   };
   if (ntile <= 0) {
