@@ -24,7 +24,7 @@ HBM_PEAK_GBS = 8000.0    # MI355X HBM3E peak, GB/s
 # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs of this script, scaled by
 # what the same counters read for its 256 MiB device copy (profiles/gemm_q4k_prefill_m512_k4096_n12288.txt,
 # profiles/gemv_q4k_decode_m1_k4096.txt, profiles/moe_block_q4k_64tok_128experts.txt). Measured once, not live: counters need the profiler attached.
-TRAFFIC_GEMM_C2 = 48.23e6 + 25.17e6
+TRAFFIC_GEMM_C2 = 49.00e6 + 25.17e6
 TRAFFIC_GEMV_C2 = 28.45e6 + 0.05e6
 TRAFFIC_GEMV_LM_HEAD = 350.25e6 + 0.62e6
 METRIC = "Q4 GEMV effective GB/s (%HBM peak); prefill GEMM int8 TOPS (%MFMA peak)"
@@ -488,7 +488,8 @@ def main():
                          "achieved": round(2.0 * 512 * 151936 * 4096 / (c3_prefill[0] * 1e-3) / 1e12, 3),
                          "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
                          "frac": round(2.0 * 512 * 151936 * 4096 / (c3_prefill[0] * 1e-3) / 1e12 / INT8_PEAK_TOPS, 5),
-                         "kernel_ms": round(c3_prefill[0], 5), "traffic": None,
+                         "kernel_ms": round(c3_prefill[0], 5), "traffic": 859.6e6 + 325.8e6,
+                         "traffic_from": "profiles/gemm_q6k_prefill_m512_k4096_n151936.txt (counter runs; not live)",
                          "algorithmic_ops_per_launch": 2.0 * 512 * 151936 * 4096}},
         "c5_fc_stack_per_layer": {
             "workload": "the seven Q4_0 FCs of one Qwen3-0.6B-shaped decoder layer (BASELINE configs[4]) through "
@@ -508,7 +509,7 @@ def main():
             "active_experts": active,
             "roofline": {"bound": "hbm", "achieved": round(moe_gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(moe_gbs / HBM_PEAK_GBS, 5), "algorithmic_bytes_per_block": moe_bytes,
-                         "traffic": 238.2e6 + 134.7e6 + 12.0e6},
+                         "traffic": 236.4e6 + 134.2e6 + 12.0e6},
             "decode_token": {"ms_per_block": round(moe_decode_ms, 5),
                              "ms_per_block_in_a_graph": round(moe_decode_graph_ms, 5),
                              "active_experts": decode_active,
