@@ -172,7 +172,10 @@ HIPQ_API int hipq_matmul_noalloc(hipq_weight_t w, const float *A, int64_t M, int
 /** One fp32 activation against several weights sharing K (the QKV layer's
  *  vector dot, float_tensor.cpp:724-798): quantizes A once. One row against up to
  *  four weights of one format (K <= 4096, fewer than 32768 rows together, device
- *  memory) is a single kernel launch for all of them. */
+ *  memory) is a single kernel launch for all of them. With more than 8 rows the Q4_0
+ *  and the Q4_K products go out four weights a launch as well (the column tiles of the
+ *  weights side by side in one grid), after the one quantization. Every output equals
+ *  what hipq_matmul gives for that weight alone, bit for bit. */
 HIPQ_API int hipq_matmul_multi(int count, const hipq_weight_t *w, const float *A,
                                int64_t M, int64_t lda, float *const *C,
                                const int64_t *ldc, int mem, void *stream);
