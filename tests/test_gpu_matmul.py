@@ -107,6 +107,30 @@ def test_q6_K_gemm_matches_oracle(hipq, cr, m, n, k):
     assert (np.abs(got - ref).max(axis=1)[rows] / scale[rows]).max() <= 2e-4
 
 
+def test_gemm_random_shapes_all_formats(hipq, cr):
+    """Prefill products at shapes drawn from a seeded generator: N from 1 upward (narrower than a
+    weight tile, between tile sizes), M between the GEMV limit and a few tiles, K one to five
+    super-blocks. Every kernel's edge handling (padding rows and columns, odd super-block counts,
+    both tile heights) is on some draw; the bar is the one of the fixed shapes."""
+    import gpu_util as gu
+    rng = np.random.RandomState(20240611)
+    for case in range(24):
+        kind = KINDS[case % 3]
+        m = int(rng.choice([9, 17, 31, 64, 65, 127, 130, 257, 300]))
+        n = int(rng.choice([1, 7, 31, 33, 100, 128, 129, 640, 1000, 4100]))
+        k = 256 * int(rng.randint(1, 6))
+        blocks = _weights(cr, kind, n, k, seed=500 + case)
+        a = synth.normal(700 + case, (m, k))
+        ref = cr.gemm(cr.oracle(), kind, a, blocks, n)
+        w = capi.Weight(kind, n, k, blocks)
+        got = gu.gpu_matmul(w, a)
+        w.destroy()
+        assert not np.isnan(got).any(), (kind, m, n, k)
+        assert gu.rel_err(got, ref) <= gu.TOL, (kind, m, n, k, gu.rel_err(got, ref))
+        if kind == "q4_0":
+            assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), (kind, m, n, k)
+
+
 def test_q4_K_gemm_tall_tiles(hipq, cr):
     """A shape for which the Q4_K GEMM picks its 128-row tiles (two rounds of 64-row
     tiles against one of 128-row tiles), with M not a multiple of the tile height."""
