@@ -63,3 +63,33 @@ def test_noalloc_rejects_what_does_not_fit(hipq, cr):
         capi.matmul_noalloc(w, a, m, c)
     assert e.value.code == -4 and "scratch" in str(e.value)
     w.destroy()
+
+
+def test_noalloc_q6_K_prefill_before_the_tile_copy_exists(hipq, cr):
+    """The Q6_K matrix-core product needs the weight's tile copy, which only an allocating call can
+    build: on a fresh weight the allocation-free call walks the rows through the GEMV engine
+    (the reference's bits); once hipq_matmul has built the copy both calls run the same kernel."""
+    import torch
+    import gpu_util as gu
+    n, k, m = 320, 512, 40
+    blocks = cr.quantize_weights(cr.oracle(), "q6_K", synth.normal(77, (n, k), 0.02))
+    w = capi.Weight("q6_K", n, k, blocks)
+    try:
+        a = synth.normal(78, (m, k))
+        da = gu.dev(a)
+        ref = cr.gemm(cr.oracle(), "q6_K", a, blocks, n)
+        first = torch.full((m, n), float("nan"), device="cuda")
+        free_before = torch.cuda.mem_get_info()[0]
+        capi.matmul_noalloc(w, da, m, first, stream=gu.stream())
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free_before
+        assert np.array_equal(first.cpu().numpy().view(np.uint32), ref.view(np.uint32))
+        full = torch.full((m, n), float("nan"), device="cuda")
+        capi.matmul(w, da, m, full, stream=gu.stream())
+        again = torch.full((m, n), float("nan"), device="cuda")
+        capi.matmul_noalloc(w, da, m, again, stream=gu.stream())
+        torch.cuda.synchronize()
+        assert np.array_equal(again.cpu().numpy(), full.cpu().numpy())
+        assert gu.rel_err(full.cpu().numpy(), ref) <= gu.TOL
+    finally:
+        w.destroy()
