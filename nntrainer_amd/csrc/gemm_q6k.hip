@@ -317,9 +317,6 @@ int launch_gemm_q6k(const hipq_weight *w, const QActTiled *qa, int M, float *C, 
    * 64-row tiles (512 tiles of twice the rows against 768 per round); they lose only where
    * there are too few of them to give every CU one. */
   const int64_t tiles128 = ((int64_t)(M + 127) / 128) * ((w->N + BN - 1) / BN);
-#ifdef XP_FORCE_TM
-  return launch_tiles6<XP_FORCE_TM>(w, qa, M, C, ldc, s);
-#endif
   if (M > 64 && tiles128 >= 256) return launch_tiles6<4>(w, qa, M, C, ldc, s);
   return launch_tiles6<2>(w, qa, M, C, ldc, s);
 }
