@@ -26,6 +26,7 @@ SYMBOLS = [
 ]
 # measurement helpers of csrc/hipq_bench.h: exported for bench.py, not part of the product ABI
 BENCH_SYMBOLS = ["hipq_time_matmul", "hipq_bench_matmul_steps", "hipq_bench_mfma_ceiling",
+                 "hipq_bench_hbm_read_ceiling",
                  "hipq_bench_tiled_bytes", "hipq_bench_quantize_tiled"]
 
 
@@ -107,6 +108,7 @@ def lib():
         fp = C.POINTER(C.c_float)
         L.hipq_bench_matmul_steps.argtypes = [i32, C.POINTER(vp), vp, i64, i64, vp, i64, i32, vp, fp, fp, fp]
         L.hipq_bench_mfma_ceiling.argtypes = [C.c_float, vp, fp, fp]
+        L.hipq_bench_hbm_read_ceiling.argtypes = [i64, i32, vp, fp]
         L.hipq_bench_tiled_bytes.argtypes = [i64, i64]
         L.hipq_bench_tiled_bytes.restype = i64
         L.hipq_bench_quantize_tiled.argtypes = [vp, i64, i64, i64, vp, vp]
@@ -323,6 +325,13 @@ def bench_tiled_bytes(m, k):
 def bench_quantize_tiled(a, m, k, out, lda=None, stream=None):
     """The tiled Q8_K form of device rows `a` into the device buffer `out` (bench_tiled_bytes)."""
     check(lib().hipq_bench_quantize_tiled(_addr(a), m, k, lda if lda is not None else k, _addr(out), stream))
+
+
+def bench_hbm_read_ceiling(nbytes=1 << 30, waves_per_simd=4, stream=None):
+    """TB/s of a kernel that only reads `nbytes` of device memory (the GEMV kernels' access pattern)."""
+    tbs = C.c_float()
+    check(lib().hipq_bench_hbm_read_ceiling(nbytes, waves_per_simd, stream, C.byref(tbs)))
+    return tbs.value
 
 
 def bench_mfma_ceiling(target_ms=2.0, stream=None):

@@ -1,8 +1,9 @@
 // SPDX-License-Identifier: Apache-2.0
 /**
  * @file   bench_kernels.hip
- * @brief  The matrix-core ceiling kernel of hipq_bench.h: what the int8 matrix
- *         instruction sustains on this device when nothing else is issued.
+ * @brief  The ceiling kernels of hipq_bench.h: what the int8 matrix instruction
+ *         sustains on this device when nothing else is issued, and what a kernel
+ *         that does nothing but read device memory gets out of it.
  */
 #include "hipq_bench.h"
 #include "hipq_internal.h"
@@ -32,7 +33,77 @@ __global__ __launch_bounds__(256) void mfma_ceiling_kernel(int iters, int *sink,
   }
 }
 
+typedef unsigned int u4 __attribute__((ext_vector_type(4)));
+
+/* Every wavefront walks its own contiguous share of the buffer in steps of DEPTH KB, DEPTH
+ * non-temporal 128-bit loads a lane in flight (each load instruction covers 1 KB of consecutive
+ * memory), the way the GEMV kernels stream a weight. */
+template <int DEPTH>
+__global__ __launch_bounds__(256) void hbm_read_ceiling_kernel(const unsigned char *p, long long kb_per_wave,
+                                                               unsigned *sink) {
+  const int lane = threadIdx.x & 63;
+  const long long wave = (long long)blockIdx.x * 4 + (threadIdx.x >> 6);
+  __amdgpu_buffer_rsrc_t r =
+    __builtin_amdgcn_make_buffer_rsrc((void *)(p + wave * kb_per_wave * 1024), 0, (int)(kb_per_wave * 1024), 0x00020000);
+  u4 acc = {0, 0, 0, 0};
+  for (long long k = 0; k + DEPTH <= kb_per_wave; k += DEPTH) {
+    u4 v[DEPTH];
+#pragma unroll
+    for (int i = 0; i < DEPTH; ++i) v[i] = __builtin_amdgcn_raw_buffer_load_b128(r, lane * 16, (int)(k + i) * 1024, 2);
+#pragma unroll
+    for (int i = 0; i < DEPTH; ++i) acc ^= v[i];
+  }
+  const unsigned x = acc[0] ^ acc[1] ^ acc[2] ^ acc[3];
+  if (x == 0x12345678u) sink[threadIdx.x] = x; /* keeps the loads alive; the buffer holds zeros */
+}
+
 } // namespace
+
+extern "C" int hipq_bench_hbm_read_ceiling(int64_t bytes, int waves_per_simd, void *stream, float *tbs) {
+  using hipq::fail;
+  if (!tbs || bytes < (int64_t)1 << 20 || bytes > (int64_t)1 << 36 || waves_per_simd < 1 || waves_per_simd > 8)
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "bad read ceiling arguments");
+  hipStream_t s = (hipStream_t)stream;
+  int dev = 0, cus = 0;
+  HIPQ_HIP(hipGetDevice(&dev));
+  HIPQ_HIP(hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev));
+  constexpr int DEPTH = 8;
+  const int wg = cus * waves_per_simd; /* four wavefronts a workgroup: one per SIMD */
+  const long long waves = (long long)wg * 4;
+  long long kb_per_wave = bytes / 1024 / waves / DEPTH * DEPTH;
+  if (kb_per_wave < DEPTH) kb_per_wave = DEPTH;
+  if (kb_per_wave * 1024 > 0x7fffffffLL) return fail(HIPQ_ERR_INVALID_ARGUMENT, "a wavefront's share exceeds 2 GiB");
+  const size_t total = (size_t)(kb_per_wave * 1024 * waves);
+  unsigned char *buf = nullptr;
+  unsigned *sink = nullptr;
+  HIPQ_HIP(hipMalloc((void **)&buf, total));
+  hipError_t e = hipMalloc((void **)&sink, 256 * sizeof(unsigned));
+  if (e == hipSuccess) e = hipMemsetAsync(buf, 0, total, s);
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  if (e == hipSuccess) e = hipEventCreate(&e0);
+  if (e == hipSuccess) e = hipEventCreate(&e1);
+  float best = 0.f;
+  for (int pass = 0; pass < 4 && e == hipSuccess; ++pass) { /* the first pass warms up; the best of the rest counts */
+    float ms = 0.f;
+    e = hipEventRecord(e0, s);
+    hipLaunchKernelGGL(hbm_read_ceiling_kernel<DEPTH>, dim3(wg), dim3(256), 0, s, buf, kb_per_wave, sink);
+    if (e == hipSuccess) e = hipGetLastError();
+    if (e == hipSuccess) e = hipEventRecord(e1, s);
+    if (e == hipSuccess) e = hipEventSynchronize(e1);
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+    if (e == hipSuccess && pass > 0 && ms > 0.f) {
+      const float r = (float)((double)total / (ms * 1e-3) / 1e12);
+      if (r > best) best = r;
+    }
+  }
+  if (e0) (void)hipEventDestroy(e0);
+  if (e1) (void)hipEventDestroy(e1);
+  if (sink) (void)hipFree(sink);
+  (void)hipFree(buf);
+  if (e != hipSuccess) return fail(HIPQ_ERR_RUNTIME, "read ceiling kernel: %s", hipGetErrorString(e));
+  *tbs = best;
+  return HIPQ_OK;
+}
 
 extern "C" int hipq_bench_mfma_ceiling(float target_ms, void *stream, float *tops, float *ghz) {
   using hipq::fail;

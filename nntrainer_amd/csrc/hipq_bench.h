@@ -4,7 +4,8 @@
  * @brief  Measurement and test helpers exported by libhipq.so for bench.py and the GPU
  *         tests only. They are not part of the product's C ABI (include/hipq.h) and
  *         replace nothing in the reference: event-timed launch loops, a matrix-core
- *         ceiling kernel, and a view of an internal buffer layout for its parity test.
+ *         and a memory-read ceiling kernel, and a view of an internal buffer layout for
+ *         its parity test.
  */
 #ifndef HIPQ_BENCH_H
 #define HIPQ_BENCH_H
@@ -40,6 +41,13 @@ HIPQ_API int hipq_bench_matmul_steps(int n_weights, const hipq_weight_t *w, cons
  *  four independent accumulators) for about `target_ms`: the int8 rate the matrix cores
  *  sustain here, in TOP/s, and the shader clock during the run in GHz. */
 HIPQ_API int hipq_bench_mfma_ceiling(float target_ms, void *stream, float *tops, float *ghz);
+
+/** A kernel that does nothing but read `bytes` of device memory (allocated, zeroed and freed
+ *  by this call; 1 GiB is four times the last-level cache) with `waves_per_simd` wavefronts on
+ *  every SIMD, each streaming its own contiguous share with eight non-temporal 128-bit loads a
+ *  lane in flight: the read rate in TB/s, best of three launches, that the memory system gives a
+ *  kernel of the GEMV kernels' access pattern. */
+HIPQ_API int hipq_bench_hbm_read_ceiling(int64_t bytes, int waves_per_simd, void *stream, float *tbs);
 
 /** The Q8_K activation quantizer in the form the Q4_K prefill product reads (rows tiled by
  *  128, 16-byte matrix operands; csrc/hipq_internal.h, QActTiled), written into ONE device

@@ -42,11 +42,14 @@
 /* The total size equals the packed ggml size; nothing is expanded in HBM.    */
 /*                                                                             */
 /* Q4_K expert weights of a mixture-of-experts block that runs on the matrix   */
-/* cores are re-laid out once more, by tiles of 32 rows (rows padded to 32):    */
-/*   qs  [N/32][K/256][4][64][16 B]: for load i of lane (n, g) the two 8-byte    */
-/*       halves g of sub-blocks 2i and 2i+1 of row n -- the 16 bytes the lane    */
-/*       feeds into two matrix steps, consecutive lanes consecutive in memory    */
-/*   hdr [N/32][K/256][32][16 B]                                                */
+/* cores are re-laid out once more, by tiles of 32 rows (rows padded to 32),   */
+/* 4608 bytes per tile and super-block, [N/32][K/256]{qs, hdr}:                */
+/*   qs  [4][64][16 B]: for load i of lane (n, g) the two 8-byte halves g of    */
+/*       sub-blocks 2i and 2i+1 of row n -- the 16 bytes the lane feeds into    */
+/*       two matrix steps, consecutive lanes consecutive in memory              */
+/*   hdr [32][16 B]: the headers of the tile's rows, right behind their nibbles */
+/*       (a wavefront's stream over a tile is one run of consecutive memory;    */
+/*       hipq_weight.hdr points at the first header, 4096 bytes behind qs)      */
 /* Such a weight serves the expert kernels only.                               */
 /* ------------------------------------------------------------------------- */
 struct hipq_weight {
@@ -259,6 +262,7 @@ int launch_quantize_weights(int dtype, const float *W, int64_t N, int64_t K,
                             void *out_blocks, hipStream_t s);
 
 /* relayout.hip ------------------------------------------------------------ */
+constexpr int EXPERT_TILE_BYTES = 4096 + 512; /* nibbles, then headers, of 32 rows and one super-block */
 int tile_expert_weight(hipq_weight *w); /* planes -> 32-row tiles, in a new allocation; synchronous */
 int ensure_gemm_tiles(hipq_weight *w);  /* adds the prefill GEMM's tile copy (allocates once; synchronous) */
 int launch_relayout(hipq_weight *w, int layout, const uint8_t *src_dev,

@@ -652,10 +652,11 @@ __device__ __forceinline__ void stage_rows(const XLds &l, const QView &a, int nr
 
 /* The weight stream. The experts' weights are stored by tiles of 32 rows: per tile
  * and super-block four 1 KB groups, group i holding for lane (n, g) the halves g
- * (weights 16g .. 16g+15) of sub-blocks 2i and 2i+1 of row n, then the 32 headers.
- * A wavefront's 128-bit load i therefore reads 1 KB of consecutive memory (whole
- * cache lines, marked non-temporal) and every lane receives exactly the bytes of its
- * two matrix steps. The loads of the next super-block are in flight during the
+ * (weights 16g .. 16g+15) of sub-blocks 2i and 2i+1 of row n, then the 32 headers
+ * (512 bytes), the super-blocks of a tile one behind the other. A wavefront's 128-bit
+ * load i therefore reads 1 KB of consecutive memory (whole cache lines, marked
+ * non-temporal), its stream over a tile is one run of consecutive memory, and every
+ * lane receives exactly the bytes of its two matrix steps. The loads of the next super-block are in flight during the
  * arithmetic of the current one, also across tiles; nothing but the activations
  * occupies LDS, so the number of resident wavefronts is bounded by registers (four
  * per SIMD for TC = 8) and one launch holds all work items of a prefill chunk. */
@@ -738,24 +739,27 @@ __device__ __forceinline__ void xr_run(int ntile, const XLds &l, int K, TileOf t
   const int lane = threadIdx.x & 63, i32 = lane & 31, g = lane >> 5;
   const int nsb = K >> 8;
   const int nv = ntile * nsb;
-  /* the current tile's nibbles and headers as buffer descriptors in scalar registers: a load
-   * names the lane's offset and a scalar offset, so no lane keeps or adds 64-bit addresses */
-  xrsrc_t rq, rh;
+  /* the current tile (nibbles and headers of its super-blocks, EXPERT_TILE_BYTES each) as a
+   * buffer descriptor in scalar registers: a load names the lane's offset and a scalar offset,
+   * so no lane keeps or adds 64-bit addresses */
+  xrsrc_t rq;
   int lt = 0, lsb = 0, issued = 0;
   auto open = [&](int t) {
     WView w;
     int c0;
     tile_of(t, w, c0);
     const int tile = c0 >> 5; /* c0 < N: rows past N are zero padding of the last tile */
-    rq = __builtin_amdgcn_make_buffer_rsrc((void *)(w.qs + (size_t)tile * (size_t)(16 * K)), 0, 16 * K, 0x00020000);
-    rh = __builtin_amdgcn_make_buffer_rsrc((void *)(w.hdr + (size_t)tile * (size_t)(nsb * 512)), 0, nsb * 512, 0x00020000);
+    rq = __builtin_amdgcn_make_buffer_rsrc((void *)(w.qs + (size_t)tile * (size_t)(nsb * hipq::EXPERT_TILE_BYTES)), 0,
+                                           nsb * hipq::EXPERT_TILE_BYTES, 0x00020000);
   };
   open(0);
   auto load = [&](XRegs &r) {
 #pragma unroll
     for (int i = 0; i < 4; ++i) /* non-temporal: every load instruction covers whole cache lines */
-      r.q[i] = __builtin_bit_cast(mv4i, __builtin_amdgcn_raw_buffer_load_b128(rq, lane * 16, lsb * 4096 + i * 1024, 2));
-    r.hd = __builtin_bit_cast(mv4i, __builtin_amdgcn_raw_buffer_load_b128(rh, i32 * 16, lsb * 512, 0));
+      r.q[i] = __builtin_bit_cast(
+        mv4i, __builtin_amdgcn_raw_buffer_load_b128(rq, lane * 16, lsb * hipq::EXPERT_TILE_BYTES + i * 1024, 2));
+    r.hd = __builtin_bit_cast(
+      mv4i, __builtin_amdgcn_raw_buffer_load_b128(rq, 4096 + i32 * 16, lsb * hipq::EXPERT_TILE_BYTES, 2));
     if (++issued >= nv) return; /* uniform: the cursor stays on the last super-block */
     if (++lsb == nsb) {
       lsb = 0;
@@ -818,7 +822,7 @@ __global__ __launch_bounds__(256, TC <= 8 ? 4 : TC <= 16 ? 2 : 1) void gate_up_m
   float *xch = (float *)(xmoe_lds + xlds_bytes(TC, K)); /* PAIRED: [2 tiles][NREG][64 lanes] */
   const int col0 = PAIRED ? (blockIdx.x * 2 + (wave & 1)) * 32 : (blockIdx.x * 4 + wave) * 32;
   const int first = PAIRED ? wave >> 1 : 0; /* 0: gate, 1: up */
-  const uint64_t dqs = (uint64_t)wu.qs - (uint64_t)wg.qs, dhdr = (uint64_t)wu.hdr - (uint64_t)wg.hdr;
+  const uint64_t dqs = (uint64_t)wu.qs - (uint64_t)wg.qs;
   auto stage = [&]() {
     if (threadIdx.x < TC) l.rows[threadIdx.x] = slot_pair[min(s0 + (int)threadIdx.x, end - 1)] / topk;
     __syncthreads();
@@ -844,7 +848,7 @@ __global__ __launch_bounds__(256, TC <= 8 ? 4 : TC <= 16 ? 2 : 1) void gate_up_m
     [&](int t, WView &w, int &c0) {
       const uint64_t isup = (uint64_t)0 - (uint64_t)((t + first) & 1);
       w.qs = (const uint8_t *)((uint64_t)wg.qs + (isup & dqs));
-      w.hdr = (const uint8_t *)((uint64_t)wg.hdr + (isup & dhdr));
+      w.hdr = nullptr; /* the headers follow the nibbles */
       w.N = wg.N;
       w.K = wg.K;
       c0 = col0;

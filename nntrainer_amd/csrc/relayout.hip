@@ -126,9 +126,10 @@ __global__ void relayout_q6_K(const uint8_t *__restrict__ src, int64_t total,
   d[i] = (uint16_t)(blk[208] | (blk[209] << 8));
 }
 
-/* planes -> tiles of 32 rows for the expert kernels: thread = one 16-byte piece */
+/* planes -> tiles of 32 rows for the expert kernels (4096 bytes of nibbles, then the 512 bytes of
+ * headers, per tile and super-block): thread = one 16-byte piece of nibbles */
 __global__ void tile_q4_K(const uint8_t *__restrict__ qs, const uint8_t *__restrict__ hdr, int N, int nsb,
-                          int64_t pieces, uint8_t *__restrict__ tq, uint8_t *__restrict__ th) {
+                          int64_t pieces, uint8_t *__restrict__ tq) {
   const int64_t p = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (p >= pieces) return;
   const int lane = (int)(p & 63), i = (int)((p >> 6) & 3);
@@ -143,9 +144,10 @@ __global__ void tile_q4_K(const uint8_t *__restrict__ qs, const uint8_t *__restr
     a = *(const uint2 *)(src + (2 * i) * 16);
     b = *(const uint2 *)(src + (2 * i + 1) * 16);
   }
-  *(uint4 *)(tq + p * 16) = make_uint4(a.x, a.y, b.x, b.y);
+  uint8_t *dst = tq + ts * hipq::EXPERT_TILE_BYTES;
+  *(uint4 *)(dst + (p & 255) * 16) = make_uint4(a.x, a.y, b.x, b.y);
   if (i == 0 && g == 0)
-    *(uint4 *)(th + (ts * 32 + (lane & 31)) * 16) =
+    *(uint4 *)(dst + 4096 + (lane & 31) * 16) =
       n < N ? *(const uint4 *)(hdr + (n * nsb + sb) * 16) : make_uint4(0, 0, 0, 0);
 }
 
@@ -269,14 +271,13 @@ int tile_expert_weight(hipq_weight *w) {
   if (w->expert_tiles) return HIPQ_OK;
   const int nsb = (int)(w->K / 256);
   const int64_t tiles = (w->N + 31) / 32;
-  const size_t q_bytes = (size_t)tiles * nsb * 4096, h_bytes = (size_t)tiles * nsb * 512;
-  const size_t o_hdr = (q_bytes + 255) & ~(size_t)255;
+  const size_t bytes = (size_t)tiles * nsb * EXPERT_TILE_BYTES;
   uint8_t *nb = nullptr;
-  hipError_t e = hipMalloc((void **)&nb, o_hdr + h_bytes);
-  if (e != hipSuccess) return fail(HIPQ_ERR_OUT_OF_MEMORY, "expert tiles of %zu bytes: %s", o_hdr + h_bytes, hipGetErrorString(e));
+  hipError_t e = hipMalloc((void **)&nb, bytes);
+  if (e != hipSuccess) return fail(HIPQ_ERR_OUT_OF_MEMORY, "expert tiles of %zu bytes: %s", bytes, hipGetErrorString(e));
   const int64_t pieces = tiles * nsb * 256;
   hipLaunchKernelGGL(tile_q4_K, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, nullptr, w->qs, w->hdr,
-                     (int)w->N, nsb, pieces, nb, nb + o_hdr);
+                     (int)w->N, nsb, pieces, nb);
   e = hipGetLastError();
   if (e == hipSuccess) e = hipDeviceSynchronize(); /* nothing may still read the planes that are freed next */
   if (e != hipSuccess) {
@@ -285,9 +286,9 @@ int tile_expert_weight(hipq_weight *w) {
   }
   (void)hipFree(w->base);
   w->base = nb;
-  w->bytes = o_hdr + h_bytes;
+  w->bytes = bytes;
   w->qs = nb;
-  w->hdr = nb + o_hdr;
+  w->hdr = nb + 4096;
   w->expert_tiles = 1;
   return HIPQ_OK;
 }
