@@ -108,7 +108,7 @@ def lib():
         fp = C.POINTER(C.c_float)
         L.hipq_bench_matmul_steps.argtypes = [i32, C.POINTER(vp), vp, i64, i64, vp, i64, i32, vp, fp, fp, fp]
         L.hipq_bench_mfma_ceiling.argtypes = [C.c_float, vp, fp, fp]
-        L.hipq_bench_hbm_read_ceiling.argtypes = [i64, i32, vp, fp]
+        L.hipq_bench_hbm_read_ceiling.argtypes = [i64, i32, i32, vp, fp]
         L.hipq_bench_tiled_bytes.argtypes = [i64, i64]
         L.hipq_bench_tiled_bytes.restype = i64
         L.hipq_bench_quantize_tiled.argtypes = [vp, i64, i64, i64, vp, vp]
@@ -327,10 +327,11 @@ def bench_quantize_tiled(a, m, k, out, lda=None, stream=None):
     check(lib().hipq_bench_quantize_tiled(_addr(a), m, k, lda if lda is not None else k, _addr(out), stream))
 
 
-def bench_hbm_read_ceiling(nbytes=1 << 30, waves_per_simd=4, stream=None):
-    """TB/s of a kernel that only reads `nbytes` of device memory (the GEMV kernels' access pattern)."""
+def bench_hbm_read_ceiling(nbytes=1 << 30, waves_per_simd=4, regions=1, stream=None):
+    """TB/s of a kernel that only reads `nbytes` of device memory (the GEMV kernels' access pattern);
+    regions > 1: that many buffers, one per launch, back to back, each read cold."""
     tbs = C.c_float()
-    check(lib().hipq_bench_hbm_read_ceiling(nbytes, waves_per_simd, stream, C.byref(tbs)))
+    check(lib().hipq_bench_hbm_read_ceiling(nbytes, regions, waves_per_simd, stream, C.byref(tbs)))
     return tbs.value
 
 

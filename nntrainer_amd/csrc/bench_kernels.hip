@@ -59,9 +59,10 @@ __global__ __launch_bounds__(256) void hbm_read_ceiling_kernel(const unsigned ch
 
 } // namespace
 
-extern "C" int hipq_bench_hbm_read_ceiling(int64_t bytes, int waves_per_simd, void *stream, float *tbs) {
+extern "C" int hipq_bench_hbm_read_ceiling(int64_t bytes, int regions, int waves_per_simd, void *stream, float *tbs) {
   using hipq::fail;
-  if (!tbs || bytes < (int64_t)1 << 20 || bytes > (int64_t)1 << 36 || waves_per_simd < 1 || waves_per_simd > 8)
+  if (!tbs || bytes < (int64_t)1 << 20 || bytes > (int64_t)1 << 33 || regions < 1 || regions > 64 ||
+      bytes * regions > (int64_t)1 << 35 || waves_per_simd < 1 || waves_per_simd > 8)
     return fail(HIPQ_ERR_INVALID_ARGUMENT, "bad read ceiling arguments");
   hipStream_t s = (hipStream_t)stream;
   int dev = 0, cus = 0;
@@ -73,27 +74,46 @@ extern "C" int hipq_bench_hbm_read_ceiling(int64_t bytes, int waves_per_simd, vo
   long long kb_per_wave = bytes / 1024 / waves / DEPTH * DEPTH;
   if (kb_per_wave < DEPTH) kb_per_wave = DEPTH;
   if (kb_per_wave * 1024 > 0x7fffffffLL) return fail(HIPQ_ERR_INVALID_ARGUMENT, "a wavefront's share exceeds 2 GiB");
-  const size_t total = (size_t)(kb_per_wave * 1024 * waves);
+  const size_t total = (size_t)(kb_per_wave * 1024 * waves); /* one region */
   unsigned char *buf = nullptr;
   unsigned *sink = nullptr;
-  HIPQ_HIP(hipMalloc((void **)&buf, total));
+  HIPQ_HIP(hipMalloc((void **)&buf, total * regions));
   hipError_t e = hipMalloc((void **)&sink, 256 * sizeof(unsigned));
-  if (e == hipSuccess) e = hipMemsetAsync(buf, 0, total, s);
+  if (e == hipSuccess) e = hipMemsetAsync(buf, 0, total * regions, s);
   hipEvent_t e0 = nullptr, e1 = nullptr;
   if (e == hipSuccess) e = hipEventCreate(&e0);
   if (e == hipSuccess) e = hipEventCreate(&e1);
+  /* One region: the first launch warms up and the best of three more counts. Several regions
+   * (together larger than the last-level cache): one round over all of them warms up, and the
+   * launches of a second round, each on memory last touched a whole round ago, are timed as one
+   * run of back-to-back launches. */
   float best = 0.f;
-  for (int pass = 0; pass < 4 && e == hipSuccess; ++pass) { /* the first pass warms up; the best of the rest counts */
-    float ms = 0.f;
-    e = hipEventRecord(e0, s);
-    hipLaunchKernelGGL(hbm_read_ceiling_kernel<DEPTH>, dim3(wg), dim3(256), 0, s, buf, kb_per_wave, sink);
-    if (e == hipSuccess) e = hipGetLastError();
-    if (e == hipSuccess) e = hipEventRecord(e1, s);
-    if (e == hipSuccess) e = hipEventSynchronize(e1);
-    if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
-    if (e == hipSuccess && pass > 0 && ms > 0.f) {
-      const float r = (float)((double)total / (ms * 1e-3) / 1e12);
-      if (r > best) best = r;
+  if (regions == 1) {
+    for (int pass = 0; pass < 4 && e == hipSuccess; ++pass) {
+      float ms = 0.f;
+      e = hipEventRecord(e0, s);
+      hipLaunchKernelGGL(hbm_read_ceiling_kernel<DEPTH>, dim3(wg), dim3(256), 0, s, buf, kb_per_wave, sink);
+      if (e == hipSuccess) e = hipGetLastError();
+      if (e == hipSuccess) e = hipEventRecord(e1, s);
+      if (e == hipSuccess) e = hipEventSynchronize(e1);
+      if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+      if (e == hipSuccess && pass > 0 && ms > 0.f) {
+        const float r = (float)((double)total / (ms * 1e-3) / 1e12);
+        if (r > best) best = r;
+      }
+    }
+  } else {
+    for (int round = 0; round < 2 && e == hipSuccess; ++round) {
+      float ms = 0.f;
+      e = hipEventRecord(e0, s);
+      for (int g = 0; g < regions; ++g)
+        hipLaunchKernelGGL(hbm_read_ceiling_kernel<DEPTH>, dim3(wg), dim3(256), 0, s, buf + (size_t)g * total,
+                           kb_per_wave, sink);
+      if (e == hipSuccess) e = hipGetLastError();
+      if (e == hipSuccess) e = hipEventRecord(e1, s);
+      if (e == hipSuccess) e = hipEventSynchronize(e1);
+      if (e == hipSuccess) e = hipEventElapsedTime(&ms, e0, e1);
+      if (e == hipSuccess && round == 1 && ms > 0.f) best = (float)((double)total * regions / (ms * 1e-3) / 1e12);
     }
   }
   if (e0) (void)hipEventDestroy(e0);

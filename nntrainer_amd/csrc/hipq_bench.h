@@ -45,9 +45,11 @@ HIPQ_API int hipq_bench_mfma_ceiling(float target_ms, void *stream, float *tops,
 /** A kernel that does nothing but read `bytes` of device memory (allocated, zeroed and freed
  *  by this call; 1 GiB is four times the last-level cache) with `waves_per_simd` wavefronts on
  *  every SIMD, each streaming its own contiguous share with eight non-temporal 128-bit loads a
- *  lane in flight: the read rate in TB/s, best of three launches, that the memory system gives a
- *  kernel of the GEMV kernels' access pattern. */
-HIPQ_API int hipq_bench_hbm_read_ceiling(int64_t bytes, int waves_per_simd, void *stream, float *tbs);
+ *  lane in flight: the read rate in TB/s that the memory system gives a kernel of the GEMV
+ *  kernels' access pattern. regions == 1: best of three launches. regions > 1: that many
+ *  buffers of `bytes` each, read one per launch in a run of back-to-back launches, every
+ *  buffer last touched a whole round earlier (a small weight read cold, launch included). */
+HIPQ_API int hipq_bench_hbm_read_ceiling(int64_t bytes, int regions, int waves_per_simd, void *stream, float *tbs);
 
 /** The Q8_K activation quantizer in the form the Q4_K prefill product reads (rows tiled by
  *  128, 16-byte matrix operands; csrc/hipq_internal.h, QActTiled), written into ONE device
