@@ -56,6 +56,24 @@ def test_small_m_matches_oracle(hipq, cr, kind, m):
 
 
 @pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("m,n,k", [(1, 8200, 12288), (3, 200, 8192), (8, 520, 9216), (1, 96, 20480),
+                                   (5, 64, 4352)])
+def test_rows_longer_than_one_chunk_match_oracle(hipq, cr, kind, m, n, k):
+    """K above 4096 runs the GEMV instance that keeps the next chunk's weights in flight while
+    the current chunk is computed: two, three and five chunks, a last chunk of 256, every group
+    size the row count selects, one to eight activation rows. Same bits as the reference."""
+    import gpu_util as gu
+    blocks = _weights(cr, kind, n, k, seed=900 + n)
+    a = synth.normal(901 + k + m, (m, k))
+    ref = cr.gemm(cr.oracle(), kind, a, blocks, n)
+    w = capi.Weight(kind, n, k, blocks)
+    got = gu.gpu_matmul(w, a)
+    w.destroy()
+    assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), \
+        "%d of %d outputs differ in bits" % ((got.view(np.uint32) != ref.view(np.uint32)).sum(), got.size)
+
+
+@pytest.mark.parametrize("kind", KINDS)
 @pytest.mark.parametrize("m,n,k", [(16, 256, 256), (64, 512, 1024), (130, 384, 512), (457, 512, 512),
                                    (459, 512, 512), (512, 1024, 2048)])
 def test_gemm_matches_oracle(hipq, cr, kind, m, n, k):
