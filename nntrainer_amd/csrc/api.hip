@@ -384,10 +384,32 @@ int matmul_tiled(const hipq_weight *w, const float *A, int64_t M, int64_t lda, f
   return hipq::launch_gemm_q4k(w, &qa, (int)M, C, ldc, s);
 }
 
+/* Three to eight rows of a large Q4_K matrix run on the matrix cores (gemm_rows_q4k.hip, the
+ * reference's bits as the GEMV engine's) off the weight's tile copy; the entry point that may not
+ * allocate takes that path only once the copy exists.
+ * phase: 0 quantizer + product, 1 product only, 2 quantizer only */
+bool wants_rows(const hipq_weight *w, int64_t M, bool may_allocate) {
+  return hipq::gemm_rows_q4k_fits(w, M) && (w->gt_base || may_allocate);
+}
+
+int matmul_rows(const hipq_weight *w, const float *A, int64_t M, int64_t lda, float *C, int64_t ldc,
+                hipStream_t s, int phase, const Scratch &sc) {
+  void *mem = nullptr;
+  int rc = sc.get(qact_bytes(1, M, w->K), &mem);
+  if (rc) return rc;
+  QAct qa = qact_carve(1, mem, M, w->K);
+  const int64_t mat_rows = (M / 4) * 4; /* the rows the reference quantizes four at a time */
+  if (phase != 1) rc = hipq::launch_quantize_q8_K_rowmma(A, M, w->K, lda, &qa, s, mat_rows);
+  if (rc || phase == 2) return rc;
+  if (!w->gt_base && (rc = hipq::ensure_gemm_tiles(const_cast<hipq_weight *>(w)))) return rc;
+  return hipq::launch_gemm_rows_q4k(w, &qa, (int)M, (int)mat_rows, C, ldc, s);
+}
+
 int matmul_device(hipq_weight_t w, const float *A, int64_t M, int64_t lda, float *C, int64_t ldc,
                   hipStream_t s, const Scratch &sc) {
   if (M == 0) return HIPQ_OK;
   if (wants_tiled(w, M, !sc.fixed)) return matmul_tiled(w, A, M, lda, C, ldc, s, 0, sc);
+  if (wants_rows(w, M, !sc.fixed)) return matmul_rows(w, A, M, lda, C, ldc, s, 0, sc);
   if (M == 1 && hipq::gemv_fuses_quantizer(w, A)) return hipq::launch_gemv_fused(w, A, C, s);
   const int is_k = w->dtype != HIPQ_Q4_0;
   void *mem = nullptr;
@@ -971,12 +993,19 @@ int hipq_time_matmul(int n_weights, const hipq_weight_t *w, const float *A, int6
   hipStream_t s = (hipStream_t)stream;
   EnqueueGuard eg(enqueue_lock(s));
   const int is_k = w[0]->dtype != HIPQ_Q4_0;
-  bool tiled = true;
-  for (int i = 0; i < n_weights; ++i) tiled = tiled && wants_tiled(w[i], M);
+  bool tiled = true, rows = true;
+  for (int i = 0; i < n_weights; ++i) {
+    tiled = tiled && wants_tiled(w[i], M);
+    rows = rows && wants_rows(w[i], M, true);
+  }
   void *memp = nullptr;
   QAct qa{};
   if (tiled) {
     if ((rc = matmul_tiled(w[0], A, M, lda, C, ldc, s, 2, Scratch{false, s}))) return rc;
+  } else if (rows) {
+    for (int i = 0; i < n_weights; ++i) /* the tile copies are built outside the timed loop */
+      if (!w[i]->gt_base && (rc = hipq::ensure_gemm_tiles(const_cast<hipq_weight *>(w[i])))) return rc;
+    if ((rc = matmul_rows(w[0], A, M, lda, C, ldc, s, 2, Scratch{false, s}))) return rc;
   } else {
     if ((rc = workspace(s, qact_bytes(is_k, M, w[0]->K), &memp))) return rc;
     qa = qact_carve(is_k, memp, M, w[0]->K);
@@ -991,6 +1020,10 @@ int hipq_time_matmul(int n_weights, const hipq_weight_t *w, const float *A, int6
     const hipq_weight *wi = w[it % n_weights];
     if (tiled) {
       rc = matmul_tiled(wi, A, M, lda, C, ldc, s, phase, Scratch{false, s});
+      continue;
+    }
+    if (rows) {
+      rc = matmul_rows(wi, A, M, lda, C, ldc, s, phase, Scratch{false, s});
       continue;
     }
     if (phase == 0 && M == 1 && hipq::gemv_fuses_quantizer(wi, A)) {

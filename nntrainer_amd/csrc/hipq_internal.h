@@ -191,7 +191,7 @@ int launch_quantize_q8_K(const float *A, int64_t M, int64_t K, int64_t lda,
  * the eight sub-block sums split into a part in 0..63 (first 8) and a multiple
  * of 64 (last 8). ql / qh are not written. */
 int launch_quantize_q8_K_rowmma(const float *A, int64_t M, int64_t K, int64_t lda, const QAct *qa,
-                                hipStream_t s);
+                                hipStream_t s, int64_t mat_rows = 0);
 /* the values of launch_quantize_q8_K, written in the tiled form; rows M .. 128 * mtiles
  * are zero-filled */
 int launch_quantize_q8_K_tiled(const float *A, int64_t M, int64_t K, int64_t lda,
@@ -227,6 +227,11 @@ int launch_gemm_q4k_multi(int count, const hipq_weight *const *w, const QActTile
 int launch_gemm_q6k(const hipq_weight *w, const QActTiled *qa, int M, float *C, int64_t ldc, hipStream_t s);
 int launch_gemm_q4k(const hipq_weight *w, const QActTiled *qa, int M, float *C,
                     int64_t ldc, hipStream_t s);
+/* gemm_rows_q4k.hip: Q4_K for 3..8 rows on the matrix cores with the reference's bits; qa in the
+ * form of launch_quantize_q8_K_rowmma, the weight with its tile copy (ensure_gemm_tiles) */
+bool gemm_rows_q4k_fits(const hipq_weight *w, int64_t M);
+int launch_gemm_rows_q4k(const hipq_weight *w, const QAct *qa, int M, int pair_rows, float *C, int64_t ldc,
+                         hipStream_t s);
 
 /* moe.hip ----------------------------------------------------------------- */
 /* Variant of the expert MLP. kind 0: h = silu(g) * u, y = down(h) (qwen_moe_layer.cpp:332-392).

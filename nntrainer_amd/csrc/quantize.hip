@@ -228,7 +228,7 @@ int launch_quantize_q8_K(const float *A, int64_t M, int64_t K, int64_t lda,
 }
 
 int launch_quantize_q8_K_rowmma(const float *A, int64_t M, int64_t K, int64_t lda, const QAct *qa,
-                                hipStream_t s) {
+                                hipStream_t s, int64_t mat_rows) {
   if (M <= 0) return HIPQ_OK;
   if (K % 256 || lda < K) return fail(HIPQ_ERR_INVALID_ARGUMENT, "Q8_K: K=%lld must be a multiple of 256 and lda >= K", (long long)K);
   if (((uintptr_t)A & 15) || (lda & 3))
@@ -237,7 +237,7 @@ int launch_quantize_q8_K_rowmma(const float *A, int64_t M, int64_t K, int64_t ld
   const int64_t total = M * nsb;
   const unsigned grid = (unsigned)((total + 3) / 4);
   hipLaunchKernelGGL(quantize_q8_K_kernel<Q8K_ROWMMA>, dim3(grid), dim3(256), 0, s, A, M, total, nsb, lda,
-                     (int64_t)0, qa->q, qa->d, nullptr, nullptr, (uint16_t *)qa->bsum, nullptr, nullptr);
+                     mat_rows, qa->q, qa->d, nullptr, nullptr, (uint16_t *)qa->bsum, nullptr, nullptr);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
 }

@@ -56,6 +56,28 @@ def test_small_m_matches_oracle(hipq, cr, kind, m):
 
 
 @pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("m,n,k", [(3, 2304, 2048), (4, 2050, 4096), (5, 2056, 2048), (8, 4100, 2048),
+                                   (7, 12288, 2048), (3, 8200, 1024), (4, 8195, 2048), (6, 1100, 768),
+                                   (8, 1024, 256), (5, 3000, 4096)])
+def test_small_m_on_large_matrices_matches_oracle(hipq, cr, kind, m, n, k):
+    """Three to eight rows against larger matrices, where Q4_K leaves the GEMV engine for the
+    matrix-core kernel of gemm_rows_q4k.hip (five rows and more from 1024 columns up, three and
+    four from 8192): rows under the reference's 4-row rule and under its row rule in one call
+    (6 = 4 + 2), one to sixteen super-blocks a row (a round of four wavefronts partly idle, a
+    single round), column counts that end inside a 32-column tile. Same bits as the reference,
+    for all three formats."""
+    import gpu_util as gu
+    blocks = _weights(cr, kind, n, k, seed=700 + n)
+    a = synth.normal(701 + k + m, (m, k))
+    ref = cr.gemm(cr.oracle(), kind, a, blocks, n)
+    w = capi.Weight(kind, n, k, blocks)
+    got = gu.gpu_matmul(w, a)
+    w.destroy()
+    assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), \
+        "%d of %d outputs differ in bits" % ((got.view(np.uint32) != ref.view(np.uint32)).sum(), got.size)
+
+
+@pytest.mark.parametrize("kind", KINDS)
 @pytest.mark.parametrize("m,n,k", [(1, 8200, 12288), (3, 200, 8192), (8, 520, 9216), (1, 96, 20480),
                                    (5, 64, 4352)])
 def test_rows_longer_than_one_chunk_match_oracle(hipq, cr, kind, m, n, k):

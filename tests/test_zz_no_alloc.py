@@ -93,3 +93,34 @@ def test_noalloc_q6_K_prefill_before_the_tile_copy_exists(hipq, cr):
         assert gu.rel_err(full.cpu().numpy(), ref) <= gu.TOL
     finally:
         w.destroy()
+
+
+def test_noalloc_q4_K_few_rows_before_and_after_the_tile_copy(hipq, cr):
+    """Five to eight rows of a Q4_K matrix run on the matrix cores off the weight's tile copy, which
+    only an allocating call can build: on a fresh weight the allocation-free call takes the GEMV
+    engine, afterwards the matrix-core kernel. Both carry the reference's bits."""
+    import torch
+    import gpu_util as gu
+    n, k, m = 1056, 1024, 6
+    blocks = cr.quantize_weights(cr.oracle(), "q4_K", synth.normal(87, (n, k), 0.02))
+    w = capi.Weight("q4_K", n, k, blocks)
+    try:
+        a = synth.normal(88, (m, k))
+        da = gu.dev(a)
+        ref = cr.gemm(cr.oracle(), "q4_K", a, blocks, n)
+        first = torch.full((m, n), float("nan"), device="cuda")
+        free_before = torch.cuda.mem_get_info()[0]
+        capi.matmul_noalloc(w, da, m, first, stream=gu.stream())
+        torch.cuda.synchronize()
+        assert torch.cuda.mem_get_info()[0] == free_before
+        assert np.array_equal(first.cpu().numpy().view(np.uint32), ref.view(np.uint32))
+        full = torch.full((m, n), float("nan"), device="cuda")
+        capi.matmul(w, da, m, full, stream=gu.stream())
+        again = torch.full((m, n), float("nan"), device="cuda")
+        capi.matmul_noalloc(w, da, m, again, stream=gu.stream())
+        torch.cuda.synchronize()
+        assert np.array_equal(full.cpu().numpy().view(np.uint32), ref.view(np.uint32))
+        assert np.array_equal(again.cpu().numpy().view(np.uint32), ref.view(np.uint32))
+    finally:
+        w.destroy()
+
