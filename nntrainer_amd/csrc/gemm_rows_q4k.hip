@@ -11,7 +11,8 @@
  * pairs of a super-block to a row's sum one after the other, the others through
  * nntr_gemv_q4_K_8x8_q8_K (:7080-7494), which adds the super-block's total. The GEMV engine
  * (gemv_device.h) does the same on the vector ALU, where a row of activations costs about
- * 4 us on a 12288 x 4096 matrix (eight rows: 37 us; one row: 8 us, the weight stream).
+ * 4 us on a 12288 x 4096 matrix (eight rows: 37 us; one row: 8 us, the weight stream); this
+ * kernel takes 12.8 us for eight.
  *
  * Here a workgroup owns 32 output columns and all rows. Its four wavefronts take one
  * super-block each per round: one v_mfma_i32_32x32x32_i8 per sub-block (the rows are the
@@ -23,7 +24,7 @@
  * vector ALU but the integer work is not. Weights come from the 32-row tile copy the prefill
  * GEMM reads (piece i of lane (n, g) = sub-block 4 g + i of row n; the two lanes of a row swap
  * halves with v_permlane32_swap so that each holds its 16 weights of sub-blocks i and 4 + i),
- * the next round's loads in flight during the current round.
+ * the loads of the next two rounds in flight during the current one.
  * Rows of one chunk only (K <= 4096: the quantized rows stay in LDS).
  */
 #include "hipq_internal.h"
@@ -42,7 +43,10 @@ constexpr int TC = 8;    /* activation rows a workgroup holds */
 constexpr int NREG = 4;  /* result registers of a matrix step that carry them */
 constexpr int SBR = 4;   /* super-blocks a round = wavefronts a workgroup */
 constexpr int NT = 64 * SBR;
-constexpr int REC_DWORDS = SBR * 8 * NREG * 64; /* [wavefront][partial 0-7][register][lane] */
+/* a round's partial sums: [wavefront][register][integer sums | min sums][lane][pair 0-3], so that a
+ * lane writes, and a chain reads, the four pairs of one kind as one 128-bit access, consecutive
+ * lanes consecutive in memory */
+constexpr int REC_DWORDS = SBR * NREG * 2 * 64 * 4;
 
 struct RowsLds {
   int8_t *q;      /* [TC][K + 16]: rows padded so that the lanes of a 128-bit read fall into different banks */
@@ -88,17 +92,34 @@ __global__ __launch_bounds__(NT, 2) void gemm_rows_q4k_kernel(WView w, QView a, 
       r.q[i] = __builtin_bit_cast(rv4i, __builtin_amdgcn_raw_buffer_load_b128(rq, lane * 16, sb * 4096 + i * 1024, 2));
     r.hd = __builtin_bit_cast(rv4i, __builtin_amdgcn_raw_buffer_load_b128(rh, i32 * 16, sb * 512, 0));
   };
-  RowsRegs WA, WB;
-  load(WA, wave);
+  /* The weights of PD + 1 rounds: the loads of the next PD rounds are in flight during a round.
+   * Every round issues its loads, past the end those of the last super-block again: with a
+   * conditional load the compiler cannot count the loads in flight and waits for all of them. */
+  constexpr int PD = 2, NB = PD + 1;
+  RowsRegs buf[NB];
+  const int rounds = (nsb + SBR - 1) / SBR;
+#pragma unroll
+  for (int p = 0; p < PD; ++p) load(buf[p], p * SBR + wave);
 
   /* the M quantized rows, while the first weights are on their way (rows M .. TC - 1 of the
    * matrix operand keep what the LDS held: a row of the product depends on its own
    * activations only, and those rows are not stored) */
   {
-    const int cpr = K >> 4;
-    for (int c = threadIdx.x; c < M * cpr; c += NT) {
-      const int r = c / cpr, o = c - r * cpr;
-      *(rv4i *)(l.q + r * (K + 16) + o * 16) = *(const rv4i *)(a.q + (size_t)r * K + o * 16);
+    const int cpr = K >> 4, np = M * cpr;
+    /* four loads before their stores, so that their latencies overlap */
+    for (int c0 = threadIdx.x; c0 < np; c0 += 4 * NT) {
+      rv4i v[4];
+      int dst[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int c = min(c0 + u * NT, np - 1);
+        const int r = c / cpr, o = c - r * cpr;
+        v[u] = *(const rv4i *)(a.q + (size_t)r * K + o * 16);
+        dst[u] = r * (K + 16) + o * 16;
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        if (c0 + u * NT < np) *(rv4i *)(l.q + dst[u]) = v[u];
     }
     for (int c = threadIdx.x; c < M * nsb * 2; c += NT)
       *(rv4i *)(l.amin + c * 16) = *(const rv4i *)((const uint8_t *)a.bsum + (size_t)c * 16);
@@ -115,7 +136,6 @@ __global__ __launch_bounds__(NT, 2) void gemm_rows_q4k_kernel(WView w, QView a, 
   const bool pairwise = cm < pair_rows;
   float acc = 0.f, accm = 0.f;
 
-  const int rounds = (nsb + SBR - 1) / SBR;
   auto round = [&](const RowsRegs &W, int rho) {
     const int sb = rho * SBR + wave;
     if (sb < nsb) { /* uniform per wavefront */
@@ -141,23 +161,33 @@ __global__ __launch_bounds__(NT, 2) void gemm_rows_q4k_kernel(WView w, QView a, 
       for (int p = 0; p < 4; ++p)
 #pragma unroll
         for (int r = 0; r < NREG; ++r) I[p][r] = 0;
+      /* With two wavefronts a SIMD nobody else hides a step's latencies: the eight operands are
+       * read from LDS up front, and step j + 1 is issued into a second result register before the
+       * sums of step j are taken. */
+      rv4i a8[8];
 #pragma unroll
-      for (int j = 0; j < 8; ++j) {
+      for (int j = 0; j < 8; ++j) a8[j] = *(const rv4i *)(pa + j * 32);
+      rv16i D[2];
+      auto step = [&](int j) {
         /* weight 2i / 2i+1 of the lane's 16 in the low / high nibble of byte i: the even ones become
          * operand bytes 0-7, the odd ones bytes 8-15 (the order the activations' 16-value groups are
          * stored in) */
         const uint32_t x0 = (uint32_t)wq[j][0], x1 = (uint32_t)wq[j][1];
         const rv4i b = {(int)(x0 & HIPQ_M4), (int)(x1 & HIPQ_M4), (int)((x0 >> 4) & HIPQ_M4),
                         (int)((x1 >> 4) & HIPQ_M4)};
-        const rv4i a8 = *(const rv4i *)(pa + j * 32);
-        const rv16i D = __builtin_amdgcn_mfma_i32_32x32x32_i8(a8, b, zero16, 0, 0, 0);
+        D[j & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(a8[j], b, zero16, 0, 0, 0);
+      };
+      step(0);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        if (j + 1 < 8) step(j + 1);
         const int scj = (int)(((j < 4 ? s03 : s47) >> (8 * (j & 3))) & 0xff);
 #pragma unroll
-        for (int r = 0; r < NREG; ++r) I[j >> 1][r] = __mul24(D[r], scj) + I[j >> 1][r];
+        for (int r = 0; r < NREG; ++r) I[j >> 1][r] = __mul24(D[j & 1][r], scj) + I[j >> 1][r];
       }
       const uint32_t mlo = (hd.w & 0x0f0f0f0fu) | ((hd.y >> 2) & 0x30303030u);
       const uint32_t mhi = ((hd.w >> 4) & 0x0f0f0f0fu) | ((hd.z >> 2) & 0x30303030u);
-      uint32_t *rec = l.rec + wave * (8 * NREG * 64) + lane;
+      float Sm[4][NREG];
 #pragma unroll
       for (int p = 0; p < 4; ++p) {
         /* the mins of pair p against the sub-block sums (both halves of the K index carry the same
@@ -166,12 +196,17 @@ __global__ __launch_bounds__(NT, 2) void gemm_rows_q4k_kernel(WView w, QView a, 
         rv8h bmin = {0, 0, 0, 0, 0, 0, 0, 0};
         bmin[2 * p] = (_Float16)(float)((mw >> (16 * (p & 1))) & 0xff);
         bmin[2 * p + 1] = (_Float16)(float)((mw >> (16 * (p & 1) + 8)) & 0xff);
-        const rv16f Sm = __builtin_amdgcn_mfma_f32_32x32x16_f16(amin, bmin, zero16f, 0, 0, 0);
+        const rv16f S = __builtin_amdgcn_mfma_f32_32x32x16_f16(amin, bmin, zero16f, 0, 0, 0);
 #pragma unroll
-        for (int r = 0; r < NREG; ++r) {
-          rec[(p * NREG + r) * 64] = (uint32_t)I[p][r];
-          rec[((4 + p) * NREG + r) * 64] = __float_as_uint(Sm[r]);
-        }
+        for (int r = 0; r < NREG; ++r) Sm[p][r] = S[r];
+      }
+      uint32_t *rec = l.rec + wave * (NREG * 2 * 256) + lane * 4;
+#pragma unroll
+      for (int r = 0; r < NREG; ++r) {
+        *(rv4i *)(rec + (r * 2) * 256) = rv4i{I[0][r], I[1][r], I[2][r], I[3][r]};
+        *(rv4i *)(rec + (r * 2 + 1) * 256) =
+          rv4i{(int)__float_as_uint(Sm[0][r]), (int)__float_as_uint(Sm[1][r]), (int)__float_as_uint(Sm[2][r]),
+               (int)__float_as_uint(Sm[3][r])};
       }
       if (g == 0) {
         l.dw[(wave * 2) * 32 + i32] = hipq_h2f((uint16_t)(hd.x & 0xffff));
@@ -179,18 +214,30 @@ __global__ __launch_bounds__(NT, 2) void gemm_rows_q4k_kernel(WView w, QView a, 
       }
     }
     __syncthreads();
-    /* the chains of this round's super-blocks, ascending */
+    /* the chains of this round's super-blocks, ascending; everything a chain reads is requested
+     * before the first step (the records of a wavefront that had no super-block are read as well
+     * and not used: a read behind a branch would wait for its own latency) */
+    rv4i ivs[SBR], mvs[SBR];
+    float dAs[SBR], dws[SBR], dms[SBR];
+#pragma unroll
+    for (int ws = 0; ws < SBR; ++ws) {
+      const uint32_t *rec = l.rec + ws * (NREG * 2 * 256) + (cr * 2) * 256 + cl * 4;
+      ivs[ws] = *(const rv4i *)rec;
+      mvs[ws] = *(const rv4i *)(rec + 256);
+      dAs[ws] = l.dA[min(rho * SBR + ws, nsb - 1) * TC + cm];
+      dws[ws] = l.dw[(ws * 2) * 32 + cn];
+      dms[ws] = l.dw[(ws * 2 + 1) * 32 + cn];
+    }
 #pragma unroll
     for (int ws = 0; ws < SBR; ++ws) {
       const int sbw = rho * SBR + ws;
       if (sbw < nsb) { /* uniform */
-        const uint32_t *rec = l.rec + ws * (8 * NREG * 64) + cr * 64 + cl;
-        const int I0 = (int)rec[0 * NREG * 64], I1 = (int)rec[1 * NREG * 64], I2 = (int)rec[2 * NREG * 64],
-                  I3 = (int)rec[3 * NREG * 64];
-        const float M0 = __uint_as_float(rec[4 * NREG * 64]), M1 = __uint_as_float(rec[5 * NREG * 64]),
-                    M2 = __uint_as_float(rec[6 * NREG * 64]), M3 = __uint_as_float(rec[7 * NREG * 64]);
-        const float dA = l.dA[sbw * TC + cm];
-        const float sd = l.dw[(ws * 2) * 32 + cn] * dA, sm = l.dw[(ws * 2 + 1) * 32 + cn] * dA;
+        const rv4i iv = ivs[ws], mv = mvs[ws];
+        const int I0 = iv[0], I1 = iv[1], I2 = iv[2], I3 = iv[3];
+        const float M0 = __int_as_float(mv[0]), M1 = __int_as_float(mv[1]), M2 = __int_as_float(mv[2]),
+                    M3 = __int_as_float(mv[3]);
+        const float dA = dAs[ws];
+        const float sd = dws[ws] * dA, sm = dms[ws] * dA;
         if (pairwise) {
           acc = fmaf((float)I0, sd, acc);
           accm = fmaf(M0, sm, accm);
@@ -209,13 +256,15 @@ __global__ __launch_bounds__(NT, 2) void gemm_rows_q4k_kernel(WView w, QView a, 
     }
     __syncthreads(); /* the next round overwrites the records */
   };
-  /* two rounds a trip so that each register set has a fixed name; all conditions are uniform */
-  for (int rho = 0; rho < rounds; rho += 2) {
-    if (rho + 1 < rounds) load(WB, (rho + 1) * SBR + wave);
-    round(WA, rho);
-    if (rho + 1 < rounds) {
-      if (rho + 2 < rounds) load(WA, (rho + 2) * SBR + wave);
-      round(WB, rho + 1);
+  /* NB rounds a trip so that each register set has a fixed name; all conditions are uniform */
+  for (int rho0 = 0; rho0 < rounds; rho0 += NB) {
+#pragma unroll
+    for (int u = 0; u < NB; ++u) {
+      const int rho = rho0 + u;
+      if (rho < rounds) {
+        load(buf[(u + PD) % NB], (rho + PD) * SBR + wave);
+        round(buf[u], rho);
+      }
     }
   }
   const int col = tile * 32 + cn;
@@ -227,9 +276,11 @@ __global__ __launch_bounds__(NT, 2) void gemm_rows_q4k_kernel(WView w, QView a, 
 namespace hipq {
 
 /* Where it beats the GEMV engine (measured, kernel us old -> new): five to eight rows from 1024
- * columns up (2048 x 1024: 5.5 -> 4.8; 4096 x 4096: 16.4 -> 11.1; 12288 x 4096: 39.0 -> 12.6;
- * 151936 x 4096: 421 -> 105), three and four rows on large matrices only (12288 x 4096: 14.2 and
- * 16.4 -> 12.5; 4096 x 4096: 7.1 and 8.7 against 10.5 and 10.8). */
+ * columns up (2048 x 1024: 5.5 -> 4.8; 4096 x 4096: 16.4 -> 9.2; 12288 x 4096: 39.0 -> 12.8;
+ * 151936 x 4096: 421 -> 94), three and four rows on large matrices only (12288 x 4096: 14.2 and
+ * 16.4 -> 12.2; 4096 x 4096: 7.1 and 8.7 against 9). A round of a workgroup takes 1.7 us, most of
+ * it the issue of its vector instructions (about 290 a wavefront and super-block: nibble
+ * expansion, scale multiplies, the chains), so the kernel runs at 2-3.6 TB/s of weights. */
 bool gemm_rows_q4k_fits(const hipq_weight *w, int64_t M) {
   if (w->dtype != HIPQ_Q4_K || w->expert_tiles || w->K > HIPQ_KCHUNK || w->K % 256) return false;
   if (M >= 5 && M <= TC) return w->N >= 1024;
