@@ -203,6 +203,16 @@ def main():
     gemv_hot_ms = capi.time_matmul(weights[:1], a1, 1, c1, 400, phase=1, stream=stream)
     gemv_gbs = gv_bytes / (gemv_ms * 1e-3) / 1e9
 
+    # ---- a batch of eight (four) decode rows against the same matrices: Q4_K on the matrix cores
+    # with the reference's bits (gemm_rows_q4k.hip) ----
+    rows_ms = {}
+    for mr in (8, 4):
+        ar = torch.randn((mr, K), generator=gen, device="cuda", dtype=torch.float32)
+        cr_ = torch.empty((mr, N), device="cuda", dtype=torch.float32)
+        capi.time_matmul(weights, ar, mr, cr_, 2 * n_copies, phase=1, stream=stream)
+        rows_ms[mr] = (capi.time_matmul(weights, ar, mr, cr_, 20 * n_copies, phase=1, stream=stream),
+                       capi.time_matmul(weights, ar, mr, cr_, 20 * n_copies, phase=0, stream=stream))
+
     # ---- the same GEMV at lm_head size (N=151936: 350 MB of Q4_K per matrix) ----
     NL = 151936
     wl32 = torch.randn((NL, K), generator=gen, device="cuda", dtype=torch.float32) * 0.02
@@ -469,6 +479,13 @@ def main():
                                      "frac_of_measured_read_ceiling": round(gemv_gbs / read_ceiling_gbs, 5),
                                      "kernel_ms": round(gemv_ms, 5), "traffic": TRAFFIC_GEMV_C2,
                                      "algorithmic_bytes_per_launch": gv_bytes}},
+        "decode_batch_rows": {
+            "workload": "Q4_K, 8 and 4 activation rows (a batch of decode steps) against the same M=1 matrices "
+                        "(K=4096 N=12288, %d copies rotated); outputs carry the reference's bits" % n_copies,
+            "kernel": "gemm_rows_q4k_kernel",
+            "rows_8_kernel_ms": round(rows_ms[8][0], 5), "rows_8_ms_per_call": round(rows_ms[8][1], 5),
+            "rows_4_kernel_ms": round(rows_ms[4][0], 5), "rows_4_ms_per_call": round(rows_ms[4][1], 5),
+            "rows_8_weight_gbs": round(gv_bytes / (rows_ms[8][0] * 1e-3) / 1e9, 2)},
         "decode_gemv_lm_head_size": {
             "workload": "Q4_K GEMV M=1 K=4096 N=151936, 3 weight copies rotated",
             "roofline": {"bound": "hbm", "kernel": "gemv_stream_kernel<Q4_K,G=4,GPW=2>",

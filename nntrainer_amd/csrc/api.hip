@@ -906,8 +906,17 @@ int hipq_matmul_multi(int count, const hipq_weight_t *w, const float *A, int64_t
   auto klass = [&](const hipq_weight *x) {
     if (x->dtype == HIPQ_Q4_0) return 0;
     if (wants_tiled(x, M)) return x->dtype == HIPQ_Q4_K ? 3 : 4; /* the two tiled forms differ in their rows' quantizer */
+    if (wants_rows(x, M, true)) return 5; /* a few rows of Q4_K on the matrix cores: the row form of the MoE kernels */
     return (x->dtype == HIPQ_Q4_K && M > 1) ? 1 : 2;
   };
+  {
+    bool first = true;
+    for (int i = 0; i < count; ++i)
+      if (klass(w[i]) == 5) {
+        if ((rc = matmul_rows(w[i], A, M, lda, C[i], ldc[i], s, first ? 0 : 1, Scratch{false, s}))) return rc;
+        first = false;
+      }
+  }
   for (int k = 3; k <= 4; ++k) {
     int members = 0;
     for (int i = 0; i < count; ++i) members += klass(w[i]) == k;

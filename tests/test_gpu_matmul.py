@@ -431,6 +431,29 @@ def test_matmul_multi_other_formats_and_prefill(hipq, cr, kind, m):
         w.destroy()
 
 
+@pytest.mark.parametrize("m", [4, 6])
+def test_matmul_multi_few_rows_mixed_paths(hipq, cr, m):
+    """A few rows against Q4_K weights of different sizes (and a Q6_K one) in one multi-weight call:
+    the large Q4_K matrices take the matrix-core kernel (one quantization in its row form shared by
+    them), the small one and the Q6_K one the GEMV engine with their own quantizations. All carry
+    the reference's bits, whatever the order of the weights in the call."""
+    import gpu_util as gu
+    import torch
+    k = 1024
+    kinds, ns = ["q4_K", "q4_K", "q6_K", "q4_K", "q4_K"], [8192, 512, 640, 1056, 8200]
+    blocks = [_weights(cr, kd, n, k, seed=95 + i) for i, (kd, n) in enumerate(zip(kinds, ns))]
+    ws = [capi.Weight(kd, n, k, b) for kd, n, b in zip(kinds, ns, blocks)]
+    a = synth.normal(99 + m, (m, k))
+    outs = [torch.full((m, n), float("nan"), device="cuda") for n in ns]
+    capi.matmul_multi(ws, gu.dev(a), m, outs, stream=gu.stream())
+    torch.cuda.synchronize()
+    for kd, n, b, o in zip(kinds, ns, blocks, outs):
+        ref = cr.gemm(cr.oracle(), kd, a, b, n)
+        assert np.array_equal(o.cpu().numpy().view(np.uint32), ref.view(np.uint32)), (kd, n)
+    for w in ws:
+        w.destroy()
+
+
 def test_matmul_multi_mixed_k_formats_prefill(hipq, cr):
     """Q4_K and Q6_K weights in one multi-weight prefill call: both take tiled Q8_K activations, but
     the reference quantizes the rows of a Q4_K product four at a time and those of a Q6_K product one
