@@ -152,9 +152,9 @@ HIPQ_API int hipq_quantize_q8_K(const float *A, int64_t M, int64_t K, int64_t ld
  *  quantized activations, another order of the fp32 sums). The first such product of a
  *  weight adds a copy of it in the kernels' load order (allocates; 0.56 bytes per weight
  *  for Q4_K, 0.875 for Q6_K), kept until hipq_weight_destroy. Q4_K with 5..8 rows and 1024
- *  columns or more (3..8 rows from 8192 columns), K <= 4096, reads the same copy: those row
+ *  columns or more (4 rows from 4096, 3 from 8192 columns) reads the same copy: those row
  *  counts run on the matrix cores as well, with the reference's bits (a batch of decode
- *  rows against a 12288 x 4096 matrix: 13 us for eight, 8 us for one). */
+ *  rows against a 12288 x 4096 matrix: 11 us for eight, 8 us for one). */
 HIPQ_API int hipq_matmul(hipq_weight_t w, const float *A, int64_t M, int64_t lda,
                          float *C, int64_t ldc, int mem, void *stream);
 

@@ -12,7 +12,7 @@
  * nntr_gemv_q4_K_8x8_q8_K (:7080-7494), which adds the super-block's total. The GEMV engine
  * (gemv_device.h) does the same on the vector ALU, where a row of activations costs about
  * 4 us on a 12288 x 4096 matrix (eight rows: 37 us; one row: 8 us, the weight stream); this
- * kernel takes 12.8 us for eight.
+ * kernel takes 11.2 us for eight.
  *
  * Here a workgroup owns 32 output columns and all rows. Its four wavefronts take one
  * super-block each per round: one v_mfma_i32_32x32x32_i8 per sub-block (the rows are the
@@ -24,8 +24,8 @@
  * vector ALU but the integer work is not. Weights come from the 32-row tile copy the prefill
  * GEMM reads (piece i of lane (n, g) = sub-block 4 g + i of row n; the two lanes of a row swap
  * halves with v_permlane32_swap so that each holds its 16 weights of sub-blocks i and 4 + i),
- * the loads of the next two rounds in flight during the current one.
- * Rows of one chunk only (K <= 4096: the quantized rows stay in LDS).
+ * the loads of the next two rounds in flight during the current one. The quantized rows are
+ * staged a round at a time (52 KB of LDS with the records: three workgroups a CU, any K).
  */
 #include "hipq_internal.h"
 #include "gemv_device.h"
@@ -48,20 +48,16 @@ constexpr int NT = 64 * SBR;
  * lanes consecutive in memory */
 constexpr int REC_DWORDS = SBR * NREG * 2 * 64 * 4;
 
-struct RowsLds {
-  int8_t *q;      /* [TC][K + 16]: rows padded so that the lanes of a 128-bit read fall into different banks */
-  uint8_t *amin;  /* [TC][nsb][32 bytes]: sub-block sums as two fp16-exact parts */
-  float *dA;      /* [nsb][TC] */
-  uint32_t *rec;  /* the round's partial sums */
-  float *dw;      /* [SBR][2][32]: d and dmin of the round's super-blocks, per column */
-};
-__host__ __device__ inline size_t rows_lds_rec_offset(int K) {
-  const size_t b = (size_t)TC * (K + 16) + (size_t)TC * (K / 256) * 32 + (size_t)TC * (K / 256) * 4;
-  return (b + 255) & ~(size_t)255;
-}
-__host__ __device__ inline size_t rows_lds_bytes(int K) {
-  return rows_lds_rec_offset(K) + (size_t)REC_DWORDS * 4 + (size_t)SBR * 2 * 32 * 4;
-}
+/* LDS of a workgroup: the quantized rows of the current and of the next round (four
+ * super-blocks of every row: int8 values, the sub-block sums as two fp16-exact parts, the
+ * scales), the round's partial sums, and d and dmin of its super-blocks per column. */
+constexpr int QROW = SBR * 256 + 16; /* a staged row, padded so that the lanes of a 128-bit read fall into different banks */
+constexpr int ACT_Q = 0, ACT_AMIN = TC * QROW, ACT_DA = ACT_AMIN + TC * SBR * 32;
+constexpr int ACT_BYTES = ACT_DA + SBR * TC * 4;
+constexpr int LDS_REC = (2 * ACT_BYTES + 255) / 256 * 256;
+constexpr int LDS_DW = LDS_REC + REC_DWORDS * 4;
+constexpr int LDS_BYTES = LDS_DW + SBR * 2 * 32 * 4;
+static_assert(ACT_BYTES % 16 == 0 && 3 * LDS_BYTES <= 160 * 1024, "three workgroups a CU");
 
 struct RowsRegs {
   rv4i q[4];
@@ -75,12 +71,8 @@ __global__ __launch_bounds__(NT, 2) void gemm_rows_q4k_kernel(WView w, QView a, 
   const int tile = blockIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const int lane = threadIdx.x & 63, i32 = lane & 31, g = lane >> 5;
-  RowsLds l;
-  l.q = (int8_t *)rows_lds;
-  l.amin = rows_lds + (size_t)TC * (K + 16);
-  l.dA = (float *)(l.amin + (size_t)TC * nsb * 32);
-  l.rec = (uint32_t *)(rows_lds + rows_lds_rec_offset(K));
-  l.dw = (float *)(l.rec + REC_DWORDS);
+  uint32_t *const lrec = (uint32_t *)(rows_lds + LDS_REC);
+  float *const ldw = (float *)(rows_lds + LDS_DW);
 
   /* the tile's nibbles and headers as buffer descriptors in scalar registers */
   const rrsrc_t rq = __builtin_amdgcn_make_buffer_rsrc((void *)(w.qs + (size_t)tile * (size_t)(16 * K)), 0, 16 * K, 0x00020000);
@@ -92,42 +84,56 @@ __global__ __launch_bounds__(NT, 2) void gemm_rows_q4k_kernel(WView w, QView a, 
       r.q[i] = __builtin_bit_cast(rv4i, __builtin_amdgcn_raw_buffer_load_b128(rq, lane * 16, sb * 4096 + i * 1024, 2));
     r.hd = __builtin_bit_cast(rv4i, __builtin_amdgcn_raw_buffer_load_b128(rh, i32 * 16, sb * 512, 0));
   };
+  /* A round's share of the M quantized rows goes through registers into one of two LDS buffers:
+   * loaded (from the cache) at the start of the previous round, stored behind that round's first
+   * barrier. Rows M .. TC - 1 repeat row M - 1 and pieces past the end of a row its last piece:
+   * every thread always issues the same loads, and what they fetch there is never used. */
+  struct ActRegs {
+    rv4i q[2], amin;
+    float dA;
+  };
+  auto act_load = [&](ActRegs &r, int rho) {
+    const int t = threadIdx.x;
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int c = t + u * NT;
+      const int row = min(c >> 6, M - 1), off = min(rho * (SBR * 256) + (c & 63) * 16, K - 16);
+      r.q[u] = *(const rv4i *)(a.q + (size_t)row * K + off);
+    }
+    {
+      const int tt = t & 63, row = min(tt >> 3, M - 1);
+      const int off = min(rho * (SBR * 32) + (tt & 7) * 16, nsb * 32 - 16);
+      r.amin = *(const rv4i *)((const uint8_t *)a.bsum + (size_t)row * nsb * 32 + off);
+    }
+    {
+      const int tt = t & 31, row = min(tt >> 2, M - 1);
+      r.dA = a.d[(size_t)row * nsb + min(rho * SBR + (tt & 3), nsb - 1)];
+    }
+  };
+  auto act_store = [&](const ActRegs &r, int which) {
+    unsigned char *base = rows_lds + which * ACT_BYTES;
+    const int t = threadIdx.x;
+#pragma unroll
+    for (int u = 0; u < 2; ++u) {
+      const int c = t + u * NT;
+      *(rv4i *)(base + ACT_Q + (c >> 6) * QROW + (c & 63) * 16) = r.q[u];
+    }
+    if (t < 64) *(rv4i *)(base + ACT_AMIN + t * 16) = r.amin; /* [row][super-block of the round][32 bytes] */
+    if (t < 32) ((float *)(base + ACT_DA))[(t & 3) * TC + (t >> 2)] = r.dA; /* [super-block][row] */
+  };
+  ActRegs AR;
+  act_load(AR, 0);
   /* The weights of PD + 1 rounds: the loads of the next PD rounds are in flight during a round.
    * Every round issues its loads, past the end those of the last super-block again: with a
-   * conditional load the compiler cannot count the loads in flight and waits for all of them. */
-  constexpr int PD = 2, NB = PD + 1;
+   * conditional load the compiler cannot count the loads in flight and waits for all of them.
+   * One round ahead keeps the kernel at 162 VGPRs, three wavefronts a SIMD as the LDS allows;
+   * two rounds ahead (182) cost a third of them: 151936 x 4096 with eight rows 91 against 75 us. */
+  constexpr int PD = 1, NB = PD + 1;
   RowsRegs buf[NB];
   const int rounds = (nsb + SBR - 1) / SBR;
 #pragma unroll
   for (int p = 0; p < PD; ++p) load(buf[p], p * SBR + wave);
-
-  /* the M quantized rows, while the first weights are on their way (rows M .. TC - 1 of the
-   * matrix operand keep what the LDS held: a row of the product depends on its own
-   * activations only, and those rows are not stored) */
-  {
-    const int cpr = K >> 4, np = M * cpr;
-    /* four loads before their stores, so that their latencies overlap */
-    for (int c0 = threadIdx.x; c0 < np; c0 += 4 * NT) {
-      rv4i v[4];
-      int dst[4];
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int c = min(c0 + u * NT, np - 1);
-        const int r = c / cpr, o = c - r * cpr;
-        v[u] = *(const rv4i *)(a.q + (size_t)r * K + o * 16);
-        dst[u] = r * (K + 16) + o * 16;
-      }
-#pragma unroll
-      for (int u = 0; u < 4; ++u)
-        if (c0 + u * NT < np) *(rv4i *)(l.q + dst[u]) = v[u];
-    }
-    for (int c = threadIdx.x; c < M * nsb * 2; c += NT)
-      *(rv4i *)(l.amin + c * 16) = *(const rv4i *)((const uint8_t *)a.bsum + (size_t)c * 16);
-    for (int c = threadIdx.x; c < M * nsb; c += NT) {
-      const int r = c / nsb, b = c - r * nsb;
-      l.dA[b * TC + r] = a.d[c];
-    }
-  }
+  act_store(AR, 0);
   __syncthreads();
 
   /* the output this thread chains: row cm, column cn; its sums sit in register cr of lane cl */
@@ -137,13 +143,14 @@ __global__ __launch_bounds__(NT, 2) void gemm_rows_q4k_kernel(WView w, QView a, 
   float acc = 0.f, accm = 0.f;
 
   auto round = [&](const RowsRegs &W, int rho) {
+    const unsigned char *act = rows_lds + (rho & 1) * ACT_BYTES;
     const int sb = rho * SBR + wave;
     if (sb < nsb) { /* uniform per wavefront */
       const rv16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
       const rv16f zero16f = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
       const int row = i32 & (TC - 1);
-      const int8_t *pa = l.q + row * (K + 16) + sb * 256 + g * 16;
-      const rv8h amin = *(const rv8h *)(l.amin + (row * nsb + sb) * 32 + g * 16);
+      const int8_t *pa = (const int8_t *)act + ACT_Q + row * QROW + wave * 256 + g * 16;
+      const rv8h amin = *(const rv8h *)(act + ACT_AMIN + (row * SBR + wave) * 32 + g * 16);
       /* wq[j]: this lane's 16 weights (8 bytes) of sub-block j */
       rv2i wq[8];
 #pragma unroll
@@ -200,7 +207,7 @@ __global__ __launch_bounds__(NT, 2) void gemm_rows_q4k_kernel(WView w, QView a, 
 #pragma unroll
         for (int r = 0; r < NREG; ++r) Sm[p][r] = S[r];
       }
-      uint32_t *rec = l.rec + wave * (NREG * 2 * 256) + lane * 4;
+      uint32_t *rec = lrec + wave * (NREG * 2 * 256) + lane * 4;
 #pragma unroll
       for (int r = 0; r < NREG; ++r) {
         *(rv4i *)(rec + (r * 2) * 256) = rv4i{I[0][r], I[1][r], I[2][r], I[3][r]};
@@ -209,11 +216,12 @@ __global__ __launch_bounds__(NT, 2) void gemm_rows_q4k_kernel(WView w, QView a, 
                (int)__float_as_uint(Sm[3][r])};
       }
       if (g == 0) {
-        l.dw[(wave * 2) * 32 + i32] = hipq_h2f((uint16_t)(hd.x & 0xffff));
-        l.dw[(wave * 2 + 1) * 32 + i32] = hipq_h2f((uint16_t)(hd.x >> 16));
+        ldw[(wave * 2) * 32 + i32] = hipq_h2f((uint16_t)(hd.x & 0xffff));
+        ldw[(wave * 2 + 1) * 32 + i32] = hipq_h2f((uint16_t)(hd.x >> 16));
       }
     }
     __syncthreads();
+    act_store(AR, (rho + 1) & 1); /* the next round's rows: that buffer was last read a round ago */
     /* the chains of this round's super-blocks, ascending; everything a chain reads is requested
      * before the first step (the records of a wavefront that had no super-block are read as well
      * and not used: a read behind a branch would wait for its own latency) */
@@ -221,12 +229,12 @@ __global__ __launch_bounds__(NT, 2) void gemm_rows_q4k_kernel(WView w, QView a, 
     float dAs[SBR], dws[SBR], dms[SBR];
 #pragma unroll
     for (int ws = 0; ws < SBR; ++ws) {
-      const uint32_t *rec = l.rec + ws * (NREG * 2 * 256) + (cr * 2) * 256 + cl * 4;
+      const uint32_t *rec = lrec + ws * (NREG * 2 * 256) + (cr * 2) * 256 + cl * 4;
       ivs[ws] = *(const rv4i *)rec;
       mvs[ws] = *(const rv4i *)(rec + 256);
-      dAs[ws] = l.dA[min(rho * SBR + ws, nsb - 1) * TC + cm];
-      dws[ws] = l.dw[(ws * 2) * 32 + cn];
-      dms[ws] = l.dw[(ws * 2 + 1) * 32 + cn];
+      dAs[ws] = ((const float *)(act + ACT_DA))[ws * TC + cm];
+      dws[ws] = ldw[(ws * 2) * 32 + cn];
+      dms[ws] = ldw[(ws * 2 + 1) * 32 + cn];
     }
 #pragma unroll
     for (int ws = 0; ws < SBR; ++ws) {
@@ -262,6 +270,7 @@ __global__ __launch_bounds__(NT, 2) void gemm_rows_q4k_kernel(WView w, QView a, 
     for (int u = 0; u < NB; ++u) {
       const int rho = rho0 + u;
       if (rho < rounds) {
+        act_load(AR, rho + 1); /* before the weights: its wait must not include theirs */
         load(buf[(u + PD) % NB], (rho + PD) * SBR + wave);
         round(buf[u], rho);
       }
@@ -276,31 +285,28 @@ __global__ __launch_bounds__(NT, 2) void gemm_rows_q4k_kernel(WView w, QView a, 
 namespace hipq {
 
 /* Where it beats the GEMV engine (measured, kernel us old -> new): five to eight rows from 1024
- * columns up (2048 x 1024: 5.5 -> 4.8; 4096 x 4096: 16.4 -> 9.2; 12288 x 4096: 39.0 -> 12.8;
- * 151936 x 4096: 421 -> 94), three and four rows on large matrices only (12288 x 4096: 14.2 and
- * 16.4 -> 12.2; 4096 x 4096: 7.1 and 8.7 against 9). A round of a workgroup takes 1.7 us, most of
- * it the issue of its vector instructions (about 290 a wavefront and super-block: nibble
- * expansion, scale multiplies, the chains), so the kernel runs at 2-3.6 TB/s of weights. */
+ * columns up (2048 x 1024: 5.5 -> 4.0; 4096 x 4096: 16.4 -> 8.3; 12288 x 4096: 39.0 -> 11.2;
+ * 151936 x 4096: 421 -> 75), four rows from 4096 columns (4096 x 4096: 8.7 -> 8.3; 12288 x 4096:
+ * 16.4 -> 11.0), three from 8192 (12288 x 4096: 14.2 -> 11; 4096 x 4096: 7.1 against 8.2). A round
+ * of a workgroup takes 1.7 us, most of it the issue of its vector instructions (about 290 a
+ * wavefront and super-block: nibble expansion, scale multiplies, the chains), so the kernel
+ * streams its weights at 2.5-4.6 TB/s. */
 bool gemm_rows_q4k_fits(const hipq_weight *w, int64_t M) {
-  if (w->dtype != HIPQ_Q4_K || w->expert_tiles || w->K > HIPQ_KCHUNK || w->K % 256) return false;
+  if (w->dtype != HIPQ_Q4_K || w->expert_tiles || w->K % 256 || 16 * w->K > 0x7fffffff) return false;
   if (M >= 5 && M <= TC) return w->N >= 1024;
-  return (M == 3 || M == 4) && w->N >= 8192;
+  return (M == 4 && w->N >= 4096) || (M == 3 && w->N >= 8192);
 }
 
 int launch_gemm_rows_q4k(const hipq_weight *w, const QAct *qa, int M, int pair_rows, float *C, int64_t ldc,
                          hipStream_t s) {
   if (!gemm_rows_q4k_fits(w, M) || qa->K != w->K)
-    return fail(HIPQ_ERR_INVALID_ARGUMENT, "the few-rows Q4_K product takes 3..8 rows of one chunk");
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "the few-rows Q4_K product takes 3..8 rows");
   if (!w->gt_base) return fail(HIPQ_ERR_INVALID_ARGUMENT, "the few-rows Q4_K product needs the weight's tile copy");
-  const size_t lds = rows_lds_bytes((int)w->K);
-  if (lds > 64 * 1024)
-    HIPQ_HIP(hipFuncSetAttribute((const void *)gemm_rows_q4k_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                 (int)lds));
   WView v = wview(w);
   v.qs = w->gt_qs;
   v.hdr = w->gt_hdr;
   const unsigned grid = (unsigned)((w->N + 31) / 32);
-  hipLaunchKernelGGL(gemm_rows_q4k_kernel, dim3(grid), dim3(NT), lds, s, v, qview(*qa), M, pair_rows, C, ldc);
+  hipLaunchKernelGGL(gemm_rows_q4k_kernel, dim3(grid), dim3(NT), LDS_BYTES, s, v, qview(*qa), M, pair_rows, C, ldc);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
 }

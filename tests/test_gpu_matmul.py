@@ -58,14 +58,15 @@ def test_small_m_matches_oracle(hipq, cr, kind, m):
 @pytest.mark.parametrize("kind", KINDS)
 @pytest.mark.parametrize("m,n,k", [(3, 2304, 2048), (4, 2050, 4096), (5, 2056, 2048), (8, 4100, 2048),
                                    (7, 12288, 2048), (3, 8200, 1024), (4, 8195, 2048), (6, 1100, 768),
-                                   (8, 1024, 256), (5, 3000, 4096)])
+                                   (8, 1024, 256), (5, 3000, 4096), (8, 1030, 8192), (6, 1024, 5376),
+                                   (4, 4100, 1280)])
 def test_small_m_on_large_matrices_matches_oracle(hipq, cr, kind, m, n, k):
     """Three to eight rows against larger matrices, where Q4_K leaves the GEMV engine for the
     matrix-core kernel of gemm_rows_q4k.hip (five rows and more from 1024 columns up, three and
     four from 8192): rows under the reference's 4-row rule and under its row rule in one call
-    (6 = 4 + 2), one to sixteen super-blocks a row (a round of four wavefronts partly idle, a
-    single round), column counts that end inside a 32-column tile. Same bits as the reference,
-    for all three formats."""
+    (6 = 4 + 2), one to 32 super-blocks a row (a round of four wavefronts partly idle, a single
+    round, rows longer than the GEMV engine's 4096-weight chunk), column counts that end inside
+    a 32-column tile. Same bits as the reference, for all three formats."""
     import gpu_util as gu
     blocks = _weights(cr, kind, n, k, seed=700 + n)
     a = synth.normal(701 + k + m, (m, k))
