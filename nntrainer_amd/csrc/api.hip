@@ -305,6 +305,8 @@ QAct qact_rows(const QAct &a, int is_k, int64_t r0, int64_t rows) {
  * keep the reference's bits). */
 bool wants_tiled(const hipq_weight *w, int64_t M, bool may_allocate = true) {
   if (w->dtype == HIPQ_Q6_K) return M > 16 && (w->gt_base || may_allocate);
+  /* up to 16 rows of a Q4_K matrix of 1024 columns or more take the few-rows kernel (wants_rows) */
+  if (hipq::gemm_rows_q4k_fits(w, M) && (w->gt_base || may_allocate)) return false;
   return w->dtype == HIPQ_Q4_K && M > 8 && w->N * (w->K / 2) < (int64_t(1) << 32);
 }
 
@@ -402,14 +404,20 @@ int matmul_rows(const hipq_weight *w, const float *A, int64_t M, int64_t lda, fl
   if (phase != 1) rc = hipq::launch_quantize_q8_K_rowmma(A, M, w->K, lda, &qa, s, mat_rows);
   if (rc || phase == 2) return rc;
   if (!w->gt_base && (rc = hipq::ensure_gemm_tiles(const_cast<hipq_weight *>(w)))) return rc;
-  return hipq::launch_gemm_rows_q4k(w, &qa, (int)M, (int)mat_rows, C, ldc, s);
+  for (int64_t r0 = 0; r0 < M && !rc; r0 += 8) { /* passes of up to eight rows */
+    const int64_t rows = (M - r0) < 8 ? (M - r0) : 8;
+    const int64_t pair = mat_rows - r0 < 0 ? 0 : (mat_rows - r0 > rows ? rows : mat_rows - r0);
+    const QAct sub = qact_rows(qa, 1, r0, rows);
+    rc = hipq::launch_gemm_rows_q4k(w, &sub, (int)rows, (int)pair, C + r0 * ldc, ldc, s);
+  }
+  return rc;
 }
 
 int matmul_device(hipq_weight_t w, const float *A, int64_t M, int64_t lda, float *C, int64_t ldc,
                   hipStream_t s, const Scratch &sc) {
   if (M == 0) return HIPQ_OK;
-  if (wants_tiled(w, M, !sc.fixed)) return matmul_tiled(w, A, M, lda, C, ldc, s, 0, sc);
   if (wants_rows(w, M, !sc.fixed)) return matmul_rows(w, A, M, lda, C, ldc, s, 0, sc);
+  if (wants_tiled(w, M, !sc.fixed)) return matmul_tiled(w, A, M, lda, C, ldc, s, 0, sc);
   if (M == 1 && hipq::gemv_fuses_quantizer(w, A)) return hipq::launch_gemv_fused(w, A, C, s);
   const int is_k = w->dtype != HIPQ_Q4_0;
   void *mem = nullptr;
@@ -905,8 +913,8 @@ int hipq_matmul_multi(int count, const hipq_weight_t *w, const float *A, int64_t
   /* one quantization per distinct activation format among the weights */
   auto klass = [&](const hipq_weight *x) {
     if (x->dtype == HIPQ_Q4_0) return 0;
-    if (wants_tiled(x, M)) return x->dtype == HIPQ_Q4_K ? 3 : 4; /* the two tiled forms differ in their rows' quantizer */
     if (wants_rows(x, M, true)) return 5; /* a few rows of Q4_K on the matrix cores: the row form of the MoE kernels */
+    if (wants_tiled(x, M)) return x->dtype == HIPQ_Q4_K ? 3 : 4; /* the two tiled forms differ in their rows' quantizer */
     return (x->dtype == HIPQ_Q4_K && M > 1) ? 1 : 2;
   };
   {

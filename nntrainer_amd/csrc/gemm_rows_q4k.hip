@@ -293,14 +293,16 @@ namespace hipq {
  * streams its weights at 2.5-4.6 TB/s. */
 bool gemm_rows_q4k_fits(const hipq_weight *w, int64_t M) {
   if (w->dtype != HIPQ_Q4_K || w->expert_tiles || w->K % 256 || 16 * w->K > 0x7fffffff) return false;
-  if (M >= 5 && M <= TC) return w->N >= 1024;
+  /* nine to sixteen rows as two passes (12288 x 4096: 22 us, against 31 us for one 64-row tile of
+   * the prefill GEMM, whose 96 workgroups leave most of the chip idle) */
+  if (M >= 5 && M <= 2 * TC) return w->N >= 1024;
   return (M == 4 && w->N >= 4096) || (M == 3 && w->N >= 8192);
 }
 
 int launch_gemm_rows_q4k(const hipq_weight *w, const QAct *qa, int M, int pair_rows, float *C, int64_t ldc,
                          hipStream_t s) {
-  if (!gemm_rows_q4k_fits(w, M) || qa->K != w->K)
-    return fail(HIPQ_ERR_INVALID_ARGUMENT, "the few-rows Q4_K product takes 3..8 rows");
+  if (M < 1 || M > TC || w->dtype != HIPQ_Q4_K || qa->K != w->K)
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "a pass of the few-rows Q4_K product takes 1..8 rows");
   if (!w->gt_base) return fail(HIPQ_ERR_INVALID_ARGUMENT, "the few-rows Q4_K product needs the weight's tile copy");
   WView v = wview(w);
   v.qs = w->gt_qs;

@@ -227,8 +227,10 @@ int launch_gemm_q4k_multi(int count, const hipq_weight *const *w, const QActTile
 int launch_gemm_q6k(const hipq_weight *w, const QActTiled *qa, int M, float *C, int64_t ldc, hipStream_t s);
 int launch_gemm_q4k(const hipq_weight *w, const QActTiled *qa, int M, float *C,
                     int64_t ldc, hipStream_t s);
-/* gemm_rows_q4k.hip: Q4_K for 3..8 rows on the matrix cores with the reference's bits; qa in the
- * form of launch_quantize_q8_K_rowmma, the weight with its tile copy (ensure_gemm_tiles) */
+/* gemm_rows_q4k.hip: Q4_K for a few rows on the matrix cores with the reference's bits; fits: the row
+ * counts and shapes that should take it (up to 16 rows, in passes of up to 8 for the launcher); qa in
+ * the form of launch_quantize_q8_K_rowmma, the first pair_rows rows under the 4-row quantizer's rule;
+ * the weight with its tile copy (ensure_gemm_tiles) */
 bool gemm_rows_q4k_fits(const hipq_weight *w, int64_t M);
 int launch_gemm_rows_q4k(const hipq_weight *w, const QAct *qa, int M, int pair_rows, float *C, int64_t ldc,
                          hipStream_t s);
