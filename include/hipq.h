@@ -160,6 +160,18 @@ HIPQ_API int hipq_quantize_q8_K(const float *A, int64_t M, int64_t K, int64_t ld
 HIPQ_API int hipq_matmul(hipq_weight_t w, const float *A, int64_t M, int64_t lda,
                          float *C, int64_t ldc, int mem, void *stream);
 
+/** `rows` independent one-row products in one call: row r of C = row r of A . W^T with the bits
+ *  of hipq_matmul(w, A + r * lda, 1, ...). Replaces the loop over batch entries of a decode step,
+ *  FullyConnectedLayer::incremental_forwarding with to - from == 1 (fc_layer.cpp:266-296: one
+ *  input_step.dot(weight, hidden_step) per entry, each an M = 1 product). It differs from
+ *  hipq_matmul with M = rows for Q4_K only, where the reference quantizes rows it multiplies
+ *  together four at a time and sums their sub-block pairs separately; rows of different batch
+ *  entries are never multiplied together there. The rows share one pass over the weights (Q4_K
+ *  against 1024 columns or more: on the matrix cores, gemm_rows_q4k.hip) and, with host memory,
+ *  one transfer each way. */
+HIPQ_API int hipq_matmul_each_row(hipq_weight_t w, const float *A, int64_t rows, int64_t lda,
+                                  float *C, int64_t ldc, int mem, void *stream);
+
 /** hipq_matmul on device buffers for callers that cannot allocate device memory:
  *  code under HIP graph capture, tight serving loops, harnesses that forbid it.
  *  It has no counterpart in the reference. The quantized activations of the call

@@ -20,7 +20,7 @@ DTYPES = {"q4_0": Q4_0, "q4_K": Q4_K, "q6_K": Q6_K}
 SYMBOLS = [
     "hipq_init", "hipq_shutdown", "hipq_last_error", "hipq_version", "hipq_weight_nbytes",
     "hipq_weight_create", "hipq_weight_destroy", "hipq_weight_dims", "hipq_quantize_q8_0",
-    "hipq_quantize_q8_K", "hipq_matmul", "hipq_matmul_noalloc", "hipq_matmul_multi", "hipq_moe_forward",
+    "hipq_quantize_q8_K", "hipq_matmul", "hipq_matmul_each_row", "hipq_matmul_noalloc", "hipq_matmul_multi", "hipq_moe_forward",
     "hipq_moe_forward_ext", "hipq_mlp_swiglu", "hipq_host_alloc", "hipq_host_free", "hipq_stream_release",
     "hipq_quantize_weights", "hipq_file_layout", "hipq_weights_from_file",
 ]
@@ -91,6 +91,7 @@ def lib():
         L.hipq_quantize_q8_0.argtypes = [vp, i64, i64, i64, vp, i32, vp]
         L.hipq_quantize_q8_K.argtypes = [vp, i64, i64, i64, i32, vp, i32, vp]
         L.hipq_matmul.argtypes = [vp, vp, i64, i64, vp, i64, i32, vp]
+        L.hipq_matmul_each_row.argtypes = [vp, vp, i64, i64, vp, i64, i32, vp]
         L.hipq_matmul_noalloc.argtypes = [vp, vp, i64, i64, vp, i64, vp]
         L.hipq_matmul_multi.argtypes = [i32, C.POINTER(vp), vp, i64, i64, C.POINTER(vp),
                                         C.POINTER(i64), i32, vp]
@@ -220,6 +221,11 @@ def quantize_q8_K(a, m, k, out, variant=Q8K_ROW, lda=None, mem=MEM_DEVICE, strea
 
 def matmul(w, a, m, c, lda=None, ldc=None, mem=MEM_DEVICE, stream=None):
     check(lib().hipq_matmul(w.handle, _addr(a), m, lda or w.k, _addr(c), ldc or w.n, mem, stream))
+
+
+def matmul_each_row(w, a, rows, c, lda=None, ldc=None, mem=MEM_DEVICE, stream=None):
+    """`rows` independent one-row products in one call (the bits of `rows` calls of matmul with m = 1)."""
+    check(lib().hipq_matmul_each_row(w.handle, _addr(a), rows, lda or w.k, _addr(c), ldc or w.n, mem, stream))
 
 
 def matmul_noalloc(w, a, m, c, lda=None, ldc=None, stream=None):

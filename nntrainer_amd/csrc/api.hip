@@ -332,18 +332,18 @@ int matmul_tiled(const hipq_weight *w, const float *A, int64_t M, int64_t lda, f
 
 /* Quantize the activations the way the reference does for this weight type. */
 int quantize_for(const hipq_weight *w, const float *A, int64_t M, int64_t lda, const QAct &qa,
-                 hipStream_t s) {
+                 hipStream_t s, bool each_row = false) {
   if (w->dtype == HIPQ_Q4_0) return hipq::launch_quantize_q8_0(A, M, w->K, lda, &qa, nullptr, s);
-  const int64_t mat_rows = (w->dtype == HIPQ_Q4_K && M > 1) ? (M / 4) * 4 : 0;
+  const int64_t mat_rows = (w->dtype == HIPQ_Q4_K && M > 1 && !each_row) ? (M / 4) * 4 : 0;
   return hipq::launch_quantize_q8_K(A, M, w->K, lda, mat_rows, &qa, nullptr, s);
 }
 
 /* Block-dot stage on already quantized activations. */
 int multiply(const hipq_weight *w, const QAct &qa, int64_t M, float *C, int64_t ldc,
-             hipStream_t s) {
+             hipStream_t s, bool each_row = false) {
   const int is_k = w->dtype != HIPQ_Q4_0;
   /* rows the reference sends through its 4-row GEMM kernel (Q4_K, M > 1) */
-  const int pair_rows = (w->dtype == HIPQ_Q4_K && M > 1) ? (int)((M / 4) * 4) : 0;
+  const int pair_rows = (w->dtype == HIPQ_Q4_K && M > 1 && !each_row) ? (int)((M / 4) * 4) : 0;
   if (M <= 8) return hipq::launch_gemv(w, &qa, (int)M, pair_rows, C, ldc, s);
   if (w->dtype == HIPQ_Q4_0 && w->K % 256 == 0) return hipq::launch_gemm(w, &qa, (int)M, C, ldc, s);
   for (int64_t r0 = 0; r0 < M; r0 += 8) {
@@ -395,12 +395,12 @@ bool wants_rows(const hipq_weight *w, int64_t M, bool may_allocate) {
 }
 
 int matmul_rows(const hipq_weight *w, const float *A, int64_t M, int64_t lda, float *C, int64_t ldc,
-                hipStream_t s, int phase, const Scratch &sc) {
+                hipStream_t s, int phase, const Scratch &sc, bool each_row = false) {
   void *mem = nullptr;
   int rc = sc.get(qact_bytes(1, M, w->K), &mem);
   if (rc) return rc;
   QAct qa = qact_carve(1, mem, M, w->K);
-  const int64_t mat_rows = (M / 4) * 4; /* the rows the reference quantizes four at a time */
+  const int64_t mat_rows = each_row ? 0 : (M / 4) * 4; /* the rows the reference quantizes four at a time */
   if (phase != 1) rc = hipq::launch_quantize_q8_K_rowmma(A, M, w->K, lda, &qa, s, mat_rows);
   if (rc || phase == 2) return rc;
   if (!w->gt_base && (rc = hipq::ensure_gemm_tiles(const_cast<hipq_weight *>(w)))) return rc;
@@ -413,20 +413,31 @@ int matmul_rows(const hipq_weight *w, const float *A, int64_t M, int64_t lda, fl
   return rc;
 }
 
+/* each_row: every row as a product of its own with M = 1 (the bits of M separate calls): for Q4_0
+ * and Q6_K that is what up to 16 rows give anyway; Q4_K drops the 4-row quantizer and the pairwise
+ * sums the reference applies to rows it multiplies together. The caller passes at most 16 rows. */
 int matmul_device(hipq_weight_t w, const float *A, int64_t M, int64_t lda, float *C, int64_t ldc,
-                  hipStream_t s, const Scratch &sc) {
+                  hipStream_t s, const Scratch &sc, bool each_row = false) {
   if (M == 0) return HIPQ_OK;
-  if (wants_rows(w, M, !sc.fixed)) return matmul_rows(w, A, M, lda, C, ldc, s, 0, sc);
-  if (wants_tiled(w, M, !sc.fixed)) return matmul_tiled(w, A, M, lda, C, ldc, s, 0, sc);
+  if (wants_rows(w, M, !sc.fixed)) return matmul_rows(w, A, M, lda, C, ldc, s, 0, sc, each_row);
+  if (!each_row && wants_tiled(w, M, !sc.fixed)) return matmul_tiled(w, A, M, lda, C, ldc, s, 0, sc);
   if (M == 1 && hipq::gemv_fuses_quantizer(w, A)) return hipq::launch_gemv_fused(w, A, C, s);
   const int is_k = w->dtype != HIPQ_Q4_0;
   void *mem = nullptr;
   int rc = sc.get(qact_bytes(is_k, M, w->K), &mem);
   if (rc) return rc;
   QAct qa = qact_carve(is_k, mem, M, w->K);
-  rc = quantize_for(w, A, M, lda, qa, s);
+  rc = quantize_for(w, A, M, lda, qa, s, each_row);
   if (rc) return rc;
-  return multiply(w, qa, M, C, ldc, s);
+  if (each_row && w->dtype == HIPQ_Q4_K && M > 8) { /* nine to sixteen rows of a small matrix: two GEMV passes */
+    for (int64_t r0 = 0; r0 < M && !rc; r0 += 8) {
+      const int64_t rows = (M - r0) < 8 ? (M - r0) : 8;
+      const QAct sub = qact_rows(qa, 1, r0, rows);
+      rc = hipq::launch_gemv(w, &sub, (int)rows, 0, C + r0 * ldc, ldc, s);
+    }
+    return rc;
+  }
+  return multiply(w, qa, M, C, ldc, s, each_row);
 }
 
 struct DevBuf {
@@ -813,6 +824,34 @@ int hipq_matmul(hipq_weight_t w, const float *A, int64_t M, int64_t lda, float *
   if ((rc = stage_copy(true, dA, (void *)A, (size_t)lda * 4, (size_t)w->K * 4, (size_t)M, s))) return rc;
   if ((rc = matmul_device(w, dA, M, w->K, dC, w->N, s, sc))) return rc;
   return stage_copy(false, dC, C, (size_t)ldc * 4, (size_t)w->N * 4, (size_t)M, s);
+}
+
+int hipq_matmul_each_row(hipq_weight_t w, const float *A, int64_t rows, int64_t lda, float *C, int64_t ldc,
+                         int mem, void *stream) {
+  int rc = require_ready();
+  if (rc) return rc;
+  if ((rc = check_matmul_args(w, A, rows, lda, C, ldc))) return rc;
+  if (mem != HIPQ_MEM_DEVICE && mem != HIPQ_MEM_HOST) return fail(HIPQ_ERR_INVALID_ARGUMENT, "unknown mem kind %d", mem);
+  if (rows == 0) return HIPQ_OK;
+  hipStream_t s = (hipStream_t)stream;
+  EnqueueGuard eg(enqueue_lock(s));
+  const Scratch sc{false, s};
+  const float *dA = A;
+  float *dC = C;
+  int64_t a_ld = lda, c_ld = ldc;
+  if (mem == HIPQ_MEM_HOST) {
+    const size_t a_bytes = ((size_t)rows * w->K * 4 + 255) & ~(size_t)255, c_bytes = (size_t)rows * w->N * 4;
+    void *io = nullptr;
+    if ((rc = io_buffer(s, a_bytes + c_bytes, &io))) return rc;
+    dA = (const float *)io, dC = (float *)((char *)io + a_bytes), a_ld = w->K, c_ld = w->N;
+    if ((rc = stage_copy(true, (void *)dA, (void *)A, (size_t)lda * 4, (size_t)w->K * 4, (size_t)rows, s))) return rc;
+  }
+  for (int64_t r0 = 0; r0 < rows && !rc; r0 += 16) { /* sixteen rows a step: the row counts that keep the M = 1 bits */
+    const int64_t n = (rows - r0) < 16 ? (rows - r0) : 16;
+    rc = matmul_device(w, dA + r0 * a_ld, n, a_ld, dC + r0 * c_ld, c_ld, s, sc, true);
+  }
+  if (rc || mem == HIPQ_MEM_DEVICE) return rc;
+  return stage_copy(false, dC, C, (size_t)ldc * 4, (size_t)w->N * 4, (size_t)rows, s);
 }
 
 int hipq_matmul_noalloc(hipq_weight_t w, const float *A, int64_t M, int64_t lda, float *C,

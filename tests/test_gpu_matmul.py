@@ -518,3 +518,44 @@ def test_bad_arguments_are_reported(hipq):
     blocks = np.zeros(capi.weight_nbytes("q4_0", 12, 64), np.uint8)
     with pytest.raises(capi.HipqError):
         capi.Weight("q4_0", 12, 64, blocks, layout=capi.LAYOUT_X8)  # N % 8 != 0 (repack returns -1)
+
+
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("rows,n,k", [(8, 1100, 1024), (5, 512, 768), (12, 2048, 512), (16, 300, 256),
+                                      (37, 1056, 1024), (3, 8200, 512), (1, 640, 256)])
+def test_matmul_each_row_has_the_bits_of_single_row_products(hipq, cr, kind, rows, n, k):
+    """hipq_matmul_each_row: the rows of a batch of decode steps against one weight in one call, every
+    row with the bits of its own M = 1 product (the reference's loop over batch entries). For Q4_K
+    that differs from hipq_matmul with M = rows (no 4-row quantizer, no pairwise sums): row 1 holds
+    +amax before -amax, where the two quantizers round differently. Large and small matrices (the
+    matrix-core kernel and the GEMV engine), more than 16 rows (several steps), strided rows, and
+    host memory."""
+    import gpu_util as gu
+    import torch
+    blocks = _weights(cr, kind, n, k, seed=500 + n)
+    a = synth.normal(501 + rows + k, (rows, k))
+    if rows > 1:
+        a[1, 3] = 7.25
+        a[1, 11] = -7.25
+    ref = np.concatenate([cr.gemm(cr.oracle(), kind, a[r:r + 1], blocks, n) for r in range(rows)], axis=0)
+    w = capi.Weight(kind, n, k, blocks)
+    try:
+        lda, ldc = k + 64, n + 32
+        da = torch.zeros((rows, lda), device="cuda")
+        da[:, :k] = gu.dev(a)
+        dc = torch.full((rows, ldc), float("nan"), device="cuda")
+        capi.matmul_each_row(w, da, rows, dc, lda=lda, ldc=ldc, stream=gu.stream())
+        torch.cuda.synchronize()
+        got = dc[:, :n].cpu().numpy()
+        assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), \
+            "%d of %d outputs differ in bits" % ((got.view(np.uint32) != ref.view(np.uint32)).sum(), got.size)
+        assert torch.isnan(dc[:, n:]).all(), "the call wrote between the rows of C"
+        host = np.full((rows, n), np.nan, np.float32)
+        capi.matmul_each_row(w, a, rows, host, mem=capi.MEM_HOST, stream=gu.stream())
+        assert np.array_equal(host.view(np.uint32), ref.view(np.uint32))
+        single = gu.gpu_matmul(w, a[1:2]) if rows > 1 else None
+        if single is not None:
+            assert np.array_equal(single.view(np.uint32), ref[1:2].view(np.uint32))
+    finally:
+        w.destroy()
+
