@@ -132,6 +132,32 @@ void FullyConnectedLayerHip::incremental_forwarding(RunLayerContext &context, un
    * for batch 1, every LLM call, that is offset 0 either way. The same rule here, so that a
    * graph that runs on both engines sees the same numbers; where it would leave the input
    * tensor (the reference then reads past its end) the call is refused instead. */
+  /* A decode step of a batch: one row per entry, the entries hidden_dim.getFeatureLen() apart on
+   * both sides. The reference multiplies them one by one (each an M = 1 product); the same
+   * products go out as ONE call that keeps each row's bits (hipq_matmul_each_row): one pass over
+   * the weights and one transfer each way instead of one per entry. */
+  const size_t stride = hidden_dim.getFeatureLen();
+  if (to - from == 1 && hidden_.batch() > 1 && stride >= input_dim.width() && stride >= hidden_dim.width() &&
+      (size_t)(hidden_.batch() - 1) * stride + input_dim.width() <= input_.size()) {
+    const int64_t K = input_dim.width(), N = weight.width();
+    NNTR_THROW_IF((int64_t)weight.height() != K, std::invalid_argument)
+      << "weight height " << weight.height() << " does not match input width " << K;
+    NNTR_THROW_IF((int64_t)hidden_dim.width() != N, std::invalid_argument)
+      << "output width " << hidden_dim.width() << " does not match unit " << N;
+    const int dtype = hipq_dtype_of(weight.getDataType());
+    NNTR_THROW_IF(dtype < 0, std::invalid_argument) << "Error: unsupported datatype";
+    const hipq_host::WeightSpec spec{dtype, hipq_host::framework_layout(dtype), N, K};
+    hipq_host::matmul_each_row(hipq_host::global_cache(), weight.getData<uint8_t>(), spec, input_.getData<float>(),
+                               hidden_.batch(), (int64_t)stride, hidden_.getData<float>(), (int64_t)stride);
+    if (!disable_bias) {
+      Tensor &bias = context.getWeight(weight_idx[FCParams::bias]);
+      for (unsigned int b = 0; b < hidden_.batch(); ++b) {
+        Tensor hidden_step = hidden_.getSharedDataTensor(hidden_step_dim, b * stride, true);
+        hidden_step.add_i(bias);
+      }
+    }
+    return;
+  }
   for (unsigned int b = 0; b < hidden_.batch(); ++b) {
     const size_t in_off = (size_t)b * hidden_dim.getFeatureLen();
     NNTR_THROW_IF(in_off + (size_t)(to - from) * input_dim.width() > input_.size(), std::invalid_argument)

@@ -132,6 +132,13 @@ void matmul(WeightCache &cache, const void *weight_bytes, const WeightSpec &spec
   check(hipq_matmul(w, A, M, lda, C, ldc, HIPQ_MEM_HOST, nullptr), "hipq_matmul");
 }
 
+void matmul_each_row(WeightCache &cache, const void *weight_bytes, const WeightSpec &spec, const float *A,
+                     int64_t rows, int64_t lda, float *C, int64_t ldc) {
+  require_runtime();
+  hipq_weight_t w = cache.get(weight_bytes, spec);
+  check(hipq_matmul_each_row(w, A, rows, lda, C, ldc, HIPQ_MEM_HOST, nullptr), "hipq_matmul_each_row");
+}
+
 void matmul_multi(WeightCache &cache, const std::vector<const void *> &weight_bytes,
                   const std::vector<WeightSpec> &specs, const float *A, int64_t M, int64_t lda,
                   const std::vector<float *> &C) {

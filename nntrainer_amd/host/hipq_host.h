@@ -106,6 +106,11 @@ WeightCache &global_cache();
 void matmul(WeightCache &cache, const void *weight_bytes, const WeightSpec &spec,
             const float *A, int64_t M, int64_t lda, float *C, int64_t ldc);
 
+/** `rows` one-row products against one weight in one call, each with the bits of matmul with
+ *  M = 1: the batch entries of a decode step (fc_layer.cpp:266-296 loops over them) */
+void matmul_each_row(WeightCache &cache, const void *weight_bytes, const WeightSpec &spec,
+                     const float *A, int64_t rows, int64_t lda, float *C, int64_t ldc);
+
 /** one activation against several weights (shared activation quantization),
  *  the vector overload of dot (float_tensor.cpp:724-798) */
 void matmul_multi(WeightCache &cache, const std::vector<const void *> &weight_bytes,

@@ -84,6 +84,31 @@ def test_fc_incremental_forwarding_prefill_then_decode(cr, tmp_path):
             assert np.all(got[b, rows:] == -12345.0)
 
 
+@pytest.mark.parametrize("kind,k,n", [("q4_K", 1024, 1056), ("q4_K", 512, 256), ("q6_K", 512, 384), ("q4_0", 512, 320)])
+def test_fc_decode_step_of_a_batch_is_one_call_with_each_entry_s_bits(cr, tmp_path, kind, k, n):
+    """A decode step (to - from == 1) of a batch of eight: the layer sends the eight rows as one
+    hipq_matmul_each_row call; every entry carries the bits of the M = 1 product the reference
+    computes for it (fc_layer.cpp:266-296), with the reference's offset rule for the input, and
+    the rest of the output is left alone."""
+    batch, height = 8, 4
+    w32 = synth.normal(7350, (n, k), 0.02)
+    blocks, fw = _framework_bytes(cr, kind, w32, n, k)
+    x = synth.normal(7351, (batch, height, k))
+    x.reshape(-1)[1 * height * n + 3] = 6.5   # entry 1: +amax before -amax (the quantizers' sign rules)
+    x.reshape(-1)[1 * height * n + 9] = -6.5
+    fw.tofile(tmp_path / "w.bin")
+    x.tofile(tmp_path / "x.bin")
+    if (batch - 1) * height * n + k > x.size:
+        pytest.skip("the reference's offset rule leaves the input tensor")
+    _run(["fc", kind, k, n, batch, height, 3, 4, tmp_path / "w.bin", tmp_path / "x.bin", "-", tmp_path / "y.bin"])
+    got = np.fromfile(tmp_path / "y.bin", np.float32).reshape(batch, height, n)
+    for b in range(batch):
+        xin = x.reshape(-1)[b * height * n:][:k].reshape(1, k)
+        ref = cr.gemm(cr.oracle(), kind, xin, blocks, n)
+        assert np.array_equal(got[b, :1].view(np.uint32), ref.view(np.uint32)), (kind, b)
+        assert np.all(got[b, 1:] == -12345.0)
+
+
 def test_fc_decode_row_is_bit_identical_to_oracle(cr, tmp_path):
     """M = 1 goes through the GEMV engine, which reproduces the reference's fp32
     evaluation order: equal bits, not just within tolerance."""
