@@ -300,11 +300,19 @@ QAct qact_rows(const QAct &a, int is_k, int64_t r0, int64_t rows) {
 /* The prefill GEMMs of the K-formats take their activations in the tiled form. The Q4_K one
  * addresses the weight planes with 32-bit byte offsets where it has no tile copy; the Q6_K
  * one reads the tile copy only, which the entry point that may not allocate cannot build
- * (such a call then walks the rows eight at a time through the GEMV engine, as every call with
- * up to 16 rows does: two or three passes over the weights cost what a 64-row tile does, and
- * keep the reference's bits). */
+ * (such a call then walks the rows eight at a time through the GEMV engine, as calls with few
+ * rows do, and keeps the reference's bits). */
 bool wants_tiled(const hipq_weight *w, int64_t M, bool may_allocate = true) {
-  if (w->dtype == HIPQ_Q6_K) return M > 16 && (w->gt_base || may_allocate);
+  if (w->dtype == HIPQ_Q6_K) {
+    /* The GEMV engine keeps the reference's bits but costs a pass over the weights per eight rows
+     * and about 1e-7 us per weight and row on the vector ALU; the matrix-core GEMM costs one 64-row
+     * tile whatever the row count (35 us, or 2e-7 us per weight). Measured, us, engine against GEMM:
+     * 151936 x 4096 with 2 / 4 / 8 / 16 rows 115 / 192 / 441 / 847 against 130; 12288 x 4096 with
+     * 8 / 16 rows 42 / 80 against 36; 4096 x 4096 with 16 rows 34 against 35. */
+    const int64_t weights = w->N * w->K;
+    const int64_t engine_rows = weights >= (int64_t(1) << 28) ? 2 : weights >= (int64_t(1) << 25) ? 8 : 16;
+    return M > engine_rows && (w->gt_base || may_allocate);
+  }
   /* up to 16 rows of a Q4_K matrix of 1024 columns or more take the few-rows kernel (wants_rows) */
   if (hipq::gemm_rows_q4k_fits(w, M) && (w->gt_base || may_allocate)) return false;
   return w->dtype == HIPQ_Q4_K && M > 8 && w->N * (w->K / 2) < (int64_t(1) << 32);

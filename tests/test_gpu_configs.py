@@ -93,6 +93,18 @@ def test_c3_q6_K_lm_head_argmax(hipq, cr):
     w.destroy()
     assert int(np.argmax(got)) == int(np.argmax(ref))  # first maximum wins on both sides
     assert np.array_equal(got.view(np.uint32), ref.view(np.uint32))
+    # a batch of four rows against the same weight: from 2^28 weights on more than two rows run on
+    # the matrix cores (the GEMV engine would take 1.5 times as long for four rows and 6.5 times for
+    # sixteen), within 1e-4 of the reference; two rows keep its bits
+    a4 = synth.normal(2, (4, k), 1.0, first=n * k + k)
+    ref4 = cr.gemm(cr.oracle(), "q6_K", a4, blocks, n)
+    w = capi.Weight("q6_K", n, k, blocks)
+    got4 = gu.gpu_matmul(w, a4)
+    got2 = gu.gpu_matmul(w, a4[:2])
+    w.destroy()
+    assert gu.rel_err(got4, ref4) <= TOL, gu.rel_err(got4, ref4)
+    assert np.array_equal(np.argmax(got4, axis=1), np.argmax(ref4, axis=1))
+    assert np.array_equal(got2.view(np.uint32), ref4[:2].view(np.uint32))
 
 
 def test_c4_moe_block(hipq, cr):

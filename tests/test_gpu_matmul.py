@@ -124,12 +124,14 @@ def test_gemm_matches_oracle(hipq, cr, kind, m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(17, 128, 256), (33, 200, 768), (64, 96, 1024), (100, 1000, 512),
-                                   (512, 4096, 4096), (1100, 8192, 512)])
+                                   (512, 4096, 4096), (1100, 8192, 512), (12, 8192, 4096)])
 def test_q6_K_gemm_matches_oracle(hipq, cr, m, n, k):
-    """The Q6_K prefill product on the matrix cores (M > 8): one and three super-blocks per row,
+    """The Q6_K prefill product on the matrix cores: one and three super-blocks per row,
     N not a multiple of the 32-row weight tiles or of the 128-column workgroup tiles, M not a
-    multiple of the tile heights, a shape that takes the 128-row tiles, and the size of a
-    Q6_K FC of a 4096-wide model. Rows up to eight keep the GEMV engine and the reference's bits."""
+    multiple of the tile heights, a shape that takes the 128-row tiles, the size of a
+    Q6_K FC of a 4096-wide model, and twelve rows against a matrix of 2^25 weights (from that
+    size on more than eight rows leave the GEMV engine). Rows up to eight keep the GEMV engine
+    and the reference's bits."""
     import gpu_util as gu
     blocks = _weights(cr, "q6_K", n, k, seed=61 + m)
     a = synth.normal(600 + m, (m, k))
