@@ -182,7 +182,10 @@ HIPQ_API int hipq_matmul_each_row(hipq_weight_t w, const float *A, int64_t rows,
  *  (M * K beyond about 7.8 million values for Q6_K weights, 14 million for Q4_0
  *  and Q4_K) returns HIPQ_ERR_NOT_SUPPORTED. The call performs no device
  *  allocation and no free and enqueues the same kernels as hipq_matmul, so
- *  results are the same bits. All calls on a GPU share that one array: calls
+ *  results are the same bits (one exception: a Q4_K product of up to 128 rows that
+ *  hipq_matmul forms in parts of K takes whole rows here when the parts' partial sums
+ *  do not fit the array as well; it then agrees to 1e-4 like every matrix-core
+ *  product). All calls on a GPU share that one array: calls
  *  whose kernels may overlap on the device (different streams) race on it. */
 HIPQ_API int hipq_matmul_noalloc(hipq_weight_t w, const float *A, int64_t M, int64_t lda,
                                  float *C, int64_t ldc, void *stream);

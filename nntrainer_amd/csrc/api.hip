@@ -379,9 +379,15 @@ int check_matmul_args(hipq_weight_t w, const float *A, int64_t M, int64_t lda, c
 int matmul_tiled(const hipq_weight *w, const float *A, int64_t M, int64_t lda, float *C, int64_t ldc,
                  hipStream_t s, int phase, const Scratch &sc) {
   void *mem = nullptr;
-  int rc = sc.get(qact_tiled_bytes(M, w->K), &mem);
+  /* room for the partial products of a product with few tiles behind the activations (the fixed
+   * scratch of the allocation-free entry point may be too small for them: then none) */
+  const size_t act_bytes = (qact_tiled_bytes(M, w->K) + 255) & ~(size_t)255;
+  size_t part_bytes = w->dtype == HIPQ_Q4_K ? hipq::gemm_q4k_split_bytes(w, M) : 0;
+  if (sc.fixed && act_bytes + part_bytes > NOALLOC_SCRATCH_BYTES) part_bytes = 0;
+  int rc = sc.get(act_bytes + part_bytes, &mem);
   if (rc) return rc;
   QActTiled qa = qact_tiled_carve(mem, M, w->K);
+  void *partials = part_bytes ? (char *)mem + act_bytes : nullptr;
   /* rows below the last multiple of four follow the 4-row quantizer for Q4_K (what the
    * reference's GEMM wrapper calls for them); its Q6_K path quantizes row by row */
   const int64_t mat_rows = w->dtype == HIPQ_Q4_K ? (M / 4) * 4 : 0;
@@ -391,7 +397,8 @@ int matmul_tiled(const hipq_weight *w, const float *A, int64_t M, int64_t lda, f
    * prefill product; the entry point that may not allocate reads the planes until it exists. */
   if (!w->gt_base && !sc.fixed && (rc = hipq::ensure_gemm_tiles(const_cast<hipq_weight *>(w)))) return rc;
   if (w->dtype == HIPQ_Q6_K) return hipq::launch_gemm_q6k(w, &qa, (int)M, C, ldc, s);
-  return hipq::launch_gemm_q4k(w, &qa, (int)M, C, ldc, s);
+  /* the copy may have been made just now: parts are used from the next call on */
+  return hipq::launch_gemm_q4k(w, &qa, (int)M, C, ldc, s, partials);
 }
 
 /* Three to eight rows of a large Q4_K matrix run on the matrix cores (gemm_rows_q4k.hip, the

@@ -215,15 +215,22 @@ __device__ __forceinline__ void epilogue(const Smem<TM> &sm, int buf, const uint
 }
 
 /* the tile (mt, nt) of one weight's product */
-template <int TM, bool TILES>
+/* KSPLIT: the tile's sum over super-blocks sb0 .. sb0 + nsbl - 1 only (a partial product; the
+ * callers add the parts). Everything the loop reads is addressed relative to its first
+ * super-block, so the part's first one becomes that by moving the bases. */
+template <int TM, bool TILES, bool KSPLIT = false>
 __device__ __forceinline__ void gemm_q4k_tile(const WView &w, const int8_t *__restrict__ qt,
                                               const uint16_t *__restrict__ amin, const float *__restrict__ dAt, int M,
-                                              int mt, int nt, float *__restrict__ C, int64_t ldc) {
+                                              int mt, int nt, float *__restrict__ C, int64_t ldc, int sb0 = 0,
+                                              int nsb_part = 0) {
+  static_assert(!KSPLIT || TILES, "partial products read the tile copy");
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   Smem<TM> &sm = *reinterpret_cast<Smem<TM> *>(smem_raw);
   constexpr int BM = 32 * TM;
   const int m0 = mt * BM, n0 = nt * BN;
-  const int nsb = w.K >> 8;
+  const int nsb_all = w.K >> 8;
+  const int first = KSPLIT ? sb0 : 0;
+  const int nsb = KSPLIT ? nsb_part : nsb_all; /* the super-blocks this call walks */
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const int i32 = lane & 31, g = lane >> 5;
@@ -231,21 +238,21 @@ __device__ __forceinline__ void gemm_q4k_tile(const WView &w, const int8_t *__re
   Src sr;
   /* the quantizer tiles by 128 rows: a 64-row tile is half mt & 1 of quantizer tile mt / 2 */
   const int qt128 = TM == 2 ? mt >> 1 : mt, hrow = TM == 2 ? mt & 1 : 0;
-  sr.qt = make_rsrc(qt + (size_t)qt128 * (2 * nsb) * QSTAGE + hrow * 8192, (uint32_t)(2 * nsb) * QSTAGE);
-  sr.amin = make_rsrc(amin + ((size_t)qt128 * nsb * 128 + hrow * 64) * 16, (uint32_t)nsb * 128 * 32);
-  sr.dAt = make_rsrc(dAt + (size_t)qt128 * nsb * 128 + hrow * 64, (uint32_t)nsb * 128 * 4);
+  sr.qt = make_rsrc(qt + ((size_t)qt128 * (2 * nsb_all) + 2 * first) * QSTAGE + hrow * 8192, (uint32_t)(2 * nsb) * QSTAGE);
+  sr.amin = make_rsrc(amin + (((size_t)qt128 * nsb_all + first) * 128 + hrow * 64) * 16, (uint32_t)nsb * 128 * 32);
+  sr.dAt = make_rsrc(dAt + ((size_t)qt128 * nsb_all + first) * 128 + hrow * 64, (uint32_t)nsb * 128 * 4);
   const int n = min(n0 + wave * 32 + i32, (int)w.N - 1);
   constexpr int HSTRIDE = TILES ? 32 : 1; /* uint4 between a column's consecutive super-block headers */
   if (TILES) {
     /* the copy pads N to 32 rows: a wavefront whose columns start below N has its tile */
     const size_t wt = (size_t)(min(n0 + wave * 32, (int)w.N - 1) >> 5);
-    sr.rq = make_rsrc(w.qs + wt * nsb * 4096, (uint32_t)nsb * 4096);
-    sr.rh = make_rsrc(w.hdr + wt * nsb * 512, (uint32_t)nsb * 512);
+    sr.rq = make_rsrc(w.qs + (wt * nsb_all + first) * 4096, (uint32_t)nsb * 4096);
+    sr.rh = make_rsrc(w.hdr + (wt * nsb_all + first) * 512, (uint32_t)nsb * 512);
     sr.wq = nullptr;
     sr.whd = nullptr;
   } else {
     sr.wq = (const uint4 *)(w.qs + (size_t)n * (w.K >> 1) + g * 64);
-    sr.whd = (const uint4 *)w.hdr + (size_t)n * nsb;
+    sr.whd = (const uint4 *)w.hdr + (size_t)n * nsb_all;
   }
   sr.wave = wave;
   sr.lane = lane;
@@ -326,6 +333,37 @@ __global__ __launch_bounds__(NT, TM == 2 ? 3 : 2) void gemm_q4k_kernel(WView w, 
   const int mt = qd % mtiles, nt = (qd / mtiles) * 8 + xcd;
   if (nt >= ntiles) return; /* uniform per workgroup */
   gemm_q4k_tile<TM, TILES>(w, qt, amin, dAt, M, mt, nt, C, ldc);
+}
+
+/* Few tiles (up to 64 rows against a matrix of a few thousand columns make under a hundred
+ * workgroups, each walking all of K: 31 us at 12288 x 4096 whatever the row count): blockIdx.y
+ * takes a part of K and writes its partial product to part[y]; split_sum_kernel adds the parts
+ * in ascending order. */
+__global__ __launch_bounds__(NT, 3) void gemm_q4k_split_kernel(WView w, const int8_t *__restrict__ qt,
+                                                               const uint16_t *__restrict__ amin,
+                                                               const float *__restrict__ dAt, int M, int mtiles,
+                                                               int ntiles, int sb_per_part, float *__restrict__ part,
+                                                               int64_t part_stride) {
+  const int id = blockIdx.x;
+  const int xcd = id & 7, qd = id >> 3;
+  const int mt = qd % mtiles, nt = (qd / mtiles) * 8 + xcd;
+  if (nt >= ntiles) return; /* uniform per workgroup */
+  const int sb0 = blockIdx.y * sb_per_part;
+  const int n = min(sb_per_part, (w.K >> 8) - sb0);
+  gemm_q4k_tile<2, true, true>(w, qt, amin, dAt, M, mt, nt, part + (int64_t)blockIdx.y * part_stride, w.N, sb0, n);
+}
+
+__global__ __launch_bounds__(256) void split_sum_kernel(const float *__restrict__ part, int parts, int64_t part_stride,
+                                                        int M, int N, float *__restrict__ C, int64_t ldc) {
+  const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4; /* N % 4 == 0 */
+  if (i >= (int64_t)M * N) return;
+  const int m = (int)(i / N), n = (int)(i - (int64_t)m * N);
+  float4 v = *(const float4 *)(part + i);
+  for (int p = 1; p < parts; ++p) {
+    const float4 u = *(const float4 *)(part + p * part_stride + i);
+    v.x += u.x, v.y += u.y, v.z += u.z, v.w += u.w;
+  }
+  *(float4 *)(C + (int64_t)m * ldc + n) = v;
 }
 
 /* Up to four weights of one K (each with its tile copy) against the same activations as ONE
@@ -417,9 +455,45 @@ int launch_gemm_q4k_multi(int count, const hipq_weight *const *w, const QActTile
   return HIPQ_OK;
 }
 
-int launch_gemm_q4k(const hipq_weight *w, const QActTiled *qa, int M, float *C, int64_t ldc, hipStream_t s) {
+/* Parts of K for a product whose 64-row tiles would leave most of the chip idle (0: none), and
+ * the bytes of partial products they need. */
+int gemm_q4k_split_parts(const hipq_weight *w, int64_t M) {
+  if (w->dtype != HIPQ_Q4_K || !w->gt_base || (w->N & 3)) return 0;
+  const int64_t tiles = ((M + 63) / 64) * ((w->N + BN - 1) / BN), nsb = w->K / 256;
+  /* measured at 12288 x 4096 (us, whole K a workgroup -> parts): 17..64 rows 31 -> 17-20, 128 rows
+   * 33 -> 28; with more than 192 tiles the parts cost what they gain (256 rows 39.4 -> 40.8) */
+  if (tiles > 192 || nsb < 8) return 0;
+  int parts = (int)(768 / tiles); /* three workgroups a CU */
+  if (parts > 8) parts = 8;
+  if (parts > nsb / 4) parts = (int)(nsb / 4);
+  return parts >= 2 ? parts : 0;
+}
+size_t gemm_q4k_split_bytes(const hipq_weight *w, int64_t M) {
+  return (size_t)gemm_q4k_split_parts(w, M) * (size_t)M * (size_t)w->N * 4;
+}
+
+int launch_gemm_q4k(const hipq_weight *w, const QActTiled *qa, int M, float *C, int64_t ldc, hipStream_t s,
+                    void *partials) {
   if ((M + 127) / 128 != qa->mtiles || qa->K != w->K)
     return fail(HIPQ_ERR_INVALID_ARGUMENT, "tiled activations do not match the matmul shape");
+  const int parts = partials ? gemm_q4k_split_parts(w, M) : 0;
+  if (parts && !(ldc & 3) && !((uintptr_t)C & 15)) {
+    const int nsb = (int)(w->K / 256), per = (nsb + parts - 1) / parts;
+    const int mtiles = (M + 63) / 64, ntiles = (int)((w->N + BN - 1) / BN), ngroups = (ntiles + 7) / 8;
+    const int64_t stride = (int64_t)M * w->N;
+    WView v = wview(w);
+    v.qs = w->gt_qs;
+    v.hdr = w->gt_hdr;
+    launch_kernel(gemm_q4k_split_kernel, dim3((unsigned)(mtiles * ngroups * 8), (unsigned)((nsb + per - 1) / per)),
+                  dim3(NT), sizeof(Smem<2>), s, v, (const int8_t *)qa->qt, (const uint16_t *)qa->amin,
+                  (const float *)qa->dAt, M, mtiles, ntiles, per, (float *)partials, stride);
+    HIPQ_HIP(hipGetLastError());
+    const int64_t quads = stride / 4;
+    hipLaunchKernelGGL(split_sum_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s,
+                       (const float *)partials, (nsb + per - 1) / per, stride, M, (int)w->N, C, ldc);
+    HIPQ_HIP(hipGetLastError());
+    return HIPQ_OK;
+  }
   /* 128-row tiles do a fifth more work per CU and time (the weight expansion is
    * shared by twice the rows) but only two workgroups fit a CU: 512 tiles per round
    * against 768 of the 64-row kind. Pick by the number of rounds. */

@@ -225,8 +225,11 @@ int launch_gemm_multi(int count, const hipq_weight *const *w, const QAct *qa, in
 int launch_gemm_q4k_multi(int count, const hipq_weight *const *w, const QActTiled *qa, int M, float *const *C,
                           const int64_t *ldc, hipStream_t s);
 int launch_gemm_q6k(const hipq_weight *w, const QActTiled *qa, int M, float *C, int64_t ldc, hipStream_t s);
+/* partials: gemm_q4k_split_bytes(w, M) bytes of device memory (or null): with few tiles the product
+ * is formed in parts of K that run side by side and are then added */
 int launch_gemm_q4k(const hipq_weight *w, const QActTiled *qa, int M, float *C,
-                    int64_t ldc, hipStream_t s);
+                    int64_t ldc, hipStream_t s, void *partials = nullptr);
+size_t gemm_q4k_split_bytes(const hipq_weight *w, int64_t M);
 /* gemm_rows_q4k.hip: Q4_K for a few rows on the matrix cores with the reference's bits; fits: the row
  * counts and shapes that should take it (up to 16 rows, in passes of up to 8 for the launcher); qa in
  * the form of launch_quantize_q8_K_rowmma, the first pair_rows rows under the 4-row quantizer's rule;

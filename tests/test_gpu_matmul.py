@@ -177,6 +177,41 @@ def test_gemm_random_shapes_all_formats(hipq, cr):
             assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), (kind, m, n, k)
 
 
+@pytest.mark.parametrize("m,n,k", [(17, 512, 2048), (40, 1000, 2304), (64, 4100, 4096), (100, 640, 3072),
+                                   (128, 1536, 2048), (33, 1001, 2048)])
+def test_q4_K_gemm_in_parts_of_k(hipq, cr, m, n, k):
+    """Few tiles (up to 128 rows against a few thousand columns): once the weight has its tile copy
+    the Q4_K prefill product is formed in parts of K that run side by side and are added in
+    ascending order. The first call (no copy yet: whole K per workgroup) and the following ones
+    (parts; nine super-blocks split 5 + 4, sixteen into four and eight parts) both within 1e-4 of
+    the reference; a strided output keeps its padding; N not a multiple of four takes no parts."""
+    import gpu_util as gu
+    import torch
+    blocks = _weights(cr, "q4_K", n, k, seed=330 + m)
+    a = synth.normal(331 + m, (m, k))
+    ref = cr.gemm(cr.oracle(), "q4_K", a, blocks, n)
+    w = capi.Weight("q4_K", n, k, blocks)
+    try:
+        first = gu.gpu_matmul(w, a)
+        assert gu.rel_err(first, ref) <= gu.TOL, gu.rel_err(first, ref)
+        ldc = n + 12
+        dc = torch.full((m, ldc), float("nan"), device="cuda")
+        capi.matmul(w, gu.dev(a), m, dc, ldc=ldc, stream=gu.stream())
+        torch.cuda.synchronize()
+        got = dc[:, :n].cpu().numpy()
+        assert not np.isnan(got).any()
+        assert gu.rel_err(got, ref) <= gu.TOL, gu.rel_err(got, ref)
+        assert torch.isnan(dc[:, n:]).all(), "the call wrote between the rows of C"
+        scale = np.abs(ref).max(axis=1)
+        assert (np.abs(got - ref).max(axis=1) / scale).max() <= 2e-4
+        again = torch.full((m, n), float("nan"), device="cuda")
+        capi.matmul_noalloc(w, gu.dev(a), m, again, stream=gu.stream())
+        torch.cuda.synchronize()
+        assert np.array_equal(again.cpu().numpy(), got), "the allocation-free call differs"
+    finally:
+        w.destroy()
+
+
 def test_q4_K_gemm_tall_tiles(hipq, cr):
     """A shape for which the Q4_K GEMM picks its 128-row tiles (two rounds of 64-row
     tiles against one of 128-row tiles), with M not a multiple of the tile height."""
