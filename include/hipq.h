@@ -149,8 +149,8 @@ HIPQ_API int hipq_quantize_q8_K(const float *A, int64_t M, int64_t K, int64_t ld
  *  Outputs carry the bits of the reference's AVX2 kernels for every Q4_0 product and for
  *  Q4_K with up to 8 rows (up to 16 against 1024 columns or more, once the weight's copy
  *  described below exists or may be made) and Q6_K with up to 16 rows (up to 8 for matrices
- *  of 2^25 weights or more, up to 2 from 2^28: there the matrix cores are several times
- *  faster); with more rows the K-formats run on the
+ *  of 2^24 weights or more, up to 4 from 2^25, up to 2 from 2^28: there the matrix cores are
+ *  faster, up to several times); with more rows the K-formats run on the
  *  int8 matrix cores and agree with the reference to 1e-4 of the output's maximum (same
  *  quantized activations, another order of the fp32 sums). The first such product of a
  *  weight adds a copy of it in the kernels' load order (allocates; 0.56 bytes per weight

@@ -306,11 +306,13 @@ bool wants_tiled(const hipq_weight *w, int64_t M, bool may_allocate = true) {
   if (w->dtype == HIPQ_Q6_K) {
     /* The GEMV engine keeps the reference's bits but costs a pass over the weights per eight rows
      * and about 1e-7 us per weight and row on the vector ALU; the matrix-core GEMM costs one 64-row
-     * tile whatever the row count (35 us, or 2e-7 us per weight). Measured, us, engine against GEMM:
-     * 151936 x 4096 with 2 / 4 / 8 / 16 rows 115 / 192 / 441 / 847 against 130; 12288 x 4096 with
-     * 8 / 16 rows 42 / 80 against 36; 4096 x 4096 with 16 rows 34 against 35. */
+     * tile whatever the row count (17-23 us in parts of K, or 2e-7 us per weight). Measured, us,
+     * engine against GEMM: 151936 x 4096 with 2 / 4 / 8 / 16 rows 115 / 192 / 441 / 847 against 130;
+     * 12288 x 4096 with 4 / 8 / 16 rows 22 / 42 / 80 against 23; 4096 x 4096 with 8 / 9 / 16 rows
+     * 19 / 25 / 34 against 17. */
     const int64_t weights = w->N * w->K;
-    const int64_t engine_rows = weights >= (int64_t(1) << 28) ? 2 : weights >= (int64_t(1) << 25) ? 8 : 16;
+    const int64_t engine_rows = weights >= (int64_t(1) << 28) ? 2 : weights >= (int64_t(1) << 25) ? 4 :
+                                weights >= (int64_t(1) << 24) ? 8 : 16;
     return M > engine_rows && (w->gt_base || may_allocate);
   }
   /* up to 16 rows of a Q4_K matrix of 1024 columns or more take the few-rows kernel (wants_rows) */
@@ -379,10 +381,18 @@ int check_matmul_args(hipq_weight_t w, const float *A, int64_t M, int64_t lda, c
 int matmul_tiled(const hipq_weight *w, const float *A, int64_t M, int64_t lda, float *C, int64_t ldc,
                  hipStream_t s, int phase, const Scratch &sc) {
   void *mem = nullptr;
+  /* The GEMM reads a tile copy of the weights (coalesced loads), made at the weight's first
+   * prefill product (before anything that depends on its existence, so that the first product has
+   * the bits of the following ones); the entry point that may not allocate reads the planes
+   * until it exists. */
+  if (!w->gt_base && !sc.fixed) {
+    const int trc = hipq::ensure_gemm_tiles(const_cast<hipq_weight *>(w));
+    if (trc) return trc;
+  }
   /* room for the partial products of a product with few tiles behind the activations (the fixed
    * scratch of the allocation-free entry point may be too small for them: then none) */
   const size_t act_bytes = (qact_tiled_bytes(M, w->K) + 255) & ~(size_t)255;
-  size_t part_bytes = w->dtype == HIPQ_Q4_K ? hipq::gemm_q4k_split_bytes(w, M) : 0;
+  size_t part_bytes = w->dtype == HIPQ_Q4_K ? hipq::gemm_q4k_split_bytes(w, M) : hipq::gemm_q6k_split_bytes(w, M);
   if (sc.fixed && act_bytes + part_bytes > NOALLOC_SCRATCH_BYTES) part_bytes = 0;
   int rc = sc.get(act_bytes + part_bytes, &mem);
   if (rc) return rc;
@@ -393,11 +403,7 @@ int matmul_tiled(const hipq_weight *w, const float *A, int64_t M, int64_t lda, f
   const int64_t mat_rows = w->dtype == HIPQ_Q4_K ? (M / 4) * 4 : 0;
   if (phase != 1) rc = hipq::launch_quantize_q8_K_tiled(A, M, w->K, lda, mat_rows, &qa, s);
   if (rc || phase == 2) return rc;
-  /* The GEMM reads a tile copy of the weights (coalesced loads), made at the weight's first
-   * prefill product; the entry point that may not allocate reads the planes until it exists. */
-  if (!w->gt_base && !sc.fixed && (rc = hipq::ensure_gemm_tiles(const_cast<hipq_weight *>(w)))) return rc;
-  if (w->dtype == HIPQ_Q6_K) return hipq::launch_gemm_q6k(w, &qa, (int)M, C, ldc, s);
-  /* the copy may have been made just now: parts are used from the next call on */
+  if (w->dtype == HIPQ_Q6_K) return hipq::launch_gemm_q6k(w, &qa, (int)M, C, ldc, s, partials);
   return hipq::launch_gemm_q4k(w, &qa, (int)M, C, ldc, s, partials);
 }
 

@@ -193,10 +193,13 @@ __device__ __forceinline__ void epilogue(const Smem6<TM> &sm, int buf, float dco
   }
 }
 
-template <int TM>
-__global__ __launch_bounds__(NT, TM == 2 ? 3 : 2) void gemm_q6k_kernel(WView w, const int8_t *__restrict__ qt,
-                                                                       const float *__restrict__ dAt, int M, int mtiles,
-                                                                       int ntiles, float *__restrict__ C, int64_t ldc) {
+/* The tile of workgroup blockIdx.x. KSPLIT: its sum over super-blocks sb0 .. sb0 + nsb_part - 1 only
+ * (a partial product; the caller adds the parts): everything the loop reads is addressed relative to
+ * its first super-block, so the part's first one becomes that by moving the bases. */
+template <int TM, bool KSPLIT>
+__device__ __forceinline__ void gemm_q6k_tile(const WView &w, const int8_t *__restrict__ qt,
+                                              const float *__restrict__ dAt, int M, int mtiles, int ntiles,
+                                              float *__restrict__ C, int64_t ldc, int sb0, int nsb_part) {
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   Smem6<TM> &sm = *reinterpret_cast<Smem6<TM> *>(smem_raw);
   constexpr int BM = 32 * TM;
@@ -205,7 +208,9 @@ __global__ __launch_bounds__(NT, TM == 2 ? 3 : 2) void gemm_q6k_kernel(WView w, 
   const int mt = qd % mtiles, nt = (qd / mtiles) * 8 + xcd;
   if (nt >= ntiles) return; /* uniform per workgroup */
   const int m0 = mt * BM, n0 = nt * BN;
-  const int nsb = w.K >> 8;
+  const int nsb_all = w.K >> 8;
+  const int first = KSPLIT ? sb0 : 0;
+  const int nsb = KSPLIT ? nsb_part : nsb_all; /* the super-blocks this call walks */
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const int i32 = lane & 31;
@@ -213,13 +218,13 @@ __global__ __launch_bounds__(NT, TM == 2 ? 3 : 2) void gemm_q6k_kernel(WView w, 
   Src6 sr;
   /* the quantizer tiles by 128 rows: a 64-row tile is half mt & 1 of quantizer tile mt / 2 */
   const int qt128 = TM == 2 ? mt >> 1 : mt, hrow = TM == 2 ? mt & 1 : 0;
-  sr.qt = make_rsrc(qt + (size_t)qt128 * (2 * nsb) * QSTAGE + hrow * 8192, (uint32_t)(2 * nsb) * QSTAGE);
-  sr.dAt = make_rsrc(dAt + (size_t)qt128 * nsb * 128 + hrow * 64, (uint32_t)nsb * 128 * 4);
+  sr.qt = make_rsrc(qt + ((size_t)qt128 * (2 * nsb_all) + 2 * first) * QSTAGE + hrow * 8192, (uint32_t)(2 * nsb) * QSTAGE);
+  sr.dAt = make_rsrc(dAt + ((size_t)qt128 * nsb_all + first) * 128 + hrow * 64, (uint32_t)nsb * 128 * 4);
   /* the copy pads N to 32 rows: a wavefront whose columns start below N has its tile */
   const size_t wt = (size_t)(min(n0 + wave * 32, (int)w.N - 1) >> 5);
-  sr.wq = make_rsrc(w.qs + wt * nsb * 4096, (uint32_t)nsb * 4096);
-  sr.wh = make_rsrc(w.qh + wt * nsb * 2048, (uint32_t)nsb * 2048);
-  sr.whd = make_rsrc(w.hdr + wt * nsb * 1024, (uint32_t)nsb * 1024);
+  sr.wq = make_rsrc(w.qs + (wt * nsb_all + first) * 4096, (uint32_t)nsb * 4096);
+  sr.wh = make_rsrc(w.qh + (wt * nsb_all + first) * 2048, (uint32_t)nsb * 2048);
+  sr.whd = make_rsrc(w.hdr + (wt * nsb_all + first) * 1024, (uint32_t)nsb * 1024);
   sr.wave = wave;
   sr.lane = lane;
 
@@ -287,6 +292,38 @@ __global__ __launch_bounds__(NT, TM == 2 ? 3 : 2) void gemm_q6k_kernel(WView w, 
     }
 }
 
+template <int TM>
+__global__ __launch_bounds__(NT, TM == 2 ? 3 : 2) void gemm_q6k_kernel(WView w, const int8_t *__restrict__ qt,
+                                                                       const float *__restrict__ dAt, int M, int mtiles,
+                                                                       int ntiles, float *__restrict__ C, int64_t ldc) {
+  gemm_q6k_tile<TM, false>(w, qt, dAt, M, mtiles, ntiles, C, ldc, 0, 0);
+}
+
+/* Few tiles (up to 128 rows against a matrix of a few thousand columns make under two hundred
+ * workgroups, each walking all of K): blockIdx.y takes a part of K and writes its partial product to
+ * part[y]; split_sum6_kernel adds the parts in ascending order. */
+__global__ __launch_bounds__(NT, 3) void gemm_q6k_split_kernel(WView w, const int8_t *__restrict__ qt,
+                                                               const float *__restrict__ dAt, int M, int mtiles,
+                                                               int ntiles, int sb_per_part, float *__restrict__ part,
+                                                               int64_t part_stride) {
+  const int sb0 = blockIdx.y * sb_per_part;
+  gemm_q6k_tile<2, true>(w, qt, dAt, M, mtiles, ntiles, part + (int64_t)blockIdx.y * part_stride, w.N, sb0,
+                         min(sb_per_part, (w.K >> 8) - sb0));
+}
+
+__global__ __launch_bounds__(256) void split_sum6_kernel(const float *__restrict__ part, int parts, int64_t part_stride,
+                                                         int M, int N, float *__restrict__ C, int64_t ldc) {
+  const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4; /* N % 4 == 0 */
+  if (i >= (int64_t)M * N) return;
+  const int m = (int)(i / N), n = (int)(i - (int64_t)m * N);
+  float4 v = *(const float4 *)(part + i);
+  for (int p = 1; p < parts; ++p) {
+    const float4 u = *(const float4 *)(part + p * part_stride + i);
+    v.x += u.x, v.y += u.y, v.z += u.z, v.w += u.w;
+  }
+  *(float4 *)(C + (int64_t)m * ldc + n) = v;
+}
+
 } // namespace
 
 namespace hipq {
@@ -307,10 +344,44 @@ static int launch_tiles6(const hipq_weight *w, const QActTiled *qa, int M, float
   return HIPQ_OK;
 }
 
-int launch_gemm_q6k(const hipq_weight *w, const QActTiled *qa, int M, float *C, int64_t ldc, hipStream_t s) {
+/* Parts of K for a product whose 64-row tiles would leave most of the chip idle (0: none), and the
+ * bytes of partial products they need (the rule of the Q4_K product, gemm_q4k.hip). */
+int gemm_q6k_split_parts(const hipq_weight *w, int64_t M) {
+  if (w->dtype != HIPQ_Q6_K || !w->gt_base || (w->N & 3)) return 0;
+  const int64_t tiles = ((M + 63) / 64) * ((w->N + BN - 1) / BN), nsb = w->K / 256;
+  if (tiles > 192 || nsb < 8) return 0;
+  int parts = (int)(768 / tiles); /* three workgroups a CU */
+  if (parts > 8) parts = 8;
+  if (parts > nsb / 4) parts = (int)(nsb / 4);
+  return parts >= 2 ? parts : 0;
+}
+size_t gemm_q6k_split_bytes(const hipq_weight *w, int64_t M) {
+  return (size_t)gemm_q6k_split_parts(w, M) * (size_t)M * (size_t)w->N * 4;
+}
+
+int launch_gemm_q6k(const hipq_weight *w, const QActTiled *qa, int M, float *C, int64_t ldc, hipStream_t s,
+                    void *partials) {
   if ((M + 127) / 128 != qa->mtiles || qa->K != w->K)
     return fail(HIPQ_ERR_INVALID_ARGUMENT, "tiled activations do not match the matmul shape");
   if (!w->gt_base) return fail(HIPQ_ERR_INVALID_ARGUMENT, "the Q6_K prefill product needs the weight's tile copy");
+  const int parts = partials ? gemm_q6k_split_parts(w, M) : 0;
+  if (parts && !(ldc & 3) && !((uintptr_t)C & 15)) {
+    const int nsb = (int)(w->K / 256), per = (nsb + parts - 1) / parts;
+    const int mtiles = (M + 63) / 64, ntiles = (int)((w->N + BN - 1) / BN), ngroups = (ntiles + 7) / 8;
+    const int64_t stride = (int64_t)M * w->N;
+    WView v = wview(w);
+    v.qs = w->gt_qs;
+    v.qh = w->gt_qh;
+    v.hdr = w->gt_hdr;
+    launch_kernel(gemm_q6k_split_kernel, dim3((unsigned)(mtiles * ngroups * 8), (unsigned)((nsb + per - 1) / per)),
+                  dim3(NT), sizeof(Smem6<2>), s, v, (const int8_t *)qa->qt, (const float *)qa->dAt, M, mtiles, ntiles,
+                  per, (float *)partials, stride);
+    HIPQ_HIP(hipGetLastError());
+    hipLaunchKernelGGL(split_sum6_kernel, dim3((unsigned)((stride / 4 + 255) / 256)), dim3(256), 0, s,
+                       (const float *)partials, (nsb + per - 1) / per, stride, M, (int)w->N, C, ldc);
+    HIPQ_HIP(hipGetLastError());
+    return HIPQ_OK;
+  }
   /* 128-row tiles halve the expansion per row (the larger part of this kernel's vector work):
    * 862 against 726 TOP/s at 2048 x 12288 x 4096, 835 against 729 at 512 x 151936 x 4096. Two
    * of their workgroups fit a CU instead of three, so they never need more rounds than the

@@ -224,7 +224,9 @@ int launch_gemm_multi(int count, const hipq_weight *const *w, const QAct *qa, in
 /* gemm_q4k.hip: Q4_K with the sub-block scales folded into two int8 digit planes */
 int launch_gemm_q4k_multi(int count, const hipq_weight *const *w, const QActTiled *qa, int M, float *const *C,
                           const int64_t *ldc, hipStream_t s);
-int launch_gemm_q6k(const hipq_weight *w, const QActTiled *qa, int M, float *C, int64_t ldc, hipStream_t s);
+int launch_gemm_q6k(const hipq_weight *w, const QActTiled *qa, int M, float *C, int64_t ldc, hipStream_t s,
+                    void *partials = nullptr);
+size_t gemm_q6k_split_bytes(const hipq_weight *w, int64_t M);
 /* partials: gemm_q4k_split_bytes(w, M) bytes of device memory (or null): with few tiles the product
  * is formed in parts of K that run side by side and are then added */
 int launch_gemm_q4k(const hipq_weight *w, const QActTiled *qa, int M, float *C,
