@@ -203,10 +203,10 @@ def main():
     gemv_hot_ms = capi.time_matmul(weights[:1], a1, 1, c1, 400, phase=1, stream=stream)
     gemv_gbs = gv_bytes / (gemv_ms * 1e-3) / 1e9
 
-    # ---- a batch of eight (four) decode rows against the same matrices: Q4_K on the matrix cores
-    # with the reference's bits (gemm_rows_q4k.hip) ----
+    # ---- a batch of decode rows against the same matrices: Q4_K on the matrix cores with the
+    # reference's bits up to sixteen rows (gemm_rows_q4k.hip), the prefill GEMM beyond ----
     rows_ms = {}
-    for mr in (8, 4):
+    for mr in (8, 4, 16, 64):
         ar = torch.randn((mr, K), generator=gen, device="cuda", dtype=torch.float32)
         cr_ = torch.empty((mr, N), device="cuda", dtype=torch.float32)
         capi.time_matmul(weights, ar, mr, cr_, 2 * n_copies, phase=1, stream=stream)
@@ -485,7 +485,11 @@ def main():
             "kernel": "gemm_rows_q4k_kernel",
             "rows_8_kernel_ms": round(rows_ms[8][0], 5), "rows_8_ms_per_call": round(rows_ms[8][1], 5),
             "rows_4_kernel_ms": round(rows_ms[4][0], 5), "rows_4_ms_per_call": round(rows_ms[4][1], 5),
-            "rows_8_weight_gbs": round(gv_bytes / (rows_ms[8][0] * 1e-3) / 1e9, 2)},
+            "rows_8_weight_gbs": round(gv_bytes / (rows_ms[8][0] * 1e-3) / 1e9, 2),
+            "rows_16_kernel_ms": round(rows_ms[16][0], 5), "rows_16_ms_per_call": round(rows_ms[16][1], 5),
+            "rows_64_kernel_ms": round(rows_ms[64][0], 5), "rows_64_ms_per_call": round(rows_ms[64][1], 5),
+            "note": "16 rows: two passes of the same kernel, still the reference's bits; 64 rows: the prefill GEMM "
+                    "in parts of K (one 64-row tile per 128 columns), within 1e-4"},
         "decode_gemv_lm_head_size": {
             "workload": "Q4_K GEMV M=1 K=4096 N=151936, 3 weight copies rotated",
             "roofline": {"bound": "hbm", "kernel": "gemv_stream_kernel<Q4_K,G=4,GPW=2>",
