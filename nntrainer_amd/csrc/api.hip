@@ -354,8 +354,14 @@ int multiply(const hipq_weight *w, const QAct &qa, int64_t M, float *C, int64_t 
   const int is_k = w->dtype != HIPQ_Q4_0;
   /* rows the reference sends through its 4-row GEMM kernel (Q4_K, M > 1) */
   const int pair_rows = (w->dtype == HIPQ_Q4_K && M > 1 && !each_row) ? (int)((M / 4) * 4) : 0;
-  if (M <= 8) return hipq::launch_gemv(w, &qa, (int)M, pair_rows, C, ldc, s);
-  if (w->dtype == HIPQ_Q4_0 && w->K % 256 == 0) return hipq::launch_gemm(w, &qa, (int)M, C, ldc, s);
+  /* Q4_0: the matrix-core GEMM carries the reference's bits like the GEMV engine, so it also takes
+   * five to eight rows where it is faster: the engine's eight-row pass costs 33 us at 12288 x 4096
+   * and 181 us at 151936 x 1024, the GEMM 29 and 72 us (smaller matrices: 8.7 against 9.3 us at
+   * 3072 x 1024, the engine stays) */
+  const bool q40_gemm = w->dtype == HIPQ_Q4_0 && w->K % 256 == 0;
+  if (M <= 8 && !(q40_gemm && M >= 5 && w->N * w->K >= (int64_t(1) << 25)))
+    return hipq::launch_gemv(w, &qa, (int)M, pair_rows, C, ldc, s);
+  if (q40_gemm) return hipq::launch_gemm(w, &qa, (int)M, C, ldc, s);
   for (int64_t r0 = 0; r0 < M; r0 += 8) {
     const int64_t rows = (M - r0) < 8 ? (M - r0) : 8;
     QAct sub = qact_rows(qa, is_k, r0, rows);
