@@ -147,8 +147,9 @@ HIPQ_API int hipq_quantize_q8_K(const float *A, int64_t M, int64_t K, int64_t ld
  *  device memory the call is a single kernel launch (the GEMV quantizes the row
  *  itself) and uses no workspace.
  *  Outputs carry the bits of the reference's AVX2 kernels for every Q4_0 product and for
- *  Q4_K with up to 8 rows (up to 16 against 1024 columns or more, once the weight's copy
- *  described below exists or may be made) and Q6_K with up to 16 rows (up to 8 for matrices
+ *  Q4_K with up to 8 rows (up to 16 against 1024 columns or more, up to 64 where
+ *  columns / 32 x rows / 8 x K / 256 <= 8192, once the weight's copy described below exists
+ *  or may be made) and Q6_K with up to 16 rows (up to 8 for matrices
  *  of 2^24 weights or more, up to 4 from 2^25, up to 2 from 2^28: there the matrix cores are
  *  faster, up to several times); with more rows the K-formats run on the
  *  int8 matrix cores and agree with the reference to 1e-4 of the output's maximum (same
@@ -157,7 +158,7 @@ HIPQ_API int hipq_quantize_q8_K(const float *A, int64_t M, int64_t K, int64_t ld
  *  for Q4_K, 0.875 for Q6_K), kept until hipq_weight_destroy. Q4_K with 5..16 rows and 1024
  *  columns or more (4 rows from 4096, 3 from 8192 columns) reads the same copy: those row
  *  counts run on the matrix cores as well, with the reference's bits (a batch of decode
- *  rows against a 12288 x 4096 matrix: 11 us for eight, 22 us for sixteen, 8 us for one). */
+ *  rows against a 12288 x 4096 matrix: 11 us for eight, 14 us for sixteen, 8 us for one). */
 HIPQ_API int hipq_matmul(hipq_weight_t w, const float *A, int64_t M, int64_t lda,
                          float *C, int64_t ldc, int mem, void *stream);
 

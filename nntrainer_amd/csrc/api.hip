@@ -431,13 +431,7 @@ int matmul_rows(const hipq_weight *w, const float *A, int64_t M, int64_t lda, fl
   if (phase != 1) rc = hipq::launch_quantize_q8_K_rowmma(A, M, w->K, lda, &qa, s, mat_rows);
   if (rc || phase == 2) return rc;
   if (!w->gt_base && (rc = hipq::ensure_gemm_tiles(const_cast<hipq_weight *>(w)))) return rc;
-  for (int64_t r0 = 0; r0 < M && !rc; r0 += 8) { /* passes of up to eight rows */
-    const int64_t rows = (M - r0) < 8 ? (M - r0) : 8;
-    const int64_t pair = mat_rows - r0 < 0 ? 0 : (mat_rows - r0 > rows ? rows : mat_rows - r0);
-    const QAct sub = qact_rows(qa, 1, r0, rows);
-    rc = hipq::launch_gemm_rows_q4k(w, &sub, (int)rows, (int)pair, C + r0 * ldc, ldc, s);
-  }
-  return rc;
+  return hipq::launch_gemm_rows_q4k(w, &qa, (int)M, (int)mat_rows, C, ldc, s); /* up to two passes of eight rows */
 }
 
 /* each_row: every row as a product of its own with M = 1 (the bits of M separate calls): for Q4_0

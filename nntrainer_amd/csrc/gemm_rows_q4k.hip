@@ -64,10 +64,18 @@ struct RowsRegs {
   rv4i hd;
 };
 
-__global__ __launch_bounds__(NT, 2) void gemm_rows_q4k_kernel(WView w, QView a, int M, int pair_rows,
+/* blockIdx.y: the pass, rows 8 y .. 8 y + 7 of the call's M_all (the first pair_all of them under
+ * the 4-row rule); the passes of one launch run side by side */
+__global__ __launch_bounds__(NT, 2) void gemm_rows_q4k_kernel(WView w, QView a, int M_all, int pair_all,
                                                               float *__restrict__ C, int64_t ldc) {
   extern __shared__ __attribute__((aligned(16))) unsigned char rows_lds[];
   const int K = w.K, nsb = K >> 8;
+  const int r0 = blockIdx.y * TC;
+  const int M = min(TC, M_all - r0), pair_rows = min(max(pair_all - r0, 0), M);
+  a.q += (size_t)r0 * K;
+  a.d += (size_t)r0 * nsb;
+  a.bsum += (size_t)r0 * (K >> 4);
+  C += (int64_t)r0 * ldc;
   const int tile = blockIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const int lane = threadIdx.x & 63, i32 = lane & 31, g = lane >> 5;
@@ -293,22 +301,30 @@ namespace hipq {
  * streams its weights at 2.5-4.6 TB/s. */
 bool gemm_rows_q4k_fits(const hipq_weight *w, int64_t M) {
   if (w->dtype != HIPQ_Q4_K || w->expert_tiles || w->K % 256 || 16 * w->K > 0x7fffffff) return false;
-  /* nine to sixteen rows as two passes (12288 x 4096: 22 us, against 31 us for one 64-row tile of
-   * the prefill GEMM, whose 96 workgroups leave most of the chip idle) */
+  /* More than eight rows: passes of eight side by side in one launch (blockIdx.y). Two passes
+   * always (12288 x 4096 with 16 rows: 14.7 us against 17.2 for the prefill GEMM in parts of K; 4096 x
+   * 4096: 8.5 against 12.5: a launch of one pass leaves half the chip idle there); up to eight where
+   * the launch stays small, measured against that GEMM (us): 4096 x 4096 with 32 / 48 rows 10.1 / 12.5
+   * against 12.7 / 13.3, 2048 x 2048 with 64 rows 6.5 against 11.0; but 12288 x 4096 with 24 rows 23.2
+   * against 18.3, 4096 x 12288 with 24 rows 24.1 against 18.1. */
   if (M >= 5 && M <= 2 * TC) return w->N >= 1024;
+  if (M > 2 * TC && M <= 8 * TC && w->N >= 1024) {
+    const int64_t tiles = (w->N + 31) / 32, passes = (M + TC - 1) / TC;
+    return tiles * passes * (w->K / 256) <= 8192;
+  }
   return (M == 4 && w->N >= 4096) || (M == 3 && w->N >= 8192);
 }
 
 int launch_gemm_rows_q4k(const hipq_weight *w, const QAct *qa, int M, int pair_rows, float *C, int64_t ldc,
                          hipStream_t s) {
-  if (M < 1 || M > TC || w->dtype != HIPQ_Q4_K || qa->K != w->K)
-    return fail(HIPQ_ERR_INVALID_ARGUMENT, "a pass of the few-rows Q4_K product takes 1..8 rows");
+  if (M < 1 || M > 8 * TC || w->dtype != HIPQ_Q4_K || qa->K != w->K)
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "the few-rows Q4_K product takes 1..64 rows");
   if (!w->gt_base) return fail(HIPQ_ERR_INVALID_ARGUMENT, "the few-rows Q4_K product needs the weight's tile copy");
   WView v = wview(w);
   v.qs = w->gt_qs;
   v.hdr = w->gt_hdr;
   const unsigned grid = (unsigned)((w->N + 31) / 32);
-  hipLaunchKernelGGL(gemm_rows_q4k_kernel, dim3(grid), dim3(NT), LDS_BYTES, s, v, qview(*qa), M, pair_rows, C, ldc);
+  hipLaunchKernelGGL(gemm_rows_q4k_kernel, dim3(grid, (unsigned)((M + TC - 1) / TC)), dim3(NT), LDS_BYTES, s, v, qview(*qa), M, pair_rows, C, ldc);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
 }

@@ -60,12 +60,14 @@ def test_small_m_matches_oracle(hipq, cr, kind, m):
                                    (7, 12288, 2048), (3, 8200, 1024), (4, 8195, 2048), (6, 1100, 768),
                                    (8, 1024, 256), (5, 3000, 4096), (8, 1030, 8192), (6, 1024, 5376),
                                    (4, 4100, 1280), (9, 1100, 1024), (14, 2048, 512), (16, 1024, 2048),
-                                   (11, 4000, 4096), (6, 32768, 1024), (8, 8200, 4096)])
+                                   (11, 4000, 4096), (6, 32768, 1024), (8, 8200, 4096), (24, 4096, 2048),
+                                   (64, 2048, 2048), (33, 1056, 4096)])
 def test_small_m_on_large_matrices_matches_oracle(hipq, cr, kind, m, n, k):
     """Three to sixteen rows against larger matrices, where Q4_K leaves the GEMV engine (and, from
     nine rows, the prefill GEMM) for the matrix-core kernel of gemm_rows_q4k.hip (five rows and
-    more from 1024 columns up, four from 4096, three from 8192; nine to sixteen rows as two
-    passes, the second with fewer rows under the 4-row rule or none): rows under the reference's
+    more from 1024 columns up, four from 4096, three from 8192; more than eight rows as passes
+    of eight side by side in one launch, up to 64 rows where the product is small, the later
+    passes with fewer rows under the 4-row rule or none): rows under the reference's
     4-row rule and under its row rule in one call
     (6 = 4 + 2), one to 32 super-blocks a row (a round of four wavefronts partly idle, a single
     round, rows longer than the GEMV engine's 4096-weight chunk), column counts that end inside
