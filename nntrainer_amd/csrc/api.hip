@@ -867,9 +867,18 @@ int hipq_matmul_each_row(hipq_weight_t w, const float *A, int64_t rows, int64_t 
     dA = (const float *)io, dC = (float *)((char *)io + a_bytes), a_ld = w->K, c_ld = w->N;
     if ((rc = stage_copy(true, (void *)dA, (void *)A, (size_t)lda * 4, (size_t)w->K * 4, (size_t)rows, s))) return rc;
   }
-  for (int64_t r0 = 0; r0 < rows && !rc; r0 += 16) { /* sixteen rows a step: the row counts that keep the M = 1 bits */
-    const int64_t n = (rows - r0) < 16 ? (rows - r0) : 16;
+  for (int64_t r0 = 0; r0 < rows && !rc;) { /* steps of row counts that keep the M = 1 bits */
+    int64_t n = (rows - r0) < 16 ? (rows - r0) : 16;
+    if (w->dtype == HIPQ_Q4_K) /* up to 64 where the few-rows kernel takes that many in one launch */
+      for (int64_t c = 64; c > 16; c -= 8) {
+        const int64_t t = (rows - r0) < c ? (rows - r0) : c;
+        if (t > 16 && wants_rows(w, t, true)) {
+          n = t;
+          break;
+        }
+      }
     rc = matmul_device(w, dA + r0 * a_ld, n, a_ld, dC + r0 * c_ld, c_ld, s, sc, true);
+    r0 += n;
   }
   if (rc || mem == HIPQ_MEM_DEVICE) return rc;
   return stage_copy(false, dC, C, (size_t)ldc * 4, (size_t)w->N * 4, (size_t)rows, s);
