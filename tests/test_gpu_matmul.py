@@ -606,3 +606,34 @@ def test_matmul_each_row_has_the_bits_of_single_row_products(hipq, cr, kind, row
     finally:
         w.destroy()
 
+
+def test_row_counts_across_the_kernel_choices(hipq, cr):
+    """hipq_matmul picks among the GEMV engine, the few-rows matrix-core kernel (one to eight passes),
+    the prefill GEMMs (whole K or parts of K) by format, row count and matrix size. Shapes drawn
+    around the thresholds from a seeded generator: every result within 1e-4 of the reference, Q4_0
+    and every product of one or two rows with its bits, a second call the bits of the first."""
+    import gpu_util as gu
+    rng = np.random.RandomState(20250117)
+    done = 0
+    while done < 36:
+        kind = KINDS[done % 3]
+        n = int(rng.choice([1000, 1024, 1056, 2048, 4096, 4100, 8192, 8200]))
+        k = int(rng.choice([256, 1024, 2048, 2304, 4096]))
+        m = int(rng.choice([1, 2, 3, 4, 5, 8, 9, 12, 16, 17, 24, 33, 48, 64, 65, 70]))
+        if m * n * k > 4e8:
+            continue
+        blocks = _weights(cr, kind, n, k, seed=1200 + done)
+        a = synth.normal(1300 + done, (m, k))
+        ref = cr.gemm(cr.oracle(), kind, a, blocks, n)
+        w = capi.Weight(kind, n, k, blocks)
+        got = gu.gpu_matmul(w, a)
+        again = gu.gpu_matmul(w, a)
+        w.destroy()
+        case = (kind, m, n, k)
+        assert not np.isnan(got).any(), case
+        assert gu.rel_err(got, ref) <= gu.TOL, (case, gu.rel_err(got, ref))
+        assert np.array_equal(got, again), case
+        if kind == "q4_0" or m <= 2:
+            assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), case
+        done += 1
+
