@@ -1,10 +1,10 @@
 // SPDX-License-Identifier: Apache-2.0
 /**
  * @file   gemm_rows_q4k.hip
- * @brief  Q4_K x Q8_K for three to eight activation rows on the int8 matrix cores,
- *         with the reference's bits.
+ * @brief  Q4_K x Q8_K for a few activation rows (three to 64, in passes of eight side by
+ *         side in one launch) on the int8 matrix cores, with the reference's bits.
  *
- * Replaces, for 3 <= M <= 8, what __ggml_q4_K_8x8_q8_K_GEMM
+ * Replaces, for 3 <= M <= 64, what __ggml_q4_K_8x8_q8_K_GEMM
  * (nntrainer/tensor/cpu_backend/ggml_interface/ggml_interface_omp.cpp:391-517 in the
  * reference checkout) does with a few rows: the rows below 4 * (M / 4) go through
  * nntr_gemm_q4_K_8x8_q8_K (nntr_ggml_impl.cpp:3261-7078), which adds the four sub-block
@@ -14,7 +14,7 @@
  * 4 us on a 12288 x 4096 matrix (eight rows: 37 us; one row: 8 us, the weight stream); this
  * kernel takes 11.2 us for eight.
  *
- * Here a workgroup owns 32 output columns and all rows. Its four wavefronts take one
+ * Here a workgroup owns 32 output columns and the eight rows of its pass (blockIdx.y). Its four wavefronts take one
  * super-block each per round: one v_mfma_i32_32x32x32_i8 per sub-block (the rows are the
  * row operand: 8 of its 32 rows are used), the 6-bit scales applied to the exact int32 sums
  * pair by pair, the mins through four v_mfma_f32_32x32x16_f16 with all but one pair's mins
@@ -24,7 +24,7 @@
  * vector ALU but the integer work is not. Weights come from the 32-row tile copy the prefill
  * GEMM reads (piece i of lane (n, g) = sub-block 4 g + i of row n; the two lanes of a row swap
  * halves with v_permlane32_swap so that each holds its 16 weights of sub-blocks i and 4 + i),
- * the loads of the next two rounds in flight during the current one. The quantized rows are
+ * the loads of the next round in flight during the current one. The quantized rows are
  * staged a round at a time (52 KB of LDS with the records: three workgroups a CU, any K).
  */
 #include "hipq_internal.h"
