@@ -354,11 +354,12 @@ int multiply(const hipq_weight *w, const QAct &qa, int64_t M, float *C, int64_t 
   const int is_k = w->dtype != HIPQ_Q4_0;
   /* rows the reference sends through its 4-row GEMM kernel (Q4_K, M > 1) */
   const int pair_rows = (w->dtype == HIPQ_Q4_K && M > 1 && !each_row) ? (int)((M / 4) * 4) : 0;
-  /* Q4_0: the matrix-core GEMM carries the reference's bits like the GEMV engine, so it also takes
-   * five to eight rows where it is faster: the engine's eight-row pass costs 33 us at 12288 x 4096
-   * and 181 us at 151936 x 1024, the GEMM 29 and 72 us (smaller matrices: 8.7 against 9.3 us at
-   * 3072 x 1024, the engine stays) */
+  /* Q4_0: every kernel carries the reference's bits, so the row count only picks the fastest. A few
+   * rows (up to 64 where the launch stays small) go to the few-rows kernel of gemm_rows_q40.hip; where
+   * that one does not apply (narrow matrices), the prefill GEMM also takes five to eight rows from
+   * 2^25 weights up, where the GEMV engine's eight-row pass is the slower of the two */
   const bool q40_gemm = w->dtype == HIPQ_Q4_0 && w->K % 256 == 0;
+  if (hipq::gemm_rows_q40_fits(w, M)) return hipq::launch_gemm_rows_q40(w, &qa, (int)M, C, ldc, s);
   if (M <= 8 && !(q40_gemm && M >= 5 && w->N * w->K >= (int64_t(1) << 25)))
     return hipq::launch_gemv(w, &qa, (int)M, pair_rows, C, ldc, s);
   if (q40_gemm) return hipq::launch_gemm(w, &qa, (int)M, C, ldc, s);
@@ -869,6 +870,7 @@ int hipq_matmul_each_row(hipq_weight_t w, const float *A, int64_t rows, int64_t 
   }
   for (int64_t r0 = 0; r0 < rows && !rc;) { /* steps of row counts that keep the M = 1 bits */
     int64_t n = (rows - r0) < 16 ? (rows - r0) : 16;
+    if (w->dtype == HIPQ_Q4_0) n = rows - r0; /* every product of this format has them */
     if (w->dtype == HIPQ_Q4_K) /* up to 64 where the few-rows kernel takes that many in one launch */
       for (int64_t c = 64; c > 16; c -= 8) {
         const int64_t t = (rows - r0) < c ? (rows - r0) : c;

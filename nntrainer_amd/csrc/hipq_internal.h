@@ -240,6 +240,12 @@ bool gemm_rows_q4k_fits(const hipq_weight *w, int64_t M);
 int launch_gemm_rows_q4k(const hipq_weight *w, const QAct *qa, int M, int pair_rows, float *C, int64_t ldc,
                          hipStream_t s);
 
+/* gemm_rows_q40.hip: Q4_0 for a few rows on the matrix cores with the reference's bits (rows are
+ * independent in this format); fits: the row counts and shapes that should take it; qa in the form
+ * of launch_quantize_q8_0; the weight's planes as they are */
+bool gemm_rows_q40_fits(const hipq_weight *w, int64_t M);
+int launch_gemm_rows_q40(const hipq_weight *w, const QAct *qa, int M, float *C, int64_t ldc, hipStream_t s);
+
 /* moe.hip ----------------------------------------------------------------- */
 /* Variant of the expert MLP. kind 0: h = silu(g) * u, y = down(h) (qwen_moe_layer.cpp:332-392).
  * kind 1: g and u take a bias, h = (g / (1 + exp(-alpha g))) * (u + 1), y = down(h) + bias

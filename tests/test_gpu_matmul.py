@@ -89,6 +89,27 @@ def test_small_m_on_large_matrices_matches_oracle(hipq, cr, kind, m, n, k):
         "%d of %d outputs differ in bits" % ((got.view(np.uint32) != ref.view(np.uint32)).sum(), got.size)
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 65553, 1024), (1, 65536, 256), (2, 12300, 512), (3, 6150, 768),
+                                   (4, 6144, 1024), (5, 3100, 1280), (7, 3072, 256), (9, 640, 256),
+                                   (12, 600, 2304), (16, 513, 1024), (17, 520, 5120), (40, 1500, 1024),
+                                   (64, 4096, 256), (57, 2050, 1280)])
+def test_q4_0_few_rows_on_the_matrix_cores_match_oracle(hipq, cr, m, n, k):
+    """Q4_0 with a few rows where gemm_rows_q40.hip takes them (one row against a wide matrix of
+    short rows, two rows from 12288 columns, three and four from 6144, five to eight from 3072,
+    nine to sixteen from 512, up to 64 while the launch stays small): one to eight passes, one to
+    five rounds of 32 blocks with the last one partly or wholly one wavefront's, column counts
+    that end inside a 32-column tile. Same bits as the reference."""
+    import gpu_util as gu
+    blocks = _weights(cr, "q4_0", n, k, seed=1300 + m)
+    a = synth.normal(1301 + k + m, (m, k))
+    ref = cr.gemm(cr.oracle(), "q4_0", a, blocks, n)
+    w = capi.Weight("q4_0", n, k, blocks)
+    got = gu.gpu_matmul(w, a)
+    w.destroy()
+    assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), \
+        "%d of %d outputs differ in bits" % ((got.view(np.uint32) != ref.view(np.uint32)).sum(), got.size)
+
+
 @pytest.mark.parametrize("kind", KINDS)
 @pytest.mark.parametrize("m,n,k", [(1, 8200, 12288), (3, 200, 8192), (8, 520, 9216), (1, 96, 20480),
                                    (5, 64, 4352)])
@@ -569,7 +590,7 @@ def test_bad_arguments_are_reported(hipq):
 
 @pytest.mark.parametrize("kind", KINDS)
 @pytest.mark.parametrize("rows,n,k", [(8, 1100, 1024), (5, 512, 768), (12, 2048, 512), (16, 300, 256),
-                                      (37, 1056, 1024), (3, 8200, 512), (1, 640, 256)])
+                                      (37, 1056, 1024), (3, 8200, 512), (1, 640, 256), (70, 1030, 512)])
 def test_matmul_each_row_has_the_bits_of_single_row_products(hipq, cr, kind, rows, n, k):
     """hipq_matmul_each_row: the rows of a batch of decode steps against one weight in one call, every
     row with the bits of its own M = 1 product (the reference's loop over batch entries). For Q4_K
