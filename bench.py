@@ -283,6 +283,10 @@ def main():
         return total
 
     c5_prefill_ms, c5_decode_ms = fc_stack(512), fc_stack(1)
+    c5_rows8_ms, c5_rows16_ms = fc_stack(8), fc_stack(16)
+    # the same model's lm_head as a Q4_0 FC (151936 x 1024): one row and a batch of eight decode rows
+    c5_head_ms, c5_head_all_ms, c5_head_bytes, _, c5_head_rows8 = gemv_case("q4_0", 151936, 1024, 4, 18, 32,
+                                                                            prefill_rows=8)
 
     def decode_layer_graph(grouped, rows=1):
         """One step's FCs of 8 layers (8 weight copies) against `rows` rows captured in a graph and
@@ -530,6 +534,12 @@ def main():
             "prefill_512_rows_in_a_graph_ms": round(c5_prefill_graph_ms, 5),
             "prefill_512_rows_in_a_graph_qkv_and_gate_up_as_one_call_each_ms": round(c5_prefill_grouped_ms, 5),
             "decode_1_row_ms": round(c5_decode_ms, 5),
+            "decode_batch_8_rows_ms": round(c5_rows8_ms, 5), "decode_batch_16_rows_ms": round(c5_rows16_ms, 5),
+            "lm_head_q4_0_n151936": {"kernel": "gemm_rows_q40_kernel (one and eight rows)",
+                                     "rows_1_kernel_ms": round(c5_head_ms, 5), "rows_1_ms_per_call": round(c5_head_all_ms, 5),
+                                     "rows_8_kernel_ms": round(c5_head_rows8[0], 5),
+                                     "rows_8_ms_per_call": round(c5_head_rows8[1], 5),
+                                     "rows_8_weight_gbs": round(c5_head_bytes / (c5_head_rows8[0] * 1e-3) / 1e9, 2)},
             "decode_1_row_in_a_graph_ms": round(c5_graph_ms, 5),
             "decode_1_row_in_a_graph_qkv_and_gate_up_as_one_launch_each_ms": round(c5_graph_grouped_ms, 5),
             "decode_1_row_in_a_graph_qkv_one_launch_up_gate_swiglu_one_launch_ms": round(c5_graph_fused_ms, 5)},

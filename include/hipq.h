@@ -158,7 +158,10 @@ HIPQ_API int hipq_quantize_q8_K(const float *A, int64_t M, int64_t K, int64_t ld
  *  for Q4_K, 0.875 for Q6_K), kept until hipq_weight_destroy. Q4_K with 5..16 rows and 1024
  *  columns or more (4 rows from 4096, 3 from 8192 columns) reads the same copy: those row
  *  counts run on the matrix cores as well, with the reference's bits (a batch of decode
- *  rows against a 12288 x 4096 matrix: 11 us for eight, 14 us for sixteen, 8 us for one). */
+ *  rows against a 12288 x 4096 matrix: 11 us for eight, 14 us for sixteen, 8 us for one).
+ *  Q4_0 has the same kind of kernel for a few rows (gemm_rows_q40.hip, off the weight as it is
+ *  stored: eight rows against 12288 x 4096 in 11 us, against 151936 x 1024 in 26 us); every Q4_0
+ *  kernel carries the reference's bits, so there the row count only selects the fastest. */
 HIPQ_API int hipq_matmul(hipq_weight_t w, const float *A, int64_t M, int64_t lda,
                          float *C, int64_t ldc, int mem, void *stream);
 
@@ -169,8 +172,8 @@ HIPQ_API int hipq_matmul(hipq_weight_t w, const float *A, int64_t M, int64_t lda
  *  hipq_matmul with M = rows for Q4_K only, where the reference quantizes rows it multiplies
  *  together four at a time and sums their sub-block pairs separately; rows of different batch
  *  entries are never multiplied together there. The rows share one pass over the weights (Q4_K
- *  against 1024 columns or more: on the matrix cores, gemm_rows_q4k.hip) and, with host memory,
- *  one transfer each way. */
+ *  against 1024 columns or more: on the matrix cores, gemm_rows_q4k.hip; Q4_0: whatever
+ *  hipq_matmul picks for that many rows) and, with host memory, one transfer each way. */
 HIPQ_API int hipq_matmul_each_row(hipq_weight_t w, const float *A, int64_t rows, int64_t lda,
                                   float *C, int64_t ldc, int mem, void *stream);
 
