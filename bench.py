@@ -353,6 +353,7 @@ def main():
     c5_graph_ms, c5_graph_grouped_ms = decode_layer_graph(0), decode_layer_graph(1)
     c5_graph_fused_ms = decode_layer_graph(2)
     c5_prefill_graph_ms, c5_prefill_grouped_ms = decode_layer_graph(0, 512), decode_layer_graph(1, 512)
+    c5_rows8_grouped_ms = decode_layer_graph(1, 8)
 
     # ---- the MoE block of configs[3]: 64 tokens, 128 experts, top-8, Q4_K ----------
     mt, mh, me, mi, mk = 64, 2048, 128, 768, 8
@@ -535,6 +536,7 @@ def main():
             "prefill_512_rows_in_a_graph_qkv_and_gate_up_as_one_call_each_ms": round(c5_prefill_grouped_ms, 5),
             "decode_1_row_ms": round(c5_decode_ms, 5),
             "decode_batch_8_rows_ms": round(c5_rows8_ms, 5), "decode_batch_16_rows_ms": round(c5_rows16_ms, 5),
+            "decode_batch_8_rows_in_a_graph_qkv_and_gate_up_as_one_launch_each_ms": round(c5_rows8_grouped_ms, 5),
             "lm_head_q4_0_n151936": {"kernel": "gemm_rows_q40_kernel (one and eight rows)",
                                      "rows_1_kernel_ms": round(c5_head_ms, 5), "rows_1_ms_per_call": round(c5_head_all_ms, 5),
                                      "rows_8_kernel_ms": round(c5_head_rows8[0], 5),

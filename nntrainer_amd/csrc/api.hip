@@ -1042,26 +1042,30 @@ int hipq_matmul_multi(int count, const hipq_weight_t *w, const float *A, int64_t
     if ((rc = workspace(s, qact_bytes(is_k, M, w[0]->K), &memp))) return rc;
     QAct qa = qact_carve(is_k, memp, M, w[0]->K);
     if ((rc = quantize_for(w[first], A, M, lda, qa, s))) return rc;
-    /* Q4_0 prefill products go out four weights a launch (Q, K, V or gate, up: one grid that
-     * fills the chip instead of three or two small ones) */
-    const bool group = k == 0 && M > 8 && w[first]->K % 256 == 0;
+    /* Q4_0 products go out four weights a launch (Q, K, V or gate, up: one grid that fills the
+     * chip instead of three or two small ones): a few rows through the few-rows kernel where the
+     * launch as a whole is wide enough for it, more than eight otherwise through the prefill GEMM */
     const hipq_weight *gw[4];
     float *gc[4];
     int64_t gl[4];
     int ng = 0;
+    auto flush = [&]() -> int {
+      int frc = HIPQ_OK;
+      if (k == 0 && ng > 1 && hipq::gemm_rows_q40_fits_multi(ng, gw, M))
+        frc = hipq::launch_gemm_rows_q40_multi(ng, gw, &qa, (int)M, gc, gl, s);
+      else if (k == 0 && M > 8 && gw[0]->K % 256 == 0)
+        frc = hipq::launch_gemm_multi(ng, gw, &qa, (int)M, gc, gl, s);
+      else
+        for (int j = 0; j < ng && !frc; ++j) frc = multiply(gw[j], qa, M, gc[j], gl[j], s);
+      ng = 0;
+      return frc;
+    };
     for (int i = 0; i < count; ++i) {
       if (klass(w[i]) != k) continue;
-      if (!group) {
-        if ((rc = multiply(w[i], qa, M, C[i], ldc[i], s))) return rc;
-        continue;
-      }
       gw[ng] = w[i], gc[ng] = C[i], gl[ng] = ldc[i];
-      if (++ng == 4) {
-        if ((rc = hipq::launch_gemm_multi(ng, gw, &qa, (int)M, gc, gl, s))) return rc;
-        ng = 0;
-      }
+      if (++ng == 4 && (rc = flush())) return rc;
     }
-    if (ng && (rc = hipq::launch_gemm_multi(ng, gw, &qa, (int)M, gc, gl, s))) return rc;
+    if (ng && (rc = flush())) return rc;
   }
   return HIPQ_OK;
 }

@@ -79,16 +79,33 @@ struct SRegs {
   uint2 dw;
 };
 
-__global__ __launch_bounds__(NT, 2) void gemm_rows_q40_kernel(WView w, QView a, int M_all, float *__restrict__ C,
-                                                              int64_t ldc) {
+/* Up to four weights of one K against the same quantized rows as ONE launch: the grid's columns are
+ * the concatenation of the weights' column tiles (Q, K, V or gate, up of a layer). */
+struct MultiRowsQ40 {
+  WView w[4];
+  float *C[4];
+  int64_t ldc[4];
+  int tile_end[4]; /* running sum of the weights' column tiles */
+};
+
+__global__ __launch_bounds__(NT, 2) void gemm_rows_q40_kernel(MultiRowsQ40 mw, QView a, int M_all) {
   extern __shared__ __attribute__((aligned(16))) unsigned char rows_lds[];
+  /* which weight this workgroup's column tile belongs to (uniform) */
+  int tile = blockIdx.x, wi = 0;
+  if (tile >= mw.tile_end[0]) wi = 1;
+  if (tile >= mw.tile_end[1]) wi = 2;
+  if (tile >= mw.tile_end[2]) wi = 3;
+  if (wi) tile -= mw.tile_end[wi - 1];
+  const WView w = wi == 0 ? mw.w[0] : wi == 1 ? mw.w[1] : wi == 2 ? mw.w[2] : mw.w[3];
+  float *__restrict__ C = wi == 0 ? mw.C[0] : wi == 1 ? mw.C[1] : wi == 2 ? mw.C[2] : mw.C[3];
+  const int64_t ldc = wi == 0 ? mw.ldc[0] : wi == 1 ? mw.ldc[1] : wi == 2 ? mw.ldc[2] : mw.ldc[3];
   const int K = w.K, nb = K >> 5;
   const int r0 = blockIdx.y * TC;
   const int M = min(TC, M_all - r0);
   a.q += (size_t)r0 * K;
   a.meta += (size_t)r0 * nb;
   C += (int64_t)r0 * ldc;
-  const int tile = blockIdx.x, n0 = tile * 32;
+  const int n0 = tile * 32;
   const int ncols = min(32, w.N - n0);
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const int lane = threadIdx.x & 63, i32 = lane & 31, g = lane >> 5;
@@ -260,27 +277,68 @@ namespace hipq {
  * 151936 x 1024 68.4 -> 49.0; with more passes the launch grows and the GEMM does not: 12288 x 4096
  * with 24 / 32 rows 25.2 / 29.6 against 28.4 / 28.5, 4096 x 4096 with 48 / 64 rows 16.5 / 20.3 against
  * 19.7 / 19.9, 151936 x 1024 with 24 rows 71.7 against 68.7, 1024 x 3072 with 64 rows 9.5 against 15.4. */
-bool gemm_rows_q40_fits(const hipq_weight *w, int64_t M) {
-  if (w->dtype != HIPQ_Q4_0 || w->K % 256 || 16 * w->K > 0x7fffffff) return false;
-  const int64_t N = w->N;
-  if (M == 1) return w->K <= 1024 && N >= 65536;
+static bool rows_q40_pay(int64_t N, int64_t K, int64_t M) {
+  if (M == 1) return K <= 1024 && N >= 65536;
   if (M == 2) return N >= 12288;
   if (M <= 4) return N >= 6144;
   if (M <= TC) return N >= 3072;
   if (M <= 2 * TC) return N >= 512;
   if (M > 8 * TC || N < 512) return false;
-  const int64_t tiles = (N + 31) / 32, passes = (M + TC - 1) / TC, rounds = (w->K / 32 + BR - 1) / BR;
+  const int64_t tiles = (N + 31) / 32, passes = (M + TC - 1) / TC, rounds = (K / 32 + BR - 1) / BR;
   return tiles * passes * (rounds + 1) <= 6000;
 }
 
-int launch_gemm_rows_q40(const hipq_weight *w, const QAct *qa, int M, float *C, int64_t ldc, hipStream_t s) {
-  if (M < 1 || M > 8 * TC || w->dtype != HIPQ_Q4_0 || qa->K != w->K || w->K % 256 || 16 * w->K > 0x7fffffff)
-    return fail(HIPQ_ERR_INVALID_ARGUMENT, "the few-rows Q4_0 product takes 1..64 rows and K in whole 256s");
-  const unsigned grid = (unsigned)((w->N + 31) / 32);
-  hipLaunchKernelGGL(gemm_rows_q40_kernel, dim3(grid, (unsigned)((M + TC - 1) / TC)), dim3(NT), LDS_BYTES, s, wview(w),
-                     qview(*qa), M, C, ldc);
+static bool rows_q40_can(const hipq_weight *w) {
+  return w->dtype == HIPQ_Q4_0 && w->K % 256 == 0 && 16 * w->K <= 0x7fffffff;
+}
+
+bool gemm_rows_q40_fits(const hipq_weight *w, int64_t M) { return rows_q40_can(w) && rows_q40_pay(w->N, w->K, M); }
+
+/* Several weights of one K in one launch: what counts is the launch's width, the columns of all of
+ * them, and the launches it replaces. The seven FCs of a Qwen3-0.6B-shaped decoder layer with Q, K, V
+ * and gate, up as one call each, replayed from a graph, us per layer with 2 / 4 / 8 / 16 / 32 rows:
+ * 31.4 / 35.3 / 37.1 / 34.9 / 35.0 with a launch per weight (or the prefill GEMM's grouped launch from
+ * nine rows) -> 23.2 / 25.4 / 26.4 / 29.8 / 32.4. */
+bool gemm_rows_q40_fits_multi(int count, const hipq_weight *const *w, int64_t M) {
+  if (count < 1 || count > 4) return false;
+  int64_t N = 0;
+  for (int i = 0; i < count; ++i) {
+    if (!rows_q40_can(w[i]) || w[i]->K != w[0]->K) return false;
+    N += (w[i]->N + 31) / 32 * 32;
+  }
+  if (count == 1) return rows_q40_pay(N, w[0]->K, M);
+  if (M < 2 || M > 8 * TC || N < 1024) return false;
+  if (M <= 2 * TC) return true;
+  const int64_t tiles = N / 32, passes = (M + TC - 1) / TC, rounds = (w[0]->K / 32 + BR - 1) / BR;
+  return tiles * passes * (rounds + 1) <= 6000;
+}
+
+int launch_gemm_rows_q40_multi(int count, const hipq_weight *const *w, const QAct *qa, int M, float *const *C,
+                               const int64_t *ldc, hipStream_t s) {
+  if (count < 1 || count > 4) return fail(HIPQ_ERR_INVALID_ARGUMENT, "the few-rows Q4_0 product takes 1 to 4 weights a launch");
+  if (M < 1 || M > 8 * TC) return fail(HIPQ_ERR_INVALID_ARGUMENT, "the few-rows Q4_0 product takes 1..64 rows");
+  MultiRowsQ40 mw;
+  int tiles = 0;
+  for (int i = 0; i < 4; ++i) {
+    const int j = i < count ? i : count - 1;
+    if (i < count) {
+      if (!rows_q40_can(w[i]) || w[i]->K != qa->K)
+        return fail(HIPQ_ERR_INVALID_ARGUMENT, "the few-rows Q4_0 product takes Q4_0 weights of the rows' K, in whole 256s");
+      tiles += (int)((w[i]->N + 31) / 32);
+    }
+    mw.w[i] = wview(w[j]);
+    mw.C[i] = C[j];
+    mw.ldc[i] = ldc[j];
+    mw.tile_end[i] = tiles; /* unused entries repeat the total: no workgroup lands in them */
+  }
+  hipLaunchKernelGGL(gemm_rows_q40_kernel, dim3((unsigned)tiles, (unsigned)((M + TC - 1) / TC)), dim3(NT), LDS_BYTES, s, mw,
+                     qview(*qa), M);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
+}
+
+int launch_gemm_rows_q40(const hipq_weight *w, const QAct *qa, int M, float *C, int64_t ldc, hipStream_t s) {
+  return launch_gemm_rows_q40_multi(1, &w, qa, M, &C, &ldc, s);
 }
 
 } // namespace hipq

@@ -245,6 +245,10 @@ int launch_gemm_rows_q4k(const hipq_weight *w, const QAct *qa, int M, int pair_r
  * of launch_quantize_q8_0; the weight's planes as they are */
 bool gemm_rows_q40_fits(const hipq_weight *w, int64_t M);
 int launch_gemm_rows_q40(const hipq_weight *w, const QAct *qa, int M, float *C, int64_t ldc, hipStream_t s);
+/* up to four weights of one K against the same rows in one launch (the column tiles side by side in the grid) */
+bool gemm_rows_q40_fits_multi(int count, const hipq_weight *const *w, int64_t M);
+int launch_gemm_rows_q40_multi(int count, const hipq_weight *const *w, const QAct *qa, int M, float *const *C,
+                               const int64_t *ldc, hipStream_t s);
 
 /* moe.hip ----------------------------------------------------------------- */
 /* Variant of the expert MLP. kind 0: h = silu(g) * u, y = down(h) (qwen_moe_layer.cpp:332-392).

@@ -526,6 +526,30 @@ def test_matmul_multi_few_rows_mixed_paths(hipq, cr, m):
         w.destroy()
 
 
+@pytest.mark.parametrize("m,k", [(2, 1024), (8, 1280), (13, 256), (16, 2048), (40, 1024), (64, 512)])
+def test_matmul_multi_q4_0_few_rows_one_launch(hipq, cr, m, k):
+    """A few rows against several Q4_0 weights of one K (Q, K, V or gate, up of a decode step of a
+    batch): the weights' column tiles side by side in one launch of the few-rows kernel, four
+    weights a launch (five make a launch of four and a single product), widths that end inside a
+    32-column tile, outputs with a row stride. Every output carries the reference's bits."""
+    import gpu_util as gu
+    import torch
+    ns = [2048, 1000, 1024, 72, 520]
+    blocks = [_weights(cr, "q4_0", n, k, seed=1400 + i) for i, n in enumerate(ns)]
+    ws = [capi.Weight("q4_0", n, k, b) for n, b in zip(ns, blocks)]
+    a = synth.normal(1410 + m, (m, k))
+    outs = [torch.full((m, n + 8 * i), float("nan"), device="cuda") for i, n in enumerate(ns)]
+    capi.matmul_multi(ws, gu.dev(a), m, outs, ldc=[n + 8 * i for i, n in enumerate(ns)], stream=gu.stream())
+    torch.cuda.synchronize()
+    for i, (n, b, o) in enumerate(zip(ns, blocks, outs)):
+        got = o.cpu().numpy()
+        ref = cr.gemm(cr.oracle(), "q4_0", a, b, n)
+        assert np.array_equal(got[:, :n].view(np.uint32), ref.view(np.uint32)), (n, gu.rel_err(got[:, :n], ref))
+        assert np.isnan(got[:, n:]).all(), "the call wrote between the rows of an output"
+    for w in ws:
+        w.destroy()
+
+
 def test_matmul_multi_mixed_k_formats_prefill(hipq, cr):
     """Q4_K and Q6_K weights in one multi-weight prefill call: both take tiled Q8_K activations, but
     the reference quantizes the rows of a Q4_K product four at a time and those of a Q6_K product one
