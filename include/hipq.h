@@ -199,10 +199,12 @@ HIPQ_API int hipq_matmul_noalloc(hipq_weight_t w, const float *A, int64_t M, int
  *  four weights of one format (K <= 4096, fewer than 32768 rows together, device
  *  memory) is a single kernel launch for all of them. With more than 8 rows the Q4_0
  *  and the Q4_K products go out four weights a launch as well (the column tiles of the
- *  weights side by side in one grid), after the one quantization; so do two or more Q4_0
- *  weights with 2 to 16 rows (a decode step of a batch; to 64 rows on narrow weights), through
- *  the few-rows kernel. Every output equals what hipq_matmul gives for that weight alone, bit
- *  for bit. */
+ *  weights side by side in one grid), after the one quantization; so do two or more Q4_0 or
+ *  Q4_K weights with 2 to 16 rows (a decode step of a batch; to 64 rows on narrow weights),
+ *  through the few-rows kernels, with the reference's bits. Every output equals what
+ *  hipq_matmul gives for that weight alone bit for bit, except where the single call of a
+ *  Q4_K weight takes the prefill GEMM for those rows (then to 1e-4, as every product of that
+ *  kernel). */
 HIPQ_API int hipq_matmul_multi(int count, const hipq_weight_t *w, const float *A,
                                int64_t M, int64_t lda, float *const *C,
                                const int64_t *ldc, int mem, void *stream);

@@ -982,19 +982,46 @@ int hipq_matmul_multi(int count, const hipq_weight_t *w, const float *A, int64_t
   if (M == 1 && hipq::gemv_fuses_quantizer_multi(count, w, A))
     return hipq::launch_gemv_fused_multi(count, w, A, C, s);
   /* one quantization per distinct activation format among the weights */
+  /* two or more Q4_K weights against a few rows: one launch of the few-rows kernel for up to four of
+   * them, where the launch as a whole is wide enough */
+  const hipq_weight *q4k[64];
+  int n_q4k = 0;
+  for (int i = 0; i < count && n_q4k < 64; ++i)
+    if (w[i]->dtype == HIPQ_Q4_K) q4k[n_q4k++] = w[i];
+  const bool q4k_rows_group = n_q4k >= 2 && n_q4k < 64 && hipq::gemm_rows_q4k_fits_multi(n_q4k, q4k, M);
   auto klass = [&](const hipq_weight *x) {
     if (x->dtype == HIPQ_Q4_0) return 0;
+    if (x->dtype == HIPQ_Q4_K && q4k_rows_group) return 5;
     if (wants_rows(x, M, true)) return 5; /* a few rows of Q4_K on the matrix cores: the row form of the MoE kernels */
     if (wants_tiled(x, M)) return x->dtype == HIPQ_Q4_K ? 3 : 4; /* the two tiled forms differ in their rows' quantizer */
     return (x->dtype == HIPQ_Q4_K && M > 1) ? 1 : 2;
   };
   {
+    const hipq_weight *gw[4];
+    float *gc[4];
+    int64_t gl[4];
+    int ng = 0;
     bool first = true;
-    for (int i = 0; i < count; ++i)
-      if (klass(w[i]) == 5) {
-        if ((rc = matmul_rows(w[i], A, M, lda, C[i], ldc[i], s, first ? 0 : 1, Scratch{false, s}))) return rc;
-        first = false;
+    QAct qa{};
+    for (int i = 0; i <= count; ++i) {
+      if (i < count && klass(w[i]) != 5) continue;
+      if (i < count) {
+        if (first) { /* the one quantization, in the row form of the matrix-core kernels */
+          if ((rc = matmul_rows(w[i], A, M, lda, C[i], ldc[i], s, 2, Scratch{false, s}))) return rc;
+          void *mem = nullptr;
+          if ((rc = workspace(s, qact_bytes(1, M, w[i]->K), &mem))) return rc;
+          qa = qact_carve(1, mem, M, w[i]->K);
+          first = false;
+        }
+        if (!w[i]->gt_base && (rc = hipq::ensure_gemm_tiles(const_cast<hipq_weight *>(w[i])))) return rc;
+        gw[ng] = w[i], gc[ng] = C[i], gl[ng] = ldc[i];
+        ++ng;
       }
+      if (ng == 4 || (i == count && ng)) {
+        if ((rc = hipq::launch_gemm_rows_q4k_multi(ng, gw, &qa, (int)M, (int)((M / 4) * 4), gc, gl, s))) return rc;
+        ng = 0;
+      }
+    }
   }
   for (int k = 3; k <= 4; ++k) {
     int members = 0;

@@ -64,11 +64,28 @@ struct RowsRegs {
   rv4i hd;
 };
 
+/* Up to four weights of one K against the same quantized rows as ONE launch: the grid's columns are
+ * the concatenation of the weights' column tiles (Q, K, V or gate, up of a layer). */
+struct MultiRowsQ4K {
+  WView w[4]; /* qs, hdr: the tile copy */
+  float *C[4];
+  int64_t ldc[4];
+  int tile_end[4]; /* running sum of the weights' column tiles */
+};
+
 /* blockIdx.y: the pass, rows 8 y .. 8 y + 7 of the call's M_all (the first pair_all of them under
  * the 4-row rule); the passes of one launch run side by side */
-__global__ __launch_bounds__(NT, 2) void gemm_rows_q4k_kernel(WView w, QView a, int M_all, int pair_all,
-                                                              float *__restrict__ C, int64_t ldc) {
+__global__ __launch_bounds__(NT, 2) void gemm_rows_q4k_kernel(MultiRowsQ4K mw, QView a, int M_all, int pair_all) {
   extern __shared__ __attribute__((aligned(16))) unsigned char rows_lds[];
+  /* which weight this workgroup's column tile belongs to (uniform) */
+  int tile = blockIdx.x, wi = 0;
+  if (tile >= mw.tile_end[0]) wi = 1;
+  if (tile >= mw.tile_end[1]) wi = 2;
+  if (tile >= mw.tile_end[2]) wi = 3;
+  if (wi) tile -= mw.tile_end[wi - 1];
+  const WView w = wi == 0 ? mw.w[0] : wi == 1 ? mw.w[1] : wi == 2 ? mw.w[2] : mw.w[3];
+  float *__restrict__ C = wi == 0 ? mw.C[0] : wi == 1 ? mw.C[1] : wi == 2 ? mw.C[2] : mw.C[3];
+  const int64_t ldc = wi == 0 ? mw.ldc[0] : wi == 1 ? mw.ldc[1] : wi == 2 ? mw.ldc[2] : mw.ldc[3];
   const int K = w.K, nsb = K >> 8;
   const int r0 = blockIdx.y * TC;
   const int M = min(TC, M_all - r0), pair_rows = min(max(pair_all - r0, 0), M);
@@ -76,7 +93,6 @@ __global__ __launch_bounds__(NT, 2) void gemm_rows_q4k_kernel(WView w, QView a, 
   a.d += (size_t)r0 * nsb;
   a.bsum += (size_t)r0 * (K >> 4);
   C += (int64_t)r0 * ldc;
-  const int tile = blockIdx.x;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
   const int lane = threadIdx.x & 63, i32 = lane & 31, g = lane >> 5;
   uint32_t *const lrec = (uint32_t *)(rows_lds + LDS_REC);
@@ -315,18 +331,52 @@ bool gemm_rows_q4k_fits(const hipq_weight *w, int64_t M) {
   return (M == 4 && w->N >= 4096) || (M == 3 && w->N >= 8192);
 }
 
-int launch_gemm_rows_q4k(const hipq_weight *w, const QAct *qa, int M, int pair_rows, float *C, int64_t ldc,
-                         hipStream_t s) {
-  if (M < 1 || M > 8 * TC || w->dtype != HIPQ_Q4_K || qa->K != w->K)
-    return fail(HIPQ_ERR_INVALID_ARGUMENT, "the few-rows Q4_K product takes 1..64 rows");
-  if (!w->gt_base) return fail(HIPQ_ERR_INVALID_ARGUMENT, "the few-rows Q4_K product needs the weight's tile copy");
-  WView v = wview(w);
-  v.qs = w->gt_qs;
-  v.hdr = w->gt_hdr;
-  const unsigned grid = (unsigned)((w->N + 31) / 32);
-  hipLaunchKernelGGL(gemm_rows_q4k_kernel, dim3(grid, (unsigned)((M + TC - 1) / TC)), dim3(NT), LDS_BYTES, s, v, qview(*qa), M, pair_rows, C, ldc);
+/* Several weights of one K in one launch (hipq_matmul_multi): what counts is the launch's width, the
+ * columns of all of them, and the launches it replaces. */
+bool gemm_rows_q4k_fits_multi(int count, const hipq_weight *const *w, int64_t M) {
+  if (count < 2 || M < 2 || M > 8 * TC) return false;
+  int64_t tiles = 0;
+  for (int i = 0; i < count; ++i) {
+    if (w[i]->dtype != HIPQ_Q4_K || w[i]->expert_tiles || w[i]->K % 256 || 16 * w[i]->K > 0x7fffffff ||
+        w[i]->K != w[0]->K)
+      return false;
+    tiles += (w[i]->N + 31) / 32;
+  }
+  if (tiles < 32) return false;
+  if (M <= 2 * TC) return true;
+  return tiles * ((M + TC - 1) / TC) * (w[0]->K / 256) <= 8192;
+}
+
+int launch_gemm_rows_q4k_multi(int count, const hipq_weight *const *w, const QAct *qa, int M, int pair_rows,
+                               float *const *C, const int64_t *ldc, hipStream_t s) {
+  if (count < 1 || count > 4) return fail(HIPQ_ERR_INVALID_ARGUMENT, "the few-rows Q4_K product takes 1 to 4 weights a launch");
+  if (M < 1 || M > 8 * TC) return fail(HIPQ_ERR_INVALID_ARGUMENT, "the few-rows Q4_K product takes 1..64 rows");
+  MultiRowsQ4K mw;
+  int tiles = 0;
+  for (int i = 0; i < 4; ++i) {
+    const int j = i < count ? i : count - 1;
+    if (i < count) {
+      if (w[i]->dtype != HIPQ_Q4_K || w[i]->expert_tiles || qa->K != w[i]->K || 16 * w[i]->K > 0x7fffffff)
+        return fail(HIPQ_ERR_INVALID_ARGUMENT, "the few-rows Q4_K product takes Q4_K weights of the rows' K");
+      if (!w[i]->gt_base) return fail(HIPQ_ERR_INVALID_ARGUMENT, "the few-rows Q4_K product needs the weight's tile copy");
+      tiles += (int)((w[i]->N + 31) / 32);
+    }
+    mw.w[i] = wview(w[j]);
+    mw.w[i].qs = w[j]->gt_qs;
+    mw.w[i].hdr = w[j]->gt_hdr;
+    mw.C[i] = C[j];
+    mw.ldc[i] = ldc[j];
+    mw.tile_end[i] = tiles; /* unused entries repeat the total: no workgroup lands in them */
+  }
+  hipLaunchKernelGGL(gemm_rows_q4k_kernel, dim3((unsigned)tiles, (unsigned)((M + TC - 1) / TC)), dim3(NT), LDS_BYTES, s, mw,
+                     qview(*qa), M, pair_rows);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
+}
+
+int launch_gemm_rows_q4k(const hipq_weight *w, const QAct *qa, int M, int pair_rows, float *C, int64_t ldc,
+                         hipStream_t s) {
+  return launch_gemm_rows_q4k_multi(1, &w, qa, M, pair_rows, &C, &ldc, s);
 }
 
 } // namespace hipq

@@ -239,6 +239,10 @@ size_t gemm_q4k_split_bytes(const hipq_weight *w, int64_t M);
 bool gemm_rows_q4k_fits(const hipq_weight *w, int64_t M);
 int launch_gemm_rows_q4k(const hipq_weight *w, const QAct *qa, int M, int pair_rows, float *C, int64_t ldc,
                          hipStream_t s);
+/* up to four weights of one K against the same rows in one launch (the column tiles side by side in the grid) */
+bool gemm_rows_q4k_fits_multi(int count, const hipq_weight *const *w, int64_t M);
+int launch_gemm_rows_q4k_multi(int count, const hipq_weight *const *w, const QAct *qa, int M, int pair_rows,
+                               float *const *C, const int64_t *ldc, hipStream_t s);
 
 /* gemm_rows_q40.hip: Q4_0 for a few rows on the matrix cores with the reference's bits (rows are
  * independent in this format); fits: the row counts and shapes that should take it; qa in the form

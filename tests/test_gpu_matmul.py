@@ -550,6 +550,33 @@ def test_matmul_multi_q4_0_few_rows_one_launch(hipq, cr, m, k):
         w.destroy()
 
 
+@pytest.mark.parametrize("m,k", [(2, 1024), (3, 512), (6, 1280), (13, 256), (16, 2048), (40, 1024)])
+def test_matmul_multi_q4_K_few_rows_one_launch(hipq, cr, m, k):
+    """The same for Q4_K weights: one quantization in the row form of the matrix-core kernels (rows
+    below 4 * (m / 4) under the 4-row rule), then the weights' column tiles side by side in one launch
+    of gemm_rows_q4k.hip, four weights a launch. The reference's bits for every output, and the bits
+    of the single-weight call where that one keeps them (the single call of a wide weight with more
+    than 16 rows takes the prefill GEMM, which agrees to 1e-4)."""
+    import gpu_util as gu
+    import torch
+    ns = [2048, 1000, 1024, 72, 520]
+    blocks = [_weights(cr, "q4_K", n, k, seed=1500 + i) for i, n in enumerate(ns)]
+    ws = [capi.Weight("q4_K", n, k, b) for n, b in zip(ns, blocks)]
+    a = synth.normal(1510 + m, (m, k))
+    a[1, 3] = 8.5
+    a[1, 7] = -8.5
+    outs = [torch.full((m, n + 8 * i), float("nan"), device="cuda") for i, n in enumerate(ns)]
+    capi.matmul_multi(ws, gu.dev(a), m, outs, ldc=[n + 8 * i for i, n in enumerate(ns)], stream=gu.stream())
+    torch.cuda.synchronize()
+    for i, (n, b, o) in enumerate(zip(ns, blocks, outs)):
+        got = o.cpu().numpy()
+        ref = cr.gemm(cr.oracle(), "q4_K", a, b, n)
+        assert np.array_equal(got[:, :n].view(np.uint32), ref.view(np.uint32)), (n, gu.rel_err(got[:, :n], ref))
+        assert np.isnan(got[:, n:]).all(), "the call wrote between the rows of an output"
+    for w in ws:
+        w.destroy()
+
+
 def test_matmul_multi_mixed_k_formats_prefill(hipq, cr):
     """Q4_K and Q6_K weights in one multi-weight prefill call: both take tiled Q8_K activations, but
     the reference quantizes the rows of a Q4_K product four at a time and those of a Q6_K product one
