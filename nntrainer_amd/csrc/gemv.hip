@@ -39,11 +39,12 @@ __global__ __launch_bounds__(256) void gemv_kernel(WView w, QView qa, int M, int
 /* Decode GEMV for large matrices: a wavefront owns GPW consecutive groups of G
  * rows. The activation row is loaded once, and the weight loads of the next
  * group are in flight while the current one is computed, so the HBM stream of a
- * wavefront never drains. One chunk only (K <= 4096). */
-template <int DT, int G, int GPW>
+ * wavefront never drains. T lanes a row (64, or 16 for rows of fewer than 64 units). One chunk only
+ * (K <= 4096). */
+template <int DT, int T, int G, int GPW>
 __global__ __launch_bounds__(256) void gemv_stream_kernel(WView w, QView qa,
                                                           float *__restrict__ C) {
-  typedef GemvCore<DT, 64, 1, G, false> E;
+  typedef GemvCore<DT, T, 1, G, false> E;
   extern __shared__ uint32_t gemv_lds[];
   const int wave = threadIdx.x >> 6;
   uint32_t *lds = gemv_lds + wave * GemvLds<DT, 1, G, false>::DWORDS;
@@ -246,12 +247,12 @@ int launch_fused_one(const hipq_weight *w, const float *x, float *C, hipStream_t
   return HIPQ_OK;
 }
 
-template <int DT, int G, int GPW>
+template <int DT, int T, int G, int GPW>
 int launch_stream(const hipq_weight *w, const QAct *qa, float *C, hipStream_t s) {
   const int rows_per_block = 4 * G * GPW;
   const unsigned grid = (unsigned)((w->N + rows_per_block - 1) / rows_per_block);
   const size_t lds = 4 * GemvLds<DT, 1, G, false>::DWORDS * sizeof(uint32_t);
-  hipLaunchKernelGGL((gemv_stream_kernel<DT, G, GPW>), dim3(grid), dim3(256), lds, s, wview(w),
+  hipLaunchKernelGGL((gemv_stream_kernel<DT, T, G, GPW>), dim3(grid), dim3(256), lds, s, wview(w),
                      qview(*qa), C);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
@@ -307,7 +308,14 @@ int launch_m1(const hipq_weight *w, const QAct *qa, float *C, int64_t ldc, hipSt
    * the next group's loads in flight gain 3 % (Q4_K) to 20 % (Q4_0); Q6_K and
    * smaller matrices are better off with more, shorter wavefronts */
   if (DT != HIPQ_Q6_K && w->N >= 32768 && w->K <= HIPQ_KCHUNK && units >= 64)
-    return launch_stream<DT, 4, 2>(w, qa, C, s);
+    return launch_stream<DT, 64, 4, 2>(w, qa, C, s);
+  /* the same for short rows (16 lanes a row, four rows side by side, eight a group): a wavefront of
+   * the plain kernel below would have four short rows for all its work. Kernel us, plain -> streamed:
+   * Q4_K 151936 x 1024 38.0 -> 31.9, 151936 x 256 27.9 -> 21.8, 65536 x 512 13.2 -> 10.7, 32768 x 1024
+   * 9.4 -> 8.0; Q4_0 32768 x 1024 8.4 -> 6.9 (wider Q4_0 matrices take the few-rows kernel); Q6_K is
+   * the slower for it (151936 x 1024 34.6 -> 38.0) and stays */
+  if (DT != HIPQ_Q6_K && w->N >= 32768 && w->K <= HIPQ_KCHUNK && units < 64)
+    return DT == HIPQ_Q4_0 ? launch_stream<DT, 16, 8, 2>(w, qa, C, s) : launch_stream<DT, 16, 8, 4>(w, qa, C, s);
   if (units < 64) { /* short rows: 16 lanes per row, 4 rows streamed at once */
     if (pick_group(w->N, 8) == 8) return launch_one<DT, 16, 1, 8, false>(w, qa, 1, 0, C, ldc, s);
     return launch_one<DT, 16, 1, 4, false>(w, qa, 1, 0, C, ldc, s);

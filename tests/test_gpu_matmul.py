@@ -111,6 +111,24 @@ def test_q4_0_few_rows_on_the_matrix_cores_match_oracle(hipq, cr, m, n, k):
 
 
 @pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("n,k", [(32800, 1024), (33000, 512), (40010, 256), (32768, 768), (50000, 1280)])
+def test_single_row_against_wide_matrices_of_short_rows(hipq, cr, kind, n, k):
+    """One row against 32768 columns or more with rows of fewer than 64 load units: Q4_0 and Q4_K
+    stream them sixteen lanes a row, eight rows a group and two or four groups a wavefront with the
+    next group's loads in flight (Q6_K keeps the plain kernel); column counts that end inside a
+    group and inside a workgroup's share. Same bits as the reference."""
+    import gpu_util as gu
+    blocks = _weights(cr, kind, n, k, seed=1600 + k)
+    a = synth.normal(1601 + n, (1, k))
+    ref = cr.gemm(cr.oracle(), kind, a, blocks, n)
+    w = capi.Weight(kind, n, k, blocks)
+    got = gu.gpu_matmul(w, a)
+    w.destroy()
+    assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), \
+        "%d of %d outputs differ in bits" % ((got.view(np.uint32) != ref.view(np.uint32)).sum(), got.size)
+
+
+@pytest.mark.parametrize("kind", KINDS)
 @pytest.mark.parametrize("m,n,k", [(1, 8200, 12288), (3, 200, 8192), (8, 520, 9216), (1, 96, 20480),
                                    (5, 64, 4352)])
 def test_rows_longer_than_one_chunk_match_oracle(hipq, cr, kind, m, n, k):
