@@ -444,6 +444,10 @@ int matmul_device(hipq_weight_t w, const float *A, int64_t M, int64_t lda, float
   if (wants_rows(w, M, !sc.fixed)) return matmul_rows(w, A, M, lda, C, ldc, s, 0, sc, each_row);
   if (!each_row && wants_tiled(w, M, !sc.fixed)) return matmul_tiled(w, A, M, lda, C, ldc, s, 0, sc);
   if (M == 1 && hipq::gemv_fuses_quantizer(w, A)) return hipq::launch_gemv_fused(w, A, C, s);
+  {
+    const hipq_weight *one = w;
+    if (hipq::gemm_rows_q40_fuses(1, &one, M, A, lda)) return hipq::launch_gemm_rows_q40_fused(1, &one, A, lda, (int)M, &C, &ldc, s);
+  }
   const int is_k = w->dtype != HIPQ_Q4_0;
   void *mem = nullptr;
   int rc = sc.get(qact_bytes(is_k, M, w->K), &mem);
@@ -1065,6 +1069,21 @@ int hipq_matmul_multi(int count, const hipq_weight_t *w, const float *A, int64_t
       }
     if (first < 0) continue;
     const int is_k = k != 0;
+    if (k == 0) { /* up to four Q4_0 weights and a few rows: one launch that quantizes the rows itself */
+      const hipq_weight *fw[4];
+      float *fc[4];
+      int64_t fl[4];
+      int nf = 0, members = 0;
+      for (int i = 0; i < count; ++i)
+        if (klass(w[i]) == 0) {
+          if (nf < 4) fw[nf] = w[i], fc[nf] = C[i], fl[nf] = ldc[i], ++nf;
+          ++members;
+        }
+      if (members <= 4 && hipq::gemm_rows_q40_fuses(nf, fw, M, A, lda)) {
+        if ((rc = hipq::launch_gemm_rows_q40_fused(nf, fw, A, lda, (int)M, fc, fl, s))) return rc;
+        continue;
+      }
+    }
     void *memp = nullptr;
     if ((rc = workspace(s, qact_bytes(is_k, M, w[0]->K), &memp))) return rc;
     QAct qa = qact_carve(is_k, memp, M, w[0]->K);
@@ -1143,6 +1162,11 @@ int hipq_time_matmul(int n_weights, const hipq_weight_t *w, const float *A, int6
     }
     if (rows) {
       rc = matmul_rows(wi, A, M, lda, C, ldc, s, phase, Scratch{false, s});
+      continue;
+    }
+    if (phase == 0 && hipq::gemm_rows_q40_fuses(1, &wi, M, A, lda)) {
+      float *cc = C;
+      rc = hipq::launch_gemm_rows_q40_fused(1, &wi, A, lda, (int)M, &cc, &ldc, s);
       continue;
     }
     if (phase == 0 && M == 1 && hipq::gemv_fuses_quantizer(wi, A)) {

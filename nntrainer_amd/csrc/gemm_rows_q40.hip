@@ -31,6 +31,7 @@
  */
 #include "hipq_internal.h"
 #include "gemv_device.h"
+#include "quantize_device.h"
 
 namespace {
 
@@ -88,7 +89,13 @@ struct MultiRowsQ40 {
   int tile_end[4]; /* running sum of the weights' column tiles */
 };
 
-__global__ __launch_bounds__(NT, 2) void gemm_rows_q40_kernel(MultiRowsQ40 mw, QView a, int M_all) {
+/* FUSED: the rows come as fp32 (Af, row stride lda) and every workgroup quantizes its pass's rows
+ * itself, a round ahead, with the arithmetic of the Q8_0 quantizer kernel (the same bits): no
+ * quantizer launch and no workspace. For launches of few workgroups, where that launch costs more
+ * than the repeated quantization. */
+template <bool FUSED>
+__global__ __launch_bounds__(NT, 2) void gemm_rows_q40_kernel(MultiRowsQ40 mw, QView a, const float *__restrict__ Af,
+                                                              int64_t lda, int M_all) {
   extern __shared__ __attribute__((aligned(16))) unsigned char rows_lds[];
   /* which weight this workgroup's column tile belongs to (uniform) */
   int tile = blockIdx.x, wi = 0;
@@ -102,8 +109,12 @@ __global__ __launch_bounds__(NT, 2) void gemm_rows_q40_kernel(MultiRowsQ40 mw, Q
   const int K = w.K, nb = K >> 5;
   const int r0 = blockIdx.y * TC;
   const int M = min(TC, M_all - r0);
-  a.q += (size_t)r0 * K;
-  a.meta += (size_t)r0 * nb;
+  if (FUSED) {
+    Af += (int64_t)r0 * lda;
+  } else {
+    a.q += (size_t)r0 * K;
+    a.meta += (size_t)r0 * nb;
+  }
   C += (int64_t)r0 * ldc;
   const int n0 = tile * 32;
   const int ncols = min(32, w.N - n0);
@@ -146,7 +157,7 @@ __global__ __launch_bounds__(NT, 2) void gemm_rows_q40_kernel(MultiRowsQ40 mw, Q
   };
   const uint16_t *const dcol = w.d + (size_t)(n0 + min(t >> 3, ncols - 1)) * nb;
   auto s_load = [&](SRegs &r, int rho) {
-    r.meta = a.meta[(size_t)min(t >> 5, M - 1) * nb + min(rho * BR + (t & 31), nb - 1)];
+    if (!FUSED) r.meta = a.meta[(size_t)min(t >> 5, M - 1) * nb + min(rho * BR + (t & 31), nb - 1)];
     r.dw = *(const uint2 *)(dcol + min(rho * BR + (t & 7) * 4, nb - 4));
   };
   auto s_store = [&](const SRegs &r) {
@@ -157,16 +168,48 @@ __global__ __launch_bounds__(NT, 2) void gemm_rows_q40_kernel(MultiRowsQ40 mw, Q
     *(qv4f *)(rows_lds + LDS_DW + ((t & 7) * 32 + (t >> 3)) * 16) = f; /* [four blocks][column][4] */
   };
 
+  /* FUSED: a thread takes one block of a round, row t / 32, block t % 32: 32 fp32 values in, its 32
+   * int8 values to LDS, the block's metadata word (fp16 scale, sum of the values) back */
+  struct FRegs {
+    float4 x[FUSED ? 8 : 1];
+  };
+  auto f_load = [&](FRegs &r, int rho) {
+    const float4 *p = (const float4 *)(Af + (int64_t)min(t >> 5, M - 1) * lda + min(rho * (BR * 32) + (t & 31) * 32, K - 32));
+#pragma unroll
+    for (int i = 0; i < 8; ++i) r.x[i] = p[i];
+  };
+  auto f_quant_store = [&](const FRegs &r) -> uint32_t {
+    float amax = 0.f;
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      amax = fmaxf(amax, fmaxf(fmaxf(fabsf(r.x[i].x), fabsf(r.x[i].y)), fmaxf(fabsf(r.x[i].z), fabsf(r.x[i].w))));
+    const float d = __fdiv_rn(amax, 127.f);
+    const float id = (amax != 0.0f) ? __fdiv_rn(127.f, amax) : 0.0f;
+    int pk[8], sum = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int q0 = (int)rintf(__fmul_rn(r.x[i].x, id)), q1 = (int)rintf(__fmul_rn(r.x[i].y, id));
+      const int q2 = (int)rintf(__fmul_rn(r.x[i].z, id)), q3 = (int)rintf(__fmul_rn(r.x[i].w, id));
+      pk[i] = pack4(q0, q1, q2, q3);
+      sum += (q0 + q1) + (q2 + q3);
+    }
+    unsigned char *dst = rows_lds + LDS_Q + (t >> 5) * QROW + (t & 31) * 32;
+    *(qv4i *)dst = qv4i{pk[0], pk[1], pk[2], pk[3]};
+    *(qv4i *)(dst + 16) = qv4i{pk[4], pk[5], pk[6], pk[7]};
+    return (uint32_t)hipq_f2h(d) | ((uint32_t)(sum & 0xffff) << 16);
+  };
+
   constexpr int PD = 1, NB = PD + 1;
   WRegs buf[NB];
   qv4i AQ[2];
+  FRegs FR;
   SRegs SR;
   const int rounds = (nb + BR - 1) / BR;
-  q_load(AQ, 0);
+  if (FUSED) f_load(FR, 0); else q_load(AQ, 0);
   s_load(SR, 0);
 #pragma unroll
   for (int p = 0; p < PD; ++p) load(buf[p], p);
-  q_store(AQ);
+  if (FUSED) SR.meta = f_quant_store(FR); else q_store(AQ);
   __syncthreads();
 
   /* the output this thread chains: row cm, column cn; its sums sit in register cr of lane cl */
@@ -217,7 +260,8 @@ __global__ __launch_bounds__(NT, 2) void gemm_rows_q40_kernel(MultiRowsQ40 mw, Q
       }
     }
     __syncthreads();
-    q_store(AQ); /* the next round's values: nobody reads this round's any more */
+    /* the next round's values: nobody reads this round's any more */
+    if (FUSED) SR.meta = f_quant_store(FR); else q_store(AQ);
     /* the chains of this round's blocks, ascending (the records of a wavefront that had no blocks
      * are read as well and not used: a read behind a branch would wait for its own latency) */
     const float *lda_ = (const float *)(rows_lds + LDS_DA) + cm * BR;
@@ -252,7 +296,8 @@ __global__ __launch_bounds__(NT, 2) void gemm_rows_q40_kernel(MultiRowsQ40 mw, Q
       const int rho = rho0 + u;
       if (rho < rounds) {
         s_store(SR); /* this round's scales: the chains of the round before have passed their barrier */
-        q_load(AQ, rho + 1); /* before the weights: their waits must not include the weights' */
+        /* before the weights: their waits must not include the weights' */
+        if (FUSED) f_load(FR, rho + 1); else q_load(AQ, rho + 1);
         s_load(SR, rho + 1);
         load(buf[(u + PD) % NB], rho + PD);
         round(buf[u], rho);
@@ -313,8 +358,9 @@ bool gemm_rows_q40_fits_multi(int count, const hipq_weight *const *w, int64_t M)
   return tiles * passes * (rounds + 1) <= 6000;
 }
 
-int launch_gemm_rows_q40_multi(int count, const hipq_weight *const *w, const QAct *qa, int M, float *const *C,
-                               const int64_t *ldc, hipStream_t s) {
+/* qa: the quantized rows, or null with the fp32 rows A (row stride lda) for the form that quantizes them itself */
+static int launch_rows_q40(int count, const hipq_weight *const *w, const QAct *qa, const float *A, int64_t lda, int M,
+                           float *const *C, const int64_t *ldc, hipStream_t s) {
   if (count < 1 || count > 4) return fail(HIPQ_ERR_INVALID_ARGUMENT, "the few-rows Q4_0 product takes 1 to 4 weights a launch");
   if (M < 1 || M > 8 * TC) return fail(HIPQ_ERR_INVALID_ARGUMENT, "the few-rows Q4_0 product takes 1..64 rows");
   MultiRowsQ40 mw;
@@ -322,7 +368,7 @@ int launch_gemm_rows_q40_multi(int count, const hipq_weight *const *w, const QAc
   for (int i = 0; i < 4; ++i) {
     const int j = i < count ? i : count - 1;
     if (i < count) {
-      if (!rows_q40_can(w[i]) || w[i]->K != qa->K)
+      if (!rows_q40_can(w[i]) || w[i]->K != (qa ? qa->K : w[0]->K))
         return fail(HIPQ_ERR_INVALID_ARGUMENT, "the few-rows Q4_0 product takes Q4_0 weights of the rows' K, in whole 256s");
       tiles += (int)((w[i]->N + 31) / 32);
     }
@@ -331,10 +377,41 @@ int launch_gemm_rows_q40_multi(int count, const hipq_weight *const *w, const QAc
     mw.ldc[i] = ldc[j];
     mw.tile_end[i] = tiles; /* unused entries repeat the total: no workgroup lands in them */
   }
-  hipLaunchKernelGGL(gemm_rows_q40_kernel, dim3((unsigned)tiles, (unsigned)((M + TC - 1) / TC)), dim3(NT), LDS_BYTES, s, mw,
-                     qview(*qa), M);
+  const dim3 grid((unsigned)tiles, (unsigned)((M + TC - 1) / TC));
+  if (qa) {
+    hipLaunchKernelGGL(gemm_rows_q40_kernel<false>, grid, dim3(NT), LDS_BYTES, s, mw, qview(*qa), (const float *)nullptr,
+                       (int64_t)0, M);
+  } else {
+    QView none{};
+    none.K = (int)w[0]->K;
+    hipLaunchKernelGGL(gemm_rows_q40_kernel<true>, grid, dim3(NT), LDS_BYTES, s, mw, none, A, lda, M);
+  }
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
+}
+
+int launch_gemm_rows_q40_multi(int count, const hipq_weight *const *w, const QAct *qa, int M, float *const *C,
+                               const int64_t *ldc, hipStream_t s) {
+  return launch_rows_q40(count, w, qa, nullptr, 0, M, C, ldc, s);
+}
+
+/* The form that quantizes the fp32 rows itself: where the launch would take the few-rows kernel
+ * anyway, is small, and K is one round: the kernel then starts a microsecond later (fp32 rows in,
+ * quantized, a barrier before the first matrix step) and saves a quantizer launch of 2.5 us.
+ * Whole calls, us, two launches -> one: 3072 x 1024 with 8 rows 7.0 -> 5.7, 2048 x 1024 with 16 rows
+ * 6.7 -> 5.5, 1024 x 1024 6.7 -> 5.6; with three rounds it loses (1024 x 3072 with 16 rows 9.4 ->
+ * 10.1), with two it gains nothing (512 x 2048 7.7 -> 7.8). */
+bool gemm_rows_q40_fuses(int count, const hipq_weight *const *w, int64_t M, const float *A, int64_t lda) {
+  if (!gemm_rows_q40_fits_multi(count, w, M) || ((uintptr_t)A & 15) || (lda & 3)) return false;
+  int64_t tiles = 0;
+  for (int i = 0; i < count; ++i) tiles += (w[i]->N + 31) / 32;
+  return w[0]->K <= BR * 32 && tiles <= 512;
+}
+
+int launch_gemm_rows_q40_fused(int count, const hipq_weight *const *w, const float *A, int64_t lda, int M,
+                               float *const *C, const int64_t *ldc, hipStream_t s) {
+  if (((uintptr_t)A & 15) || (lda & 3)) return fail(HIPQ_ERR_INVALID_ARGUMENT, "activation rows must be 16-byte aligned");
+  return launch_rows_q40(count, w, nullptr, A, lda, M, C, ldc, s);
 }
 
 int launch_gemm_rows_q40(const hipq_weight *w, const QAct *qa, int M, float *C, int64_t ldc, hipStream_t s) {

@@ -253,6 +253,11 @@ int launch_gemm_rows_q40(const hipq_weight *w, const QAct *qa, int M, float *C, 
 bool gemm_rows_q40_fits_multi(int count, const hipq_weight *const *w, int64_t M);
 int launch_gemm_rows_q40_multi(int count, const hipq_weight *const *w, const QAct *qa, int M, float *const *C,
                                const int64_t *ldc, hipStream_t s);
+/* the same on the fp32 rows themselves (the workgroups quantize them: no quantizer launch, no workspace),
+ * for small launches; fuses: whether a product should take it */
+bool gemm_rows_q40_fuses(int count, const hipq_weight *const *w, int64_t M, const float *A, int64_t lda);
+int launch_gemm_rows_q40_fused(int count, const hipq_weight *const *w, const float *A, int64_t lda, int M,
+                               float *const *C, const int64_t *ldc, hipStream_t s);
 
 /* moe.hip ----------------------------------------------------------------- */
 /* Variant of the expert MLP. kind 0: h = silu(g) * u, y = down(h) (qwen_moe_layer.cpp:332-392).
