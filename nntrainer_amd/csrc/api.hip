@@ -1053,6 +1053,20 @@ int hipq_matmul_multi(int count, const hipq_weight_t *w, const float *A, int64_t
       if (ng && (rc = hipq::launch_gemm_q4k_multi(ng, gw, &qa, (int)M, gc, gl, s))) return rc;
       continue;
     }
+    if (members > 1) {
+      /* the products after the first read the activations the first one quantized: the workspace must
+       * not grow (and move) between them, so it is sized for the largest member first (a product of
+       * few tiles keeps its partial products of parts of K behind the activations) */
+      size_t parts_max = 0;
+      for (int i = 0; i < count; ++i) {
+        if (klass(w[i]) != k) continue;
+        if (!w[i]->gt_base && (rc = hipq::ensure_gemm_tiles(const_cast<hipq_weight *>(w[i])))) return rc;
+        const size_t pb = w[i]->dtype == HIPQ_Q4_K ? hipq::gemm_q4k_split_bytes(w[i], M) : hipq::gemm_q6k_split_bytes(w[i], M);
+        if (pb > parts_max) parts_max = pb;
+      }
+      void *reserve = nullptr;
+      if ((rc = workspace(s, ((qact_tiled_bytes(M, w[0]->K) + 255) & ~(size_t)255) + parts_max, &reserve))) return rc;
+    }
     bool first = true;
     for (int i = 0; i < count; ++i)
       if (klass(w[i]) == k) {

@@ -595,6 +595,34 @@ def test_matmul_multi_q4_K_few_rows_one_launch(hipq, cr, m, k):
         w.destroy()
 
 
+@pytest.mark.parametrize("ns", [[72, 3072], [3072, 72, 1000]])
+def test_matmul_multi_q6_K_members_of_different_size_share_the_quantization(hipq, cr, ns):
+    """Q6_K weights of one multi-weight call share the quantized rows of the first one's product. A
+    product of few tiles keeps its partial products of parts of K behind those rows in the same
+    workspace, and a later, larger member needs more of it: the workspace is sized for the largest
+    member before the first product, so that it does not move between them. A fresh stream, so that
+    the workspace starts empty."""
+    import gpu_util as gu
+    import torch
+    m, k = 65, 2048
+    blocks = [_weights(cr, "q6_K", n, k, seed=1700 + i) for i, n in enumerate(ns)]
+    ws = [capi.Weight("q6_K", n, k, b) for n, b in zip(ns, blocks)]
+    a = synth.normal(1710, (m, k))
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        da = gu.dev(a)
+        outs = [torch.full((m, n), float("nan"), device="cuda") for n in ns]
+        side.synchronize()
+        capi.matmul_multi(ws, da, m, outs, stream=side.cuda_stream)
+        side.synchronize()
+    for n, b, o in zip(ns, blocks, outs):
+        got = o.cpu().numpy()
+        assert not np.isnan(got).any()
+        assert gu.rel_err(got, cr.gemm(cr.oracle(), "q6_K", a, b, n)) <= gu.TOL, n
+    for w in ws:
+        w.destroy()
+
+
 def test_matmul_multi_mixed_k_formats_prefill(hipq, cr):
     """Q4_K and Q6_K weights in one multi-weight prefill call: both take tiled Q8_K activations, but
     the reference quantizes the rows of a Q4_K product four at a time and those of a Q6_K product one
