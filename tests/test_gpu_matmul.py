@@ -623,6 +623,51 @@ def test_matmul_multi_q6_K_members_of_different_size_share_the_quantization(hipq
         w.destroy()
 
 
+def test_matmul_multi_seeded_mixed_calls(hipq, cr):
+    """Forty multi-weight calls drawn from a seeded generator: one to seven weights of mixed formats
+    and widths, one to 130 rows, every second call on a stream of its own (an empty workspace).
+    Whatever grouping the call chooses (one launch for several weights, shared quantizations, parts
+    of K), every output is within 1e-4 of the reference and Q4_0 outputs carry its bits."""
+    import gpu_util as gu
+    import torch
+    rng = np.random.default_rng(7)
+    cache = {}
+
+    def blocks_of(kind, n, k):
+        if (kind, n, k) not in cache:
+            cache[(kind, n, k)] = _weights(cr, kind, n, k, seed=2000 + n + k + len(kind))
+        return cache[(kind, n, k)]
+
+    for it in range(40):
+        k = int(rng.choice([256, 512, 1024, 1280, 2048]))
+        cnt = int(rng.integers(1, 8))
+        kinds = [str(rng.choice(["q4_0", "q4_0", "q4_K", "q4_K", "q6_K"])) for _ in range(cnt)]
+        ns = [int(rng.choice([72, 256, 520, 1000, 1024, 2048, 3072, 4100])) for _ in range(cnt)]
+        m = int(rng.choice([1, 2, 3, 4, 5, 8, 9, 13, 16, 17, 31, 40, 64, 65, 130]))
+        a = synth.normal(3000 + it, (m, k))
+        if m > 1:
+            a[1, 3] = 7.5
+            a[1, 9] = -7.5
+        blocks = [blocks_of(kd, n, k) for kd, n in zip(kinds, ns)]
+        ws = [capi.Weight(kd, n, k, b) for kd, n, b in zip(kinds, ns, blocks)]
+        outs = [torch.full((m, n), float("nan"), device="cuda") for n in ns]
+        da = gu.dev(a)
+        st = torch.cuda.Stream() if it % 2 else torch.cuda.current_stream()
+        torch.cuda.synchronize()
+        capi.matmul_multi(ws, da, m, outs, stream=st.cuda_stream)
+        torch.cuda.synchronize()
+        for kd, n, b, o in zip(kinds, ns, blocks, outs):
+            got = o.cpu().numpy()
+            ref = cr.gemm(cr.oracle(), kd, a, b, n)
+            case = (it, m, k, kd, n)
+            assert not np.isnan(got).any(), case
+            assert gu.rel_err(got, ref) <= gu.TOL, case
+            if kd == "q4_0":
+                assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), case
+        for w in ws:
+            w.destroy()
+
+
 def test_matmul_multi_mixed_k_formats_prefill(hipq, cr):
     """Q4_K and Q6_K weights in one multi-weight prefill call: both take tiled Q8_K activations, but
     the reference quantizes the rows of a Q4_K product four at a time and those of a Q6_K product one
