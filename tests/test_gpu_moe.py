@@ -58,6 +58,49 @@ def test_moe_matches_oracle(hipq, cr, t, h, i, e, k):
         w.destroy()
 
 
+def test_moe_seeded_blocks(hipq, cr):
+    """Twenty-four blocks drawn from a seeded generator: one to 130 tokens, 4 to 64 experts, top-1 to
+    top-8, hidden sizes 256 to 2048, a third of them with one expert favoured by every token, every
+    second one on a stream of its own. Expert choices identical, outputs within 2e-6."""
+    import gpu_util as gu
+    import torch
+    rng = np.random.default_rng(5)
+    cache = {}
+    for it in range(24):
+        h = int(rng.choice([256, 512, 1024, 2048]))
+        i = int(rng.choice([256, 512, 768]))
+        e = int(rng.choice([4, 8, 16, 32, 64]))
+        k = min(int(rng.choice([1, 2, 4, 8])), e)
+        t = int(rng.choice([1, 2, 3, 7, 8, 9, 16, 17, 31, 40, 64, 100, 130]))
+        if (e, i, h) not in cache:
+            if len(cache) > 4:
+                cache.clear()
+            cache[(e, i, h)] = _experts(cr, e, i, h, seed=100 + h)
+        gate, up, down = cache[(e, i, h)]
+        x = synth.normal(7000 + it, (t, h))
+        logits = synth.normal(7100 + it, (t, e))
+        if rng.random() < 0.3:
+            logits[:, int(rng.integers(0, e))] += 6.0
+        ref_y, ref_idx, _ = cr.moe_forward(x, logits, gate, up, down, k)
+        wg = [capi.Weight("q4_K", i, h, b) for b in gate]
+        wu = [capi.Weight("q4_K", i, h, b) for b in up]
+        wd = [capi.Weight("q4_K", h, i, b) for b in down]
+        dx, dl = gu.dev(x), gu.dev(logits)
+        y = torch.full((t, h), float("nan"), device="cuda")
+        idx = torch.zeros((t, k), dtype=torch.int32, device="cuda")
+        st = torch.cuda.Stream() if it % 2 else torch.cuda.current_stream()
+        torch.cuda.synchronize()
+        capi.moe_forward(t, h, i, e, k, wg, wu, wd, dx, y, router_logits=dl, topk_idx=idx, stream=st.cuda_stream)
+        torch.cuda.synchronize()
+        case = (it, t, h, i, e, k)
+        assert np.array_equal(idx.cpu().numpy(), ref_idx), case
+        got = y.cpu().numpy()
+        assert not np.isnan(got).any(), case
+        assert gu.rel_err(got, ref_y) <= 2e-6, (case, gu.rel_err(got, ref_y))
+        for w in wg + wu + wd:
+            w.destroy()
+
+
 @pytest.mark.parametrize("t,h,i,e,k", [(64, 512, 256, 32, 2), (64, 256, 256, 16, 2), (96, 256, 256, 8, 2)])
 def test_moe_skewed_routing(hipq, cr, t, h, i, e, k):
     """Every token chooses expert 0: it holds far more slots than a work item (8, 16 or
