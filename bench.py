@@ -355,6 +355,54 @@ def main():
     c5_prefill_graph_ms, c5_prefill_grouped_ms = decode_layer_graph(0, 512), decode_layer_graph(1, 512)
     c5_rows8_grouped_ms = decode_layer_graph(1, 8)
 
+    def q4k_qkv_rows(rows, copies=6):
+        """Q, K, V of a 4096-wide layer with grouped-query attention (4096, 1024, 1024 x 4096, Q4_K) against
+        `rows` rows as ONE hipq_matmul_multi call, replayed from a graph: milliseconds per call."""
+        ns_ = (4096, 1024, 1024)
+        sets_ = []
+        for _ in range(copies):
+            ws_ = []
+            for n_ in ns_:
+                w32_ = torch.randn((n_, K), generator=gen, device="cuda", dtype=torch.float32) * 0.02
+                b_ = torch.empty(capi.weight_nbytes("q4_K", n_, K), dtype=torch.uint8, device="cuda")
+                capi.quantize_weights("q4_K", w32_, n_, K, b_, stream=stream)
+                torch.cuda.synchronize()
+                ws_.append(capi.Weight("q4_K", n_, K, b_, mem=capi.MEM_DEVICE))
+            sets_.append(ws_)
+        x_ = torch.randn((rows, K), generator=gen, device="cuda")
+        cs_ = [torch.empty((rows, n_), device="cuda") for n_ in ns_]
+
+        def step(st):
+            for ws_ in sets_:
+                capi.matmul_multi(ws_, x_, rows, cs_, stream=st)
+
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            step(side.cuda_stream)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=side):
+            step(side.cuda_stream)
+        for _ in range(3):
+            graph.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for _ in range(20):
+            graph.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / (20 * copies)
+        del graph
+        for ws_ in sets_:
+            for w_ in ws_:
+                w_.destroy()
+        return ms
+
+    q4k_qkv_ms = {r_: q4k_qkv_rows(r_) for r_ in (1, 8, 16)}
+
     # ---- the MoE block of configs[3]: 64 tokens, 128 experts, top-8, Q4_K ----------
     mt, mh, me, mi, mk = 64, 2048, 128, 768, 8
 
@@ -493,8 +541,12 @@ def main():
             "rows_8_weight_gbs": round(gv_bytes / (rows_ms[8][0] * 1e-3) / 1e9, 2),
             "rows_16_kernel_ms": round(rows_ms[16][0], 5), "rows_16_ms_per_call": round(rows_ms[16][1], 5),
             "rows_64_kernel_ms": round(rows_ms[64][0], 5), "rows_64_ms_per_call": round(rows_ms[64][1], 5),
+            "qkv_4096_1024_1024_as_one_call_in_a_graph_ms": {"rows_1": round(q4k_qkv_ms[1], 5),
+                                                             "rows_8": round(q4k_qkv_ms[8], 5),
+                                                             "rows_16": round(q4k_qkv_ms[16], 5)},
             "note": "16 rows: two passes of the same kernel, still the reference's bits; 64 rows: the prefill GEMM "
-                    "in parts of K (one 64-row tile per 128 columns), within 1e-4"},
+                    "in parts of K (one 64-row tile per 128 columns), within 1e-4; qkv: three Q4_K weights of a layer "
+                    "through hipq_matmul_multi, one quantization and one launch of the few-rows kernel for all three"},
         "decode_gemv_lm_head_size": {
             "workload": "Q4_K GEMV M=1 K=4096 N=151936, 3 weight copies rotated",
             "roofline": {"bound": "hbm", "kernel": "gemv_stream_kernel<Q4_K,G=4,GPW=2>",
