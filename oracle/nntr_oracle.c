@@ -15,6 +15,7 @@
 
 #include <math.h>
 #include <stdlib.h>
+#include <xmmintrin.h>
 #include <string.h>
 #ifdef _OPENMP
 #include <omp.h>
@@ -847,22 +848,10 @@ static void gemv_serial(int kind, int N, int K, const float *a, const uint8_t *w
     c[n] = kind == 12 ? dot_q4_K_q8_K(w + (size_t)n * rb, qa, nb, 0) : dot_q6_K_q8_K(w + (size_t)n * rb, qa, nb);
 }
 
-/* Applications/CausalLM/layers/qwen_moe_layer.cpp:394-503 with :332-392 (renormalize
- * = 1, the incremental path) and :161-259 (renormalize = 0, the forwarding path, which
- * uses the softmax values of the selected experts as they are).
- * Routing: softmax over the E logits (subtract row max, exp, divide by the row
- * sum), top-k by descending probability, weights divided by their sum if renormalize.
- * Expert e, token t (one at a time, M = 1): g = x.Wgate, u = x.Wup,
- * h = (sigmoid(g) * g) * u with sigmoid evaluated in double and cast
- * (nntrainer/layers/acti_func.h:286-288, 400-405), o = h.Wdown, contribution =
- * o * weight. Contributions are added into y in ascending expert order. */
-static void moe_forward_impl(int kind, int renormalize, int T, int H, int I, int E, int topk, const float *x,
-                             const float *logits, const void *const *gate, const void *const *up,
-                             const void *const *down, const float *gate_bias, const float *up_bias,
-                             const float *down_bias, int gpt_oss, float alpha, float *y, int32_t *topk_idx,
-                             float *topk_w) {
-  int32_t *idx = (int32_t *)malloc(sizeof(int32_t) * (size_t)T * topk);
-  float *wt = (float *)malloc(sizeof(float) * (size_t)T * topk);
+/* Routing shared by every variant of the block: softmax over the E logits, top-k by
+ * descending probability (ties to the lower index), weights divided by their sum if
+ * renormalize. idx, wt [T x topk]. */
+static void moe_route(int renormalize, int T, int E, int topk, const float *logits, int32_t *idx, float *wt) {
   float *p = (float *)malloc(sizeof(float) * (size_t)E);
   char *taken = (char *)malloc((size_t)E);
   for (int t = 0; t < T; ++t) {
@@ -892,6 +881,25 @@ static void moe_forward_impl(int kind, int renormalize, int T, int H, int I, int
   }
   free(p);
   free(taken);
+}
+
+/* Applications/CausalLM/layers/qwen_moe_layer.cpp:394-503 with :332-392 (renormalize
+ * = 1, the incremental path) and :161-259 (renormalize = 0, the forwarding path, which
+ * uses the softmax values of the selected experts as they are).
+ * Routing: softmax over the E logits (subtract row max, exp, divide by the row
+ * sum), top-k by descending probability, weights divided by their sum if renormalize.
+ * Expert e, token t (one at a time, M = 1): g = x.Wgate, u = x.Wup,
+ * h = (sigmoid(g) * g) * u with sigmoid evaluated in double and cast
+ * (nntrainer/layers/acti_func.h:286-288, 400-405), o = h.Wdown, contribution =
+ * o * weight. Contributions are added into y in ascending expert order. */
+static void moe_forward_impl(int kind, int renormalize, int T, int H, int I, int E, int topk, const float *x,
+                             const float *logits, const void *const *gate, const void *const *up,
+                             const void *const *down, const float *gate_bias, const float *up_bias,
+                             const float *down_bias, int gpt_oss, float alpha, float *y, int32_t *topk_idx,
+                             float *topk_w) {
+  int32_t *idx = (int32_t *)malloc(sizeof(int32_t) * (size_t)T * topk);
+  float *wt = (float *)malloc(sizeof(float) * (size_t)T * topk);
+  moe_route(renormalize, T, E, topk, logits, idx, wt);
   if (topk_idx) memcpy(topk_idx, idx, sizeof(int32_t) * (size_t)T * topk);
   if (topk_w) memcpy(topk_w, wt, sizeof(float) * (size_t)T * topk);
 
@@ -989,6 +997,167 @@ void orc_moe_forward_q4_K(int T, int H, int I, int E, int topk, const float *x,
  * exponential, avx2_impl.cpp:304-311, within the path's tolerance of this one). */
 void orc_swiglu(int64_t n, float *x, const float *y, const float *z) {
   for (int64_t i = 0; i < n; ++i) x[i] = (y[i] / (1.f + expf(-y[i]))) * z[i];
+}
+
+/* ------------------------------------------------------------------------- */
+/* nntrainer::swiglu as an x86 build of the reference evaluates it             */
+/* ------------------------------------------------------------------------- */
+
+/* avx2_approx_exp_e2lookup<8>, nntrainer/tensor/cpu_backend/x86/avx2_impl.cpp:227-294:
+ * e^x = 2^(k/8) * 2^f with k = nearest integer of 8x/ln2 (read out of the mantissa of
+ * x' + 1.5*2^23), 2^(k/8) from an eight-entry table of bit patterns plus k shifted into
+ * the exponent, and 2^f - 1 by a cubic in the remainder. One lane of the vector code,
+ * operation by operation; the table is the one a C++17 build carries (:166-174). */
+static inline float approx_exp_x86(float x) {
+  static const uint32_t tbl[8] = {0x3f800000u, 0x3f7b95c2u, 0x3f7837f0u, 0x3f75fed7u,
+                                  0x3f7504f3u, 0x3f75672au, 0x3f7744fdu, 0x3f7ac0c7u};
+  const float arg_min = -87.0f, arg_max = +88.3762626647949f; /* :142-143 */
+  const double ln2 = 0.69314718055994530942; /* M_LN2, what numbers::ln2_v<double> is in a C++17 build (:132-137) */
+  const float to_k = (float)(1.0 / ln2 * 8);
+  const float k_max = (float)(arg_max / ln2 * 8);
+  const float c0 = 0x1.c6af84b912394p-5f / 8 / 8 / 8, c1 = 0x1.ebfce50fac4f3p-3f / 8 / 8,
+              c2 = 0x1.62e42ff0c52d6p-1f / 8;
+  x = x > arg_min ? x : arg_min; /* _mm256_max_ps(xs, MIN) */
+  x = x * to_k;
+  x = x < k_max ? x : k_max;     /* _mm256_min_ps(xs, MAX) */
+  float xi = x + 0x1.8p23f;
+  const uint32_t bits = f32_bits(xi);
+  xi = xi - 0x1.8p23f;
+  const float fr = x - xi;
+  const float sc = bits_f32(tbl[bits & 7u] + (bits << 20));
+  const float q0 = fmaf(fr, c0, c1);
+  const float fr2 = fr * fr;
+  const float q2 = fr * c2;
+  const float pl = fmaf(q0, fr2, q2);
+  return fmaf(pl, sc, sc);
+}
+
+/* avx2::swiglu, avx2_impl.cpp:297-304 and 906-947: X = (Y / (exp'(-Y) + 1)) * Z with the
+ * exponential above, denormals read and written as zero while it runs (:909-910). Every
+ * lane of the 16-wide, 8-wide and masked steps does the same arithmetic. */
+void orc_swiglu_x86(int64_t n, float *x, const float *y, const float *z) {
+  const unsigned csr = _mm_getcsr();
+  _mm_setcsr(csr | 0x8040u);
+  for (int64_t i = 0; i < n; ++i) {
+    const float inv = approx_exp_x86(-y[i]) + 1.0f;
+    x[i] = (y[i] / inv) * z[i];
+  }
+  _mm_setcsr(csr);
+}
+
+/* avx2::swiglu with alpha, avx2_impl.cpp:306-316 and 950-993: the exponent is -(alpha * Y). */
+void orc_swiglu_alpha_x86(int64_t n, float *x, const float *y, const float *z, float alpha) {
+  const unsigned csr = _mm_getcsr();
+  _mm_setcsr(csr | 0x8040u);
+  for (int64_t i = 0; i < n; ++i) {
+    const float ay = alpha * y[i];
+    const float inv = approx_exp_x86(-ay) + 1.0f;
+    x[i] = (y[i] / inv) * z[i];
+  }
+  _mm_setcsr(csr);
+}
+
+/* ------------------------------------------------------------------------- */
+/* the cached mixture-of-experts layers                                       */
+/* ------------------------------------------------------------------------- */
+
+static void gemm_kind(int kind, int M, int N, int K, const float *A, const void *W, float *C) {
+  if (kind == 2)
+    orc_gemm_q4_0(M, N, K, A, W, C);
+  else if (kind == 12)
+    orc_gemm_q4_K(M, N, K, A, W, C);
+  else
+    orc_gemm_q6_K(M, N, K, A, W, C);
+}
+
+/* CachedSlimMoELayer::incremental_forwarding with compute_expert_forward
+ * (Applications/CausalLM/layers/qwen_moe_layer_cached.cpp:266-470, 176-265) and, with
+ * gpt_oss = 1, CachedSlimGptOssMoELayer (gpt_oss_moe_layer_cached.cpp:193-426, 438-530).
+ * Routing as in the plain layers (softmax, top-k, renormalised). Then per expert, in
+ * ascending id, ONE product with M = the number of its tokens (their rows gathered in
+ * ascending token order; one token: its row where it lies): so rows [0, 4*(M/4)) take
+ * the 4-row quantizer and the GEMM kernel's fp32 order and the others the row forms,
+ * as in every M > 1 product of the path.
+ *   Qwen: one token h = (sigmoid(g) * g) * u with the double-precision sigmoid of the
+ *         activation function (:236-241); more tokens nntrainer::swiglu, the x86 form
+ *         above (:242-250).
+ *   GPT-OSS: g += gate_bias, g = min(g, limit); u += up_bias, u = clamp(u, -limit, limit);
+ *         u += 1; nntrainer::swiglu with alpha for every token count; the down product
+ *         takes down_bias (:497-530).
+ * The expert's weighted rows go into its own zero-filled [T x H] tensor (0 + w * o) and
+ * the experts' tensors are added in ascending order (:456-464). */
+void orc_moe_forward_cached(int kind, int gpt_oss, int T, int H, int I, int E, int topk, const float *x,
+                            const float *logits, const void *const *gate, const void *const *up,
+                            const void *const *down, const float *gate_bias, const float *up_bias,
+                            const float *down_bias, float alpha, float limit, float *y, int32_t *topk_idx,
+                            float *topk_w) {
+  int32_t *idx = (int32_t *)malloc(sizeof(int32_t) * (size_t)T * topk);
+  float *wt = (float *)malloc(sizeof(float) * (size_t)T * topk);
+  moe_route(1, T, E, topk, logits, idx, wt);
+  if (topk_idx) memcpy(topk_idx, idx, sizeof(int32_t) * (size_t)T * topk);
+  if (topk_w) memcpy(topk_w, wt, sizeof(float) * (size_t)T * topk);
+
+  int *tok = (int *)malloc(sizeof(int) * (size_t)T);
+  float *tw = (float *)malloc(sizeof(float) * (size_t)T);
+  float *tin = (float *)malloc(sizeof(float) * (size_t)T * H);
+  float *g = (float *)malloc(sizeof(float) * (size_t)T * I);
+  float *u = (float *)malloc(sizeof(float) * (size_t)T * I);
+  float *h = (float *)malloc(sizeof(float) * (size_t)T * I);
+  float *o = (float *)malloc(sizeof(float) * (size_t)T * H);
+  float *eo = (float *)malloc(sizeof(float) * (size_t)T * H);
+  int first = 1;
+  for (int e = 0; e < E; ++e) {
+    int n = 0;
+    for (int t = 0; t < T; ++t)
+      for (int k = 0; k < topk; ++k)
+        if (idx[t * topk + k] == e) {
+          tok[n] = t;
+          tw[n] = wt[t * topk + k];
+          ++n;
+        }
+    if (!n) continue;
+    for (int i = 0; i < n; ++i) memcpy(tin + (size_t)i * H, x + (size_t)tok[i] * H, sizeof(float) * (size_t)H);
+    gemm_kind(kind, n, I, H, tin, gate[e], g);
+    gemm_kind(kind, n, I, H, tin, up[e], u);
+    if (gpt_oss) {
+      for (int i = 0; i < n; ++i)
+        for (int c = 0; c < I; ++c) {
+          float gv = g[(size_t)i * I + c] + gate_bias[(size_t)e * I + c];
+          gv = gv < limit ? gv : limit; /* clamp(lowest, limit): max with lowest changes nothing */
+          float uv = u[(size_t)i * I + c] + up_bias[(size_t)e * I + c];
+          uv = uv > -limit ? uv : -limit;
+          uv = uv < limit ? uv : limit;
+          g[(size_t)i * I + c] = gv;
+          u[(size_t)i * I + c] = uv + 1.f;
+        }
+      for (int i = 0; i < n; ++i)
+        orc_swiglu_alpha_x86(I, h + (size_t)i * I, g + (size_t)i * I, u + (size_t)i * I, alpha);
+    } else if (n == 1) {
+      for (int c = 0; c < I; ++c) {
+        const float en = (float)exp((double)(-g[c]));
+        const float sig = (float)(1.0 / (1.0 + (double)en));
+        h[c] = (sig * g[c]) * u[c];
+      }
+    } else {
+      for (int i = 0; i < n; ++i) orc_swiglu_x86(I, h + (size_t)i * I, g + (size_t)i * I, u + (size_t)i * I);
+    }
+    gemm_kind(kind, n, H, I, h, down[e], o);
+    memset(eo, 0, sizeof(float) * (size_t)T * H);
+    for (int i = 0; i < n; ++i)
+      for (int c = 0; c < H; ++c) {
+        float v = o[(size_t)i * H + c];
+        if (gpt_oss) v = v + down_bias[(size_t)e * H + c];
+        v = v * tw[i];
+        eo[(size_t)tok[i] * H + c] = eo[(size_t)tok[i] * H + c] + v;
+      }
+    if (first) {
+      memcpy(y, eo, sizeof(float) * (size_t)T * H);
+      first = 0;
+    } else
+      for (size_t j = 0; j < (size_t)T * H; ++j) y[j] = y[j] + eo[j];
+  }
+  if (first) memset(y, 0, sizeof(float) * (size_t)T * H);
+  free(tok); free(tw); free(tin); free(g); free(u); free(h); free(o); free(eo); free(idx); free(wt);
 }
 
 void orc_set_threads(int n) {

@@ -114,6 +114,18 @@ void orc_moe_forward_q4_K(int T, int H, int I, int E, int topk, const float *x,
                           float *y, int32_t *topk_idx, float *topk_w);
 
 void orc_swiglu(int64_t n, float *x, const float *y, const float *z);
+/* nntrainer::swiglu as the x86 back-end evaluates it (table-and-cubic exponential, denormals
+ * as zero): nntrainer/tensor/cpu_backend/x86/avx2_impl.cpp:227-316, 906-993. */
+void orc_swiglu_x86(int64_t n, float *x, const float *y, const float *z);
+void orc_swiglu_alpha_x86(int64_t n, float *x, const float *y, const float *z, float alpha);
+/* The cached layers: one product per expert with M = its token count, swiglu by token count,
+ * GPT-OSS with its clamps. qwen_moe_layer_cached.cpp:176-470, gpt_oss_moe_layer_cached.cpp:193-530.
+ * Biases [E x I], [E x I], [E x H] (gpt_oss = 1 only). */
+void orc_moe_forward_cached(int kind, int gpt_oss, int T, int H, int I, int E, int topk, const float *x,
+                            const float *logits, const void *const *gate, const void *const *up,
+                            const void *const *down, const float *gate_bias, const float *up_bias,
+                            const float *down_bias, float alpha, float limit, float *y, int32_t *topk_idx,
+                            float *topk_w);
 void orc_set_threads(int n);
 
 #ifdef __cplusplus

@@ -9,6 +9,7 @@
  *         to pin the C restatement in oracle/nntr_oracle.c and by bench.py's
  *         cpu_baseline leg. It is never linked into the product.
  */
+#include <avx2_impl.h>
 #include <ggml_interface.h>
 #include <nntr_ggml_impl.h>
 #include <nntr_ggml_impl_common.h>
@@ -16,6 +17,9 @@
 #include <cstddef>
 #include <cstdint>
 #include <omp.h>
+#ifdef REF_SHIM_MIXED
+#include <bs_thread_pool_manager.hpp>
+#endif
 
 extern "C" {
 
@@ -120,7 +124,30 @@ float ref_vec_dot_q6_K_q8_K(unsigned K, const void *vq6, const void *vq8) {
   return nntrainer::__ggml_vec_dot_q6_K_q8_K(K, vq6, vq8);
 }
 
-/** Thread control for the timed baseline (the wrappers use OpenMP). */
+/** nntrainer::swiglu of an x86 build, x86_compute_backend.cpp:286-292 -> avx2_impl.cpp:906-993. */
+void ref_swiglu(unsigned n, float *x, const float *y, const float *z) {
+  nntrainer::avx2::swiglu(n, x, y, z);
+}
+void ref_swiglu_alpha(unsigned n, float *x, const float *y, const float *z,
+                      float alpha) {
+  nntrainer::avx2::swiglu(n, x, y, z, alpha);
+}
+/** nntrainer::clamp of an x86 build, avx2_impl.cpp:1811-1833. */
+void ref_clamp(const float *in, float *out, size_t n, float lo, float hi) {
+  nntrainer::avx2::clamp(in, out, n, lo, hi);
+}
+
+/** Thread control for the timed baseline. The OpenMP front-end takes its count from
+ * OpenMP; the thread-pool front-end sizes its pool itself
+ * (bs_thread_pool_manager.hpp:41) and reports it here. */
 void ref_set_threads(int n) { omp_set_num_threads(n); }
+#ifdef REF_SHIM_MIXED
+int ref_max_threads(void) {
+  return (int)nntrainer::ThreadPoolManager::Global().getThreadPool().get_thread_count();
+}
+int ref_front_end_is_thread_pool(void) { return 1; }
+#else
 int ref_max_threads(void) { return omp_get_max_threads(); }
+int ref_front_end_is_thread_pool(void) { return 0; }
+#endif
 }

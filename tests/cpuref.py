@@ -242,3 +242,47 @@ def swiglu(y, z):
     x = np.empty_like(y)
     lib.orc_swiglu(_c.c_int64(y.size), _ptr(x), _ptr(y), _ptr(z))
     return x
+
+
+def swiglu_x86(lib, y, z, alpha=None):
+    """nntrainer::swiglu as the x86 back-end evaluates it (approximate exponential): the oracle's
+    restatement, or the reference library's own routine."""
+    y = np.ascontiguousarray(y, np.float32)
+    z = np.ascontiguousarray(z, np.float32)
+    x = np.zeros_like(y)
+    if lib is oracle():
+        if alpha is None:
+            lib.orc_swiglu_x86(_c.c_int64(y.size), _ptr(x), _ptr(y), _ptr(z))
+        else:
+            lib.orc_swiglu_alpha_x86(_c.c_int64(y.size), _ptr(x), _ptr(y), _ptr(z), _c.c_float(alpha))
+    elif alpha is None:
+        lib.ref_swiglu(_c.c_uint(y.size), _ptr(x), _ptr(y), _ptr(z))
+    else:
+        lib.ref_swiglu_alpha(_c.c_uint(y.size), _ptr(x), _ptr(y), _ptr(z), _c.c_float(alpha))
+    return x
+
+
+def moe_forward_cached(x, logits, gate, up, down, topk, kind="q4_K", gpt_oss=False, gate_bias=None, up_bias=None,
+                       down_bias=None, alpha=1.702, limit=7.0):
+    """Oracle of the cached layers (moe_cached_slim; gpt_oss_moe_slim_cached with gpt_oss=True):
+    one product per expert over its tokens, swiglu by token count, GPT-OSS with its clamps."""
+    lib = oracle()
+    x = np.ascontiguousarray(x, np.float32)
+    logits = np.ascontiguousarray(logits, np.float32)
+    t, h = x.shape
+    e = logits.shape[1]
+    nbytes, blk = BLOCK_BYTES[kind]
+    i = gate[0].size // ((h // blk) * nbytes)
+    if gpt_oss:
+        gb, ub, db = (np.ascontiguousarray(b, np.float32) for b in (gate_bias, up_bias, down_bias))
+    else:
+        gb = ub = db = np.zeros(1, np.float32)
+    arr = lambda lst: (_c.c_void_p * e)(*[w.ctypes.data for w in lst])
+    y = np.zeros((t, h), np.float32)
+    idx = np.zeros((t, topk), np.int32)
+    wt = np.zeros((t, topk), np.float32)
+    lib.orc_moe_forward_cached(_i32({"q4_0": 2, "q4_K": 12, "q6_K": 14}[kind]), _i32(1 if gpt_oss else 0), _i32(t),
+                               _i32(h), _i32(i), _i32(e), _i32(topk), _ptr(x), _ptr(logits), arr(gate), arr(up),
+                               arr(down), _ptr(gb), _ptr(ub), _ptr(db), _c.c_float(alpha), _c.c_float(limit),
+                               _ptr(y), _ptr(idx), _ptr(wt))
+    return y, idx, wt

@@ -62,6 +62,12 @@ def main():
         mo = cr.quantize_act(o, kind, x, "mat")
         inter = np.stack([cr.interleave4(kind, mo[4 * g:4 * g + 4], 1024) for g in range(len(x) // 4)])
         assert np.array_equal(inter, cr.quantize_act(r, kind, x, "mat"))
+    ys, zs = t._swiglu_inputs()
+    for alpha in (None, 1.702):
+        assert np.array_equal(cr.swiglu_x86(o, ys, zs, alpha).view(np.uint32), cr.swiglu_x86(r, ys, zs, alpha).view(np.uint32))
+    # the cached mixture-of-experts oracle against the same block composed from the reference's routines
+    for gpt_oss in (False, True):
+        t.test_cached_moe_equals_composition_of_reference_routines(gpt_oss)
     json.dump(t._digest_cases(), open(os.path.join(HERE, "oracle_digests.json"), "w"), indent=1, sort_keys=True)
     print("wrote oracle_digests.json")
 

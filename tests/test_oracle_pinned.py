@@ -272,6 +272,135 @@ def test_gpt_oss_moe_reduces_to_known_cases():
     assert np.abs(ya - yc).max() / np.abs(ya).max() > 1e-2
 
 
+def _swiglu_inputs():
+    rng = np.random.default_rng(12)
+    y = np.concatenate([rng.normal(0, s, 4099).astype(np.float32) for s in (0.05, 1, 6, 40)]
+                       + [np.array([0, -0.0, 87.0, -87.0, 88.5, -88.5, 200, -200, 1e-39, -1e-39, 3e-38], np.float32)])
+    z = rng.normal(0, 2, y.size).astype(np.float32)
+    return y, z
+
+
+@needs_ref
+@pytest.mark.parametrize("alpha", [None, 1.702, 1.0])
+def test_x86_swiglu_bits_match_reference(alpha):
+    """orc_swiglu_x86 / orc_swiglu_alpha_x86 against avx2::swiglu of the reference build, bit for
+    bit: small, ordinary and saturating arguments, denormals (read as zero while the routine
+    runs), and lengths that end in the 8-wide and the masked step."""
+    y, z = _swiglu_inputs()
+    for n in (y.size, 16, 24, 29, 7, 1):
+        a = cr.swiglu_x86(cr.oracle(), y[:n], z[:n], alpha)
+        b = cr.swiglu_x86(cr.ref(), y[:n], z[:n], alpha)
+        assert np.array_equal(a.view(np.uint32), b.view(np.uint32)), n
+
+
+@needs_ref
+def test_x86_swiglu_distance_from_the_expf_form():
+    """How far the reference's x86 swiglu is from the expf form the C5 decoder's CPU leg and the
+    dense-MLP oracle use: measured on gate values of the range a decoder produces (|y| up to 40),
+    relative to the largest output. This number is what lets a 1e-4 test use either form."""
+    y, z = _swiglu_inputs()
+    keep = np.abs(y) < 60
+    approx = cr.swiglu_x86(cr.ref(), y[keep], z[keep])
+    exact = cr.swiglu(y[keep], z[keep])
+    dist = np.abs(approx.astype(np.float64) - exact).max() / np.abs(exact).max()
+    assert dist <= 2e-6, dist
+    rel = np.abs(approx.astype(np.float64) - exact) / np.maximum(np.abs(exact), 1e-30)
+    assert rel[np.abs(exact) > 1e-3].max() <= 1e-5
+
+
+def _cached_moe_case(kind="q4_K", t=13, h=256, i=256, e=6, k=2, seed=500):
+    o = cr.oracle()
+    gate = [cr.quantize_weights(o, kind, synth.normal(seed + 3 * x, (i, h), 0.02)) for x in range(e)]
+    up = [cr.quantize_weights(o, kind, synth.normal(seed + 1 + 3 * x, (i, h), 0.02)) for x in range(e)]
+    down = [cr.quantize_weights(o, kind, synth.normal(seed + 2 + 3 * x, (h, i), 0.02)) for x in range(e)]
+    x = synth.normal(seed + 100, (t, h))
+    logits = synth.normal(seed + 101, (t, e))
+    logits[0] = [9, 8, 0, 0, 0, 0][:e] if e >= 2 else logits[0]  # expert 0 and 1 certainly used
+    return gate, up, down, x, logits
+
+
+@needs_ref
+@pytest.mark.parametrize("gpt_oss", [False, True])
+def test_cached_moe_equals_composition_of_reference_routines(gpt_oss):
+    """orc_moe_forward_cached against the cached layers' expert forward rebuilt here from the
+    reference library's own routines: per expert one ref_gemm over its gathered tokens (its 4-row
+    and leftover-row paths), ref_swiglu / the activation function by token count (Qwen) or the
+    bias, ref_clamp, + 1 and ref_swiglu with alpha (GPT-OSS), one more ref_gemm, the routing weight,
+    and the experts' [T x H] tensors added in ascending order. Bit for bit. Token counts per
+    expert range over 1, 2..3 (leftover rows only), 4 and more (both paths)."""
+    o, r = cr.oracle(), cr.ref()
+    kind, t, h, i, e, k = "q4_K", 13, 256, 256, 6, 2
+    gate, up, down, x, logits = _cached_moe_case(kind, t, h, i, e, k)
+    logits[:, 5] = -30.0
+    logits[3, 5] = 30.0  # expert 5 gets exactly one token
+    gb, ub, db = synth.normal(601, (e, i), 3.0), synth.normal(602, (e, i), 3.0), synth.normal(603, (e, h), 0.3)
+    y, idx, wt = cr.moe_forward_cached(x, logits, gate, up, down, k, kind, gpt_oss, gb, ub, db)
+    counts = np.bincount(idx.ravel(), minlength=e)
+    assert counts[5] == 1 and (counts >= 4).any() and ((counts > 1) & (counts % 4 != 0)).any()
+    f32 = np.float32
+    want = None
+    import ctypes as c
+    for ee in range(e):
+        toks = [(tt, wt[tt, kk]) for tt in range(t) for kk in range(k) if idx[tt, kk] == ee]
+        if not toks:
+            continue
+        tin = np.stack([x[tt] for tt, _ in toks])
+        g = cr.gemm(r, kind, tin, gate[ee], i)
+        u = cr.gemm(r, kind, tin, up[ee], i)
+        if gpt_oss:
+            g = (g + gb[ee]).astype(f32)
+            u = (u + ub[ee]).astype(f32)
+            gc, uc = np.empty_like(g), np.empty_like(u)
+            r.ref_clamp(cr._ptr(g), cr._ptr(gc), c.c_size_t(g.size), c.c_float(np.finfo(f32).min), c.c_float(7.0))
+            r.ref_clamp(cr._ptr(u), cr._ptr(uc), c.c_size_t(u.size), c.c_float(-7.0), c.c_float(7.0))
+            uc = (uc + f32(1)).astype(f32)
+            hh = np.stack([cr.swiglu_x86(r, gc[j], uc[j], 1.702) for j in range(len(toks))])
+        elif len(toks) == 1:
+            en = np.exp(-g.astype(np.float64)).astype(f32)
+            sig = (1.0 / (1.0 + en.astype(np.float64))).astype(f32)
+            hh = ((sig * g).astype(f32) * u).astype(f32)
+        else:
+            hh = np.stack([cr.swiglu_x86(r, g[j], u[j]) for j in range(len(toks))])
+        od = cr.gemm(r, kind, hh, down[ee], h)
+        if gpt_oss:
+            od = (od + db[ee]).astype(f32)
+        eo = np.zeros((t, h), f32)
+        for j, (tt, ww) in enumerate(toks):
+            eo[tt] = eo[tt] + (od[j] * f32(ww)).astype(f32)
+        want = eo if want is None else (want + eo).astype(f32)
+    assert np.array_equal(y.view(np.uint32), want.view(np.uint32))
+    if gpt_oss:  # the clamps are live: pre-activations beyond the limit exist in this case
+        g0 = cr.gemm(o, kind, x, gate[0], i) + gb[0]
+        assert (g0 > 7).any() and (np.abs(cr.gemm(o, kind, x, up[0], i) + ub[0]) > 7).any()
+
+
+def test_cached_moe_reduces_to_the_per_token_layer():
+    """Without the reference library: with one token every expert sees one row, where the cached
+    Qwen layer evaluates exactly what the per-token layer does (same products, the activation
+    function's sigmoid): the two oracles must agree bit for bit. With more tokens they differ only
+    by the 4-row products' fp32 order and the approximate exponential: 2e-5 of the largest output.
+    For GPT-OSS with limits beyond every pre-activation the same holds against the unclamped block,
+    and with limit = 7 on large biases the outputs must differ (the clamp acts)."""
+    kind, t, h, i, e, k = "q4_K", 9, 256, 256, 6, 2
+    gate, up, down, x, logits = _cached_moe_case(kind, t, h, i, e, k, seed=700)
+    y1, idx1, wt1 = cr.moe_forward_cached(x[:1], logits[:1], gate, up, down, k, kind)
+    y0, idx0, wt0 = cr.moe_forward(x[:1], logits[:1], gate, up, down, k, kind)
+    assert np.array_equal(idx1, idx0) and np.array_equal(wt1, wt0)
+    assert np.array_equal(y1.view(np.uint32), y0.view(np.uint32))
+    y, idx, wt = cr.moe_forward_cached(x, logits, gate, up, down, k, kind)
+    yp, idxp, wtp = cr.moe_forward(x, logits, gate, up, down, k, kind)
+    assert np.array_equal(idx, idxp) and np.array_equal(wt, wtp)
+    assert 0 < np.abs(y - yp).max() <= 2e-5 * np.abs(yp).max()
+    gb, ub, db = synth.normal(801, (e, i), 0.3), synth.normal(802, (e, i), 0.3), synth.normal(803, (e, h), 0.3)
+    yg, _, _ = cr.moe_forward_cached(x, logits, gate, up, down, k, kind, True, gb, ub, db, limit=1e30)
+    yu, _, _ = cr.moe_forward_gpt_oss(x, logits, gate, up, down, gb, ub, db, k)
+    assert np.abs(yg - yu).max() <= 2e-5 * np.abs(yu).max()
+    big = synth.normal(804, (e, i), 4.0)
+    yc, _, _ = cr.moe_forward_cached(x, logits, gate, up, down, k, kind, True, big, big, db, limit=7.0)
+    yn, _, _ = cr.moe_forward_cached(x, logits, gate, up, down, k, kind, True, big, big, db, limit=1e30)
+    assert np.abs(yc - yn).max() > 1e-2 * np.abs(yn).max()
+
+
 # ------------------------------------------------------------------ 3. golden digests
 def _digest_cases():
     o = cr.oracle()
@@ -287,6 +416,14 @@ def _digest_cases():
     out["q8_K_row"] = synth.digest(cr.quantize_act(o, "q8_K", x, "row"))
     out["q8_K_mat"] = synth.digest(cr.quantize_act(o, "q8_K", x, "mat"))
     out["input_w"] = synth.digest(_w(20, 64, 1024))
+    ys, zs = _swiglu_inputs()
+    out["swiglu_x86"] = synth.digest(cr.swiglu_x86(o, ys, zs))
+    out["swiglu_alpha_x86"] = synth.digest(cr.swiglu_x86(o, ys, zs, 1.702))
+    gate, up, down, x, logits = _cached_moe_case()
+    e, i, h = len(gate), 256, 256
+    out["moe_cached_qwen"] = synth.digest(cr.moe_forward_cached(x, logits, gate, up, down, 2)[0])
+    gb, ub, db = synth.normal(601, (e, i), 3.0), synth.normal(602, (e, i), 3.0), synth.normal(603, (e, h), 0.3)
+    out["moe_cached_gpt_oss"] = synth.digest(cr.moe_forward_cached(x, logits, gate, up, down, 2, "q4_K", True, gb, ub, db)[0])
     return out
 
 
