@@ -180,17 +180,26 @@ HIPQ_API int hipq_matmul_each_row(hipq_weight_t w, const float *A, int64_t rows,
 /** hipq_matmul on device buffers for callers that cannot allocate device memory:
  *  code under HIP graph capture, tight serving loops, harnesses that forbid it.
  *  It has no counterpart in the reference. The quantized activations of the call
- *  live in a fixed array of 16 MiB inside the library's device code (each GPU the
+ *  live in a fixed array inside the library's device code (32 MiB; each GPU the
  *  library runs on holds one until the process ends) instead of the per-stream
- *  workspace that hipq_matmul grows on demand; a call that needs more
- *  (M * K beyond about 7.8 million values for Q6_K weights, 14 million for Q4_0
+ *  workspace that hipq_matmul grows on demand. The array has four slots of 8 MiB,
+ *  one for each of the first four streams that use this entry point (a fifth stream
+ *  gets HIPQ_ERR_NOT_SUPPORTED until hipq_stream_release has given a slot back), so calls
+ *  on different streams do not share memory; calls on ONE stream run in order and share
+ *  its slot, which keeps the last call's contents. A call that needs more than a slot
+ *  (M * K beyond about 3.9 million values for Q6_K weights, 7 million for Q4_0
  *  and Q4_K) returns HIPQ_ERR_NOT_SUPPORTED. The call performs no device
  *  allocation and no free and enqueues the same kernels as hipq_matmul, so
- *  results are the same bits (one exception: a Q4_K product of up to 128 rows that
- *  hipq_matmul forms in parts of K takes whole rows here when the parts' partial sums
- *  do not fit the array as well; it then agrees to 1e-4 like every matrix-core
- *  product). All calls on a GPU share that one array: calls
- *  whose kernels may overlap on the device (different streams) race on it. */
+ *  results are the same bits wherever the same kernel runs. Where the two may take
+ *  different kernels: a weight that has no tile copy yet (only an allocating call builds
+ *  one) goes through the GEMV engine here, which carries the reference's bits where
+ *  hipq_matmul's matrix-core product agrees to 1e-4; and a Q4_K or Q6_K product of up to
+ *  128 rows that hipq_matmul forms in parts of K takes whole rows here when the parts'
+ *  partial sums do not fit the slot beside the activations, or when C is not 16-byte
+ *  aligned with ldc a multiple of four (both entry points then): the fp32 sums then have
+ *  another order, within the 1e-4 of every matrix-core product. Results of the K-formats'
+ *  matrix-core products are therefore stable to the tolerance, not to the bit, across ldc,
+ *  alignment and entry point. */
 HIPQ_API int hipq_matmul_noalloc(hipq_weight_t w, const float *A, int64_t M, int64_t lda,
                                  float *C, int64_t ldc, void *stream);
 
@@ -262,10 +271,17 @@ HIPQ_API int hipq_moe_forward(const hipq_moe_desc *desc, const hipq_weight_t *ga
  *    here all experts stay in HBM) and in running one batched product per expert, which is how
  *    this library runs every MoE; routing, expert arithmetic and the ascending-expert sum are
  *    the same.
+ *    Against the cached layer's own arithmetic (rows [0, 4*(n/4)) of an expert's n tokens through
+ *    the 4-row quantizer and GEMM order, nntrainer::swiglu with the x86 back-end's approximate
+ *    exponential for n > 1) the outputs agree to 1e-4 of the largest, not to the bit: every
+ *    (token, expert) pair here has the bits of its own M = 1 products.
  *  - HIPQ_MOE_GPT_OSS: GptOssMoELayer (gpt_oss_moe_layer.cpp:372-449, 452-568): the router
  *    logits take router_bias [E]; per expert g = gate(x) + gate_bias[e], u = up(x) + up_bias[e],
- *    h = (g / (1 + exp(-alpha g))) * (u + 1), y_e = down(h) + down_bias[e]; no clamping (the
- *    reference has it commented out); top-k weights renormalised per desc->renormalize. */
+ *    h = (g / (1 + exp(-alpha g))) * (u + 1), y_e = down(h) + down_bias[e]; top-k weights
+ *    renormalised per desc->renormalize. `limit` > 0 clamps the biased pre-activations first,
+ *    g = min(g, limit), u = min(max(u, -limit), limit): the cached layer does so with limit 7
+ *    (gpt_oss_moe_layer_cached.cpp:497-507, gpt_oss_moe_layer_cached.h:137), the uncached
+ *    one has the same two lines commented out (gpt_oss_moe_layer.cpp:414, 419) and passes 0. */
 enum { HIPQ_MOE_QWEN = 0, HIPQ_MOE_GPT_OSS = 1 };
 typedef struct hipq_moe_ext {
   int32_t variant;          /* HIPQ_MOE_*                                    */
@@ -274,6 +290,10 @@ typedef struct hipq_moe_ext {
   const float *gate_bias;   /* [E x I], gpt_oss                              */
   const float *up_bias;     /* [E x I], gpt_oss                              */
   const float *down_bias;   /* [E x H], gpt_oss                              */
+  float limit;              /* gpt_oss: 0 = no clamp, > 0 as above           */
+  int32_t biases_on_device; /* non-zero: the four bias pointers are device memory
+                               whatever `mem` says (a layer uploads them once,
+                               hipq_device_alloc / hipq_device_upload)         */
 } hipq_moe_ext;
 HIPQ_API int hipq_moe_forward_ext(const hipq_moe_desc *desc, const hipq_moe_ext *ext,
                                   const hipq_weight_t *gate, const hipq_weight_t *up,
@@ -281,6 +301,15 @@ HIPQ_API int hipq_moe_forward_ext(const hipq_moe_desc *desc, const hipq_moe_ext 
                                   const float *router_logits, const float *router_weight,
                                   float *y, int32_t *topk_idx, float *topk_w, int mem,
                                   void *stream);
+
+/** Device memory for a caller that has no HIP runtime of its own (the framework plug-in keeps
+ *  the biases of a GPT-OSS block and activations that stay on the GPU between two of its layers
+ *  in it). No counterpart in the reference: its tensors are host memory only. upload / download
+ *  are ordered on `stream` and return when the host bytes have been read / written. */
+HIPQ_API int hipq_device_alloc(void **ptr, size_t bytes);
+HIPQ_API int hipq_device_free(void *ptr);
+HIPQ_API int hipq_device_upload(void *dst_device, const void *src_host, size_t bytes, void *stream);
+HIPQ_API int hipq_device_download(void *dst_host, const void *src_device, size_t bytes, void *stream);
 
 /** Page-locked host memory, zero-filled: what a context's MemAllocator hands the framework's
  *  memory pool (MemAllocator::alloc / free, nntrainer/mem_allocator.cpp:22-30; set by the
@@ -291,8 +320,12 @@ HIPQ_API int hipq_host_alloc(void **ptr, size_t bytes);
 HIPQ_API int hipq_host_free(void *ptr);
 
 /** Frees the scratch the library keeps for a stream (it grows on demand with the calls made on
- *  the stream and is otherwise kept until hipq_shutdown). Call it before destroying a stream
- *  that calls were made on; waits for the stream. No counterpart in the reference, whose OpenCL
+ *  the stream and is otherwise kept until hipq_shutdown) and gives back the stream's slot of the
+ *  allocation-free entry point's array. Call it before destroying a stream
+ *  that calls were made on; waits for the stream. When a call needs more scratch than the stream
+ *  has, the library allocates a larger block (hipMalloc: not possible while the stream is being
+ *  captured into a graph, so run a call of the largest shape once before capturing) and keeps the
+ *  smaller one until a later call on the stream finds the stream drained. No counterpart in the reference, whose OpenCL
  *  back-end has one queue (opencl_command_queue_manager.cpp). */
 HIPQ_API int hipq_stream_release(void *stream);
 

@@ -23,6 +23,7 @@ SYMBOLS = [
     "hipq_quantize_q8_K", "hipq_matmul", "hipq_matmul_each_row", "hipq_matmul_noalloc", "hipq_matmul_multi", "hipq_moe_forward",
     "hipq_moe_forward_ext", "hipq_mlp_swiglu", "hipq_host_alloc", "hipq_host_free", "hipq_stream_release",
     "hipq_quantize_weights", "hipq_file_layout", "hipq_weights_from_file",
+    "hipq_device_alloc", "hipq_device_free", "hipq_device_upload", "hipq_device_download",
 ]
 # measurement helpers of csrc/hipq_bench.h: exported for bench.py, not part of the product ABI
 BENCH_SYMBOLS = ["hipq_time_matmul", "hipq_bench_matmul_steps", "hipq_bench_mfma_ceiling",
@@ -51,7 +52,8 @@ class MoeDesc(C.Structure):
 
 class MoeExt(C.Structure):
     _fields_ = [("variant", C.c_int32), ("alpha", C.c_float), ("router_bias", C.c_void_p),
-                ("gate_bias", C.c_void_p), ("up_bias", C.c_void_p), ("down_bias", C.c_void_p)]
+                ("gate_bias", C.c_void_p), ("up_bias", C.c_void_p), ("down_bias", C.c_void_p),
+                ("limit", C.c_float), ("biases_on_device", C.c_int32)]
 
 
 MOE_QWEN, MOE_GPT_OSS = 0, 1
@@ -275,10 +277,13 @@ def moe_forward(tokens, hidden, inter, experts, topk, gate, up, down, x, y, rout
 
 def moe_forward_gpt_oss(tokens, hidden, inter, experts, topk, gate, up, down, x, y, gate_bias, up_bias,
                         down_bias, alpha=1.702, router_logits=None, router_weight=None, router_bias=None,
-                        topk_idx=None, topk_w=None, renormalize=True, mem=MEM_DEVICE, stream=None):
-    """The GPT-OSS block: biased router and projections, (g / (1 + exp(-alpha g))) * (u + 1)."""
+                        topk_idx=None, topk_w=None, renormalize=True, mem=MEM_DEVICE, stream=None, limit=0.0,
+                        biases_on_device=False):
+    """The GPT-OSS block: biased router and projections, (g / (1 + exp(-alpha g))) * (u + 1);
+    limit > 0: the cached layer's clamps on the biased gate and up values."""
     d = MoeDesc(tokens, hidden, inter, experts, topk, 1 if renormalize else 0)
-    ext = MoeExt(MOE_GPT_OSS, alpha, _addr(router_bias), _addr(gate_bias), _addr(up_bias), _addr(down_bias))
+    ext = MoeExt(MOE_GPT_OSS, alpha, _addr(router_bias), _addr(gate_bias), _addr(up_bias), _addr(down_bias),
+                 limit, 1 if biases_on_device else 0)
     ex = gate if isinstance(gate, Experts) else Experts(gate, up, down)
     check(lib().hipq_moe_forward_ext(C.byref(d), C.byref(ext), ex.gate, ex.up, ex.down, _addr(x),
                                      _addr(router_logits), _addr(router_weight), _addr(y),

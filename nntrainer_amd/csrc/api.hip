@@ -25,13 +25,15 @@
 #include "hipq_bench.h"
 #include "hipq_internal.h"
 
-/* Scratch of hipq_matmul_noalloc: quantized activations of one call. Every GPU the
- * library runs on holds its own copy of the array at its own address until the
- * process ends; in host code the array's name is only a stand-in, the address
- * comes from hipGetSymbolAddress with that device current (hipq_init). */
-constexpr size_t NOALLOC_SCRATCH_BYTES = (size_t)16 << 20;
+/* Scratch of hipq_matmul_noalloc: quantized activations (and partial products) of one call.
+ * Four slots, one per stream that uses the entry point, so that calls on different streams
+ * do not share memory. Every GPU the library runs on holds its own copy of the array at its
+ * own address until the process ends; in host code the array's name is only a stand-in, the
+ * address comes from hipGetSymbolAddress with that device current (hipq_init). */
+constexpr int NOALLOC_SLOTS = 4;
+constexpr size_t NOALLOC_SCRATCH_BYTES = (size_t)8 << 20; /* one slot: the most one call may need */
 constexpr int MAX_DEVICES = 64;
-static __device__ __align__(256) unsigned char scratch[NOALLOC_SCRATCH_BYTES];
+static __device__ __align__(256) unsigned char scratch[NOALLOC_SLOTS * NOALLOC_SCRATCH_BYTES];
 
 namespace {
 
@@ -40,6 +42,12 @@ thread_local char tl_error[768] = "";
 struct Workspace {
   void *ptr = nullptr;
   size_t bytes = 0;
+  /* Blocks a call outgrew. They are not freed where they are replaced: kernels already queued
+   * read them, and the call that asked may still hold pointers into them. They go when a later
+   * call on the stream starts (after the stream has drained) or the stream is released. */
+  std::vector<void *> retired;
+  int depth = 0;           /* public entry points active on this stream (they nest) */
+  uint64_t generation = 0; /* counts the times ptr has changed */
   /* device copies of a host-memory call's operands (the kernels' own scratch is ptr) */
   void *io = nullptr;
   size_t io_bytes = 0;
@@ -59,7 +67,9 @@ struct State {
   bool ready = false;
   int device = -1;
   void *scratch_ptr[MAX_DEVICES] = {}; /* device address of `scratch`, per device */
-  std::recursive_mutex noalloc_enqueue; /* calls that share the scratch submit one at a time */
+  std::recursive_mutex noalloc_enqueue; /* calls of the allocation-free entry point submit one at a time */
+  hipStream_t noalloc_stream[NOALLOC_SLOTS] = {}; /* which stream owns which slot of `scratch` */
+  bool noalloc_taken[NOALLOC_SLOTS] = {};
   std::unordered_map<hipStream_t, Workspace> ws;
   /* one table of expert weight views per MoE layer, found by its first gate weight */
   std::unordered_map<const hipq_weight *, MoeTable> moe_tables;
@@ -97,28 +107,68 @@ int require_ready() {
 }
 
 /* Per-stream scratch, grown on demand. Work queued on one stream runs in order,
- * so consecutive calls on a stream may share it; different streams never do. */
+ * so consecutive calls on a stream may share it; different streams never do.
+ * A request the block cannot serve gets a new block; the old one is retired, not freed, so
+ * nothing that was carved out of it earlier in the same call (or is read by kernels already
+ * queued) loses its memory. What a larger block does not carry over is the old block's
+ * CONTENTS: a call that shares quantized activations between several products reserves the
+ * largest request first (one reservation per entry point) and checks workspace_generation()
+ * before it reuses them. */
 int workspace(hipStream_t s, size_t bytes, void **out) {
   std::lock_guard<std::mutex> lk(g.mu);
   Workspace &w = g.ws[s];
   if (w.bytes < bytes) {
-    if (w.ptr) {
-      HIPQ_HIP(hipStreamSynchronize(s));
-      HIPQ_HIP(hipFree(w.ptr));
-      w.ptr = nullptr;
-      w.bytes = 0;
-    }
     size_t want = (bytes + ((size_t)1 << 20) - 1) & ~(((size_t)1 << 20) - 1);
-    hipError_t e = hipMalloc(&w.ptr, want);
-    if (e != hipSuccess) {
-      w.ptr = nullptr;
+    void *fresh = nullptr;
+    hipError_t e = hipMalloc(&fresh, want);
+    if (e != hipSuccess)
       return fail(HIPQ_ERR_OUT_OF_MEMORY, "workspace of %zu bytes: %s", want, hipGetErrorString(e));
-    }
+    if (w.ptr) w.retired.push_back(w.ptr);
+    w.ptr = fresh;
     w.bytes = want;
+    ++w.generation;
   }
   *out = w.ptr;
   return HIPQ_OK;
 }
+
+uint64_t workspace_generation(hipStream_t s) {
+  std::lock_guard<std::mutex> lk(g.mu);
+  return g.ws[s].generation;
+}
+
+/* A call that reuses activations it quantized earlier names the generation it saw then. */
+int workspace_unmoved(hipStream_t s, uint64_t generation) {
+  if (workspace_generation(s) == generation) return HIPQ_OK;
+  return fail(HIPQ_ERR_RUNTIME,
+              "internal: the stream's workspace was replaced between the quantization of a call's shared "
+              "activations and a product that reads them (a request larger than the call's reservation)");
+}
+
+/* Marks a public entry point's stay on a stream. The outermost one frees the blocks earlier
+ * calls retired, once the stream has drained -- unless the stream is being captured into a
+ * graph, where nothing may wait; they then stay until a later call. */
+struct CallScope {
+  hipStream_t s;
+  explicit CallScope(hipStream_t s_) : s(s_) {
+    std::lock_guard<std::mutex> lk(g.mu);
+    Workspace &w = g.ws[s];
+    if (w.depth++ == 0 && !w.retired.empty()) {
+      hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+      if (hipStreamIsCapturing(s, &cs) != hipSuccess) (void)hipGetLastError();
+      if (cs == hipStreamCaptureStatusNone && hipStreamSynchronize(s) == hipSuccess) {
+        for (void *p : w.retired) (void)hipFree(p);
+        w.retired.clear();
+      }
+    }
+  }
+  ~CallScope() {
+    std::lock_guard<std::mutex> lk(g.mu);
+    --g.ws[s].depth;
+  }
+  CallScope(const CallScope &) = delete;
+  CallScope &operator=(const CallScope &) = delete;
+};
 
 int io_buffer(hipStream_t s, size_t bytes, void **out) {
   std::lock_guard<std::mutex> lk(g.mu);
@@ -325,17 +375,41 @@ bool wants_tiled(const hipq_weight *w, int64_t M, bool may_allocate = true) {
 struct Scratch {
   bool fixed;
   hipStream_t s;
+  void *slot = nullptr; /* fixed: this stream's part of the static array */
   int get(size_t bytes, void **out) const {
     if (!fixed) return workspace(s, bytes, out);
     if (bytes > NOALLOC_SCRATCH_BYTES)
       return fail(HIPQ_ERR_NOT_SUPPORTED,
                   "this matmul needs %zu bytes of scratch for its quantized activations; the "
-                  "allocation-free entry point holds %zu",
+                  "allocation-free entry point holds %zu a stream",
                   bytes, NOALLOC_SCRATCH_BYTES);
-    *out = g.scratch_ptr[g.device];
+    *out = slot;
     return HIPQ_OK;
   }
 };
+
+/* The slot of the static array that belongs to stream s (the first four streams that use the
+ * allocation-free entry point get one each, until hipq_stream_release gives it back). */
+int noalloc_slot(hipStream_t s, void **out) {
+  std::lock_guard<std::mutex> lk(g.mu);
+  int free_slot = -1;
+  for (int i = 0; i < NOALLOC_SLOTS; ++i) {
+    if (g.noalloc_taken[i] && g.noalloc_stream[i] == s) {
+      *out = (char *)g.scratch_ptr[g.device] + (size_t)i * NOALLOC_SCRATCH_BYTES;
+      return HIPQ_OK;
+    }
+    if (!g.noalloc_taken[i] && free_slot < 0) free_slot = i;
+  }
+  if (free_slot < 0)
+    return fail(HIPQ_ERR_NOT_SUPPORTED,
+                "%d streams already use the allocation-free entry point, one slot of its scratch each; "
+                "hipq_stream_release gives a stream's slot back",
+                NOALLOC_SLOTS);
+  g.noalloc_taken[free_slot] = true;
+  g.noalloc_stream[free_slot] = s;
+  *out = (char *)g.scratch_ptr[g.device] + (size_t)free_slot * NOALLOC_SCRATCH_BYTES;
+  return HIPQ_OK;
+}
 
 int matmul_tiled(const hipq_weight *w, const float *A, int64_t M, int64_t lda, float *C, int64_t ldc,
                  hipStream_t s, int phase, const Scratch &sc);
@@ -527,8 +601,10 @@ int hipq_shutdown(void) {
   for (auto &kv : g.ws) {
     if (kv.second.ptr) (void)hipFree(kv.second.ptr);
     if (kv.second.io) (void)hipFree(kv.second.io);
+    for (void *p : kv.second.retired) (void)hipFree(p);
   }
   g.ws.clear();
+  for (int i = 0; i < NOALLOC_SLOTS; ++i) g.noalloc_taken[i] = false;
   {
     std::lock_guard<std::mutex> rl(g_ring.mu);
     if (g_ring.base) {
@@ -550,14 +626,21 @@ int hipq_stream_release(void *stream) {
   if (rc) return rc;
   hipStream_t s = (hipStream_t)stream;
   std::lock_guard<std::mutex> lk(g.mu);
+  for (int i = 0; i < NOALLOC_SLOTS; ++i) /* its slot of the allocation-free scratch, if it has one */
+    if (g.noalloc_taken[i] && g.noalloc_stream[i] == s) {
+      HIPQ_HIP(hipStreamSynchronize(s));
+      g.noalloc_taken[i] = false;
+    }
   auto it = g.ws.find(s);
   if (it == g.ws.end()) return HIPQ_OK;
   /* a caller that still enqueues on the stream from another thread holds the lock: refuse */
   std::unique_lock<std::recursive_mutex> el(it->second.enqueue, std::try_to_lock);
-  if (!el.owns_lock()) return fail(HIPQ_ERR_INVALID_ARGUMENT, "the stream is in use by another call");
+  if (!el.owns_lock() || it->second.depth)
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "the stream is in use by another call");
   HIPQ_HIP(hipStreamSynchronize(s));
   if (it->second.ptr) (void)hipFree(it->second.ptr);
   if (it->second.io) (void)hipFree(it->second.io);
+  for (void *p : it->second.retired) (void)hipFree(p);
   el.unlock();
   el.release();
   g.ws.erase(it);
@@ -837,6 +920,7 @@ int hipq_matmul(hipq_weight_t w, const float *A, int64_t M, int64_t lda, float *
   if ((rc = check_matmul_args(w, A, M, lda, C, ldc))) return rc;
   hipStream_t s = (hipStream_t)stream;
   EnqueueGuard eg(enqueue_lock(s));
+  CallScope call(s);
   const Scratch sc{false, s};
   if (mem == HIPQ_MEM_DEVICE) return matmul_device(w, A, M, lda, C, ldc, s, sc);
   if (mem != HIPQ_MEM_HOST) return fail(HIPQ_ERR_INVALID_ARGUMENT, "unknown mem kind %d", mem);
@@ -861,6 +945,7 @@ int hipq_matmul_each_row(hipq_weight_t w, const float *A, int64_t rows, int64_t 
   if (rows == 0) return HIPQ_OK;
   hipStream_t s = (hipStream_t)stream;
   EnqueueGuard eg(enqueue_lock(s));
+  CallScope call(s);
   const Scratch sc{false, s};
   const float *dA = A;
   float *dC = C;
@@ -896,10 +981,12 @@ int hipq_matmul_noalloc(hipq_weight_t w, const float *A, int64_t M, int64_t lda,
   if (rc) return rc;
   if ((rc = check_matmul_args(w, A, M, lda, C, ldc))) return rc;
   hipStream_t s = (hipStream_t)stream;
-  /* one scratch per GPU: calls submit one at a time; the kernels of two calls on
-   * different streams would still race on it, which is the caller's to avoid */
+  /* calls submit one at a time; each stream has its own slot of the scratch, so the kernels of
+   * calls on different streams do not share memory (two calls on ONE stream run in order) */
   EnqueueGuard eg(g.noalloc_enqueue);
-  return matmul_device(w, A, M, lda, C, ldc, s, Scratch{true, s});
+  void *slot = nullptr;
+  if ((rc = noalloc_slot(s, &slot))) return rc;
+  return matmul_device(w, A, M, lda, C, ldc, s, Scratch{true, s, slot});
 }
 
 int hipq_mlp_swiglu(hipq_weight_t w_act, hipq_weight_t w_mul, const float *A, int64_t M, int64_t lda,
@@ -915,6 +1002,7 @@ int hipq_mlp_swiglu(hipq_weight_t w_act, hipq_weight_t w_mul, const float *A, in
   if (M == 0) return HIPQ_OK;
   hipStream_t s = (hipStream_t)stream;
   EnqueueGuard eg(enqueue_lock(s));
+  CallScope call(s);
   const int64_t N = w_act->N, K = w_act->K;
   const size_t a_bytes = ((size_t)M * K * 4 + 255) & ~(size_t)255, o_bytes = ((size_t)M * N * 4 + 255) & ~(size_t)255;
   if (mem == HIPQ_MEM_DEVICE && M == 1 && hipq::gemv_fuses_swiglu(w_act, w_mul, A))
@@ -959,6 +1047,7 @@ int hipq_matmul_multi(int count, const hipq_weight_t *w, const float *A, int64_t
   if (M == 0) return HIPQ_OK;
   hipStream_t s = (hipStream_t)stream;
   EnqueueGuard eg(enqueue_lock(s));
+  CallScope call(s);
   if (mem == HIPQ_MEM_HOST) {
     /* the activation crosses once, the products run as for device memory, the outputs return */
     const int64_t Kh = w[0]->K;
@@ -985,6 +1074,30 @@ int hipq_matmul_multi(int count, const hipq_weight_t *w, const float *A, int64_t
   }
   if (M == 1 && hipq::gemv_fuses_quantizer_multi(count, w, A))
     return hipq::launch_gemv_fused_multi(count, w, A, C, s);
+  /* ONE reservation for the whole call, before anything is quantized: the largest scratch any
+   * member's product asks for (its quantized rows in the plane, row or tiled form, and behind the
+   * tiled form the partial products of a product in parts of K, which depend on the weight's tile
+   * copy: that is built first). Members of a group read the rows the group's first product
+   * quantized, so the block must not be replaced between them; `gen` is checked before every
+   * product that reuses them. */
+  uint64_t gen = 0;
+  {
+    size_t need = 0;
+    for (int i = 0; i < count; ++i) {
+      const hipq_weight *x = w[i];
+      size_t n = qact_bytes(x->dtype != HIPQ_Q4_0, M, x->K);
+      if (x->dtype != HIPQ_Q4_0 && wants_tiled(x, M)) {
+        if (!x->gt_base && (rc = hipq::ensure_gemm_tiles(const_cast<hipq_weight *>(x)))) return rc;
+        const size_t parts = x->dtype == HIPQ_Q4_K ? hipq::gemm_q4k_split_bytes(x, M) : hipq::gemm_q6k_split_bytes(x, M);
+        const size_t tiled = ((qact_tiled_bytes(M, x->K) + 255) & ~(size_t)255) + parts;
+        if (tiled > n) n = tiled;
+      }
+      if (n > need) need = n;
+    }
+    void *reserve = nullptr;
+    if ((rc = workspace(s, need, &reserve))) return rc;
+    gen = workspace_generation(s);
+  }
   /* one quantization per distinct activation format among the weights */
   /* two or more Q4_K weights against a few rows: one launch of the few-rows kernel for up to four of
    * them, where the launch as a whole is wide enough */
@@ -1022,6 +1135,7 @@ int hipq_matmul_multi(int count, const hipq_weight_t *w, const float *A, int64_t
         ++ng;
       }
       if (ng == 4 || (i == count && ng)) {
+        if ((rc = workspace_unmoved(s, gen))) return rc;
         if ((rc = hipq::launch_gemm_rows_q4k_multi(ng, gw, &qa, (int)M, (int)((M / 4) * 4), gc, gl, s))) return rc;
         ng = 0;
       }
@@ -1046,30 +1160,20 @@ int hipq_matmul_multi(int count, const hipq_weight_t *w, const float *A, int64_t
         if (!w[i]->gt_base && (rc = hipq::ensure_gemm_tiles(const_cast<hipq_weight *>(w[i])))) return rc;
         gw[ng] = w[i], gc[ng] = C[i], gl[ng] = ldc[i];
         if (++ng == 4) {
+          if ((rc = workspace_unmoved(s, gen))) return rc;
           if ((rc = hipq::launch_gemm_q4k_multi(ng, gw, &qa, (int)M, gc, gl, s))) return rc;
           ng = 0;
         }
       }
+      if (ng && (rc = workspace_unmoved(s, gen))) return rc;
       if (ng && (rc = hipq::launch_gemm_q4k_multi(ng, gw, &qa, (int)M, gc, gl, s))) return rc;
       continue;
-    }
-    if (members > 1) {
-      /* the products after the first read the activations the first one quantized: the workspace must
-       * not grow (and move) between them, so it is sized for the largest member first (a product of
-       * few tiles keeps its partial products of parts of K behind the activations) */
-      size_t parts_max = 0;
-      for (int i = 0; i < count; ++i) {
-        if (klass(w[i]) != k) continue;
-        if (!w[i]->gt_base && (rc = hipq::ensure_gemm_tiles(const_cast<hipq_weight *>(w[i])))) return rc;
-        const size_t pb = w[i]->dtype == HIPQ_Q4_K ? hipq::gemm_q4k_split_bytes(w[i], M) : hipq::gemm_q6k_split_bytes(w[i], M);
-        if (pb > parts_max) parts_max = pb;
-      }
-      void *reserve = nullptr;
-      if ((rc = workspace(s, ((qact_tiled_bytes(M, w[0]->K) + 255) & ~(size_t)255) + parts_max, &reserve))) return rc;
     }
     bool first = true;
     for (int i = 0; i < count; ++i)
       if (klass(w[i]) == k) {
+        /* the products after the first read the rows the first one quantized */
+        if (!first && (rc = workspace_unmoved(s, gen))) return rc;
         if ((rc = matmul_tiled(w[i], A, M, lda, C[i], ldc[i], s, first ? 0 : 1, Scratch{false, s}))) return rc;
         first = false;
       }
@@ -1110,7 +1214,8 @@ int hipq_matmul_multi(int count, const hipq_weight_t *w, const float *A, int64_t
     int64_t gl[4];
     int ng = 0;
     auto flush = [&]() -> int {
-      int frc = HIPQ_OK;
+      int frc = workspace_unmoved(s, gen);
+      if (frc) return frc;
       if (k == 0 && ng > 1 && hipq::gemm_rows_q40_fits_multi(ng, gw, M))
         frc = hipq::launch_gemm_rows_q40_multi(ng, gw, &qa, (int)M, gc, gl, s);
       else if (k == 0 && M > 8 && gw[0]->K % 256 == 0)
@@ -1144,6 +1249,7 @@ int hipq_time_matmul(int n_weights, const hipq_weight_t *w, const float *A, int6
   }
   hipStream_t s = (hipStream_t)stream;
   EnqueueGuard eg(enqueue_lock(s));
+  CallScope call(s);
   const int is_k = w[0]->dtype != HIPQ_Q4_0;
   bool tiled = true, rows = true;
   for (int i = 0; i < n_weights; ++i) {
@@ -1153,6 +1259,15 @@ int hipq_time_matmul(int n_weights, const hipq_weight_t *w, const float *A, int6
   void *memp = nullptr;
   QAct qa{};
   if (tiled) {
+    /* the loop multiplies every weight with the rows quantized here: reserve for the largest first */
+    size_t need = 0;
+    for (int i = 0; i < n_weights; ++i) {
+      if (!w[i]->gt_base && (rc = hipq::ensure_gemm_tiles(const_cast<hipq_weight *>(w[i])))) return rc;
+      const size_t parts = w[i]->dtype == HIPQ_Q4_K ? hipq::gemm_q4k_split_bytes(w[i], M) : hipq::gemm_q6k_split_bytes(w[i], M);
+      const size_t n = ((qact_tiled_bytes(M, w[i]->K) + 255) & ~(size_t)255) + parts;
+      if (n > need) need = n;
+    }
+    if ((rc = workspace(s, need, &memp))) return rc;
     if ((rc = matmul_tiled(w[0], A, M, lda, C, ldc, s, 2, Scratch{false, s}))) return rc;
   } else if (rows) {
     for (int i = 0; i < n_weights; ++i) /* the tile copies are built outside the timed loop */
@@ -1163,6 +1278,7 @@ int hipq_time_matmul(int n_weights, const hipq_weight_t *w, const float *A, int6
     qa = qact_carve(is_k, memp, M, w[0]->K);
     if ((rc = quantize_for(w[0], A, M, lda, qa, s))) return rc;
   }
+  const uint64_t gen = workspace_generation(s);
   hipEvent_t e0, e1;
   HIPQ_HIP(hipEventCreate(&e0));
   HIPQ_HIP(hipEventCreate(&e1));
@@ -1170,6 +1286,7 @@ int hipq_time_matmul(int n_weights, const hipq_weight_t *w, const float *A, int6
   HIPQ_HIP(hipEventRecord(e0, s));
   for (int it = 0; it < iters && !rc; ++it) {
     const hipq_weight *wi = w[it % n_weights];
+    if (phase == 1 && (rc = workspace_unmoved(s, gen))) break;
     if (tiled) {
       rc = matmul_tiled(wi, A, M, lda, C, ldc, s, phase, Scratch{false, s});
       continue;
@@ -1216,6 +1333,7 @@ int hipq_bench_matmul_steps(int n_weights, const hipq_weight_t *w, const float *
   }
   hipStream_t s = (hipStream_t)stream;
   EnqueueGuard eg(enqueue_lock(s));
+  CallScope call(s);
   const Scratch sc{false, s};
   /* one untimed call first: workspace and tile copies exist before the events */
   for (int i = 0; i < n_weights; ++i)
@@ -1315,6 +1433,7 @@ int hipq_moe_forward_ext(const hipq_moe_desc *desc, const hipq_moe_ext *ext, con
   if (d.tokens == 0) return HIPQ_OK;
   hipStream_t s = (hipStream_t)stream;
   EnqueueGuard eg(enqueue_lock(s));
+  CallScope call(s);
 
   /* device table of the 3E weight views, rebuilt only when the handles change; moe_mu keeps
    * the table from being rebuilt or freed by another thread before the launches below are in
@@ -1359,6 +1478,7 @@ int hipq_moe_forward_ext(const hipq_moe_desc *desc, const hipq_moe_ext *ext, con
   a.down = down;
   a.epi.kind = x_.variant;
   a.epi.alpha = x_.alpha;
+  a.epi.limit = x_.variant == HIPQ_MOE_GPT_OSS ? x_.limit : 0.f;
   a.epi.gate_bias = x_.gate_bias;
   a.epi.up_bias = x_.up_bias;
   a.epi.down_bias = x_.down_bias;
@@ -1375,39 +1495,90 @@ int hipq_moe_forward_ext(const hipq_moe_desc *desc, const hipq_moe_ext *ext, con
     return hipq::launch_moe(&a, ws, ws_bytes, dev_views, s);
   }
   if (mem != HIPQ_MEM_HOST) return fail(HIPQ_ERR_INVALID_ARGUMENT, "unknown mem kind %d", mem);
-  DevBuf dx, dr, dy, di, dw, dbr, dbg, dbu, dbd;
-  auto to_device = [&](DevBuf &b, const float *src, size_t n, const float **dst) -> int {
-    if (!src) return HIPQ_OK;
-    if (int r = b.alloc(n * 4)) return r;
-    HIPQ_HIP(hipMemcpy(b.p, src, n * 4, hipMemcpyHostToDevice));
-    *dst = (const float *)b.p;
-    return HIPQ_OK;
-  };
-  if ((rc = to_device(dbr, x_.router_bias, E, &a.router_bias))) return rc;
-  if (x_.variant == HIPQ_MOE_GPT_OSS) {
-    if ((rc = to_device(dbg, x_.gate_bias, E * I, &a.epi.gate_bias))) return rc;
-    if ((rc = to_device(dbu, x_.up_bias, E * I, &a.epi.up_bias))) return rc;
-    if ((rc = to_device(dbd, x_.down_bias, E * H, &a.epi.down_bias))) return rc;
+  /* host operands: device copies in the stream's operand buffer (no allocation per call); biases
+   * the caller keeps on the device are used where they are */
+  const bool gpt = x_.variant == HIPQ_MOE_GPT_OSS;
+  const bool host_biases = !x_.biases_on_device;
+  auto up256 = [](size_t n) { return (n + 255) & ~(size_t)255; };
+  const size_t n_router = router_logits ? T * E : H * E;
+  const size_t o_x = 0, o_r = o_x + up256(T * H * 4), o_y = o_r + up256(n_router * 4), o_i = o_y + up256(T * H * 4),
+               o_w = o_i + up256(T * k * 4), o_br = o_w + up256(T * k * 4),
+               o_bg = o_br + (host_biases && x_.router_bias ? up256(E * 4) : 0),
+               o_bu = o_bg + (host_biases && gpt ? up256(E * I * 4) : 0),
+               o_bd = o_bu + (host_biases && gpt ? up256(E * I * 4) : 0),
+               total = o_bd + (host_biases && gpt ? up256(E * H * 4) : 0);
+  void *io = nullptr;
+  if ((rc = io_buffer(s, total, &io))) return rc;
+  char *base = (char *)io;
+  if (host_biases) {
+    if (x_.router_bias) {
+      if ((rc = stage_copy(true, base + o_br, (void *)x_.router_bias, E * 4, E * 4, 1, s))) return rc;
+      a.router_bias = (const float *)(base + o_br);
+    }
+    if (gpt) {
+      if ((rc = stage_copy(true, base + o_bg, (void *)x_.gate_bias, I * 4, I * 4, E, s))) return rc;
+      if ((rc = stage_copy(true, base + o_bu, (void *)x_.up_bias, I * 4, I * 4, E, s))) return rc;
+      if ((rc = stage_copy(true, base + o_bd, (void *)x_.down_bias, H * 4, H * 4, E, s))) return rc;
+      a.epi.gate_bias = (const float *)(base + o_bg);
+      a.epi.up_bias = (const float *)(base + o_bu);
+      a.epi.down_bias = (const float *)(base + o_bd);
+    }
   }
-  if ((rc = dx.alloc(T * H * 4))) return rc;
-  if ((rc = dr.alloc((router_logits ? T * E : H * E) * 4))) return rc;
-  if ((rc = dy.alloc(T * H * 4))) return rc;
-  if ((rc = di.alloc(T * k * 4))) return rc;
-  if ((rc = dw.alloc(T * k * 4))) return rc;
-  if ((rc = stage_copy(true, dx.p, (void *)x, H * 4, H * 4, T, s))) return rc;
-  HIPQ_HIP(hipMemcpy(dr.p, router_logits ? router_logits : router_weight,
-                     (router_logits ? T * E : H * E) * 4, hipMemcpyHostToDevice));
-  a.x = (const float *)dx.p;
-  a.router_logits = router_logits ? (const float *)dr.p : nullptr;
-  a.router_weight = router_weight ? (const float *)dr.p : nullptr;
-  a.y = (float *)dy.p;
-  a.topk_idx = (int32_t *)di.p;
-  a.topk_w = (float *)dw.p;
+  if ((rc = stage_copy(true, base + o_x, (void *)x, H * 4, H * 4, T, s))) return rc;
+  /* logits [T x E] or the router weight [H x E] */
+  if ((rc = stage_copy(true, base + o_r, (void *)(router_logits ? router_logits : router_weight), E * 4, E * 4,
+                       router_logits ? T : H, s)))
+    return rc;
+  a.x = (const float *)(base + o_x);
+  a.router_logits = router_logits ? (const float *)(base + o_r) : nullptr;
+  a.router_weight = router_weight ? (const float *)(base + o_r) : nullptr;
+  a.y = (float *)(base + o_y);
+  a.topk_idx = (int32_t *)(base + o_i);
+  a.topk_w = (float *)(base + o_w);
   if ((rc = hipq::launch_moe(&a, ws, ws_bytes, dev_views, s))) return rc;
-  if ((rc = stage_copy(false, dy.p, y, H * 4, H * 4, T, s))) return rc;
-  if (topk_idx) HIPQ_HIP(hipMemcpy(topk_idx, di.p, T * k * 4, hipMemcpyDeviceToHost));
-  if (topk_w) HIPQ_HIP(hipMemcpy(topk_w, dw.p, T * k * 4, hipMemcpyDeviceToHost));
+  if ((rc = stage_copy(false, base + o_y, y, H * 4, H * 4, T, s))) return rc;
+  if (topk_idx && (rc = stage_copy(false, base + o_i, topk_idx, k * 4, k * 4, T, s))) return rc;
+  if (topk_w && (rc = stage_copy(false, base + o_w, topk_w, k * 4, k * 4, T, s))) return rc;
   return HIPQ_OK;
+}
+
+/* ---- device memory for callers without a HIP runtime of their own ------------ */
+
+int hipq_device_alloc(void **ptr, size_t bytes) {
+  int rc = require_ready();
+  if (rc) return rc;
+  if (!ptr) return fail(HIPQ_ERR_INVALID_ARGUMENT, "null argument");
+  *ptr = nullptr;
+  hipError_t e = hipMalloc(ptr, bytes ? bytes : 16);
+  if (e != hipSuccess) {
+    *ptr = nullptr;
+    return fail(HIPQ_ERR_OUT_OF_MEMORY, "hipMalloc(%zu): %s", bytes, hipGetErrorString(e));
+  }
+  return HIPQ_OK;
+}
+
+int hipq_device_free(void *ptr) {
+  if (!ptr) return HIPQ_OK;
+  int rc = require_ready();
+  if (rc) return rc;
+  HIPQ_HIP(hipFree(ptr)); /* waits for the device's work that may still read it */
+  return HIPQ_OK;
+}
+
+int hipq_device_upload(void *dst_device, const void *src_host, size_t bytes, void *stream) {
+  int rc = require_ready();
+  if (rc) return rc;
+  if (!dst_device || !src_host) return fail(HIPQ_ERR_INVALID_ARGUMENT, "null argument");
+  if ((rc = stage_copy(true, dst_device, (void *)src_host, bytes, bytes, 1, (hipStream_t)stream))) return rc;
+  HIPQ_HIP(hipStreamSynchronize((hipStream_t)stream)); /* page-locked sources are read by the DMA engine later */
+  return HIPQ_OK;
+}
+
+int hipq_device_download(void *dst_host, const void *src_device, size_t bytes, void *stream) {
+  int rc = require_ready();
+  if (rc) return rc;
+  if (!dst_host || !src_device) return fail(HIPQ_ERR_INVALID_ARGUMENT, "null argument");
+  return stage_copy(false, (void *)src_device, dst_host, bytes, bytes, 1, (hipStream_t)stream);
 }
 
 /* ---- offline weight quantizers ---------------------------------------------- */

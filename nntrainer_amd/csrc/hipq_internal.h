@@ -262,10 +262,13 @@ int launch_gemm_rows_q40_fused(int count, const hipq_weight *const *w, const flo
 /* moe.hip ----------------------------------------------------------------- */
 /* Variant of the expert MLP. kind 0: h = silu(g) * u, y = down(h) (qwen_moe_layer.cpp:332-392).
  * kind 1: g and u take a bias, h = (g / (1 + exp(-alpha g))) * (u + 1), y = down(h) + bias
- * (gpt_oss_moe_layer.cpp:372-449). Biases are device pointers, [E][I], [E][I], [E][H]. */
+ * (gpt_oss_moe_layer.cpp:372-449); with limit > 0 the biased g and u are clamped first, g to
+ * at most limit and u to [-limit, limit] (gpt_oss_moe_layer_cached.cpp:497-507). Biases are
+ * device pointers, [E][I], [E][I], [E][H]. */
 struct MoeEpi {
   const float *gate_bias, *up_bias, *down_bias;
   float alpha;
+  float limit;
   int kind;
 };
 struct MoeArgs {

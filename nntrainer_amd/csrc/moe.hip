@@ -397,12 +397,18 @@ __device__ __forceinline__ float silu_ref(float g) {
 
 /* The activation between the projections and the bias of the down projection, by expert
  * variant (hipq_internal.h, MoeEpi). For the biased variant the value of column col of expert
- * e is (g / (1 + exp(-alpha g))) * (u + 1) with g and u the biased products, in fp32
- * (gpt_oss_moe_layer.cpp:406-437; swiglu with alpha, fallback_internal.cpp:425-432). */
+ * e is (g / (1 + exp(-alpha g))) * (u + 1) with g and u the biased (and, for the cached layer,
+ * clamped) products, in fp32 (gpt_oss_moe_layer.cpp:406-437; swiglu with alpha,
+ * fallback_internal.cpp:425-432). */
 __device__ __forceinline__ float moe_act(const hipq::MoeEpi &ep, int e, int I, int col, float g, float u) {
   if (ep.kind == 0) return silu_ref(g) * u;
   g = g + ep.gate_bias[(size_t)e * I + col];
   u = u + ep.up_bias[(size_t)e * I + col];
+  if (ep.limit > 0.f) { /* the cached layer's clamps, gpt_oss_moe_layer_cached.cpp:497-507 */
+    g = g < ep.limit ? g : ep.limit;
+    u = u > -ep.limit ? u : -ep.limit;
+    u = u < ep.limit ? u : ep.limit;
+  }
   u = u + 1.f;
   return (g / (1.f + expf(-ep.alpha * g))) * u;
 }

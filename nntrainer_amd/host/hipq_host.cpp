@@ -173,6 +173,25 @@ hipq_weight_t upload(const void *host_bytes, const WeightSpec &spec) {
   return w;
 }
 
+float *device_floats(const float *host, size_t n) {
+  require_runtime();
+  if (!host)
+    throw std::invalid_argument("[hipq] device_floats: the tensor has no data");
+  void *p = nullptr;
+  check(hipq_device_alloc(&p, n * sizeof(float)), "hipq_device_alloc");
+  const int rc = hipq_device_upload(p, host, n * sizeof(float), nullptr);
+  if (rc != HIPQ_OK) {
+    hipq_device_free(p);
+    check(rc, "hipq_device_upload");
+  }
+  return static_cast<float *>(p);
+}
+
+void device_release(void *p) noexcept {
+  if (p)
+    hipq_device_free(p);
+}
+
 void release(hipq_weight_t w) noexcept {
   if (w)
     hipq_weight_destroy(w);
@@ -196,6 +215,8 @@ void moe_forward_resident(const MoeShape &shape, const hipq_weight_t *gate, cons
   ext.gate_bias = extras ? extras->gate_bias : nullptr;
   ext.up_bias = extras ? extras->up_bias : nullptr;
   ext.down_bias = extras ? extras->down_bias : nullptr;
+  ext.limit = extras ? extras->limit : 0.f;
+  ext.biases_on_device = extras && extras->biases_on_device ? 1 : 0;
   check(hipq_moe_forward_ext(&desc, &ext, gate, up, down, x, nullptr, router_weight, y, nullptr, nullptr,
                              HIPQ_MEM_HOST, nullptr),
         "hipq_moe_forward");

@@ -131,9 +131,15 @@ struct MoeShape {
 struct MoeExtras {
   bool gpt_oss = false;
   float alpha = 1.702f;
+  float limit = 0.f; /* > 0: the cached layer's clamps on the biased gate and up values */
   const float *router_bias = nullptr;
   const float *gate_bias = nullptr, *up_bias = nullptr, *down_bias = nullptr;
+  bool biases_on_device = false; /* the four pointers above are device copies (device_floats) */
 };
+
+/** A device copy of n floats the caller owns; freed with device_release. */
+float *device_floats(const float *host, size_t n);
+void device_release(void *p) noexcept;
 
 /** A device copy that the caller owns (not entered into a cache): for weights whose host bytes
  *  come and go (virtual tensors), where an address is no identity. */

@@ -17,6 +17,7 @@ static constexpr unsigned int SINGLE_INOUT_IDX = 0;
 MoELayerHip::~MoELayerHip() {
   for (hipq_weight_t w : resident)
     hipq_host::release(w);
+  drop_device_biases();
 }
 
 void MoELayerHip::setProperty(const std::vector<std::string> &values) {
@@ -170,26 +171,39 @@ void MoELayerHip::run(RunLayerContext &context, const float *x, float *y, unsign
 
   hipq_host::MoeExtras extras;
   if (gpt_oss) {
-    bias_gate.resize((size_t)E * intermediate);
-    bias_up.resize((size_t)E * intermediate);
-    bias_down.resize((size_t)E * hidden);
-    for (unsigned int e = 0; e < E; ++e) {
-      with_bytes(expert_gate_bias_indices[e], [&](Tensor &t) {
-        std::memcpy(&bias_gate[(size_t)e * intermediate], t.getData<float>(), (size_t)intermediate * 4);
-      });
-      with_bytes(expert_up_bias_indices[e], [&](Tensor &t) {
-        std::memcpy(&bias_up[(size_t)e * intermediate], t.getData<float>(), (size_t)intermediate * 4);
-      });
-      with_bytes(expert_down_bias_indices[e], [&](Tensor &t) {
-        std::memcpy(&bias_down[(size_t)e * hidden], t.getData<float>(), (size_t)hidden * 4);
-      });
+    /* the biases go to the device once, with the weights: [E x I], [E x I], [E x H] gathered from
+     * the experts' tensors, and the router's [E]; read() drops them as it drops the weights */
+    if (!dev_bias_gate) {
+      std::vector<float> bias_gate((size_t)E * intermediate), bias_up((size_t)E * intermediate),
+        bias_down((size_t)E * hidden);
+      for (unsigned int e = 0; e < E; ++e) {
+        with_bytes(expert_gate_bias_indices[e], [&](Tensor &t) {
+          std::memcpy(&bias_gate[(size_t)e * intermediate], t.getData<float>(), (size_t)intermediate * 4);
+        });
+        with_bytes(expert_up_bias_indices[e], [&](Tensor &t) {
+          std::memcpy(&bias_up[(size_t)e * intermediate], t.getData<float>(), (size_t)intermediate * 4);
+        });
+        with_bytes(expert_down_bias_indices[e], [&](Tensor &t) {
+          std::memcpy(&bias_down[(size_t)e * hidden], t.getData<float>(), (size_t)hidden * 4);
+        });
+      }
+      dev_bias_gate = hipq_host::device_floats(bias_gate.data(), bias_gate.size());
+      dev_bias_up = hipq_host::device_floats(bias_up.data(), bias_up.size());
+      dev_bias_down = hipq_host::device_floats(bias_down.data(), bias_down.size());
     }
+    if (with_router_bias && !dev_bias_router)
+      dev_bias_router = hipq_host::device_floats(context.getWeight(gate_bias_idx).getData<float>(), E);
     extras.gpt_oss = true;
     extras.alpha = 1.702f; /* gpt_oss_moe_layer.h:126 */
-    extras.gate_bias = bias_gate.data();
-    extras.up_bias = bias_up.data();
-    extras.down_bias = bias_down.data();
-    extras.router_bias = with_router_bias ? context.getWeight(gate_bias_idx).getData<float>() : nullptr;
+    /* only the cached layer clamps (gpt_oss_moe_layer_cached.cpp:497-507, limit 7.0 from
+     * gpt_oss_moe_layer_cached.h:137); the uncached one has the two lines commented out
+     * (gpt_oss_moe_layer.cpp:414, 419) */
+    extras.limit = cached ? 7.0f : 0.f;
+    extras.gate_bias = dev_bias_gate;
+    extras.up_bias = dev_bias_up;
+    extras.down_bias = dev_bias_down;
+    extras.router_bias = with_router_bias ? dev_bias_router : nullptr;
+    extras.biases_on_device = true;
   }
 
   if (cached) {
@@ -265,6 +279,14 @@ void MoELayerHip::incremental_forwarding(RunLayerContext &context, unsigned int 
   }
 }
 
+void MoELayerHip::drop_device_biases() noexcept {
+  hipq_host::device_release(dev_bias_gate);
+  hipq_host::device_release(dev_bias_up);
+  hipq_host::device_release(dev_bias_down);
+  hipq_host::device_release(dev_bias_router);
+  dev_bias_gate = dev_bias_up = dev_bias_down = dev_bias_router = nullptr;
+}
+
 void MoELayerHip::calcDerivative(RunLayerContext &) {
   throw exception::not_supported("MoELayerHip does not support backwarding");
 }
@@ -279,6 +301,7 @@ void MoELayerHip::calcGradient(RunLayerContext &) {
     for (hipq_weight_t w : resident)                                                                \
       hipq_host::release(w);                                                                        \
     resident.clear();                                                                               \
+    drop_device_biases();                                                                           \
   } while (0)
 
 void MoELayerHip::read(std::ifstream &file, RunLayerContext &run_context, bool opt_var,

@@ -94,7 +94,10 @@ private:
   std::vector<unsigned int> expert_gate_bias_indices;
   std::vector<unsigned int> expert_up_bias_indices;
   std::vector<unsigned int> expert_down_bias_indices;
-  std::vector<float> bias_gate, bias_up, bias_down; /* [E x I], [E x I], [E x H], gathered per call */
+  /* device copies of the biases, [E x I], [E x I], [E x H] and the router's [E]: made at the first
+   * step, dropped when the framework reads the layer's weights again */
+  float *dev_bias_gate = nullptr, *dev_bias_up = nullptr, *dev_bias_down = nullptr, *dev_bias_router = nullptr;
+  void drop_device_biases() noexcept;
   /* cached: device copies this layer owns, gate | up | down, made at an expert's first use */
   std::vector<hipq_weight_t> resident;
 };

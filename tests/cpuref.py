@@ -286,3 +286,19 @@ def moe_forward_cached(x, logits, gate, up, down, topk, kind="q4_K", gpt_oss=Fal
                                arr(down), _ptr(gb), _ptr(ub), _ptr(db), _c.c_float(alpha), _c.c_float(limit),
                                _ptr(y), _ptr(idx), _ptr(wt))
     return y, idx, wt
+
+
+def router_logits(x, wr, topk, bias=None):
+    """x . wr in fp32, as the layers form their router logits (input.dot(gate_weights),
+    qwen_moe_layer.cpp:436). The order of the fp32 sums is the BLAS's there and the device's here,
+    so a case must not sit on a routing tie: the softmax values of the last expert taken and the
+    first one left out differ by far more than such rounding can move them."""
+    x = np.ascontiguousarray(x, np.float32)
+    wr = np.ascontiguousarray(wr, np.float32)
+    logits = (x @ wr).astype(np.float32)
+    if bias is not None:
+        logits = (logits + np.asarray(bias, np.float32)).astype(np.float32)
+    p = np.exp(logits.astype(np.float64) - logits.max(1, keepdims=True))
+    p = np.sort(p / p.sum(1, keepdims=True), axis=1)[:, ::-1]
+    assert (p[:, topk - 1] - p[:, topk] > 1e-4 * p[:, 0]).all(), "routing tie in the test case"
+    return logits
