@@ -5,8 +5,10 @@ A step is one pass of the hot path over one batch: hipq_matmul on device-residen
 inputs = activation quantizer (fp32 -> Q8_K) + Q4_K x Q8_K block-dot GEMM, at the
 prefill shape BASELINE.json quotes its metric on (configs[1]: M=512, K=4096,
 N=12288). Prints ONE JSON line. Also measured and attached to the same line: the
-decode GEMV (M=1) over the same matrix at HBM-resident size, kernel-only timings
-with HIP events, and the reference CPU path timed on this box's host cores.
+decode GEMV (M=1) over the same matrix at HBM-resident size and over a sweep of widths,
+the kernels' own durations (start and stop events attached to every launch), the FC stack
+of the whole 28-layer decoder of configs[4], host-memory calls, and the reference CPU path
+timed on this box's host cores with both of its thread front-ends.
 """
 import argparse
 import ctypes
@@ -28,6 +30,48 @@ TRAFFIC_GEMM_C2 = 49.00e6 + 25.17e6
 TRAFFIC_GEMV_C2 = 28.45e6 + 0.05e6
 TRAFFIC_GEMV_LM_HEAD = 350.25e6 + 0.62e6
 METRIC = "Q4 GEMV effective GB/s (%HBM peak); prefill GEMM int8 TOPS (%MFMA peak)"
+
+
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
+
+
+def cpu_baseline_thread_pool(blocks_host, a_host, budget_s=8.0):
+    """The same product through the reference's default x86 front-end (ggml_interface_mixed.cpp:532-638):
+    a pool of hardware_concurrency() threads (bs_thread_pool_manager.hpp:41), whatever share of the
+    machine this process has. Its thread count is what the pool reports."""
+    import numpy as np
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    so = os.path.join(ROOT, "oracle", "_ref", "libnntr_ref_mixed.so")
+    if not os.path.exists(so):
+        return None
+    lib = ctypes.CDLL(so)
+    lib.ref_init()
+    b = np.zeros_like(blocks_host)
+    lib.ref_repack_q4_K_x8(ctypes.c_void_p(b.ctypes.data), ctypes.c_void_p(blocks_host.ctypes.data),
+                           ctypes.c_size_t(blocks_host.size), ctypes.c_uint(N), ctypes.c_uint(K))
+    c = np.zeros((M, N), np.float32)
+    run = lambda: lib.ref_gemm_q4_K(ctypes.c_uint(M), ctypes.c_uint(N), ctypes.c_uint(K),
+                                    ctypes.c_void_p(a_host.ctypes.data), ctypes.c_void_p(b.ctypes.data),
+                                    ctypes.c_void_p(c.ctypes.data))
+    run()
+    t0, reps = time.perf_counter(), 0
+    while True:
+        run()
+        reps += 1
+        el = time.perf_counter() - t0
+        if el > budget_s or reps >= 400:
+            break
+    sec = el / reps
+    return {"value": round(2.0 * M * N * K / sec / 1e12, 4), "unit": "TOPS", "threads": int(lib.ref_max_threads()),
+            "kind": "reference", "front_end": "thread pool of hardware_concurrency() threads (the x86 default)",
+            "sample": "%d full passes (%.2f s each), same inputs" % (reps, sec)}
 
 
 def cpu_baseline(blocks_host, a_host, gpu_out, budget_s=12.0):
@@ -70,6 +114,8 @@ def cpu_baseline(blocks_host, a_host, gpu_out, budget_s=12.0):
     sec = el / reps
     err = float(np.abs(gpu_out - c).max() / np.abs(c).max())
     return {"value": round(2.0 * M * N * K / sec / 1e12, 4), "unit": "TOPS", "cores": cores, "kind": kind,
+            "front_end": "OpenMP, hardware_concurrency() / 2 threads for a GEMM (ggml_interface_omp.cpp:331, 434)",
+            "cpu_model": cpu_model(), "cpus_visible": os.cpu_count(),
             "sample": "%d full passes of the same M=%d K=%d N=%d Q4_K matmul (%.2f s each), same inputs"
                       % (reps, M, K, N, sec),
             "gpu_vs_cpu_max_rel_err": err}
@@ -124,9 +170,18 @@ def main():
     stream = torch.cuda.current_stream().cuda_stream
     gen = torch.Generator(device="cuda").manual_seed(1)
 
-    # synthetic inputs, generated and quantized on the device
-    w32 = torch.randn((N, K), generator=gen, device="cuda", dtype=torch.float32) * 0.02
-    a = torch.randn((M, K), generator=gen, device="cuda", dtype=torch.float32)
+    # The headline's inputs are configs[1] as the parity test of the same configuration draws them
+    # (tests/test_gpu_configs.py::test_c2_q4_K_prefill_gemm): the repository's bit-reproducible generator,
+    # stream 1, weights N(0, 0.02) from sample 0 and activations N(0, 1) behind them; quantized on the
+    # device by the byte-exact weight quantizer. The other sections below draw theirs from torch's
+    # generator on the device (not the tests' data; shapes and distributions as stated there).
+    from nntrainer_amd import synth
+    w32_host = synth.normal(1, (N, K), 0.02)
+    a_host_in = synth.normal(1, (M, K), 1.0, first=N * K)
+    input_digest = {"weights_fp32": synth.digest(w32_host), "activations_fp32": synth.digest(a_host_in)}
+    w32 = torch.from_numpy(w32_host).cuda()
+    a = torch.from_numpy(a_host_in).cuda()
+    del w32_host
     blocks = torch.empty(capi.weight_nbytes("q4_K", N, K), dtype=torch.uint8, device="cuda")
     capi.quantize_weights("q4_K", w32, N, K, blocks, stream=stream)
     torch.cuda.synchronize()
@@ -135,27 +190,49 @@ def main():
     del w32
     c = torch.empty((M, N), device="cuda", dtype=torch.float32)
 
+    def timed(ws_, a_, m_, c_, iters):
+        """(ms per call, {kernel: (launches, mean ms)}, ms of the kernels that are not the activation
+        quantizer per call, name of the longest of them): `iters` hipq_matmul calls between two events,
+        then the same calls again with a start and a stop event attached to every launch."""
+        call_ms = capi.matmul_loop(ws_, a_, m_, c_, iters, stream=stream)
+        with capi.LaunchTiming(4 * (iters + len(ws_)) + 16) as lt:
+            capi.matmul_loop(ws_, a_, m_, c_, iters, stream=stream)
+        kern = lt.by_kernel()
+        calls = iters + len(ws_)
+        prod = {k_: v_ for k_, v_ in kern.items() if "quantize" not in k_}
+        prod_ms = sum(cnt * mean for cnt, mean in prod.values()) / calls
+        main_k = max(prod, key=lambda k_: prod[k_][0] * prod[k_][1]) if prod else ""
+        return call_ms, kern, prod_ms, main_k
+
     # ---- the timed region: K steps of the whole hot path -------------------
-    # A block = K steps of hipq_matmul, bracketed by synchronize() on both sides (wall clock) and
-    # by two HIP events on the launch stream, nothing else in the stream: ms_per_step. Each
-    # block is followed by an instrumented one over the same weights, in which every launch
-    # carries its own start and stop event (the kernel's own duration, as a kernel trace reports
-    # it): roofline.kernel_ms and quantizer_ms. Attaching events to a launch delays the next
-    # launch by several microseconds, so the instrumented block's own total is reported beside
-    # the figures and is not the step time. Blocks are repeated and medians reported: 20 steps
-    # are 1.5 ms, short enough for the clock state of the moment to move one block by percents.
+    # A block = `steps` calls of hipq_matmul from a C loop (hipq_bench_matmul_loop of libhipq_bench.so,
+    # which links the product library and calls its public entry point), bracketed by synchronize() on
+    # both sides (wall clock) and by two HIP events on the launch stream, nothing else in the stream:
+    # ms_per_step. Each block is followed by the same loop with the library's kernel timing switched on
+    # (hipq_launch_timing_begin / _end: every launch carries its own start and stop event, the kernel's
+    # own duration as a kernel trace reports it): roofline.kernel_ms and quantizer_ms. Attaching events
+    # to a launch delays the next launch by several microseconds, so the timed loop's own total is not
+    # the step time. Blocks are repeated and medians reported: 20 steps are 1.5 ms, short enough for
+    # the clock state of the moment to move one block by percents.
     for i in range(args.warmup):
         capi.matmul(weights[i % n_copies], a, M, c, stream=stream)
     torch.cuda.synchronize()
     blocks_timed, blocks_instr = [], []
+    gemm_kernel_name = ""
     for rep in range(5):
         torch.cuda.synchronize()
         t0 = time.perf_counter()
-        ev_step = capi.time_matmul(weights, a, M, c, args.steps, phase=0, stream=stream)
+        ev_step = capi.matmul_loop(weights, a, M, c, args.steps, stream=stream)
         torch.cuda.synchronize()
-        wall = (time.perf_counter() - t0) / args.steps
+        wall = (time.perf_counter() - t0) / (args.steps + n_copies)  # the loop makes one untimed call per weight first
         blocks_timed.append((ev_step, wall))
-        blocks_instr.append(capi.bench_matmul_steps(weights, a, M, c, args.steps, stream=stream))
+        with capi.LaunchTiming(4 * (args.steps + n_copies)) as lt:
+            capi.matmul_loop(weights, a, M, c, args.steps, stream=stream)
+        kern = lt.by_kernel()
+        q_ms = sum(mean for k_, (cnt, mean) in kern.items() if "quantize" in k_)
+        g_name = max((k_ for k_ in kern if "quantize" not in k_), key=lambda k_: kern[k_][1])
+        blocks_instr.append((q_ms + kern[g_name][1], q_ms, kern[g_name][1]))
+        gemm_kernel_name = g_name
     blocks_timed.sort()
     step_ms = blocks_timed[len(blocks_timed) // 2][0]
     blocks_instr.sort(key=lambda b: b[2])
@@ -194,13 +271,13 @@ def main():
     capi.host_free(pc)
 
     # ---- decode GEMV over the same matrix, weights rotating through HBM ----
+    # One row against a matrix of this size is ONE launch (the workgroups quantize the row themselves
+    # while their weights are on the way): kernel_ms is that kernel's own duration.
     a1 = a[:1].contiguous()
     c1 = torch.empty((1, N), device="cuda", dtype=torch.float32)
     gv_bytes = N * K * 144 // 256 + 4 * K + 4 * N
-    capi.time_matmul(weights, a1, 1, c1, 2 * n_copies, phase=0, stream=stream)
-    gemv_ms = capi.time_matmul(weights, a1, 1, c1, 40 * n_copies, phase=1, stream=stream)
-    gemv_all_ms = capi.time_matmul(weights, a1, 1, c1, 40 * n_copies, phase=0, stream=stream)
-    gemv_hot_ms = capi.time_matmul(weights[:1], a1, 1, c1, 400, phase=1, stream=stream)
+    gemv_all_ms, gemv_kern, gemv_ms, gemv_kernel_name = timed(weights, a1, 1, c1, 40 * n_copies)
+    _, _, gemv_hot_ms, _ = timed(weights[:1], a1, 1, c1, 400)
     gemv_gbs = gv_bytes / (gemv_ms * 1e-3) / 1e9
 
     # ---- a batch of decode rows against the same matrices: Q4_K on the matrix cores with the
@@ -209,25 +286,35 @@ def main():
     for mr in (8, 4, 16, 64):
         ar = torch.randn((mr, K), generator=gen, device="cuda", dtype=torch.float32)
         cr_ = torch.empty((mr, N), device="cuda", dtype=torch.float32)
-        capi.time_matmul(weights, ar, mr, cr_, 2 * n_copies, phase=1, stream=stream)
-        rows_ms[mr] = (capi.time_matmul(weights, ar, mr, cr_, 20 * n_copies, phase=1, stream=stream),
-                       capi.time_matmul(weights, ar, mr, cr_, 20 * n_copies, phase=0, stream=stream))
+        call_, _, prod_, _ = timed(weights, ar, mr, cr_, 20 * n_copies)
+        rows_ms[mr] = (prod_, call_)
 
-    # ---- the same GEMV at lm_head size (N=151936: 350 MB of Q4_K per matrix) ----
-    NL = 151936
-    wl32 = torch.randn((NL, K), generator=gen, device="cuda", dtype=torch.float32) * 0.02
-    blocks_l = torch.empty(capi.weight_nbytes("q4_K", NL, K), dtype=torch.uint8, device="cuda")
-    capi.quantize_weights("q4_K", wl32, NL, K, blocks_l, stream=stream)
-    torch.cuda.synchronize()
-    del wl32
-    big = [capi.Weight("q4_K", NL, K, blocks_l, mem=capi.MEM_DEVICE) for _ in range(3)]
-    cl = torch.empty((1, NL), device="cuda", dtype=torch.float32)
-    capi.time_matmul(big, a1, 1, cl, 6, phase=1, stream=stream)
-    big_ms = capi.time_matmul(big, a1, 1, cl, 60, phase=1, stream=stream)
-    big_bytes = NL * K * 144 // 256 + 4 * K + 4 * NL
+    # ---- the Q4_K decode GEMV over widths from 4096 to the lm_head's: where the kernel meets the HBM
+    # bound. Per width: copies that together exceed twice the last-level cache, the product kernel's own
+    # duration against the algorithmic bytes (weights + 4K + 4N), and the whole call.
+    sweep = []
+    for n_ in (4096, 12288, 32768, 65536, 151936):
+        w32_ = torch.randn((n_, K), generator=gen, device="cuda", dtype=torch.float32) * 0.02
+        b_ = torch.empty(capi.weight_nbytes("q4_K", n_, K), dtype=torch.uint8, device="cuda")
+        capi.quantize_weights("q4_K", w32_, n_, K, b_, stream=stream)
+        torch.cuda.synchronize()
+        del w32_
+        by_ = n_ * K * 144 // 256 + 4 * K + 4 * n_
+        copies_ = max(3, min(64, (600 << 20) // by_ + 1))
+        ws_ = [capi.Weight("q4_K", n_, K, b_, mem=capi.MEM_DEVICE) for _ in range(copies_)]
+        cn_ = torch.empty((1, n_), device="cuda")
+        call_, _, prod_, name_ = timed(ws_, a1, 1, cn_, max(60, 6 * copies_))
+        for w_ in ws_:
+            w_.destroy()
+        del b_
+        sweep.append({"N": n_, "copies": copies_, "kernel": name_, "kernel_ms": round(prod_, 5),
+                      "ms_per_call": round(call_, 5), "algorithmic_bytes": by_,
+                      "kernel_gbs": round(by_ / (prod_ * 1e-3) / 1e9, 1),
+                      "frac": round(by_ / (prod_ * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)})
+    big_ms = sweep[-1]["kernel_ms"]
+    big_bytes = sweep[-1]["algorithmic_bytes"]
     big_gbs = big_bytes / (big_ms * 1e-3) / 1e9
-    for w in big:
-        w.destroy()
+    big_kernel_name = sweep[-1]["kernel"]
 
     # ---- the other GEMV configurations: C1 (Q4_0, 4096 x 4096) and C3 (Q6_K lm_head) ----
     def gemv_case(kind, n, k, copies, bytes_per_weight_num, bytes_per_weight_den, prefill_rows=0):
@@ -239,9 +326,7 @@ def main():
         ws_ = [capi.Weight(kind, n, k, b_, mem=capi.MEM_DEVICE) for _ in range(copies)]
         a_ = torch.randn((1, k), generator=gen, device="cuda")
         c_ = torch.empty((1, n), device="cuda")
-        capi.time_matmul(ws_, a_, 1, c_, 2 * copies, phase=1, stream=stream)
-        ms_ = capi.time_matmul(ws_, a_, 1, c_, max(60, 4 * copies), phase=1, stream=stream)
-        all_ms_ = capi.time_matmul(ws_, a_, 1, c_, max(60, 4 * copies), phase=0, stream=stream)
+        all_ms_, _, ms_, _ = timed(ws_, a_, 1, c_, max(60, 4 * copies))
         capi.matmul(ws_[0], a_, 1, c_, stream=stream)
         torch.cuda.synchronize()
         host_ = None if args.no_cpu else (b_.cpu().numpy(), a_.cpu().numpy(), c_.cpu().numpy())
@@ -250,11 +335,8 @@ def main():
             # the same weights against `prefill_rows` rows: the matrix-core product of the format
             ap_ = torch.randn((prefill_rows, k), generator=gen, device="cuda")
             cp_ = torch.empty((prefill_rows, n), device="cuda")
-            capi.time_matmul(ws_, ap_, prefill_rows, cp_, 2 * copies, phase=0, stream=stream)
-            pre_ = (sorted(capi.time_matmul(ws_, ap_, prefill_rows, cp_, 6 * copies, phase=1, stream=stream)
-                           for _ in range(3))[1],
-                    sorted(capi.time_matmul(ws_, ap_, prefill_rows, cp_, 6 * copies, phase=0, stream=stream)
-                           for _ in range(3))[1])
+            runs_ = sorted((timed(ws_, ap_, prefill_rows, cp_, 6 * copies) for _ in range(3)), key=lambda r_: r_[2])
+            pre_ = (runs_[1][2], runs_[1][0], runs_[1][3])
             del ap_, cp_
         for w_ in ws_:
             w_.destroy()
@@ -276,8 +358,7 @@ def main():
             ws_ = [capi.Weight("q4_0", n_, k_, b_, mem=capi.MEM_DEVICE) for _ in range(8)]
             a_ = torch.randn((rows, k_), generator=gen, device="cuda")
             c_ = torch.empty((rows, n_), device="cuda")
-            capi.time_matmul(ws_, a_, rows, c_, 16, phase=0, stream=stream)
-            total += capi.time_matmul(ws_, a_, rows, c_, 80, phase=0, stream=stream)
+            total += capi.matmul_loop(ws_, a_, rows, c_, 80, stream=stream)
             for w_ in ws_:
                 w_.destroy()
         return total
@@ -354,6 +435,127 @@ def main():
     c5_graph_fused_ms = decode_layer_graph(2)
     c5_prefill_graph_ms, c5_prefill_grouped_ms = decode_layer_graph(0, 512), decode_layer_graph(1, 512)
     c5_rows8_grouped_ms = decode_layer_graph(1, 8)
+
+    def whole_model(rows, with_head):
+        """The FCs of all 28 decoder layers of configs[4] (Q, K, V as one call, the output projection,
+        gate and up as one call, the down projection: what the context's qkv_layer and grouped FCs make
+        of a layer) and, with_head, the model's lm_head as a Q4_0 FC on one row (the last one of a
+        prompt), captured into ONE graph per model copy; two copies of the model (2 x 248 MB of FC
+        weights) replayed in turn, so that a step does not find its weights in the last-level cache.
+        Milliseconds per step."""
+        shapes = [(2048, 1024), (1024, 1024), (1024, 1024), (1024, 2048), (3072, 1024), (3072, 1024), (1024, 3072)]
+        models = []
+        for _ in range(2):
+            layers = []
+            for _l in range(28):
+                ws_ = []
+                for n_, k_ in shapes:
+                    w32_ = torch.randn((n_, k_), generator=gen, device="cuda", dtype=torch.float32) * 0.02
+                    b_ = torch.empty(capi.weight_nbytes("q4_0", n_, k_), dtype=torch.uint8, device="cuda")
+                    capi.quantize_weights("q4_0", w32_, n_, k_, b_, stream=stream)
+                    torch.cuda.synchronize()
+                    ws_.append(capi.Weight("q4_0", n_, k_, b_, mem=capi.MEM_DEVICE))
+                layers.append(ws_)
+            head = None
+            if with_head:
+                w32_ = torch.randn((151936, 1024), generator=gen, device="cuda", dtype=torch.float32) * 0.02
+                b_ = torch.empty(capi.weight_nbytes("q4_0", 151936, 1024), dtype=torch.uint8, device="cuda")
+                capi.quantize_weights("q4_0", w32_, 151936, 1024, b_, stream=stream)
+                torch.cuda.synchronize()
+                head = capi.Weight("q4_0", 151936, 1024, b_, mem=capi.MEM_DEVICE)
+                del w32_, b_
+            models.append((layers, head))
+        xs_ = {k_: torch.randn((rows, k_), generator=gen, device="cuda") for k_ in (1024, 2048, 3072)}
+        cs_ = [torch.empty((rows, n_), device="cuda") for n_, _ in shapes]
+        logits_ = torch.empty((1, 151936), device="cuda")
+
+        def step(st, model):
+            layers, head = model
+            for ws_ in layers:
+                capi.matmul_multi(ws_[0:3], xs_[1024], rows, cs_[0:3], stream=st)
+                capi.matmul(ws_[3], xs_[2048], rows, cs_[3], stream=st)
+                capi.matmul_multi(ws_[4:6], xs_[1024], rows, cs_[4:6], stream=st)
+                capi.matmul(ws_[6], xs_[3072], rows, cs_[6], stream=st)
+            if head is not None:
+                capi.matmul(head, xs_[1024][rows - 1:rows], 1, logits_, stream=st)
+
+        side = torch.cuda.Stream()
+        side.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(side):
+            for model in models:
+                step(side.cuda_stream, model)
+        torch.cuda.current_stream().wait_stream(side)
+        torch.cuda.synchronize()
+        graphs = []
+        for model in models:
+            g_ = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g_, stream=side):
+                step(side.cuda_stream, model)
+            graphs.append(g_)
+        for _ in range(2):
+            for g_ in graphs:
+                g_.replay()
+        torch.cuda.synchronize()
+        e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        reps = 10
+        e0.record()
+        for _ in range(reps):
+            for g_ in graphs:
+                g_.replay()
+        e1.record()
+        torch.cuda.synchronize()
+        ms = e0.elapsed_time(e1) / (reps * len(graphs))
+        del graphs
+        for layers, head in models:
+            for ws_ in layers:
+                for w_ in ws_:
+                    w_.destroy()
+            if head is not None:
+                head.destroy()
+        return ms
+
+    c5_model_decode_ms, c5_model_decode_head_ms = whole_model(1, False), whole_model(1, True)
+    c5_model_prefill_ms = whole_model(512, True)
+
+    # ---- one decode row through host memory (what the Layer API hands over): microseconds per call,
+    # page-locked (memory of the context's allocator) and pageable, against the same call on device
+    # memory, for the shapes of C1, C3 and the largest FC of C5
+    def host_row_us(kind, n_, k_):
+        w32_ = torch.randn((n_, k_), generator=gen, device="cuda", dtype=torch.float32) * 0.02
+        b_ = torch.empty(capi.weight_nbytes(kind, n_, k_), dtype=torch.uint8, device="cuda")
+        capi.quantize_weights(kind, w32_, n_, k_, b_, stream=stream)
+        torch.cuda.synchronize()
+        del w32_
+        w_ = capi.Weight(kind, n_, k_, b_, mem=capi.MEM_DEVICE)
+        xr = np.random.default_rng(5).standard_normal((1, k_)).astype(np.float32)
+        yr = np.empty((1, n_), np.float32)
+        px, py = capi.host_alloc(k_ * 4), capi.host_alloc(n_ * 4)
+        np.ctypeslib.as_array(ctypes.cast(px, ctypes.POINTER(ctypes.c_float)), (1, k_))[:] = xr
+        dx_, dy_ = torch.from_numpy(xr).cuda(), torch.empty((1, n_), device="cuda")
+
+        def med(fn, reps=41):
+            ts = []
+            for _ in range(reps + 4):
+                t0 = time.perf_counter()
+                fn()
+                ts.append((time.perf_counter() - t0) * 1e6)
+            return sorted(ts[4:])[reps // 2]
+
+        def dev_call():
+            capi.matmul(w_, dx_, 1, dy_, stream=stream)
+            torch.cuda.synchronize()
+
+        out_ = {"page_locked": round(med(lambda: capi.matmul(w_, px, 1, py, mem=capi.MEM_HOST)), 2),
+                "pageable": round(med(lambda: capi.matmul(w_, xr, 1, yr, mem=capi.MEM_HOST)), 2),
+                "device_memory_call_and_synchronize": round(med(dev_call), 2)}
+        capi.host_free(px)
+        capi.host_free(py)
+        w_.destroy()
+        return out_
+
+    decode_row_us = {"c1_q4_0_4096x4096": host_row_us("q4_0", 4096, 4096),
+                     "c5_q4_0_3072x1024": host_row_us("q4_0", 3072, 1024),
+                     "c3_q6_K_151936x4096": host_row_us("q6_K", 151936, 4096)}
 
     def q4k_qkv_rows(rows, copies=6):
         """Q, K, V of a 4096-wide layer with grouped-query attention (4096, 1024, 1024 x 4096, Q4_K) against
@@ -492,9 +694,11 @@ def main():
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "int8",
         "data": "synthetic",
         "config": {"workload": "Q4_K x Q8_K prefill GEMM, M=512 K=4096 N=12288 (BASELINE configs[1]); "
-                               "step = activation quantizer + block-dot GEMM on HBM-resident inputs",
-                   "M": M, "K": K, "N": N, "weight_copies_rotated": n_copies},
-        "roofline": {"bound": "mfma", "kernel": "gemm_q4k_kernel<2, true>", "achieved": round(gemm_tops, 3),
+                               "step = activation quantizer + block-dot GEMM on HBM-resident inputs; inputs: the "
+                               "repository's bit-reproducible generator, stream 1 (weights N(0, 0.02), activations "
+                               "N(0, 1) behind them), the data of tests/test_gpu_configs.py::test_c2_q4_K_prefill_gemm",
+                   "M": M, "K": K, "N": N, "weight_copies_rotated": n_copies, "input_digest": input_digest},
+        "roofline": {"bound": "mfma", "kernel": gemm_kernel_name, "achieved": round(gemm_tops, 3),
                      "peak": INT8_PEAK_TOPS, "unit": "TOP/s", "frac": round(gemm_tops / INT8_PEAK_TOPS, 5),
                      "kernel_ms": round(gemm_ms, 5), "traffic": TRAFFIC_GEMM_C2,
                      "traffic_from": "profiles/gemm_q4k_prefill_m512_k4096_n12288.txt (counter runs; not live)",
@@ -507,16 +711,19 @@ def main():
                            "pageable_ms_per_step": round(pageable_ms, 4),
                            "pageable_tops": round(ops / (pageable_ms * 1e-3) / 1e12, 2),
                            "page_locked_ms_per_step": round(pinned_ms, 4),
-                           "page_locked_tops": round(ops / (pinned_ms * 1e-3) / 1e12, 2)},
-        "timing": {"method": "median of 5 blocks of `steps` hipq_matmul calls, two HIP events on the launch stream "
-                             "around each block (synchronize on both sides): ms_per_step; every block is followed "
-                             "by an instrumented block of the same calls whose launches carry their own start and "
-                             "stop events: roofline.kernel_ms and quantizer_ms are the kernels' own durations "
-                             "(median block), ms_per_step - kernel_ms - quantizer_ms the time between kernels",
+                           "page_locked_tops": round(ops / (pinned_ms * 1e-3) / 1e12, 2),
+                           "decode_row_us": decode_row_us},
+        "timing": {"method": "median of 5 blocks; a block is a C loop of `steps` calls of the public hipq_matmul "
+                             "(hipq_bench_matmul_loop in libhipq_bench.so, which links libhipq.so) with two HIP "
+                             "events on the launch stream around it (synchronize on both sides): ms_per_step; every "
+                             "block is followed by the same loop under hipq_launch_timing_begin / _end, where every "
+                             "launch carries its own start and stop event: roofline.kernel_ms and quantizer_ms are "
+                             "the kernels' own mean durations (median block), ms_per_step - kernel_ms - quantizer_ms "
+                             "the time between kernels",
                    "blocks_ms_per_step": [round(b[0], 5) for b in blocks_timed],
                    "blocks_wall_clock_ms_per_step": [round(b[1] * 1e3, 5) for b in blocks_timed],
-                   "instrumented_blocks_ms_per_step": [round(b[0], 5) for b in blocks_instr],
-                   "instrumented_blocks_kernel_ms": [round(b[2], 5) for b in blocks_instr],
+                   "kernel_timing_blocks_quantizer_plus_kernel_ms": [round(b[0], 5) for b in blocks_instr],
+                   "kernel_timing_blocks_kernel_ms": [round(b[2], 5) for b in blocks_instr],
                    "consistent": bool(gemm_ms + quant_ms <= step_ms)},
         "hbm_read_ceiling": {"value": round(read_ceiling_gbs, 1), "unit": "GB/s",
                              "method": "a kernel that only reads 1 GiB of device memory, four wavefronts a SIMD, each "
@@ -526,7 +733,8 @@ def main():
                         "value": round(gv_bytes / (gemv_all_ms * 1e-3) / 1e9, 2), "unit": "GB/s",
                         "ms_per_call": round(gemv_all_ms, 5),
                         "cache_hot_kernel_ms": round(gemv_hot_ms, 5),
-                        "roofline": {"bound": "hbm", "kernel": "gemv_kernel<Q4_K,T=64,R=1,G=4>",
+                        "kernels": {k_: [v_[0], round(v_[1], 5)] for k_, v_ in gemv_kern.items()},
+                        "roofline": {"bound": "hbm", "kernel": gemv_kernel_name,
                                      "achieved": round(gemv_gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                                      "frac": round(gemv_gbs / HBM_PEAK_GBS, 5),
                                      "frac_of_measured_read_ceiling": round(gemv_gbs / read_ceiling_gbs, 5),
@@ -547,9 +755,15 @@ def main():
             "note": "16 rows: two passes of the same kernel, still the reference's bits; 64 rows: the prefill GEMM "
                     "in parts of K (one 64-row tile per 128 columns), within 1e-4; qkv: three Q4_K weights of a layer "
                     "through hipq_matmul_multi, one quantization and one launch of the few-rows kernel for all three"},
+        "decode_gemv_size_sweep": {
+            "workload": "Q4_K GEMV M=1 K=4096 over N = 4096 .. 151936, weight copies of more than twice the last-level "
+                        "cache rotated; kernel_ms = the product kernel's own duration (one launch that quantizes the row "
+                        "itself below 32768 columns; from there the quantizer is a launch of its own, counted in "
+                        "ms_per_call only); frac = algorithmic bytes / kernel_ms / 8 TB/s",
+            "points": sweep},
         "decode_gemv_lm_head_size": {
-            "workload": "Q4_K GEMV M=1 K=4096 N=151936, 3 weight copies rotated",
-            "roofline": {"bound": "hbm", "kernel": "gemv_stream_kernel<Q4_K,G=4,GPW=2>",
+            "workload": "Q4_K GEMV M=1 K=4096 N=151936 (the last point of the sweep), %d weight copies rotated" % sweep[-1]["copies"],
+            "roofline": {"bound": "hbm", "kernel": big_kernel_name,
                          "achieved": round(big_gbs, 2), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                          "frac": round(big_gbs / HBM_PEAK_GBS, 5),
                          "frac_of_measured_read_ceiling": round(big_gbs / read_ceiling_gbs, 5),
@@ -573,7 +787,7 @@ def main():
             "workload": "Q6_K x Q8_K prefill GEMM, M=512 K=4096 N=151936 (the C3 weights against 512 rows), "
                         "2 weight copies rotated",
             "ms_per_call": round(c3_prefill[1], 5),
-            "roofline": {"bound": "mfma", "kernel": "gemm_q6k_kernel<4>",
+            "roofline": {"bound": "mfma", "kernel": c3_prefill[2],
                          "achieved": round(2.0 * 512 * 151936 * 4096 / (c3_prefill[0] * 1e-3) / 1e12, 3),
                          "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
                          "frac": round(2.0 * 512 * 151936 * 4096 / (c3_prefill[0] * 1e-3) / 1e12 / INT8_PEAK_TOPS, 5),
@@ -597,6 +811,25 @@ def main():
             "decode_1_row_in_a_graph_ms": round(c5_graph_ms, 5),
             "decode_1_row_in_a_graph_qkv_and_gate_up_as_one_launch_each_ms": round(c5_graph_grouped_ms, 5),
             "decode_1_row_in_a_graph_qkv_one_launch_up_gate_swiglu_one_launch_ms": round(c5_graph_fused_ms, 5)},
+        "c5_whole_model": {
+            "workload": "the FCs of all 28 layers of the Qwen3-0.6B-shaped decoder of BASELINE configs[4] (Q4_0; Q, K, V "
+                        "as one call, O, gate and up as one call, down), one graph per model copy, two copies replayed "
+                        "in turn (the FC weights of one are 248 MB, about the last-level cache); lm_head = the model's "
+                        "151936 x 1024 head as a Q4_0 FC on one row",
+            "decode_ms_per_token_fcs": round(c5_model_decode_ms, 5),
+            "decode_fc_gbs": round(247726080 / (c5_model_decode_ms * 1e-3) / 1e9, 1),
+            "decode_roofline": {"bound": "hbm", "achieved": round(247726080 / (c5_model_decode_ms * 1e-3) / 1e9, 1),
+                                "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                                "frac": round(247726080 / (c5_model_decode_ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 5),
+                                "algorithmic_bytes_per_token": 247726080, "launches_per_token": 112},
+            "decode_ms_per_token_fcs_and_lm_head": round(c5_model_decode_head_ms, 5),
+            "decode_fcs_and_lm_head_gbs": round((247726080 + 151936 * 1024 * 18 // 32) / (c5_model_decode_head_ms * 1e-3) / 1e9, 1),
+            "prefill_512_ms_fcs_and_lm_head": round(c5_model_prefill_ms, 5),
+            "prefill_roofline": {"bound": "mfma", "achieved": round(450971566080 / (c5_model_prefill_ms * 1e-3) / 1e12, 1),
+                                 "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                                 "frac": round(450971566080 / (c5_model_prefill_ms * 1e-3) / 1e12 / INT8_PEAK_TOPS, 5),
+                                 "algorithmic_ops": 450971566080,
+                                 "note": "the lm_head row's time is inside the figure, its ops are not"}},
         "moe_block": {
             "workload": "MoE FFN block (BASELINE configs[3]): 64 tokens, hidden 2048, 128 experts x "
                         "(gate/up 2048->768, down 768->2048) Q4_K, top-8; router, sort, experts, combine; "
@@ -617,6 +850,7 @@ def main():
         capi.matmul(weights[0], a, M, c, stream=stream)
         torch.cuda.synchronize()
         out["cpu_baseline"] = cpu_baseline(blocks.cpu().numpy(), a.cpu().numpy(), c.cpu().numpy())
+        out["cpu_baseline_thread_pool"] = cpu_baseline_thread_pool(blocks.cpu().numpy(), a.cpu().numpy())
         out["cpu_baseline_gemv"] = {
             "c1_q4_0_m1_k4096_n4096": cpu_gemv_baseline("q4_0", 4096, 4096, c1_host, c1_bytes),
             "c3_q6_K_m1_k4096_n151936": cpu_gemv_baseline("q6_K", 151936, 4096, c3_host, c3_bytes)}

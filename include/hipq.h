@@ -319,6 +319,18 @@ HIPQ_API int hipq_device_download(void *dst_host, const void *src_device, size_t
 HIPQ_API int hipq_host_alloc(void **ptr, size_t bytes);
 HIPQ_API int hipq_host_free(void *ptr);
 
+/** Kernel timing without an external tracer. Between _begin and _end every kernel that calls of
+ *  the SAME THREAD launch carries a start and a stop event of its own (attached to the dispatch:
+ *  no marker packets between the kernels), up to max_launches of them. _end waits for the timed
+ *  launches and returns how many there were (*count), and for the first `capacity` of them, in
+ *  launch order, the kernel's own duration in milliseconds and the kernel as its launch site in
+ *  this library's source names it (names may be NULL; the strings are literals of the library). What a kernel trace reports for the same launches. A launch
+ *  that carries events delays the one behind it by a few microseconds, so the time of a whole call
+ *  is taken without this switched on. No counterpart in the reference, whose profiler brackets
+ *  host calls (nntrainer/utils/profiler.h). */
+HIPQ_API int hipq_launch_timing_begin(int max_launches);
+HIPQ_API int hipq_launch_timing_end(int capacity, int *count, float *ms, const char **names);
+
 /** Frees the scratch the library keeps for a stream (it grows on demand with the calls made on
  *  the stream and is otherwise kept until hipq_shutdown) and gives back the stream's slot of the
  *  allocation-free entry point's array. Call it before destroying a stream

@@ -24,11 +24,12 @@ SYMBOLS = [
     "hipq_moe_forward_ext", "hipq_mlp_swiglu", "hipq_host_alloc", "hipq_host_free", "hipq_stream_release",
     "hipq_quantize_weights", "hipq_file_layout", "hipq_weights_from_file",
     "hipq_device_alloc", "hipq_device_free", "hipq_device_upload", "hipq_device_download",
+    "hipq_launch_timing_begin", "hipq_launch_timing_end",
 ]
-# measurement helpers of csrc/hipq_bench.h: exported for bench.py, not part of the product ABI
-BENCH_SYMBOLS = ["hipq_time_matmul", "hipq_bench_matmul_steps", "hipq_bench_mfma_ceiling",
-                 "hipq_bench_hbm_read_ceiling",
-                 "hipq_bench_tiled_bytes", "hipq_bench_quantize_tiled"]
+# measurement and test helpers of csrc/hipq_bench.h: a library of their own (libhipq_bench.so)
+# that links the product library; not part of the product
+BENCH_SYMBOLS = ["hipq_bench_matmul_loop", "hipq_bench_mfma_ceiling", "hipq_bench_hbm_read_ceiling",
+                 "hipq_bench_tiled_bytes", "hipq_bench_quantize_tiled", "hipq_bench_last_error"]
 
 
 class HipqError(RuntimeError):
@@ -106,15 +107,12 @@ def lib():
         L.hipq_host_alloc.argtypes = [C.POINTER(vp), C.c_size_t]
         L.hipq_host_free.argtypes = [vp]
         L.hipq_stream_release.argtypes = [vp]
-        L.hipq_time_matmul.argtypes = [i32, C.POINTER(vp), vp, i64, i64, vp, i64, i32, i32, vp,
-                                       C.POINTER(C.c_float)]
-        fp = C.POINTER(C.c_float)
-        L.hipq_bench_matmul_steps.argtypes = [i32, C.POINTER(vp), vp, i64, i64, vp, i64, i32, vp, fp, fp, fp]
-        L.hipq_bench_mfma_ceiling.argtypes = [C.c_float, vp, fp, fp]
-        L.hipq_bench_hbm_read_ceiling.argtypes = [i64, i32, i32, vp, fp]
-        L.hipq_bench_tiled_bytes.argtypes = [i64, i64]
-        L.hipq_bench_tiled_bytes.restype = i64
-        L.hipq_bench_quantize_tiled.argtypes = [vp, i64, i64, i64, vp, vp]
+        L.hipq_device_alloc.argtypes = [C.POINTER(vp), C.c_size_t]
+        L.hipq_device_free.argtypes = [vp]
+        L.hipq_device_upload.argtypes = [vp, vp, C.c_size_t, vp]
+        L.hipq_device_download.argtypes = [vp, vp, C.c_size_t, vp]
+        L.hipq_launch_timing_begin.argtypes = [i32]
+        L.hipq_launch_timing_end.argtypes = [i32, C.POINTER(i32), C.POINTER(C.c_float), C.POINTER(C.c_char_p)]
         _lib = L
     return _lib
 
@@ -305,29 +303,97 @@ def stream_release(stream=None):
     check(lib().hipq_stream_release(stream))
 
 
-def time_matmul(ws, a, m, c, iters, phase=0, stream=None):
-    """Average milliseconds per call, HIP events on `stream`, rotating over `ws`."""
+_bench = None
+
+
+def bench_lib():
+    """libhipq_bench.so: measurement and test helpers beside the product library."""
+    global _bench
+    if _bench is None:
+        lib()  # the helpers link the product library
+        path = os.path.join(os.path.dirname(LIB_PATH), "libhipq_bench.so")
+        if not os.path.exists(path):
+            raise FileNotFoundError("%s is missing: build it with `make -C %s`" % (path, CSRC))
+        B = C.CDLL(path)
+        vp, i64, i32, fp = C.c_void_p, C.c_int64, C.c_int, C.POINTER(C.c_float)
+        B.hipq_bench_last_error.restype = C.c_char_p
+        B.hipq_bench_matmul_loop.argtypes = [i32, C.POINTER(vp), vp, i64, i64, vp, i64, i32, vp, fp]
+        B.hipq_bench_mfma_ceiling.argtypes = [C.c_float, vp, fp, fp]
+        B.hipq_bench_hbm_read_ceiling.argtypes = [i64, i32, i32, vp, fp]
+        B.hipq_bench_tiled_bytes.argtypes = [i64, i64]
+        B.hipq_bench_tiled_bytes.restype = i64
+        B.hipq_bench_quantize_tiled.argtypes = [vp, i64, i64, i64, vp, vp]
+        _bench = B
+    return _bench
+
+
+def _bcheck(rc):
+    if rc != 0:
+        raise HipqError(rc, bench_lib().hipq_bench_last_error().decode())
+
+
+def matmul_loop(ws, a, m, c, iters, stream=None):
+    """Average milliseconds per call of `iters` hipq_matmul calls rotating over `ws`, two HIP events
+    on `stream` around the loop (after one untimed call per weight)."""
     n = len(ws)
     hs = (C.c_void_p * n)(*[w.handle.value for w in ws])
     ms = C.c_float()
-    check(lib().hipq_time_matmul(n, hs, _addr(a), m, ws[0].k, _addr(c), ws[0].n, iters, phase,
-                                 stream, C.byref(ms)))
+    _bcheck(bench_lib().hipq_bench_matmul_loop(n, hs, _addr(a), m, ws[0].k, _addr(c), ws[0].n, iters, stream,
+                                               C.byref(ms)))
     return ms.value
 
 
-def bench_matmul_steps(ws, a, m, c, steps, stream=None):
-    """(total, quantizer, product) milliseconds per step of `steps` whole matmuls, all three
-    from the same launches (events on `stream` between the kernels)."""
-    n = len(ws)
-    hs = (C.c_void_p * n)(*[w.handle.value for w in ws])
-    t, q, p = C.c_float(), C.c_float(), C.c_float()
-    check(lib().hipq_bench_matmul_steps(n, hs, _addr(a), m, ws[0].k, _addr(c), ws[0].n, steps, stream,
-                                        C.byref(t), C.byref(q), C.byref(p)))
-    return t.value / steps, q.value / steps, p.value / steps
+class LaunchTiming:
+    """with LaunchTiming(n) as t: ...calls...; afterwards t.launches = [(kernel name, ms), ...] in
+    launch order: the kernels' own durations (hipq_launch_timing_begin / _end)."""
+
+    def __init__(self, max_launches):
+        self.max = int(max_launches)
+        self.launches = []
+
+    def __enter__(self):
+        check(lib().hipq_launch_timing_begin(self.max))
+        return self
+
+    def __exit__(self, *exc):
+        n = C.c_int()
+        ms = (C.c_float * self.max)()
+        names = (C.c_char_p * self.max)()
+        rc = lib().hipq_launch_timing_end(self.max, C.byref(n), ms, names)
+        if exc[0] is None:
+            check(rc)
+        k = min(n.value, self.max)
+        self.launches = [((names[i] or b"").decode(), ms[i]) for i in range(k)]
+        return False
+
+    @staticmethod
+    def _demangle(names):
+        mangled = sorted({n for n in names if n.startswith("_Z")})
+        if not mangled:
+            return {}
+        try:
+            out = subprocess.run(["c++filt"] + mangled, capture_output=True, text=True, timeout=30).stdout.splitlines()
+            return dict(zip(mangled, out)) if len(out) == len(mangled) else {}
+        except (OSError, subprocess.SubprocessError):
+            return {}
+
+    def by_kernel(self):
+        """{short kernel name: (launches, mean ms)}; the short name drops arguments and namespaces."""
+        acc = {}
+        plain = self._demangle([n for n, _ in self.launches])
+        for name, ms in self.launches:
+            name = plain.get(name, name)
+            if name.endswith(" [clone .kd]"):
+                name = name[:-len(" [clone .kd]")]
+            short = name.split("(")[0].replace("(anonymous namespace)::", "").replace("void ", "").strip()
+            short = short.replace("hipq::", "")
+            cnt, tot = acc.get(short, (0, 0.0))
+            acc[short] = (cnt + 1, tot + ms)
+        return {k: (c, t / c) for k, (c, t) in acc.items()}
 
 
 def bench_tiled_bytes(m, k):
-    n = lib().hipq_bench_tiled_bytes(m, k)
+    n = bench_lib().hipq_bench_tiled_bytes(m, k)
     if n < 0:
         raise HipqError(int(n), "bad shape")
     return int(n)
@@ -335,19 +401,19 @@ def bench_tiled_bytes(m, k):
 
 def bench_quantize_tiled(a, m, k, out, lda=None, stream=None):
     """The tiled Q8_K form of device rows `a` into the device buffer `out` (bench_tiled_bytes)."""
-    check(lib().hipq_bench_quantize_tiled(_addr(a), m, k, lda if lda is not None else k, _addr(out), stream))
+    _bcheck(bench_lib().hipq_bench_quantize_tiled(_addr(a), m, k, lda if lda is not None else k, _addr(out), stream))
 
 
 def bench_hbm_read_ceiling(nbytes=1 << 30, waves_per_simd=4, regions=1, stream=None):
     """TB/s of a kernel that only reads `nbytes` of device memory (the GEMV kernels' access pattern);
     regions > 1: that many buffers, one per launch, back to back, each read cold."""
     tbs = C.c_float()
-    check(lib().hipq_bench_hbm_read_ceiling(nbytes, regions, waves_per_simd, stream, C.byref(tbs)))
+    _bcheck(bench_lib().hipq_bench_hbm_read_ceiling(nbytes, regions, waves_per_simd, stream, C.byref(tbs)))
     return tbs.value
 
 
 def bench_mfma_ceiling(target_ms=2.0, stream=None):
     """(TOP/s, GHz) of a kernel that issues nothing but the int8 matrix instruction."""
     tops, ghz = C.c_float(), C.c_float()
-    check(lib().hipq_bench_mfma_ceiling(target_ms, stream, C.byref(tops), C.byref(ghz)))
+    _bcheck(bench_lib().hipq_bench_mfma_ceiling(target_ms, stream, C.byref(tops), C.byref(ghz)))
     return tops.value, ghz.value

@@ -22,7 +22,6 @@
 #include <unordered_map>
 #include <vector>
 
-#include "hipq_bench.h"
 #include "hipq_internal.h"
 
 /* Scratch of hipq_matmul_noalloc: quantized activations (and partial products) of one call.
@@ -83,7 +82,7 @@ State g;
 } // namespace
 
 namespace hipq {
-thread_local const LaunchTimer *launch_timer = nullptr;
+thread_local LaunchLog launch_log;
 
 int fail(int code, const char *fmt, ...) {
   va_list ap;
@@ -1235,157 +1234,47 @@ int hipq_matmul_multi(int count, const hipq_weight_t *w, const float *A, int64_t
   return HIPQ_OK;
 }
 
-int hipq_time_matmul(int n_weights, const hipq_weight_t *w, const float *A, int64_t M, int64_t lda,
-                     float *C, int64_t ldc, int iters, int phase, void *stream,
-                     float *ms_per_call) {
+/* ---- kernel timing ------------------------------------------------------------ */
+
+int hipq_launch_timing_begin(int max_launches) {
   int rc = require_ready();
   if (rc) return rc;
-  if (n_weights <= 0 || !w || iters <= 0 || !ms_per_call || phase < 0 || phase > 2)
-    return fail(HIPQ_ERR_INVALID_ARGUMENT, "bad timing arguments");
-  for (int i = 0; i < n_weights; ++i) {
-    if ((rc = check_matmul_args(w[i], A, M, lda, C, ldc))) return rc;
-    if (w[i]->K != w[0]->K || w[i]->dtype != w[0]->dtype)
-      return fail(HIPQ_ERR_INVALID_ARGUMENT, "timed weights must share dtype and K");
+  if (max_launches <= 0 || max_launches > (1 << 20)) return fail(HIPQ_ERR_INVALID_ARGUMENT, "max_launches = %d", max_launches);
+  hipq::LaunchLog &lg = hipq::launch_log;
+  if (lg.on) return fail(HIPQ_ERR_INVALID_ARGUMENT, "kernel timing is already on for this thread");
+  while (lg.ev.size() < (size_t)2 * max_launches) {
+    hipEvent_t e;
+    HIPQ_HIP(hipEventCreate(&e));
+    lg.ev.push_back(e);
   }
-  hipStream_t s = (hipStream_t)stream;
-  EnqueueGuard eg(enqueue_lock(s));
-  CallScope call(s);
-  const int is_k = w[0]->dtype != HIPQ_Q4_0;
-  bool tiled = true, rows = true;
-  for (int i = 0; i < n_weights; ++i) {
-    tiled = tiled && wants_tiled(w[i], M);
-    rows = rows && wants_rows(w[i], M, true);
+  lg.fn.assign((size_t)max_launches, nullptr);
+  /* events beyond this call's limit stay in the pool but are not used */
+  while (lg.ev.size() > (size_t)2 * max_launches) {
+    (void)hipEventDestroy(lg.ev.back());
+    lg.ev.pop_back();
   }
-  void *memp = nullptr;
-  QAct qa{};
-  if (tiled) {
-    /* the loop multiplies every weight with the rows quantized here: reserve for the largest first */
-    size_t need = 0;
-    for (int i = 0; i < n_weights; ++i) {
-      if (!w[i]->gt_base && (rc = hipq::ensure_gemm_tiles(const_cast<hipq_weight *>(w[i])))) return rc;
-      const size_t parts = w[i]->dtype == HIPQ_Q4_K ? hipq::gemm_q4k_split_bytes(w[i], M) : hipq::gemm_q6k_split_bytes(w[i], M);
-      const size_t n = ((qact_tiled_bytes(M, w[i]->K) + 255) & ~(size_t)255) + parts;
-      if (n > need) need = n;
-    }
-    if ((rc = workspace(s, need, &memp))) return rc;
-    if ((rc = matmul_tiled(w[0], A, M, lda, C, ldc, s, 2, Scratch{false, s}))) return rc;
-  } else if (rows) {
-    for (int i = 0; i < n_weights; ++i) /* the tile copies are built outside the timed loop */
-      if (!w[i]->gt_base && (rc = hipq::ensure_gemm_tiles(const_cast<hipq_weight *>(w[i])))) return rc;
-    if ((rc = matmul_rows(w[0], A, M, lda, C, ldc, s, 2, Scratch{false, s}))) return rc;
-  } else {
-    if ((rc = workspace(s, qact_bytes(is_k, M, w[0]->K), &memp))) return rc;
-    qa = qact_carve(is_k, memp, M, w[0]->K);
-    if ((rc = quantize_for(w[0], A, M, lda, qa, s))) return rc;
-  }
-  const uint64_t gen = workspace_generation(s);
-  hipEvent_t e0, e1;
-  HIPQ_HIP(hipEventCreate(&e0));
-  HIPQ_HIP(hipEventCreate(&e1));
-  HIPQ_HIP(hipStreamSynchronize(s));
-  HIPQ_HIP(hipEventRecord(e0, s));
-  for (int it = 0; it < iters && !rc; ++it) {
-    const hipq_weight *wi = w[it % n_weights];
-    if (phase == 1 && (rc = workspace_unmoved(s, gen))) break;
-    if (tiled) {
-      rc = matmul_tiled(wi, A, M, lda, C, ldc, s, phase, Scratch{false, s});
-      continue;
-    }
-    if (rows) {
-      rc = matmul_rows(wi, A, M, lda, C, ldc, s, phase, Scratch{false, s});
-      continue;
-    }
-    if (phase == 0 && hipq::gemm_rows_q40_fuses(1, &wi, M, A, lda)) {
-      float *cc = C;
-      rc = hipq::launch_gemm_rows_q40_fused(1, &wi, A, lda, (int)M, &cc, &ldc, s);
-      continue;
-    }
-    if (phase == 0 && M == 1 && hipq::gemv_fuses_quantizer(wi, A)) {
-      rc = hipq::launch_gemv_fused(wi, A, C, s);
-      continue;
-    }
-    if (phase == 0 || phase == 2) rc = quantize_for(wi, A, M, lda, qa, s);
-    if (!rc && (phase == 0 || phase == 1)) rc = multiply(wi, qa, M, C, ldc, s);
-  }
-  hipError_t er = hipEventRecord(e1, s);
-  if (er == hipSuccess) er = hipEventSynchronize(e1);
-  float ms = 0.f;
-  if (er == hipSuccess) er = hipEventElapsedTime(&ms, e0, e1);
-  (void)hipEventDestroy(e0);
-  (void)hipEventDestroy(e1);
-  if (rc) return rc;
-  if (er != hipSuccess) return fail(HIPQ_ERR_RUNTIME, "timing: %s", hipGetErrorString(er));
-  *ms_per_call = ms / (float)iters;
+  lg.count = 0;
+  lg.dropped = 0;
+  lg.on = true;
   return HIPQ_OK;
 }
 
-int hipq_bench_matmul_steps(int n_weights, const hipq_weight_t *w, const float *A, int64_t M, int64_t lda,
-                            float *C, int64_t ldc, int steps, void *stream, float *total_ms,
-                            float *quantizer_ms, float *product_ms) {
-  int rc = require_ready();
-  if (rc) return rc;
-  if (n_weights <= 0 || !w || steps <= 0 || steps > 100000 || !total_ms || !quantizer_ms || !product_ms)
-    return fail(HIPQ_ERR_INVALID_ARGUMENT, "bad timing arguments");
-  for (int i = 0; i < n_weights; ++i) {
-    if ((rc = check_matmul_args(w[i], A, M, lda, C, ldc))) return rc;
-    if (!wants_tiled(w[i], M))
-      return fail(HIPQ_ERR_NOT_SUPPORTED, "the step timer covers the tiled Q4_K prefill product");
+int hipq_launch_timing_end(int capacity, int *count, float *ms, const char **names) {
+  hipq::LaunchLog &lg = hipq::launch_log;
+  if (!lg.on) return fail(HIPQ_ERR_INVALID_ARGUMENT, "kernel timing is not on for this thread");
+  lg.on = false;
+  if (!count || capacity < 0 || (capacity && !ms)) return fail(HIPQ_ERR_INVALID_ARGUMENT, "bad argument");
+  *count = lg.count;
+  const int n = lg.count < capacity ? lg.count : capacity;
+  for (int i = 0; i < n; ++i) {
+    HIPQ_HIP(hipEventSynchronize(lg.ev[2 * i + 1]));
+    HIPQ_HIP(hipEventElapsedTime(&ms[i], lg.ev[2 * i], lg.ev[2 * i + 1]));
+    if (names) names[i] = lg.fn[i] ? lg.fn[i] : "";
   }
-  hipStream_t s = (hipStream_t)stream;
-  EnqueueGuard eg(enqueue_lock(s));
-  CallScope call(s);
-  const Scratch sc{false, s};
-  /* one untimed call first: workspace and tile copies exist before the events */
-  for (int i = 0; i < n_weights; ++i)
-    if ((rc = matmul_tiled(w[i], A, M, lda, C, ldc, s, 0, sc))) return rc;
-  /* Two events before and behind the block give the steps' total; every launch carries a
-   * start and a stop event of its own (hipq_internal.h, LaunchTimer), which hold the kernel's
-   * own time without putting marker packets between the kernels. */
-  std::vector<hipEvent_t> ev((size_t)4 * steps + 2);
-  for (auto &e : ev) HIPQ_HIP(hipEventCreate(&e));
-  HIPQ_HIP(hipStreamSynchronize(s));
-  hipError_t er = hipEventRecord(ev[4 * steps], s);
-  for (int it = 0; it < steps && !rc && er == hipSuccess; ++it) {
-    const hipq_weight *wi = w[it % n_weights];
-    const hipq::LaunchTimer tq{ev[4 * it], ev[4 * it + 1]}, tp{ev[4 * it + 2], ev[4 * it + 3]};
-    hipq::launch_timer = &tq;
-    rc = matmul_tiled(wi, A, M, lda, C, ldc, s, 2, sc);
-    hipq::launch_timer = &tp;
-    if (!rc) rc = matmul_tiled(wi, A, M, lda, C, ldc, s, 1, sc);
-    hipq::launch_timer = nullptr;
-  }
-  if (er == hipSuccess) er = hipEventRecord(ev[4 * steps + 1], s);
-  if (er == hipSuccess) er = hipEventSynchronize(ev[4 * steps + 1]);
-  double q = 0.0, p = 0.0;
-  float total = 0.f;
-  for (int it = 0; it < steps && !rc && er == hipSuccess; ++it) {
-    float a = 0.f, b = 0.f;
-    er = hipEventElapsedTime(&a, ev[4 * it], ev[4 * it + 1]);
-    if (er == hipSuccess) er = hipEventElapsedTime(&b, ev[4 * it + 2], ev[4 * it + 3]);
-    q += a;
-    p += b;
-  }
-  if (!rc && er == hipSuccess) er = hipEventElapsedTime(&total, ev[4 * steps], ev[4 * steps + 1]);
-  for (auto &e : ev) (void)hipEventDestroy(e);
-  if (rc) return rc;
-  if (er != hipSuccess) return fail(HIPQ_ERR_RUNTIME, "timing: %s", hipGetErrorString(er));
-  *total_ms = total;
-  *quantizer_ms = (float)q;
-  *product_ms = (float)p;
+  if (lg.dropped)
+    return fail(HIPQ_ERR_NOT_SUPPORTED, "%d launches beyond the %d the timing was opened for were not timed", lg.dropped,
+                (int)lg.fn.size());
   return HIPQ_OK;
-}
-
-int64_t hipq_bench_tiled_bytes(int64_t M, int64_t K) {
-  if (M <= 0 || K <= 0 || K % 256) return HIPQ_ERR_INVALID_ARGUMENT;
-  return (int64_t)qact_tiled_bytes(M, K);
-}
-
-int hipq_bench_quantize_tiled(const float *A, int64_t M, int64_t K, int64_t lda, void *out, void *stream) {
-  int rc = require_ready();
-  if (rc) return rc;
-  if (!A || !out || M <= 0 || K <= 0) return fail(HIPQ_ERR_INVALID_ARGUMENT, "bad argument");
-  const QActTiled qa = qact_tiled_carve(out, M, K);
-  return hipq::launch_quantize_q8_K_tiled(A, M, K, lda, (M / 4) * 4, &qa, (hipStream_t)stream);
 }
 
 /* ---- mixture of experts ---------------------------------------------------- */

@@ -381,7 +381,7 @@ int launch_gemm_multi(int count, const hipq_weight *const *w, const QAct *qa, in
     mw.tile_end[i] = tiles; /* unused entries repeat the total: no workgroup lands in them */
   }
   const dim3 grid((unsigned)tiles, (unsigned)((M + BM - 1) / BM));
-  hipLaunchKernelGGL(gemm_q40_kernel, grid, dim3(NT), 0, s, mw, qview(*qa), M);
+  hipq::launch_kernel("gemm_q40_kernel", gemm_q40_kernel, grid, dim3(NT), 0, s, mw, qview(*qa), M);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
 }

@@ -409,10 +409,10 @@ int launch_tiles(const hipq_weight *w, const QActTiled *qa, int M, float *C, int
   if (w->gt_base) { /* the tile copy, where the weight has one */
     v.qs = w->gt_qs;
     v.hdr = w->gt_hdr;
-    launch_kernel(gemm_q4k_kernel<TM, true>, dim3(grid), dim3(NT), sizeof(Smem<TM>), s, v, (const int8_t *)qa->qt,
+    hipq::launch_kernel(TM == 2 ? "gemm_q4k_kernel<2, true>" : "gemm_q4k_kernel<4, true>", gemm_q4k_kernel<TM, true>, dim3(grid), dim3(NT), sizeof(Smem<TM>), s, v, (const int8_t *)qa->qt,
                   (const uint16_t *)qa->amin, (const float *)qa->dAt, M, mtiles, ntiles, C, ldc);
   } else
-    launch_kernel(gemm_q4k_kernel<TM, false>, dim3(grid), dim3(NT), sizeof(Smem<TM>), s, v, (const int8_t *)qa->qt,
+    hipq::launch_kernel(TM == 2 ? "gemm_q4k_kernel<2, false>" : "gemm_q4k_kernel<4, false>", gemm_q4k_kernel<TM, false>, dim3(grid), dim3(NT), sizeof(Smem<TM>), s, v, (const int8_t *)qa->qt,
                   (const uint16_t *)qa->amin, (const float *)qa->dAt, M, mtiles, ntiles, C, ldc);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
@@ -444,11 +444,11 @@ int launch_gemm_q4k_multi(int count, const hipq_weight *const *w, const QActTile
   const int ngroups = (tiles + 7) / 8;
   if (rounds128 * 6 < rounds64 * 5) {
     const int mtiles = (M + 127) / 128;
-    hipLaunchKernelGGL(gemm_q4k_multi_kernel<4>, dim3((unsigned)(mtiles * ngroups * 8)), dim3(NT), sizeof(Smem<4>), s, mw,
+    hipq::launch_kernel("gemm_q4k_multi_kernel<4>", gemm_q4k_multi_kernel<4>, dim3((unsigned)(mtiles * ngroups * 8)), dim3(NT), sizeof(Smem<4>), s, mw,
                        (const int8_t *)qa->qt, (const uint16_t *)qa->amin, (const float *)qa->dAt, M, mtiles);
   } else {
     const int mtiles = (M + 63) / 64;
-    hipLaunchKernelGGL(gemm_q4k_multi_kernel<2>, dim3((unsigned)(mtiles * ngroups * 8)), dim3(NT), sizeof(Smem<2>), s, mw,
+    hipq::launch_kernel("gemm_q4k_multi_kernel<2>", gemm_q4k_multi_kernel<2>, dim3((unsigned)(mtiles * ngroups * 8)), dim3(NT), sizeof(Smem<2>), s, mw,
                        (const int8_t *)qa->qt, (const uint16_t *)qa->amin, (const float *)qa->dAt, M, mtiles);
   }
   HIPQ_HIP(hipGetLastError());
@@ -484,12 +484,12 @@ int launch_gemm_q4k(const hipq_weight *w, const QActTiled *qa, int M, float *C, 
     WView v = wview(w);
     v.qs = w->gt_qs;
     v.hdr = w->gt_hdr;
-    launch_kernel(gemm_q4k_split_kernel, dim3((unsigned)(mtiles * ngroups * 8), (unsigned)((nsb + per - 1) / per)),
+    hipq::launch_kernel("gemm_q4k_split_kernel", gemm_q4k_split_kernel, dim3((unsigned)(mtiles * ngroups * 8), (unsigned)((nsb + per - 1) / per)),
                   dim3(NT), sizeof(Smem<2>), s, v, (const int8_t *)qa->qt, (const uint16_t *)qa->amin,
                   (const float *)qa->dAt, M, mtiles, ntiles, per, (float *)partials, stride);
     HIPQ_HIP(hipGetLastError());
     const int64_t quads = stride / 4;
-    hipLaunchKernelGGL(split_sum_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s,
+    hipq::launch_kernel("split_sum_kernel", split_sum_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s,
                        (const float *)partials, (nsb + per - 1) / per, stride, M, (int)w->N, C, ldc);
     HIPQ_HIP(hipGetLastError());
     return HIPQ_OK;

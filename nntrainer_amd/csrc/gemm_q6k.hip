@@ -338,7 +338,7 @@ static int launch_tiles6(const hipq_weight *w, const QActTiled *qa, int M, float
   v.qs = w->gt_qs;
   v.qh = w->gt_qh;
   v.hdr = w->gt_hdr;
-  launch_kernel(gemm_q6k_kernel<TM>, dim3(grid), dim3(NT), sizeof(Smem6<TM>), s, v, (const int8_t *)qa->qt,
+  hipq::launch_kernel(TM == 2 ? "gemm_q6k_kernel<2>" : "gemm_q6k_kernel<4>", gemm_q6k_kernel<TM>, dim3(grid), dim3(NT), sizeof(Smem6<TM>), s, v, (const int8_t *)qa->qt,
                 (const float *)qa->dAt, M, mtiles, ntiles, C, ldc);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
@@ -373,11 +373,11 @@ int launch_gemm_q6k(const hipq_weight *w, const QActTiled *qa, int M, float *C, 
     v.qs = w->gt_qs;
     v.qh = w->gt_qh;
     v.hdr = w->gt_hdr;
-    launch_kernel(gemm_q6k_split_kernel, dim3((unsigned)(mtiles * ngroups * 8), (unsigned)((nsb + per - 1) / per)),
+    hipq::launch_kernel("gemm_q6k_split_kernel", gemm_q6k_split_kernel, dim3((unsigned)(mtiles * ngroups * 8), (unsigned)((nsb + per - 1) / per)),
                   dim3(NT), sizeof(Smem6<2>), s, v, (const int8_t *)qa->qt, (const float *)qa->dAt, M, mtiles, ntiles,
                   per, (float *)partials, stride);
     HIPQ_HIP(hipGetLastError());
-    hipLaunchKernelGGL(split_sum6_kernel, dim3((unsigned)((stride / 4 + 255) / 256)), dim3(256), 0, s,
+    hipq::launch_kernel("split_sum6_kernel", split_sum6_kernel, dim3((unsigned)((stride / 4 + 255) / 256)), dim3(256), 0, s,
                        (const float *)partials, (nsb + per - 1) / per, stride, M, (int)w->N, C, ldc);
     HIPQ_HIP(hipGetLastError());
     return HIPQ_OK;

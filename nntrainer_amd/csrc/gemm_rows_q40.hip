@@ -379,12 +379,12 @@ static int launch_rows_q40(int count, const hipq_weight *const *w, const QAct *q
   }
   const dim3 grid((unsigned)tiles, (unsigned)((M + TC - 1) / TC));
   if (qa) {
-    hipLaunchKernelGGL(gemm_rows_q40_kernel<false>, grid, dim3(NT), LDS_BYTES, s, mw, qview(*qa), (const float *)nullptr,
+    hipq::launch_kernel("gemm_rows_q40_kernel<false>", gemm_rows_q40_kernel<false>, grid, dim3(NT), LDS_BYTES, s, mw, qview(*qa), (const float *)nullptr,
                        (int64_t)0, M);
   } else {
     QView none{};
     none.K = (int)w[0]->K;
-    hipLaunchKernelGGL(gemm_rows_q40_kernel<true>, grid, dim3(NT), LDS_BYTES, s, mw, none, A, lda, M);
+    hipq::launch_kernel("gemm_rows_q40_kernel<true>", gemm_rows_q40_kernel<true>, grid, dim3(NT), LDS_BYTES, s, mw, none, A, lda, M);
   }
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;

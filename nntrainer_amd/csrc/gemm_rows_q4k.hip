@@ -368,7 +368,7 @@ int launch_gemm_rows_q4k_multi(int count, const hipq_weight *const *w, const QAc
     mw.ldc[i] = ldc[j];
     mw.tile_end[i] = tiles; /* unused entries repeat the total: no workgroup lands in them */
   }
-  hipLaunchKernelGGL(gemm_rows_q4k_kernel, dim3((unsigned)tiles, (unsigned)((M + TC - 1) / TC)), dim3(NT), LDS_BYTES, s, mw,
+  hipq::launch_kernel("gemm_rows_q4k_kernel", gemm_rows_q4k_kernel, dim3((unsigned)tiles, (unsigned)((M + TC - 1) / TC)), dim3(NT), LDS_BYTES, s, mw,
                      qview(*qa), M, pair_rows);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;

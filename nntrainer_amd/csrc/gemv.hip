@@ -233,7 +233,7 @@ int launch_fused_many(int count, const hipq_weight *const *w, const float *x, fl
     mw.end[i] = blocks;
   }
   const size_t lds = fused_act_bytes<DT>((int)w[0]->K) + 4 * GemvLds<DT, 1, G, false>::DWORDS * sizeof(uint32_t);
-  hipLaunchKernelGGL((gemv_fused_multi_kernel<DT, T, G>), dim3((unsigned)blocks), dim3(256), lds, s, mw, x);
+  hipq::launch_kernel("gemv_fused_multi_kernel<DT, T, G>", (gemv_fused_multi_kernel<DT, T, G>), dim3((unsigned)blocks), dim3(256), lds, s, mw, x);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
 }
@@ -242,7 +242,7 @@ template <int DT, int T, int G>
 int launch_fused_one(const hipq_weight *w, const float *x, float *C, hipStream_t s) {
   const unsigned grid = (unsigned)((w->N + 4 * G - 1) / (4 * G));
   const size_t lds = fused_act_bytes<DT>((int)w->K) + 4 * GemvLds<DT, 1, G, false>::DWORDS * sizeof(uint32_t);
-  hipLaunchKernelGGL((gemv_fused_kernel<DT, T, G>), dim3(grid), dim3(256), lds, s, wview(w), x, C);
+  hipq::launch_kernel("gemv_fused_kernel<DT, T, G>", (gemv_fused_kernel<DT, T, G>), dim3(grid), dim3(256), lds, s, wview(w), x, C);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
 }
@@ -252,7 +252,7 @@ int launch_stream(const hipq_weight *w, const QAct *qa, float *C, hipStream_t s)
   const int rows_per_block = 4 * G * GPW;
   const unsigned grid = (unsigned)((w->N + rows_per_block - 1) / rows_per_block);
   const size_t lds = 4 * GemvLds<DT, 1, G, false>::DWORDS * sizeof(uint32_t);
-  hipLaunchKernelGGL((gemv_stream_kernel<DT, T, G, GPW>), dim3(grid), dim3(256), lds, s, wview(w),
+  hipq::launch_kernel("gemv_stream_kernel<DT, T, G, GPW>", (gemv_stream_kernel<DT, T, G, GPW>), dim3(grid), dim3(256), lds, s, wview(w),
                      qview(*qa), C);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
@@ -263,7 +263,7 @@ int launch_one(const hipq_weight *w, const QAct *qa, int M, int pair_rows, float
                hipStream_t s) {
   const unsigned grid = (unsigned)((w->N + 4 * G - 1) / (4 * G));
   const size_t lds = 4 * GemvLds<DT, R, G, PW>::DWORDS * sizeof(uint32_t);
-  hipLaunchKernelGGL((gemv_kernel<DT, T, R, G, PW>), dim3(grid), dim3(256), lds, s, wview(w),
+  hipq::launch_kernel("gemv_kernel<DT, T, R, G, PW>", (gemv_kernel<DT, T, R, G, PW>), dim3(grid), dim3(256), lds, s, wview(w),
                      qview(*qa), M, pair_rows, C, ldc);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
@@ -282,7 +282,7 @@ int launch_fused_swiglu_one(const hipq_weight *wa, const hipq_weight *wm, const 
                             hipStream_t s) {
   const unsigned grid = (unsigned)((wa->N + 4 * G - 1) / (4 * G));
   const size_t lds = fused_act_bytes<DT>((int)wa->K) + 4 * GemvLds<DT, 1, G, false>::DWORDS * sizeof(uint32_t);
-  hipLaunchKernelGGL((gemv_fused_swiglu_kernel<DT, T, G>), dim3(grid), dim3(256), lds, s, wview(wa), wview(wm), x,
+  hipq::launch_kernel("gemv_fused_swiglu_kernel<DT, T, G>", (gemv_fused_swiglu_kernel<DT, T, G>), dim3(grid), dim3(256), lds, s, wview(wa), wview(wm), x,
                      out);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
@@ -467,7 +467,7 @@ __global__ __launch_bounds__(256) void swiglu_rows_kernel(const float *__restric
 
 int launch_swiglu_rows(const float *y, const float *z, int64_t M, int64_t N, float *out, int64_t ldo, hipStream_t s) {
   const int64_t n = M * N;
-  hipLaunchKernelGGL(swiglu_rows_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, y, z, n, N, ldo, out);
+  hipq::launch_kernel("swiglu_rows_kernel", swiglu_rows_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, s, y, z, n, N, ldo, out);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
 }

@@ -1,11 +1,11 @@
 /* SPDX-License-Identifier: Apache-2.0 */
 /**
  * @file   hipq_bench.h
- * @brief  Measurement and test helpers exported by libhipq.so for bench.py and the GPU
- *         tests only. They are not part of the product's C ABI (include/hipq.h) and
- *         replace nothing in the reference: event-timed launch loops, a matrix-core
- *         and a memory-read ceiling kernel, and a view of an internal buffer layout for
- *         its parity test.
+ * @brief  Measurement and test helpers of libhipq_bench.so, a library of its own beside
+ *         libhipq.so, for bench.py and the GPU tests only. They are not part of the
+ *         product's C ABI (include/hipq.h) and replace nothing in the reference: an
+ *         event-timed loop of hipq_matmul calls, a matrix-core and a memory-read ceiling
+ *         kernel, and a view of an internal buffer layout for its parity test.
  */
 #ifndef HIPQ_BENCH_H
 #define HIPQ_BENCH_H
@@ -16,26 +16,16 @@
 extern "C" {
 #endif
 
-/** Runs the matmul `iters` times on device buffers, rotating over `n_weights` handles
- *  (distinct copies defeat the last-level cache), brackets the launches with HIP events
- *  recorded on `stream` and returns the average milliseconds per call.
- *  phase 0: whole call (activation quantizer + block-dot kernel);
- *  phase 1: block-dot kernel only, on activations quantized once beforehand;
- *  phase 2: activation quantizer only. */
-HIPQ_API int hipq_time_matmul(int n_weights, const hipq_weight_t *w, const float *A, int64_t M,
-                              int64_t lda, float *C, int64_t ldc, int iters, int phase, void *stream,
-                              float *ms_per_call);
-
-/** `steps` whole matmuls (activation quantizer, then block-dot kernel) as hipq_matmul
- *  enqueues them on `stream`. total_ms: between one event recorded before the first
- *  quantizer and one behind the last product (nothing else is put into the stream, so the
- *  kernels follow each other as they do in a caller's loop). quantizer_ms, product_ms: sums
- *  of the kernels' own durations, taken from a start and a stop event attached to each of
- *  the same launches (hipExtLaunchKernelGGL): what a kernel trace reports for them.
- *  total >= quantizer + product; the difference is the time between the kernels. */
-HIPQ_API int hipq_bench_matmul_steps(int n_weights, const hipq_weight_t *w, const float *A, int64_t M,
-                                     int64_t lda, float *C, int64_t ldc, int steps, void *stream,
-                                     float *total_ms, float *quantizer_ms, float *product_ms);
+/** `iters` calls of hipq_matmul on device buffers, rotating over `n_weights` handles (distinct
+ *  copies defeat the last-level cache), after one untimed call per weight; two HIP events recorded
+ *  on `stream` before the first and behind the last call; returns the average milliseconds per
+ *  call. Nothing else is put into the stream, so the kernels follow each other as they do in a
+ *  caller's loop. The kernels' own durations come from hipq_launch_timing_begin / _end
+ *  (include/hipq.h) around such a loop. */
+HIPQ_API int hipq_bench_matmul_loop(int n_weights, const hipq_weight_t *w, const float *A, int64_t M,
+                                    int64_t lda, float *C, int64_t ldc, int iters, void *stream,
+                                    float *ms_per_call);
+HIPQ_API const char *hipq_bench_last_error(void);
 
 /** Nothing but v_mfma_i32_32x32x32_i8 on every SIMD of the device (three wavefronts each,
  *  four independent accumulators) for about `target_ms`: the int8 rate the matrix cores

@@ -11,6 +11,7 @@
 
 #include <hip/hip_fp16.h>
 #include <hip/hip_runtime.h>
+#include <vector>
 #include <hip/hip_ext.h>
 #include <stdint.h>
 
@@ -151,21 +152,29 @@ namespace hipq {
 /* error plumbing (api.hip) */
 int fail(int code, const char *fmt, ...);
 
-/* Measurement hook of the prefill product's two launches (hipq_bench.h): while a thread has
- * set launch_timer, a launch made through launch_kernel attaches the two events to the
- * dispatch itself, which then hold the kernel's own start and end (no marker packets in the
- * stream between the kernels). Null outside the bench helper. */
-struct LaunchTimer {
-  hipEvent_t start, stop;
+/* Kernel timing (hipq_launch_timing_begin / _end of include/hipq.h): while the calling thread
+ * has it switched on, every launch made through launch_kernel attaches a start and a stop event of
+ * its own to the dispatch, which then hold the kernel's own start and end (no marker packets in
+ * the stream between the kernels), and notes which kernel it was. Off otherwise: one thread-local
+ * load per launch. */
+struct LaunchLog {
+  bool on = false;
+  int count = 0, dropped = 0;
+  std::vector<hipEvent_t> ev;     /* 2 per launch: start, stop */
+  std::vector<const char *> fn;   /* the kernel as its launch site names it (a string literal) */
 };
-extern thread_local const LaunchTimer *launch_timer;
+extern thread_local LaunchLog launch_log;
 template <typename... KArgs, typename... Args>
-inline void launch_kernel(void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t lds, hipStream_t s, Args... args) {
-  const LaunchTimer *t = launch_timer;
-  if (t)
-    hipExtLaunchKernelGGL(kernel, grid, block, lds, s, t->start, t->stop, 0, args...);
-  else
-    hipLaunchKernelGGL(kernel, grid, block, lds, s, args...);
+inline void launch_kernel(const char *name, void (*kernel)(KArgs...), dim3 grid, dim3 block, size_t lds, hipStream_t s,
+                          Args... args) {
+  LaunchLog &lg = launch_log;
+  if (lg.on && (size_t)(2 * lg.count + 1) < lg.ev.size()) {
+    hipExtLaunchKernelGGL(kernel, grid, block, lds, s, lg.ev[2 * lg.count], lg.ev[2 * lg.count + 1], 0, args...);
+    lg.fn[lg.count++] = name;
+    return;
+  }
+  if (lg.on) ++lg.dropped;
+  hipLaunchKernelGGL(kernel, grid, block, lds, s, args...);
 }
 #define HIPQ_HIP(call)                                                        \
   do {                                                                        \

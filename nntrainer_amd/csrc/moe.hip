@@ -984,12 +984,12 @@ void launch_gate_up(const hipq_moe_desc &d, const hipq::MoeEpi &ep, const WView 
   if (d.hidden > KC) {
     const dim3 grid((d.intermediate + 7) / 8, d.experts);
     const size_t lds_long = 4 * GemvLds<DT, RTOK, 2, false>::DWORDS * sizeof(uint32_t);
-    hipLaunchKernelGGL((gate_up_long_kernel<DT>), grid, dim3(256), lds_long, s, views, d.experts,
+    hipq::launch_kernel("gate_up_long_kernel<DT>", (gate_up_long_kernel<DT>), grid, dim3(256), lds_long, s, views, d.experts,
                        qview(xq), b.offsets, b.slot_pair, d.topk, d.intermediate, b.h, ep);
     return;
   }
   const dim3 grid((d.intermediate + 4 * G * CPW - 1) / (4 * G * CPW), d.experts);
-  hipLaunchKernelGGL((gate_up_kernel<DT, T, KC, G, CPW>), grid, dim3(256), lds, s, views, d.experts,
+  hipq::launch_kernel("gate_up_kernel<DT, T, KC, G, CPW>", (gate_up_kernel<DT, T, KC, G, CPW>), grid, dim3(256), lds, s, views, d.experts,
                      qview(xq), b.offsets, b.slot_pair, d.topk, d.intermediate, b.h, ep);
 }
 template <int DT, int T, int KC, int G>
@@ -999,12 +999,12 @@ void launch_down(const hipq_moe_desc &d, const hipq::MoeEpi &ep, const WView *vi
   if (d.intermediate > KC) {
     const dim3 grid((d.hidden + 7) / 8, d.experts);
     const size_t lds_long = 4 * GemvLds<DT, RTOK, 2, false>::DWORDS * sizeof(uint32_t);
-    hipLaunchKernelGGL((down_long_kernel<DT>), grid, dim3(256), lds_long, s, views, d.experts,
+    hipq::launch_kernel("down_long_kernel<DT>", (down_long_kernel<DT>), grid, dim3(256), lds_long, s, views, d.experts,
                        qview(hq), b.offsets, b.slot_pair, b.wgt, d.hidden, b.contrib, ep);
     return;
   }
   const dim3 grid((d.hidden + 4 * G * CPW - 1) / (4 * G * CPW), d.experts);
-  hipLaunchKernelGGL((down_kernel<DT, T, KC, G, CPW>), grid, dim3(256), lds, s, views, d.experts,
+  hipq::launch_kernel("down_kernel<DT, T, KC, G, CPW>", (down_kernel<DT, T, KC, G, CPW>), grid, dim3(256), lds, s, views, d.experts,
                      qview(hq), b.offsets, b.slot_pair, b.wgt, d.hidden, b.contrib, ep);
 }
 
@@ -1062,11 +1062,11 @@ int launch_grouped_mma(const hipq::MoeArgs *a, const MoeBufs &b, const WView *vi
   if (lds_g > 64 * 1024) /* beyond the default limit of a launch */
     HIPQ_HIP(hipFuncSetAttribute(kg, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_g));
   if (few)
-    hipLaunchKernelGGL((gate_up_mma_kernel<TC, true>), dim3((d.intermediate + 63) / 64, max_items), dim3(256), lds_g,
+    hipq::launch_kernel("gate_up_mma_kernel<TC, true>", (gate_up_mma_kernel<TC, true>), dim3((d.intermediate + 63) / 64, max_items), dim3(256), lds_g,
                        s, views, d.experts, qview(xq), b.offsets, b.items, b.slot_pair, d.topk, d.intermediate,
                        b.h, a->epi);
   else
-    hipLaunchKernelGGL((gate_up_mma_kernel<TC, false>), dim3((d.intermediate + 127) / 128, max_items), dim3(256),
+    hipq::launch_kernel("gate_up_mma_kernel<TC, false>", (gate_up_mma_kernel<TC, false>), dim3((d.intermediate + 127) / 128, max_items), dim3(256),
                        lds_g, s, views, d.experts, qview(xq), b.offsets, b.items, b.slot_pair, d.topk,
                        d.intermediate, b.h, a->epi);
   HIPQ_HIP(hipGetLastError());
@@ -1085,10 +1085,10 @@ int launch_grouped_mma(const hipq::MoeArgs *a, const MoeBufs &b, const WView *vi
   const int ct = few ? 1 : 2;
   const dim3 gd((d.hidden + 128 * ct - 1) / (128 * ct), max_items);
   if (qh)
-    hipLaunchKernelGGL((down_mma_kernel<TC, true>), gd, dim3(256), lds_d, s, views, d.experts, qview(hq), b.h,
+    hipq::launch_kernel("down_mma_kernel<TC, true>", (down_mma_kernel<TC, true>), gd, dim3(256), lds_d, s, views, d.experts, qview(hq), b.h,
                        b.offsets, b.items, b.slot_pair, b.wgt, d.hidden, b.contrib, ct, a->epi);
   else
-    hipLaunchKernelGGL((down_mma_kernel<TC, false>), gd, dim3(256), lds_d, s, views, d.experts, qview(hq), b.h,
+    hipq::launch_kernel("down_mma_kernel<TC, false>", (down_mma_kernel<TC, false>), gd, dim3(256), lds_d, s, views, d.experts, qview(hq), b.h,
                        b.offsets, b.items, b.slot_pair, b.wgt, d.hidden, b.contrib, ct, a->epi);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
@@ -1154,7 +1154,7 @@ int launch_moe(const MoeArgs *a, void *workspace, size_t workspace_bytes, const 
 
   const float *logits = a->router_logits;
   if (!logits) {
-    hipLaunchKernelGGL(router_logits_kernel, dim3(T), dim3(256), 0, s, a->x, a->router_weight,
+    hipq::launch_kernel("router_logits_kernel", router_logits_kernel, dim3(T), dim3(256), 0, s, a->x, a->router_weight,
                        d.hidden, E, a->router_bias, b.logits);
     HIPQ_HIP(hipGetLastError());
     logits = b.logits;
@@ -1176,10 +1176,10 @@ int launch_moe(const MoeArgs *a, void *workspace, size_t workspace_bytes, const 
     const unsigned qblocks = mma ? (unsigned)((xqa.n_sb + 15) / 16) : 0;
     auto launch = [&](auto fused, auto plain) {
       if (mma)
-        hipLaunchKernelGGL(fused, dim3(1 + qblocks), dim3(1024), 0, s, logits, T, E, d.topk, d.renormalize, idx,
+        hipq::launch_kernel("fused", fused, dim3(1 + qblocks), dim3(1024), 0, s, logits, T, E, d.topk, d.renormalize, idx,
                            wgt, b.offsets, b.slot_pair, b.tok_slots, chunk, b.items, xqa);
       else
-        hipLaunchKernelGGL(plain, dim3(1), dim3(1024), 0, s, logits, T, E, d.topk, d.renormalize, idx, wgt,
+        hipq::launch_kernel("plain", plain, dim3(1), dim3(1024), 0, s, logits, T, E, d.topk, d.renormalize, idx, wgt,
                            b.offsets, b.slot_pair, b.tok_slots, chunk, b.items);
     };
     if (E <= 128) launch(route_sort_quantize_kernel<2>, route_sort_kernel<2>);
@@ -1191,10 +1191,10 @@ int launch_moe(const MoeArgs *a, void *workspace, size_t workspace_bytes, const 
     const unsigned qblocks = mma ? (unsigned)((xqa.n_sb + 3) / 4) : 0;
     auto launch = [&](auto fused, auto plain) {
       if (mma)
-        hipLaunchKernelGGL(fused, dim3(rblocks + qblocks), dim3(256), 0, s, logits, T, E, d.topk, d.renormalize,
+        hipq::launch_kernel("fused", fused, dim3(rblocks + qblocks), dim3(256), 0, s, logits, T, E, d.topk, d.renormalize,
                            idx, wgt, rblocks, xqa);
       else
-        hipLaunchKernelGGL(plain, dim3(rblocks), dim3(256), 0, s, logits, T, E, d.topk, d.renormalize, idx, wgt);
+        hipq::launch_kernel("plain", plain, dim3(rblocks), dim3(256), 0, s, logits, T, E, d.topk, d.renormalize, idx, wgt);
     };
     if (E <= 128) launch(route_quantize_kernel<2>, route_kernel<2>);
     else if (E <= 256) launch(route_quantize_kernel<4>, route_kernel<4>);
@@ -1204,13 +1204,13 @@ int launch_moe(const MoeArgs *a, void *workspace, size_t workspace_bytes, const 
   if (T <= 16 && E <= 1024) {
     /* routed and sorted above */
   } else if (P <= 16384 && E <= 1024) {
-    hipLaunchKernelGGL(sort_pairs_kernel, dim3(1), dim3(1024), 0, s, idx, P, E, d.topk, b.offsets,
+    hipq::launch_kernel("sort_pairs_kernel", sort_pairs_kernel, dim3(1), dim3(1024), 0, s, idx, P, E, d.topk, b.offsets,
                        b.slot_pair, b.tok_slots, chunk, b.items);
   } else {
-    hipLaunchKernelGGL(fill_int_kernel, dim3((E + 255) / 256), dim3(256), 0, s, b.counts, E, 0);
-    hipLaunchKernelGGL(count_kernel, dim3((P + 255) / 256), dim3(256), 0, s, idx, P, b.counts);
-    hipLaunchKernelGGL(scan_kernel, dim3(1), dim3(64), 0, s, b.counts, E, b.offsets, b.cursor, chunk, b.items);
-    hipLaunchKernelGGL(scatter_kernel, dim3((P + 255) / 256), dim3(256), 0, s, idx, P, d.topk, b.offsets,
+    hipq::launch_kernel("fill_int_kernel", fill_int_kernel, dim3((E + 255) / 256), dim3(256), 0, s, b.counts, E, 0);
+    hipq::launch_kernel("count_kernel", count_kernel, dim3((P + 255) / 256), dim3(256), 0, s, idx, P, b.counts);
+    hipq::launch_kernel("scan_kernel", scan_kernel, dim3(1), dim3(64), 0, s, b.counts, E, b.offsets, b.cursor, chunk, b.items);
+    hipq::launch_kernel("scatter_kernel", scatter_kernel, dim3((P + 255) / 256), dim3(256), 0, s, idx, P, d.topk, b.offsets,
                        b.cursor, b.slot_pair, b.tok_slots);
   }
   HIPQ_HIP(hipGetLastError());
@@ -1231,7 +1231,7 @@ int launch_moe(const MoeArgs *a, void *workspace, size_t workspace_bytes, const 
   else
     rc = launch_grouped<HIPQ_Q6_K>(a, b, views, xq, hq, s);
   if (rc) return rc;
-  hipLaunchKernelGGL(combine_kernel, dim3((d.hidden + 255) / 256, T), dim3(256), 0, s, b.tok_slots,
+  hipq::launch_kernel("combine_kernel", combine_kernel, dim3((d.hidden + 255) / 256, T), dim3(256), 0, s, b.tok_slots,
                      d.topk, d.hidden, b.contrib, a->y);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;

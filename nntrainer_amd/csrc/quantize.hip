@@ -196,10 +196,10 @@ int launch_quantize_q8_0(const float *A, int64_t M, int64_t K, int64_t lda,
   const int64_t threads = total * 8;
   const unsigned grid = (unsigned)((threads + 255) / 256);
   if (canonical_out)
-    hipLaunchKernelGGL(quantize_q8_0_kernel<true>, dim3(grid), dim3(256), 0, s, A, total, nb, lda,
+    hipq::launch_kernel("quantize_q8_0_kernel<true>", quantize_q8_0_kernel<true>, dim3(grid), dim3(256), 0, s, A, total, nb, lda,
                        nullptr, nullptr, (uint8_t *)canonical_out);
   else
-    hipLaunchKernelGGL(quantize_q8_0_kernel<false>, dim3(grid), dim3(256), 0, s, A, total, nb, lda,
+    hipq::launch_kernel("quantize_q8_0_kernel<false>", quantize_q8_0_kernel<false>, dim3(grid), dim3(256), 0, s, A, total, nb, lda,
                        qa->q, qa->meta, nullptr);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
@@ -216,11 +216,11 @@ int launch_quantize_q8_K(const float *A, int64_t M, int64_t K, int64_t lda,
   const int64_t total = M * nsb;
   const unsigned grid = (unsigned)((total + 3) / 4);
   if (canonical_out)
-    hipLaunchKernelGGL(quantize_q8_K_kernel<Q8K_CANONICAL>, dim3(grid), dim3(256), 0, s, A, M, total,
+    hipq::launch_kernel("quantize_q8_K_kernel<Q8K_CANONICAL>", quantize_q8_K_kernel<Q8K_CANONICAL>, dim3(grid), dim3(256), 0, s, A, M, total,
                        nsb, lda, mat_rows, nullptr, nullptr, nullptr, (uint8_t *)canonical_out, nullptr, nullptr,
                        nullptr);
   else
-    hipLaunchKernelGGL(quantize_q8_K_kernel<Q8K_PLANES>, dim3(grid), dim3(256), 0, s, A, M, total, nsb,
+    hipq::launch_kernel("quantize_q8_K_kernel<Q8K_PLANES>", quantize_q8_K_kernel<Q8K_PLANES>, dim3(grid), dim3(256), 0, s, A, M, total, nsb,
                        lda, mat_rows, qa->q, qa->d, qa->bsum, nullptr, nullptr, (uint16_t *)qa->ql,
                        (uint16_t *)qa->qh);
   HIPQ_HIP(hipGetLastError());
@@ -236,7 +236,7 @@ int launch_quantize_q8_K_rowmma(const float *A, int64_t M, int64_t K, int64_t ld
   const int nsb = (int)(K / 256);
   const int64_t total = M * nsb;
   const unsigned grid = (unsigned)((total + 3) / 4);
-  hipLaunchKernelGGL(quantize_q8_K_kernel<Q8K_ROWMMA>, dim3(grid), dim3(256), 0, s, A, M, total, nsb, lda,
+  hipq::launch_kernel("quantize_q8_K_kernel<Q8K_ROWMMA>", quantize_q8_K_kernel<Q8K_ROWMMA>, dim3(grid), dim3(256), 0, s, A, M, total, nsb, lda,
                      mat_rows, qa->q, qa->d, nullptr, nullptr, (uint16_t *)qa->bsum, nullptr, nullptr);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
@@ -251,7 +251,7 @@ int launch_quantize_q8_K_tiled(const float *A, int64_t M, int64_t K, int64_t lda
   const int nsb = (int)(K / 256);
   const int64_t units = (int64_t)qa->mtiles * 32 * nsb; /* (row quad, super-block) pairs, padding rows included */
   const unsigned grid = (unsigned)((units + 3) / 4);
-  launch_kernel(quantize_q8_K_tiled_kernel, dim3(grid), dim3(256), 0, s, A, M, units, (int)nsb, lda, mat_rows, qa->qt,
+  hipq::launch_kernel("quantize_q8_K_tiled_kernel", quantize_q8_K_tiled_kernel, dim3(grid), dim3(256), 0, s, A, M, units, (int)nsb, lda, mat_rows, qa->qt,
                 qa->dAt, qa->amin);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;

@@ -246,11 +246,11 @@ int ensure_gemm_tiles(hipq_weight *w) {
     return fail(HIPQ_ERR_OUT_OF_MEMORY, "GEMM tiles of %zu bytes: %s", q_bytes + x_bytes + h_bytes, hipGetErrorString(e));
   if (q6) {
     const int64_t lanes = tiles * nsb * 64;
-    hipLaunchKernelGGL(gemm_tile_q6_K, dim3((unsigned)((lanes + 255) / 256)), dim3(256), 0, nullptr, w->qs, w->qh, w->sc,
+    hipq::launch_kernel("gemm_tile_q6_K", gemm_tile_q6_K, dim3((unsigned)((lanes + 255) / 256)), dim3(256), 0, nullptr, w->qs, w->qh, w->sc,
                        w->d, (int)w->N, nsb, (int64_t)w->N * nsb, lanes, nb, nb + q_bytes, nb + q_bytes + x_bytes);
   } else {
     const int64_t pieces = tiles * nsb * 256;
-    hipLaunchKernelGGL(gemm_tile_q4_K, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, nullptr, w->qs, w->hdr,
+    hipq::launch_kernel("gemm_tile_q4_K", gemm_tile_q4_K, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, nullptr, w->qs, w->hdr,
                        (int)w->N, nsb, pieces, nb, nb + q_bytes);
   }
   e = hipGetLastError();
@@ -276,7 +276,7 @@ int tile_expert_weight(hipq_weight *w) {
   hipError_t e = hipMalloc((void **)&nb, bytes);
   if (e != hipSuccess) return fail(HIPQ_ERR_OUT_OF_MEMORY, "expert tiles of %zu bytes: %s", bytes, hipGetErrorString(e));
   const int64_t pieces = tiles * nsb * 256;
-  hipLaunchKernelGGL(tile_q4_K, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, nullptr, w->qs, w->hdr,
+  hipq::launch_kernel("tile_q4_K", tile_q4_K, dim3((unsigned)((pieces + 255) / 256)), dim3(256), 0, nullptr, w->qs, w->hdr,
                      (int)w->N, nsb, pieces, nb);
   e = hipGetLastError();
   if (e == hipSuccess) e = hipDeviceSynchronize(); /* nothing may still read the planes that are freed next */
@@ -298,16 +298,16 @@ int launch_relayout(hipq_weight *w, int layout, const uint8_t *src, hipStream_t 
   if (w->dtype == HIPQ_Q4_0) {
     const int nb = (int)(w->K / 32);
     const int64_t total = w->N * nb;
-    hipLaunchKernelGGL(relayout_q4_0, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, src,
+    hipq::launch_kernel("relayout_q4_0", relayout_q4_0, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, src,
                        x8, w->N, nb, (uint8_t *)w->qs, (uint16_t *)w->d);
   } else if (w->dtype == HIPQ_Q4_K) {
     const int nb = (int)(w->K / 256);
     const int64_t total = w->N * nb;
-    hipLaunchKernelGGL(relayout_q4_K, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, src,
+    hipq::launch_kernel("relayout_q4_K", relayout_q4_K, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, src,
                        x8, w->N, nb, (uint8_t *)w->qs, (uint8_t *)w->hdr);
   } else {
     const int64_t total = w->N * (w->K / 256);
-    hipLaunchKernelGGL(relayout_q6_K, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, src,
+    hipq::launch_kernel("relayout_q6_K", relayout_q6_K, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, s, src,
                        total, (uint8_t *)w->qs, (uint8_t *)w->qh, (int8_t *)w->sc,
                        (uint16_t *)w->d);
   }

@@ -305,15 +305,15 @@ int launch_quantize_weights(int dtype, const float *W, int64_t N, int64_t K, voi
                             hipStream_t s) {
   if (dtype == HIPQ_Q4_0) {
     const int64_t nblk = N * (K / 32);
-    hipLaunchKernelGGL(quantize_w_q4_0, dim3((unsigned)((nblk + 255) / 256)), dim3(256), 0, s, W,
+    hipq::launch_kernel("quantize_w_q4_0", quantize_w_q4_0, dim3((unsigned)((nblk + 255) / 256)), dim3(256), 0, s, W,
                        nblk, (uint8_t *)out);
   } else if (dtype == HIPQ_Q4_K) {
     const int64_t nblk = N * (K / 256);
-    hipLaunchKernelGGL(quantize_w_q4_K, dim3((unsigned)((nblk + 63) / 64)), dim3(64), 0, s, W, nblk,
+    hipq::launch_kernel("quantize_w_q4_K", quantize_w_q4_K, dim3((unsigned)((nblk + 63) / 64)), dim3(64), 0, s, W, nblk,
                        (uint8_t *)out);
   } else if (dtype == HIPQ_Q6_K) {
     const int64_t nblk = N * (K / 256);
-    hipLaunchKernelGGL(quantize_w_q6_K, dim3((unsigned)((nblk + 63) / 64)), dim3(64), 0, s, W, nblk,
+    hipq::launch_kernel("quantize_w_q6_K", quantize_w_q6_K, dim3((unsigned)((nblk + 63) / 64)), dim3(64), 0, s, W, nblk,
                        (uint8_t *)out);
   } else {
     return fail(HIPQ_ERR_INVALID_ARGUMENT, "unknown weight dtype %d", dtype);

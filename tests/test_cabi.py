@@ -23,6 +23,21 @@ def test_header_symbols_are_exported():
         assert getattr(lib, n) is not None
 
 
+def test_product_library_exports_exactly_the_header(tmp_path):
+    """libhipq.so exports the functions include/hipq.h declares and no others; the measurement
+    and test helpers live in libhipq_bench.so, which links it."""
+    import subprocess
+    out = subprocess.run(["nm", "-D", "--defined-only", capi.LIB_PATH], capture_output=True, text=True, check=True).stdout
+    exported = sorted(line.split()[-1] for line in out.splitlines() if " T " in line)
+    assert exported == _declared(), set(exported) ^ set(_declared())
+    bench = os.path.join(os.path.dirname(capi.LIB_PATH), "libhipq_bench.so")
+    out = subprocess.run(["nm", "-D", "--defined-only", bench], capture_output=True, text=True, check=True).stdout
+    have = {line.split()[-1] for line in out.splitlines() if " T " in line}
+    assert set(capi.BENCH_SYMBOLS) <= have
+    needed = subprocess.run(["readelf", "-d", bench], capture_output=True, text=True, check=True).stdout
+    assert "libhipq.so" in needed
+
+
 def test_weight_size_rules():
     # 18 B / 32, 144 B / 256, 210 B / 256 (q4_0_tensor.h:20-31, q4_k_tensor.h:25-33, q6_k_tensor.h:25-32)
     assert capi.weight_nbytes("q4_0", 4096, 4096) == 9437184
