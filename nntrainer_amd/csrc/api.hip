@@ -50,6 +50,12 @@ struct Workspace {
   /* device copies of a host-memory call's operands (the kernels' own scratch is ptr) */
   void *io = nullptr;
   size_t io_bytes = 0;
+  /* page-locked staging of a decode step's pageable operands (DirectIO) */
+  void *pin = nullptr;
+  size_t pin_bytes = 0;
+  /* a page-locked word the last launch of such a call writes and the host polls */
+  uint32_t *done = nullptr;
+  uint32_t done_seq = 0;
   /* held while a call enqueues its launches: two threads that name the same stream
    * must not interleave their kernels (the second would quantize into the scratch
    * the first one's product has not read yet) */
@@ -231,6 +237,172 @@ bool is_pinned(const void *p) {
   }
   return at.type == hipMemoryTypeHost;
 }
+
+/* The address the GPU uses for page-locked host memory (null if p is none). */
+void *pinned_device_ptr(const void *p) {
+  hipPointerAttribute_t at;
+  if (hipPointerGetAttributes(&at, p) != hipSuccess) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  if (at.type != hipMemoryTypeHost) return nullptr;
+  void *d = nullptr;
+  if (hipHostGetDevicePointer(&d, const_cast<void *>(p), 0) != hipSuccess) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  return d;
+}
+
+/* A few rows of page-locked host memory into a dense device buffer, by a kernel: each value
+ * crosses the bus once, and a launch costs less than a copy engine's start. */
+__global__ __launch_bounds__(256) void fetch_rows_kernel(const float *__restrict__ src, int64_t lds, float *__restrict__ dst,
+                                                         int K, int rows) {
+  const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+  if (i >= (int64_t)rows * K) return;
+  const int r = (int)(i / K), c = (int)(i - (int64_t)r * K); /* K % 4 == 0 */
+  *(float4 *)(dst + i) = *(const float4 *)(src + r * lds + c);
+}
+
+/* The stream's page-locked staging buffer, grown on demand (the stream is idle when it grows: the
+ * calls that use it are synchronous and hold the stream's enqueue lock). */
+int pinned_staging(hipStream_t s, size_t bytes, void **out) {
+  std::lock_guard<std::mutex> lk(g.mu);
+  Workspace &w = g.ws[s];
+  if (w.pin_bytes < bytes) {
+    if (w.pin) {
+      HIPQ_HIP(hipStreamSynchronize(s));
+      HIPQ_HIP(hipHostFree(w.pin));
+      w.pin = nullptr;
+      w.pin_bytes = 0;
+    }
+    const size_t want = (bytes + ((size_t)1 << 16) - 1) & ~(((size_t)1 << 16) - 1);
+    hipError_t e = hipHostMalloc(&w.pin, want, hipHostMallocDefault);
+    if (e != hipSuccess) {
+      w.pin = nullptr;
+      return fail(HIPQ_ERR_OUT_OF_MEMORY, "page-locked staging of %zu bytes: %s", want, hipGetErrorString(e));
+    }
+    w.pin_bytes = want;
+  }
+  *out = w.pin;
+  return HIPQ_OK;
+}
+
+/* The end of a short synchronous call: a one-thread kernel behind the call's launches writes the
+ * call's number into a page-locked word and the host polls that word. Waking a thread out of
+ * hipStreamSynchronize costs several microseconds more than the poll sees the store; a call that
+ * takes longer than the poll is patient falls back to the stream's wait. */
+__global__ void signal_done_kernel(uint32_t *word, uint32_t value) {
+  __hip_atomic_store(word, value, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+int wait_done(hipStream_t s) {
+  uint32_t *word = nullptr, seq = 0;
+  {
+    std::lock_guard<std::mutex> lk(g.mu);
+    Workspace &w = g.ws[s];
+    if (!w.done) {
+      hipError_t e = hipHostMalloc((void **)&w.done, 64, hipHostMallocDefault);
+      if (e != hipSuccess) {
+        w.done = nullptr;
+        (void)hipGetLastError();
+      } else
+        *w.done = 0;
+    }
+    word = w.done;
+    seq = ++w.done_seq;
+  }
+  if (!word) {
+    HIPQ_HIP(hipStreamSynchronize(s));
+    return HIPQ_OK;
+  }
+  hipq::launch_kernel("signal_done_kernel", signal_done_kernel, dim3(1), dim3(1), 0, s, (uint32_t *)pinned_device_ptr(word), seq);
+  HIPQ_HIP(hipGetLastError());
+  for (int spin = 0; spin < 200000; ++spin) { /* about a tenth of a millisecond */
+    if (__atomic_load_n(word, __ATOMIC_ACQUIRE) == seq) return HIPQ_OK;
+    __builtin_ia32_pause();
+  }
+  HIPQ_HIP(hipStreamSynchronize(s));
+  return HIPQ_OK;
+}
+
+/* A decode step's host operands without a copy engine. Up to eight rows and small outputs (what an
+ * FC sees while tokens are generated): the rows are fetched into device memory by a small kernel,
+ * the product kernels write their outputs straight into host memory, and one wait ends the call --
+ * two launches and a wait instead of a copy in, the launches, one copy out per output and the wait.
+ * Page-locked operands (the context's allocator) are used where they lie; pageable ones pass through
+ * the stream's page-locked staging buffer with a memcpy on either side. */
+constexpr int64_t DIRECT_ROWS = 8;
+constexpr size_t DIRECT_BYTES = (size_t)1 << 20; /* rows in, and all outputs together */
+struct DirectIO {
+  struct Out {
+    float *host, *dev; /* where the caller wants it; where the kernels write (device-side address) */
+    int64_t hld, dld, N;
+    float *bounce; /* host address of the staging the kernels write, or null */
+  };
+  hipStream_t s = nullptr;
+  int64_t rows = 0;
+  const float *a_dev = nullptr; /* device-side address of the rows to fetch */
+  int64_t a_ld = 0;
+  std::vector<Out> outs;
+
+  /* false: the call does not qualify (too many rows or bytes, odd K) and takes the copy engines */
+  bool begin(hipStream_t stream, const float *A, int64_t M, int64_t lda, int64_t K, int count, float *const *C,
+             const int64_t *ldc, const int64_t *Ns, int *rc) {
+    *rc = HIPQ_OK;
+    if (M < 1 || M > DIRECT_ROWS || (K & 3) || (size_t)M * K * 4 > DIRECT_BYTES) return false;
+    size_t out_bytes = 0, stage_bytes = 0;
+    for (int i = 0; i < count; ++i) out_bytes += (size_t)M * Ns[i] * 4;
+    if (out_bytes > DIRECT_BYTES) return false;
+    s = stream;
+    rows = M;
+    const bool a_direct = !(lda & 3) && !((uintptr_t)A & 15) && pinned_device_ptr(A);
+    if (!a_direct) stage_bytes += ((size_t)M * K * 4 + 255) & ~(size_t)255;
+    outs.resize(count);
+    for (int i = 0; i < count; ++i) {
+      outs[i] = Out{C[i], (float *)pinned_device_ptr(C[i]), ldc[i], ldc[i], Ns[i], nullptr};
+      if (!outs[i].dev) stage_bytes += ((size_t)M * Ns[i] * 4 + 255) & ~(size_t)255;
+    }
+    char *stage = nullptr;
+    if (stage_bytes) {
+      void *p = nullptr;
+      if ((*rc = pinned_staging(s, stage_bytes, &p))) return false;
+      stage = (char *)p;
+    }
+    if (a_direct) {
+      a_dev = (const float *)pinned_device_ptr(A);
+      a_ld = lda;
+    } else {
+      for (int64_t r = 0; r < M; ++r) memcpy(stage + (size_t)r * K * 4, A + r * lda, (size_t)K * 4);
+      a_dev = (const float *)pinned_device_ptr(stage);
+      a_ld = K;
+      stage += ((size_t)M * K * 4 + 255) & ~(size_t)255;
+    }
+    for (Out &o : outs)
+      if (!o.dev) {
+        o.bounce = (float *)stage;
+        o.dev = (float *)pinned_device_ptr(stage);
+        o.dld = o.N;
+        stage += ((size_t)M * o.N * 4 + 255) & ~(size_t)255;
+      }
+    return true;
+  }
+  /* the rows into dense device memory dst [rows x K] */
+  int fetch(float *dst, int64_t K) const {
+    const int64_t quads = rows * K / 4;
+    hipq::launch_kernel("fetch_rows_kernel", fetch_rows_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, s, a_dev,
+                        a_ld, dst, (int)K, (int)rows);
+    HIPQ_HIP(hipGetLastError());
+    return HIPQ_OK;
+  }
+  /* waits for the kernels; staged outputs go to where the caller wants them */
+  int finish() const {
+    if (int rc = wait_done(s)) return rc;
+    for (const Out &o : outs)
+      if (o.bounce)
+        for (int64_t r = 0; r < rows; ++r) memcpy(o.host + r * o.hld, o.bounce + r * o.N, (size_t)o.N * 4);
+    return HIPQ_OK;
+  }
+};
 
 /* rows x width bytes between host (pitch hpitch) and a dense device buffer, in order on s.
  * to_device: the copy is queued when this returns (the host bytes have been read). Otherwise
@@ -600,6 +772,8 @@ int hipq_shutdown(void) {
   for (auto &kv : g.ws) {
     if (kv.second.ptr) (void)hipFree(kv.second.ptr);
     if (kv.second.io) (void)hipFree(kv.second.io);
+    if (kv.second.pin) (void)hipHostFree(kv.second.pin);
+    if (kv.second.done) (void)hipHostFree(kv.second.done);
     for (void *p : kv.second.retired) (void)hipFree(p);
   }
   g.ws.clear();
@@ -639,6 +813,8 @@ int hipq_stream_release(void *stream) {
   HIPQ_HIP(hipStreamSynchronize(s));
   if (it->second.ptr) (void)hipFree(it->second.ptr);
   if (it->second.io) (void)hipFree(it->second.io);
+  if (it->second.pin) (void)hipHostFree(it->second.pin);
+  if (it->second.done) (void)hipHostFree(it->second.done);
   for (void *p : it->second.retired) (void)hipFree(p);
   el.unlock();
   el.release();
@@ -930,6 +1106,15 @@ int hipq_matmul(hipq_weight_t w, const float *A, int64_t M, int64_t lda, float *
   void *io = nullptr;
   if ((rc = io_buffer(s, a_bytes + c_bytes, &io))) return rc;
   float *dA = (float *)io, *dC = (float *)((char *)io + a_bytes);
+  {
+    DirectIO dio; /* a decode step's rows: no copy engine */
+    if (dio.begin(s, A, M, lda, w->K, 1, &C, &ldc, &w->N, &rc)) {
+      if ((rc = dio.fetch(dA, w->K))) return rc;
+      if ((rc = matmul_device(w, dA, M, w->K, dio.outs[0].dev, dio.outs[0].dld, s, sc))) return rc;
+      return dio.finish();
+    }
+    if (rc) return rc;
+  }
   if ((rc = stage_copy(true, dA, (void *)A, (size_t)lda * 4, (size_t)w->K * 4, (size_t)M, s))) return rc;
   if ((rc = matmul_device(w, dA, M, w->K, dC, w->N, s, sc))) return rc;
   return stage_copy(false, dC, C, (size_t)ldc * 4, (size_t)w->N * 4, (size_t)M, s);
@@ -949,12 +1134,19 @@ int hipq_matmul_each_row(hipq_weight_t w, const float *A, int64_t rows, int64_t 
   const float *dA = A;
   float *dC = C;
   int64_t a_ld = lda, c_ld = ldc;
+  bool direct = false;
+  DirectIO dio;
   if (mem == HIPQ_MEM_HOST) {
     const size_t a_bytes = ((size_t)rows * w->K * 4 + 255) & ~(size_t)255, c_bytes = (size_t)rows * w->N * 4;
     void *io = nullptr;
     if ((rc = io_buffer(s, a_bytes + c_bytes, &io))) return rc;
     dA = (const float *)io, dC = (float *)((char *)io + a_bytes), a_ld = w->K, c_ld = w->N;
-    if ((rc = stage_copy(true, (void *)dA, (void *)A, (size_t)lda * 4, (size_t)w->K * 4, (size_t)rows, s))) return rc;
+    if (dio.begin(s, A, rows, lda, w->K, 1, &C, &ldc, &w->N, &rc)) { /* a decode step's rows: no copy engine */
+      if ((rc = dio.fetch((float *)io, w->K))) return rc;
+      dC = dio.outs[0].dev, c_ld = dio.outs[0].dld;
+      direct = true;
+    } else if (rc || (rc = stage_copy(true, (void *)dA, (void *)A, (size_t)lda * 4, (size_t)w->K * 4, (size_t)rows, s)))
+      return rc;
   }
   for (int64_t r0 = 0; r0 < rows && !rc;) { /* steps of row counts that keep the M = 1 bits */
     int64_t n = (rows - r0) < 16 ? (rows - r0) : 16;
@@ -971,6 +1163,7 @@ int hipq_matmul_each_row(hipq_weight_t w, const float *A, int64_t rows, int64_t 
     r0 += n;
   }
   if (rc || mem == HIPQ_MEM_DEVICE) return rc;
+  if (direct) return dio.finish();
   return stage_copy(false, dC, C, (size_t)ldc * 4, (size_t)w->N * 4, (size_t)rows, s);
 }
 
@@ -1014,12 +1207,20 @@ int hipq_mlp_swiglu(hipq_weight_t w_act, hipq_weight_t w_mul, const float *A, in
         *dO = (float *)((char *)dZ + o_bytes);
   const float *a_dev = A;
   int64_t a_ld = lda;
+  float *h_out = nullptr; /* a decode step's output: the device-side address the kernels write */
+  int64_t h_ld = 0;
+  DirectIO dio;
   if (mem == HIPQ_MEM_HOST) {
-    if ((rc = stage_copy(true, dA, (void *)A, (size_t)lda * 4, (size_t)K * 4, (size_t)M, s))) return rc;
+    if (dio.begin(s, A, M, lda, K, 1, &out, &ldo, &N, &rc)) {
+      if ((rc = dio.fetch(dA, K))) return rc;
+      h_out = dio.outs[0].dev, h_ld = dio.outs[0].dld;
+    } else if (rc || (rc = stage_copy(true, dA, (void *)A, (size_t)lda * 4, (size_t)K * 4, (size_t)M, s)))
+      return rc;
     a_dev = dA;
     a_ld = K;
     if (M == 1 && hipq::gemv_fuses_swiglu(w_act, w_mul, dA)) {
-      if ((rc = hipq::launch_gemv_fused_swiglu(w_act, w_mul, dA, dO, s))) return rc;
+      if ((rc = hipq::launch_gemv_fused_swiglu(w_act, w_mul, dA, h_out ? h_out : dO, s))) return rc;
+      if (h_out) return dio.finish();
       return stage_copy(false, dO, out, (size_t)ldo * 4, (size_t)N * 4, 1, s);
     }
   }
@@ -1028,6 +1229,10 @@ int hipq_mlp_swiglu(hipq_weight_t w_act, hipq_weight_t w_mul, const float *A, in
   const int64_t lds[2] = {N, N};
   if ((rc = hipq_matmul_multi(2, ws, a_dev, M, a_ld, cs, lds, HIPQ_MEM_DEVICE, stream))) return rc;
   if (mem == HIPQ_MEM_DEVICE) return hipq::launch_swiglu_rows(dY, dZ, M, N, out, ldo, s);
+  if (h_out) {
+    if ((rc = hipq::launch_swiglu_rows(dY, dZ, M, N, h_out, h_ld, s))) return rc;
+    return dio.finish();
+  }
   if ((rc = hipq::launch_swiglu_rows(dY, dZ, M, N, dO, N, s))) return rc;
   return stage_copy(false, dO, out, (size_t)ldo * 4, (size_t)N * 4, (size_t)M, s);
 }
@@ -1058,9 +1263,21 @@ int hipq_matmul_multi(int count, const hipq_weight_t *w, const float *A, int64_t
     }
     void *io = nullptr;
     if ((rc = io_buffer(s, total, &io))) return rc;
-    if ((rc = stage_copy(true, io, (void *)A, (size_t)lda * 4, (size_t)Kh * 4, (size_t)M, s))) return rc;
     std::vector<float *> dC(count);
     std::vector<int64_t> dld(count);
+    /* a decode step's rows: fetched by a kernel, the outputs written by the product kernels */
+    DirectIO dio;
+    std::vector<int64_t> ns(count);
+    for (int i = 0; i < count; ++i) ns[i] = w[i]->N;
+    if (dio.begin(s, A, M, lda, Kh, count, C, ldc, ns.data(), &rc)) {
+      for (int i = 0; i < count; ++i) dC[i] = dio.outs[i].dev, dld[i] = dio.outs[i].dld;
+      if ((rc = dio.fetch((float *)io, Kh))) return rc;
+      if ((rc = hipq_matmul_multi(count, w, (const float *)io, M, Kh, dC.data(), dld.data(), HIPQ_MEM_DEVICE, stream)))
+        return rc;
+      return dio.finish();
+    }
+    if (rc) return rc;
+    if ((rc = stage_copy(true, io, (void *)A, (size_t)lda * 4, (size_t)Kh * 4, (size_t)M, s))) return rc;
     for (int i = 0; i < count; ++i) {
       dC[i] = (float *)((char *)io + off[i]);
       dld[i] = w[i]->N;

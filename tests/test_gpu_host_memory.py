@@ -97,3 +97,86 @@ def test_stream_release(hipq, cr):
         capi.stream_release(st.cuda_stream)
     capi.stream_release(st.cuda_stream)  # nothing kept: a no-op
     w.destroy()
+
+
+class _Pinned:
+    """A float32 array in page-locked memory of the context's allocator."""
+
+    def __init__(self, shape, fill=None):
+        self.n = int(np.prod(shape))
+        self.addr = capi.host_alloc(self.n * 4)
+        self.arr = np.ctypeslib.as_array(ctypes.cast(self.addr, ctypes.POINTER(ctypes.c_float)), tuple(shape))
+        if fill is not None:
+            self.arr[...] = fill
+
+    def free(self):
+        capi.host_free(self.addr)
+
+
+@pytest.mark.parametrize("kind,m,k,n,lda_pad,ldc_pad", [
+    ("q4_0", 1, 1024, 3072, 0, 0),      # one launch that quantizes the row itself
+    ("q4_K", 1, 4096, 4096, 0, 0),
+    ("q6_K", 1, 1024, 40000, 0, 0),     # two launches (vocabulary-sized)
+    ("q4_K", 3, 2048, 1024, 8, 4),      # strided rows on both sides
+    ("q4_0", 8, 1024, 3072, 0, 12),
+    ("q4_K", 8, 4096, 12288, 0, 0),     # the few-rows matrix-core kernel
+    ("q4_0", 9, 1024, 3072, 0, 0),      # one row more than the direct path takes: through the copy engines
+])
+def test_a_few_page_locked_rows_take_no_copy(hipq, cr, kind, m, k, n, lda_pad, ldc_pad):
+    """Up to eight rows in page-locked memory (a decode step through the Layer API): the rows are
+    fetched by a kernel and the product kernels write the host tensor directly. Same bits as the
+    device-memory call; the padding of strided rows stays untouched; two calls in a row."""
+    blocks = cr.quantize_weights(cr.oracle(), kind, synth.normal(9400 + n % 89, (n, k), 0.02))
+    w = capi.Weight(kind, n, k, blocks)
+    a = synth.normal(9401 + m, (m, k))
+    want = _device_result(w, a)
+    lda, ldc = k + lda_pad, n + ldc_pad
+    pa, pc = _Pinned((m, lda), 7e9), _Pinned((m, ldc), -3.5)
+    try:
+        pa.arr[:, :k] = a
+        for _ in range(2):
+            pc.arr[:, :n] = np.nan
+            capi.matmul(w, pa.addr, m, pc.addr, lda=lda, ldc=ldc, mem=capi.MEM_HOST)
+            assert np.array_equal(pc.arr[:, :n].view(np.uint32), want.view(np.uint32))
+            assert np.all(pc.arr[:, n:] == np.float32(-3.5))
+        # the rows of a decode step of a batch: each with the bits of its own one-row product
+        pc.arr[:, :n] = np.nan
+        capi.matmul_each_row(w, pa.addr, m, pc.addr, lda=lda, ldc=ldc, mem=capi.MEM_HOST)
+        for r in range(m):
+            assert np.array_equal(pc.arr[r, :n].view(np.uint32), _device_result(w, a[r:r + 1])[0].view(np.uint32)), r
+    finally:
+        pa.free()
+        pc.free()
+        w.destroy()
+
+
+@pytest.mark.parametrize("kind,m", [("q4_0", 1), ("q4_K", 1), ("q4_0", 4), ("q4_K", 8), ("q6_K", 2)])
+def test_grouped_calls_on_a_few_page_locked_rows(hipq, cr, kind, m):
+    """hipq_matmul_multi (Q, K, V) and hipq_mlp_swiglu (up, gate and the activation) with a decode
+    step's page-locked operands: outputs written by the kernels, the bits of the device calls."""
+    import gpu_util as gu
+    import torch
+    k, ns = 1024, (2048, 1024, 1024)
+    ws = [capi.Weight(kind, n, k, cr.quantize_weights(cr.oracle(), kind, synth.normal(9500 + j, (n, k), 0.05)))
+          for j, n in enumerate(ns)]
+    a = synth.normal(9510 + m, (m, k))
+    pa = _Pinned((m, k), a)
+    pcs = [_Pinned((m, n), np.nan) for n in ns]
+    po = _Pinned((m, ns[1]), np.nan)
+    try:
+        capi.matmul_multi(ws, pa.addr, m, [p.addr for p in pcs], mem=capi.MEM_HOST)
+        dev = [torch.full((m, n), float("nan"), device="cuda") for n in ns]
+        capi.matmul_multi(ws, gu.dev(a), m, dev, stream=gu.stream())
+        torch.cuda.synchronize()
+        for p, d in zip(pcs, dev):
+            assert np.array_equal(p.arr.view(np.uint32), d.cpu().numpy().view(np.uint32))
+        capi.mlp_swiglu(ws[1], ws[2], pa.addr, m, po.addr, mem=capi.MEM_HOST)
+        want = torch.full((m, ns[1]), float("nan"), device="cuda")
+        capi.mlp_swiglu(ws[1], ws[2], gu.dev(a), m, want, stream=gu.stream())
+        torch.cuda.synchronize()
+        assert np.array_equal(po.arr.view(np.uint32), want.cpu().numpy().view(np.uint32))
+    finally:
+        for p in [pa, po] + pcs:
+            p.free()
+        for w in ws:
+            w.destroy()
