@@ -294,6 +294,9 @@ typedef struct hipq_moe_ext {
   int32_t biases_on_device; /* non-zero: the four bias pointers are device memory
                                whatever `mem` says (a layer uploads them once,
                                hipq_device_alloc / hipq_device_upload)         */
+  int32_t router_on_device; /* non-zero: router_weight is device memory whatever
+                               `mem` says (1 MB at 2048 x 128: not worth a copy
+                               per call)                                       */
 } hipq_moe_ext;
 HIPQ_API int hipq_moe_forward_ext(const hipq_moe_desc *desc, const hipq_moe_ext *ext,
                                   const hipq_weight_t *gate, const hipq_weight_t *up,

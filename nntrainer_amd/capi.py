@@ -54,7 +54,7 @@ class MoeDesc(C.Structure):
 class MoeExt(C.Structure):
     _fields_ = [("variant", C.c_int32), ("alpha", C.c_float), ("router_bias", C.c_void_p),
                 ("gate_bias", C.c_void_p), ("up_bias", C.c_void_p), ("down_bias", C.c_void_p),
-                ("limit", C.c_float), ("biases_on_device", C.c_int32)]
+                ("limit", C.c_float), ("biases_on_device", C.c_int32), ("router_on_device", C.c_int32)]
 
 
 MOE_QWEN, MOE_GPT_OSS = 0, 1
@@ -281,7 +281,7 @@ def moe_forward_gpt_oss(tokens, hidden, inter, experts, topk, gate, up, down, x,
     limit > 0: the cached layer's clamps on the biased gate and up values."""
     d = MoeDesc(tokens, hidden, inter, experts, topk, 1 if renormalize else 0)
     ext = MoeExt(MOE_GPT_OSS, alpha, _addr(router_bias), _addr(gate_bias), _addr(up_bias), _addr(down_bias),
-                 limit, 1 if biases_on_device else 0)
+                 limit, 1 if biases_on_device else 0, 0)
     ex = gate if isinstance(gate, Experts) else Experts(gate, up, down)
     check(lib().hipq_moe_forward_ext(C.byref(d), C.byref(ext), ex.gate, ex.up, ex.down, _addr(x),
                                      _addr(router_logits), _addr(router_weight), _addr(y),

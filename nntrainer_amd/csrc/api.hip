@@ -1602,13 +1602,15 @@ int hipq_moe_forward_ext(const hipq_moe_desc *desc, const hipq_moe_ext *ext, con
   }
   if (mem != HIPQ_MEM_HOST) return fail(HIPQ_ERR_INVALID_ARGUMENT, "unknown mem kind %d", mem);
   /* host operands: device copies in the stream's operand buffer (no allocation per call); biases
-   * the caller keeps on the device are used where they are */
+   * and a router weight the caller keeps on the device are used where they are; a decode step's
+   * few rows take no copy engine (DirectIO) */
   const bool gpt = x_.variant == HIPQ_MOE_GPT_OSS;
   const bool host_biases = !x_.biases_on_device;
+  const bool host_router = router_logits || !x_.router_on_device;
   auto up256 = [](size_t n) { return (n + 255) & ~(size_t)255; };
   const size_t n_router = router_logits ? T * E : H * E;
-  const size_t o_x = 0, o_r = o_x + up256(T * H * 4), o_y = o_r + up256(n_router * 4), o_i = o_y + up256(T * H * 4),
-               o_w = o_i + up256(T * k * 4), o_br = o_w + up256(T * k * 4),
+  const size_t o_x = 0, o_r = o_x + up256(T * H * 4), o_y = o_r + (host_router ? up256(n_router * 4) : 0),
+               o_i = o_y + up256(T * H * 4), o_w = o_i + up256(T * k * 4), o_br = o_w + up256(T * k * 4),
                o_bg = o_br + (host_biases && x_.router_bias ? up256(E * 4) : 0),
                o_bu = o_bg + (host_biases && gpt ? up256(E * I * 4) : 0),
                o_bd = o_bu + (host_biases && gpt ? up256(E * I * 4) : 0),
@@ -1630,17 +1632,32 @@ int hipq_moe_forward_ext(const hipq_moe_desc *desc, const hipq_moe_ext *ext, con
       a.epi.down_bias = (const float *)(base + o_bd);
     }
   }
-  if ((rc = stage_copy(true, base + o_x, (void *)x, H * 4, H * 4, T, s))) return rc;
   /* logits [T x E] or the router weight [H x E] */
-  if ((rc = stage_copy(true, base + o_r, (void *)(router_logits ? router_logits : router_weight), E * 4, E * 4,
-                       router_logits ? T : H, s)))
-    return rc;
+  if (host_router) {
+    if ((rc = stage_copy(true, base + o_r, (void *)(router_logits ? router_logits : router_weight), E * 4, E * 4,
+                         router_logits ? T : H, s)))
+      return rc;
+    a.router_logits = router_logits ? (const float *)(base + o_r) : nullptr;
+    a.router_weight = router_weight ? (const float *)(base + o_r) : nullptr;
+  } else {
+    a.router_logits = nullptr;
+    a.router_weight = router_weight;
+  }
   a.x = (const float *)(base + o_x);
-  a.router_logits = router_logits ? (const float *)(base + o_r) : nullptr;
-  a.router_weight = router_weight ? (const float *)(base + o_r) : nullptr;
-  a.y = (float *)(base + o_y);
   a.topk_idx = (int32_t *)(base + o_i);
   a.topk_w = (float *)(base + o_w);
+  DirectIO dio;
+  const int64_t h64 = (int64_t)H;
+  if (!topk_idx && !topk_w && dio.begin(s, x, (int64_t)T, h64, h64, 1, &y, &h64, &h64, &rc)) {
+    if ((rc = dio.fetch((float *)(base + o_x), h64))) return rc;
+    a.y = dio.outs[0].dev;
+    if (dio.outs[0].dld != h64) return fail(HIPQ_ERR_RUNTIME, "internal: strided output of a decode step's MoE block");
+    if ((rc = hipq::launch_moe(&a, ws, ws_bytes, dev_views, s))) return rc;
+    return dio.finish();
+  }
+  if (rc) return rc;
+  if ((rc = stage_copy(true, base + o_x, (void *)x, H * 4, H * 4, T, s))) return rc;
+  a.y = (float *)(base + o_y);
   if ((rc = hipq::launch_moe(&a, ws, ws_bytes, dev_views, s))) return rc;
   if ((rc = stage_copy(false, base + o_y, y, H * 4, H * 4, T, s))) return rc;
   if (topk_idx && (rc = stage_copy(false, base + o_i, topk_idx, k * 4, k * 4, T, s))) return rc;

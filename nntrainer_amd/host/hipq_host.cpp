@@ -192,6 +192,23 @@ void device_release(void *p) noexcept {
     hipq_device_free(p);
 }
 
+const float *DeviceMirror::get(const float *host, size_t n) {
+  const uint64_t t = sample_tag(host, (int64_t)(n * sizeof(float)));
+  if (dev && src == host && count == n && tag == t)
+    return dev;
+  drop();
+  dev = device_floats(host, n);
+  src = host;
+  count = n;
+  tag = t;
+  return dev;
+}
+
+void DeviceMirror::drop() noexcept {
+  device_release(dev);
+  dev = nullptr;
+}
+
 void release(hipq_weight_t w) noexcept {
   if (w)
     hipq_weight_destroy(w);
@@ -217,6 +234,7 @@ void moe_forward_resident(const MoeShape &shape, const hipq_weight_t *gate, cons
   ext.down_bias = extras ? extras->down_bias : nullptr;
   ext.limit = extras ? extras->limit : 0.f;
   ext.biases_on_device = extras && extras->biases_on_device ? 1 : 0;
+  ext.router_on_device = extras && extras->router_on_device ? 1 : 0;
   check(hipq_moe_forward_ext(&desc, &ext, gate, up, down, x, nullptr, router_weight, y, nullptr, nullptr,
                              HIPQ_MEM_HOST, nullptr),
         "hipq_moe_forward");

@@ -135,11 +135,30 @@ struct MoeExtras {
   const float *router_bias = nullptr;
   const float *gate_bias = nullptr, *up_bias = nullptr, *down_bias = nullptr;
   bool biases_on_device = false; /* the four pointers above are device copies (device_floats) */
+  bool router_on_device = false; /* router_weight of the call is a device copy */
 };
 
 /** A device copy of n floats the caller owns; freed with device_release. */
 float *device_floats(const float *host, size_t n);
 void device_release(void *p) noexcept;
+
+/** A device copy of a host tensor of floats that follows its source: made at the first get(),
+ *  made again when the source's address, size or sampled content has changed. */
+class DeviceMirror {
+public:
+  DeviceMirror() = default;
+  ~DeviceMirror() { drop(); }
+  DeviceMirror(const DeviceMirror &) = delete;
+  DeviceMirror &operator=(const DeviceMirror &) = delete;
+  const float *get(const float *host, size_t n);
+  void drop() noexcept;
+
+private:
+  float *dev = nullptr;
+  const float *src = nullptr;
+  size_t count = 0;
+  uint64_t tag = 0;
+};
 
 /** A device copy that the caller owns (not entered into a cache): for weights whose host bytes
  *  come and go (virtual tensors), where an address is no identity. */

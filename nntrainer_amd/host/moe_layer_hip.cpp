@@ -157,7 +157,8 @@ void MoELayerHip::run(RunLayerContext &context, const float *x, float *y, unsign
   shape.experts = (int)E;
   shape.topk = (int)topk;
   shape.renormalize = renormalize;
-  const float *router = context.getWeight(gate_idx).getData<float>();
+  /* the router weight stays on the device between steps (1 MB at 2048 x 128) */
+  const float *router = dev_router.get(context.getWeight(gate_idx).getData<float>(), (size_t)hidden * E);
 
   /* a virtual tensor has bytes only between activate() and deactivate() */
   auto with_bytes = [&](unsigned int idx, auto use) {
@@ -170,6 +171,7 @@ void MoELayerHip::run(RunLayerContext &context, const float *x, float *y, unsign
   };
 
   hipq_host::MoeExtras extras;
+  extras.router_on_device = true;
   if (gpt_oss) {
     /* the biases go to the device once, with the weights: [E x I], [E x I], [E x H] gathered from
      * the experts' tensors, and the router's [E]; read() drops them as it drops the weights */
@@ -285,6 +287,7 @@ void MoELayerHip::drop_device_biases() noexcept {
   hipq_host::device_release(dev_bias_down);
   hipq_host::device_release(dev_bias_router);
   dev_bias_gate = dev_bias_up = dev_bias_down = dev_bias_router = nullptr;
+  dev_router.drop();
 }
 
 void MoELayerHip::calcDerivative(RunLayerContext &) {

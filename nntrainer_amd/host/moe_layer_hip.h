@@ -34,6 +34,8 @@
 
 #include <hipq.h>
 
+#include "hipq_host.h"
+
 #include "nntr_api.h"
 
 namespace nntrainer {
@@ -98,6 +100,7 @@ private:
    * step, dropped when the framework reads the layer's weights again */
   float *dev_bias_gate = nullptr, *dev_bias_up = nullptr, *dev_bias_down = nullptr, *dev_bias_router = nullptr;
   void drop_device_biases() noexcept;
+  hipq_host::DeviceMirror dev_router; /* the fp32 router weight [hidden x experts] */
   /* cached: device copies this layer owns, gate | up | down, made at an expert's first use */
   std::vector<hipq_weight_t> resident;
 };

@@ -244,3 +244,43 @@ def test_moe_router_weight_path(hipq, cr):
     assert gu.rel_err(y.cpu().numpy(), ref_y) <= gu.TOL  # logits differ in the last bits only
     for w in wg + wu + wd:
         w.destroy()
+
+
+@pytest.mark.parametrize("t,pinned", [(1, True), (5, True), (8, False), (9, False)])
+def test_moe_decode_step_in_host_memory(hipq, cr, t, pinned):
+    """A decode step's MoE block with x and y in host memory (page-locked: read and written where
+    they lie; pageable: through the stream's staging buffer; nine tokens: through the copy engines):
+    the bits of the device-memory call, with the router weight given in host memory."""
+    import ctypes
+    import gpu_util as gu
+    import torch
+    h, i, e, k = 512, 256, 8, 2
+    gate, up, down = _experts(cr, e, i, h, seed=5200)
+    wg = [capi.Weight("q4_K", i, h, b) for b in gate]
+    wu = [capi.Weight("q4_K", i, h, b) for b in up]
+    wd = [capi.Weight("q4_K", h, i, b) for b in down]
+    x = synth.normal(5300 + t, (t, h))
+    wr = synth.normal(5301, (h, e), 0.1)
+    want = torch.full((t, h), float("nan"), device="cuda")
+    capi.moe_forward(t, h, i, e, k, wg, wu, wd, gu.dev(x), want, router_weight=gu.dev(wr), stream=gu.stream())
+    torch.cuda.synchronize()
+    if pinned:
+        px, py = capi.host_alloc(t * h * 4), capi.host_alloc(t * h * 4)
+        xa = np.ctypeslib.as_array(ctypes.cast(px, ctypes.POINTER(ctypes.c_float)), (t, h))
+        ya = np.ctypeslib.as_array(ctypes.cast(py, ctypes.POINTER(ctypes.c_float)), (t, h))
+        xa[:] = x
+        xin, yout = px, py
+    else:
+        ya = np.full((t, h), np.nan, np.float32)
+        xin, yout = x, ya
+    try:
+        for _ in range(2):
+            ya[:] = np.nan
+            capi.moe_forward(t, h, i, e, k, wg, wu, wd, xin, yout, router_weight=wr, mem=capi.MEM_HOST)
+            assert np.array_equal(ya.view(np.uint32), want.cpu().numpy().view(np.uint32))
+    finally:
+        if pinned:
+            capi.host_free(px)
+            capi.host_free(py)
+        for w in wg + wu + wd:
+            w.destroy()
