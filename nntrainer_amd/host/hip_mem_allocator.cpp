@@ -19,11 +19,17 @@ void HipMemAllocator::alloc(void **ptr, size_t size, size_t /*alignment*/) {
     size = 1; /* the default allocator logs and allocates nothing useful; a valid pointer is kinder */
   if (hipq_host::runtime_available()) {
     void *p = nullptr;
-    hipq_host::check(hipq_host_alloc(&p, size), "hipq_host_alloc");
-    std::lock_guard<std::mutex> lock(mtx);
-    pinned.insert(p);
-    *ptr = p;
-    return;
+    const int rc = hipq_host_alloc(&p, size);
+    if (rc == HIPQ_OK) {
+      std::lock_guard<std::mutex> lock(mtx);
+      pinned.insert(p);
+      *ptr = p;
+      return;
+    }
+    /* a pool larger than the system lets a process page-lock (a multi-GB model): ordinary memory
+     * serves as well, its tensors cross through the library's page-locked staging instead */
+    if (rc != HIPQ_ERR_OUT_OF_MEMORY)
+      hipq_host::check(rc, "hipq_host_alloc");
   }
   *ptr = std::calloc(size, 1);
   if (!*ptr)

@@ -24,8 +24,9 @@ public:
   HipMemAllocator() = default;
   ~HipMemAllocator() override = default;
   /** zero-filled like the default allocator's calloc; `alignment` is met by any page-locked
-   *  allocation (page aligned). Without a usable device the memory is ordinary host memory: the
-   *  framework must still be able to build and inspect a model. */
+   *  allocation (page aligned). Without a usable device, or when the runtime cannot page-lock
+   *  that much, the memory is ordinary host memory: the framework must still be able to build
+   *  and inspect a model, and pageable tensors cross through the library's own staging. */
   void alloc(void **ptr, size_t size, size_t alignment) override;
   void free(void *ptr) override;
   std::string getName() override { return "gpu"; }
