@@ -24,10 +24,11 @@ M, K, N = 512, 4096, 12288
 INT8_PEAK_TOPS = 5000.0  # MI355X dense int8 matrix peak, TOP/s
 HBM_PEAK_GBS = 8000.0    # MI355X HBM3E peak, GB/s
 # HBM bytes per launch from rocprofv3 FETCH_SIZE / WRITE_SIZE counter runs of this script, scaled by
-# what the same counters read for its 256 MiB device copy (profiles/gemm_q4k_prefill_m512_k4096_n12288.txt,
+# what the same counters read for kernels of known size in the same run (a 1 GiB read-only kernel, a 1 GiB
+# fill, its 256 MiB device copies) (profiles/gemm_q4k_prefill_m512_k4096_n12288.txt,
 # profiles/gemv_q4k_decode_m1_k4096.txt, profiles/moe_block_q4k_64tok_128experts.txt). Measured once, not live: counters need the profiler attached.
-TRAFFIC_GEMM_C2 = 49.00e6 + 25.17e6
-TRAFFIC_GEMV_C2 = 28.45e6 + 0.05e6
+TRAFFIC_GEMM_C2 = 49.04e6 + 25.17e6
+TRAFFIC_GEMV_C2 = 28.57e6 + 0.05e6
 TRAFFIC_GEMV_LM_HEAD = 350.25e6 + 0.62e6
 METRIC = "Q4 GEMV effective GB/s (%HBM peak); prefill GEMM int8 TOPS (%MFMA peak)"
 
@@ -791,7 +792,7 @@ def main():
                          "achieved": round(2.0 * 512 * 151936 * 4096 / (c3_prefill[0] * 1e-3) / 1e12, 3),
                          "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
                          "frac": round(2.0 * 512 * 151936 * 4096 / (c3_prefill[0] * 1e-3) / 1e12 / INT8_PEAK_TOPS, 5),
-                         "kernel_ms": round(c3_prefill[0], 5), "traffic": 859.6e6 + 325.8e6,
+                         "kernel_ms": round(c3_prefill[0], 5), "traffic": 860.0e6 + 325.8e6,
                          "traffic_from": "profiles/gemm_q6k_prefill_m512_k4096_n151936.txt (counter runs; not live)",
                          "algorithmic_ops_per_launch": 2.0 * 512 * 151936 * 4096}},
         "c5_fc_stack_per_layer": {
@@ -840,7 +841,7 @@ def main():
                          "frac": round(moe_gbs / HBM_PEAK_GBS, 5),
                          "frac_of_measured_read_ceiling": round(moe_gbs / read_ceiling_gbs, 5),
                          "algorithmic_bytes_per_block": moe_bytes,
-                         "traffic": 235.9e6 + 134.3e6 + 12.0e6},
+                         "traffic": 232.4e6 + 133.0e6 + 11.4e6},
             "decode_token": {"ms_per_block": round(moe_decode_ms, 5),
                              "ms_per_block_in_a_graph": round(moe_decode_graph_ms, 5),
                              "active_experts": decode_active,
