@@ -20,7 +20,12 @@
  * Memory: `mem` says where the caller's buffers live. HIPQ_MEM_DEVICE buffers are
  * device pointers; the call only enqueues work on `stream` and returns.
  * HIPQ_MEM_HOST buffers are ordinary host memory; the call copies in, runs,
- * copies out and returns when the result is in the host buffer.
+ * copies out and returns when the result is in the host buffer. A call of a
+ * few rows (a decode step: up to eight rows, at most 1 MiB of outputs) uses no
+ * copy engine: a kernel reads the rows from page-locked memory (memory of
+ * hipq_host_alloc as it is, other memory through a page-locked staging buffer),
+ * the product kernels write the outputs there, and the call returns when the
+ * last kernel has set a flag in page-locked memory.
  * `stream` is a hipStream_t passed as void* (NULL = the default stream).
  */
 #ifndef HIPQ_H
