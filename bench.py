@@ -151,6 +151,29 @@ def cpu_gemv_baseline(kind, n, k, host, nbytes, budget_s=4.0):
             "gpu_output_bit_identical": bool(np.array_equal(gpu_out.view(np.uint32), c.view(np.uint32)))}
 
 
+def plugin_c5_layer():
+    """The quantized FCs of one C5 decoder layer through libnntrainer_hip_context.so (layers created by the
+    context's factories, run with incremental_forwarding on host tensors): microseconds per layer."""
+    import subprocess
+    lib = os.path.join(ROOT, "nntrainer_amd", "lib")
+    exe, plugin = os.path.join(lib, "hipq_host_selftest"), os.path.join(lib, "libnntrainer_hip_context.so")
+    if not (os.path.exists(exe) and os.path.exists(plugin)):
+        return {"skipped": "the plug-in is not built (python -c 'import __graft_entry__ as g; g.build()')"}
+    try:
+        r = subprocess.run([exe, plugin, "c5layer", "200"], capture_output=True, text=True, timeout=180)
+        if r.returncode != 0:
+            return {"failed": (r.stdout + r.stderr)[-300:]}
+        res = json.loads(r.stdout.strip().splitlines()[-1])
+    except Exception as e:  # the bench line must still be printed
+        return {"failed": repr(e)[:300]}
+    res["workload"] = ("one Qwen3-0.6B-shaped decoder layer (BASELINE configs[4]), Q4_0 weights, through the context "
+                       "plug-in: layers from its factories, incremental_forwarding on host tensors, every call "
+                       "synchronous; as the seven fully_connected layers of an unchanged graph and as qkv_layer + "
+                       "fully_connected + mlp_swiglu + fully_connected; tensors in ordinary memory and in memory of the "
+                       "context's allocator (page-locked); one decode row, and a prefill of 512 rows; wall clock per layer")
+    return res
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -160,6 +183,10 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no multi-GPU part (run with --gpus 1)")
+
+    # ---- a C5 decoder layer's FCs through the framework plug-in (the layer API, host tensors, every
+    # call synchronous): the plug-in's own driver as a child process, before this process touches the GPU
+    plugin_layer = plugin_c5_layer()
 
     import numpy as np
     import torch
@@ -831,6 +858,7 @@ def main():
                                  "frac": round(450971566080 / (c5_model_prefill_ms * 1e-3) / 1e12 / INT8_PEAK_TOPS, 5),
                                  "algorithmic_ops": 450971566080,
                                  "note": "the lm_head row's time is inside the figure, its ops are not"}},
+        "c5_layer_through_plugin": plugin_layer,
         "moe_block": {
             "workload": "MoE FFN block (BASELINE configs[3]): 64 tokens, hidden 2048, 128 experts x "
                         "(gate/up 2048->768, down 768->2048) Q4_K, top-8; router, sort, experts, combine; "

@@ -32,10 +32,18 @@
  *   lmhead <dtype> <K> <unit> <batch> <height> <from> <to> <table> <input> <out>
  *   embed <dtype> <in_dim> <out_dim> <batch> <width> <from> <to> <table> <ids> <out>
  *                            tie_word_embeddings in its two modes
+ *   c5layer <iterations>     times the quantized FCs of one Qwen3-0.6B-shaped decoder layer (hidden 1024,
+ *                            Q 2048, K and V 1024, feed-forward 3072, Q4_0) through the layer API, every call
+ *                            synchronous on host tensors as the framework makes it: as seven fully_connected
+ *                            layers (what an unchanged graph gives) and as qkv_layer + fully_connected +
+ *                            mlp_swiglu + fully_connected; one decode row and a prefill of 512 rows; tensors in
+ *                            ordinary memory and in memory of the context's allocator. Prints one JSON object.
+ *                            Weights are pseudo-random blocks: the mode measures time, the other modes results.
  * The test suite compares the written outputs with expected values it computes itself.
  */
 #include <dlfcn.h>
 
+#include <chrono>
 #include <cstdio>
 #include <cstdlib>
 #include <fstream>
@@ -513,14 +521,124 @@ static int run_tie(Context *ctx, bool lmhead, char **a) {
   return 0;
 }
 
+/* ---- c5layer ------------------------------------------------------------------------- */
+namespace {
+struct BuiltLayer {
+  std::unique_ptr<Layer> layer;
+  std::unique_ptr<InitLayerContext> ic;
+  std::unique_ptr<RunLayerContext> rc;
+  unsigned n_out = 1;
+};
+
+/* x8-repacked Q4_0 as the layer's weight tensor holds it: groups of 144 bytes, eight fp16 scales
+ * (2^-8 here), then 128 bytes of nibbles */
+void fill_q4_0x8(uint8_t *p, size_t bytes, uint32_t seed) {
+  uint32_t x = seed * 2654435761u + 12345u;
+  for (size_t g = 0; g + 144 <= bytes; g += 144) {
+    for (int i = 0; i < 8; ++i) {
+      p[g + 2 * i] = 0x00;
+      p[g + 2 * i + 1] = 0x1c;
+    }
+    for (int i = 16; i < 144; ++i) {
+      x = x * 1664525u + 1013904223u;
+      p[g + i] = (uint8_t)(x >> 24);
+    }
+  }
+}
+
+BuiltLayer build(Context *ctx, const std::string &type, const std::vector<std::string> &props, unsigned height,
+                 unsigned K, unsigned n_out, uint32_t seed, const std::shared_ptr<MemAllocator> &ma) {
+  BuiltLayer b;
+  b.layer = ctx->createLayerObject(type, props);
+  b.ic = std::make_unique<InitLayerContext>(std::vector<TensorDim>{TensorDim(1, 1, height, K)}, type, Tformat::NCHW,
+                                            Tdatatype::Q4_0, Tdatatype::FP32);
+  b.layer->finalize(*b.ic);
+  b.rc = std::make_unique<RunLayerContext>(*b.ic);
+  b.n_out = n_out;
+  for (unsigned i = 0; i < b.rc->getNumWeights(); ++i)
+    fill_q4_0x8(b.rc->getWeight(i).getData<uint8_t>(), mirror_tensor_bytes(b.rc->getWeight(i).getDim()), seed + i);
+  float *in = b.rc->getInput(0).getData<float>();
+  for (size_t i = 0; i < (size_t)height * K; ++i)
+    in[i] = (float)((int)((i * 2654435761u) >> 20 & 0xfff) - 2048) / 2048.f;
+  if (ma) { /* activations and outputs in the pool the context's allocator serves */
+    auto place = [&](Tensor &t) {
+      void *p = nullptr;
+      ma->alloc(&p, mirror_tensor_bytes(t.getDim()), 64);
+      t.mirror_move_to(p, [ma](void *q) { ma->free(q); });
+    };
+    place(b.rc->getInput(0));
+    for (unsigned o = 0; o < n_out; ++o)
+      place(b.rc->getOutput(o));
+  }
+  return b;
+}
+
+double time_chain(std::vector<BuiltLayer> &chain, bool decode, int iters) {
+  auto once = [&]() {
+    for (auto &b : chain) {
+      if (decode)
+        b.layer->incremental_forwarding(*b.rc, 3, 4, false);
+      else
+        b.layer->incremental_forwarding(*b.rc, 0, b.rc->getInput(0).height(), false);
+    }
+  };
+  for (int i = 0; i < 3; ++i)
+    once();
+  const auto t0 = std::chrono::steady_clock::now();
+  for (int i = 0; i < iters; ++i)
+    once();
+  const auto t1 = std::chrono::steady_clock::now();
+  return std::chrono::duration<double, std::micro>(t1 - t0).count() / iters;
+}
+} // namespace
+
+static int run_c5layer(Context *ctx, int iters) {
+  const unsigned D = 1024, NQ = 2048, NKV = 1024, FF = 3072;
+  auto ma = ctx->getContextData() ? ctx->getContextData()->getMemAllocator() : nullptr;
+  auto unit = [](unsigned n) { return std::vector<std::string>{"unit=" + std::to_string(n), "disable_bias=true"}; };
+  std::printf("{");
+  bool first = true;
+  for (int pinned = 0; pinned < 2; ++pinned) {
+    for (int decode = 1; decode >= 0; --decode) {
+      const unsigned h = decode ? 8 : 512;
+      const auto mem = pinned ? ma : std::shared_ptr<MemAllocator>();
+      std::vector<BuiltLayer> seven, four;
+      seven.push_back(build(ctx, "fully_connected", unit(NQ), h, D, 1, 1, mem));
+      seven.push_back(build(ctx, "fully_connected", unit(NKV), h, D, 1, 2, mem));
+      seven.push_back(build(ctx, "fully_connected", unit(NKV), h, D, 1, 3, mem));
+      seven.push_back(build(ctx, "fully_connected", unit(D), h, NQ, 1, 4, mem));
+      seven.push_back(build(ctx, "fully_connected", unit(FF), h, D, 1, 5, mem));
+      seven.push_back(build(ctx, "fully_connected", unit(FF), h, D, 1, 6, mem));
+      seven.push_back(build(ctx, "fully_connected", unit(D), h, FF, 1, 7, mem));
+      four.push_back(build(ctx, "qkv_layer",
+                           {"q_unit=" + std::to_string(NQ), "k_unit=" + std::to_string(NKV),
+                            "v_unit=" + std::to_string(NKV)},
+                           h, D, 3, 11, mem));
+      four.push_back(build(ctx, "fully_connected", unit(D), h, NQ, 1, 14, mem));
+      four.push_back(build(ctx, "mlp_swiglu", unit(FF), h, D, 1, 15, mem));
+      four.push_back(build(ctx, "fully_connected", unit(D), h, FF, 1, 17, mem));
+      const int n = decode ? iters : (iters + 9) / 10;
+      const double t7 = time_chain(seven, decode, n), t4 = time_chain(four, decode, n);
+      std::printf("%s\"%s_%s_seven_fully_connected_us\": %.2f, \"%s_%s_qkv_fc_mlp_swiglu_fc_us\": %.2f", first ? "" : ", ",
+                  decode ? "decode_row" : "prefill_512_rows", pinned ? "allocator_memory" : "ordinary_memory", t7,
+                  decode ? "decode_row" : "prefill_512_rows", pinned ? "allocator_memory" : "ordinary_memory", t4);
+      first = false;
+    }
+  }
+  std::printf("}\n");
+  return 0;
+}
+
 int main(int argc, char **argv) {
   if (argc < 3) {
-    std::printf("usage: %s <plugin.so> api | fc ... | moe ...\n", argv[0]);
+    std::printf("usage: %s <plugin.so> api | c5layer <iterations> | fc ... | moe ...\n", argv[0]);
     return 2;
   }
   try {
     Context *ctx = load_context(argv[1]);
     const std::string mode = argv[2];
+    if (mode == "c5layer" && argc == 4)
+      return run_c5layer(ctx, std::atoi(argv[3]));
     if (mode == "api")
       return run_api(ctx);
     if (mode == "fc" && argc == 14)

@@ -149,6 +149,31 @@ inline size_t mirror_tensor_bytes(const TensorDim &d) {
 /** where a layer's weights are read from (nntrainer/utils/util_func.h:43) */
 using ReadSource = std::variant<std::ifstream *, const char *>;
 
+/** The bytes of a tensor: the stand-in's own memory, or memory that a driver took from a
+ *  MemAllocator, as the framework hands a context's allocator to its memory pool (engine.h:82-84,
+ *  tensor/memory_pool.h:110). */
+class MirrorBytes {
+public:
+  explicit MirrorBytes(size_t n) : own(n), p(own.data()), n(n) {}
+  explicit MirrorBytes(const std::vector<uint8_t> &v) : own(v), p(own.data()), n(own.size()) {}
+  MirrorBytes(void *external, size_t n, std::function<void(void *)> release) :
+    p(static_cast<uint8_t *>(external)), n(n), release(std::move(release)) {}
+  MirrorBytes(const MirrorBytes &) = delete;
+  MirrorBytes &operator=(const MirrorBytes &) = delete;
+  ~MirrorBytes() {
+    if (release)
+      release(p);
+  }
+  uint8_t *data() { return p; }
+  size_t size() const { return n; }
+
+private:
+  std::vector<uint8_t> own;
+  uint8_t *p;
+  size_t n;
+  std::function<void(void *)> release;
+};
+
 /** Host tensor: a view (offset + dims) into shared storage. */
 class Tensor {
 public:
@@ -167,7 +192,15 @@ public:
   }
 
   Tensor() = default;
-  explicit Tensor(const TensorDim &d) : dim(d), store(std::make_shared<std::vector<uint8_t>>(mirror_tensor_bytes(d))) {}
+  explicit Tensor(const TensorDim &d) : dim(d), store(std::make_shared<MirrorBytes>(mirror_tensor_bytes(d))) {}
+  /** moves the tensor's bytes into `external` (of at least its size), released through `release` with the last view */
+  void mirror_move_to(void *external, std::function<void(void *)> release) {
+    const size_t n = mirror_tensor_bytes(dim);
+    if (store)
+      std::memcpy(external, getData<uint8_t>(), n);
+    store = std::make_shared<MirrorBytes>(external, n, std::move(release));
+    offset_bytes = 0;
+  }
   /** a virtual tensor (requestWeight(..., is_virtual = true)): its bytes live in the model file
    *  until activate() maps them in and are gone again after deactivate() (tensor.h:1979-1993).
    *  Here the "file" is a second buffer that a test fills through mirror_file_bytes(). */
@@ -180,7 +213,7 @@ public:
   }
   void activate() {
     if (is_virtual && !store)
-      store = std::make_shared<std::vector<uint8_t>>(*file);
+      store = std::make_shared<MirrorBytes>(*file);
   }
   void deactivate() {
     if (is_virtual)
@@ -242,7 +275,7 @@ public:
 
 private:
   TensorDim dim;
-  std::shared_ptr<std::vector<uint8_t>> store;
+  std::shared_ptr<MirrorBytes> store;
   size_t offset_bytes = 0;
   bool is_virtual = false;
   std::shared_ptr<std::vector<uint8_t>> file;
