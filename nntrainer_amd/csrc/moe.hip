@@ -28,7 +28,9 @@
  * Q4_K experts whose rows fit the LDS run on the matrix cores, 8 to 32 tokens of
  * an expert per work item; the other formats and longer rows use the decode
  * GEMV's engine, four tokens per pass over an expert's weights. Both carry the
- * reference's bits for every single-row product.
+ * reference's bits for every single-row product. Chunks of 17 to a few dozen tokens
+ * over many experts take a form without the sort (gate_up_self_kernel below): four
+ * launches, one workgroup row per expert.
  */
 #include "gemv_device.h"
 #include "quantize_device.h"
@@ -48,6 +50,7 @@ struct MoeBufs {
   float *h;       /* [P][I] by slot */
   float *contrib; /* [P][H] by slot */
   void *xq_mem, *hq_mem;
+  const int32_t *idx_used = nullptr; /* where this call's routing wrote the expert ids */
 };
 
 size_t up256(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -108,7 +111,7 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const float *__restr
 /* Routing of token t by one wavefront: softmax, top-k, optional renormalisation. */
 template <int MAXV> /* logits per lane: E <= 64 * MAXV */
 __device__ __forceinline__ void route_token(const float *__restrict__ logits, int t, int E, int topk,
-                                            int renorm, int32_t *idx, float *wgt) {
+                                            int renorm, int32_t *idx, float *wgt, int *by_expert = nullptr) {
   const int lane = threadIdx.x & 63;
   float p[MAXV];
   const float *lg = logits + (size_t)t * E;
@@ -181,6 +184,13 @@ __device__ __forceinline__ void route_token(const float *__restrict__ logits, in
       myw = bv;
       myi = bi;
     }
+  }
+  if (by_expert) {
+    /* the token's pairs in ascending expert id, the order in which its contributions are added
+     * (tok_slots, for the forms that number the rows of h by pair instead of by sorted slot) */
+    int r = 0;
+    for (int j = 0; j < topk; ++j) r += __shfl(myi, j, 64) < myi;
+    if (lane < topk) by_expert[(size_t)t * topk + r] = t * topk + lane;
   }
   if (lane < topk) {
     idx[(size_t)t * topk + lane] = myi;
@@ -322,14 +332,14 @@ template <int MAXV>
 __global__ __launch_bounds__(256) void route_quantize_kernel(const float *__restrict__ logits, int T, int E,
                                                              int topk, int renorm, int32_t *__restrict__ idx,
                                                              float *__restrict__ wgt, int route_blocks,
-                                                             XQuant xq) {
+                                                             XQuant xq, int *__restrict__ by_expert) {
   if ((int)blockIdx.x >= route_blocks) {
     quantize_x(xq, T, blockIdx.x - route_blocks);
     return;
   }
   const int t = blockIdx.x * 4 + (threadIdx.x >> 6);
   if (t >= T) return; /* uniform per wavefront */
-  route_token<MAXV>(logits, t, E, topk, renorm, idx, wgt);
+  route_token<MAXV>(logits, t, E, topk, renorm, idx, wgt, by_expert);
 }
 
 template <int MAXV>
@@ -606,6 +616,7 @@ struct XLds {
   uint8_t *amin; /* [TC][nsb][32 bytes] */
   float *dA;     /* [nsb][TC] */
   int *rows;     /* [TC] source rows of the item */
+  int *pairs;    /* the item's (token, k) pairs, where the workgroup finds them itself (the forms without a sort) */
 };
 __host__ __device__ inline size_t xlds_bytes(int TC, int K) {
   const size_t b = (size_t)TC * (K + 16) + (size_t)TC * (K / 256) * 32 + (size_t)TC * (K / 256) * 4 + TC * 4;
@@ -617,6 +628,7 @@ __device__ __forceinline__ XLds xlds_carve(unsigned char *base, int TC, int K) {
   l.amin = (uint8_t *)base + (size_t)TC * (K + 16);
   l.dA = (float *)(l.amin + (size_t)TC * (K / 256) * 32);
   l.rows = (int *)(l.dA + (size_t)TC * (K / 256));
+  l.pairs = nullptr;
   return l;
 }
 
@@ -950,6 +962,194 @@ __global__ __launch_bounds__(256, TC <= 8 ? 4 : TC <= 16 ? 2 : 1) void down_mma_
     stage);
 }
 
+/* ---- The block without a pair sort ------------------------------------------------------
+ * For chunks of a few dozen tokens the sort is a launch of its own (4-5 us of a block of 80) and
+ * puts three dependent reads (item, offsets, pairs) in front of every workgroup's first weight
+ * load. Here a workgroup is given (expert, chunk of 16 of its pairs) by its block id and finds the
+ * pairs itself in the routing's idx[P] (a few KB: every thread compares its share, ranks by pair
+ * number come from a prefix sum over the workgroup). Rows of h and of the contributions are
+ * numbered by pair, and the routing writes each token's pairs in ascending expert id for the
+ * combine. An expert with up to 8 pairs runs the 8-row form of the matrix step, one with 9 to 16
+ * the 16-row form, so either is ONE workgroup per column block: its weights cross HBM once and the
+ * number of streaming workgroups is the number of active experts whatever the routing (with 128
+ * experts and 768 intermediate columns exactly three on every CU). Experts with more than 16 pairs
+ * continue in the next row of the grid (blockIdx.y / E); rows whose chunk is empty leave after the
+ * scan. */
+constexpr int SELF_TC = 16;     /* pairs per chunk */
+constexpr int SELF_HEAD = 128;  /* bytes of LDS in front of the rows: pairs[16], tokens[16] */
+
+__device__ __forceinline__ int self_scan(const int32_t *__restrict__ idx, int P, int topk, int e, int chunk,
+                                         int *pairs, int *rows) {
+  __shared__ int wtot[4];
+  const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
+  const int pp = (P + 255) >> 8; /* pairs per thread, consecutive: thread order is pair order */
+  int m = 0;
+  uint32_t mask = 0;
+  for (int u = 0; u < pp; ++u) {
+    const int i = t * pp + u;
+    if (i < P && idx[i] == e) mask |= 1u << u, ++m;
+  }
+  int inc = m;
+#pragma unroll
+  for (int d = 1; d < 64; d <<= 1) {
+    const int v = __shfl_up(inc, d, 64);
+    if (lane >= d) inc += v;
+  }
+  if (lane == 63) wtot[wave] = inc;
+  __syncthreads();
+  int base = 0, total = 0;
+#pragma unroll
+  for (int w = 0; w < 4; ++w) {
+    base += w < wave ? wtot[w] : 0;
+    total += wtot[w];
+  }
+  int r = base + inc - m - chunk * SELF_TC;
+  for (int u = 0; u < pp; ++u)
+    if (mask >> u & 1) {
+      if (r >= 0 && r < SELF_TC) {
+        pairs[r] = t * pp + u;
+        rows[r] = (t * pp + u) / topk;
+      }
+      ++r;
+    }
+  __syncthreads();
+  return total;
+}
+
+template <int TC>
+__device__ __forceinline__ void gate_up_self_pass(unsigned char *lds, int n, int e, const WView *__restrict__ views,
+                                                  int E_, const QView &xq, int I, float *__restrict__ h,
+                                                  const hipq::MoeEpi &ep) {
+  constexpr int NREG = TC / 2;
+  const WView wg = views[e], wu = views[E_ + e];
+  const int K = wg.K;
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
+  XLds l = xlds_carve(lds + SELF_HEAD, TC, K);
+  l.pairs = (int *)lds;
+  l.rows = l.pairs + SELF_TC;
+  const int col0 = (blockIdx.x * 4 + wave) * 32;
+  const uint64_t dqs = (uint64_t)wu.qs - (uint64_t)wg.qs;
+  auto stage = [&]() {
+    stage_rows<TC>(l, xq, n);
+    __syncthreads();
+  };
+  if (col0 >= I) { /* uniform per wavefront; it still takes part in the barrier */
+    stage();
+    return;
+  }
+  float gate[NREG], up[NREG];
+  xr_run<TC, NREG, XPD>(
+    2, l, K,
+    [&](int t, WView &w, int &c0) {
+      const uint64_t isup = (uint64_t)0 - (uint64_t)(t & 1);
+      w.qs = (const uint8_t *)((uint64_t)wg.qs + (isup & dqs));
+      w.hdr = nullptr; /* the headers follow the nibbles */
+      w.N = wg.N;
+      w.K = wg.K;
+      c0 = col0;
+    },
+    [&](int t, const float(&out)[NREG]) {
+      if (t == 0) {
+#pragma unroll
+        for (int r = 0; r < NREG; ++r) gate[r] = out[r];
+      } else {
+#pragma unroll
+        for (int r = 0; r < NREG; ++r) up[r] = out[r];
+      }
+    },
+    stage);
+  const int col = col0 + (lane & 31);
+#pragma unroll
+  for (int r = 0; r < NREG; ++r) {
+    const int tok = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+    if (col < I && tok < n) h[(size_t)l.pairs[tok] * I + col] = moe_act(ep, e, I, col, gate[r], up[r]);
+  }
+}
+
+__global__ __launch_bounds__(256, 4) void gate_up_self_kernel(const WView *__restrict__ views, int E_, QView xq,
+                                                              const int32_t *__restrict__ idx, int P, int topk, int I,
+                                                              float *__restrict__ h, hipq::MoeEpi ep) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char xmoe_lds[];
+  const int e = blockIdx.y % E_, chunk = blockIdx.y / E_;
+  int *pairs = (int *)xmoe_lds;
+  const int total = self_scan(idx, P, topk, e, chunk, pairs, pairs + SELF_TC);
+  const int n = min(SELF_TC, total - chunk * SELF_TC);
+  if (n <= 0) return; /* uniform per workgroup */
+  if (n <= 8)
+    gate_up_self_pass<8>(xmoe_lds, n, e, views, E_, xq, I, h, ep);
+  else
+    gate_up_self_pass<16>(xmoe_lds, n, e, views, E_, xq, I, h, ep);
+}
+
+/* The rows of h come as fp32 and the workgroup quantizes those of its chunk itself while its first
+ * weights are on their way (the QH form of down_mma_kernel). */
+template <int TC>
+__device__ __forceinline__ void down_self_pass(unsigned char *lds, int n, int e, const WView *__restrict__ views,
+                                               int E_, const float *__restrict__ hf, const float *__restrict__ wgt,
+                                               int H, float *__restrict__ contrib, const hipq::MoeEpi &ep) {
+  constexpr int NREG = TC / 2, CT = 2;
+  const WView wd = views[2 * E_ + e];
+  const int K = wd.K;
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
+  XLds l = xlds_carve(lds + SELF_HEAD, TC, K);
+  l.pairs = (int *)lds;
+  l.rows = l.pairs + SELF_TC;
+  const int col0 = (blockIdx.x * 4 + wave) * 32 * CT;
+  const int ntile = min(CT, (H - col0 + 31) / 32);
+  auto stage = [&]() {
+    /* rows past the chunk's end stay as they are: a row of the matrix product depends on its own
+     * activations only, and those rows are not stored */
+    const int nsb = K >> 8;
+    for (int u = wave; u < n * nsb; u += 4) { /* uniform per wavefront */
+      const int r = u / nsb, b = u - r * nsb;
+      const float4 xv = *(const float4 *)(hf + (size_t)l.pairs[r] * K + b * 256 + lane * 4);
+      hipq_quantize_q8_K_values<Q8K_ROWMMA>(xv, 0, b, b, nsb, 0, l.q + (size_t)r * (K + 16), l.dA + r, nullptr,
+                                            nullptr, (uint16_t *)(l.amin + (size_t)r * nsb * 32), nullptr, nullptr,
+                                            TC);
+    }
+    __syncthreads();
+  };
+  if (ntile <= 0) {
+    stage();
+    return;
+  }
+  xr_run<TC, NREG, XPD>(
+    ntile, l, K,
+    [&](int t, WView &w, int &c0) {
+      w = wd;
+      c0 = col0 + 32 * t;
+    },
+    [&](int t, const float(&out)[NREG]) {
+      const int col = col0 + 32 * t + (lane & 31);
+#pragma unroll
+      for (int r = 0; r < NREG; ++r) {
+        const int tok = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+        if (col < H && tok < n) {
+          const int pair = l.pairs[tok];
+          contrib[(size_t)pair * H + col] = moe_out(ep, e, H, col, out[r], wgt[pair]);
+        }
+      }
+    },
+    stage);
+}
+
+__global__ __launch_bounds__(256, 4) void down_self_kernel(const WView *__restrict__ views, int E_,
+                                                           const float *__restrict__ hf,
+                                                           const int32_t *__restrict__ idx, int P, int topk,
+                                                           const float *__restrict__ wgt, int H,
+                                                           float *__restrict__ contrib, hipq::MoeEpi ep) {
+  extern __shared__ __attribute__((aligned(16))) unsigned char xmoe_lds[];
+  const int e = blockIdx.y % E_, chunk = blockIdx.y / E_;
+  int *pairs = (int *)xmoe_lds;
+  const int total = self_scan(idx, P, topk, e, chunk, pairs, pairs + SELF_TC);
+  const int n = min(SELF_TC, total - chunk * SELF_TC);
+  if (n <= 0) return; /* uniform per workgroup */
+  if (n <= 8)
+    down_self_pass<8>(xmoe_lds, n, e, views, E_, hf, wgt, H, contrib, ep);
+  else
+    down_self_pass<16>(xmoe_lds, n, e, views, E_, hf, wgt, H, contrib, ep);
+}
+
 /* y[t][c] = sum of the token's contributions, ascending expert id */
 __global__ __launch_bounds__(256) void combine_kernel(const int *__restrict__ tok_slots, int topk,
                                                       int H, const float *__restrict__ contrib,
@@ -1045,6 +1245,39 @@ template <int DT> struct DownLauncher {
 
 constexpr size_t XLDS_MAX = 160 * 1024; /* LDS of a CU */
 
+/* Few work items: halve the gate/up stream of a wavefront and give the down product
+ * one column tile per wavefront instead of two (its rows are short), so that more
+ * wavefronts share the weights' bytes. */
+bool mma_few(const hipq_moe_desc &d, int TC) {
+  const int64_t P = (int64_t)d.tokens * d.topk;
+  const int64_t max_items = (P < d.experts ? P : d.experts) + P / TC;
+  return max_items * ((d.intermediate + 127) / 128) * 4 <= 2048;
+}
+/* The block without a pair sort: the regime of 8-token chunks (a mean expert has at most four
+ * pairs), more tokens than the one-launch routing and sort of a decode step takes, an idx[] that
+ * a workgroup scans in one go, and rows short enough that four workgroups of the 16-row form fit
+ * a CU's LDS. */
+bool mma_self(const hipq_moe_desc &d, int TC) {
+  const int64_t P = (int64_t)d.tokens * d.topk;
+  const int kmax = d.hidden > d.intermediate ? d.hidden : d.intermediate;
+  return TC == 8 && !mma_few(d, TC) && d.tokens > 16 && P <= 1024 && d.topk <= 64 &&
+         4 * (SELF_HEAD + xlds_bytes(SELF_TC, kmax)) <= XLDS_MAX;
+}
+int launch_self_mma(const hipq::MoeArgs *a, const MoeBufs &b, const WView *views, const QAct &xq, hipStream_t s) {
+  const hipq_moe_desc &d = a->desc;
+  const int P = d.tokens * d.topk;
+  const unsigned gy = (unsigned)(((d.tokens + SELF_TC - 1) / SELF_TC) * d.experts); /* an expert has at most T pairs */
+  const size_t lds_g = SELF_HEAD + xlds_bytes(SELF_TC, d.hidden), lds_d = SELF_HEAD + xlds_bytes(SELF_TC, d.intermediate);
+  hipq::launch_kernel("gate_up_self_kernel", gate_up_self_kernel, dim3((d.intermediate + 127) / 128, gy), dim3(256), lds_g, s,
+                      views, d.experts, qview(xq), b.idx_used, P, d.topk, d.intermediate, b.h, a->epi);
+  HIPQ_HIP(hipGetLastError());
+  hipq::launch_kernel("down_self_kernel", down_self_kernel, dim3((d.hidden + 255) / 256, gy), dim3(256), lds_d, s, views,
+                      d.experts, (const float *)b.h, b.idx_used, P, d.topk, (const float *)b.wgt, d.hidden, b.contrib,
+                      a->epi);
+  HIPQ_HIP(hipGetLastError());
+  return HIPQ_OK;
+}
+
 template <int TC>
 int launch_grouped_mma(const hipq::MoeArgs *a, const MoeBufs &b, const WView *views, const QAct &xq,
                        const QAct &hq, hipStream_t s) {
@@ -1052,10 +1285,7 @@ int launch_grouped_mma(const hipq::MoeArgs *a, const MoeBufs &b, const WView *vi
   const int64_t P = (int64_t)d.tokens * d.topk;
   /* an upper bound of the work items: one per active expert and one per full chunk */
   const int max_items = (int)((P < d.experts ? P : d.experts) + P / TC);
-  /* Few work items: halve the gate/up stream of a wavefront and give the down product
-   * one column tile per wavefront instead of two (its rows are short), so that more
-   * wavefronts share the weights' bytes. */
-  const bool few = (int64_t)max_items * ((d.intermediate + 127) / 128) * 4 <= 2048;
+  const bool few = mma_few(d, TC);
   const size_t lds_g = xlds_bytes(TC, d.hidden) + (few ? TC * 256 : 0);
   const size_t lds_d = xlds_bytes(TC, d.intermediate);
   const void *kg = few ? (const void *)gate_up_mma_kernel<TC, true> : (const void *)gate_up_mma_kernel<TC, false>;
@@ -1164,6 +1394,8 @@ int launch_moe(const MoeArgs *a, void *workspace, size_t workspace_bytes, const 
   int32_t *idx = a->topk_idx ? a->topk_idx : b.idx;
   float *wgt = a->topk_w ? a->topk_w : b.wgt;
   b.wgt = wgt;
+  b.idx_used = idx;
+  const bool self = mma && mma_self(d, chunk); /* no pair sort: the expert kernels find their pairs in idx */
   /* the router is instantiated for 2, 4 and 16 logits per lane (E <= 128, 256, 1024):
    * a short kernel whose code is mostly fetched cold, so its length is its time.
    * For the matrix-core expert kernels the same launch quantizes x. */
@@ -1192,7 +1424,7 @@ int launch_moe(const MoeArgs *a, void *workspace, size_t workspace_bytes, const 
     auto launch = [&](auto fused, auto plain) {
       if (mma)
         hipq::launch_kernel("fused", fused, dim3(rblocks + qblocks), dim3(256), 0, s, logits, T, E, d.topk, d.renormalize,
-                           idx, wgt, rblocks, xqa);
+                           idx, wgt, rblocks, xqa, self ? b.tok_slots : (int *)nullptr);
       else
         hipq::launch_kernel("plain", plain, dim3(rblocks), dim3(256), 0, s, logits, T, E, d.topk, d.renormalize, idx, wgt);
     };
@@ -1201,8 +1433,8 @@ int launch_moe(const MoeArgs *a, void *workspace, size_t workspace_bytes, const 
     else launch(route_quantize_kernel<16>, route_kernel<16>);
     HIPQ_HIP(hipGetLastError());
   }
-  if (T <= 16 && E <= 1024) {
-    /* routed and sorted above */
+  if ((T <= 16 && E <= 1024) || self) {
+    /* routed and sorted above, or no sort needed */
   } else if (P <= 16384 && E <= 1024) {
     hipq::launch_kernel("sort_pairs_kernel", sort_pairs_kernel, dim3(1), dim3(1024), 0, s, idx, P, E, d.topk, b.offsets,
                        b.slot_pair, b.tok_slots, chunk, b.items);
@@ -1219,7 +1451,9 @@ int launch_moe(const MoeArgs *a, void *workspace, size_t workspace_bytes, const 
            : is_k ? launch_quantize_q8_K(a->x, T, d.hidden, d.hidden, 0, &xq, nullptr, s)
                   : launch_quantize_q8_0(a->x, T, d.hidden, d.hidden, &xq, nullptr, s);
   if (rc) return rc;
-  if (mma) {
+  if (self) {
+    rc = launch_self_mma(a, b, views, xq, s);
+  } else if (mma) {
     const int tc = chunk;
     rc = tc == 8    ? launch_grouped_mma<8>(a, b, views, xq, hq, s)
          : tc == 16 ? launch_grouped_mma<16>(a, b, views, xq, hq, s)

@@ -129,6 +129,41 @@ def test_moe_skewed_routing(hipq, cr, t, h, i, e, k):
         w.destroy()
 
 
+def test_moe_block_without_a_pair_sort_with_crowded_experts(hipq, cr):
+    """40 tokens over 48 experts, 1024 intermediate columns: the regime in which the expert kernels
+    find their pairs in the routing's output themselves. Expert 0 is chosen by every token (three
+    chunks of 16, 16 and 8 pairs: the later rows of the grid), expert 1 by the first twelve (one
+    chunk in the 16-row form), the others by a few (the 8-row form) or by none."""
+    import gpu_util as gu
+    import torch
+    t, h, i, e, k = 40, 256, 1024, 48, 4
+    gate, up, down = _experts(cr, e, i, h, seed=8000)
+    x = synth.normal(8100, (t, h))
+    logits = synth.normal(8101, (t, e))
+    logits[:, 0] += 9.0
+    logits[:12, 1] += 8.0
+    logits[:, 40:] -= 20.0  # experts nobody chooses
+    ref_y, ref_idx, ref_w = cr.moe_forward(x, logits, gate, up, down, k)
+    counts = np.bincount(ref_idx.ravel(), minlength=e)
+    assert counts[0] == 40 and 12 <= counts[1] <= 16 and (counts[40:] == 0).all() and (counts[2:40] <= 8).all()
+    wg = [capi.Weight("q4_K", i, h, b) for b in gate]
+    wu = [capi.Weight("q4_K", i, h, b) for b in up]
+    wd = [capi.Weight("q4_K", h, i, b) for b in down]
+    y = torch.full((t, h), float("nan"), device="cuda")
+    idx = torch.zeros((t, k), dtype=torch.int32, device="cuda")
+    for rep in range(2):  # the second call reuses the workspace the first one left
+        y.fill_(float("nan"))
+        capi.moe_forward(t, h, i, e, k, wg, wu, wd, gu.dev(x), y, router_logits=gu.dev(logits), topk_idx=idx,
+                         stream=gu.stream())
+        torch.cuda.synchronize()
+        assert np.array_equal(idx.cpu().numpy(), ref_idx)
+        got = y.cpu().numpy()
+        assert not np.isnan(got).any()
+        assert gu.rel_err(got, ref_y) <= 2e-6, gu.rel_err(got, ref_y)
+    for w in wg + wu + wd:
+        w.destroy()
+
+
 def test_moe_long_chunk_uses_the_multi_kernel_sort(hipq, cr):
     """More than 16384 (token, expert) pairs: the pairs are counted, scanned and
     scattered by separate kernels, which also list the work items."""
