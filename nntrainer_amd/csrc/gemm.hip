@@ -64,10 +64,15 @@ struct SmemQ40 { /* one of the two chunk buffers */
 };
 static_assert(sizeof(SmemQ40) * 2 * 2 <= 160 * 1024, "two workgroups per CU, two buffers each");
 
-__device__ __forceinline__ uint32_t nib_to_s8(uint32_t x) {
-  /* per byte: (nibble value 0..15) - 8 as int8, no carries between bytes */
-  return ((x | 0x80808080u) - 0x08080808u) ^ 0x80808080u;
-}
+/* A weight q - 8 enters the matrix instruction as 16 (q - 8): with bit 3 of every nibble flipped the
+ * nibble IS q - 8 in two's complement, and in the high half of a byte that is the int8 value
+ * 16 (q - 8) - one exclusive-or for eight weights, then a mask for the odd and a shift and a mask
+ * for the even ones (how the reference reads its repacked blocks, nntr_ggml_impl.cpp:3233-3240). The
+ * sums are 16 times too large, exactly (|16 dot| < 2^20), and the weight scales are staged as dw / 16
+ * (a power of two: fl((dw / 16) da) = fl(dw da) / 16 for every fp16 pair of scales), so
+ * fma(float(16 dot), fl(dw da) / 16, acc) has the operands' exact product of the reference's
+ * fma(float(dot), fl(dw da), acc) and rounds to the same bits. */
+constexpr uint32_t HIPQ_MHI = 0xf0f0f0f0u;
 
 /* One chunk of a workgroup's inputs, as loaded (registers of one thread). Every thread takes the
  * same share of the staging, so that no wavefront keeps the others waiting at the barrier. */
@@ -138,16 +143,17 @@ __device__ __forceinline__ void store_chunk(const Chunk &c, SmemQ40 &sm) {
      * elements 0..7 (g = 0) and 16..23 (g = 2), dwords 2, 3 elements 8..15 (g = 1) and 24..31 (g = 3). */
     const int h = t & 1;
     int8_t *dst = sm.b + (t >> 4) * LDS_STRIDE + h * 64 + ((t >> 1) & 7) * 8;
-    *(v2i *)dst = v2i{(int)nib_to_s8(c.x.x & HIPQ_M4), (int)nib_to_s8(c.x.y & HIPQ_M4)};
-    *(v2i *)(dst + 128) = v2i{(int)nib_to_s8((c.x.x >> 4) & HIPQ_M4), (int)nib_to_s8((c.x.y >> 4) & HIPQ_M4)};
+    const uint32_t x0 = c.x.x ^ 0x88888888u, x1 = c.x.y ^ 0x88888888u;
+    *(v2i *)dst = v2i{(int)((x0 << 4) & HIPQ_MHI), (int)((x1 << 4) & HIPQ_MHI)};
+    *(v2i *)(dst + 128) = v2i{(int)(x0 & HIPQ_MHI), (int)(x1 & HIPQ_MHI)};
   }
   const uint32_t s4[4] = {c.sc.x, c.sc.y, c.sc.z, c.sc.w};
   if (t < 32) {
     float f[8];
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      f[2 * i] = hipq_h2f((uint16_t)(s4[i] & 0xffff));
-      f[2 * i + 1] = hipq_h2f((uint16_t)(s4[i] >> 16));
+      f[2 * i] = hipq_h2f((uint16_t)(s4[i] & 0xffff)) * 0.0625f; /* exact: see above */
+      f[2 * i + 1] = hipq_h2f((uint16_t)(s4[i] >> 16)) * 0.0625f;
     }
     float4 *dst = (float4 *)(sm.dw + t * 8);
     dst[0] = float4{f[0], f[1], f[2], f[3]};
