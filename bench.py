@@ -869,7 +869,7 @@ def main():
                          "frac": round(moe_gbs / HBM_PEAK_GBS, 5),
                          "frac_of_measured_read_ceiling": round(moe_gbs / read_ceiling_gbs, 5),
                          "algorithmic_bytes_per_block": moe_bytes,
-                         "traffic": 232.4e6 + 133.0e6 + 11.4e6},
+                         "traffic": 232.4e6 + 133.2e6 + 11.3e6},
             "decode_token": {"ms_per_block": round(moe_decode_ms, 5),
                              "ms_per_block_in_a_graph": round(moe_decode_graph_ms, 5),
                              "active_experts": decode_active,
