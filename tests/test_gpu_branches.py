@@ -111,7 +111,9 @@ def _gpt_oss_case(cr, kind, t, h, i, e, k, seed):
 
 @pytest.mark.parametrize("kind,t,h,i,e,k", [("q4_K", 8, 256, 256, 8, 2), ("q4_K", 64, 512, 256, 16, 4),
                                             ("q4_K", 1, 2048, 768, 16, 4), ("q4_0", 9, 256, 512, 8, 4),
-                                            ("q6_K", 5, 512, 256, 4, 2)])
+                                            ("q6_K", 5, 512, 256, 4, 2),
+                                            # 40 tokens over 48 experts and 1024 columns: the block without a pair sort
+                                            ("q4_K", 40, 256, 1024, 48, 4)])
 def test_gpt_oss_moe_matches_oracle(hipq, cr, kind, t, h, i, e, k):
     """hipq_moe_forward_ext, GPT-OSS variant (gpt_oss_moe_layer.cpp:372-449, 452-568): biased
     projections, swiglu with alpha on (gate, up + 1), biased down projection. The integer and
