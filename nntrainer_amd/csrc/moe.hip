@@ -108,10 +108,11 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const float *__restr
   }
 }
 
-/* Routing of token t by one wavefront: softmax, top-k, optional renormalisation. */
+/* Routing of token t by one wavefront: softmax, top-k, optional renormalisation, into registers:
+ * lane kk < topk ends up with the kk-th choice's expert and weight. */
 template <int MAXV> /* logits per lane: E <= 64 * MAXV */
-__device__ __forceinline__ void route_token(const float *__restrict__ logits, int t, int E, int topk,
-                                            int renorm, int32_t *idx, float *wgt, int *by_expert = nullptr) {
+__device__ __forceinline__ void route_token_regs(const float *__restrict__ logits, int t, int E, int topk,
+                                                 int renorm, int &myi, float &myw) {
   const int lane = threadIdx.x & 63;
   float p[MAXV];
   const float *lg = logits + (size_t)t * E;
@@ -149,8 +150,8 @@ __device__ __forceinline__ void route_token(const float *__restrict__ logits, in
     if (!(p[i] == p[i])) p[i] = 0.f;
   }
   float ksum = 0.f;
-  float myw = 0.f; /* lane kk keeps the kk-th weight */
-  int myi = 0;
+  myw = 0.f; /* lane kk keeps the kk-th weight */
+  myi = 0;
   for (int kk = 0; kk < topk; ++kk) {
     float bv = -2.f;
     int bi = 0x7fffffff;
@@ -185,16 +186,33 @@ __device__ __forceinline__ void route_token(const float *__restrict__ logits, in
       myi = bi;
     }
   }
+  if (renorm) myw = __fdiv_rn(myw, ksum);
+}
+
+/* the rank of lane kk's expert among the token's topk, ascending expert id (lanes below topk) */
+__device__ __forceinline__ int rank_by_expert(int myi, int topk) {
+  int r = 0;
+  for (int j = 0; j < topk; ++j) r += __shfl(myi, j, 64) < myi;
+  return r;
+}
+
+/* ... and written out */
+template <int MAXV>
+__device__ __forceinline__ void route_token(const float *__restrict__ logits, int t, int E, int topk,
+                                            int renorm, int32_t *idx, float *wgt, int *by_expert = nullptr) {
+  const int lane = threadIdx.x & 63;
+  int myi;
+  float myw;
+  route_token_regs<MAXV>(logits, t, E, topk, renorm, myi, myw);
   if (by_expert) {
     /* the token's pairs in ascending expert id, the order in which its contributions are added
      * (tok_slots, for the forms that number the rows of h by pair instead of by sorted slot) */
-    int r = 0;
-    for (int j = 0; j < topk; ++j) r += __shfl(myi, j, 64) < myi;
+    const int r = rank_by_expert(myi, topk);
     if (lane < topk) by_expert[(size_t)t * topk + r] = t * topk + lane;
   }
   if (lane < topk) {
     idx[(size_t)t * topk + lane] = myi;
-    wgt[(size_t)t * topk + lane] = renorm ? __fdiv_rn(myw, ksum) : myw;
+    wgt[(size_t)t * topk + lane] = myw;
   }
 }
 
@@ -899,6 +917,97 @@ __global__ __launch_bounds__(256, TC <= 8 ? 4 : TC <= 16 ? 2 : 1) void gate_up_m
   }
 }
 
+/* One token (a decode step), the routing inside the gate/up launch: every wavefront routes the
+ * token itself (the same arithmetic on the same logits, so all agree), the workgroup takes the
+ * expert whose rank in ascending id is its blockIdx.y, quantizes the row of x into its LDS while
+ * its first weights are on their way, and goes on as the paired form of gate_up_mma_kernel.
+ * Workgroup (0, 0) writes the routing's outputs and the few table entries the down product and
+ * the combine read. One launch (7-8 us of a block of 25) less than routing, sort and quantization
+ * as a launch of their own. */
+template <int MAXV>
+__global__ __launch_bounds__(256, 4) void gate_up_one_token_kernel(
+  const float *__restrict__ logits, int E, int topk, int renorm, int32_t *__restrict__ idx, float *__restrict__ wgt,
+  int *__restrict__ offsets, int *__restrict__ slot_pair, int *__restrict__ tok_slots, int *__restrict__ items,
+  const float *__restrict__ x, const WView *__restrict__ views, int I, float *__restrict__ h, hipq::MoeEpi ep) {
+  constexpr int TC = 8, NREG = TC / 2;
+  extern __shared__ __attribute__((aligned(16))) unsigned char xmoe_lds[];
+  const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
+  int myi;
+  float myw;
+  route_token_regs<MAXV>(logits, 0, E, topk, renorm, myi, myw);
+  const int rank = rank_by_expert(myi, topk);
+  const int item = blockIdx.y; /* < topk */
+  const unsigned long long owner = __ballot(lane < topk && rank == item);
+  const int e = __shfl(myi, __ffsll((long long)owner) - 1, 64);
+  if (blockIdx.x == 0 && blockIdx.y == 0 && wave == 0) {
+    if (lane < topk) {
+      idx[lane] = myi;
+      wgt[lane] = myw;
+      slot_pair[rank] = lane; /* slots in ascending expert id; one token: pair = its k */
+      tok_slots[rank] = rank;
+      offsets[myi + 1] = rank + 1; /* the end of the expert's slots: all the later kernels read of offsets */
+      items[2 + 2 * rank] = myi;
+      items[3 + 2 * rank] = rank;
+    }
+    if (lane == 0) items[0] = topk;
+  }
+  const WView wg = views[e], wu = views[E + e];
+  const int K = wg.K;
+  const XLds l = xlds_carve(xmoe_lds, TC, K);
+  float *xch = (float *)(xmoe_lds + xlds_bytes(TC, K)); /* [2 tiles][NREG][64 lanes] */
+  const int col0 = (blockIdx.x * 2 + (wave & 1)) * 32;
+  const int first = wave >> 1; /* 0: gate, 1: up */
+  const uint64_t dqs = (uint64_t)wu.qs - (uint64_t)wg.qs;
+  auto stage = [&]() {
+    /* rows 1 .. 7 of the matrix operand keep what the LDS held: a row of the product depends on
+     * its own activations only, and those rows are not stored */
+    const int nsb = K >> 8;
+    for (int b = wave; b < nsb; b += 4) { /* uniform per wavefront */
+      const float4 xv = *(const float4 *)(x + b * 256 + lane * 4);
+      hipq_quantize_q8_K_values<Q8K_ROWMMA>(xv, 0, b, b, nsb, 0, l.q, l.dA, nullptr, nullptr, (uint16_t *)l.amin,
+                                            nullptr, nullptr, TC);
+    }
+    __syncthreads();
+  };
+  float gate[NREG], up[NREG];
+  auto store = [&]() {
+    const int col = col0 + (lane & 31);
+    if (col < I && lane < 32) h[(size_t)item * I + col] = moe_act(ep, e, I, col, gate[0], up[0]);
+  };
+  if (col0 >= I) { /* uniform per wavefront; it still takes part in the barriers */
+    stage();
+    __syncthreads();
+    return;
+  }
+  xr_run<TC, NREG, XPD>(
+    1, l, K,
+    [&](int t, WView &w, int &c0) {
+      const uint64_t isup = (uint64_t)0 - (uint64_t)((t + first) & 1);
+      w.qs = (const uint8_t *)((uint64_t)wg.qs + (isup & dqs));
+      w.hdr = nullptr; /* the headers follow the nibbles */
+      w.N = wg.N;
+      w.K = wg.K;
+      c0 = col0;
+    },
+    [&](int t, const float(&out)[NREG]) {
+      if (t + first == 0) {
+#pragma unroll
+        for (int r = 0; r < NREG; ++r) gate[r] = out[r];
+      } else {
+#pragma unroll
+        for (int r = 0; r < NREG; ++r) up[r] = out[r];
+      }
+    },
+    stage);
+  float *mine = xch + (wave & 1) * (NREG * 64) + lane;
+  if (first == 0) mine[0] = gate[0];
+  __syncthreads();
+  if (first == 1) {
+    gate[0] = mine[0];
+    store();
+  }
+}
+
 /* QH: the rows of h come as fp32 (hf) and the workgroup quantizes those of its item
  * itself while its first weights are on their way, with the quantizer kernel's
  * arithmetic. Every column workgroup of an item repeats that, which pays with few
@@ -1280,7 +1389,7 @@ int launch_self_mma(const hipq::MoeArgs *a, const MoeBufs &b, const WView *views
 
 template <int TC>
 int launch_grouped_mma(const hipq::MoeArgs *a, const MoeBufs &b, const WView *views, const QAct &xq,
-                       const QAct &hq, hipStream_t s) {
+                       const QAct &hq, hipStream_t s, bool gate_up_done = false) {
   const hipq_moe_desc &d = a->desc;
   const int64_t P = (int64_t)d.tokens * d.topk;
   /* an upper bound of the work items: one per active expert and one per full chunk */
@@ -1291,7 +1400,9 @@ int launch_grouped_mma(const hipq::MoeArgs *a, const MoeBufs &b, const WView *vi
   const void *kg = few ? (const void *)gate_up_mma_kernel<TC, true> : (const void *)gate_up_mma_kernel<TC, false>;
   if (lds_g > 64 * 1024) /* beyond the default limit of a launch */
     HIPQ_HIP(hipFuncSetAttribute(kg, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_g));
-  if (few)
+  if (gate_up_done) {
+    /* h is there: the routing launch formed it (gate_up_one_token_kernel) */
+  } else if (few)
     hipq::launch_kernel("gate_up_mma_kernel<TC, true>", (gate_up_mma_kernel<TC, true>), dim3((d.intermediate + 63) / 64, max_items), dim3(256), lds_g,
                        s, views, d.experts, qview(xq), b.offsets, b.items, b.slot_pair, d.topk, d.intermediate,
                        b.h, a->epi);
@@ -1404,7 +1515,26 @@ int launch_moe(const MoeArgs *a, void *workspace, size_t workspace_bytes, const 
   const XQuant xqa = {a->x, (int64_t)T * (d.hidden / 256), d.hidden / 256, xq.q, xq.d, (uint16_t *)xq.bsum};
   if (mma && (((uintptr_t)a->x & 15) != 0))
     return fail(HIPQ_ERR_INVALID_ARGUMENT, "activation rows must be 16-byte aligned");
-  if (T <= 16 && E <= 1024) {
+  /* one token on the matrix-core path: routing, the quantization of x and gate/up as one launch */
+  const bool one_token = mma && T == 1 && chunk == 8 && mma_few(d, 8) && E <= 1024 && d.topk <= 64;
+  if (one_token) {
+    const size_t lds_g = xlds_bytes(8, d.hidden) + 8 * 256;
+    if (lds_g > 64 * 1024) {
+      const void *k = E <= 128   ? (const void *)gate_up_one_token_kernel<2>
+                      : E <= 256 ? (const void *)gate_up_one_token_kernel<4>
+                                 : (const void *)gate_up_one_token_kernel<16>;
+      HIPQ_HIP(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_g));
+    }
+    const dim3 grid((unsigned)((d.intermediate + 63) / 64), (unsigned)d.topk);
+    auto launch = [&](auto k, const char *name) {
+      hipq::launch_kernel(name, k, grid, dim3(256), lds_g, s, logits, E, d.topk, d.renormalize, idx, wgt, b.offsets,
+                          b.slot_pair, b.tok_slots, b.items, a->x, views, d.intermediate, b.h, a->epi);
+    };
+    if (E <= 128) launch(gate_up_one_token_kernel<2>, "gate_up_one_token_kernel<2>");
+    else if (E <= 256) launch(gate_up_one_token_kernel<4>, "gate_up_one_token_kernel<4>");
+    else launch(gate_up_one_token_kernel<16>, "gate_up_one_token_kernel<16>");
+    HIPQ_HIP(hipGetLastError());
+  } else if (T <= 16 && E <= 1024) {
     const unsigned qblocks = mma ? (unsigned)((xqa.n_sb + 15) / 16) : 0;
     auto launch = [&](auto fused, auto plain) {
       if (mma)
@@ -1433,7 +1563,7 @@ int launch_moe(const MoeArgs *a, void *workspace, size_t workspace_bytes, const 
     else launch(route_quantize_kernel<16>, route_kernel<16>);
     HIPQ_HIP(hipGetLastError());
   }
-  if ((T <= 16 && E <= 1024) || self) {
+  if ((T <= 16 && E <= 1024) || self || one_token) {
     /* routed and sorted above, or no sort needed */
   } else if (P <= 16384 && E <= 1024) {
     hipq::launch_kernel("sort_pairs_kernel", sort_pairs_kernel, dim3(1), dim3(1024), 0, s, idx, P, E, d.topk, b.offsets,
@@ -1455,7 +1585,7 @@ int launch_moe(const MoeArgs *a, void *workspace, size_t workspace_bytes, const 
     rc = launch_self_mma(a, b, views, xq, s);
   } else if (mma) {
     const int tc = chunk;
-    rc = tc == 8    ? launch_grouped_mma<8>(a, b, views, xq, hq, s)
+    rc = tc == 8    ? launch_grouped_mma<8>(a, b, views, xq, hq, s, one_token)
          : tc == 16 ? launch_grouped_mma<16>(a, b, views, xq, hq, s)
                     : launch_grouped_mma<32>(a, b, views, xq, hq, s);
   } else if (dt == HIPQ_Q4_0)
