@@ -1126,11 +1126,10 @@ __device__ __forceinline__ int self_scan(const int32_t *__restrict__ idx, int P,
 }
 
 template <int TC>
-__device__ __forceinline__ void gate_up_self_pass(unsigned char *lds, int n, int e, const WView *__restrict__ views,
-                                                  int E_, const QView &xq, int I, float *__restrict__ h,
+__device__ __forceinline__ void gate_up_self_pass(unsigned char *lds, int n, int e, const WView &wg, const WView &wu,
+                                                  const QView &xq, int I, float *__restrict__ h,
                                                   const hipq::MoeEpi &ep) {
   constexpr int NREG = TC / 2;
-  const WView wg = views[e], wu = views[E_ + e];
   const int K = wg.K;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
   XLds l = xlds_carve(lds + SELF_HEAD, TC, K);
@@ -1180,24 +1179,24 @@ __global__ __launch_bounds__(256, 4) void gate_up_self_kernel(const WView *__res
                                                               float *__restrict__ h, hipq::MoeEpi ep) {
   extern __shared__ __attribute__((aligned(16))) unsigned char xmoe_lds[];
   const int e = blockIdx.y % E_, chunk = blockIdx.y / E_;
+  const WView wg = views[e], wu = views[E_ + e]; /* asked for before the scan: they are there when it ends */
   int *pairs = (int *)xmoe_lds;
   const int total = self_scan(idx, P, topk, e, chunk, pairs, pairs + SELF_TC);
   const int n = min(SELF_TC, total - chunk * SELF_TC);
   if (n <= 0) return; /* uniform per workgroup */
   if (n <= 8)
-    gate_up_self_pass<8>(xmoe_lds, n, e, views, E_, xq, I, h, ep);
+    gate_up_self_pass<8>(xmoe_lds, n, e, wg, wu, xq, I, h, ep);
   else
-    gate_up_self_pass<16>(xmoe_lds, n, e, views, E_, xq, I, h, ep);
+    gate_up_self_pass<16>(xmoe_lds, n, e, wg, wu, xq, I, h, ep);
 }
 
 /* The rows of h come as fp32 and the workgroup quantizes those of its chunk itself while its first
  * weights are on their way (the QH form of down_mma_kernel). */
 template <int TC>
-__device__ __forceinline__ void down_self_pass(unsigned char *lds, int n, int e, const WView *__restrict__ views,
-                                               int E_, const float *__restrict__ hf, const float *__restrict__ wgt,
+__device__ __forceinline__ void down_self_pass(unsigned char *lds, int n, int e, const WView &wd,
+                                               const float *__restrict__ hf, const float *__restrict__ wgt,
                                                int H, float *__restrict__ contrib, const hipq::MoeEpi &ep) {
   constexpr int NREG = TC / 2, CT = 2;
-  const WView wd = views[2 * E_ + e];
   const int K = wd.K;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
   XLds l = xlds_carve(lds + SELF_HEAD, TC, K);
@@ -1249,14 +1248,15 @@ __global__ __launch_bounds__(256, 4) void down_self_kernel(const WView *__restri
                                                            float *__restrict__ contrib, hipq::MoeEpi ep) {
   extern __shared__ __attribute__((aligned(16))) unsigned char xmoe_lds[];
   const int e = blockIdx.y % E_, chunk = blockIdx.y / E_;
+  const WView wd = views[2 * E_ + e]; /* asked for before the scan */
   int *pairs = (int *)xmoe_lds;
   const int total = self_scan(idx, P, topk, e, chunk, pairs, pairs + SELF_TC);
   const int n = min(SELF_TC, total - chunk * SELF_TC);
   if (n <= 0) return; /* uniform per workgroup */
   if (n <= 8)
-    down_self_pass<8>(xmoe_lds, n, e, views, E_, hf, wgt, H, contrib, ep);
+    down_self_pass<8>(xmoe_lds, n, e, wd, hf, wgt, H, contrib, ep);
   else
-    down_self_pass<16>(xmoe_lds, n, e, views, E_, hf, wgt, H, contrib, ep);
+    down_self_pass<16>(xmoe_lds, n, e, wd, hf, wgt, H, contrib, ep);
 }
 
 /* y[t][c] = sum of the token's contributions, ascending expert id */
