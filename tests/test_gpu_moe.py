@@ -160,6 +160,13 @@ def test_moe_block_without_a_pair_sort_with_crowded_experts(hipq, cr):
         got = y.cpu().numpy()
         assert not np.isnan(got).any()
         assert gu.rel_err(got, ref_y) <= 2e-6, gu.rel_err(got, ref_y)
+    # the same block with every operand in host memory: the bits of the device-memory call
+    yh = np.full((t, h), np.nan, np.float32)
+    idxh = np.zeros((t, k), np.int32)
+    capi.moe_forward(t, h, i, e, k, wg, wu, wd, x, yh, router_logits=logits, topk_idx=idxh, mem=capi.MEM_HOST,
+                     stream=gu.stream())
+    assert np.array_equal(idxh, ref_idx)
+    assert np.array_equal(yh.view(np.uint32), got.view(np.uint32))
     for w in wg + wu + wd:
         w.destroy()
 
