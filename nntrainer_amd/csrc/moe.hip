@@ -94,17 +94,99 @@ size_t carve(const hipq_moe_desc &d, int is_k, uint8_t *base, MoeBufs *b) {
 }
 
 /* logits[t][e] = sum_h x[t][h] * Wr[h][e] (+ bias[e], added after the sum as the reference
- * adds it to the finished product, gpt_oss_moe_layer.cpp:500-503) */
-__global__ __launch_bounds__(256) void router_logits_kernel(const float *__restrict__ x,
-                                                            const float *__restrict__ wr, int H,
-                                                            int E, const float *__restrict__ bias,
-                                                            float *__restrict__ logits) {
+ * adds it to the finished product, gpt_oss_moe_layer.cpp:500-503): one thread per logit, one
+ * chain over h. For expert counts that are no multiple of four. */
+__global__ __launch_bounds__(256) void router_logits_scalar_kernel(const float *__restrict__ x,
+                                                                   const float *__restrict__ wr, int H,
+                                                                   int E, const float *__restrict__ bias,
+                                                                   float *__restrict__ logits) {
   const int t = blockIdx.x;
   const float *xt = x + (size_t)t * H;
   for (int e = threadIdx.x; e < E; e += blockDim.x) {
     float acc = 0.f;
     for (int h = 0; h < H; ++h) acc = fmaf(xt[h], wr[(size_t)h * E + e], acc);
     logits[(size_t)t * E + e] = bias ? acc + bias[e] : acc;
+  }
+}
+
+/* The same for E % 4 == 0, which is every model on this path. The single chain is bound by the
+ * latency of its loads (2048 dependent rounds: 28 us for ONE token against 24 us for the rest of
+ * the block), and one workgroup per token by what one CU can pull out of the cache (Wr is 1 MB:
+ * 12 us). Here a workgroup takes sixteen experts (64 bytes of every row of Wr) and up to four
+ * tokens, whose rows of x it first copies to LDS. Four lanes read a row's 64 bytes, sixteen rows
+ * an instruction (sixteen half lines, not sixty-four separate ones), the four wavefronts take the
+ * rows in turn, sixteen loads are in flight and each is used for all the tokens. The partial sums
+ * meet in a fixed order: over the sixteen row lanes by exchanges, over the wavefronts through LDS.
+ * The matrix is read by E / 16 CUs side by side, each its own columns. (The reference's order of
+ * the sum is its BLAS library's and not specified.) */
+constexpr int ROUTER_TB = 4; /* tokens per workgroup, at most */
+template <int TBN> /* tokens of this workgroup: 1, 2 or 4 */
+__global__ __launch_bounds__(256) void router_logits_kernel(const float *__restrict__ x,
+                                                            const float *__restrict__ wr, int T, int H,
+                                                            int E, const float *__restrict__ bias,
+                                                            float *__restrict__ logits) {
+  extern __shared__ __attribute__((aligned(16))) float router_x[]; /* [token][H], then 256 floats of partial sums */
+  constexpr int JU = 4; /* groups of four rows a lane has in flight: sixteen loads */
+  const int t0 = blockIdx.y * TBN;
+  for (int i = threadIdx.x * 4; i < TBN * H; i += 256 * 4) { /* H % 4 == 0 */
+    const int tb = i / H, h = i - tb * H;
+    *(float4 *)(router_x + i) = *(const float4 *)(x + (size_t)min(t0 + tb, T - 1) * H + h);
+  }
+  __syncthreads();
+  float *part = router_x + TBN * H; /* [wavefront 4][token][16 experts] */
+  const int e4n = E >> 2;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int r = lane >> 2, q = lane & 3;
+  const int c = min((int)blockIdx.x * 4 + q, e4n - 1); /* columns past the end repeat the last; not stored */
+  float acc[TBN][4];
+#pragma unroll
+  for (int tb = 0; tb < TBN; ++tb) acc[tb][0] = acc[tb][1] = acc[tb][2] = acc[tb][3] = 0.f;
+  const float4 *w4 = (const float4 *)wr + c;
+  /* this lane's rows: h = 256 j + 64 wave + 4 r + i, i = 0 .. 3 (its x values are one 128-bit LDS read) */
+  for (int h = 64 * wave + 4 * r; h < H; h += 256 * JU) {
+    float4 w[JU][4];
+#pragma unroll
+    for (int j = 0; j < JU; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) w[j][i] = w4[(size_t)min(h + 256 * j + i, H - 1) * e4n];
+#pragma unroll
+    for (int j = 0; j < JU; ++j) {
+      if (h + 256 * j < H) { /* H % 4 == 0: the four rows are in or out together */
+#pragma unroll
+        for (int tb = 0; tb < TBN; ++tb) {
+          const float4 xv = *(const float4 *)(router_x + tb * H + h + 256 * j);
+          const float xs[4] = {xv.x, xv.y, xv.z, xv.w};
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            acc[tb][0] = fmaf(xs[i], w[j][i].x, acc[tb][0]);
+            acc[tb][1] = fmaf(xs[i], w[j][i].y, acc[tb][1]);
+            acc[tb][2] = fmaf(xs[i], w[j][i].z, acc[tb][2]);
+            acc[tb][3] = fmaf(xs[i], w[j][i].w, acc[tb][3]);
+          }
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int tb = 0; tb < TBN; ++tb) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float v = acc[tb][j];
+      v += __shfl_xor(v, 4, 64);
+      v += __shfl_xor(v, 8, 64);
+      v += __shfl_xor(v, 16, 64);
+      v += __shfl_xor(v, 32, 64);
+      if (r == 0) part[(wave * TBN + tb) * 16 + q * 4 + j] = v;
+    }
+  }
+  __syncthreads();
+  if (threadIdx.x < TBN * 16) {
+    const int tb = threadIdx.x >> 4, el = threadIdx.x & 15, e = blockIdx.x * 16 + el;
+    if (t0 + tb < T && e < E) {
+      float sum = part[tb * 16 + el];
+      for (int w = 1; w < 4; ++w) sum += part[(w * TBN + tb) * 16 + el];
+      logits[(size_t)(t0 + tb) * E + e] = bias ? sum + bias[e] : sum;
+    }
   }
 }
 
@@ -1495,8 +1577,23 @@ int launch_moe(const MoeArgs *a, void *workspace, size_t workspace_bytes, const 
 
   const float *logits = a->router_logits;
   if (!logits) {
-    hipq::launch_kernel("router_logits_kernel", router_logits_kernel, dim3(T), dim3(256), 0, s, a->x, a->router_weight,
-                       d.hidden, E, a->router_bias, b.logits);
+    /* the rows of x of a workgroup's tokens go to LDS: four tokens, or as many as there are or fit 64 KB */
+    int tb_n = d.hidden > 0 ? (int)std::min<int64_t>(std::min(ROUTER_TB, T), 16000 / d.hidden) : 0;
+    tb_n = tb_n >= 4 ? 4 : tb_n >= 2 ? 2 : tb_n;
+    if ((E & 3) || (d.hidden & 3) || tb_n < 1 || (((uintptr_t)a->router_weight | (uintptr_t)a->x) & 15)) {
+      hipq::launch_kernel("router_logits_scalar_kernel", router_logits_scalar_kernel, dim3(T), dim3(256), 0, s, a->x,
+                          a->router_weight, d.hidden, E, a->router_bias, b.logits);
+    } else {
+      const dim3 grid((E / 4 + 3) / 4, (T + tb_n - 1) / tb_n);
+      const size_t lds = ((size_t)tb_n * d.hidden + 256) * sizeof(float);
+      auto launch = [&](auto k, const char *name) {
+        hipq::launch_kernel(name, k, grid, dim3(256), lds, s, a->x, a->router_weight, T, d.hidden, E, a->router_bias,
+                            b.logits);
+      };
+      if (tb_n == 4) launch(router_logits_kernel<4>, "router_logits_kernel<4>");
+      else if (tb_n == 2) launch(router_logits_kernel<2>, "router_logits_kernel<2>");
+      else launch(router_logits_kernel<1>, "router_logits_kernel<1>");
+    }
     HIPQ_HIP(hipGetLastError());
     logits = b.logits;
   }
