@@ -699,6 +699,23 @@ def main():
     moe_graph_ms = moe_graph_time(mt)
     moe_decode_ms, decode_active = moe_time(1)
     moe_decode_graph_ms = moe_graph_time(1)
+
+    def moe_router_time(tokens, reps=40):
+        """The block given the router's weight instead of its logits (the layer API's case)."""
+        wr = torch.randn((mh, me), generator=gen, device="cuda") * 0.05
+        x_, y_ = mx[:tokens], my[:tokens]
+        for i in range(4):
+            capi.moe_forward(tokens, mh, mi, me, mk, sets[i % 2], None, None, x_, y_, router_weight=wr, stream=stream)
+        torch.cuda.synchronize()
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ev0.record()
+        for i in range(reps):
+            capi.moe_forward(tokens, mh, mi, me, mk, sets[i % 2], None, None, x_, y_, router_weight=wr, stream=stream)
+        ev1.record()
+        torch.cuda.synchronize()
+        return ev0.elapsed_time(ev1) / reps
+
+    moe_router_ms, moe_router_decode_ms = moe_router_time(mt), moe_router_time(1)
     moe_bytes = active * 3 * (mi * mh * 144 // 256) + 2 * mt * mh * 4
     moe_gbs = moe_bytes / (moe_ms * 1e-3) / 1e9
     moe_decode_bytes = decode_active * 3 * (mi * mh * 144 // 256) + 2 * mh * 4
@@ -873,7 +890,11 @@ def main():
             "decode_token": {"ms_per_block": round(moe_decode_ms, 5),
                              "ms_per_block_in_a_graph": round(moe_decode_graph_ms, 5),
                              "active_experts": decode_active,
-                             "gbs": round(moe_decode_bytes / (moe_decode_ms * 1e-3) / 1e9, 2)}},
+                             "gbs": round(moe_decode_bytes / (moe_decode_ms * 1e-3) / 1e9, 2)},
+            "from_the_router_weight": {"note": "the same blocks given the router's weight [hidden x experts] instead of its "
+                                               "logits: one more launch (router_logits_kernel)",
+                                       "ms_per_block": round(moe_router_ms, 5),
+                                       "decode_token_ms_per_block": round(moe_router_decode_ms, 5)}},
     }
     if not args.no_cpu:
         capi.matmul(weights[0], a, M, c, stream=stream)
