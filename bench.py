@@ -151,6 +151,27 @@ def cpu_gemv_baseline(kind, n, k, host, nbytes, budget_s=4.0):
             "gpu_output_bit_identical": bool(np.array_equal(gpu_out.view(np.uint32), c.view(np.uint32)))}
 
 
+def plugin_moe_layer():
+    """One qwen_moe layer of the C3 shape through libnntrainer_hip_context.so: router, routing and the three
+    expert products in one incremental_forwarding call on host tensors; microseconds per call."""
+    import subprocess
+    lib = os.path.join(ROOT, "nntrainer_amd", "lib")
+    exe, plugin = os.path.join(lib, "hipq_host_selftest"), os.path.join(lib, "libnntrainer_hip_context.so")
+    if not (os.path.exists(exe) and os.path.exists(plugin)):
+        return {"skipped": "the plug-in is not built (python -c 'import __graft_entry__ as g; g.build()')"}
+    try:
+        r = subprocess.run([exe, plugin, "moelayer", "200"], capture_output=True, text=True, timeout=180)
+        if r.returncode != 0:
+            return {"failed": (r.stdout + r.stderr)[-300:]}
+        res = json.loads(r.stdout.strip().splitlines()[-1])
+    except Exception as e:  # the bench line must still be printed
+        return {"failed": repr(e)[:300]}
+    res["workload"] = ("one qwen_moe layer, hidden 2048, 128 experts of 768, top 8, Q4_K (BASELINE configs[2]'s "
+                       "block), created by the context's factory; incremental_forwarding on host tensors, the router's "
+                       "weight given; one decode token and a chunk of 64 tokens; wall clock per call")
+    return res
+
+
 def plugin_c5_layer():
     """The quantized FCs of one C5 decoder layer through libnntrainer_hip_context.so (layers created by the
     context's factories, run with incremental_forwarding on host tensors): microseconds per layer."""
@@ -187,6 +208,7 @@ def main():
     # ---- a C5 decoder layer's FCs through the framework plug-in (the layer API, host tensors, every
     # call synchronous): the plug-in's own driver as a child process, before this process touches the GPU
     plugin_layer = plugin_c5_layer()
+    plugin_moe = plugin_moe_layer()
 
     import numpy as np
     import torch
@@ -876,6 +898,7 @@ def main():
                                  "algorithmic_ops": 450971566080,
                                  "note": "the lm_head row's time is inside the figure, its ops are not"}},
         "c5_layer_through_plugin": plugin_layer,
+        "moe_layer_through_plugin": plugin_moe,
         "moe_block": {
             "workload": "MoE FFN block (BASELINE configs[3]): 64 tokens, hidden 2048, 128 experts x "
                         "(gate/up 2048->768, down 768->2048) Q4_K, top-8; router, sort, experts, combine; "

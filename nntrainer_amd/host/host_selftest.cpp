@@ -39,6 +39,8 @@
  *                            mlp_swiglu + fully_connected; one decode row and a prefill of 512 rows; tensors in
  *                            ordinary memory and in memory of the context's allocator. Prints one JSON object.
  *                            Weights are pseudo-random blocks: the mode measures time, the other modes results.
+ *   moelayer <iterations>    the same for one qwen_moe layer of the Qwen3-30B-A3B shape (hidden 2048, 128 experts of
+ *                            768, top 8, Q4_K): one decode token and a chunk of 64 tokens per call
  * The test suite compares the written outputs with expected values it computes itself.
  */
 #include <dlfcn.h>
@@ -629,9 +631,73 @@ static int run_c5layer(Context *ctx, int iters) {
   return 0;
 }
 
+static int run_moelayer(Context *ctx, int iters) {
+  const unsigned H = 2048, I = 768, E = 128, K = 8;
+  auto ma = ctx->getContextData() ? ctx->getContextData()->getMemAllocator() : nullptr;
+  std::printf("{");
+  bool first = true;
+  for (int pinned = 0; pinned < 2; ++pinned) {
+    for (unsigned T : {1u, 64u}) {
+      auto layer = ctx->createLayerObject("qwen_moe", {"num_experts=" + std::to_string(E),
+                                                        "num_experts_per_token=" + std::to_string(K),
+                                                        "unit=" + std::to_string(I), "moe_activation=swish"});
+      InitLayerContext ic({TensorDim(1, 1, T, H)}, "moe", Tformat::NCHW, Tdatatype::Q4_K, Tdatatype::FP32);
+      layer->finalize(ic);
+      RunLayerContext rc(ic);
+      uint32_t x = 12345u + T;
+      float *wr = rc.getWeight(0).getData<float>();
+      for (size_t i = 0; i < (size_t)H * E; ++i) {
+        x = x * 1664525u + 1013904223u;
+        wr[i] = ((int)(x >> 20) - 2048) / 40960.f;
+      }
+      for (unsigned w = 1; w < rc.getNumWeights(); ++w) {
+        /* x8-repacked Q4_K as the tensor holds it: groups of 1152 bytes, eight fp16 scales and eight
+         * fp16 mins (2^-8 here), then 96 bytes of 6-bit scales and 1024 of nibbles */
+        uint8_t *p = rc.getWeight(w).getData<uint8_t>();
+        const size_t bytes = mirror_tensor_bytes(rc.getWeight(w).getDim());
+        for (size_t g = 0; g + 1152 <= bytes; g += 1152) {
+          for (int i = 0; i < 16; ++i) {
+            p[g + 2 * i] = 0x00;
+            p[g + 2 * i + 1] = 0x1c;
+          }
+          for (int i = 32; i < 1152; ++i) {
+            x = x * 1664525u + 1013904223u;
+            p[g + i] = (uint8_t)(x >> 24);
+          }
+        }
+      }
+      float *in = rc.getInput(0).getData<float>();
+      for (size_t i = 0; i < (size_t)T * H; ++i)
+        in[i] = (float)((int)((i * 2654435761u) >> 20 & 0xfff) - 2048) / 2048.f;
+      if (pinned && ma) {
+        auto place = [&](Tensor &t) {
+          void *q = nullptr;
+          ma->alloc(&q, mirror_tensor_bytes(t.getDim()), 64);
+          t.mirror_move_to(q, [ma](void *r) { ma->free(r); });
+        };
+        place(rc.getInput(0));
+        place(rc.getOutput(0));
+      }
+      const int n = T == 1 ? iters : (iters + 3) / 4;
+      for (int i = 0; i < 3; ++i)
+        layer->incremental_forwarding(rc, 0, T, false);
+      const auto t0 = std::chrono::steady_clock::now();
+      for (int i = 0; i < n; ++i)
+        layer->incremental_forwarding(rc, 0, T, false);
+      const auto t1 = std::chrono::steady_clock::now();
+      std::printf("%s\"%s_%s_us\": %.2f", first ? "" : ", ", T == 1 ? "decode_token" : "chunk_of_64_tokens",
+                  pinned ? "allocator_memory" : "ordinary_memory",
+                  std::chrono::duration<double, std::micro>(t1 - t0).count() / n);
+      first = false;
+    }
+  }
+  std::printf("}\n");
+  return 0;
+}
+
 int main(int argc, char **argv) {
   if (argc < 3) {
-    std::printf("usage: %s <plugin.so> api | c5layer <iterations> | fc ... | moe ...\n", argv[0]);
+    std::printf("usage: %s <plugin.so> api | c5layer <iterations> | moelayer <iterations> | fc ... | moe ...\n", argv[0]);
     return 2;
   }
   try {
@@ -639,6 +705,8 @@ int main(int argc, char **argv) {
     const std::string mode = argv[2];
     if (mode == "c5layer" && argc == 4)
       return run_c5layer(ctx, std::atoi(argv[3]));
+    if (mode == "moelayer" && argc == 4)
+      return run_moelayer(ctx, std::atoi(argv[3]));
     if (mode == "api")
       return run_api(ctx);
     if (mode == "fc" && argc == 14)
