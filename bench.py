@@ -189,8 +189,9 @@ def plugin_c5_layer():
         return {"failed": repr(e)[:300]}
     res["workload"] = ("one Qwen3-0.6B-shaped decoder layer (BASELINE configs[4]), Q4_0 weights, through the context "
                        "plug-in: layers from its factories, incremental_forwarding on host tensors, every call "
-                       "synchronous; as the seven fully_connected layers of an unchanged graph and as qkv_layer + "
-                       "fully_connected + mlp_swiglu + fully_connected; tensors in ordinary memory and in memory of the "
+                       "synchronous; as the seven fully_connected layers of an unchanged graph, as qkv_layer + "
+                       "fully_connected + mlp_swiglu + fully_connected, and as qkv_layer + fully_connected + mlp_swiglu "
+                       "with down_unit (the whole MLP one call, hidden rows kept on the device); tensors in ordinary memory and in memory of the "
                        "context's allocator (page-locked); one decode row, and a prefill of 512 rows; wall clock per layer")
     return res
 

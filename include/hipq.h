@@ -234,6 +234,17 @@ HIPQ_API int hipq_matmul_multi(int count, const hipq_weight_t *w, const float *A
 HIPQ_API int hipq_mlp_swiglu(hipq_weight_t w_act, hipq_weight_t w_mul, const float *A, int64_t M,
                              int64_t lda, float *out, int64_t ldo, int mem, void *stream);
 
+/** The whole gated MLP of a decoder layer: out[M x Nd] = swiglu(A . W_act^T, A . W_mul^T) . W_down^T,
+ *  the four layers "ffn_up", "ffn_gate", "swiglu" and "ffn_down" of CausalLM::createMlp
+ *  (Applications/CausalLM/causal_lm.cpp:671-705) as one call. The hidden activation [M x N] stays in
+ *  device memory between the gated half and the down projection: with host operands only A goes in
+ *  and only out comes back, where the two calls (hipq_mlp_swiglu, hipq_matmul) move the hidden rows
+ *  out and in again and wait once more. W_down has K = N of the other two. Every value equals what
+ *  those two calls give bit for bit (the same kernels on the same operands). */
+HIPQ_API int hipq_mlp_swiglu_down(hipq_weight_t w_act, hipq_weight_t w_mul, hipq_weight_t w_down,
+                                  const float *A, int64_t M, int64_t lda, float *out, int64_t ldo,
+                                  int mem, void *stream);
+
 /** Mixture-of-experts feed-forward block (MoELayer::incremental_forwarding,
  *  qwen_moe_layer.cpp:394-503): softmax over E router logits, top-k, weights
  *  renormalised to sum 1, per (token, expert) SwiGLU MLP

@@ -21,7 +21,7 @@ SYMBOLS = [
     "hipq_init", "hipq_shutdown", "hipq_last_error", "hipq_version", "hipq_weight_nbytes",
     "hipq_weight_create", "hipq_weight_destroy", "hipq_weight_dims", "hipq_quantize_q8_0",
     "hipq_quantize_q8_K", "hipq_matmul", "hipq_matmul_each_row", "hipq_matmul_noalloc", "hipq_matmul_multi", "hipq_moe_forward",
-    "hipq_moe_forward_ext", "hipq_mlp_swiglu", "hipq_host_alloc", "hipq_host_free", "hipq_stream_release",
+    "hipq_moe_forward_ext", "hipq_mlp_swiglu", "hipq_mlp_swiglu_down", "hipq_host_alloc", "hipq_host_free", "hipq_stream_release",
     "hipq_quantize_weights", "hipq_file_layout", "hipq_weights_from_file",
     "hipq_device_alloc", "hipq_device_free", "hipq_device_upload", "hipq_device_download",
     "hipq_launch_timing_begin", "hipq_launch_timing_end",
@@ -104,6 +104,7 @@ def lib():
                                            C.POINTER(vp), vp, vp, vp, vp, vp, vp, i32, vp]
         L.hipq_quantize_weights.argtypes = [i32, vp, i64, i64, vp, i32, vp]
         L.hipq_mlp_swiglu.argtypes = [vp, vp, vp, i64, i64, vp, i64, i32, vp]
+        L.hipq_mlp_swiglu_down.argtypes = [vp, vp, vp, vp, i64, i64, vp, i64, i32, vp]
         L.hipq_host_alloc.argtypes = [C.POINTER(vp), C.c_size_t]
         L.hipq_host_free.argtypes = [vp]
         L.hipq_stream_release.argtypes = [vp]
@@ -246,6 +247,12 @@ def mlp_swiglu(w_act, w_mul, a, m, out, lda=None, ldo=None, mem=MEM_DEVICE, stre
     """out = swiglu(a . w_act^T, a . w_mul^T): the gated half of a dense MLP in one call."""
     check(lib().hipq_mlp_swiglu(w_act.handle, w_mul.handle, _addr(a), m, lda or w_act.k, _addr(out),
                                 ldo or w_act.n, mem, stream))
+
+
+def mlp_swiglu_down(w_act, w_mul, w_down, a, m, out, lda=None, ldo=None, mem=MEM_DEVICE, stream=None):
+    """out = swiglu(a . w_act^T, a . w_mul^T) . w_down^T: the gated MLP of a decoder layer in one call."""
+    check(lib().hipq_mlp_swiglu_down(w_act.handle, w_mul.handle, w_down.handle, _addr(a), m, lda or w_act.k,
+                                     _addr(out), ldo or w_down.n, mem, stream))
 
 
 def quantize_weights(dtype, w, n, k, out, mem=MEM_DEVICE, stream=None):

@@ -1237,6 +1237,66 @@ int hipq_mlp_swiglu(hipq_weight_t w_act, hipq_weight_t w_mul, const float *A, in
   return stage_copy(false, dO, out, (size_t)ldo * 4, (size_t)N * 4, (size_t)M, s);
 }
 
+int hipq_mlp_swiglu_down(hipq_weight_t w_act, hipq_weight_t w_mul, hipq_weight_t w_down, const float *A, int64_t M,
+                         int64_t lda, float *out, int64_t ldo, int mem, void *stream) {
+  int rc = require_ready();
+  if (rc) return rc;
+  if (!w_act || !w_mul || !w_down) return fail(HIPQ_ERR_INVALID_ARGUMENT, "null weight");
+  if ((rc = check_matmul_args(w_act, A, M, lda, out, w_act->N))) return rc;
+  if ((rc = check_matmul_args(w_mul, A, M, lda, out, w_mul->N))) return rc;
+  if (w_act->K != w_mul->K || w_act->N != w_mul->N)
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "the two projections differ in shape");
+  if (w_down->K != w_act->N)
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "the down projection takes %lld values a row, the gated half gives %lld",
+                (long long)w_down->K, (long long)w_act->N);
+  if ((rc = check_matmul_args(w_down, A, M, w_down->K, out, ldo))) return rc;
+  if (mem != HIPQ_MEM_DEVICE && mem != HIPQ_MEM_HOST)
+    return fail(HIPQ_ERR_INVALID_ARGUMENT, "unknown mem kind %d", mem);
+  if (M == 0) return HIPQ_OK;
+  hipStream_t s = (hipStream_t)stream;
+  EnqueueGuard eg(enqueue_lock(s));
+  CallScope call(s);
+  const int64_t N = w_act->N, K = w_act->K, Nd = w_down->N;
+  /* one operand buffer for the whole call: the input rows (host operands), the two products, the hidden
+   * rows and the output rows (host operands) */
+  const size_t a_bytes = ((size_t)M * K * 4 + 255) & ~(size_t)255, h_bytes = ((size_t)M * N * 4 + 255) & ~(size_t)255,
+               o_bytes = ((size_t)M * Nd * 4 + 255) & ~(size_t)255;
+  void *io = nullptr;
+  if ((rc = io_buffer(s, a_bytes + 3 * h_bytes + o_bytes, &io))) return rc;
+  float *dA = (float *)io, *dY = (float *)((char *)io + a_bytes), *dZ = (float *)((char *)dY + h_bytes),
+        *dH = (float *)((char *)dZ + h_bytes), *dO = (float *)((char *)dH + h_bytes);
+  const float *a_dev = A;
+  int64_t a_ld = lda;
+  float *o_dev = out;
+  int64_t o_ld = ldo;
+  DirectIO dio;
+  bool direct = false;
+  if (mem == HIPQ_MEM_HOST) {
+    if (dio.begin(s, A, M, lda, K, 1, &out, &ldo, &Nd, &rc)) { /* a decode step's rows: no copy engine */
+      if ((rc = dio.fetch(dA, K))) return rc;
+      o_dev = dio.outs[0].dev, o_ld = dio.outs[0].dld;
+      direct = true;
+    } else {
+      if (rc || (rc = stage_copy(true, dA, (void *)A, (size_t)lda * 4, (size_t)K * 4, (size_t)M, s))) return rc;
+      o_dev = dO, o_ld = Nd;
+    }
+    a_dev = dA, a_ld = K;
+  }
+  if (M == 1 && hipq::gemv_fuses_swiglu(w_act, w_mul, a_dev)) {
+    if ((rc = hipq::launch_gemv_fused_swiglu(w_act, w_mul, a_dev, dH, s))) return rc;
+  } else {
+    const hipq_weight_t ws[2] = {w_act, w_mul};
+    float *const cs[2] = {dY, dZ};
+    const int64_t lds[2] = {N, N};
+    if ((rc = hipq_matmul_multi(2, ws, a_dev, M, a_ld, cs, lds, HIPQ_MEM_DEVICE, stream))) return rc;
+    if ((rc = hipq::launch_swiglu_rows(dY, dZ, M, N, dH, N, s))) return rc;
+  }
+  if ((rc = hipq_matmul(w_down, dH, M, N, o_dev, o_ld, HIPQ_MEM_DEVICE, stream))) return rc;
+  if (mem == HIPQ_MEM_DEVICE) return HIPQ_OK;
+  if (direct) return dio.finish();
+  return stage_copy(false, dO, out, (size_t)ldo * 4, (size_t)Nd * 4, (size_t)M, s);
+}
+
 int hipq_matmul_multi(int count, const hipq_weight_t *w, const float *A, int64_t M, int64_t lda,
                       float *const *C, const int64_t *ldc, int mem, void *stream) {
   int rc = require_ready();

@@ -163,6 +163,14 @@ void mlp_swiglu(WeightCache &cache, const void *act_bytes, const void *mul_bytes
   check(hipq_mlp_swiglu(wa, wm, A, M, lda, out, ldo, HIPQ_MEM_HOST, nullptr), "hipq_mlp_swiglu");
 }
 
+void mlp_swiglu_down(WeightCache &cache, const void *act_bytes, const void *mul_bytes, const WeightSpec &spec,
+                     const void *down_bytes, const WeightSpec &down_spec, const float *A, int64_t M, int64_t lda,
+                     float *out, int64_t ldo) {
+  require_runtime();
+  hipq_weight_t wa = cache.get(act_bytes, spec), wm = cache.get(mul_bytes, spec), wd = cache.get(down_bytes, down_spec);
+  check(hipq_mlp_swiglu_down(wa, wm, wd, A, M, lda, out, ldo, HIPQ_MEM_HOST, nullptr), "hipq_mlp_swiglu_down");
+}
+
 hipq_weight_t upload(const void *host_bytes, const WeightSpec &spec) {
   require_runtime();
   if (!host_bytes)

@@ -120,6 +120,10 @@ void matmul_multi(WeightCache &cache, const std::vector<const void *> &weight_by
 /** out[M x N] = swiglu(A . Wact^T, A . Wmul^T), both weights of one spec (hipq_mlp_swiglu) */
 void mlp_swiglu(WeightCache &cache, const void *act_bytes, const void *mul_bytes, const WeightSpec &spec,
                 const float *A, int64_t M, int64_t lda, float *out, int64_t ldo);
+/** out[M x Nd] = swiglu(A . Wact^T, A . Wmul^T) . Wdown^T (hipq_mlp_swiglu_down): the hidden rows stay on the device */
+void mlp_swiglu_down(WeightCache &cache, const void *act_bytes, const void *mul_bytes, const WeightSpec &spec,
+                     const void *down_bytes, const WeightSpec &down_spec, const float *A, int64_t M, int64_t lda,
+                     float *out, int64_t ldo);
 
 struct MoeShape {
   int tokens, hidden, intermediate, experts, topk;

@@ -27,8 +27,9 @@
  *   qkv <dtype> <K> <Nq> <Nk> <Nv> <height> <from> <to> <weights> <input> <out>
  *                            qkv_layer; <weights> holds q, k, v; <out> the three outputs one after
  *                            the other
- *   mlp <dtype> <K> <unit> <batch> <height> <from> <to> <weights> <input> <out>
- *                            mlp_swiglu; <weights> holds the up then the gate matrix
+ *   mlp <dtype> <K> <unit> <batch> <height> <from> <to> <weights> <input> <out> [<down_unit>]
+ *                            mlp_swiglu; <weights> holds the up then the gate matrix, with <down_unit> the down
+ *                            projection's after them (the whole MLP as one layer)
  *   lmhead <dtype> <K> <unit> <batch> <height> <from> <to> <table> <input> <out>
  *   embed <dtype> <in_dim> <out_dim> <batch> <width> <from> <to> <table> <ids> <out>
  *                            tie_word_embeddings in its two modes
@@ -46,6 +47,7 @@
 #include <dlfcn.h>
 
 #include <chrono>
+#include <cstring>
 #include <cstdio>
 #include <cstdlib>
 #include <fstream>
@@ -301,6 +303,16 @@ static int run_api(Context *ctx) {
     EXPECT(ic.getWeightRequests()[1].dim == TensorDim(1, 1, 1024, 3072));
     EXPECT(ic.getOutputDimensions()[0] == TensorDim(1, 1, 4, 3072));
     EXPECT_THROW(ctx->createLayerObject("mlp_swiglu", {"unit=8", "disable_bias=false"}), exception::not_supported);
+    /* with down_unit: the whole MLP, the down projection's weight third, the output as wide as the model */
+    auto whole = ctx->createLayerObject("mlp_swiglu", {"unit=3072", "down_unit=1024", "disable_bias=true"});
+    InitLayerContext iw({TensorDim(1, 1, 4, 1024)}, "l0_ffn", Tformat::NCHW, Tdatatype::Q4_0, Tdatatype::FP32);
+    whole->finalize(iw);
+    EXPECT(iw.getWeightRequests().size() == 3 && iw.getWeightRequests()[2].name == "l0_ffn:down_weight");
+    EXPECT(iw.getWeightRequests()[2].dim == TensorDim(1, 1, 3072, 1024));
+    EXPECT(iw.getOutputDimensions()[0] == TensorDim(1, 1, 4, 1024));
+    auto odd = ctx->createLayerObject("mlp_swiglu", {"unit=3000", "down_unit=1024"});
+    InitLayerContext io({TensorDim(1, 1, 4, 1024)}, "odd", Tformat::NCHW, Tdatatype::Q4_K, Tdatatype::FP32);
+    EXPECT_THROW(odd->finalize(io), std::invalid_argument);
   }
   /* inference only */
   {
@@ -467,12 +479,16 @@ static int run_qkv(Context *ctx, char **a) {
   return 0;
 }
 
-static int run_mlp(Context *ctx, char **a) {
+static int run_mlp(Context *ctx, char **a, unsigned down_unit) {
   const std::string dt = a[0];
   const unsigned K = std::atoi(a[1]), N = std::atoi(a[2]), batch = std::atoi(a[3]), height = std::atoi(a[4]),
                  from = std::atoi(a[5]), to = std::atoi(a[6]);
   const std::string wpath = a[7], ipath = a[8], opath = a[9];
-  auto layer = ctx->createLayerObject("mlp_swiglu", {"unit=" + std::to_string(N), "disable_bias=true"});
+  std::vector<std::string> props = {"unit=" + std::to_string(N), "disable_bias=true"};
+  if (down_unit)
+    props.push_back("down_unit=" + std::to_string(down_unit));
+  const unsigned W = down_unit ? down_unit : N; /* the output's width */
+  auto layer = ctx->createLayerObject("mlp_swiglu", props);
   InitLayerContext ic({TensorDim(batch, 1, height, K)}, "mlp", Tformat::NCHW, dtype_of(dt), Tdatatype::FP32);
   layer->finalize(ic);
   RunLayerContext rc(ic);
@@ -482,13 +498,13 @@ static int run_mlp(Context *ctx, char **a) {
   }
   read_into(ipath, rc.getInput(0).getData<float>(), (size_t)batch * height * K * 4);
   float *out = rc.getOutput(0).getData<float>();
-  for (size_t i = 0; i < (size_t)batch * height * N; ++i)
+  for (size_t i = 0; i < (size_t)batch * height * W; ++i)
     out[i] = -12345.f;
   if (from == 0 && to == 0)
     layer->forwarding(rc, false);
   else
     layer->incremental_forwarding(rc, from, to, false);
-  write_from(opath, out, (size_t)batch * height * N * 4);
+  write_from(opath, out, (size_t)batch * height * W * 4);
   std::printf("MLP DONE\n");
   return 0;
 }
@@ -599,12 +615,12 @@ static int run_c5layer(Context *ctx, int iters) {
   auto ma = ctx->getContextData() ? ctx->getContextData()->getMemAllocator() : nullptr;
   auto unit = [](unsigned n) { return std::vector<std::string>{"unit=" + std::to_string(n), "disable_bias=true"}; };
   std::printf("{");
-  bool first = true;
+  bool first = true, fused_equal = true;
   for (int pinned = 0; pinned < 2; ++pinned) {
     for (int decode = 1; decode >= 0; --decode) {
       const unsigned h = decode ? 8 : 512;
       const auto mem = pinned ? ma : std::shared_ptr<MemAllocator>();
-      std::vector<BuiltLayer> seven, four;
+      std::vector<BuiltLayer> seven, four, three;
       seven.push_back(build(ctx, "fully_connected", unit(NQ), h, D, 1, 1, mem));
       seven.push_back(build(ctx, "fully_connected", unit(NKV), h, D, 1, 2, mem));
       seven.push_back(build(ctx, "fully_connected", unit(NKV), h, D, 1, 3, mem));
@@ -619,16 +635,39 @@ static int run_c5layer(Context *ctx, int iters) {
       four.push_back(build(ctx, "fully_connected", unit(D), h, NQ, 1, 14, mem));
       four.push_back(build(ctx, "mlp_swiglu", unit(FF), h, D, 1, 15, mem));
       four.push_back(build(ctx, "fully_connected", unit(D), h, FF, 1, 17, mem));
+      /* the whole MLP as one layer: the same three weights as four[2] and four[3] */
+      std::vector<std::string> mlp_props = unit(FF);
+      mlp_props.push_back("down_unit=" + std::to_string(D));
+      three.push_back(build(ctx, "qkv_layer",
+                            {"q_unit=" + std::to_string(NQ), "k_unit=" + std::to_string(NKV),
+                             "v_unit=" + std::to_string(NKV)},
+                            h, D, 3, 11, mem));
+      three.push_back(build(ctx, "fully_connected", unit(D), h, NQ, 1, 14, mem));
+      three.push_back(build(ctx, "mlp_swiglu", mlp_props, h, D, 1, 15, mem));
       const int n = decode ? iters : (iters + 9) / 10;
-      const double t7 = time_chain(seven, decode, n), t4 = time_chain(four, decode, n);
-      std::printf("%s\"%s_%s_seven_fully_connected_us\": %.2f, \"%s_%s_qkv_fc_mlp_swiglu_fc_us\": %.2f", first ? "" : ", ",
-                  decode ? "decode_row" : "prefill_512_rows", pinned ? "allocator_memory" : "ordinary_memory", t7,
-                  decode ? "decode_row" : "prefill_512_rows", pinned ? "allocator_memory" : "ordinary_memory", t4);
+      const double t7 = time_chain(seven, decode, n), t4 = time_chain(four, decode, n),
+                   t3 = time_chain(three, decode, n);
+      /* the one-layer MLP against the two layers it replaces, the hidden rows handed over on the host */
+      {
+        const unsigned rows = decode ? 1 : h;
+        std::memcpy(four[3].rc->getInput(0).getData<float>(), four[2].rc->getOutput(0).getData<float>(),
+                    (size_t)rows * FF * sizeof(float));
+        four[3].layer->incremental_forwarding(*four[3].rc, decode ? 3 : 0, decode ? 4 : h, false);
+        if (std::memcmp(four[3].rc->getOutput(0).getData<float>(), three[2].rc->getOutput(0).getData<float>(),
+                        (size_t)rows * D * sizeof(float)) != 0)
+          fused_equal = false;
+      }
+      const char *rows_name = decode ? "decode_row" : "prefill_512_rows";
+      const char *mem_name = pinned ? "allocator_memory" : "ordinary_memory";
+      std::printf("%s\"%s_%s_seven_fully_connected_us\": %.2f, \"%s_%s_qkv_fc_mlp_swiglu_fc_us\": %.2f, "
+                  "\"%s_%s_qkv_fc_mlp_us\": %.2f",
+                  first ? "" : ", ", rows_name, mem_name, t7, rows_name, mem_name, t4, rows_name, mem_name, t3);
       first = false;
     }
   }
-  std::printf("}\n");
-  return 0;
+  std::printf(", \"one_layer_mlp_equals_mlp_swiglu_then_fully_connected_bit_for_bit\": %s}\n",
+              fused_equal ? "true" : "false");
+  return fused_equal ? 0 : 1;
 }
 
 static int run_moelayer(Context *ctx, int iters) {
@@ -719,8 +758,8 @@ int main(int argc, char **argv) {
       return run_moex(ctx, argv + 3);
     if (mode == "qkv" && argc == 14)
       return run_qkv(ctx, argv + 3);
-    if (mode == "mlp" && argc == 13)
-      return run_mlp(ctx, argv + 3);
+    if (mode == "mlp" && (argc == 13 || argc == 14))
+      return run_mlp(ctx, argv + 3, argc == 14 ? (unsigned)std::atoi(argv[13]) : 0);
     if ((mode == "lmhead" || mode == "embed") && argc == 13)
       return run_tie(ctx, mode == "lmhead", argv + 3);
     std::printf("bad arguments for mode %s (argc %d)\n", mode.c_str(), argc);

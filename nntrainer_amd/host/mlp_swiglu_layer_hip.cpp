@@ -17,6 +17,8 @@ void MlpSwiGLULayerHip::setProperty(const std::vector<std::string> &values) {
     const std::string &key = kv.first, &val = kv.second;
     if (key == "unit") {
       unit = hipq_host::parse_positive(key, val);
+    } else if (key == "down_unit") {
+      down_unit = hipq_host::parse_positive(key, val);
     } else if (key == "disable_bias") {
       NNTR_THROW_IF(!hipq_host::parse_bool(key, val), exception::not_supported)
         << "MlpSwiGLULayerHip has no bias (the application's MLP FCs disable it, causal_lm.cpp:675-686)";
@@ -48,9 +50,13 @@ void MlpSwiGLULayerHip::finalize(InitLayerContext &context) {
   NNTR_THROW_IF(in_dim.width() % block != 0, std::invalid_argument)
     << "input width " << in_dim.width() << " is not a multiple of the quantization block " << block;
 
+  NNTR_THROW_IF(down_unit && unit % block != 0, std::invalid_argument)
+    << "unit " << unit << " is not a multiple of the quantization block " << block
+    << " (the rows the down projection takes)";
+
   std::vector<TensorDim> output_dims(1);
   output_dims[0] = in_dim;
-  output_dims[0].width(unit);
+  output_dims[0].width(down_unit ? down_unit : unit);
   output_dims[0].setTensorType({context.getFormat(), context.getActivationDataType()});
   context.setOutputDimensions(output_dims);
 
@@ -60,6 +66,12 @@ void MlpSwiGLULayerHip::finalize(InitLayerContext &context) {
                                                  "up_weight", true);
   weight_idx[Params::gate] = context.requestWeight(weight_dim, Initializer::NONE, WeightRegularizer::NONE, 1.0f,
                                                    0.0f, "gate_weight", true);
+  if (down_unit) {
+    TensorDim down_dim(1, 1, unit, down_unit,
+                       TensorDim::TensorType(context.getFormat(), context.getWeightDataType()), 0b0011);
+    weight_idx[Params::down] = context.requestWeight(down_dim, Initializer::NONE, WeightRegularizer::NONE, 1.0f,
+                                                     0.0f, "down_weight", true);
+  }
 }
 
 void MlpSwiGLULayerHip::run(RunLayerContext &context, const float *x, float *y, unsigned int rows) const {
@@ -69,6 +81,14 @@ void MlpSwiGLULayerHip::run(RunLayerContext &context, const float *x, float *y, 
   NNTR_THROW_IF(dtype < 0, std::invalid_argument) << "Error: unsupported datatype";
   const int64_t K = wu.height(), N = wu.width();
   const hipq_host::WeightSpec spec{dtype, hipq_host::framework_layout(dtype), N, K};
+  if (down_unit) {
+    const Tensor &wd = context.getWeight(weight_idx[Params::down]);
+    const hipq_host::WeightSpec dspec{dtype, hipq_host::framework_layout(dtype), (int64_t)wd.width(),
+                                      (int64_t)wd.height()};
+    hipq_host::mlp_swiglu_down(hipq_host::global_cache(), wu.getData<uint8_t>(), wg.getData<uint8_t>(), spec,
+                               wd.getData<uint8_t>(), dspec, x, rows, K, y, dspec.N);
+    return;
+  }
   hipq_host::mlp_swiglu(hipq_host::global_cache(), wu.getData<uint8_t>(), wg.getData<uint8_t>(), spec, x, rows, K, y,
                         N);
 }

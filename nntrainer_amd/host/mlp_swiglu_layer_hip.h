@@ -13,6 +13,12 @@
  * the MLP's hidden size). It requests "up_weight" then "gate_weight", [in_width x unit] of the
  * model's weight type: the order in which the two FCs' weights lie in a model file, so files
  * written for the three-layer form load unchanged.
+ *
+ * With the property `down_unit` (the model's width) the layer is the whole MLP of createMlp
+ * (causal_lm.cpp:671-705), the FC "ffn_down" included: it requests "down_weight" [unit x down_unit]
+ * after the other two (again the file's order), its output is [rows x down_unit], and the hidden
+ * rows never leave the device (hipq_mlp_swiglu_down): one call and one wait where the layers
+ * "mlp_swiglu" + "fully_connected" move the hidden rows to the host and back.
  */
 #ifndef HIPQ_MLP_SWIGLU_LAYER_HIP_H
 #define HIPQ_MLP_SWIGLU_LAYER_HIP_H
@@ -50,11 +56,12 @@ public:
   inline static const std::string type = "mlp_swiglu";
 
 private:
-  enum Params { up, gate };
+  enum Params { up, gate, down };
   void run(RunLayerContext &context, const float *x, float *y, unsigned int rows) const;
 
   unsigned int unit = 0;
-  std::array<unsigned int, 2> weight_idx = {0, 0};
+  unsigned int down_unit = 0; /* 0: the gated half only */
+  std::array<unsigned int, 3> weight_idx = {0, 0, 0};
 };
 
 } // namespace nntrainer

@@ -171,6 +171,52 @@ def test_gpt_oss_moe_router_bias_and_host_memory(hipq, cr):
         w.destroy()
 
 
+@pytest.mark.parametrize("kind,m,k,n,nd", [("q4_0", 1, 1024, 3072, 1024), ("q4_K", 1, 2048, 768, 2048),
+                                           ("q6_K", 3, 512, 256, 512), ("q4_0", 24, 1024, 3072, 1024),
+                                           ("q4_K", 5, 1024, 512, 768), ("q4_K", 80, 1024, 1024, 512),
+                                           ("q4_0", 1, 96, 320, 64)])
+@pytest.mark.parametrize("mem", ["device", "host"])
+def test_mlp_swiglu_down_is_the_two_calls_and_matches_the_oracle(hipq, cr, kind, m, k, n, nd, mem):
+    """hipq_mlp_swiglu_down: out = swiglu(a . Wup^T, a . Wgate^T) . Wdown^T, the four layers of
+    CausalLM::createMlp (causal_lm.cpp:671-705) as one call. Bit for bit what hipq_mlp_swiglu followed by
+    hipq_matmul give, and within the fp32 tolerance of the oracle's products, its swiglu and its down
+    product on the oracle's own hidden rows."""
+    import gpu_util as gu
+    import torch
+    wa = cr.quantize_weights(cr.oracle(), kind, synth.normal(8800 + n, (n, k), 0.05))
+    wm = cr.quantize_weights(cr.oracle(), kind, synth.normal(8801 + n, (n, k), 0.05))
+    wd = cr.quantize_weights(cr.oracle(), kind, synth.normal(8802 + n, (nd, n), 0.05))
+    a = synth.normal(8803 + m, (m, k))
+    hidden = cr.swiglu(cr.gemm(cr.oracle(), kind, a, wa, n), cr.gemm(cr.oracle(), kind, a, wm, n))
+    ref = cr.gemm(cr.oracle(), kind, hidden, wd, nd)
+    ha, hm, hd = capi.Weight(kind, n, k, wa), capi.Weight(kind, n, k, wm), capi.Weight(kind, nd, n, wd)
+    try:
+        two = torch.full((m, nd), float("nan"), device="cuda")
+        h = torch.full((m, n), float("nan"), device="cuda")
+        capi.mlp_swiglu(ha, hm, gu.dev(a), m, h, stream=gu.stream())
+        capi.matmul(hd, h, m, two, stream=gu.stream())
+        torch.cuda.synchronize()
+        if mem == "device":
+            ldo = nd + 4
+            out = torch.full((m, ldo), float("nan"), device="cuda")
+            capi.mlp_swiglu_down(ha, hm, hd, gu.dev(a), m, out, ldo=ldo, stream=gu.stream())
+            torch.cuda.synchronize()
+            assert torch.isnan(out[:, nd:]).all(), "the call wrote between the rows of the output"
+            got = out[:, :nd].cpu().numpy()
+        else:
+            got = np.full((m, nd), np.nan, np.float32)
+            capi.mlp_swiglu_down(ha, hm, hd, a, m, got, mem=capi.MEM_HOST)
+        assert not np.isnan(got).any()
+        assert np.array_equal(got.view(np.uint32), two.cpu().numpy().view(np.uint32))
+        assert gu.rel_err(got, ref) <= gu.TOL, gu.rel_err(got, ref)
+        if k != n:
+            with pytest.raises(capi.HipqError):   # a down projection that does not fit the hidden rows
+                capi.mlp_swiglu_down(ha, hm, ha, gu.dev(a), m, two, stream=gu.stream())
+    finally:
+        for w in (ha, hm, hd):
+            w.destroy()
+
+
 @pytest.mark.parametrize("kind,m,k,n", [("q4_0", 1, 1024, 3072), ("q4_K", 1, 2048, 768), ("q6_K", 1, 1024, 512),
                                         ("q4_0", 1, 96, 320),      # K below one chunk unit: not fused
                                         ("q4_0", 24, 1024, 3072), ("q4_K", 5, 1024, 512)])

@@ -175,6 +175,12 @@ def test_grouped_calls_on_a_few_page_locked_rows(hipq, cr, kind, m):
         capi.mlp_swiglu(ws[1], ws[2], gu.dev(a), m, want, stream=gu.stream())
         torch.cuda.synchronize()
         assert np.array_equal(po.arr.view(np.uint32), want.cpu().numpy().view(np.uint32))
+        # the whole MLP in one call: the hidden rows stay on the device, the output is written in place
+        capi.mlp_swiglu_down(ws[1], ws[2], ws[0], pa.addr, m, pcs[0].addr, mem=capi.MEM_HOST)
+        whole = torch.full((m, ns[0]), float("nan"), device="cuda")
+        capi.matmul(ws[0], want, m, whole, stream=gu.stream())
+        torch.cuda.synchronize()
+        assert np.array_equal(pcs[0].arr.view(np.uint32), whole.cpu().numpy().view(np.uint32))
     finally:
         for p in [pa, po] + pcs:
             p.free()

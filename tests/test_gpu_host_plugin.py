@@ -387,3 +387,30 @@ def test_mlp_swiglu_layer(cr, tmp_path, kind, k, n, batch, height, frm, to):
         ref = cr.swiglu(y, z)
         assert np.abs(got[b, :rows] - ref).max() / np.abs(ref).max() <= TOL
         assert np.all(got[b, rows:] == -12345.0)
+
+
+@pytest.mark.parametrize("kind,k,n,nd,batch,height,frm,to", [("q4_0", 1024, 3072, 1024, 1, 1, 5, 6),   # decode row
+                                                             ("q4_K", 1024, 768, 1024, 1, 20, 0, 0),    # forwarding
+                                                             ("q4_0", 512, 256, 512, 2, 8, 0, 5)])      # prefill step
+def test_mlp_swiglu_layer_with_the_down_projection(cr, tmp_path, kind, k, n, nd, batch, height, frm, to):
+    """mlp_swiglu with down_unit: the four layers of CausalLM::createMlp (causal_lm.cpp:671-705) as one, the
+    hidden rows never on the host; weights in the file order of the three FCs."""
+    up, fup = _framework_bytes(cr, kind, synth.normal(8600, (n, k), 0.05), n, k)
+    gate, fgate = _framework_bytes(cr, kind, synth.normal(8601, (n, k), 0.05), n, k)
+    down, fdown = _framework_bytes(cr, kind, synth.normal(8602, (nd, n), 0.05), nd, n)
+    x = synth.normal(8603 + height, (batch, height, k))
+    with open(tmp_path / "w.bin", "wb") as f:
+        f.write(fup.tobytes())
+        f.write(fgate.tobytes())
+        f.write(fdown.tobytes())
+    x.tofile(tmp_path / "x.bin")
+    out = _run(["mlp", kind, k, n, batch, height, frm, to, tmp_path / "w.bin", tmp_path / "x.bin", tmp_path / "y.bin",
+                nd])
+    assert "MLP DONE" in out
+    got = np.fromfile(tmp_path / "y.bin", np.float32).reshape(batch, height, nd)
+    rows = height if to == 0 else to - frm
+    for b in range(batch):
+        hidden = cr.swiglu(cr.gemm(cr.oracle(), kind, x[b, :rows], up, n), cr.gemm(cr.oracle(), kind, x[b, :rows], gate, n))
+        ref = cr.gemm(cr.oracle(), kind, hidden, down, nd)
+        assert np.abs(got[b, :rows] - ref).max() / np.abs(ref).max() <= TOL
+        assert np.all(got[b, rows:] == -12345.0)
