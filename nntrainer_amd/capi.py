@@ -235,12 +235,12 @@ def matmul_noalloc(w, a, m, c, lda=None, ldc=None, stream=None):
     check(lib().hipq_matmul_noalloc(w.handle, _addr(a), m, lda or w.k, _addr(c), ldc or w.n, stream))
 
 
-def matmul_multi(ws, a, m, cs, ldc=None, mem=MEM_DEVICE, stream=None):
+def matmul_multi(ws, a, m, cs, ldc=None, mem=MEM_DEVICE, stream=None, lda=None):
     n = len(ws)
     hs = (C.c_void_p * n)(*[w.handle.value for w in ws])
     cp = (C.c_void_p * n)(*[_addr(c) for c in cs])
     ld = (C.c_int64 * n)(*(ldc if ldc is not None else [w.n for w in ws]))
-    check(lib().hipq_matmul_multi(n, hs, _addr(a), m, ws[0].k, cp, ld, mem, stream))
+    check(lib().hipq_matmul_multi(n, hs, _addr(a), m, lda or ws[0].k, cp, ld, mem, stream))
 
 
 def mlp_swiglu(w_act, w_mul, a, m, out, lda=None, ldo=None, mem=MEM_DEVICE, stream=None):

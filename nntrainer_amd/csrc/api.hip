@@ -56,6 +56,10 @@ struct Workspace {
   /* a page-locked word the last launch of such a call writes and the host polls */
   uint32_t *done = nullptr;
   uint32_t done_seq = 0;
+  /* a second stream and an event: a prefill's finished rows go back to page-locked host memory on it
+   * while the kernels work on the following rows (RowSteps) */
+  hipStream_t copy = nullptr;
+  hipEvent_t step_done = nullptr;
   /* held while a call enqueues its launches: two threads that name the same stream
    * must not interleave their kernels (the second would quantize into the scratch
    * the first one's product has not read yet) */
@@ -493,6 +497,74 @@ int stage_copy(bool to_device, void *dev, void *host, size_t hpitch, size_t widt
   return HIPQ_OK;
 }
 
+/* Rows of a host-memory call in steps. With page-locked operands the copies are asynchronous, and
+ * the link carries both directions at once: while the kernels work on one step's rows, the copy
+ * engines take the step before out (on a second stream) and, behind the kernels, bring the next
+ * one in. A call of 512 rows and more is cut into steps of 256 (the last one takes the remainder)
+ * where the caller says that every step's product has the bits of the whole call's, and where the
+ * outputs are at least twice the input and 16 MiB: measured on page-locked memory (us, one piece -> steps),
+ * 12288 x 4096 with 512 / 1024 / 2048 rows 675 -> 613 / 1315 -> 1102 / 2598 -> 2081, 4096 x 1024
+ * 229 -> 225 / 428 -> 400 / 825 -> 754; with the input the larger side (1024 x 3072: 190 -> 214 /
+ * 347 -> 395 / 661 -> 763) the steps' extra waits cost more than the little output they hide. */
+struct RowSteps {
+  static constexpr int64_t STEP = 256;
+  static constexpr int64_t MIN_OUT_BYTES = (int64_t)16 << 20; /* below, a step's copy is too short to hide anything */
+  hipStream_t s = nullptr, cs = nullptr;
+  hipEvent_t ev = nullptr;
+  int64_t M = 0, step = 0; /* step 0: the whole call in one piece */
+  bool pending = false;
+
+  int plan(hipStream_t stream, int64_t rows, bool steps_keep_bits, const float *A, int64_t in_cols, int count,
+           float *const *C, int64_t out_cols) {
+    s = stream;
+    M = rows;
+    step = 0;
+    if (!steps_keep_bits || rows < 2 * STEP || out_cols < 2 * in_cols || rows * out_cols * 4 < MIN_OUT_BYTES ||
+        !is_pinned(A))
+      return HIPQ_OK;
+    for (int i = 0; i < count; ++i)
+      if (!is_pinned(C[i])) return HIPQ_OK;
+    {
+      std::lock_guard<std::mutex> lk(g.mu);
+      Workspace &w = g.ws[s];
+      if (!w.copy) HIPQ_HIP(hipStreamCreateWithFlags(&w.copy, hipStreamNonBlocking));
+      if (!w.step_done) HIPQ_HIP(hipEventCreateWithFlags(&w.step_done, hipEventDisableTiming));
+      cs = w.copy;
+      ev = w.step_done;
+    }
+    step = STEP;
+    return HIPQ_OK;
+  }
+  /* the rows of the piece that starts at r0 */
+  int64_t rows_at(int64_t r0) const { return (!step || M - r0 < 2 * step) ? M - r0 : step; }
+  int in(float *dev, const float *host, int64_t lda, int64_t K, int64_t r0, int64_t n) const {
+    return stage_copy(true, dev + r0 * K, (void *)(host + r0 * lda), (size_t)lda * 4, (size_t)K * 4, (size_t)n, s);
+  }
+  /* rows [r0, r0 + n) of a dense device result [M x N] to the caller's matrix; in one piece this returns
+   * with the host bytes written, in steps finish() does */
+  int out(const float *dev, float *host, int64_t ldc, int64_t N, int64_t r0, int64_t n, bool first_of_step = true) {
+    if (!step)
+      return stage_copy(false, (void *)(dev + r0 * N), host + r0 * ldc, (size_t)ldc * 4, (size_t)N * 4, (size_t)n, s);
+    if (first_of_step) {
+      HIPQ_HIP(hipEventRecord(ev, s));
+      HIPQ_HIP(hipStreamWaitEvent(cs, ev, 0));
+    }
+    pending = true;
+    HIPQ_HIP(hipMemcpy2DAsync(host + r0 * ldc, (size_t)ldc * 4, dev + r0 * N, (size_t)N * 4, (size_t)N * 4, (size_t)n,
+                              hipMemcpyDeviceToHost, cs));
+    return HIPQ_OK;
+  }
+  int finish() {
+    if (!pending) return HIPQ_OK;
+    pending = false;
+    HIPQ_HIP(hipStreamSynchronize(cs));
+    return HIPQ_OK;
+  }
+  ~RowSteps() { /* a call that fails half way still owns the caller's memory until its copies end */
+    if (pending) (void)hipStreamSynchronize(cs);
+  }
+};
+
 std::recursive_mutex &enqueue_lock(hipStream_t s) {
   std::lock_guard<std::mutex> lk(g.mu);
   return g.ws[s].enqueue; /* nodes of the map do not move */
@@ -711,6 +783,29 @@ int matmul_device(hipq_weight_t w, const float *A, int64_t M, int64_t lda, float
   return multiply(w, qa, M, C, ldc, s, each_row);
 }
 
+/* Whether the products of a call of M rows against these weights have the same bits when the rows are
+ * multiplied in steps of RowSteps::STEP (the last one up to twice that). Q4_0: every kernel has the
+ * reference's bits, always. Q4_K and Q6_K: where the whole call and every step take the prefill GEMM
+ * on whole K (a row's sums there depend on neither the other rows nor the tile height; a product in
+ * parts of K adds in another order). The weights' tile copies are made here, as the products would. */
+int steps_keep_bits(int count, const hipq_weight_t *w, int64_t M, bool *keep) {
+  *keep = false;
+  if (M < 2 * RowSteps::STEP) return HIPQ_OK;
+  const int64_t sizes[3] = {M, RowSteps::STEP, RowSteps::STEP + M % RowSteps::STEP};
+  for (int i = 0; i < count; ++i) {
+    if (w[i]->dtype == HIPQ_Q4_0) continue;
+    for (int64_t m : sizes)
+      if (!wants_tiled(w[i], m)) return HIPQ_OK;
+    if (!w[i]->gt_base)
+      if (int rc = hipq::ensure_gemm_tiles(const_cast<hipq_weight *>(w[i]))) return rc;
+    for (int64_t m : sizes)
+      if (w[i]->dtype == HIPQ_Q4_K ? hipq::gemm_q4k_split_bytes(w[i], m) : hipq::gemm_q6k_split_bytes(w[i], m))
+        return HIPQ_OK;
+  }
+  *keep = true;
+  return HIPQ_OK;
+}
+
 struct DevBuf {
   void *p = nullptr;
   ~DevBuf() {
@@ -774,6 +869,8 @@ int hipq_shutdown(void) {
     if (kv.second.io) (void)hipFree(kv.second.io);
     if (kv.second.pin) (void)hipHostFree(kv.second.pin);
     if (kv.second.done) (void)hipHostFree(kv.second.done);
+    if (kv.second.step_done) (void)hipEventDestroy(kv.second.step_done);
+    if (kv.second.copy) (void)hipStreamDestroy(kv.second.copy);
     for (void *p : kv.second.retired) (void)hipFree(p);
   }
   g.ws.clear();
@@ -815,6 +912,8 @@ int hipq_stream_release(void *stream) {
   if (it->second.io) (void)hipFree(it->second.io);
   if (it->second.pin) (void)hipHostFree(it->second.pin);
   if (it->second.done) (void)hipHostFree(it->second.done);
+  if (it->second.step_done) (void)hipEventDestroy(it->second.step_done);
+  if (it->second.copy) (void)hipStreamDestroy(it->second.copy);
   for (void *p : it->second.retired) (void)hipFree(p);
   el.unlock();
   el.release();
@@ -1115,9 +1214,18 @@ int hipq_matmul(hipq_weight_t w, const float *A, int64_t M, int64_t lda, float *
     }
     if (rc) return rc;
   }
-  if ((rc = stage_copy(true, dA, (void *)A, (size_t)lda * 4, (size_t)w->K * 4, (size_t)M, s))) return rc;
-  if ((rc = matmul_device(w, dA, M, w->K, dC, w->N, s, sc))) return rc;
-  return stage_copy(false, dC, C, (size_t)ldc * 4, (size_t)w->N * 4, (size_t)M, s);
+  bool keep = false;
+  if ((rc = steps_keep_bits(1, &w, M, &keep))) return rc;
+  RowSteps steps;
+  if ((rc = steps.plan(s, M, keep, A, w->K, 1, &C, w->N))) return rc;
+  for (int64_t r0 = 0; r0 < M;) {
+    const int64_t n = steps.rows_at(r0);
+    if ((rc = steps.in(dA, A, lda, w->K, r0, n))) return rc;
+    if ((rc = matmul_device(w, dA + r0 * w->K, n, w->K, dC + r0 * w->N, w->N, s, sc))) return rc;
+    if ((rc = steps.out(dC, C, ldc, w->N, r0, n))) return rc;
+    r0 += n;
+  }
+  return steps.finish();
 }
 
 int hipq_matmul_each_row(hipq_weight_t w, const float *A, int64_t rows, int64_t lda, float *C, int64_t ldc,
@@ -1214,8 +1322,8 @@ int hipq_mlp_swiglu(hipq_weight_t w_act, hipq_weight_t w_mul, const float *A, in
     if (dio.begin(s, A, M, lda, K, 1, &out, &ldo, &N, &rc)) {
       if ((rc = dio.fetch(dA, K))) return rc;
       h_out = dio.outs[0].dev, h_ld = dio.outs[0].dld;
-    } else if (rc || (rc = stage_copy(true, dA, (void *)A, (size_t)lda * 4, (size_t)K * 4, (size_t)M, s)))
-      return rc;
+    } else if (rc || (M == 1 && (rc = stage_copy(true, dA, (void *)A, (size_t)lda * 4, (size_t)K * 4, 1, s))))
+      return rc; /* more rows cross below, in steps */
     a_dev = dA;
     a_ld = K;
     if (M == 1 && hipq::gemv_fuses_swiglu(w_act, w_mul, dA)) {
@@ -1227,14 +1335,26 @@ int hipq_mlp_swiglu(hipq_weight_t w_act, hipq_weight_t w_mul, const float *A, in
   const hipq_weight_t ws[2] = {w_act, w_mul};
   float *const cs[2] = {dY, dZ};
   const int64_t lds[2] = {N, N};
+  if (mem == HIPQ_MEM_HOST && !h_out) { /* rows through the copy engines, in steps where that keeps the bits */
+    bool keep = false;
+    if ((rc = steps_keep_bits(2, ws, M, &keep))) return rc;
+    RowSteps steps;
+    if ((rc = steps.plan(s, M, keep, A, K, 1, &out, N))) return rc;
+    for (int64_t r0 = 0; r0 < M;) {
+      const int64_t n = steps.rows_at(r0);
+      float *const cr[2] = {dY + r0 * N, dZ + r0 * N};
+      if (M > 1 && (rc = steps.in(dA, A, lda, K, r0, n))) return rc;
+      if ((rc = hipq_matmul_multi(2, ws, dA + r0 * K, n, K, cr, lds, HIPQ_MEM_DEVICE, stream))) return rc;
+      if ((rc = hipq::launch_swiglu_rows(cr[0], cr[1], n, N, dO + r0 * N, N, s))) return rc;
+      if ((rc = steps.out(dO, out, ldo, N, r0, n))) return rc;
+      r0 += n;
+    }
+    return steps.finish();
+  }
   if ((rc = hipq_matmul_multi(2, ws, a_dev, M, a_ld, cs, lds, HIPQ_MEM_DEVICE, stream))) return rc;
   if (mem == HIPQ_MEM_DEVICE) return hipq::launch_swiglu_rows(dY, dZ, M, N, out, ldo, s);
-  if (h_out) {
-    if ((rc = hipq::launch_swiglu_rows(dY, dZ, M, N, h_out, h_ld, s))) return rc;
-    return dio.finish();
-  }
-  if ((rc = hipq::launch_swiglu_rows(dY, dZ, M, N, dO, N, s))) return rc;
-  return stage_copy(false, dO, out, (size_t)ldo * 4, (size_t)N * 4, (size_t)M, s);
+  if ((rc = hipq::launch_swiglu_rows(dY, dZ, M, N, h_out, h_ld, s))) return rc;
+  return dio.finish();
 }
 
 int hipq_mlp_swiglu_down(hipq_weight_t w_act, hipq_weight_t w_mul, hipq_weight_t w_down, const float *A, int64_t M,
@@ -1277,24 +1397,44 @@ int hipq_mlp_swiglu_down(hipq_weight_t w_act, hipq_weight_t w_mul, hipq_weight_t
       o_dev = dio.outs[0].dev, o_ld = dio.outs[0].dld;
       direct = true;
     } else {
-      if (rc || (rc = stage_copy(true, dA, (void *)A, (size_t)lda * 4, (size_t)K * 4, (size_t)M, s))) return rc;
+      if (rc) return rc;
       o_dev = dO, o_ld = Nd;
     }
     a_dev = dA, a_ld = K;
   }
-  if (M == 1 && hipq::gemv_fuses_swiglu(w_act, w_mul, a_dev)) {
-    if ((rc = hipq::launch_gemv_fused_swiglu(w_act, w_mul, a_dev, dH, s))) return rc;
-  } else {
-    const hipq_weight_t ws[2] = {w_act, w_mul};
-    float *const cs[2] = {dY, dZ};
-    const int64_t lds[2] = {N, N};
-    if ((rc = hipq_matmul_multi(2, ws, a_dev, M, a_ld, cs, lds, HIPQ_MEM_DEVICE, stream))) return rc;
-    if ((rc = hipq::launch_swiglu_rows(dY, dZ, M, N, dH, N, s))) return rc;
+  const hipq_weight_t ws[2] = {w_act, w_mul};
+  const int64_t lds[2] = {N, N};
+  /* rows [r0, r0 + n): the gated half into dH, the down projection into the output */
+  auto rows = [&](int64_t r0, int64_t n) -> int {
+    const float *a = a_dev + r0 * a_ld;
+    int rr;
+    if (n == 1 && hipq::gemv_fuses_swiglu(w_act, w_mul, a)) {
+      if ((rr = hipq::launch_gemv_fused_swiglu(w_act, w_mul, a, dH + r0 * N, s))) return rr;
+    } else {
+      float *const cr[2] = {dY + r0 * N, dZ + r0 * N};
+      if ((rr = hipq_matmul_multi(2, ws, a, n, a_ld, cr, lds, HIPQ_MEM_DEVICE, stream))) return rr;
+      if ((rr = hipq::launch_swiglu_rows(cr[0], cr[1], n, N, dH + r0 * N, N, s))) return rr;
+    }
+    return hipq_matmul(w_down, dH + r0 * N, n, N, o_dev + r0 * o_ld, o_ld, HIPQ_MEM_DEVICE, stream);
+  };
+  if (mem == HIPQ_MEM_DEVICE || direct) {
+    if ((rc = rows(0, M))) return rc;
+    return direct ? dio.finish() : HIPQ_OK;
   }
-  if ((rc = hipq_matmul(w_down, dH, M, N, o_dev, o_ld, HIPQ_MEM_DEVICE, stream))) return rc;
-  if (mem == HIPQ_MEM_DEVICE) return HIPQ_OK;
-  if (direct) return dio.finish();
-  return stage_copy(false, dO, out, (size_t)ldo * 4, (size_t)Nd * 4, (size_t)M, s);
+  /* host rows through the copy engines, in steps where that keeps the bits */
+  const hipq_weight_t all[3] = {w_act, w_mul, w_down};
+  bool keep = false;
+  if ((rc = steps_keep_bits(3, all, M, &keep))) return rc;
+  RowSteps steps;
+  if ((rc = steps.plan(s, M, keep, A, K, 1, &out, Nd))) return rc;
+  for (int64_t r0 = 0; r0 < M;) {
+    const int64_t n = steps.rows_at(r0);
+    if ((rc = steps.in(dA, A, lda, K, r0, n))) return rc;
+    if ((rc = rows(r0, n))) return rc;
+    if ((rc = steps.out(dO, out, ldo, Nd, r0, n))) return rc;
+    r0 += n;
+  }
+  return steps.finish();
 }
 
 int hipq_matmul_multi(int count, const hipq_weight_t *w, const float *A, int64_t M, int64_t lda,
@@ -1337,16 +1477,30 @@ int hipq_matmul_multi(int count, const hipq_weight_t *w, const float *A, int64_t
       return dio.finish();
     }
     if (rc) return rc;
-    if ((rc = stage_copy(true, io, (void *)A, (size_t)lda * 4, (size_t)Kh * 4, (size_t)M, s))) return rc;
     for (int i = 0; i < count; ++i) {
       dC[i] = (float *)((char *)io + off[i]);
       dld[i] = w[i]->N;
     }
-    if ((rc = hipq_matmul_multi(count, w, (const float *)io, M, Kh, dC.data(), dld.data(), HIPQ_MEM_DEVICE, stream)))
-      return rc;
-    for (int i = 0; i < count; ++i)
-      if ((rc = stage_copy(false, dC[i], C[i], (size_t)ldc[i] * 4, (size_t)w[i]->N * 4, (size_t)M, s))) return rc;
-    return HIPQ_OK;
+    /* rows through the copy engines, in steps where that keeps the bits */
+    bool keep = false;
+    if ((rc = steps_keep_bits(count, w, M, &keep))) return rc;
+    RowSteps steps;
+    int64_t out_cols = 0;
+    for (int i = 0; i < count; ++i) out_cols += w[i]->N;
+    if ((rc = steps.plan(s, M, keep, A, Kh, count, C, out_cols))) return rc;
+    std::vector<float *> dCr(count);
+    for (int64_t r0 = 0; r0 < M;) {
+      const int64_t n = steps.rows_at(r0);
+      if ((rc = steps.in((float *)io, A, lda, Kh, r0, n))) return rc;
+      for (int i = 0; i < count; ++i) dCr[i] = dC[i] + r0 * dld[i];
+      if ((rc = hipq_matmul_multi(count, w, (const float *)io + r0 * Kh, n, Kh, dCr.data(), dld.data(), HIPQ_MEM_DEVICE,
+                                  stream)))
+        return rc;
+      for (int i = 0; i < count; ++i)
+        if ((rc = steps.out(dC[i], C[i], ldc[i], w[i]->N, r0, n, i == 0))) return rc;
+      r0 += n;
+    }
+    return steps.finish();
   }
   if (M == 1 && hipq::gemv_fuses_quantizer_multi(count, w, A))
     return hipq::launch_gemv_fused_multi(count, w, A, C, s);

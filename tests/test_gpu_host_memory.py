@@ -186,3 +186,63 @@ def test_grouped_calls_on_a_few_page_locked_rows(hipq, cr, kind, m):
             p.free()
         for w in ws:
             w.destroy()
+
+
+@pytest.mark.parametrize("kind,m,k,n,pad", [
+    ("q4_0", 1400, 1024, 3072, 0),      # five steps of 256 rows, the last of 376
+    ("q4_0", 2100, 1024, 2048, 8),      # eight steps; strided rows on both sides
+    ("q4_K", 700, 2048, 12288, 0),      # every step takes the prefill GEMM on whole K: two steps
+    ("q4_K", 1100, 2048, 4096, 0),      # a step would run in parts of K (other bits): one piece
+    ("q6_K", 1100, 1024, 4096, 4),
+    ("q4_0", 512, 1024, 3072, 0),       # outputs of 6 MB: one piece
+])
+def test_prefill_rows_in_steps_give_the_device_bits(hipq, cr, kind, m, k, n, pad):
+    """512 rows and more in page-locked memory with outputs of 16 MiB and at least twice the input cross in
+    steps of 256: a step's rows come in and the step before goes out while the kernels work. Every entry point that takes host rows gives the bits of its
+    device-memory call on the whole matrix, twice in a row."""
+    import gpu_util as gu
+    import torch
+    nd = 1024
+    mk = lambda j, rows, cols: capi.Weight(kind, rows, cols, cr.quantize_weights(
+        cr.oracle(), kind, synth.normal(9700 + j, (rows, cols), 0.05)))
+    w, w2, wd = mk(0, n, k), mk(1, n, k), mk(2, nd, n)
+    a = synth.normal(9710 + m, (m, k))
+    lda, ldc = k + pad, n + pad
+    pa = _Pinned((m, lda), 7e9)
+    pa.arr[:, :k] = a
+    pc, pc2, po, pd = _Pinned((m, ldc)), _Pinned((m, n)), _Pinned((m, n)), _Pinned((m, nd))
+    try:
+        da = gu.dev(a)
+        want = torch.empty((m, n), device="cuda")
+        want2 = torch.empty((m, n), device="cuda")
+        capi.matmul_multi([w, w2], da, m, [want, want2], stream=gu.stream())
+        single = torch.empty((m, n), device="cuda")
+        capi.matmul(w, da, m, single, stream=gu.stream())
+        act = torch.empty((m, n), device="cuda")
+        capi.mlp_swiglu(w, w2, da, m, act, stream=gu.stream())
+        down = torch.empty((m, nd), device="cuda")
+        capi.mlp_swiglu_down(w, w2, wd, da, m, down, stream=gu.stream())
+        torch.cuda.synchronize()
+        bits = lambda t: t.cpu().numpy().view(np.uint32)
+        for _ in range(2):
+            pc.arr[...] = -3.5
+            pc.arr[:, :n] = np.nan
+            capi.matmul(w, pa.addr, m, pc.addr, lda=lda, ldc=ldc, mem=capi.MEM_HOST)
+            assert np.array_equal(pc.arr[:, :n].view(np.uint32), bits(single))
+            assert np.all(pc.arr[:, n:] == np.float32(-3.5)), "the padding of the output rows was written"
+            pc.arr[...] = np.nan
+            pc2.arr[...] = np.nan
+            capi.matmul_multi([w, w2], pa.addr, m, [pc.addr, pc2.addr], lda=lda, ldc=[ldc, n], mem=capi.MEM_HOST)
+            assert np.array_equal(pc.arr[:, :n].view(np.uint32), bits(want))
+            assert np.array_equal(pc2.arr.view(np.uint32), bits(want2))
+            po.arr[...] = np.nan
+            capi.mlp_swiglu(w, w2, pa.addr, m, po.addr, lda=lda, mem=capi.MEM_HOST)
+            assert np.array_equal(po.arr.view(np.uint32), bits(act))
+            pd.arr[...] = np.nan
+            capi.mlp_swiglu_down(w, w2, wd, pa.addr, m, pd.addr, lda=lda, mem=capi.MEM_HOST)
+            assert np.array_equal(pd.arr.view(np.uint32), bits(down))
+    finally:
+        for p in (pa, pc, pc2, po, pd):
+            p.free()
+        for x in (w, w2, wd):
+            x.destroy()
