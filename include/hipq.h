@@ -332,7 +332,10 @@ HIPQ_API int hipq_device_download(void *dst_host, const void *src_device, size_t
 
 /** Page-locked host memory, zero-filled: what a context's MemAllocator hands the framework's
  *  memory pool (MemAllocator::alloc / free, nntrainer/mem_allocator.cpp:22-30; set by the
- *  context, cl_context.cpp:83). Tensors that live in it cross to the GPU by DMA as they are;
+ *  context, cl_context.cpp:83). Tensors that live in it cross to the GPU by DMA as they are
+ *  (a prefill of 512 rows and more with 16 MiB of outputs in steps of 256 rows, a step's output
+ *  leaving on a second stream of the library's while the next step's rows arrive and are
+ *  multiplied; a decode step of up to eight rows without a copy engine at all);
  *  any other host memory passed with HIPQ_MEM_HOST goes through a pinned staging ring inside
  *  the library (8 MiB), at the speed of a host memcpy. */
 HIPQ_API int hipq_host_alloc(void **ptr, size_t bytes);
