@@ -52,7 +52,7 @@ WeightCache::~WeightCache() { clear(); }
 
 /* Eight 8-byte words of the buffer (both ends and six in between) folded into one:
  * cheap enough for every forward call, and a rewritten weight differs in them. */
-static uint64_t sample_tag(const void *bytes, int64_t n) {
+uint64_t WeightCache::sample(const void *bytes, int64_t n) {
   const unsigned char *p = static_cast<const unsigned char *>(bytes);
   uint64_t tag = 0x9e3779b97f4a7c15ull ^ (uint64_t)n;
   if (n < 8)
@@ -73,7 +73,7 @@ hipq_weight_t WeightCache::get(const void *host_bytes, const WeightSpec &spec) {
   const int64_t nbytes = hipq_weight_nbytes(spec.dtype, spec.N, spec.K);
   if (nbytes < 0)
     check((int)nbytes, "hipq_weight_nbytes");
-  const uint64_t tag = sample_tag(host_bytes, nbytes);
+  const uint64_t tag = sample(host_bytes, nbytes);
   std::lock_guard<std::mutex> lock(mtx);
   auto it = map.find(host_bytes);
   if (it != map.end()) {
@@ -84,6 +84,7 @@ hipq_weight_t WeightCache::get(const void *host_bytes, const WeightSpec &spec) {
     /* the allocator handed the address to another tensor, or the bytes were rewritten: replace */
     hipq_weight_destroy(it->second.w);
     map.erase(it);
+    freed.fetch_add(1, std::memory_order_release);
   }
   hipq_weight_t w = nullptr;
   check(hipq_weight_create(spec.dtype, spec.layout, spec.N, spec.K, host_bytes, HIPQ_MEM_HOST, &w),
@@ -99,12 +100,15 @@ void WeightCache::invalidate(const void *host_bytes) {
     return;
   hipq_weight_destroy(it->second.w);
   map.erase(it);
+  freed.fetch_add(1, std::memory_order_release);
 }
 
 void WeightCache::clear() {
   std::lock_guard<std::mutex> lock(mtx);
   for (auto &kv : map)
     hipq_weight_destroy(kv.second.w);
+  if (!map.empty())
+    freed.fetch_add(1, std::memory_order_release);
   map.clear();
 }
 
@@ -201,7 +205,7 @@ void device_release(void *p) noexcept {
 }
 
 const float *DeviceMirror::get(const float *host, size_t n) {
-  const uint64_t t = sample_tag(host, (int64_t)(n * sizeof(float)));
+  const uint64_t t = WeightCache::sample(host, (int64_t)(n * sizeof(float)));
   if (dev && src == host && count == n && tag == t)
     return dev;
   drop();
@@ -252,7 +256,7 @@ void moe_forward(WeightCache &cache, const MoeShape &shape, int dtype,
                  const std::vector<const void *> &gate_bytes,
                  const std::vector<const void *> &up_bytes,
                  const std::vector<const void *> &down_bytes, const float *x,
-                 const float *router_weight, float *y, const MoeExtras *extras) {
+                 const float *router_weight, float *y, const MoeExtras *extras, HandleMemo *memo) {
   require_runtime();
   const size_t E = (size_t)shape.experts;
   if (gate_bytes.size() != E || up_bytes.size() != E || down_bytes.size() != E)
@@ -260,13 +264,43 @@ void moe_forward(WeightCache &cache, const MoeShape &shape, int dtype,
   const int layout = framework_layout(dtype);
   const WeightSpec gu{dtype, layout, shape.intermediate, shape.hidden};
   const WeightSpec dn{dtype, layout, shape.hidden, shape.intermediate};
-  std::vector<hipq_weight_t> g(E), u(E), d(E);
-  for (size_t e = 0; e < E; ++e) {
-    g[e] = cache.get(gate_bytes[e], gu);
-    u[e] = cache.get(up_bytes[e], gu);
-    d[e] = cache.get(down_bytes[e], dn);
+  HandleMemo local;
+  HandleMemo &m = memo ? *memo : local;
+  /* gate, up and down handles in one array: [0, E), [E, 2E), [2E, 3E) */
+  const bool known = m.w.size() == 3 * E && m.epoch == cache.epoch();
+  if (!known) {
+    m.bytes.assign(3 * E, nullptr);
+    m.tags.assign(3 * E, 0);
+    m.w.assign(3 * E, nullptr);
   }
-  moe_forward_resident(shape, g.data(), u.data(), d.data(), x, router_weight, y, extras);
+  const int64_t nb_gu = hipq_weight_nbytes(gu.dtype, gu.N, gu.K), nb_dn = hipq_weight_nbytes(dn.dtype, dn.N, dn.K);
+  bool replaced = false;
+  auto resolve = [&](size_t i, const void *bytes, const WeightSpec &spec, int64_t nbytes) {
+    if (!bytes)
+      throw std::invalid_argument("[hipq] weight tensor has no data");
+    const uint64_t tag = nbytes >= 0 ? WeightCache::sample(bytes, nbytes) : 0;
+    if (known && m.bytes[i] == bytes && m.tags[i] == tag)
+      return; /* the tensor of the last call, unchanged: its handle stands */
+    const uint64_t before = cache.epoch();
+    m.w[i] = cache.get(bytes, spec);
+    replaced |= cache.epoch() != before;
+    m.bytes[i] = bytes;
+    m.tags[i] = tag;
+  };
+  for (size_t e = 0; e < E; ++e) {
+    resolve(e, gate_bytes[e], gu, nb_gu);
+    resolve(E + e, up_bytes[e], gu, nb_gu);
+    resolve(2 * E + e, down_bytes[e], dn, nb_dn);
+  }
+  /* a replacement freed a device copy: handles resolved before it in this call may be that copy */
+  if (replaced)
+    for (size_t e = 0; e < E; ++e) {
+      m.w[e] = cache.get(gate_bytes[e], gu);
+      m.w[E + e] = cache.get(up_bytes[e], gu);
+      m.w[2 * E + e] = cache.get(down_bytes[e], dn);
+    }
+  m.epoch = cache.epoch();
+  moe_forward_resident(shape, m.w.data(), m.w.data() + E, m.w.data() + 2 * E, x, router_weight, y, extras);
 }
 
 } // namespace hipq_host

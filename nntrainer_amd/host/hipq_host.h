@@ -21,6 +21,7 @@
 #define HIPQ_HOST_H
 
 #include <cstdint>
+#include <atomic>
 #include <mutex>
 #include <stdexcept>
 #include <string>
@@ -83,6 +84,11 @@ public:
   void invalidate(const void *host_bytes);
   void clear();
   size_t size() const;
+  /** counts the device copies this cache has freed: a handle taken from get() while the count read
+   *  n is still alive as long as it reads n */
+  uint64_t epoch() const { return freed.load(std::memory_order_acquire); }
+  /** the sample get() compares (eight words of the buffer) */
+  static uint64_t sample(const void *host_bytes, int64_t nbytes);
 
 private:
   struct Entry {
@@ -92,6 +98,18 @@ private:
   };
   mutable std::mutex mtx;
   std::unordered_map<const void *, Entry> map;
+  std::atomic<uint64_t> freed{0};
+};
+
+/** The handles of a layer's many weights from its last call (a MoE layer's 3 x experts): a call finds
+ *  them again by comparing each tensor's address and sample, without the cache's lock and hash look-up
+ *  per weight (128 experts: 384 of them a call, which cost more than the rest of a decode step's host
+ *  work). Valid while the cache has freed nothing since. */
+struct HandleMemo {
+  std::vector<const void *> bytes;
+  std::vector<uint64_t> tags;
+  std::vector<hipq_weight_t> w;
+  uint64_t epoch = ~(uint64_t)0;
 };
 
 /** process-wide cache used by the layers */
@@ -178,7 +196,8 @@ void moe_forward(WeightCache &cache, const MoeShape &shape, int dtype,
                  const std::vector<const void *> &gate_bytes,
                  const std::vector<const void *> &up_bytes,
                  const std::vector<const void *> &down_bytes, const float *x,
-                 const float *router_weight, float *y, const MoeExtras *extras = nullptr);
+                 const float *router_weight, float *y, const MoeExtras *extras = nullptr,
+                 HandleMemo *memo = nullptr);
 
 /** the same block on device copies the caller already holds (experts entries each) */
 void moe_forward_resident(const MoeShape &shape, const hipq_weight_t *gate, const hipq_weight_t *up,

@@ -17,9 +17,10 @@
  *                            forwarding with weight A, then the weight tensor's bytes are replaced
  *                            by B in place -- through Layer::read as the model loader does it, or
  *                            behind the layer's back -- and forwarding runs again
- *   moe <dtype> <T> <H> <I> <E> <k> <incremental> <router> <experts> <input> <out>
+ *   moe <dtype> <T> <H> <I> <E> <k> <incremental> <router> <experts> <input> <out> [<experts_b> <out_b>]
  *                            the same for qwen_moe; <experts> holds up_e, gate_e,
- *                            down_e for e = 0.. in the order the layer requests them
+ *                            down_e for e = 0.. in the order the layer requests them; with <experts_b> the
+ *                            expert tensors are then overwritten in place with that file and the layer runs again
  *   moex <type> <dtype> <T> <H> <I> <E> <k> <incremental> <weights> <input> <out>
  *                            any of the MoE layer types; <weights> holds every weight in the order
  *                            the layer requests them and is loaded through Layer::read (which is how
@@ -379,7 +380,7 @@ static int run_fc_reload(Context *ctx, char **a) {
   return 0;
 }
 
-static int run_moe(Context *ctx, char **a) {
+static int run_moe(Context *ctx, char **a, char **second) {
   const std::string dt = a[0];
   const unsigned T = std::atoi(a[1]), H = std::atoi(a[2]), I = std::atoi(a[3]), E = std::atoi(a[4]),
                  k = std::atoi(a[5]), incremental = std::atoi(a[6]);
@@ -408,6 +409,16 @@ static int run_moe(Context *ctx, char **a) {
   else
     layer->forwarding(rc, false);
   write_from(opath, rc.getOutput(0).getData<float>(), (size_t)T * H * 4);
+  if (second) { /* other experts at the same addresses: the layer must not serve the old device copies */
+    std::ifstream f(second[0], std::ios::binary);
+    for (unsigned i = 1; i < rc.getNumWeights(); ++i)
+      f.read(rc.getWeight(i).getData<char>(), mirror_tensor_bytes(rc.getWeight(i).getDim()));
+    if (incremental)
+      layer->incremental_forwarding(rc, 0, T, false);
+    else
+      layer->forwarding(rc, false);
+    write_from(second[1], rc.getOutput(0).getData<float>(), (size_t)T * H * 4);
+  }
   std::printf("MOE DONE\n");
   return 0;
 }
@@ -750,8 +761,8 @@ int main(int argc, char **argv) {
       return run_api(ctx);
     if (mode == "fc" && argc == 14)
       return run_fc(ctx, argv + 3);
-    if (mode == "moe" && argc == 14)
-      return run_moe(ctx, argv + 3);
+    if (mode == "moe" && (argc == 14 || argc == 16))
+      return run_moe(ctx, argv + 3, argc == 16 ? argv + 14 : nullptr);
     if (mode == "fcreload" && argc == 13)
       return run_fc_reload(ctx, argv + 3);
     if (mode == "moex" && argc == 14)

@@ -236,7 +236,7 @@ void MoELayerHip::run(RunLayerContext &context, const float *x, float *y, unsign
     u[e] = context.getWeight(expert_up_proj_indices[e]).getData<uint8_t>();
     d[e] = context.getWeight(expert_down_proj_indices[e]).getData<uint8_t>();
   }
-  hipq_host::moe_forward(hipq_host::global_cache(), shape, weight_dtype, g, u, d, x, router, y, &extras);
+  hipq_host::moe_forward(hipq_host::global_cache(), shape, weight_dtype, g, u, d, x, router, y, &extras, &handles);
 }
 
 void MoELayerHip::forwarding(RunLayerContext &context, bool training) {

@@ -103,6 +103,7 @@ private:
   hipq_host::DeviceMirror dev_router; /* the fp32 router weight [hidden x experts] */
   /* cached: device copies this layer owns, gate | up | down, made at an expert's first use */
   std::vector<hipq_weight_t> resident;
+  hipq_host::HandleMemo handles; /* the uncached layers' expert handles from the last call */
 };
 
 /** "moe_cached_slim" */

@@ -414,3 +414,32 @@ def test_mlp_swiglu_layer_with_the_down_projection(cr, tmp_path, kind, k, n, nd,
         ref = cr.gemm(cr.oracle(), kind, hidden, down, nd)
         assert np.abs(got[b, :rows] - ref).max() / np.abs(ref).max() <= TOL
         assert np.all(got[b, rows:] == -12345.0)
+
+
+def test_moe_sees_expert_weights_rewritten_in_place(cr, tmp_path):
+    """The MoE layer remembers its experts' device handles between calls; experts whose bytes change at the
+    same addresses (a second model read into the same tensors) must be uploaded again."""
+    t, h, i, e, k = 6, 512, 256, 8, 2
+    sets = []
+    for base in (7900, 7950):
+        gate = [cr.quantize_weights(cr.oracle(), "q4_K", synth.normal(base + 3 * x, (i, h), 0.02)) for x in range(e)]
+        up = [cr.quantize_weights(cr.oracle(), "q4_K", synth.normal(base + 3 * x + 1, (i, h), 0.02)) for x in range(e)]
+        down = [cr.quantize_weights(cr.oracle(), "q4_K", synth.normal(base + 3 * x + 2, (h, i), 0.02)) for x in range(e)]
+        sets.append((gate, up, down))
+    xin = synth.normal(7990, (t, h))
+    wr = synth.normal(7991, (h, e), 0.1)
+    logits = cr.router_logits(xin, wr, k)
+    wr.tofile(tmp_path / "router.bin")
+    for name, (gate, up, down) in zip(("a.bin", "b.bin"), sets):
+        with open(tmp_path / name, "wb") as f:
+            for x in range(e):
+                f.write(cr.repack_x8(cr.oracle(), "q4_K", up[x], i, h).tobytes())
+                f.write(cr.repack_x8(cr.oracle(), "q4_K", gate[x], i, h).tobytes())
+                f.write(cr.repack_x8(cr.oracle(), "q4_K", down[x], h, i).tobytes())
+    xin.tofile(tmp_path / "x.bin")
+    _run(["moe", "q4_K", t, h, i, e, k, 1, tmp_path / "router.bin", tmp_path / "a.bin", tmp_path / "x.bin",
+          tmp_path / "ya.bin", tmp_path / "b.bin", tmp_path / "yb.bin"])
+    for name, (gate, up, down) in zip(("ya.bin", "yb.bin"), sets):
+        ref_y, _, _ = cr.moe_forward(xin, logits, gate, up, down, k)
+        got = np.fromfile(tmp_path / name, np.float32).reshape(t, h)
+        assert np.abs(got - ref_y).max() / np.abs(ref_y).max() <= TOL, name
