@@ -21,7 +21,7 @@
  * device pointers; the call only enqueues work on `stream` and returns.
  * HIPQ_MEM_HOST buffers are ordinary host memory; the call copies in, runs,
  * copies out and returns when the result is in the host buffer. A call of a
- * few rows (a decode step: up to eight rows, at most 1 MiB of outputs) uses no
+ * few rows (a decode step or a short chunk: up to 128 rows, at most 2 MiB a side) uses no
  * copy engine: a kernel reads the rows from page-locked memory (memory of
  * hipq_host_alloc as it is, other memory through a page-locked staging buffer),
  * the product kernels write the outputs there, and the call returns when the
@@ -335,7 +335,7 @@ HIPQ_API int hipq_device_download(void *dst_host, const void *src_device, size_t
  *  context, cl_context.cpp:83). Tensors that live in it cross to the GPU by DMA as they are
  *  (a prefill of 512 rows and more with 16 MiB of outputs in steps of 256 rows, a step's output
  *  leaving on a second stream of the library's while the next step's rows arrive and are
- *  multiplied; a decode step of up to eight rows without a copy engine at all);
+ *  multiplied; up to 128 rows of at most 2 MiB a side without a copy engine at all);
  *  any other host memory passed with HIPQ_MEM_HOST goes through a pinned staging ring inside
  *  the library (8 MiB), at the speed of a host memcpy. */
 HIPQ_API int hipq_host_alloc(void **ptr, size_t bytes);

@@ -329,14 +329,17 @@ int wait_done(hipStream_t s) {
   return HIPQ_OK;
 }
 
-/* A decode step's host operands without a copy engine. Up to eight rows and small outputs (what an
- * FC sees while tokens are generated): the rows are fetched into device memory by a small kernel,
- * the product kernels write their outputs straight into host memory, and one wait ends the call --
- * two launches and a wait instead of a copy in, the launches, one copy out per output and the wait.
- * Page-locked operands (the context's allocator) are used where they lie; pageable ones pass through
- * the stream's page-locked staging buffer with a memcpy on either side. */
-constexpr int64_t DIRECT_ROWS = 8;
-constexpr size_t DIRECT_BYTES = (size_t)1 << 20; /* rows in, and all outputs together */
+/* A few rows of host operands without a copy engine. Up to 128 rows and 2 MiB a side (what an FC sees
+ * while tokens are generated, and a short prefill chunk): the rows are fetched into device memory by a
+ * small kernel, the product kernels write their outputs straight into host memory, and one wait ends
+ * the call -- two launches and a wait instead of a copy in, the launches, one copy out per output and
+ * the wait. Page-locked operands (the context's allocator) are used where they lie; pageable ones pass
+ * through the stream's page-locked staging buffer with a memcpy on either side. Measured on page-locked
+ * operands, us a call, copy engines -> this path: Q4_0 3072 x 1024 with 9 / 16 / 32 / 64 / 128 rows
+ * 32 -> 19 / 34 -> 21 / 41 -> 28 / 52 -> 40 / 70 -> 60, Q4_K 4096 x 4096 42 -> 28 / 45 -> 32 / 56 -> 45 /
+ * 78 -> 69 / 120 -> 115; at 256 rows the copy engines are level or ahead (111 against 105, 199 against 206). */
+constexpr int64_t DIRECT_ROWS = 128;
+constexpr size_t DIRECT_BYTES = (size_t)2 << 20; /* rows in, and all outputs together */
 struct DirectIO {
   struct Out {
     float *host, *dev; /* where the caller wants it; where the kernels write (device-side address) */

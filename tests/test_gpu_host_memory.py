@@ -120,10 +120,16 @@ class _Pinned:
     ("q4_K", 3, 2048, 1024, 8, 4),      # strided rows on both sides
     ("q4_0", 8, 1024, 3072, 0, 12),
     ("q4_K", 8, 4096, 12288, 0, 0),     # the few-rows matrix-core kernel
-    ("q4_0", 9, 1024, 3072, 0, 0),      # one row more than the direct path takes: through the copy engines
+    ("q4_0", 9, 1024, 3072, 0, 0),
+    ("q4_K", 64, 4096, 4096, 0, 8),     # a short prefill chunk: 1 MiB each way
+    ("q6_K", 100, 1024, 2048, 4, 0),
+    ("q4_0", 128, 1024, 3072, 0, 0),    # the most rows this path takes
+    ("q4_0", 129, 1024, 3072, 0, 0),    # one row more: through the copy engines
+    ("q4_0", 100, 1024, 8192, 0, 0),    # outputs beyond 2 MiB: through the copy engines
 ])
 def test_a_few_page_locked_rows_take_no_copy(hipq, cr, kind, m, k, n, lda_pad, ldc_pad):
-    """Up to eight rows in page-locked memory (a decode step through the Layer API): the rows are
+    """Up to 128 rows and 2 MiB a side in page-locked memory (a decode step or a short chunk through the
+    Layer API): the rows are
     fetched by a kernel and the product kernels write the host tensor directly. Same bits as the
     device-memory call; the padding of strided rows stays untouched; two calls in a row."""
     blocks = cr.quantize_weights(cr.oracle(), kind, synth.normal(9400 + n % 89, (n, k), 0.02))
