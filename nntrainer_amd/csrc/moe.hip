@@ -115,40 +115,69 @@ __global__ __launch_bounds__(256) void router_logits_scalar_kernel(const float *
  * 12 us). Here a workgroup takes sixteen experts (64 bytes of every row of Wr) and up to four
  * tokens, whose rows of x it first copies to LDS. Four lanes read a row's 64 bytes, sixteen rows
  * an instruction (sixteen half lines, not sixty-four separate ones), the four wavefronts take the
- * rows in turn, sixteen loads are in flight and each is used for all the tokens. The partial sums
+ * rows in turn, thirty-two loads are in flight (issued before the rows of x are copied) and each is
+ * used for all the tokens. The partial sums
  * meet in a fixed order: over the sixteen row lanes by exchanges, over the wavefronts through LDS.
  * The matrix is read by E / 16 CUs side by side, each its own columns. (The reference's order of
  * the sum is its BLAS library's and not specified.) */
 constexpr int ROUTER_TB = 4; /* tokens per workgroup, at most */
+constexpr size_t router_lds_bytes(int tb_n, int H) { return ((size_t)tb_n * H + 256 * (size_t)tb_n) * sizeof(float); }
 template <int TBN> /* tokens of this workgroup: 1, 2 or 4 */
 __global__ __launch_bounds__(256) void router_logits_kernel(const float *__restrict__ x,
                                                             const float *__restrict__ wr, int T, int H,
                                                             int E, const float *__restrict__ bias,
                                                             float *__restrict__ logits) {
-  extern __shared__ __attribute__((aligned(16))) float router_x[]; /* [token][H], then 256 floats of partial sums */
-  constexpr int JU = 4; /* groups of four rows a lane has in flight: sixteen loads */
+  extern __shared__ __attribute__((aligned(16))) float router_x[]; /* [token][H], then the partial sums */
+  constexpr int JU = 8; /* groups of four rows a lane has in flight: thirty-two loads (all of H = 2048 at once) */
   const int t0 = blockIdx.y * TBN;
-  for (int i = threadIdx.x * 4; i < TBN * H; i += 256 * 4) { /* H % 4 == 0 */
-    const int tb = i / H, h = i - tb * H;
-    *(float4 *)(router_x + i) = *(const float4 *)(x + (size_t)min(t0 + tb, T - 1) * H + h);
-  }
-  __syncthreads();
-  float *part = router_x + TBN * H; /* [wavefront 4][token][16 experts] */
+  float *part = router_x + TBN * H; /* [wavefront 4][row of 16 lanes 4][token][16 experts] */
   const int e4n = E >> 2;
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
   const int r = lane >> 2, q = lane & 3;
   const int c = min((int)blockIdx.x * 4 + q, e4n - 1); /* columns past the end repeat the last; not stored */
+  /* this lane's rows: h = 256 j + 64 wave + 4 r + i, i = 0 .. 3 (its x values are one 128-bit LDS read) */
+  int h = 64 * wave + 4 * r;
+  const bool whole = (H & 255) == 0; /* then a group of rows 256 j .. 256 j + 255 is in or out as one (uniform) */
+  float4 w[JU][4];
+  auto load_w = [&](int h0) {
+    if (whole) {
+      const float4 *p = (const float4 *)wr + c + (size_t)h0 * e4n;
+#pragma unroll
+      for (int j = 0; j < JU; ++j)
+        if (256 * j + (h0 & ~255) < H) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) w[j][i] = p[(size_t)(256 * j + i) * e4n];
+        }
+    } else {
+#pragma unroll
+      for (int j = 0; j < JU; ++j)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) w[j][i] = ((const float4 *)wr + c)[(size_t)min(h0 + 256 * j + i, H - 1) * e4n];
+    }
+  };
+  /* the first rows of Wr are on their way while the tokens' rows of x go to LDS, 2 * TBN loads of a lane at a
+   * time (one after the other they cost a round trip each: 2.4 us for four rows of 2048) */
+  load_w(h);
+  const float *xrow[TBN];
+#pragma unroll
+  for (int tb = 0; tb < TBN; ++tb) xrow[tb] = x + (size_t)min(t0 + tb, T - 1) * H;
+  for (int hx0 = threadIdx.x * 4; hx0 < H; hx0 += 2048) { /* H % 4 == 0 */
+    float4 v[TBN][2];
+#pragma unroll
+    for (int tb = 0; tb < TBN; ++tb)
+#pragma unroll
+      for (int u = 0; u < 2; ++u) v[tb][u] = *(const float4 *)(xrow[tb] + min(hx0 + 1024 * u, H - 4));
+#pragma unroll
+    for (int tb = 0; tb < TBN; ++tb)
+#pragma unroll
+      for (int u = 0; u < 2; ++u)
+        if (hx0 + 1024 * u < H) *(float4 *)(router_x + tb * H + hx0 + 1024 * u) = v[tb][u];
+  }
+  __syncthreads();
   float acc[TBN][4];
 #pragma unroll
   for (int tb = 0; tb < TBN; ++tb) acc[tb][0] = acc[tb][1] = acc[tb][2] = acc[tb][3] = 0.f;
-  const float4 *w4 = (const float4 *)wr + c;
-  /* this lane's rows: h = 256 j + 64 wave + 4 r + i, i = 0 .. 3 (its x values are one 128-bit LDS read) */
-  for (int h = 64 * wave + 4 * r; h < H; h += 256 * JU) {
-    float4 w[JU][4];
-#pragma unroll
-    for (int j = 0; j < JU; ++j)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) w[j][i] = w4[(size_t)min(h + 256 * j + i, H - 1) * e4n];
+  for (; h < H; h += 256 * JU) {
 #pragma unroll
     for (int j = 0; j < JU; ++j) {
       if (h + 256 * j < H) { /* H % 4 == 0: the four rows are in or out together */
@@ -166,17 +195,20 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const float *__restr
         }
       }
     }
+    if (h + 256 * JU < H) load_w(h + 256 * JU);
   }
+  /* The partial sums meet in a fixed order: the four lanes of a column quarter inside a row of sixteen lanes by
+   * two shifted adds (lanes 12 .. 15 of the row then hold the row's sums), the sixteen rows of the workgroup
+   * through LDS. (Exchanges across the whole wavefront, four a value, took 2.2 us of this kernel's 8.) */
+  const int row16 = lane >> 4;
 #pragma unroll
   for (int tb = 0; tb < TBN; ++tb) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       float v = acc[tb][j];
-      v += __shfl_xor(v, 4, 64);
-      v += __shfl_xor(v, 8, 64);
-      v += __shfl_xor(v, 16, 64);
-      v += __shfl_xor(v, 32, 64);
-      if (r == 0) part[(wave * TBN + tb) * 16 + q * 4 + j] = v;
+      v += hipq_dpp_f<0x114>(v); /* row_shr:4 */
+      v += hipq_dpp_f<0x118>(v); /* row_shr:8 */
+      if ((lane & 12) == 12) part[((wave * 4 + row16) * TBN + tb) * 16 + q * 4 + j] = v;
     }
   }
   __syncthreads();
@@ -184,7 +216,7 @@ __global__ __launch_bounds__(256) void router_logits_kernel(const float *__restr
     const int tb = threadIdx.x >> 4, el = threadIdx.x & 15, e = blockIdx.x * 16 + el;
     if (t0 + tb < T && e < E) {
       float sum = part[tb * 16 + el];
-      for (int w = 1; w < 4; ++w) sum += part[(w * TBN + tb) * 16 + el];
+      for (int p = 1; p < 16; ++p) sum += part[(p * TBN + tb) * 16 + el];
       logits[(size_t)(t0 + tb) * E + e] = bias ? sum + bias[e] : sum;
     }
   }
@@ -1577,15 +1609,15 @@ int launch_moe(const MoeArgs *a, void *workspace, size_t workspace_bytes, const 
 
   const float *logits = a->router_logits;
   if (!logits) {
-    /* the rows of x of a workgroup's tokens go to LDS: four tokens, or as many as there are or fit 64 KB */
-    int tb_n = d.hidden > 0 ? (int)std::min<int64_t>(std::min(ROUTER_TB, T), 16000 / d.hidden) : 0;
+    /* the rows of x of a workgroup's tokens go to LDS: four tokens, or as many as there are or fit 64 KB with the partial sums */
+    int tb_n = d.hidden > 0 ? (int)std::min<int64_t>(std::min(ROUTER_TB, T), 15000 / d.hidden) : 0;
     tb_n = tb_n >= 4 ? 4 : tb_n >= 2 ? 2 : tb_n;
     if ((E & 3) || (d.hidden & 3) || tb_n < 1 || (((uintptr_t)a->router_weight | (uintptr_t)a->x) & 15)) {
       hipq::launch_kernel("router_logits_scalar_kernel", router_logits_scalar_kernel, dim3(T), dim3(256), 0, s, a->x,
                           a->router_weight, d.hidden, E, a->router_bias, b.logits);
     } else {
       const dim3 grid((E / 4 + 3) / 4, (T + tb_n - 1) / tb_n);
-      const size_t lds = ((size_t)tb_n * d.hidden + 256) * sizeof(float);
+      const size_t lds = router_lds_bytes(tb_n, d.hidden);
       auto launch = [&](auto k, const char *name) {
         hipq::launch_kernel(name, k, grid, dim3(256), lds, s, a->x, a->router_weight, T, d.hidden, E, a->router_bias,
                             b.logits);
