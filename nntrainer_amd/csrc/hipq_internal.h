@@ -380,6 +380,40 @@ template <int T> __device__ __forceinline__ float hipq_group_max(float v) {
   return v;
 }
 
+/* The same reductions over the whole wavefront with a wave-uniform result, without the two
+ * exchanges through the LDS crossbar that the last steps of the group forms take (about two hundred
+ * clocks each when a lone wavefront waits for them): after the four steps inside the rows of sixteen
+ * lanes, row_bcast:15 hands every row's value to the next row (rows 1 and 3 take it), row_bcast:31
+ * hands row 1's to rows 2 and 3, and lane 63 holds the total, which a scalar read broadcasts. The
+ * sum associates as the exchange form does, (R3 + R2) + (R1 + R0) over the rows' totals, so it has
+ * that form's bits. */
+template <int CTRL, int ROWS> __device__ __forceinline__ int hipq_dpp_rows_i(int v) {
+  return __builtin_amdgcn_update_dpp(v, v, CTRL, ROWS, 0xf, false); /* rows outside ROWS keep v */
+}
+__device__ __forceinline__ float hipq_wave_max(float v) {
+  v = hipq_group_max<16>(v);
+  v = fmaxf(v, __builtin_bit_cast(float, hipq_dpp_rows_i<0x142, 0xa>(__builtin_bit_cast(int, v))));
+  v = fmaxf(v, __builtin_bit_cast(float, hipq_dpp_rows_i<0x143, 0xc>(__builtin_bit_cast(int, v))));
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+__device__ __forceinline__ int hipq_wave_min_i(int v) {
+  v = min(v, hipq_dpp_i<HIPQ_DPP_XOR1>(v));
+  v = min(v, hipq_dpp_i<HIPQ_DPP_XOR2>(v));
+  v = min(v, hipq_dpp_i<HIPQ_DPP_HALF_MIRROR>(v));
+  v = min(v, hipq_dpp_i<HIPQ_DPP_MIRROR>(v));
+  v = min(v, hipq_dpp_rows_i<0x142, 0xa>(v));
+  v = min(v, hipq_dpp_rows_i<0x143, 0xc>(v));
+  return __builtin_amdgcn_readlane(v, 63);
+}
+__device__ __forceinline__ float hipq_wave_sum(float v) {
+  v = hipq_group_sum<16>(v);
+  const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x142, 0xa, 0xf, false));
+  v = v + r1; /* rows 0 and 2 add zero */
+  const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x143, 0xc, 0xf, false));
+  v = v + r2;
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
+}
+
 /* Loads of weight data name the global address space. A pointer that a kernel
  * read from memory (a table of weight views) is generic to the compiler, which
  * then emits flat loads; those count against the LDS counter as well, so every

@@ -242,7 +242,7 @@ __device__ __forceinline__ void route_token_regs(const float *__restrict__ logit
       mx = fmaxf(mx, p[i]);
     }
   }
-  mx = hipq_group_max<64>(mx);
+  mx = hipq_wave_max(mx);
   float sum = 0.f;
 #pragma unroll
   for (int i = 0; i < MAXV; ++i) {
@@ -252,7 +252,7 @@ __device__ __forceinline__ void route_token_regs(const float *__restrict__ logit
       sum += p[i];
     }
   }
-  sum = hipq_group_sum<64>(sum);
+  sum = hipq_wave_sum(sum);
 #pragma unroll
   for (int i = 0; i < MAXV; ++i) {
     const int e = lane + 64 * i;
@@ -277,15 +277,11 @@ __device__ __forceinline__ void route_token_regs(const float *__restrict__ logit
         bi = e;
       }
     }
-    /* the wavefront's maximum, then the lowest expert id that holds it */
-    const float mxv = hipq_group_max<64>(bv);
-    int cand = bv == mxv ? bi : 0x7fffffff;
-    cand = min(cand, hipq_dpp_i<HIPQ_DPP_XOR1>(cand));
-    cand = min(cand, hipq_dpp_i<HIPQ_DPP_XOR2>(cand));
-    cand = min(cand, hipq_dpp_i<HIPQ_DPP_HALF_MIRROR>(cand));
-    cand = min(cand, hipq_dpp_i<HIPQ_DPP_MIRROR>(cand));
-    cand = min(cand, __shfl_xor(cand, 16, 64));
-    cand = min(cand, __shfl_xor(cand, 32, 64));
+    /* the wavefront's maximum, then the lowest expert id that holds it: mostly one lane's */
+    const float mxv = hipq_wave_max(bv);
+    const unsigned long long holders = __ballot(bv == mxv);
+    const int cand = __popcll(holders) == 1 ? __builtin_amdgcn_readlane(bi, __ffsll((long long)holders) - 1)
+                                            : hipq_wave_min_i(bv == mxv ? bi : 0x7fffffff);
     bv = mxv;
     bi = cand;
     /* every lane now agrees on (bv, bi); retire it in its owner */
@@ -301,6 +297,84 @@ __device__ __forceinline__ void route_token_regs(const float *__restrict__ logit
     }
   }
   if (renorm) myw = __fdiv_rn(myw, ksum);
+}
+
+/* The SET of token 0's topk experts without the exponentials and without a selection round per expert:
+ * mask[i] bit l = expert 64 i + l is one of them. Returns false when the shortcut cannot promise the set
+ * of route_token_regs, and the caller runs that. The probability p = fdiv(float(exp(double(v))), sum) with
+ * v = logit - max <= 0 is monotone in v, so the sets can differ only if the topk-th and the next
+ * probability round to the same float while their logits differ (the tie then goes to the lower expert
+ * id). With v_topk - v_next > 1e-6 the two exponentials differ by more than eight float spacings and stay
+ * apart through both roundings; with v_topk > -75 nothing underflows. A NaN or an infinite maximum among
+ * the logits, and equal values on the two sides of the cut, take the full routine as well.
+ * The topk-th largest v is the topk-th smallest magnitude |v| (as an integer: the bits of a float order
+ * like its magnitude), found one bit at a time from counts over the wavefront: 31 steps of two compares
+ * and a few scalar instructions, where a round of selection per expert is two dependent reductions over
+ * the wavefront each (2.6 us for eight experts of 128, against 0.7 us). */
+template <int MAXV>
+__device__ __forceinline__ bool topk_set_fast(const float *__restrict__ lg, int E, int topk,
+                                              unsigned long long (&mask)[MAXV]) {
+  const int lane = threadIdx.x & 63;
+  float v[MAXV];
+  float mx = -INFINITY;
+  bool nan = false;
+#pragma unroll
+  for (int i = 0; i < MAXV; ++i) {
+    v[i] = -INFINITY;
+    if (64 * i < E) {
+      const int e = lane + 64 * i;
+      if (e < E) v[i] = lg[e];
+      nan |= !(v[i] == v[i]);
+      mx = fmaxf(mx, v[i]);
+    }
+  }
+  if (__ballot(nan)) return false;
+  mx = hipq_wave_max(mx);
+  if (!(fabsf(mx) < INFINITY)) return false; /* uniform: an infinite logit makes differences undefined */
+  int mag[MAXV]; /* |logit - max| as an integer; no expert's: beyond every float */
+#pragma unroll
+  for (int i = 0; i < MAXV; ++i) {
+    const int e = lane + 64 * i;
+    mag[i] = (64 * i < E && e < E) ? (int)(__float_as_uint(v[i] - mx) & 0x7fffffffu) : 0x7fffffff;
+  }
+  auto count_le = [&](int t) {
+    int n = 0;
+#pragma unroll
+    for (int i = 0; i < MAXV; ++i)
+      if (64 * i < E) n += __popcll(__ballot(mag[i] <= t));
+    return n;
+  };
+  int cut = 0; /* the smallest t with topk magnitudes <= t */
+  for (int bit = 30; bit >= 0; --bit)
+    if (count_le(cut | ((1 << bit) - 1)) < topk) cut |= 1 << bit;
+  if (count_le(cut) != topk) return false; /* equal values across the cut: the tie rule decides (uniform) */
+  int beyond = 0x7fffffff;
+#pragma unroll
+  for (int i = 0; i < MAXV; ++i) beyond = min(beyond, mag[i] > cut ? mag[i] : 0x7fffffff);
+  beyond = hipq_wave_min_i(beyond); /* the next magnitude, or 0x7fffffff when every expert is selected */
+#pragma unroll
+  for (int i = 0; i < MAXV; ++i) mask[i] = 64 * i < E ? __ballot(mag[i] <= cut) : 0ull;
+  const float v_cut = __uint_as_float((uint32_t)cut);
+  if (!(v_cut < 75.f)) return false;
+  return beyond == 0x7fffffff || __uint_as_float((uint32_t)beyond) - v_cut > 1e-6f;
+}
+
+/* expert number `item` of the set in ascending id */
+template <int MAXV> __device__ __forceinline__ int nth_of_set(const unsigned long long (&mask)[MAXV], int item) {
+  int e = 0;
+  bool found = false;
+#pragma unroll
+  for (int i = 0; i < MAXV; ++i) {
+    const int c = __popcll(mask[i]);
+    if (!found && item < c) {
+      unsigned long long m = mask[i];
+      for (int j = 0; j < item; ++j) m &= m - 1; /* drop the item lowest */
+      e = 64 * i + __ffsll((long long)m) - 1;
+      found = true;
+    }
+    if (!found) item -= c;
+  }
+  return e;
 }
 
 /* the rank of lane kk's expert among the token's topk, ascending expert id (lanes below topk) */
@@ -1031,13 +1105,14 @@ __global__ __launch_bounds__(256, TC <= 8 ? 4 : TC <= 16 ? 2 : 1) void gate_up_m
   }
 }
 
-/* One token (a decode step), the routing inside the gate/up launch: every wavefront routes the
- * token itself (the same arithmetic on the same logits, so all agree), the workgroup takes the
+/* One token (a decode step), the routing inside the gate/up launch: every wavefront finds the
+ * token's set of experts itself (the same arithmetic on the same logits, so all agree; without the
+ * softmax's exponentials where topk_set_fast can promise the same set), the workgroup takes the
  * expert whose rank in ascending id is its blockIdx.y, quantizes the row of x into its LDS while
  * its first weights are on their way, and goes on as the paired form of gate_up_mma_kernel.
- * Workgroup (0, 0) writes the routing's outputs and the few table entries the down product and
- * the combine read. One launch (7-8 us of a block of 25) less than routing, sort and quantization
- * as a launch of their own. */
+ * One workgroup more than the columns need routes the token in full and writes the routing's
+ * outputs and the few table entries the down product and the combine read. One launch (7-8 us of
+ * a block of 25) less than routing, sort and quantization as a launch of their own. */
 template <int MAXV>
 __global__ __launch_bounds__(256, 4) void gate_up_one_token_kernel(
   const float *__restrict__ logits, int E, int topk, int renorm, int32_t *__restrict__ idx, float *__restrict__ wgt,
@@ -1048,23 +1123,38 @@ __global__ __launch_bounds__(256, 4) void gate_up_one_token_kernel(
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
   int myi;
   float myw;
-  route_token_regs<MAXV>(logits, 0, E, topk, renorm, myi, myw);
-  const int rank = rank_by_expert(myi, topk);
-  const int item = blockIdx.y; /* < topk */
-  const unsigned long long owner = __ballot(lane < topk && rank == item);
-  const int e = __shfl(myi, __ffsll((long long)owner) - 1, 64);
-  if (blockIdx.x == 0 && blockIdx.y == 0 && wave == 0) {
-    if (lane < topk) {
-      idx[lane] = myi;
-      wgt[lane] = myw;
-      slot_pair[rank] = lane; /* slots in ascending expert id; one token: pair = its k */
-      tok_slots[rank] = rank;
-      offsets[myi + 1] = rank + 1; /* the end of the expert's slots: all the later kernels read of offsets */
-      items[2 + 2 * rank] = myi;
-      items[3 + 2 * rank] = rank;
+  if (blockIdx.x == gridDim.x - 1) {
+    /* the extra column of the grid: its first workgroup's first wavefront routes the token in full and
+     * writes what the launches behind this one read; it multiplies nothing */
+    if (blockIdx.y == 0 && wave == 0) {
+      route_token_regs<MAXV>(logits, 0, E, topk, renorm, myi, myw);
+      const int rank = rank_by_expert(myi, topk);
+      if (lane < topk) {
+        idx[lane] = myi;
+        wgt[lane] = myw;
+        slot_pair[rank] = lane; /* slots in ascending expert id; one token: pair = its k */
+        tok_slots[rank] = rank;
+        offsets[myi + 1] = rank + 1; /* the end of the expert's slots: all the later kernels read of offsets */
+        items[2 + 2 * rank] = myi;
+        items[3 + 2 * rank] = rank;
+      }
+      if (lane == 0) items[0] = topk;
     }
-    if (lane == 0) items[0] = topk;
+    return; /* uniform per workgroup */
   }
+  /* the other workgroups need the set of experts only, which mostly needs no exponential */
+  const int item = blockIdx.y; /* < topk */
+  unsigned long long set[MAXV];
+  int e;
+  if (topk_set_fast<MAXV>(logits, E, topk, set)) {
+    e = nth_of_set<MAXV>(set, item);
+  } else {
+    route_token_regs<MAXV>(logits, 0, E, topk, renorm, myi, myw);
+    const int rank = rank_by_expert(myi, topk);
+    const unsigned long long owner = __ballot(lane < topk && rank == item);
+    e = __shfl(myi, __ffsll((long long)owner) - 1, 64);
+  }
+  e = __builtin_amdgcn_readfirstlane(e);
   const WView wg = views[e], wu = views[E + e];
   const int K = wg.K;
   const XLds l = xlds_carve(xmoe_lds, TC, K);
@@ -1654,7 +1744,8 @@ int launch_moe(const MoeArgs *a, void *workspace, size_t workspace_bytes, const 
                                  : (const void *)gate_up_one_token_kernel<16>;
       HIPQ_HIP(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_g));
     }
-    const dim3 grid((unsigned)((d.intermediate + 63) / 64), (unsigned)d.topk);
+    /* one block column more than the columns of h need: the routing's outputs are written there */
+    const dim3 grid((unsigned)((d.intermediate + 63) / 64) + 1, (unsigned)d.topk);
     auto launch = [&](auto k, const char *name) {
       hipq::launch_kernel(name, k, grid, dim3(256), lds_g, s, logits, E, d.topk, d.renormalize, idx, wgt, b.offsets,
                           b.slot_pair, b.tok_slots, b.items, a->x, views, d.intermediate, b.h, a->epi);
