@@ -891,9 +891,13 @@ struct XRegs {
   mv4i hd;
 };
 
+/* One super-block's terms for the NREG rows of a lane: the integer sum fi (as a float) with its factor
+ * si = d * dA, and the mins' sum fm with its factor sm = dmin * dA. The caller adds them to its chains,
+ * acc = fma(fi, si, acc) and accm = fma(fm, sm, accm), in super-block order. */
 template <int TC, int NREG>
-__device__ __forceinline__ void xr_super_block(const XRegs &W, const XLds &l, int K, int sb, int i32, int g,
-                                               float (&acc)[NREG], float (&accm)[NREG]) {
+__device__ __forceinline__ void xr_sb_terms(const XRegs &W, const XLds &l, int K, int sb, int i32, int g,
+                                            float (&fi)[NREG], float (&si)[NREG], float (&fm)[NREG],
+                                            float (&sm)[NREG]) {
   const mv16i zero16 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
   const mv16f zero16f = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
   const int nsb = K >> 8;
@@ -948,9 +952,22 @@ __device__ __forceinline__ void xr_super_block(const XRegs &W, const XLds &l, in
     for (int e = 0; e < 4; ++e) {
       const int r = 4 * q4 + e;
       const float dA = __int_as_float(dv[q4][e]);
-      acc[r] = fmaf((float)I[r], dw * dA, acc[r]);
-      accm[r] = fmaf(Sm[r], dmin * dA, accm[r]);
+      fi[r] = (float)I[r];
+      si[r] = dw * dA;
+      fm[r] = Sm[r];
+      sm[r] = dmin * dA;
     }
+  }
+}
+template <int TC, int NREG>
+__device__ __forceinline__ void xr_super_block(const XRegs &W, const XLds &l, int K, int sb, int i32, int g,
+                                               float (&acc)[NREG], float (&accm)[NREG]) {
+  float fi[NREG], si[NREG], fm[NREG], sm[NREG];
+  xr_sb_terms<TC, NREG>(W, l, K, sb, i32, g, fi, si, fm, sm);
+#pragma unroll
+  for (int r = 0; r < NREG; ++r) {
+    acc[r] = fmaf(fi[r], si[r], acc[r]);
+    accm[r] = fmaf(fm[r], sm[r], accm[r]);
   }
 }
 
@@ -1117,7 +1134,7 @@ template <int MAXV>
 __global__ __launch_bounds__(256, 4) void gate_up_one_token_kernel(
   const float *__restrict__ logits, int E, int topk, int renorm, int32_t *__restrict__ idx, float *__restrict__ wgt,
   int *__restrict__ offsets, int *__restrict__ slot_pair, int *__restrict__ tok_slots, int *__restrict__ items,
-  const float *__restrict__ x, const WView *__restrict__ views, int I, float *__restrict__ h, hipq::MoeEpi ep) {
+  const float *__restrict__ x, const WView *__restrict__ views, int H, int I, float *__restrict__ h, hipq::MoeEpi ep) {
   constexpr int TC = 8, NREG = TC / 2;
   extern __shared__ __attribute__((aligned(16))) unsigned char xmoe_lds[];
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
@@ -1142,6 +1159,13 @@ __global__ __launch_bounds__(256, 4) void gate_up_one_token_kernel(
     }
     return; /* uniform per workgroup */
   }
+  /* this wavefront's share of the row of x is asked for first: it has arrived when the routing is done */
+  constexpr int XPRE = 4; /* super-blocks a wavefront holds ahead: rows of up to 4096 values */
+  const int nsb_x = H >> 8;
+  float4 xpre[XPRE];
+#pragma unroll
+  for (int j = 0; j < XPRE; ++j)
+    if (wave + 4 * j < nsb_x) xpre[j] = *(const float4 *)(x + (wave + 4 * j) * 256 + lane * 4);
   /* the other workgroups need the set of experts only, which mostly needs no exponential */
   const int item = blockIdx.y; /* < topk */
   unsigned long long set[MAXV];
@@ -1166,7 +1190,14 @@ __global__ __launch_bounds__(256, 4) void gate_up_one_token_kernel(
     /* rows 1 .. 7 of the matrix operand keep what the LDS held: a row of the product depends on
      * its own activations only, and those rows are not stored */
     const int nsb = K >> 8;
-    for (int b = wave; b < nsb; b += 4) { /* uniform per wavefront */
+#pragma unroll
+    for (int j = 0; j < XPRE; ++j) {
+      const int b = wave + 4 * j;
+      if (b < nsb) /* uniform per wavefront */
+        hipq_quantize_q8_K_values<Q8K_ROWMMA>(xpre[j], 0, b, b, nsb, 0, l.q, l.dA, nullptr, nullptr,
+                                              (uint16_t *)l.amin, nullptr, nullptr, TC);
+    }
+    for (int b = wave + 4 * XPRE; b < nsb; b += 4) { /* longer rows: the rest as it comes */
       const float4 xv = *(const float4 *)(x + b * 256 + lane * 4);
       hipq_quantize_q8_K_values<Q8K_ROWMMA>(xv, 0, b, b, nsb, 0, l.q, l.dA, nullptr, nullptr, (uint16_t *)l.amin,
                                             nullptr, nullptr, TC);
@@ -1748,7 +1779,7 @@ int launch_moe(const MoeArgs *a, void *workspace, size_t workspace_bytes, const 
     const dim3 grid((unsigned)((d.intermediate + 63) / 64) + 1, (unsigned)d.topk);
     auto launch = [&](auto k, const char *name) {
       hipq::launch_kernel(name, k, grid, dim3(256), lds_g, s, logits, E, d.topk, d.renormalize, idx, wgt, b.offsets,
-                          b.slot_pair, b.tok_slots, b.items, a->x, views, d.intermediate, b.h, a->epi);
+                          b.slot_pair, b.tok_slots, b.items, a->x, views, d.hidden, d.intermediate, b.h, a->epi);
     };
     if (E <= 128) launch(gate_up_one_token_kernel<2>, "gate_up_one_token_kernel<2>");
     else if (E <= 256) launch(gate_up_one_token_kernel<4>, "gate_up_one_token_kernel<4>");
