@@ -579,9 +579,11 @@ template <int DT, int T, int R, int G, bool PW, int KC = HIPQ_KCHUNK> struct Gem
   } else if (DT == HIPQ_Q6_K) {
     /* ((a0+a4)+(a2+a6)) + ((a1+a5)+(a3+a7)) */
     float v = acc;
-    v = v + __shfl_xor(v, 4, 64);
-    v = v + __shfl_xor(v, 2, 64);
-    v = v + __shfl_xor(v, 1, 64);
+    /* lane l of the eight takes lanes l + 4, l + 2, l + 1 in turn (row_shl): for l = 0, the only one
+     * stored, the sums of the exchange with lanes l ^ 4, l ^ 2, l ^ 1, without the LDS crossbar */
+    v = v + hipq_dpp_f<0x104>(v);
+    v = v + hipq_dpp_f<0x102>(v);
+    v = v + hipq_dpp_f<0x101>(v);
     out.v = v;
     out.valid = chain && l == 0;
   } else {

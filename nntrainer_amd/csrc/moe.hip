@@ -380,7 +380,7 @@ template <int MAXV> __device__ __forceinline__ int nth_of_set(const unsigned lon
 /* the rank of lane kk's expert among the token's topk, ascending expert id (lanes below topk) */
 __device__ __forceinline__ int rank_by_expert(int myi, int topk) {
   int r = 0;
-  for (int j = 0; j < topk; ++j) r += __shfl(myi, j, 64) < myi;
+  for (int j = 0; j < topk; ++j) r += __builtin_amdgcn_readlane(myi, j) < myi;
   return r;
 }
 
@@ -1122,6 +1122,9 @@ __global__ __launch_bounds__(256, TC <= 8 ? 4 : TC <= 16 ? 2 : 1) void gate_up_m
   }
 }
 
+/* floats of LDS one of (gate, up) needs for the terms of the second half of K in the one-token kernel */
+__host__ __device__ constexpr int one_token_terms(int K) { return ((K >> 8) / 2 + 1) * 128; }
+
 /* One token (a decode step), the routing inside the gate/up launch: every wavefront finds the
  * token's set of experts itself (the same arithmetic on the same logits, so all agree; without the
  * softmax's exponentials where topk_set_fast can promise the same set), the workgroup takes the
@@ -1182,14 +1185,21 @@ __global__ __launch_bounds__(256, 4) void gate_up_one_token_kernel(
   const WView wg = views[e], wu = views[E + e];
   const int K = wg.K;
   const XLds l = xlds_carve(xmoe_lds, TC, K);
-  float *xch = (float *)(xmoe_lds + xlds_bytes(TC, K)); /* [2 tiles][NREG][64 lanes] */
-  const int col0 = (blockIdx.x * 2 + (wave & 1)) * 32;
-  const int first = wave >> 1; /* 0: gate, 1: up */
-  const uint64_t dqs = (uint64_t)wu.qs - (uint64_t)wg.qs;
+  /* One tile of 32 columns a workgroup, a wavefront for each of (gate, up) x (first, second half of K):
+   * with one wavefront per SIMD a super-block's eight matrix steps wait for each other, so half the
+   * super-blocks per wavefront halve the stream's time. The chain of fp32 sums keeps the reference's
+   * order: the second half's wavefront leaves its super-blocks' terms in LDS, and the first half's adds
+   * them to its own after the barrier, one super-block after the other. */
+  const int col0 = blockIdx.x * 32; /* < I: the grid has as many columns (and the one that routes) */
+  const int first = wave >> 1, half = wave & 1; /* 0: gate, 1: up; which half of K */
+  const int i32 = lane & 31, g = lane >> 5;
+  const int nsb = K >> 8, n0 = (nsb + 1) >> 1; /* the first half's super-blocks */
+  const int sb0 = half ? n0 : 0, cnt = half ? nsb - n0 : n0;
+  float *terms = (float *)(xmoe_lds + xlds_bytes(TC, K)); /* [gate, up][super-block of the second half][4 terms][32 columns] */
+  float *xch = terms + 2 * one_token_terms(K);            /* [32 columns] the gate values */
   auto stage = [&]() {
     /* rows 1 .. 7 of the matrix operand keep what the LDS held: a row of the product depends on
      * its own activations only, and those rows are not stored */
-    const int nsb = K >> 8;
 #pragma unroll
     for (int j = 0; j < XPRE; ++j) {
       const int b = wave + 4 * j;
@@ -1204,42 +1214,56 @@ __global__ __launch_bounds__(256, 4) void gate_up_one_token_kernel(
     }
     __syncthreads();
   };
-  float gate[NREG], up[NREG];
-  auto store = [&]() {
-    const int col = col0 + (lane & 31);
-    if (col < I && lane < 32) h[(size_t)item * I + col] = moe_act(ep, e, I, col, gate[0], up[0]);
+  /* the tile (nibbles and headers of its super-blocks) as a buffer descriptor in scalar registers */
+  const uint8_t *qs = first ? wu.qs : wg.qs;
+  const xrsrc_t rq = __builtin_amdgcn_make_buffer_rsrc(
+    (void *)(qs + (size_t)(col0 >> 5) * (size_t)(nsb * hipq::EXPERT_TILE_BYTES)), 0, nsb * hipq::EXPERT_TILE_BYTES,
+    0x00020000);
+  auto load = [&](XRegs &r, int sb) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) /* non-temporal: every load instruction covers whole cache lines */
+      r.q[i] = __builtin_bit_cast(
+        mv4i, __builtin_amdgcn_raw_buffer_load_b128(rq, lane * 16, sb * hipq::EXPERT_TILE_BYTES + i * 1024, 2));
+    r.hd = __builtin_bit_cast(
+      mv4i, __builtin_amdgcn_raw_buffer_load_b128(rq, 4096 + i32 * 16, sb * hipq::EXPERT_TILE_BYTES, 2));
   };
-  if (col0 >= I) { /* uniform per wavefront; it still takes part in the barriers */
-    stage();
-    __syncthreads();
-    return;
-  }
-  xr_run<TC, NREG, XPD>(
-    1, l, K,
-    [&](int t, WView &w, int &c0) {
-      const uint64_t isup = (uint64_t)0 - (uint64_t)((t + first) & 1);
-      w.qs = (const uint8_t *)((uint64_t)wg.qs + (isup & dqs));
-      w.hdr = nullptr; /* the headers follow the nibbles */
-      w.N = wg.N;
-      w.K = wg.K;
-      c0 = col0;
-    },
-    [&](int t, const float(&out)[NREG]) {
-      if (t + first == 0) {
+  XRegs buf[2];
+  if (cnt > 0) load(buf[0], sb0);
+  stage(); /* the row of x is quantized while the first weights are on their way */
+  float acc = 0.f, accm = 0.f;
+  for (int u0 = 0; u0 < cnt; u0 += 2) {
 #pragma unroll
-        for (int r = 0; r < NREG; ++r) gate[r] = out[r];
-      } else {
-#pragma unroll
-        for (int r = 0; r < NREG; ++r) up[r] = out[r];
+    for (int k = 0; k < 2; ++k) {
+      const int u = u0 + k;
+      if (u < cnt) { /* uniform per wavefront */
+        if (u + 1 < cnt) load(buf[(k + 1) & 1], sb0 + u + 1);
+        float fi[NREG], si[NREG], fm[NREG], sm[NREG];
+        xr_sb_terms<TC, NREG>(buf[k], l, K, sb0 + u, i32, g, fi, si, fm, sm);
+        if (half == 0) {
+          acc = fmaf(fi[0], si[0], acc);
+          accm = fmaf(fm[0], sm[0], accm);
+        } else if (lane < 32) {
+          float *t = terms + (size_t)((first * one_token_terms(K) / 128 + u) * 4) * 32 + lane;
+          t[0] = fi[0], t[32] = si[0], t[64] = fm[0], t[96] = sm[0];
+        }
       }
-    },
-    stage);
-  float *mine = xch + (wave & 1) * (NREG * 64) + lane;
-  if (first == 0) mine[0] = gate[0];
+    }
+  }
   __syncthreads();
-  if (first == 1) {
-    gate[0] = mine[0];
-    store();
+  float out = 0.f;
+  if (half == 0) {
+    for (int u = 0; u < nsb - n0; ++u) {
+      const float *t = terms + (size_t)((first * one_token_terms(K) / 128 + u) * 4) * 32 + i32;
+      acc = fmaf(t[0], t[32], acc);
+      accm = fmaf(t[64], t[96], accm);
+    }
+    out = acc - accm;
+    if (first == 0 && lane < 32) xch[lane] = out;
+  }
+  __syncthreads();
+  if (first == 1 && half == 0 && lane < 32) {
+    const int col = col0 + lane;
+    if (col < I) h[(size_t)item * I + col] = moe_act(ep, e, I, col, xch[lane], out);
   }
 }
 
@@ -1768,7 +1792,7 @@ int launch_moe(const MoeArgs *a, void *workspace, size_t workspace_bytes, const 
   /* one token on the matrix-core path: routing, the quantization of x and gate/up as one launch */
   const bool one_token = mma && T == 1 && chunk == 8 && mma_few(d, 8) && E <= 1024 && d.topk <= 64;
   if (one_token) {
-    const size_t lds_g = xlds_bytes(8, d.hidden) + 8 * 256;
+    const size_t lds_g = xlds_bytes(8, d.hidden) + (2 * (size_t)one_token_terms(d.hidden) + 32) * sizeof(float);
     if (lds_g > 64 * 1024) {
       const void *k = E <= 128   ? (const void *)gate_up_one_token_kernel<2>
                       : E <= 256 ? (const void *)gate_up_one_token_kernel<4>
@@ -1776,7 +1800,7 @@ int launch_moe(const MoeArgs *a, void *workspace, size_t workspace_bytes, const 
       HIPQ_HIP(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_g));
     }
     /* one block column more than the columns of h need: the routing's outputs are written there */
-    const dim3 grid((unsigned)((d.intermediate + 63) / 64) + 1, (unsigned)d.topk);
+    const dim3 grid((unsigned)((d.intermediate + 31) / 32) + 1, (unsigned)d.topk);
     auto launch = [&](auto k, const char *name) {
       hipq::launch_kernel(name, k, grid, dim3(256), lds_g, s, logits, E, d.topk, d.renormalize, idx, wgt, b.offsets,
                           b.slot_pair, b.tok_slots, b.items, a->x, views, d.hidden, d.intermediate, b.h, a->epi);

@@ -80,7 +80,7 @@ __device__ __forceinline__ void hipq_quantize_q8_K_values(
   const float x[4] = {xv.x, xv.y, xv.z, xv.w};
 
   float amax = fmaxf(fmaxf(fabsf(x[0]), fabsf(x[1])), fmaxf(fabsf(x[2]), fabsf(x[3])));
-  amax = hipq_group_max<64>(amax);
+  amax = hipq_wave_max(amax); /* the same value in every lane, without an exchange through LDS */
 
   int q[4];
   float d;
@@ -110,7 +110,7 @@ __device__ __forceinline__ void hipq_quantize_q8_K_values(
       }
     const unsigned long long mask = __ballot(has);
     const int first = __ffsll((long long)mask) - 1;
-    const float vmax = __shfl(cand, first, HIPQ_WAVE);
+    const float vmax = __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, cand), first));
     const float iscale = __fdiv_rn(-127.f, vmax);
     d = __fdiv_rn(1.f, iscale);
 #pragma unroll
@@ -133,7 +133,7 @@ __device__ __forceinline__ void hipq_quantize_q8_K_values(
     const uint4 op = hipq_quad_operand(q);
     if ((lane & 3) == 0) *(uint4 *)(q_out + sb * 256 + (lane >> 2) * 16) = op;
     if (lane == 0) d_out[sb * d_stride] = d;
-    const int bs = gsum + __shfl_xor(gsum, 4, HIPQ_WAVE); /* two 16-value groups = one sub-block */
+    const int bs = gsum + hipq_dpp_i<0x104>(gsum); /* row_shl:4: lane l takes lane l + 4; two 16-value groups = one sub-block (read in lanes 0 and 8 of a row) */
     if ((lane & 7) == 0) {
       const int l6 = bs & 63;
       amin_out[sb * 16 + (lane >> 3)] = __half_as_ushort(__float2half_rn((float)l6));
