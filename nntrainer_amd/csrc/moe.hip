@@ -1312,6 +1312,14 @@ __global__ __launch_bounds__(256, TC <= 8 ? 4 : TC <= 16 ? 2 : 1) void down_mma_
     stage();
     return;
   }
+  /* the routing weights of this lane's rows are asked for now: two dependent reads that would
+   * otherwise stand between the last super-block and the store */
+  float wrow[NREG];
+#pragma unroll
+  for (int r = 0; r < NREG; ++r) {
+    const int tok = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
+    wrow[r] = wgt[slot_pair[min(s0 + tok, end - 1)]];
+  }
   xr_run<TC, NREG, XPD>(
     ntile, l, K,
     [&](int t, WView &w, int &c0) {
@@ -1323,8 +1331,7 @@ __global__ __launch_bounds__(256, TC <= 8 ? 4 : TC <= 16 ? 2 : 1) void down_mma_
 #pragma unroll
       for (int r = 0; r < NREG; ++r) {
         const int tok = 8 * (r >> 2) + 4 * (lane >> 5) + (r & 3);
-        if (col < H && s0 + tok < end)
-          contrib[(size_t)(s0 + tok) * H + col] = moe_out(ep, e, H, col, out[r], wgt[slot_pair[s0 + tok]]);
+        if (col < H && s0 + tok < end) contrib[(size_t)(s0 + tok) * H + col] = moe_out(ep, e, H, col, out[r], wrow[r]);
       }
     },
     stage);
