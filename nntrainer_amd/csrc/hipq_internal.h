@@ -414,6 +414,18 @@ __device__ __forceinline__ float hipq_wave_sum(float v) {
   return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), 63));
 }
 
+/* Inclusive prefix sum over the lanes of a wavefront by shifted adds inside the rows of sixteen
+ * lanes (row_shr 1, 2, 4, 8: lanes without a source add zero) and the two row-broadcast steps. */
+__device__ __forceinline__ int hipq_wave_prefix_sum_i(int v) {
+  v += hipq_dpp_i<0x111>(v);
+  v += hipq_dpp_i<0x112>(v);
+  v += hipq_dpp_i<0x114>(v);
+  v += hipq_dpp_i<0x118>(v);
+  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xa, 0xf, false); /* rows 1 and 3 take the total of the row before */
+  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xc, 0xf, false); /* rows 2 and 3 take the total of rows 0 and 1 */
+  return v;
+}
+
 /* Loads of weight data name the global address space. A pointer that a kernel
  * read from memory (a table of weight views) is generic to the compiler, which
  * then emits flat loads; those count against the LDS counter as well, so every

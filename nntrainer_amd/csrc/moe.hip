@@ -1292,13 +1292,24 @@ __global__ __launch_bounds__(256, TC <= 8 ? 4 : TC <= 16 ? 2 : 1) void down_mma_
     if (QH) {
       /* rows past the item's end stay as they are: a row of the matrix product
        * depends on its own activations only, and those rows are not stored */
-      const int nsb = K >> 8;
-      for (int u = wave; u < (end - s0) * nsb; u += 4) { /* uniform per wavefront */
-        const int r = u / nsb, b = u - r * nsb;
-        const float4 xv = *(const float4 *)(hf + (size_t)(s0 + r) * K + b * 256 + lane * 4);
-        hipq_quantize_q8_K_values<Q8K_ROWMMA>(xv, 0, b, b, nsb, 0, l.q + (size_t)r * (K + 16), l.dA + r, nullptr,
-                                              nullptr, (uint16_t *)(l.amin + (size_t)r * nsb * 32), nullptr,
-                                              nullptr, TC);
+      const int nsb = K >> 8, units = (end - s0) * nsb;
+      for (int u0 = wave; u0 < units; u0 += 16) { /* uniform per wavefront; four loads, then four quantizations */
+        float4 xv[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const int u = min(u0 + 4 * k, units - 1), r = u / nsb, b = u - r * nsb;
+          xv[k] = *(const float4 *)(hf + (size_t)(s0 + r) * K + b * 256 + lane * 4);
+        }
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+          const int u = u0 + 4 * k;
+          if (u < units) {
+            const int r = u / nsb, b = u - r * nsb;
+            hipq_quantize_q8_K_values<Q8K_ROWMMA>(xv[k], 0, b, b, nsb, 0, l.q + (size_t)r * (K + 16), l.dA + r,
+                                                  nullptr, nullptr, (uint16_t *)(l.amin + (size_t)r * nsb * 32),
+                                                  nullptr, nullptr, TC);
+          }
+        }
       }
       __syncthreads();
       return;
@@ -1364,12 +1375,7 @@ __device__ __forceinline__ int self_scan(const int32_t *__restrict__ idx, int P,
     const int i = t * pp + u;
     if (i < P && idx[i] == e) mask |= 1u << u, ++m;
   }
-  int inc = m;
-#pragma unroll
-  for (int d = 1; d < 64; d <<= 1) {
-    const int v = __shfl_up(inc, d, 64);
-    if (lane >= d) inc += v;
-  }
+  const int inc = hipq_wave_prefix_sum_i(m); /* inclusive, over the lanes */
   if (lane == 63) wtot[wave] = inc;
   __syncthreads();
   int base = 0, total = 0;
@@ -1473,13 +1479,27 @@ __device__ __forceinline__ void down_self_pass(unsigned char *lds, int n, int e,
   auto stage = [&]() {
     /* rows past the chunk's end stay as they are: a row of the matrix product depends on its own
      * activations only, and those rows are not stored */
-    const int nsb = K >> 8;
-    for (int u = wave; u < n * nsb; u += 4) { /* uniform per wavefront */
-      const int r = u / nsb, b = u - r * nsb;
-      const float4 xv = *(const float4 *)(hf + (size_t)l.pairs[r] * K + b * 256 + lane * 4);
-      hipq_quantize_q8_K_values<Q8K_ROWMMA>(xv, 0, b, b, nsb, 0, l.q + (size_t)r * (K + 16), l.dA + r, nullptr,
-                                            nullptr, (uint16_t *)(l.amin + (size_t)r * nsb * 32), nullptr, nullptr,
-                                            TC);
+    const int nsb = K >> 8, units = n * nsb;
+    /* a wavefront's (row, super-block) units four at a time: the four loads first, then the four
+     * quantizations (one after the other, a unit's load is a round trip of its own: 4-6 us of this
+     * kernel's start with three rows of three super-blocks) */
+    for (int u0 = wave; u0 < units; u0 += 16) { /* uniform per wavefront */
+      float4 xv[4];
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const int u = min(u0 + 4 * k, units - 1), r = u / nsb, b = u - r * nsb;
+        xv[k] = *(const float4 *)(hf + (size_t)l.pairs[r] * K + b * 256 + lane * 4);
+      }
+#pragma unroll
+      for (int k = 0; k < 4; ++k) {
+        const int u = u0 + 4 * k;
+        if (u < units) {
+          const int r = u / nsb, b = u - r * nsb;
+          hipq_quantize_q8_K_values<Q8K_ROWMMA>(xv[k], 0, b, b, nsb, 0, l.q + (size_t)r * (K + 16), l.dA + r, nullptr,
+                                                nullptr, (uint16_t *)(l.amin + (size_t)r * nsb * 32), nullptr,
+                                                nullptr, TC);
+        }
+      }
     }
     __syncthreads();
   };
