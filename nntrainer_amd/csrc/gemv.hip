@@ -81,9 +81,11 @@ template <int DT> __host__ __device__ constexpr int fused_act_bytes(int K) {
   return ((DT == HIPQ_Q4_0 ? K + K / 8 : 2 * K + K / 8 + K / 64) + 15) & ~15;
 }
 
-template <int DT, int T, int G, int NW, typename Store>
+template <int DT, int T, int G, int NW, int WV = 4, typename Store>
 __device__ __forceinline__ void gemv_fused_rows(const WView (&wv)[NW], const float *__restrict__ x, int block,
                                                 Store store) {
+  static_assert(WV == 4 || (DT != HIPQ_Q4_0 && WV == 12), "wavefronts a workgroup");
+  constexpr int XP = 16 / WV + (16 % WV != 0); /* super-blocks of the row a wavefront quantizes, at most (K <= 4096) */
   typedef GemvCore<DT, T, 1, G, false> E;
   const WView &w = wv[0];
   extern __shared__ __attribute__((aligned(16))) uint32_t gemv_lds[];
@@ -91,7 +93,7 @@ __device__ __forceinline__ void gemv_fused_rows(const WView (&wv)[NW], const flo
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   uint8_t *ap = (uint8_t *)gemv_lds;
   uint32_t *lds = gemv_lds + fused_act_bytes<DT>(K) / 4 + wave * GemvLds<DT, 1, G, false>::DWORDS;
-  const int row0 = (block * 4 + wave) * G;
+  const int row0 = (block * WV + wave) * G;
   const int arow[1] = {0};
 
   /* the row first (it comes from the cache), then the weights: the wait for the row
@@ -105,7 +107,7 @@ __device__ __forceinline__ void gemv_fused_rows(const WView (&wv)[NW], const flo
   } else {
     const int nsb = K >> 8;
 #pragma unroll
-    for (int p = 0; p < 4; ++p) xs[p] = *(const float4 *)(x + min(wave + 4 * p, nsb - 1) * 256 + lane * 4);
+    for (int p = 0; p < XP; ++p) xs[p] = *(const float4 *)(x + min(wave + WV * p, nsb - 1) * 256 + lane * 4);
   }
   typename E::Wts W[NW];
 #pragma unroll
@@ -147,8 +149,8 @@ __device__ __forceinline__ void gemv_fused_rows(const WView (&wv)[NW], const flo
     qa.qh = (const uint8_t *)qh;
     const int nsb = K >> 8;
 #pragma unroll
-    for (int p = 0; p < 4; ++p) {
-      const int sb = wave + 4 * p;
+    for (int p = 0; p < XP; ++p) {
+      const int sb = wave + WV * p;
       if (sb >= nsb) break; /* uniform per wavefront */
       hipq_quantize_q8_K_values < DT == HIPQ_Q4_K ? Q8K_DIGITS : Q8K_BYTES > (xs[p], 0, sb, sb, nsb, 0, q, d, bsum,
                                                                              nullptr, nullptr, ql, qh);
@@ -202,6 +204,14 @@ __global__ __launch_bounds__(256) void gemv_fused_kernel(WView w, const float *_
                                                          float *__restrict__ C) {
   gemv_fused_body<DT, T, G>(w, x, C, (int)blockIdx.x);
 }
+/* The same with WV wavefronts a workgroup: one workgroup a CU quantizes the row once where three of four
+ * wavefronts each would quantize it three times (see launch_fused for where that pays). */
+template <int DT, int T, int G, int WV>
+__global__ __launch_bounds__(64 * WV) void gemv_fused_wide_kernel(WView w, const float *__restrict__ x,
+                                                                  float *__restrict__ C) {
+  const WView wv[1] = {w};
+  gemv_fused_rows<DT, T, G, 1, WV>(wv, x, (int)blockIdx.x, [&](int row, const GemvOut(&o)[1]) { C[row] = o[0].v; });
+}
 
 /* Up to four weights of one format and K on the same row, one launch: the
  * workgroups of weight i are blocks end[i-1] .. end[i]-1 of the grid. */
@@ -234,6 +244,15 @@ int launch_fused_many(int count, const hipq_weight *const *w, const float *x, fl
   }
   const size_t lds = fused_act_bytes<DT>((int)w[0]->K) + 4 * GemvLds<DT, 1, G, false>::DWORDS * sizeof(uint32_t);
   hipq::launch_kernel("gemv_fused_multi_kernel<DT, T, G>", (gemv_fused_multi_kernel<DT, T, G>), dim3((unsigned)blocks), dim3(256), lds, s, mw, x);
+  HIPQ_HIP(hipGetLastError());
+  return HIPQ_OK;
+}
+
+template <int DT, int T, int G, int WV>
+int launch_fused_wide(const hipq_weight *w, const float *x, float *C, hipStream_t s) {
+  const unsigned grid = (unsigned)((w->N + WV * G - 1) / (WV * G));
+  const size_t lds = fused_act_bytes<DT>((int)w->K) + WV * GemvLds<DT, 1, G, false>::DWORDS * sizeof(uint32_t);
+  hipq::launch_kernel("gemv_fused_wide_kernel<DT, T, G, WV>", (gemv_fused_wide_kernel<DT, T, G, WV>), dim3(grid), dim3(64 * WV), lds, s, wview(w), x, C);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
 }
@@ -340,6 +359,14 @@ template <int DT> int launch_fused(const hipq_weight *w, const float *x, float *
   if (units < 64) {
     if (pick_group(w->N, 8) == 8) return launch_fused_one<DT, 16, 8>(w, x, C, s);
     return launch_fused_one<DT, 16, 4>(w, x, C, s);
+  }
+  if constexpr (DT == HIPQ_Q4_K) {
+    /* Four rows a wavefront and at most one workgroup of twelve wavefronts a CU (256 of them): the row is
+     * quantized once a CU instead of three times. Measured, us a call, four -> twelve wavefronts:
+     * 10240 x 4096 9.3 -> 8.5, 11008 x 4096 9.5 -> 8.8, 12288 x 4096 9.7 -> 9.2, 12288 x 2048 6.1 -> 5.6; with
+     * more rows than one round of such workgroups it loses (14336 x 4096 11.0 -> 13.5), and Q6_K loses
+     * everywhere (12288 x 4096 11.8 -> 12.1). */
+    if (pick_group(w->N, 8) == 4 && (w->N + 47) / 48 <= 256) return launch_fused_wide<DT, 64, 4, 12>(w, x, C, s);
   }
   switch (pick_group(w->N, 8)) {
   case 8:
