@@ -1364,16 +1364,38 @@ __global__ __launch_bounds__(256, TC <= 8 ? 4 : TC <= 16 ? 2 : 1) void down_mma_
 constexpr int SELF_TC = 16;     /* pairs per chunk */
 constexpr int SELF_HEAD = 128;  /* bytes of LDS in front of the rows: pairs[16], tokens[16] */
 
-__device__ __forceinline__ int self_scan(const int32_t *__restrict__ idx, int P, int topk, int e, int chunk,
-                                         int *pairs, int *rows) {
+/* The scan of the routing's output in two parts, so that a workgroup can ask for other things
+ * between them: the loads of idx (up to four pairs per thread in registers; longer lists are read
+ * in the second part), then the counting. */
+struct SelfAsk {
+  int v[4];
+};
+
+__device__ __forceinline__ SelfAsk self_scan_ask(const int32_t *__restrict__ idx, int P) {
+  const int t = threadIdx.x;
+  const int pp = (P + 255) >> 8; /* pairs per thread, consecutive: thread order is pair order */
+  SelfAsk a;
+#pragma unroll
+  for (int u = 0; u < 4; ++u) a.v[u] = idx[min(t * pp + min(u, pp - 1), P - 1)];
+  return a;
+}
+
+__device__ __forceinline__ int self_scan(const SelfAsk &a, const int32_t *__restrict__ idx, int P, int topk, int e,
+                                         int chunk, int *pairs, int *rows) {
   __shared__ int wtot[4];
   const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-  const int pp = (P + 255) >> 8; /* pairs per thread, consecutive: thread order is pair order */
+  const int pp = (P + 255) >> 8;
   int m = 0;
   uint32_t mask = 0;
-  for (int u = 0; u < pp; ++u) {
-    const int i = t * pp + u;
-    if (i < P && idx[i] == e) mask |= 1u << u, ++m;
+  if (pp <= 4) { /* uniform */
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (u < pp && t * pp + u < P && a.v[u] == e) mask |= 1u << u, ++m;
+  } else {
+    for (int u = 0; u < pp; ++u) {
+      const int i = t * pp + u;
+      if (i < P && idx[i] == e) mask |= 1u << u, ++m;
+    }
   }
   const int inc = hipq_wave_prefix_sum_i(m); /* inclusive, over the lanes */
   if (lane == 63) wtot[wave] = inc;
@@ -1397,10 +1419,35 @@ __device__ __forceinline__ int self_scan(const int32_t *__restrict__ idx, int P,
   return total;
 }
 
+/* Load instructions that touch every cache line of a wavefront's first NT super-blocks of column
+ * tile `tile` (a lane per 128 bytes, one instruction a super-block), so that the lines are on their
+ * way to the caches while the workgroup finds its pairs and stages its rows. The values come back in
+ * NT registers, which self_touched() takes behind the staging's barrier. */
+/* One super-block: touching two or three made the block 1-4 us slower (the lines do not stay in
+ * the L2 until they are used). */
+constexpr int SELF_TOUCH = 1;
+template <int NT> struct SelfTouch {
+  int v[NT];
+};
+template <int NT> __device__ __forceinline__ void self_touch(SelfTouch<NT> &t, const WView &w, int tile) {
+  const int nsb = w.K >> 8, lane = threadIdx.x & 63;
+  const xrsrc_t rq =
+    __builtin_amdgcn_make_buffer_rsrc((void *)(w.qs + (size_t)tile * (size_t)(nsb * hipq::EXPERT_TILE_BYTES)), 0,
+                                      min(NT, nsb) * hipq::EXPERT_TILE_BYTES, 0x00020000);
+#pragma unroll
+  for (int i = 0; i < NT; ++i) /* lanes past a super-block's end, and super-blocks past the tile's, read nothing */
+    t.v[i] = __builtin_amdgcn_raw_buffer_load_b32(rq, lane < hipq::EXPERT_TILE_BYTES / 128 ? lane * 128 : 0x7fffff00,
+                                                  i * hipq::EXPERT_TILE_BYTES, 0);
+}
+template <int NT> __device__ __forceinline__ void self_touched(const SelfTouch<NT> &t) {
+#pragma unroll
+  for (int i = 0; i < NT; ++i) asm volatile("" ::"v"(t.v[i]));
+}
+
 template <int TC>
 __device__ __forceinline__ void gate_up_self_pass(unsigned char *lds, int n, int e, const WView &wg, const WView &wu,
                                                   const QView &xq, int I, float *__restrict__ h,
-                                                  const hipq::MoeEpi &ep) {
+                                                  const hipq::MoeEpi &ep, const SelfTouch<SELF_TOUCH> &touched) {
   constexpr int NREG = TC / 2;
   const int K = wg.K;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
@@ -1412,6 +1459,7 @@ __device__ __forceinline__ void gate_up_self_pass(unsigned char *lds, int n, int
   auto stage = [&]() {
     stage_rows<TC>(l, xq, n);
     __syncthreads();
+    self_touched(touched);
   };
   if (col0 >= I) { /* uniform per wavefront; it still takes part in the barrier */
     stage();
@@ -1451,15 +1499,21 @@ __global__ __launch_bounds__(256, 4) void gate_up_self_kernel(const WView *__res
                                                               float *__restrict__ h, hipq::MoeEpi ep) {
   extern __shared__ __attribute__((aligned(16))) unsigned char xmoe_lds[];
   const int e = blockIdx.y % E_, chunk = blockIdx.y / E_;
-  const WView wg = views[e], wu = views[E_ + e]; /* asked for before the scan: they are there when it ends */
+  const SelfAsk ask = self_scan_ask(idx, P);
+  const WView wg = views[e], wu = views[E_ + e];
+  /* a workgroup of the first chunk row has work unless nobody chose its expert: its first
+   * weights start towards the L2 before it knows its pairs */
+  const int col0 = (blockIdx.x * 4 + (int)(threadIdx.x >> 6)) * 32;
+  SelfTouch<SELF_TOUCH> touched = {};
+  if (chunk == 0 && col0 < I) self_touch(touched, wg, __builtin_amdgcn_readfirstlane(col0 >> 5));
   int *pairs = (int *)xmoe_lds;
-  const int total = self_scan(idx, P, topk, e, chunk, pairs, pairs + SELF_TC);
+  const int total = self_scan(ask, idx, P, topk, e, chunk, pairs, pairs + SELF_TC);
   const int n = min(SELF_TC, total - chunk * SELF_TC);
   if (n <= 0) return; /* uniform per workgroup */
   if (n <= 8)
-    gate_up_self_pass<8>(xmoe_lds, n, e, wg, wu, xq, I, h, ep);
+    gate_up_self_pass<8>(xmoe_lds, n, e, wg, wu, xq, I, h, ep, touched);
   else
-    gate_up_self_pass<16>(xmoe_lds, n, e, wg, wu, xq, I, h, ep);
+    gate_up_self_pass<16>(xmoe_lds, n, e, wg, wu, xq, I, h, ep, touched);
 }
 
 /* The rows of h come as fp32 and the workgroup quantizes those of its chunk itself while its first
@@ -1467,7 +1521,8 @@ __global__ __launch_bounds__(256, 4) void gate_up_self_kernel(const WView *__res
 template <int TC>
 __device__ __forceinline__ void down_self_pass(unsigned char *lds, int n, int e, const WView &wd,
                                                const float *__restrict__ hf, const float *__restrict__ wgt,
-                                               int H, float *__restrict__ contrib, const hipq::MoeEpi &ep) {
+                                               int H, float *__restrict__ contrib, const hipq::MoeEpi &ep,
+                                               const SelfTouch<SELF_TOUCH> &touched) {
   constexpr int NREG = TC / 2, CT = 2;
   const int K = wd.K;
   const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
@@ -1502,6 +1557,7 @@ __device__ __forceinline__ void down_self_pass(unsigned char *lds, int n, int e,
       }
     }
     __syncthreads();
+    self_touched(touched);
   };
   if (ntile <= 0) {
     stage();
@@ -1534,15 +1590,19 @@ __global__ __launch_bounds__(256, 4) void down_self_kernel(const WView *__restri
                                                            float *__restrict__ contrib, hipq::MoeEpi ep) {
   extern __shared__ __attribute__((aligned(16))) unsigned char xmoe_lds[];
   const int e = blockIdx.y % E_, chunk = blockIdx.y / E_;
-  const WView wd = views[2 * E_ + e]; /* asked for before the scan */
+  const SelfAsk ask = self_scan_ask(idx, P);
+  const WView wd = views[2 * E_ + e];
+  const int col0 = (blockIdx.x * 4 + (int)(threadIdx.x >> 6)) * 64; /* two column tiles per wavefront */
+  SelfTouch<SELF_TOUCH> touched = {};
+  if (chunk == 0 && col0 < H) self_touch(touched, wd, __builtin_amdgcn_readfirstlane(col0 >> 5));
   int *pairs = (int *)xmoe_lds;
-  const int total = self_scan(idx, P, topk, e, chunk, pairs, pairs + SELF_TC);
+  const int total = self_scan(ask, idx, P, topk, e, chunk, pairs, pairs + SELF_TC);
   const int n = min(SELF_TC, total - chunk * SELF_TC);
   if (n <= 0) return; /* uniform per workgroup */
   if (n <= 8)
-    down_self_pass<8>(xmoe_lds, n, e, wd, hf, wgt, H, contrib, ep);
+    down_self_pass<8>(xmoe_lds, n, e, wd, hf, wgt, H, contrib, ep, touched);
   else
-    down_self_pass<16>(xmoe_lds, n, e, wd, hf, wgt, H, contrib, ep);
+    down_self_pass<16>(xmoe_lds, n, e, wd, hf, wgt, H, contrib, ep, touched);
 }
 
 /* y[t][c] = sum of the token's contributions, ascending expert id */
