@@ -83,7 +83,7 @@ template <int DT> __host__ __device__ constexpr int fused_act_bytes(int K) {
 
 template <int DT, int T, int G, int NW, int WV = 4, typename Store>
 __device__ __forceinline__ void gemv_fused_rows(const WView (&wv)[NW], const float *__restrict__ x, int block,
-                                                Store store, bool late = false) {
+                                                Store store, int late = 0) {
   static_assert(WV == 4 || (DT != HIPQ_Q4_0 && WV == 12), "wavefronts a workgroup");
   constexpr int XP = 16 / WV + (16 % WV != 0); /* super-blocks of the row a wavefront quantizes, at most (K <= 4096) */
   typedef GemvCore<DT, T, 1, G, false> E;
@@ -109,7 +109,8 @@ __device__ __forceinline__ void gemv_fused_rows(const WView (&wv)[NW], const flo
 #pragma unroll
     for (int p = 0; p < XP; ++p) xs[p] = *(const float4 *)(x + min(wave + WV * p, nsb - 1) * 256 + lane * 4);
   }
-  /* late (uniform): the weights are asked for behind the row's quantization instead of in front of it.
+  /* late (uniform) 1: the weights are asked for behind the row's quantization instead of in front of it; 2: the
+   * first half of the wavefront's rows in front, the other half behind.
    * A wavefront's weight loads fill the CU's queue of outstanding requests, and a wavefront that is still
    * issuing them has not begun to quantize its share of the row, for which the whole workgroup waits at
    * the barrier: from 16 M weights on the quantization first is faster (us a call, Q4_K 14336 x 4096
@@ -117,9 +118,13 @@ __device__ __forceinline__ void gemv_fused_rows(const WView (&wv)[NW], const flo
    * 4096 x 4096 7.0 -> 6.4); a matrix of a few MB is served from one round of loads either way, and there
    * the overlap of the two latencies is worth as much (2048 x 2048 4.12 against 4.16-4.37). */
   typename E::Wts W[NW];
+  constexpr int HP = E::NP / 2; /* late == 2: the first half of a wavefront's passes in front, the rest behind */
   if (!late) {
 #pragma unroll
     for (int i = 0; i < NW; ++i) E::load_w(W[i], wv[i], row0, 0, K);
+  } else if (late == 2) {
+#pragma unroll
+    for (int i = 0; i < NW; ++i) E::template load_w<0, HP>(W[i], wv[i], row0, 0, K);
   }
 
   QView qa;
@@ -165,9 +170,12 @@ __device__ __forceinline__ void gemv_fused_rows(const WView (&wv)[NW], const flo
                                                                              nullptr, nullptr, ql, qh);
     }
   }
-  if (late) {
+  if (late == 1) {
 #pragma unroll
     for (int i = 0; i < NW; ++i) E::load_w(W[i], wv[i], row0, 0, K);
+  } else if (late == 2) {
+#pragma unroll
+    for (int i = 0; i < NW; ++i) E::template load_w<HP, E::NP>(W[i], wv[i], row0, 0, K);
   }
   __syncthreads();
 
@@ -189,7 +197,7 @@ __device__ __forceinline__ void gemv_fused_rows(const WView (&wv)[NW], const flo
 
 template <int DT, int T, int G>
 __device__ __forceinline__ void gemv_fused_body(const WView &w, const float *__restrict__ x,
-                                                float *__restrict__ C, int block, bool late = false) {
+                                                float *__restrict__ C, int block, int late = 0) {
   const WView wv[1] = {w};
   gemv_fused_rows<DT, T, G, 1>(wv, x, block, [&](int row, const GemvOut(&o)[1]) { C[row] = o[0].v; }, late);
 }
@@ -204,18 +212,21 @@ __device__ __forceinline__ void gemv_fused_body(const WView &w, const float *__r
 template <int DT, int T, int G>
 __global__ __launch_bounds__(256) void gemv_fused_swiglu_kernel(WView wact, WView wmul,
                                                                 const float *__restrict__ x,
-                                                                float *__restrict__ out) {
+                                                                float *__restrict__ out, int late) {
   const WView wv[2] = {wact, wmul};
-  gemv_fused_rows<DT, T, G, 2>(wv, x, (int)blockIdx.x, [&](int row, const GemvOut(&o)[2]) {
-    const float y = o[0].v, z = o[1].v;
-    out[row] = (y / (1.f + expf(-y))) * z;
-  });
+  gemv_fused_rows<DT, T, G, 2>(
+    wv, x, (int)blockIdx.x,
+    [&](int row, const GemvOut(&o)[2]) {
+      const float y = o[0].v, z = o[1].v;
+      out[row] = (y / (1.f + expf(-y))) * z;
+    },
+    late);
 }
 
 template <int DT, int T, int G>
 __global__ __launch_bounds__(256) void gemv_fused_kernel(WView w, const float *__restrict__ x,
                                                          float *__restrict__ C, int late) {
-  gemv_fused_body<DT, T, G>(w, x, C, (int)blockIdx.x, late != 0);
+  gemv_fused_body<DT, T, G>(w, x, C, (int)blockIdx.x, late);
 }
 /* The same with WV wavefronts a workgroup: one workgroup a CU quantizes the row once where three of four
  * wavefronts each would quantize it three times (see launch_fused for where that pays). */
@@ -224,7 +235,7 @@ __global__ __launch_bounds__(64 * WV) void gemv_fused_wide_kernel(WView w, const
                                                                   float *__restrict__ C, int late) {
   const WView wv[1] = {w};
   gemv_fused_rows<DT, T, G, 1, WV>(
-    wv, x, (int)blockIdx.x, [&](int row, const GemvOut(&o)[1]) { C[row] = o[0].v; }, late != 0);
+    wv, x, (int)blockIdx.x, [&](int row, const GemvOut(&o)[1]) { C[row] = o[0].v; }, late);
 }
 
 /* Up to four weights of one format and K on the same row, one launch: the
@@ -236,41 +247,58 @@ struct FusedMulti {
   int end[FUSED_MAXW];
 };
 template <int DT, int T, int G>
-__global__ __launch_bounds__(256) void gemv_fused_multi_kernel(FusedMulti mw, const float *__restrict__ x) {
+__global__ __launch_bounds__(256) void gemv_fused_multi_kernel(FusedMulti mw, const float *__restrict__ x, int late) {
   const int b = (int)blockIdx.x;
   int i = 0;
 #pragma unroll
   for (int k = 0; k + 1 < FUSED_MAXW; ++k) i += b >= mw.end[k];
   const int first = i ? mw.end[i - 1] : 0;
-  gemv_fused_body<DT, T, G>(mw.w[i], x, mw.C[i], b - first);
+  gemv_fused_body<DT, T, G>(mw.w[i], x, mw.C[i], b - first, late);
 }
+
+/* Where a wavefront asks for its weights (gemv_fused_rows' `late`): in front of the row's quantization below
+ * 16 M weights, behind it above; and with rows of 4096 the first half in front and the rest behind where that
+ * measured faster (us a call, behind -> half and half: Q4_K in the twelve-wavefront form 10240 x 4096 8.8 -> 8.45,
+ * 12288 x 4096 9.35 -> 8.8, but 12288 x 2048 5.8 -> 6.05; four wavefronts, 13312 .. 16384 x 4096 the same within
+ * 0.2, 20480 14.3 -> 13.5, 24576 15.6 -> 14.8, 28672 16.9 -> 16.6; Q4_0 8192 x 4096 9.0 -> 8.9, 12288 10.7 -> 9.95;
+ * Q6_K 4096 x 4096 6.8 -> 6.65, 8192 9.65 -> 8.7, 12288 the same, 16384 13.8 -> 14.0). */
+static inline int fused_weights_late(const hipq_weight *w, bool wide = false) {
+  if (w->N * w->K < ((int64_t)1 << 24)) return 0;
+  if (w->K < 4096) return 1;
+  if (w->dtype == HIPQ_Q4_K) return wide || w->N >= 20480 ? 2 : 1;
+  if (w->dtype == HIPQ_Q4_0) return w->N >= 8192 ? 2 : 1;
+  return w->N <= 8192 ? 2 : 1;
+}
+/* the same for launches of several matrices on one row (their weights counted together) */
+static inline int fused_weights_late(int64_t weights) { return weights >= ((int64_t)1 << 24) ? 1 : 0; }
 
 template <int DT, int T, int G>
 int launch_fused_many(int count, const hipq_weight *const *w, const float *x, float *const *C, hipStream_t s) {
   FusedMulti mw;
   int blocks = 0;
+  int64_t weights = 0;
   for (int i = 0; i < FUSED_MAXW; ++i) {
     const int j = i < count ? i : count - 1;
     mw.w[i] = wview(w[j]);
     mw.C[i] = C[j];
-    if (i < count) blocks += (int)((w[i]->N + 4 * G - 1) / (4 * G));
+    if (i < count) blocks += (int)((w[i]->N + 4 * G - 1) / (4 * G)), weights += w[i]->N * w[i]->K;
     mw.end[i] = blocks;
   }
   const size_t lds = fused_act_bytes<DT>((int)w[0]->K) + 4 * GemvLds<DT, 1, G, false>::DWORDS * sizeof(uint32_t);
-  hipq::launch_kernel("gemv_fused_multi_kernel<DT, T, G>", (gemv_fused_multi_kernel<DT, T, G>), dim3((unsigned)blocks), dim3(256), lds, s, mw, x);
+  hipq::launch_kernel("gemv_fused_multi_kernel<DT, T, G>", (gemv_fused_multi_kernel<DT, T, G>), dim3((unsigned)blocks), dim3(256), lds, s, mw, x,
+                      fused_weights_late(weights));
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
 }
 
 /* whether a fused launch asks for its weights behind the row's quantization (gemv_fused_rows) */
-static inline int fused_weights_late(const hipq_weight *w) { return w->N * w->K >= ((int64_t)1 << 24) ? 1 : 0; }
 
 template <int DT, int T, int G, int WV>
 int launch_fused_wide(const hipq_weight *w, const float *x, float *C, hipStream_t s) {
   const unsigned grid = (unsigned)((w->N + WV * G - 1) / (WV * G));
   const size_t lds = fused_act_bytes<DT>((int)w->K) + WV * GemvLds<DT, 1, G, false>::DWORDS * sizeof(uint32_t);
   hipq::launch_kernel("gemv_fused_wide_kernel<DT, T, G, WV>", (gemv_fused_wide_kernel<DT, T, G, WV>), dim3(grid), dim3(64 * WV), lds, s, wview(w), x, C,
-                      fused_weights_late(w));
+                      fused_weights_late(w, true));
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
 }
@@ -321,7 +349,7 @@ int launch_fused_swiglu_one(const hipq_weight *wa, const hipq_weight *wm, const 
   const unsigned grid = (unsigned)((wa->N + 4 * G - 1) / (4 * G));
   const size_t lds = fused_act_bytes<DT>((int)wa->K) + 4 * GemvLds<DT, 1, G, false>::DWORDS * sizeof(uint32_t);
   hipq::launch_kernel("gemv_fused_swiglu_kernel<DT, T, G>", (gemv_fused_swiglu_kernel<DT, T, G>), dim3(grid), dim3(256), lds, s, wview(wa), wview(wm), x,
-                     out);
+                     out, fused_weights_late(2 * wa->N * wa->K));
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
 }

@@ -471,11 +471,12 @@ template <int DT, int T, int R, int G, bool PW, int KC = HIPQ_KCHUNK> struct Gem
                                                   int k0, int kc) {
     F::load_act(A, qa, arow, (threadIdx.x & 63) % T, k0, kc);
   }
-  /* issue the loads of the G weight rows from row0 (clamped to the matrix) */
+  /* issue the loads of the G weight rows from row0 (clamped to the matrix); P0, P1: of passes P0 .. P1 - 1 only */
+  template <int P0 = 0, int P1 = NP>
   __device__ static __forceinline__ void load_w(Wts &w, const WView &wv, int row0, int k0, int kc) {
     const int lane = threadIdx.x & 63, tl = lane % T;
 #pragma unroll
-    for (int pass = 0; pass < NP; ++pass) {
+    for (int pass = P0; pass < P1; ++pass) {
       const int g = pass * RW + lane / T;
       F::load_w(w.W[pass], wv, min(row0 + g, wv.N - 1), tl, k0, kc);
     }
