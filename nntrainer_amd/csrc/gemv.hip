@@ -17,6 +17,8 @@
  * HBM: per output column it reads the column's packed weights exactly once,
  * 16 bytes per lane per load, all loads of a group in flight together.
  */
+#include <type_traits>
+
 #include "gemv_device.h"
 #include "quantize_device.h"
 
@@ -81,15 +83,18 @@ template <int DT> __host__ __device__ constexpr int fused_act_bytes(int K) {
   return ((DT == HIPQ_Q4_0 ? K + K / 8 : 2 * K + K / 8 + K / 64) + 15) & ~15;
 }
 
-template <int DT, int T, int G, int NW, int WV = 4, typename Store>
+template <int DT, int T, int G, int NW, int LATE, int FK, int WV = 4, typename Store>
 __device__ __forceinline__ void gemv_fused_rows(const WView (&wv)[NW], const float *__restrict__ x, int block,
-                                                Store store, int late = 0) {
+                                                Store store) {
   static_assert(WV == 4 || (DT != HIPQ_Q4_0 && WV == 12), "wavefronts a workgroup");
   constexpr int XP = 16 / WV + (16 % WV != 0); /* super-blocks of the row a wavefront quantizes, at most (K <= 4096) */
   typedef GemvCore<DT, T, 1, G, false> E;
   const WView &w = wv[0];
   extern __shared__ __attribute__((aligned(16))) uint32_t gemv_lds[];
-  const int K = w.K;
+  /* FK: the row length the launcher has seen, where it is one of the usual ones (0: any). With the length a
+   * constant every load of the row and of the weights is issued unconditionally, and the waits can count them:
+   * a load behind a condition makes every wait in front of it a wait for nearly all loads in flight. */
+  const int K = FK ? FK : w.K;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
   uint8_t *ap = (uint8_t *)gemv_lds;
   uint32_t *lds = gemv_lds + fused_act_bytes<DT>(K) / 4 + wave * GemvLds<DT, 1, G, false>::DWORDS;
@@ -109,20 +114,19 @@ __device__ __forceinline__ void gemv_fused_rows(const WView (&wv)[NW], const flo
 #pragma unroll
     for (int p = 0; p < XP; ++p) xs[p] = *(const float4 *)(x + min(wave + WV * p, nsb - 1) * 256 + lane * 4);
   }
-  /* late (uniform) 1: the weights are asked for behind the row's quantization instead of in front of it; 2: the
-   * first half of the wavefront's rows in front, the other half behind.
-   * A wavefront's weight loads fill the CU's queue of outstanding requests, and a wavefront that is still
-   * issuing them has not begun to quantize its share of the row, for which the whole workgroup waits at
-   * the barrier: from 16 M weights on the quantization first is faster (us a call, Q4_K 14336 x 4096
-   * 10.9 -> 9.7, 12288 x 4096 in the twelve-wavefront form 9.2 -> 8.65, Q4_0 4096 x 4096 7.14 -> 6.78, Q6_K
-   * 4096 x 4096 7.0 -> 6.4); a matrix of a few MB is served from one round of loads either way, and there
-   * the overlap of the two latencies is worth as much (2048 x 2048 4.12 against 4.16-4.37). */
+  /* LATE 0: the weights are asked for in front of the row's quantization; 1: behind it; 2: the first half of
+   * the wavefront's rows in front, the other half behind. A template parameter: chosen at run time, the
+   * places' loads end in different registers that are copied where the paths meet, which waits for every
+   * load in front of the barrier; this way they stay in flight across it and each pass of the arithmetic
+   * waits for its own. Which is fastest depends on the row length and the size (fused_weights_late): the
+   * row's quantization wants its own loads back first and the weights' requests out early, and a wavefront
+   * that issues sixteen loads in front of it is late for the barrier the workgroup waits at. */
   typename E::Wts W[NW];
-  constexpr int HP = E::NP / 2; /* late == 2: the first half of a wavefront's passes in front, the rest behind */
-  if (!late) {
+  constexpr int HP = E::NP / 2; /* LATE == 2: the first half of a wavefront's passes in front, the rest behind */
+  if constexpr (LATE == 0) {
 #pragma unroll
     for (int i = 0; i < NW; ++i) E::load_w(W[i], wv[i], row0, 0, K);
-  } else if (late == 2) {
+  } else if constexpr (LATE == 2) {
 #pragma unroll
     for (int i = 0; i < NW; ++i) E::template load_w<0, HP>(W[i], wv[i], row0, 0, K);
   }
@@ -170,10 +174,10 @@ __device__ __forceinline__ void gemv_fused_rows(const WView (&wv)[NW], const flo
                                                                              nullptr, nullptr, ql, qh);
     }
   }
-  if (late == 1) {
+  if constexpr (LATE == 1) {
 #pragma unroll
     for (int i = 0; i < NW; ++i) E::load_w(W[i], wv[i], row0, 0, K);
-  } else if (late == 2) {
+  } else if constexpr (LATE == 2) {
 #pragma unroll
     for (int i = 0; i < NW; ++i) E::template load_w<HP, E::NP>(W[i], wv[i], row0, 0, K);
   }
@@ -195,11 +199,11 @@ __device__ __forceinline__ void gemv_fused_rows(const WView (&wv)[NW], const flo
   if (o[0].valid && row0 + o[0].g < w.N) store(row0 + o[0].g, o);
 }
 
-template <int DT, int T, int G>
+template <int DT, int T, int G, int LATE, int FK>
 __device__ __forceinline__ void gemv_fused_body(const WView &w, const float *__restrict__ x,
-                                                float *__restrict__ C, int block, int late = 0) {
+                                                float *__restrict__ C, int block) {
   const WView wv[1] = {w};
-  gemv_fused_rows<DT, T, G, 1>(wv, x, block, [&](int row, const GemvOut(&o)[1]) { C[row] = o[0].v; }, late);
+  gemv_fused_rows<DT, T, G, 1, LATE, FK>(wv, x, block, [&](int row, const GemvOut(&o)[1]) { C[row] = o[0].v; });
 }
 
 /* out[n] = silu(x . Wact[n]) * (x . Wmul[n]): the two projections of a gated MLP and the
@@ -209,33 +213,30 @@ __device__ __forceinline__ void gemv_fused_body(const WView &w, const float *__r
  * (X = (Y / (1 + exp(-Y))) * Z in fp32, fallback_internal.cpp:417-423), applied by
  * SwiGLULayer::incremental_forwarding to the outputs of ffn_up (Y) and ffn_gate (Z)
  * (Applications/CausalLM/layers/swiglu.cpp:40-62, causal_lm.cpp:690-695). */
-template <int DT, int T, int G>
+template <int DT, int T, int G, int LATE, int FK>
 __global__ __launch_bounds__(256) void gemv_fused_swiglu_kernel(WView wact, WView wmul,
                                                                 const float *__restrict__ x,
-                                                                float *__restrict__ out, int late) {
+                                                                float *__restrict__ out) {
   const WView wv[2] = {wact, wmul};
-  gemv_fused_rows<DT, T, G, 2>(
-    wv, x, (int)blockIdx.x,
-    [&](int row, const GemvOut(&o)[2]) {
-      const float y = o[0].v, z = o[1].v;
-      out[row] = (y / (1.f + expf(-y))) * z;
-    },
-    late);
+  gemv_fused_rows<DT, T, G, 2, LATE, FK>(wv, x, (int)blockIdx.x, [&](int row, const GemvOut(&o)[2]) {
+    const float y = o[0].v, z = o[1].v;
+    out[row] = (y / (1.f + expf(-y))) * z;
+  });
 }
 
-template <int DT, int T, int G>
+template <int DT, int T, int G, int LATE, int FK>
 __global__ __launch_bounds__(256) void gemv_fused_kernel(WView w, const float *__restrict__ x,
-                                                         float *__restrict__ C, int late) {
-  gemv_fused_body<DT, T, G>(w, x, C, (int)blockIdx.x, late);
+                                                         float *__restrict__ C) {
+  gemv_fused_body<DT, T, G, LATE, FK>(w, x, C, (int)blockIdx.x);
 }
 /* The same with WV wavefronts a workgroup: one workgroup a CU quantizes the row once where three of four
  * wavefronts each would quantize it three times (see launch_fused for where that pays). */
-template <int DT, int T, int G, int WV>
+template <int DT, int T, int G, int WV, int LATE, int FK>
 __global__ __launch_bounds__(64 * WV) void gemv_fused_wide_kernel(WView w, const float *__restrict__ x,
-                                                                  float *__restrict__ C, int late) {
+                                                                  float *__restrict__ C) {
   const WView wv[1] = {w};
-  gemv_fused_rows<DT, T, G, 1, WV>(
-    wv, x, (int)blockIdx.x, [&](int row, const GemvOut(&o)[1]) { C[row] = o[0].v; }, late);
+  gemv_fused_rows<DT, T, G, 1, LATE, FK, WV>(wv, x, (int)blockIdx.x,
+                                         [&](int row, const GemvOut(&o)[1]) { C[row] = o[0].v; });
 }
 
 /* Up to four weights of one format and K on the same row, one launch: the
@@ -246,31 +247,52 @@ struct FusedMulti {
   float *C[FUSED_MAXW];
   int end[FUSED_MAXW];
 };
-template <int DT, int T, int G>
-__global__ __launch_bounds__(256) void gemv_fused_multi_kernel(FusedMulti mw, const float *__restrict__ x, int late) {
+template <int DT, int T, int G, int LATE, int FK>
+__global__ __launch_bounds__(256) void gemv_fused_multi_kernel(FusedMulti mw, const float *__restrict__ x) {
   const int b = (int)blockIdx.x;
   int i = 0;
 #pragma unroll
   for (int k = 0; k + 1 < FUSED_MAXW; ++k) i += b >= mw.end[k];
   const int first = i ? mw.end[i - 1] : 0;
-  gemv_fused_body<DT, T, G>(mw.w[i], x, mw.C[i], b - first, late);
+  gemv_fused_body<DT, T, G, LATE, FK>(mw.w[i], x, mw.C[i], b - first);
 }
 
-/* Where a wavefront asks for its weights (gemv_fused_rows' `late`): in front of the row's quantization below
- * 16 M weights, behind it above; and with rows of 4096 the first half in front and the rest behind where that
- * measured faster (us a call, behind -> half and half: Q4_K in the twelve-wavefront form 10240 x 4096 8.8 -> 8.45,
- * 12288 x 4096 9.35 -> 8.8, but 12288 x 2048 5.8 -> 6.05; four wavefronts, 13312 .. 16384 x 4096 the same within
- * 0.2, 20480 14.3 -> 13.5, 24576 15.6 -> 14.8, 28672 16.9 -> 16.6; Q4_0 8192 x 4096 9.0 -> 8.9, 12288 10.7 -> 9.95;
- * Q6_K 4096 x 4096 6.8 -> 6.65, 8192 9.65 -> 8.7, 12288 the same, 16384 13.8 -> 14.0). */
-static inline int fused_weights_late(const hipq_weight *w, bool wide = false) {
-  if (w->N * w->K < ((int64_t)1 << 24)) return 0;
-  if (w->K < 4096) return 1;
-  if (w->dtype == HIPQ_Q4_K) return wide || w->N >= 20480 ? 2 : 1;
-  if (w->dtype == HIPQ_Q4_0) return w->N >= 8192 ? 2 : 1;
-  return w->N <= 8192 ? 2 : 1;
+/* Where a wavefront asks for its weights (gemv_fused_rows' LATE), by the row length and the weights of the
+ * launch (all its matrices together). Measured with the usual row lengths as constants (us a call, in front /
+ * behind / half and half): Q4_K 2048 x 4096 4.35 / 4.57 / 4.3, 4096 x 4096 5.35 / 5.25 / 5.2, 12288 x 4096
+ * 8.1 / 8.1 / 7.65, 14336 x 4096 9.95 / 9.15 / 8.8, 24576 x 4096 13.3 / 13.7 / 12.65, 8192 x 3072 7.2 / 6.45 / 6.25,
+ * 12288 x 2048 5.15 / 4.35 / 4.7, 16384 x 2048 6.65 / 5.65 / 6.3, 4096 x 2048 4.2 / 4.1 / 4.25; Q6_K 4096 x 4096
+ * 5.75 / 5.85 / 5.0, 8192 x 4096 8.3 / 7.9 / 7.6; Q4_0 12288 x 4096 9.7 / 10.0 / 9.4, the C5 shapes (1024 .. 3072
+ * rows of 1024 .. 3072) the same within 0.1 (in front 4.0-4.6); gate and up with the SwiGLU 11008 x 4096 13.9 /
+ * 14.2 / 13.1, 8192 x 2048 7.45 / 6.4 / 6.9; Q, K, V of 4096 + 1024 + 1024 x 4096 6.7 / 6.5 / 6.3. */
+static inline int fused_weights_late(int64_t K, int64_t weights) {
+  if (K == 4096) return 2;
+  if (weights < ((int64_t)1 << 24)) return 0;
+  return K >= 3072 ? 2 : 1;
 }
-/* the same for launches of several matrices on one row (their weights counted together) */
-static inline int fused_weights_late(int64_t weights) { return weights >= ((int64_t)1 << 24) ? 1 : 0; }
+
+/* f(LATE, FK) with the two as compile-time constants. Rows of 16 lanes a row (under 2048 weights) have one
+ * pass of weight rows a wavefront: no half and half. */
+template <int T, typename F> void with_late(int late, int64_t K, F f) {
+  auto go = [&](auto L) {
+    if (T == 64 && K == 4096)
+      f(L, std::integral_constant<int, T == 64 ? 4096 : 0>{});
+    else if (T == 64 && K == 3072)
+      f(L, std::integral_constant<int, T == 64 ? 3072 : 0>{});
+    else if (T == 64 && K == 2048)
+      f(L, std::integral_constant<int, T == 64 ? 2048 : 0>{});
+    else if (T == 16 && K == 1024)
+      f(L, std::integral_constant<int, T == 16 ? 1024 : 0>{});
+    else
+      f(L, std::integral_constant<int, 0>{});
+  };
+  if (late == 2 && T == 64)
+    go(std::integral_constant<int, T == 64 ? 2 : 1>{});
+  else if (late)
+    go(std::integral_constant<int, 1>{});
+  else
+    go(std::integral_constant<int, 0>{});
+}
 
 template <int DT, int T, int G>
 int launch_fused_many(int count, const hipq_weight *const *w, const float *x, float *const *C, hipStream_t s) {
@@ -285,20 +307,22 @@ int launch_fused_many(int count, const hipq_weight *const *w, const float *x, fl
     mw.end[i] = blocks;
   }
   const size_t lds = fused_act_bytes<DT>((int)w[0]->K) + 4 * GemvLds<DT, 1, G, false>::DWORDS * sizeof(uint32_t);
-  hipq::launch_kernel("gemv_fused_multi_kernel<DT, T, G>", (gemv_fused_multi_kernel<DT, T, G>), dim3((unsigned)blocks), dim3(256), lds, s, mw, x,
-                      fused_weights_late(weights));
+  with_late<T>(fused_weights_late(w[0]->K, weights), w[0]->K, [&](auto L, auto FK) {
+    hipq::launch_kernel("gemv_fused_multi_kernel<DT, T, G, LATE, FK>", (gemv_fused_multi_kernel<DT, T, G, decltype(L)::value, decltype(FK)::value>),
+                        dim3((unsigned)blocks), dim3(256), lds, s, mw, x);
+  });
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
 }
-
-/* whether a fused launch asks for its weights behind the row's quantization (gemv_fused_rows) */
 
 template <int DT, int T, int G, int WV>
 int launch_fused_wide(const hipq_weight *w, const float *x, float *C, hipStream_t s) {
   const unsigned grid = (unsigned)((w->N + WV * G - 1) / (WV * G));
   const size_t lds = fused_act_bytes<DT>((int)w->K) + WV * GemvLds<DT, 1, G, false>::DWORDS * sizeof(uint32_t);
-  hipq::launch_kernel("gemv_fused_wide_kernel<DT, T, G, WV>", (gemv_fused_wide_kernel<DT, T, G, WV>), dim3(grid), dim3(64 * WV), lds, s, wview(w), x, C,
-                      fused_weights_late(w, true));
+  with_late<T>(fused_weights_late(w->K, w->N * w->K), w->K, [&](auto L, auto FK) {
+    hipq::launch_kernel("gemv_fused_wide_kernel<DT, T, G, WV, LATE, FK>", (gemv_fused_wide_kernel<DT, T, G, WV, decltype(L)::value, decltype(FK)::value>),
+                        dim3(grid), dim3(64 * WV), lds, s, wview(w), x, C);
+  });
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
 }
@@ -307,8 +331,11 @@ template <int DT, int T, int G>
 int launch_fused_one(const hipq_weight *w, const float *x, float *C, hipStream_t s) {
   const unsigned grid = (unsigned)((w->N + 4 * G - 1) / (4 * G));
   const size_t lds = fused_act_bytes<DT>((int)w->K) + 4 * GemvLds<DT, 1, G, false>::DWORDS * sizeof(uint32_t);
-  hipq::launch_kernel("gemv_fused_kernel<DT, T, G>", (gemv_fused_kernel<DT, T, G>), dim3(grid), dim3(256), lds, s, wview(w), x, C,
-                      fused_weights_late(w));
+  with_late<T>(fused_weights_late(w->K, w->N * w->K), w->K, [&](auto L, auto FK) {
+    constexpr int LATE = decltype(L)::value == 2 && G < 2 ? 0 : decltype(L)::value; /* half and half takes two passes */
+    hipq::launch_kernel("gemv_fused_kernel<DT, T, G, LATE, FK>", (gemv_fused_kernel<DT, T, G, LATE, decltype(FK)::value>), dim3(grid),
+                        dim3(256), lds, s, wview(w), x, C);
+  });
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
 }
@@ -348,8 +375,10 @@ int launch_fused_swiglu_one(const hipq_weight *wa, const hipq_weight *wm, const 
                             hipStream_t s) {
   const unsigned grid = (unsigned)((wa->N + 4 * G - 1) / (4 * G));
   const size_t lds = fused_act_bytes<DT>((int)wa->K) + 4 * GemvLds<DT, 1, G, false>::DWORDS * sizeof(uint32_t);
-  hipq::launch_kernel("gemv_fused_swiglu_kernel<DT, T, G>", (gemv_fused_swiglu_kernel<DT, T, G>), dim3(grid), dim3(256), lds, s, wview(wa), wview(wm), x,
-                     out, fused_weights_late(2 * wa->N * wa->K));
+  with_late<T>(fused_weights_late(wa->K, 2 * wa->N * wa->K), wa->K, [&](auto L, auto FK) {
+    hipq::launch_kernel("gemv_fused_swiglu_kernel<DT, T, G, LATE, FK>", (gemv_fused_swiglu_kernel<DT, T, G, decltype(L)::value, decltype(FK)::value>),
+                        dim3(grid), dim3(256), lds, s, wview(wa), wview(wm), x, out);
+  });
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
 }
