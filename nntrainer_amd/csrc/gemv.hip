@@ -43,7 +43,7 @@ __global__ __launch_bounds__(256) void gemv_kernel(WView w, QView qa, int M, int
  * group are in flight while the current one is computed, so the HBM stream of a
  * wavefront never drains. T lanes a row (64, or 16 for rows of fewer than 64 units). One chunk only
  * (K <= 4096). */
-template <int DT, int T, int G, int GPW>
+template <int DT, int T, int G, int GPW, int FK>
 __global__ __launch_bounds__(256) void gemv_stream_kernel(WView w, QView qa,
                                                           float *__restrict__ C) {
   typedef GemvCore<DT, T, 1, G, false> E;
@@ -52,17 +52,25 @@ __global__ __launch_bounds__(256) void gemv_stream_kernel(WView w, QView qa,
   uint32_t *lds = gemv_lds + wave * GemvLds<DT, 1, G, false>::DWORDS;
   const int first = (blockIdx.x * 4 + wave) * GPW * G;
   if (first >= w.N) return; /* uniform per wavefront; all syncs below are wavefront-local */
-  const int K = w.K;
+  /* FK: the row length where the launcher has seen one of the usual ones (0: any). With it a constant, and the
+   * next group's loads issued whether or not the matrix still has those rows (a row past the end is read as
+   * the last one), no load sits behind a condition and the waits of a group's arithmetic leave the next
+   * group's loads in flight; behind a condition they were waited for with everything else. */
+  const int K = FK ? FK : w.K;
   const int arow[1] = {0};
   typename E::Wts W[2];
-  E::load_w(W[0], w, first, 0, K); /* before the activations, whose loads are followed by arithmetic */
   typename E::Act A;
+  /* the activations' loads first and nothing moved across: a load that the arithmetic needs and that is
+   * issued behind the weights' has to wait for all of them */
   E::load_act(A, qa, arow, 0, K);
+  __builtin_amdgcn_sched_barrier(0);
+  E::load_w(W[0], w, first, 0, K);
 #pragma unroll
   for (int i = 0; i < GPW; ++i) {
     const int row0 = first + i * G;
     if (row0 >= w.N) break; /* uniform */
-    if (i + 1 < GPW && row0 + G < w.N) E::load_w(W[(i + 1) & 1], w, row0 + G, 0, K);
+    if (i + 1 < GPW) E::load_w(W[(i + 1) & 1], w, row0 + G, 0, K);
+    __builtin_amdgcn_sched_barrier(0);
     typename E::Chain c = E::begin(arow, 0);
     E::compute(W[i & 1], A, K, lds);
     hipq_wave_lds_sync();
@@ -345,8 +353,13 @@ int launch_stream(const hipq_weight *w, const QAct *qa, float *C, hipStream_t s)
   const int rows_per_block = 4 * G * GPW;
   const unsigned grid = (unsigned)((w->N + rows_per_block - 1) / rows_per_block);
   const size_t lds = 4 * GemvLds<DT, 1, G, false>::DWORDS * sizeof(uint32_t);
-  hipq::launch_kernel("gemv_stream_kernel<DT, T, G, GPW>", (gemv_stream_kernel<DT, T, G, GPW>), dim3(grid), dim3(256), lds, s, wview(w),
-                     qview(*qa), C);
+  constexpr int USUAL = T == 64 ? 4096 : 1024; /* the row length that has an instance of its own */
+  if (w->K == USUAL)
+    hipq::launch_kernel("gemv_stream_kernel<DT, T, G, GPW, K>", (gemv_stream_kernel<DT, T, G, GPW, USUAL>), dim3(grid), dim3(256),
+                        lds, s, wview(w), qview(*qa), C);
+  else
+    hipq::launch_kernel("gemv_stream_kernel<DT, T, G, GPW, 0>", (gemv_stream_kernel<DT, T, G, GPW, 0>), dim3(grid), dim3(256), lds,
+                        s, wview(w), qview(*qa), C);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
 }
