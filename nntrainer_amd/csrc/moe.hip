@@ -231,19 +231,19 @@ __device__ __forceinline__ void route_token_regs(const float *__restrict__ logit
   float p[MAXV];
   const float *lg = logits + (size_t)t * E;
   float mx = -INFINITY;
-  /* the guards on 64 * i are uniform: rounds past E cost nothing (the double
-   * exponential is a few hundred instructions) */
+  /* every lane's loads at once and unconditionally (a lane without an expert reads the last one's): behind
+   * a condition each load is a round trip of its own */
+#pragma unroll
+  for (int i = 0; i < MAXV; ++i) p[i] = lg[min(lane + 64 * i, E - 1)];
 #pragma unroll
   for (int i = 0; i < MAXV; ++i) {
-    p[i] = -INFINITY;
-    if (64 * i < E) {
-      const int e = lane + 64 * i;
-      if (e < E) p[i] = lg[e];
-      mx = fmaxf(mx, p[i]);
-    }
+    if (lane + 64 * i >= E) p[i] = -INFINITY;
+    if (64 * i < E) mx = fmaxf(mx, p[i]);
   }
   mx = hipq_wave_max(mx);
   float sum = 0.f;
+  /* the guards on 64 * i are uniform: rounds past E cost nothing (the double exponential is a few hundred
+   * instructions) */
 #pragma unroll
   for (int i = 0; i < MAXV; ++i) {
     if (64 * i < E) {
@@ -319,11 +319,11 @@ __device__ __forceinline__ bool topk_set_fast(const float *__restrict__ lg, int 
   float mx = -INFINITY;
   bool nan = false;
 #pragma unroll
+  for (int i = 0; i < MAXV; ++i) v[i] = lg[min(lane + 64 * i, E - 1)]; /* all loads at once, see route_token_regs */
+#pragma unroll
   for (int i = 0; i < MAXV; ++i) {
-    v[i] = -INFINITY;
+    if (lane + 64 * i >= E) v[i] = -INFINITY;
     if (64 * i < E) {
-      const int e = lane + 64 * i;
-      if (e < E) v[i] = lg[e];
       nan |= !(v[i] == v[i]);
       mx = fmaxf(mx, v[i]);
     }
