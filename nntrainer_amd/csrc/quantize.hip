@@ -90,10 +90,15 @@ __global__ __launch_bounds__(256) void quantize_q8_K_tiled_kernel(
   const int b = (int)(unit - mq * nsb);
   const int64_t m = mq * 4 + (lane >> 4);
   float x[4][4];
+  /* the four loads at once and unconditionally (a row past M reads the last one and is zeroed after): behind a
+   * condition they went out two at a time, each pair a round trip of its own */
+  const float *src = A + (m < M ? m : M - 1) * lda + (int64_t)b * 256 + 4 * l16;
+  float4 v4[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) v4[i] = *(const float4 *)(src + 64 * i);
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-    if (m < M) v = *(const float4 *)(A + m * lda + (int64_t)b * 256 + 64 * i + 4 * l16);
+    const float4 v = m < M ? v4[i] : make_float4(0.f, 0.f, 0.f, 0.f);
     x[i][0] = v.x, x[i][1] = v.y, x[i][2] = v.z, x[i][3] = v.w;
   }
   float amax = 0.f;
