@@ -1227,8 +1227,11 @@ __global__ __launch_bounds__(256, 4) void gate_up_one_token_kernel(
     r.hd = __builtin_bit_cast(
       mv4i, __builtin_amdgcn_raw_buffer_load_b128(rq, 4096 + i32 * 16, sb * hipq::EXPERT_TILE_BYTES, 2));
   };
+  /* Every step issues its loads whether or not a super-block is left: past the wavefront's last one the loads
+   * name the descriptor's end and return zeros without touching memory. Behind a condition the waits could
+   * not count them, and every super-block's arithmetic waited for the loads just issued for the next. */
   XRegs buf[2];
-  if (cnt > 0) load(buf[0], sb0);
+  load(buf[0], cnt > 0 ? sb0 : nsb);
   stage(); /* the row of x is quantized while the first weights are on their way */
   float acc = 0.f, accm = 0.f;
   for (int u0 = 0; u0 < cnt; u0 += 2) {
@@ -1236,7 +1239,7 @@ __global__ __launch_bounds__(256, 4) void gate_up_one_token_kernel(
     for (int k = 0; k < 2; ++k) {
       const int u = u0 + k;
       if (u < cnt) { /* uniform per wavefront */
-        if (u + 1 < cnt) load(buf[(k + 1) & 1], sb0 + u + 1);
+        load(buf[(k + 1) & 1], u + 1 < cnt ? sb0 + u + 1 : nsb);
         float fi[NREG], si[NREG], fm[NREG], sm[NREG];
         xr_sb_terms<TC, NREG>(buf[k], l, K, sb0 + u, i32, g, fi, si, fm, sm);
         if (half == 0) {
