@@ -24,7 +24,7 @@
 
 namespace {
 
-template <int DT, int T, int R, int G, bool PW>
+template <int DT, int T, int R, int G, bool PW, int FK>
 __global__ __launch_bounds__(256) void gemv_kernel(WView w, QView qa, int M, int pair_rows,
                                                    float *__restrict__ C, int64_t ldc) {
   extern __shared__ uint32_t gemv_lds[];
@@ -34,7 +34,7 @@ __global__ __launch_bounds__(256) void gemv_kernel(WView w, QView qa, int M, int
   int arow[R];
 #pragma unroll
   for (int r = 0; r < R; ++r) arow[r] = r < M ? r : M - 1;
-  const GemvOut o = gemv_engine<DT, T, R, G, PW>(w, row0, qa, arow, pair_rows, lds);
+  const GemvOut o = gemv_engine<DT, T, R, G, PW, HIPQ_KCHUNK, FK>(w, row0, qa, arow, pair_rows, lds);
   if (o.valid && row0 + o.g < w.N && o.r < M) C[(int64_t)o.r * ldc + row0 + o.g] = o.v;
 }
 
@@ -369,8 +369,13 @@ int launch_one(const hipq_weight *w, const QAct *qa, int M, int pair_rows, float
                hipStream_t s) {
   const unsigned grid = (unsigned)((w->N + 4 * G - 1) / (4 * G));
   const size_t lds = 4 * GemvLds<DT, R, G, PW>::DWORDS * sizeof(uint32_t);
-  hipq::launch_kernel("gemv_kernel<DT, T, R, G, PW>", (gemv_kernel<DT, T, R, G, PW>), dim3(grid), dim3(256), lds, s, wview(w),
-                     qview(*qa), M, pair_rows, C, ldc);
+  constexpr int USUAL = T == 64 ? 4096 : 1024; /* the row length that has an instance of its own */
+  if (w->K == USUAL)
+    hipq::launch_kernel("gemv_kernel<DT, T, R, G, PW, K>", (gemv_kernel<DT, T, R, G, PW, USUAL>), dim3(grid), dim3(256), lds, s,
+                        wview(w), qview(*qa), M, pair_rows, C, ldc);
+  else
+    hipq::launch_kernel("gemv_kernel<DT, T, R, G, PW, 0>", (gemv_kernel<DT, T, R, G, PW, 0>), dim3(grid), dim3(256), lds, s,
+                        wview(w), qview(*qa), M, pair_rows, C, ldc);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
 }

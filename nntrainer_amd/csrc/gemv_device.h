@@ -595,12 +595,28 @@ template <int DT, int T, int R, int G, bool PW, int KC = HIPQ_KCHUNK> struct Gem
   }
 };
 
-template <int DT, int T, int R, int G, bool PW, int KC = HIPQ_KCHUNK>
+template <int DT, int T, int R, int G, bool PW, int KC = HIPQ_KCHUNK, int FK = 0>
 __device__ __forceinline__ GemvOut gemv_engine(const WView &w, int row0, const QView &qa,
                                                const int (&arow)[R], int pair_rows,
                                                uint32_t *lds) {
   typedef GemvCore<DT, T, R, G, PW, KC> E;
   typename E::Chain c = E::begin(arow, pair_rows);
+  if constexpr (FK != 0) {
+    /* FK: the row length, where the launcher has seen one of the usual ones (one chunk). With it a constant no
+     * load sits behind a condition and the waits can count them: the activations' loads first, nothing moved
+     * across, then the weights', and each pass over the weight rows waits for its own loads only. */
+    typename E::Act A;
+    E::load_act(A, qa, arow, 0, FK);
+    __builtin_amdgcn_sched_barrier(0);
+    typename E::Wts W;
+    E::load_w(W, w, row0, 0, FK);
+    __builtin_amdgcn_sched_barrier(0);
+    E::compute(W, A, FK, lds);
+    hipq_wave_lds_sync();
+    E::chain(c, FK, lds);
+    hipq_wave_lds_sync();
+    return E::finish(c);
+  }
   auto chunk = [&](int k0, int kc) {
     /* the weights first: the activations' loads are followed by arithmetic on what
      * they return, and in the other order the weight loads would be issued only
