@@ -295,7 +295,7 @@ def main():
     # what the int8 matrix instruction sustains on this device with nothing else issued
     ceiling_tops, ceiling_ghz = capi.bench_mfma_ceiling(2.0, stream=stream)
     # what a kernel that only reads gets out of device memory (1 GiB, the GEMV kernels' access pattern)
-    read_ceiling_gbs = capi.bench_hbm_read_ceiling(1 << 30, 4, stream=stream) * 1e3
+    read_ceiling_gbs = max(capi.bench_hbm_read_ceiling(1 << 30, wps, stream=stream) for wps in (1, 2, 4)) * 1e3
 
     # ---- the same step with operands in host memory (what the Layer API hands over) --------
     # Not `value`: the PCIe-inclusive rate of the whole call, activations in and outputs back
@@ -794,9 +794,10 @@ def main():
                    "kernel_timing_blocks_kernel_ms": [round(b[2], 5) for b in blocks_instr],
                    "consistent": bool(gemm_ms + quant_ms <= step_ms)},
         "hbm_read_ceiling": {"value": round(read_ceiling_gbs, 1), "unit": "GB/s",
-                             "method": "a kernel that only reads 1 GiB of device memory, four wavefronts a SIMD, each "
-                                       "streaming its own consecutive share with eight non-temporal 128-bit loads a "
-                                       "lane in flight; best of three launches"},
+                             "method": "a kernel that only reads 1 GiB of device memory, each wavefront streaming its own "
+                                       "consecutive share with four to eight non-temporal 128-bit loads a lane in "
+                                       "flight (the next four asked for before the last four are used); the best of "
+                                       "one, two and four wavefronts a SIMD, three launches each"},
         "decode_gemv": {"workload": "Q4_K GEMV M=1 K=4096 N=12288, %d weight copies rotated" % n_copies,
                         "value": round(gv_bytes / (gemv_all_ms * 1e-3) / 1e9, 2), "unit": "GB/s",
                         "ms_per_call": round(gemv_all_ms, 5),

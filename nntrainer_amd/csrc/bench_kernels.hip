@@ -46,12 +46,24 @@ __global__ __launch_bounds__(256) void hbm_read_ceiling_kernel(const unsigned ch
   __amdgpu_buffer_rsrc_t r =
     __builtin_amdgcn_make_buffer_rsrc((void *)(p + wave * kb_per_wave * 1024), 0, (int)(kb_per_wave * 1024), 0x00020000);
   u4 acc = {0, 0, 0, 0};
+  /* two halves of DEPTH / 2 loads in turn, the next half asked for before the current one is consumed, so that
+   * the wavefront always has loads in flight; past its share's end the loads name the descriptor's end and
+   * return zeros without touching memory (unconditional, so that the waits can count them) */
+  constexpr int HALF = DEPTH / 2;
+  u4 a[HALF], b[HALF];
+#pragma unroll
+  for (int i = 0; i < HALF; ++i) a[i] = __builtin_amdgcn_raw_buffer_load_b128(r, lane * 16, i * 1024, 2);
   for (long long k = 0; k + DEPTH <= kb_per_wave; k += DEPTH) {
-    u4 v[DEPTH];
 #pragma unroll
-    for (int i = 0; i < DEPTH; ++i) v[i] = __builtin_amdgcn_raw_buffer_load_b128(r, lane * 16, (int)(k + i) * 1024, 2);
+    for (int i = 0; i < HALF; ++i)
+      b[i] = __builtin_amdgcn_raw_buffer_load_b128(r, lane * 16, (int)(k + HALF + i) * 1024, 2);
 #pragma unroll
-    for (int i = 0; i < DEPTH; ++i) acc ^= v[i];
+    for (int i = 0; i < HALF; ++i) acc ^= a[i];
+#pragma unroll
+    for (int i = 0; i < HALF; ++i)
+      a[i] = __builtin_amdgcn_raw_buffer_load_b128(r, lane * 16, (int)(k + DEPTH + i) * 1024, 2);
+#pragma unroll
+    for (int i = 0; i < HALF; ++i) acc ^= b[i];
   }
   const unsigned x = acc[0] ^ acc[1] ^ acc[2] ^ acc[3];
   if (x == 0x12345678u) sink[threadIdx.x] = x; /* keeps the loads alive; the buffer holds zeros */
