@@ -418,9 +418,12 @@ template <int DT>
 int launch_m1(const hipq_weight *w, const QAct *qa, float *C, int64_t ldc, hipStream_t s) {
   const int64_t units = w->K / GemvRec<DT, false>::UNIT;
   /* measured on lm_head-sized matrices (N = 151936): two groups per wavefront with
-   * the next group's loads in flight gain 3 % (Q4_K) to 20 % (Q4_0); Q6_K and
-   * smaller matrices are better off with more, shorter wavefronts */
-  if (DT != HIPQ_Q6_K && w->N >= 32768 && w->K <= HIPQ_KCHUNK && units >= 64)
+   * the next group's loads in flight gain 3 % (Q4_K) to 20 % (Q4_0) over the plain kernel whose loads the
+   * waits cannot count (any row length); Q6_K and smaller matrices are better off with more, shorter
+   * wavefronts, and so are rows of 4096 now that the plain kernel's waits count every load (us a call with
+   * the quantizer's launch, streamed -> plain: Q4_K 32768 x 4096 17.6 -> 16.1, 65536 29.0 -> 26.4, 151936
+   * 57.2 -> 53.9; Q4_0 32768 20.1 -> 17.7, 151936 59.0 -> 57.0) */
+  if (DT != HIPQ_Q6_K && w->N >= 32768 && w->K < HIPQ_KCHUNK && units >= 64)
     return launch_stream<DT, 64, 4, 2>(w, qa, C, s);
   /* the same for short rows (16 lanes a row, four rows side by side, eight a group): a wavefront of
    * the plain kernel below would have four short rows for all its work. Kernel us, plain -> streamed:
