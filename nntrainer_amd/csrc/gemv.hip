@@ -473,7 +473,9 @@ template <int DT> int launch_fused(const hipq_weight *w, const float *x, float *
   case 2:
     return launch_fused_one<DT, 64, 2>(w, x, C, s);
   default:
-    if (DT == HIPQ_Q4_0) return launch_fused_one<DT, 64, 2>(w, x, C, s);
+    /* Q4_0 rows are short work for a wavefront: two of them, unless that leaves CUs without a workgroup (1024 rows
+     * of 3072: 4.6 -> 4.4 us a call, of 4096: 5.5 -> 5.1; 1536 rows of 3072: 4.6 against 4.8) */
+    if (DT == HIPQ_Q4_0 && w->N > 1024) return launch_fused_one<DT, 64, 2>(w, x, C, s);
     return launch_fused_one<DT, 64, 1>(w, x, C, s);
   }
 }
