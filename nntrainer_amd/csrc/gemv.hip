@@ -458,13 +458,24 @@ template <int DT> int launch_fused(const hipq_weight *w, const float *x, float *
     return launch_fused_one<DT, 16, 4>(w, x, C, s);
   }
   if constexpr (DT == HIPQ_Q4_K) {
-    /* Four rows a wavefront and at most one workgroup of twelve wavefronts a CU (256 of them): the row is
-     * quantized once a CU instead of three times. Measured, us a call, four -> twelve wavefronts:
-     * 10240 x 4096 9.3 -> 8.5, 11008 x 4096 9.5 -> 8.8, 12288 x 4096 9.7 -> 9.2, 12288 x 2048 6.1 -> 5.6; with
-     * more rows than one round of such workgroups it loses (14336 x 4096 11.0 -> 13.5), and Q6_K loses
-     * everywhere (12288 x 4096 11.8 -> 12.1). */
+    /* Workgroups of twelve wavefronts quantize the row once where three of four wavefronts each would
+     * quantize it three times. With rows of 4096 and every load counted by the waits, two rows a wavefront
+     * (24 a workgroup) are the fastest form wherever the workgroups fill the CUs' rounds evenly (us a call,
+     * four wavefronts of four rows / twelve of four / twelve of two: 3072 rows 4.6 / 6.1 / 4.5, 5120 5.85 / 6.4 /
+     * 4.75, 6144 5.8 / 6.4 / 4.9, 11008 7.6 / 7.5 / 7.05, 12288 7.35 / 7.65 / 7.1, 18432 10.65 / 11.8 / 9.35, 24576
+     * 12.6 / 12.7 / 11.5), and four wavefronts of four rows where the last round would be short (7168 5.95 / 6.55 /
+     * 6.75, 8192 5.9 / 6.65 / 6.9, 20480 10.9 / 11.85 / 11.35). Other row lengths keep the form measured for them
+     * (twelve wavefronts of four rows up to one round: 12288 x 2048 6.1 -> 5.6 when it was introduced). */
+    if (w->K == HIPQ_KCHUNK && w->N >= 2048) {
+      const int64_t wgs = (w->N + 23) / 24, rest = wgs % 256;
+      if (wgs <= 256 || rest == 0 || rest >= 128) return launch_fused_wide<DT, 64, 2, 12>(w, x, C, s);
+      return launch_fused_one<DT, 64, 4>(w, x, C, s);
+    }
     if (pick_group(w->N, 8) == 4 && (w->N + 47) / 48 <= 256) return launch_fused_wide<DT, 64, 4, 12>(w, x, C, s);
   }
+  /* Q4_0 with rows of 4096: four rows a wavefront from 4096 rows on (4096 x 4096 6.65 -> 6.25 us a call, 6144 x 4096
+   * 7.65 -> 7.3) */
+  if (DT == HIPQ_Q4_0 && w->K == HIPQ_KCHUNK && w->N >= 4096) return launch_fused_one<DT, 64, 4>(w, x, C, s);
   switch (pick_group(w->N, 8)) {
   case 8:
     return launch_fused_one<DT, 64, 8>(w, x, C, s);
