@@ -39,6 +39,28 @@ def test_gemv_matches_oracle(hipq, cr, kind, n, k):
 
 
 @pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("n,k", [(6150, 4096), (8200, 4096), (12290, 4096), (2050, 3072), (1024, 3072),
+                                 (3000, 2304), (2100, 2560), (9000, 2048), (33000, 4096), (33000, 2048),
+                                 (1000, 1024), (40000, 1024)])
+def test_single_row_against_the_instances_by_row_length(hipq, cr, kind, n, k):
+    """One row against shapes chosen by what the library picks for them: the kernels with the row length as
+    a constant (1024, 2048, 3072, 4096) and the ones that take any length (2304, 2560),
+    workgroups of twelve wavefronts whose last one hangs over the matrix's end (6150, 12290), four wavefronts
+    of four rows (8200), the plain and the streamed kernel behind the quantizer's launch (33000 and 40000
+    columns). Same bits as the reference's row product."""
+    import gpu_util as gu
+    blocks = _weights(cr, kind, n, k, seed=900 + n % 97)
+    a = synth.normal(950 + k % 89, (1, k))
+    ref = cr.gemm(cr.oracle(), kind, a, blocks, n)
+    w = capi.Weight(kind, n, k, blocks)
+    got = gu.gpu_matmul(w, a)
+    w.destroy()
+    assert not np.isnan(got).any()
+    assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), \
+        "%d of %d outputs differ in bits" % ((got.view(np.uint32) != ref.view(np.uint32)).sum(), got.size)
+
+
+@pytest.mark.parametrize("kind", KINDS)
 @pytest.mark.parametrize("m", [2, 3, 4, 5, 7, 8])
 def test_small_m_matches_oracle(hipq, cr, kind, m):
     """M = 2..8 runs the multi-row GEMV; rows below 4*(M/4) of a Q4_K matmul must be
