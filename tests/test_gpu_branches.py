@@ -219,7 +219,11 @@ def test_mlp_swiglu_down_is_the_two_calls_and_matches_the_oracle(hipq, cr, kind,
 
 @pytest.mark.parametrize("kind,m,k,n", [("q4_0", 1, 1024, 3072), ("q4_K", 1, 2048, 768), ("q6_K", 1, 1024, 512),
                                         ("q4_0", 1, 96, 320),      # K below one chunk unit: not fused
-                                        ("q4_0", 24, 1024, 3072), ("q4_K", 5, 1024, 512)])
+                                        ("q4_0", 24, 1024, 3072), ("q4_K", 5, 1024, 512),
+                                        # one row, the row length a constant of the launch (4096, 3072) or not (2304),
+                                        # the weights asked for in front of, behind and around the row's quantization
+                                        ("q4_K", 1, 4096, 2200), ("q4_K", 1, 3072, 3000), ("q6_K", 1, 4096, 1100),
+                                        ("q4_0", 1, 4096, 2100), ("q4_K", 1, 2304, 1000), ("q4_K", 1, 2048, 4100)])
 @pytest.mark.parametrize("mem", ["device", "host"])
 def test_mlp_swiglu_matches_oracle(hipq, cr, kind, m, k, n, mem):
     """hipq_mlp_swiglu: out = swiglu(a . Wact^T, a . Wmul^T) (swiglu.cpp:40-62 on the outputs of

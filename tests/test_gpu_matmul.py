@@ -566,6 +566,29 @@ def test_matmul_multi_few_rows_mixed_paths(hipq, cr, m):
         w.destroy()
 
 
+@pytest.mark.parametrize("kind", KINDS)
+@pytest.mark.parametrize("k", [4096, 3072, 2304, 1024])
+def test_matmul_multi_one_row_one_launch_by_row_length(hipq, cr, kind, k):
+    """One row against the Q, K, V of a layer (one launch that quantizes the row itself): the launch with the
+    row length as a constant (4096, 3072, 1024) and for any length (2304), widths that end inside a
+    wavefront's group of rows. Every output carries the reference's bits."""
+    import gpu_util as gu
+    import torch
+    ns = [4100, 1024, 1030] if k >= 3072 else [2050, 520, 512]
+    blocks = [_weights(cr, kind, n, k, seed=1450 + i) for i, n in enumerate(ns)]
+    ws = [capi.Weight(kind, n, k, b) for n, b in zip(ns, blocks)]
+    a = synth.normal(1460 + k % 13, (1, k))
+    outs = [torch.full((1, n), float("nan"), device="cuda") for n in ns]
+    capi.matmul_multi(ws, gu.dev(a), 1, outs, stream=gu.stream())
+    torch.cuda.synchronize()
+    for n, b, o in zip(ns, blocks, outs):
+        got = o.cpu().numpy()
+        ref = cr.gemm(cr.oracle(), kind, a, b, n)
+        assert np.array_equal(got.view(np.uint32), ref.view(np.uint32)), (n, gu.rel_err(got, ref))
+    for w in ws:
+        w.destroy()
+
+
 @pytest.mark.parametrize("m,k", [(2, 1024), (8, 1280), (13, 256), (16, 2048), (40, 1024), (64, 512)])
 def test_matmul_multi_q4_0_few_rows_one_launch(hipq, cr, m, k):
     """A few rows against several Q4_0 weights of one K (Q, K, V or gate, up of a decode step of a
