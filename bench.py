@@ -292,10 +292,6 @@ def main():
     ops = 2.0 * M * N * K
     value = ops / sec / 1e12
     gemm_tops = ops / (gemm_ms * 1e-3) / 1e12
-    # what the int8 matrix instruction sustains on this device with nothing else issued
-    ceiling_tops, ceiling_ghz = capi.bench_mfma_ceiling(2.0, stream=stream)
-    # what a kernel that only reads gets out of device memory (1 GiB, the GEMV kernels' access pattern)
-    read_ceiling_gbs = max(capi.bench_hbm_read_ceiling(1 << 30, wps, stream=stream) for wps in (1, 2, 4)) * 1e3
 
     # ---- the same step with operands in host memory (what the Layer API hands over) --------
     # Not `value`: the PCIe-inclusive rate of the whole call, activations in and outputs back
@@ -755,6 +751,14 @@ def main():
         dst.copy_(src)
     torch.cuda.synchronize()
     del src, dst
+
+    # ---- the two ceilings, after everything else: for a second or two after milliseconds of nothing but matrix
+    # instructions or reads the device serves host copies more slowly (the page-locked C2 call took 0.86-0.98 ms
+    # instead of 0.62 ms when it was measured right behind them)
+    # what the int8 matrix instruction sustains on this device with nothing else issued
+    ceiling_tops, ceiling_ghz = capi.bench_mfma_ceiling(2.0, stream=stream)
+    # what a kernel that only reads gets out of device memory (1 GiB, the GEMV kernels' access pattern)
+    read_ceiling_gbs = max(capi.bench_hbm_read_ceiling(1 << 30, wps, stream=stream) for wps in (1, 2, 4)) * 1e3
 
     out = {
         "metric": METRIC, "value": round(value, 3), "unit": "TOPS", "n_gpus": 1,
