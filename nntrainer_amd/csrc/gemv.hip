@@ -17,6 +17,7 @@
  * HBM: per output column it reads the column's packed weights exactly once,
  * 16 bytes per lane per load, all loads of a group in flight together.
  */
+#include <string>
 #include <type_traits>
 
 #include "gemv_device.h"
@@ -265,6 +266,19 @@ __global__ __launch_bounds__(256) void gemv_fused_multi_kernel(FusedMulti mw, co
   gemv_fused_body<DT, T, G, LATE, FK>(mw.w[i], x, mw.C[i], b - first);
 }
 
+/* The name a launch is noted under, with the instance's template arguments as numbers (what a kernel trace
+ * prints): built once per instance. */
+template <int FAMILY, int... V> const char *kernel_name(const char *base) { /* FAMILY: one number a kernel template */
+  static const std::string name = [&] {
+    std::string n = std::string(base) + "<";
+    const int v[] = {V...};
+    for (size_t i = 0; i < sizeof(v) / sizeof(v[0]); ++i) n += (i ? ", " : "") + std::to_string(v[i]);
+    (void)FAMILY;
+    return n + ">";
+  }();
+  return name.c_str();
+}
+
 /* Where a wavefront asks for its weights (gemv_fused_rows' LATE), by the row length and the weights of the
  * launch (all its matrices together). Measured with the usual row lengths as constants (us a call, in front /
  * behind / half and half): Q4_K 2048 x 4096 4.35 / 4.57 / 4.3, 4096 x 4096 5.35 / 5.25 / 5.2, 12288 x 4096
@@ -316,7 +330,8 @@ int launch_fused_many(int count, const hipq_weight *const *w, const float *x, fl
   }
   const size_t lds = fused_act_bytes<DT>((int)w[0]->K) + 4 * GemvLds<DT, 1, G, false>::DWORDS * sizeof(uint32_t);
   with_late<T>(fused_weights_late(w[0]->K, weights), w[0]->K, [&](auto L, auto FK) {
-    hipq::launch_kernel("gemv_fused_multi_kernel<DT, T, G, LATE, FK>", (gemv_fused_multi_kernel<DT, T, G, decltype(L)::value, decltype(FK)::value>),
+    hipq::launch_kernel(kernel_name<1, DT, T, G, decltype(L)::value, decltype(FK)::value>("gemv_fused_multi_kernel"),
+                        (gemv_fused_multi_kernel<DT, T, G, decltype(L)::value, decltype(FK)::value>),
                         dim3((unsigned)blocks), dim3(256), lds, s, mw, x);
   });
   HIPQ_HIP(hipGetLastError());
@@ -328,7 +343,8 @@ int launch_fused_wide(const hipq_weight *w, const float *x, float *C, hipStream_
   const unsigned grid = (unsigned)((w->N + WV * G - 1) / (WV * G));
   const size_t lds = fused_act_bytes<DT>((int)w->K) + WV * GemvLds<DT, 1, G, false>::DWORDS * sizeof(uint32_t);
   with_late<T>(fused_weights_late(w->K, w->N * w->K), w->K, [&](auto L, auto FK) {
-    hipq::launch_kernel("gemv_fused_wide_kernel<DT, T, G, WV, LATE, FK>", (gemv_fused_wide_kernel<DT, T, G, WV, decltype(L)::value, decltype(FK)::value>),
+    hipq::launch_kernel(kernel_name<2, DT, T, G, WV, decltype(L)::value, decltype(FK)::value>("gemv_fused_wide_kernel"),
+                        (gemv_fused_wide_kernel<DT, T, G, WV, decltype(L)::value, decltype(FK)::value>),
                         dim3(grid), dim3(64 * WV), lds, s, wview(w), x, C);
   });
   HIPQ_HIP(hipGetLastError());
@@ -341,7 +357,8 @@ int launch_fused_one(const hipq_weight *w, const float *x, float *C, hipStream_t
   const size_t lds = fused_act_bytes<DT>((int)w->K) + 4 * GemvLds<DT, 1, G, false>::DWORDS * sizeof(uint32_t);
   with_late<T>(fused_weights_late(w->K, w->N * w->K), w->K, [&](auto L, auto FK) {
     constexpr int LATE = decltype(L)::value == 2 && G < 2 ? 0 : decltype(L)::value; /* half and half takes two passes */
-    hipq::launch_kernel("gemv_fused_kernel<DT, T, G, LATE, FK>", (gemv_fused_kernel<DT, T, G, LATE, decltype(FK)::value>), dim3(grid),
+    hipq::launch_kernel(kernel_name<3, DT, T, G, LATE, decltype(FK)::value>("gemv_fused_kernel"),
+                        (gemv_fused_kernel<DT, T, G, LATE, decltype(FK)::value>), dim3(grid),
                         dim3(256), lds, s, wview(w), x, C);
   });
   HIPQ_HIP(hipGetLastError());
@@ -355,10 +372,10 @@ int launch_stream(const hipq_weight *w, const QAct *qa, float *C, hipStream_t s)
   const size_t lds = 4 * GemvLds<DT, 1, G, false>::DWORDS * sizeof(uint32_t);
   constexpr int USUAL = T == 64 ? 4096 : 1024; /* the row length that has an instance of its own */
   if (w->K == USUAL)
-    hipq::launch_kernel("gemv_stream_kernel<DT, T, G, GPW, K>", (gemv_stream_kernel<DT, T, G, GPW, USUAL>), dim3(grid), dim3(256),
+    hipq::launch_kernel(kernel_name<4, DT, T, G, GPW, USUAL>("gemv_stream_kernel"), (gemv_stream_kernel<DT, T, G, GPW, USUAL>), dim3(grid), dim3(256),
                         lds, s, wview(w), qview(*qa), C);
   else
-    hipq::launch_kernel("gemv_stream_kernel<DT, T, G, GPW, 0>", (gemv_stream_kernel<DT, T, G, GPW, 0>), dim3(grid), dim3(256), lds,
+    hipq::launch_kernel(kernel_name<4, DT, T, G, GPW, 0>("gemv_stream_kernel"), (gemv_stream_kernel<DT, T, G, GPW, 0>), dim3(grid), dim3(256), lds,
                         s, wview(w), qview(*qa), C);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
@@ -371,10 +388,10 @@ int launch_one(const hipq_weight *w, const QAct *qa, int M, int pair_rows, float
   const size_t lds = 4 * GemvLds<DT, R, G, PW>::DWORDS * sizeof(uint32_t);
   constexpr int USUAL = T == 64 ? 4096 : 1024; /* the row length that has an instance of its own */
   if (w->K == USUAL)
-    hipq::launch_kernel("gemv_kernel<DT, T, R, G, PW, K>", (gemv_kernel<DT, T, R, G, PW, USUAL>), dim3(grid), dim3(256), lds, s,
+    hipq::launch_kernel(kernel_name<5, DT, T, R, G, PW, USUAL>("gemv_kernel"), (gemv_kernel<DT, T, R, G, PW, USUAL>), dim3(grid), dim3(256), lds, s,
                         wview(w), qview(*qa), M, pair_rows, C, ldc);
   else
-    hipq::launch_kernel("gemv_kernel<DT, T, R, G, PW, 0>", (gemv_kernel<DT, T, R, G, PW, 0>), dim3(grid), dim3(256), lds, s,
+    hipq::launch_kernel(kernel_name<5, DT, T, R, G, PW, 0>("gemv_kernel"), (gemv_kernel<DT, T, R, G, PW, 0>), dim3(grid), dim3(256), lds, s,
                         wview(w), qview(*qa), M, pair_rows, C, ldc);
   HIPQ_HIP(hipGetLastError());
   return HIPQ_OK;
@@ -394,7 +411,8 @@ int launch_fused_swiglu_one(const hipq_weight *wa, const hipq_weight *wm, const 
   const unsigned grid = (unsigned)((wa->N + 4 * G - 1) / (4 * G));
   const size_t lds = fused_act_bytes<DT>((int)wa->K) + 4 * GemvLds<DT, 1, G, false>::DWORDS * sizeof(uint32_t);
   with_late<T>(fused_weights_late(wa->K, 2 * wa->N * wa->K), wa->K, [&](auto L, auto FK) {
-    hipq::launch_kernel("gemv_fused_swiglu_kernel<DT, T, G, LATE, FK>", (gemv_fused_swiglu_kernel<DT, T, G, decltype(L)::value, decltype(FK)::value>),
+    hipq::launch_kernel(kernel_name<6, DT, T, G, decltype(L)::value, decltype(FK)::value>("gemv_fused_swiglu_kernel"),
+                        (gemv_fused_swiglu_kernel<DT, T, G, decltype(L)::value, decltype(FK)::value>),
                         dim3(grid), dim3(256), lds, s, wview(wa), wview(wm), x, out);
   });
   HIPQ_HIP(hipGetLastError());
