@@ -876,7 +876,7 @@ def main():
             "decode_1_row_ms": round(c5_decode_ms, 5),
             "decode_batch_8_rows_ms": round(c5_rows8_ms, 5), "decode_batch_16_rows_ms": round(c5_rows16_ms, 5),
             "decode_batch_8_rows_in_a_graph_qkv_and_gate_up_as_one_launch_each_ms": round(c5_rows8_grouped_ms, 5),
-            "lm_head_q4_0_n151936": {"kernel": "gemm_rows_q40_kernel (one and eight rows)",
+            "lm_head_q4_0_n151936": {"kernel": "gemv_stream_kernel (one row, behind the quantizer's launch), gemm_rows_q40_kernel (eight rows)",
                                      "rows_1_kernel_ms": round(c5_head_ms, 5), "rows_1_ms_per_call": round(c5_head_all_ms, 5),
                                      "rows_8_kernel_ms": round(c5_head_rows8[0], 5),
                                      "rows_8_ms_per_call": round(c5_head_rows8[1], 5),

@@ -323,7 +323,7 @@ namespace hipq {
  * with 24 / 32 rows 25.2 / 29.6 against 28.4 / 28.5, 4096 x 4096 with 48 / 64 rows 16.5 / 20.3 against
  * 19.7 / 19.9, 151936 x 1024 with 24 rows 71.7 against 68.7, 1024 x 3072 with 64 rows 9.5 against 15.4. */
 static bool rows_q40_pay(int64_t N, int64_t K, int64_t M) {
-  if (M == 1) return K <= 1024 && N >= 65536;
+  if (M == 1) return false; /* the streamed GEMV, since its waits count every load: 151936 x 1024 28.5 -> 18.3 us a call, 65536 x 1024 15.2 -> 10.6 */
   if (M == 2) return N >= 12288;
   if (M <= 4) return N >= 6144;
   if (M <= TC) return N >= 3072;
