@@ -390,6 +390,12 @@ int launch_one(const hipq_weight *w, const QAct *qa, int M, int pair_rows, float
   if (w->K == USUAL)
     hipq::launch_kernel(kernel_name<5, DT, T, R, G, PW, USUAL>("gemv_kernel"), (gemv_kernel<DT, T, R, G, PW, USUAL>), dim3(grid), dim3(256), lds, s,
                         wview(w), qview(*qa), M, pair_rows, C, ldc);
+  else if (R == 1 && T == 64 && w->K == 2048) /* one row: two more lengths */
+    hipq::launch_kernel(kernel_name<5, DT, T, R, G, PW, 2048>("gemv_kernel"), (gemv_kernel<DT, T, R, G, PW, R == 1 && T == 64 ? 2048 : 0>), dim3(grid),
+                        dim3(256), lds, s, wview(w), qview(*qa), M, pair_rows, C, ldc);
+  else if (R == 1 && T == 64 && w->K == 3072)
+    hipq::launch_kernel(kernel_name<5, DT, T, R, G, PW, 3072>("gemv_kernel"), (gemv_kernel<DT, T, R, G, PW, R == 1 && T == 64 ? 3072 : 0>), dim3(grid),
+                        dim3(256), lds, s, wview(w), qview(*qa), M, pair_rows, C, ldc);
   else
     hipq::launch_kernel(kernel_name<5, DT, T, R, G, PW, 0>("gemv_kernel"), (gemv_kernel<DT, T, R, G, PW, 0>), dim3(grid), dim3(256), lds, s,
                         wview(w), qview(*qa), M, pair_rows, C, ldc);
@@ -440,8 +446,10 @@ int launch_m1(const hipq_weight *w, const QAct *qa, float *C, int64_t ldc, hipSt
    * waits cannot count (any row length); Q6_K and smaller matrices are better off with more, shorter
    * wavefronts, and so are rows of 4096 now that the plain kernel's waits count every load (us a call with
    * the quantizer's launch, streamed -> plain: Q4_K 32768 x 4096 17.6 -> 16.1, 65536 29.0 -> 26.4, 151936
-   * 57.2 -> 53.9; Q4_0 32768 20.1 -> 17.7, 151936 59.0 -> 57.0) */
-  if (DT != HIPQ_Q6_K && w->N >= 32768 && w->K < HIPQ_KCHUNK && units >= 64)
+   * 57.2 -> 53.9; Q4_0 32768 20.1 -> 17.7, 151936 59.0 -> 57.0), and rows of 2048 and 3072, which the plain kernel
+   * has as constants for one row too (Q4_K 151936 x 2048 35 -> 29, 65536 x 2048 18.6 -> 15.5, 151936 x 3072 47.7 -> 46.2;
+   * Q4_0 151936 x 2048 39.7 -> 31) */
+  if (DT != HIPQ_Q6_K && w->N >= 32768 && w->K < HIPQ_KCHUNK && w->K != 2048 && w->K != 3072 && units >= 64)
     return launch_stream<DT, 64, 4, 2>(w, qa, C, s);
   /* the same for short rows (16 lanes a row, four rows side by side, eight a group): a wavefront of
    * the plain kernel below would have four short rows for all its work. Kernel us, plain -> streamed:
