@@ -497,11 +497,14 @@ template <int DT> int launch_fused(const hipq_weight *w, const float *x, float *
       if (wgs <= 256 || rest == 0 || rest >= 128) return launch_fused_wide<DT, 64, 2, 12>(w, x, C, s);
       return launch_fused_one<DT, 64, 4>(w, x, C, s);
     }
+    /* shorter rows: twelve wavefronts of two rows up to one round of them (6144 x 2048 4.85 -> 4.1 us a call,
+     * 4096 x 2048 4.3 -> 4.1, 3072 x 3072 5.3 -> 5.05), of four rows up to one round of those */
+    if (w->N >= 2048 && (w->N + 23) / 24 <= 256) return launch_fused_wide<DT, 64, 2, 12>(w, x, C, s);
     if (pick_group(w->N, 8) == 4 && (w->N + 47) / 48 <= 256) return launch_fused_wide<DT, 64, 4, 12>(w, x, C, s);
   }
-  /* Q4_0 with rows of 4096: four rows a wavefront from 4096 rows on (4096 x 4096 6.65 -> 6.25 us a call, 6144 x 4096
-   * 7.65 -> 7.3) */
-  if (DT == HIPQ_Q4_0 && w->K == HIPQ_KCHUNK && w->N >= 4096) return launch_fused_one<DT, 64, 4>(w, x, C, s);
+  /* Q4_0: four rows a wavefront from 4096 rows on (4096 x 4096 6.65 -> 6.25 us a call, 6144 x 4096 7.65 -> 7.3,
+   * 4096 x 2048 4.4 -> 4.15, 6144 x 2048 4.9 -> 4.6) */
+  if (DT == HIPQ_Q4_0 && w->N >= 4096) return launch_fused_one<DT, 64, 4>(w, x, C, s);
   switch (pick_group(w->N, 8)) {
   case 8:
     return launch_fused_one<DT, 64, 8>(w, x, C, s);
