@@ -321,10 +321,18 @@ namespace hipq {
  * 12288 x 4096 28.3 -> 17.6, 4096 x 4096 19.4 -> 10.9, 1024 x 3072 15.1 -> 9.4, 1024 x 1024 8.5 -> 6.7,
  * 151936 x 1024 68.4 -> 49.0; with more passes the launch grows and the GEMM does not: 12288 x 4096
  * with 24 / 32 rows 25.2 / 29.6 against 28.4 / 28.5, 4096 x 4096 with 48 / 64 rows 16.5 / 20.3 against
- * 19.7 / 19.9, 151936 x 1024 with 24 rows 71.7 against 68.7, 1024 x 3072 with 64 rows 9.5 against 15.4. */
+ * 19.7 / 19.9, 151936 x 1024 with 24 rows 71.7 against 68.7, 1024 x 3072 with 64 rows 9.5 against 15.4.
+ * Against the engine with its row lengths compiled in (calls in a row on one stream, us, engine
+ * against this kernel): two rows 12288 x 4096 12.2 / 13.1, 12288 x 2048 9.2 / 9.6, 32768 x 4096 22.0 /
+ * 21.6, 65536 x 2048 24.9 / 22.8, 151936 x 2048 49.2 / 43.0; three and four rows 6144 x 4096 10.5 / 10.8,
+ * 12288 x 4096 14.3 / 13.2, 4096 x 2048 7.1 / 7.7, 12288 x 2048 10.9 / 9.6. Where the kernel quantizes
+ * the rows itself (K of one round, up to 512 tiles) it is one launch against the engine's two, and
+ * two to four rows take it from 512 columns: 512 ... 3072 x 1024 7.0 / 5.3, 6144 x 1024 7.1 / 5.5. */
 static bool rows_q40_pay(int64_t N, int64_t K, int64_t M) {
   if (M == 1) return false; /* the streamed GEMV, since its waits count every load: 151936 x 1024 28.5 -> 18.3 us a call, 65536 x 1024 15.2 -> 10.6 */
-  if (M == 2) return N >= 12288;
+  const bool quantizes = K <= BR * 32 && (N + 31) / 32 <= 512; /* one launch: the form that takes the fp32 rows */
+  if (M <= 4 && quantizes) return N >= 512;
+  if (M == 2) return N >= (K <= BR * 32 ? 12288 : 32768);
   if (M <= 4) return N >= 6144;
   if (M <= TC) return N >= 3072;
   if (M <= 2 * TC) return N >= 512;

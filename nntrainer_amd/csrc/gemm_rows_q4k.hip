@@ -310,7 +310,8 @@ namespace hipq {
 
 /* Where it beats the GEMV engine (measured, kernel us old -> new): five to eight rows from 1024
  * columns up (2048 x 1024: 5.5 -> 4.0; 4096 x 4096: 16.4 -> 8.3; 12288 x 4096: 39.0 -> 11.2;
- * 151936 x 4096: 421 -> 75), four rows from 4096 columns (4096 x 4096: 8.7 -> 8.3; 12288 x 4096:
+ * 151936 x 4096: 421 -> 75); with fewer rows where the last lines of the rule below say (at first four
+ * rows from 4096 columns, 4096 x 4096: 8.7 -> 8.3; 12288 x 4096:
  * 16.4 -> 11.0), three from 8192 (12288 x 4096: 14.2 -> 11; 4096 x 4096: 7.1 against 8.2). A round
  * of a workgroup takes 1.7 us, most of it the issue of its vector instructions (about 290 a
  * wavefront and super-block: nibble expansion, scale multiplies, the chains), so the kernel
@@ -328,7 +329,16 @@ bool gemm_rows_q4k_fits(const hipq_weight *w, int64_t M) {
     const int64_t tiles = (w->N + 31) / 32, passes = (M + TC - 1) / TC;
     return tiles * passes * (w->K / 256) <= 8192;
   }
-  return (M == 4 && w->N >= 4096) || (M == 3 && w->N >= 8192);
+  /* Two to four rows against the engine with its row lengths compiled in (calls in a row on one
+   * stream, us, engine / this kernel). Four rows: 4096 x 4096 10.4 / 11.2, 6144 x 4096 11.7 / 11.4,
+   * 6144 x 2048 8.6 / 8.5, 12288 x 2048 12.3 / 9.9. Three: 8192 x 4096 11.0 / 11.5, 12288 x 4096 13.5 /
+   * 13.4, 32768 x 4096 24.3 / 22.1, 12288 x 2048 11.2 / 9.8, 6144 x 2048 7.9 / 8.4. Two rows stay with
+   * the engine (12288 x 4096 10.5 / 13.5, 32768 x 4096 18.0 / 22.0) but for rows of 1024, where the
+   * engine's wavefronts hold a quarter of a row each: 16384 x 1024 10.9 / 8.3. */
+  const bool long_rows = w->K >= 4096;
+  if (M == 4) return w->N >= (long_rows ? 6144 : 4096);
+  if (M == 3) return w->N >= (long_rows ? 12288 : 8192);
+  return M == 2 && w->K <= 1024 && w->N >= 16384;
 }
 
 /* Several weights of one K in one launch (hipq_matmul_multi): what counts is the launch's width, the

@@ -83,11 +83,13 @@ def test_small_m_matches_oracle(hipq, cr, kind, m):
                                    (8, 1024, 256), (5, 3000, 4096), (8, 1030, 8192), (6, 1024, 5376),
                                    (4, 4100, 1280), (9, 1100, 1024), (14, 2048, 512), (16, 1024, 2048),
                                    (11, 4000, 4096), (6, 32768, 1024), (8, 8200, 4096), (24, 4096, 2048),
-                                   (64, 2048, 2048), (33, 1056, 4096)])
+                                   (64, 2048, 2048), (33, 1056, 4096), (2, 16400, 1024), (4, 6150, 4096),
+                                   (3, 12290, 4096), (4, 4100, 4096), (2, 33000, 2048)])
 def test_small_m_on_large_matrices_matches_oracle(hipq, cr, kind, m, n, k):
     """Three to sixteen rows against larger matrices, where Q4_K leaves the GEMV engine (and, from
     nine rows, the prefill GEMM) for the matrix-core kernel of gemm_rows_q4k.hip (five rows and
-    more from 1024 columns up, four from 4096, three from 8192; more than eight rows as passes
+    more from 1024 columns up, four from 4096 or, with rows of 4096, 6144, three from 8192 or 12288,
+    two against 16384 rows of 1024; more than eight rows as passes
     of eight side by side in one launch, up to 64 rows where the product is small, the later
     passes with fewer rows under the 4-row rule or none): rows under the reference's
     4-row rule and under its row rule in one call
@@ -112,12 +114,14 @@ def test_small_m_on_large_matrices_matches_oracle(hipq, cr, kind, m, n, k):
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 65553, 1024), (1, 65536, 256), (2, 12300, 512), (3, 6150, 768),
+                                   (2, 600, 1024), (3, 16000, 512), (4, 2050, 768), (2, 16500, 1024),
                                    (4, 6144, 1024), (5, 3100, 1280), (7, 3072, 256), (9, 640, 256),
                                    (12, 600, 2304), (16, 513, 1024), (17, 520, 5120), (40, 1500, 1024),
                                    (64, 4096, 256), (57, 2050, 1280)])
 def test_q4_0_few_rows_on_the_matrix_cores_match_oracle(hipq, cr, m, n, k):
     """Q4_0 with a few rows where gemm_rows_q40.hip takes them (one row against a wide matrix of
-    short rows, two rows from 12288 columns, three and four from 6144, five to eight from 3072,
+    short rows, two rows from 12288 columns of 1024 or 32768 longer ones, three and four from 6144,
+    two to four from 512 where the kernel quantizes the rows itself, five to eight from 3072,
     nine to sixteen from 512, up to 64 while the launch stays small): one to eight passes, one to
     five rounds of 32 blocks with the last one partly or wholly one wavefront's, column counts
     that end inside a 32-column tile. Same bits as the reference."""
