@@ -327,11 +327,12 @@ namespace hipq {
  * 21.6, 65536 x 2048 24.9 / 22.8, 151936 x 2048 49.2 / 43.0; three and four rows 6144 x 4096 10.5 / 10.8,
  * 12288 x 4096 14.3 / 13.2, 4096 x 2048 7.1 / 7.7, 12288 x 2048 10.9 / 9.6. Where the kernel quantizes
  * the rows itself (K of one round, up to 512 tiles) it is one launch against the engine's two, and
- * two to four rows take it from 512 columns: 512 ... 3072 x 1024 7.0 / 5.3, 6144 x 1024 7.1 / 5.5. */
+ * two to eight rows take it from 512 columns: 512 ... 3072 x 1024 with two to four 7.0 / 5.3, 6144 x
+ * 1024 7.1 / 5.5, 3072 x 1024 with six and eight 8.0 / 5.5. */
 static bool rows_q40_pay(int64_t N, int64_t K, int64_t M) {
   if (M == 1) return false; /* the streamed GEMV, since its waits count every load: 151936 x 1024 28.5 -> 18.3 us a call, 65536 x 1024 15.2 -> 10.6 */
   const bool quantizes = K <= BR * 32 && (N + 31) / 32 <= 512; /* one launch: the form that takes the fp32 rows */
-  if (M <= 4 && quantizes) return N >= 512;
+  if (M <= TC && quantizes) return N >= 512;
   if (M == 2) return N >= (K <= BR * 32 ? 12288 : 32768);
   if (M <= 4) return N >= 6144;
   if (M <= TC) return N >= 3072;

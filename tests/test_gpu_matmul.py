@@ -115,13 +115,14 @@ def test_small_m_on_large_matrices_matches_oracle(hipq, cr, kind, m, n, k):
 
 @pytest.mark.parametrize("m,n,k", [(1, 65553, 1024), (1, 65536, 256), (2, 12300, 512), (3, 6150, 768),
                                    (2, 600, 1024), (3, 16000, 512), (4, 2050, 768), (2, 16500, 1024),
+                                   (6, 1030, 1024), (8, 2048, 512), (5, 520, 768),
                                    (4, 6144, 1024), (5, 3100, 1280), (7, 3072, 256), (9, 640, 256),
                                    (12, 600, 2304), (16, 513, 1024), (17, 520, 5120), (40, 1500, 1024),
                                    (64, 4096, 256), (57, 2050, 1280)])
 def test_q4_0_few_rows_on_the_matrix_cores_match_oracle(hipq, cr, m, n, k):
     """Q4_0 with a few rows where gemm_rows_q40.hip takes them (one row against a wide matrix of
     short rows, two rows from 12288 columns of 1024 or 32768 longer ones, three and four from 6144,
-    two to four from 512 where the kernel quantizes the rows itself, five to eight from 3072,
+    two to eight from 512 where the kernel quantizes the rows itself, five to eight from 3072,
     nine to sixteen from 512, up to 64 while the launch stays small): one to eight passes, one to
     five rounds of 32 blocks with the last one partly or wholly one wavefront's, column counts
     that end inside a 32-column tile. Same bits as the reference."""
